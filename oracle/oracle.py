@@ -1,0 +1,254 @@
+"""ctypes loader for the CPU oracle (test infrastructure only).
+
+Loads oracle/libpto_oracle.so (the plain-C restatement of the reference's CPU-simulation ops)
+and, when it has been built, oracle/_ref/libpto_ref.so (the reference's own headers compiled
+behind a C ABI).  Only tests, the smoke check and the benchmark's CPU-baseline leg import this.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = os.path.join(_HERE, "libpto_oracle.so")
+_REF = os.path.join(_HERE, "_ref", "libpto_ref.so")
+
+BL_ROW, BL_COL = 0, 1
+SL_NONE, SL_ROW, SL_COL = 0, 1, 2
+
+
+class Layout(C.Structure):
+    _fields_ = [("rows", C.c_int32), ("cols", C.c_int32), ("blayout", C.c_int32), ("slayout", C.c_int32),
+                ("inner_rows", C.c_int32), ("inner_cols", C.c_int32)]
+
+
+def build(ref=True):
+    """Compile the oracle (and the reference shim when the reference tree is present)."""
+    subprocess.run(["make", "-s", "-C", _HERE], check=True)
+    if ref and os.path.isdir(os.environ.get("PTO_REFERENCE", "/root/reference")):
+        subprocess.run(["make", "-s", "-C", _HERE, "ref"], check=True)
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB):
+            build(ref=False)
+        L = C.CDLL(_LIB)
+        L.po_make_layout.restype = Layout
+        L.po_make_layout.argtypes = [C.c_int] * 6
+        L.po_tile_offset.restype = C.c_size_t
+        L.po_tile_offset.argtypes = [C.POINTER(Layout), C.c_size_t, C.c_size_t]
+        L.po_f32_to_f16_rne.restype = C.c_uint16
+        L.po_f32_to_f16_rne.argtypes = [C.c_uint32]
+        L.po_f32_to_f16_rna.restype = C.c_uint16
+        L.po_f32_to_f16_rna.argtypes = [C.c_uint32]
+        L.po_f32_to_bf16_rne.restype = C.c_uint16
+        L.po_f32_to_bf16_rne.argtypes = [C.c_uint32]
+        L.po_tgather_mask.restype = C.c_size_t
+        L.po_online_cpus.restype = C.c_int
+        for name in ("po_tcvt_f32_f16", "po_tcvt_f32_bf16", "po_tcvt_f16_f32"):
+            getattr(L, name).argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+            getattr(L, name).restype = None
+        L.po_tcvt_f32_s32.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        L.po_gather_rows.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_int]
+        L.po_gather_rows.restype = None
+        L.po_gemm_f16f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 7
+        L.po_gemm_f16f32.restype = None
+        L.po_fa_auto_f32.argtypes = [C.c_void_p] * 4 + [C.c_int] * 3
+        L.po_fa_auto_f32.restype = None
+        L.po_fa_stream_f16.argtypes = [C.c_void_p] * 6 + [C.c_int] * 8
+        L.po_fa_stream_f16.restype = None
+        L.po_result_cmp_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.POINTER(C.c_double),
+                                        C.POINTER(C.c_size_t)]
+        L.po_result_cmp_f32.restype = C.c_int
+        _lib = L
+    return _lib
+
+
+def ref():
+    """The compiled reference, or None when oracle/_ref has not been built."""
+    if not os.path.exists(_REF):
+        return None
+    return C.CDLL(_REF)
+
+
+def online_cpus():
+    return lib().po_online_cpus()
+
+
+# ------------------------------------------------------------------ layouts
+def make_layout(rows, cols, blayout=BL_ROW, slayout=SL_NONE, elem_bytes=2, fractal_bytes=512):
+    return lib().po_make_layout(rows, cols, blayout, slayout, elem_bytes, fractal_bytes)
+
+
+def tile_offset(L, r, c):
+    return lib().po_tile_offset(C.byref(L), r, c)
+
+
+def _i64x5(v):
+    return (C.c_int64 * 5)(*[int(x) for x in v])
+
+
+def tload(L, dtype, gm, shape, stride, valid_row=None, valid_col=None, pad=0):
+    """Returns the tile's linear storage after TLOAD (or None where the reference asserts)."""
+    gm = np.ascontiguousarray(gm)
+    tile = np.zeros(L.rows * L.cols, dtype=dtype)
+    padv = np.array([pad], dtype=dtype)
+    vr = L.rows if valid_row is None else valid_row
+    vc = L.cols if valid_col is None else valid_col
+    rc = lib().po_tload(_p(tile), C.byref(L), C.c_int(tile.itemsize), _p(gm), _i64x5(shape), _i64x5(stride),
+                        C.c_int(vr), C.c_int(vc), _p(padv))
+    return tile if rc == 0 else None
+
+
+def tstore(out, shape, stride, tile, L, valid_row=None, valid_col=None):
+    vr = L.rows if valid_row is None else valid_row
+    vc = L.cols if valid_col is None else valid_col
+    return lib().po_tstore(_p(out), _i64x5(shape), _i64x5(stride), _p(tile), C.byref(L), C.c_int(tile.itemsize),
+                           C.c_int(vr), C.c_int(vc))
+
+
+def textract(Ld, dvr, dvc, src, Ls, svr, svc, idx_row, idx_col, mode=0):
+    dst = np.zeros(Ld.rows * Ld.cols, dtype=src.dtype)
+    rc = lib().po_textract(_p(dst), C.byref(Ld), C.c_int(dvr), C.c_int(dvc), _p(src), C.byref(Ls), C.c_int(svr),
+                           C.c_int(svc), C.c_int(src.itemsize), C.c_int(idx_row), C.c_int(idx_col), C.c_int(mode))
+    return dst if rc == 0 else None
+
+
+def tmov(Ld, src, Ls, valid_row, valid_col):
+    dst = np.zeros(Ld.rows * Ld.cols, dtype=src.dtype)
+    lib().po_tmov(_p(dst), C.byref(Ld), _p(src), C.byref(Ls), C.c_int(src.itemsize), C.c_int(valid_row),
+                  C.c_int(valid_col))
+    return dst
+
+
+def tmatmul(a, La, b, Lb, Lc, M, N, K, acc=None, bias=None, threads=0):
+    """a, b are tile storages (uint16 fp16 bits, float32 or int8); returns the Acc tile storage."""
+    L = lib()
+    if a.dtype == np.uint16:
+        dst = np.zeros(Lc.rows * Lc.cols, dtype=np.float32)
+        if bias is not None:
+            L.po_tmatmul_bias_f16(_p(dst), C.byref(Lc), _p(a), C.byref(La), _p(b), C.byref(Lb), _p(bias), C.c_int(M),
+                                  C.c_int(N), C.c_int(K), C.c_int(threads))
+            return dst
+        fn = L.po_tmatmul_f16
+    elif a.dtype == np.float32:
+        dst = np.zeros(Lc.rows * Lc.cols, dtype=np.float32)
+        fn = L.po_tmatmul_f32
+    else:
+        dst = np.zeros(Lc.rows * Lc.cols, dtype=np.int32)
+        fn = L.po_tmatmul_s8
+    fn(_p(dst), _p(acc) if acc is not None else None, C.byref(Lc), _p(a), C.byref(La), _p(b), C.byref(Lb),
+       C.c_int(M), C.c_int(N), C.c_int(K), C.c_int(threads))
+    return dst
+
+
+def gemm_f16f32(A, B, base_k=64, row0=0, row1=0, threads=0):
+    """A [m,k] fp16, B [n,k] fp16 (column-major k x n) -> C [m,n] fp32 (rows outside [row0,row1) left 0)."""
+    A = np.ascontiguousarray(A).view(np.uint16)
+    B = np.ascontiguousarray(B).view(np.uint16)
+    m, k = A.shape
+    n = B.shape[0]
+    Cm = np.zeros((m, n), dtype=np.float32)
+    lib().po_gemm_f16f32(_p(Cm), _p(A), _p(B), m, n, k, base_k, row0, row1, threads)
+    return Cm
+
+
+# --------------------------------------------------------------- conversion
+def tcvt_f32_f16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().po_tcvt_f32_f16(_p(out), _p(x), x.size)
+    return out
+
+
+def tcvt_f32_bf16(x):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.uint16)
+    lib().po_tcvt_f32_bf16(_p(out), _p(x), x.size)
+    return out
+
+
+def tcvt_f16_f32(h):
+    h = np.ascontiguousarray(h).view(np.uint16)
+    out = np.empty(h.shape, dtype=np.float32)
+    lib().po_tcvt_f16_f32(_p(out), _p(h), h.size)
+    return out
+
+
+def tcvt_f32_s32(x, round_mode):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty(x.shape, dtype=np.int32)
+    lib().po_tcvt_f32_s32(_p(out), _p(x), x.size, round_mode)
+    return out
+
+
+# ------------------------------------------------------------------- gather
+def tgather_index(Ld, src0, L0, idx, L1, valid_row, valid_col):
+    dst = np.zeros(Ld.rows * Ld.cols, dtype=src0.dtype)
+    idx = np.ascontiguousarray(idx, dtype=np.int32)
+    lib().po_tgather_index(_p(dst), C.byref(Ld), _p(src0), C.byref(L0), _p(idx), C.byref(L1),
+                           C.c_int(src0.itemsize), C.c_int(valid_row), C.c_int(valid_col))
+    return dst
+
+
+def tgather_mask(Ld, src, Ls, valid_row, valid_col, pattern):
+    dst = np.zeros(Ld.rows * Ld.cols, dtype=src.dtype)
+    n = lib().po_tgather_mask(_p(dst), C.byref(Ld), _p(src), C.byref(Ls), C.c_int(src.itemsize), C.c_int(valid_row),
+                              C.c_int(valid_col), C.c_int(pattern))
+    return dst, n
+
+
+def mgather(Ld, gm, idx, Li, valid_row, valid_col):
+    dst = np.zeros(Ld.rows * Ld.cols, dtype=gm.dtype)
+    idx = np.ascontiguousarray(idx, dtype=np.int32)
+    lib().po_mgather(_p(dst), C.byref(Ld), _p(gm), _p(idx), C.byref(Li), C.c_int(gm.itemsize), C.c_int(valid_row),
+                     C.c_int(valid_col))
+    return dst
+
+
+def gather_rows(table, idx):
+    table = np.ascontiguousarray(table)
+    idx = np.ascontiguousarray(idx, dtype=np.int32)
+    out = np.empty((idx.size, table.shape[1]), dtype=table.dtype)
+    lib().po_gather_rows(_p(out), _p(table), _p(idx), idx.size, table.shape[0], table.shape[1], table.itemsize)
+    return out
+
+
+# ---------------------------------------------------------------- attention
+def fa_auto_f32(q, k, v, threads=0):
+    q, k, v = (np.ascontiguousarray(t, dtype=np.float32) for t in (q, k, v))
+    out = np.empty_like(q)
+    lib().po_fa_auto_f32(_p(out), _p(q), _p(k), _p(v), q.shape[0], q.shape[1], threads)
+    return out
+
+
+def fa_stream_f16(q, k, v, tile_s1=128, causal=False, q_offset=0, round_away=True, threads=0):
+    """One head: q [S0,D], k,v [S1,D] fp16 -> (o fp32 [S0,D], row_max [S0], row_sum [S0])."""
+    q, k, v = (np.ascontiguousarray(t).view(np.uint16) for t in (q, k, v))
+    S0, D = q.shape
+    S1 = k.shape[0]
+    o = np.empty((S0, D), dtype=np.float32)
+    rmax = np.empty(S0, dtype=np.float32)
+    rsum = np.empty(S0, dtype=np.float32)
+    lib().po_fa_stream_f16(_p(o), _p(rmax), _p(rsum), _p(q), _p(k), _p(v), S0, S1, D, tile_s1, int(causal),
+                           q_offset, int(round_away), threads)
+    return o, rmax, rsum
+
+
+def result_cmp(expect, actual, eps):
+    e = np.ascontiguousarray(expect, dtype=np.float32)
+    a = np.ascontiguousarray(actual, dtype=np.float32)
+    md = C.c_double()
+    nb = C.c_size_t()
+    ok = lib().po_result_cmp_f32(_p(e), _p(a), e.size, eps, C.byref(md), C.byref(nb))
+    return bool(ok), md.value, nb.value

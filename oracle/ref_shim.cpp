@@ -1,0 +1,343 @@
+// C-ABI harness around the REFERENCE's own CPU-simulation headers.
+// TEST INFRASTRUCTURE ONLY.  Compiled by oracle/Makefile (target `ref`) with
+//   clang++ -std=c++20 -D__CPU_SIM -I<reference>/include
+// from the reference sources where they lie; the output (oracle/_ref/libpto_ref.so)
+// is used to validate the plain-C restatement in pto_oracle.c and as the CPU
+// baseline of the benchmark.  Nothing from the reference is copied here: this file
+// only instantiates its public templates (pto::Tile, pto::GlobalTensor, TLOAD, ...)
+// at the shapes the tests use.
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <memory>
+#include <pto/pto-inst.hpp>
+
+using namespace pto;
+
+namespace {
+
+template <typename T, int R, int C>
+using GmND = GlobalTensor<T, Shape<1, 1, 1, R, C>, Stride<R * C, R * C, R * C, C, 1>, Layout::ND>;
+// column-major view of a buffer stored [C][R]
+template <typename T, int R, int C>
+using GmDN = GlobalTensor<T, Shape<1, 1, 1, R, C>, Stride<R * C, R * C, R * C, 1, R>, Layout::DN>;
+
+// ---- GEMM tile path: TLOAD(ND->Nz A, DN->Zn B) -> TEXTRACT -> TMATMUL[_ACC] per K-step -> TSTORE ----
+// A [M,K] row-major fp16, B stored [N,K] (column-major K x N), C [M,N] fp32.  KS = K-step
+// (one TMATMUL for the first step, TMATMUL_ACC after), as the manual GEMM kernel does.
+template <int M, int K, int N, int KS>
+void gemm_tile(float *c, const uint16_t *a, const uint16_t *b)
+{
+    using MatA = Tile<TileType::Mat, half, M, KS, BLayout::ColMajor, M, KS, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, half, KS, N, BLayout::RowMajor, KS, N, SLayout::ColMajor>;
+    using L = TileLeft<half, M, KS, M, KS>;
+    using R = TileRight<half, KS, N, KS, N>;
+    using Acc = TileAcc<float, M, N, M, N>;
+    using GA = GlobalTensor<half, Shape<1, 1, 1, M, KS>, Stride<M * K, M * K, M * K, K, 1>, Layout::ND>;
+    using GB = GlobalTensor<half, Shape<1, 1, 1, KS, N>, Stride<N * K, N * K, N * K, 1, K>, Layout::DN>;
+    auto am = std::make_unique<MatA>();
+    auto bm = std::make_unique<MatB>();
+    auto al = std::make_unique<L>();
+    auto br = std::make_unique<R>();
+    auto acc = std::make_unique<Acc>();
+    for (int k0 = 0; k0 < K; k0 += KS) {
+        GA ga(reinterpret_cast<half *>(const_cast<uint16_t *>(a)) + k0);
+        GB gb(reinterpret_cast<half *>(const_cast<uint16_t *>(b)) + k0);
+        TLOAD(*am, ga);
+        TLOAD(*bm, gb);
+        TEXTRACT(*al, *am, 0, 0);
+        TEXTRACT(*br, *bm, 0, 0);
+        if (k0 == 0)
+            TMATMUL(*acc, *al, *br);
+        else
+            TMATMUL_ACC(*acc, *acc, *al, *br);
+    }
+    GmND<float, M, N> gc(c);
+    TSTORE(gc, *acc);
+}
+
+// ---- valid-region matmul as in the tmatmul ST: plain [vM,vK] x [vK,vN], both row-major ----
+template <typename TO, typename TI, int vM, int vK, int vN, bool kBias>
+void matmul_valid(TO *out, const TI *a, const TI *b, const TO *bias)
+{
+    constexpr int al = sizeof(TI) == 1 ? 32 : 16;
+    constexpr int M = (vM + al - 1) / al * al, K = (vK + al - 1) / al * al, N = (vN + al - 1) / al * al;
+    using MatA = Tile<TileType::Mat, TI, M, K, BLayout::ColMajor, vM, vK, SLayout::RowMajor, 512>;
+    using MatB = Tile<TileType::Mat, TI, K, N, BLayout::ColMajor, vK, vN, SLayout::RowMajor, 512>;
+    using L = TileLeft<TI, M, K, vM, vK>;
+    using R = TileRight<TI, K, N, vK, vN>;
+    using Acc = TileAcc<TO, M, N, vM, vN>;
+    using Bias = Tile<TileType::Bias, TO, 1, N, BLayout::RowMajor, 1, vN>;
+    auto am = std::make_unique<MatA>();
+    auto bm = std::make_unique<MatB>();
+    auto lt = std::make_unique<L>();
+    auto rt = std::make_unique<R>();
+    auto acc = std::make_unique<Acc>();
+    GmND<TI, vM, vK> ga(const_cast<TI *>(a));
+    GmND<TI, vK, vN> gb(const_cast<TI *>(b));
+    TLOAD(*am, ga);
+    TLOAD(*bm, gb);
+    TMOV(*lt, *am);
+    TMOV(*rt, *bm);
+    if constexpr (kBias) {
+        auto bt = std::make_unique<Bias>();
+        GlobalTensor<TO, Shape<1, 1, 1, 1, vN>, Stride<vN, vN, vN, vN, 1>> gbias(const_cast<TO *>(bias));
+        TLOAD(*bt, gbias);
+        TMATMUL_BIAS(*acc, *lt, *rt, *bt);
+    } else {
+        TMATMUL(*acc, *lt, *rt);
+    }
+    GmND<TO, vM, vN> gc(out);
+    TSTORE(gc, *acc);
+}
+
+// ---- elementwise conversion over an [R,C] row-major tensor, one Vec tile ----
+template <typename D, typename S, int R, int C>
+void cvt_tile(D *dst, const S *src)
+{
+    using TS = Tile<TileType::Vec, S, R, C, BLayout::RowMajor>;
+    using TD = Tile<TileType::Vec, D, R, C, BLayout::RowMajor>;
+    auto s = std::make_unique<TS>();
+    auto d = std::make_unique<TD>();
+    GmND<S, R, C> gs(const_cast<S *>(src));
+    GmND<D, R, C> gd(dst);
+    TLOAD(*s, gs);
+    TCVT(*d, *s, RoundMode::CAST_RINT);
+    TSTORE(gd, *d);
+}
+
+// ---- index gather: dst[R,C] = src0[R0,C0].flat[idx[R,C]] ----
+template <typename T, int R0, int C0, int R, int C>
+void gather_index(T *dst, const T *src0, const int32_t *idx)
+{
+    using T0 = Tile<TileType::Vec, T, R0, C0, BLayout::RowMajor>;
+    using TI = Tile<TileType::Vec, int32_t, R, C, BLayout::RowMajor>;
+    using TD = Tile<TileType::Vec, T, R, C, BLayout::RowMajor>;
+    auto s0 = std::make_unique<T0>();
+    auto ti = std::make_unique<TI>();
+    auto td = std::make_unique<TD>();
+    GmND<T, R0, C0> g0(const_cast<T *>(src0));
+    GmND<int32_t, R, C> gi(const_cast<int32_t *>(idx));
+    GmND<T, R, C> gd(dst);
+    TLOAD(*s0, g0);
+    TLOAD(*ti, gi);
+    TGATHER(*td, *s0, *ti);
+    TSTORE(gd, *td);
+}
+
+// ---- mask gather over [R,C] -> [R, C/div] ----
+template <typename T, int R, int C, MaskPattern P, int Div>
+void gather_mask(T *dst, const T *src)
+{
+    using TS = Tile<TileType::Vec, T, R, C, BLayout::RowMajor>;
+    using TD = Tile<TileType::Vec, T, R, C / Div, BLayout::RowMajor>;
+    auto s = std::make_unique<TS>();
+    auto d = std::make_unique<TD>();
+    GmND<T, R, C> gs(const_cast<T *>(src));
+    GmND<T, R, C / Div> gd(dst);
+    TLOAD(*s, gs);
+    TGATHER<TD, TS, P>(*d, *s);
+    TSTORE(gd, *d);
+}
+
+// ---- MGATHER: dst[R,C] = gm[idx[R,C]] ----
+template <typename T, int R, int C, int GN>
+void mgather(T *dst, const T *gm, const int32_t *idx)
+{
+    using TI = Tile<TileType::Vec, int32_t, R, C, BLayout::RowMajor>;
+    using TD = Tile<TileType::Vec, T, R, C, BLayout::RowMajor>;
+    auto ti = std::make_unique<TI>();
+    auto td = std::make_unique<TD>();
+    GmND<int32_t, R, C> gi(const_cast<int32_t *>(idx));
+    GmND<T, 1, GN> gsrc(const_cast<T *>(gm));
+    GmND<T, R, C> gd(dst);
+    TLOAD(*ti, gi);
+    MGATHER(*td, gsrc, *ti);
+    TSTORE(gd, *td);
+}
+
+// ---- suffix-window TEXTRACT Mat(Nz) [R,C] -> Left [R-r0, C-c0] -> plain out ----
+template <int R, int C, int R0, int C0>
+void extract_suffix(uint16_t *out, const uint16_t *in)
+{
+    using Src = Tile<TileType::Mat, half, R, C, BLayout::ColMajor, R, C, SLayout::RowMajor>;
+    using Dst = TileLeft<half, R, C, R - R0, C - C0>;
+    using Pl = Tile<TileType::Vec, half, R, C, BLayout::RowMajor, R - R0, C - C0>;
+    auto s = std::make_unique<Src>();
+    auto d = std::make_unique<Dst>();
+    auto p = std::make_unique<Pl>();
+    GmND<half, R, C> gs(reinterpret_cast<half *>(const_cast<uint16_t *>(in)));
+    TLOAD(*s, gs);
+    TEXTRACT(*d, *s, R0, C0);
+    TMOV(*p, *d);
+    GlobalTensor<half, Shape<1, 1, 1, R - R0, C - C0>,
+                 Stride<(R - R0) * (C - C0), (R - R0) * (C - C0), (R - R0) * (C - C0), C - C0, 1>>
+        go(reinterpret_cast<half *>(out));
+    TSTORE(go, *p);
+}
+
+// ---- raw tile images: what TLOAD leaves in tile storage (layout + pad) ----
+template <typename TileT, typename GmT>
+void load_image(typename TileT::DType *image, typename TileT::DType *gm)
+{
+    auto t = std::make_unique<TileT>();
+    GmT g(gm);
+    TLOAD(*t, g);
+    std::memcpy(image, t->data(), sizeof(typename TileT::DType) * TileT::Numel);
+}
+
+// ---- Auto-Mode attention on one [S,D] fp32 head (the op sequence of the tflashattn ST) ----
+template <int S, int D>
+void fa_auto(float *out, const float *q, const float *k, const float *v)
+{
+    using QP = Tile<TileType::Vec, float, S, D, BLayout::RowMajor, S, D, SLayout::NoneBox>;
+    using KT = Tile<TileType::Vec, float, D, S, BLayout::RowMajor, D, S, SLayout::NoneBox>;
+    using SP = Tile<TileType::Vec, float, S, S, BLayout::RowMajor, S, S, SLayout::NoneBox>;
+    using RR = Tile<TileType::Vec, float, S, S, BLayout::ColMajor, S, S, SLayout::NoneBox>;
+    auto qt = std::make_unique<QP>();
+    auto kt = std::make_unique<QP>();
+    auto vt = std::make_unique<QP>();
+    auto ktt = std::make_unique<KT>();
+    auto ql = std::make_unique<TileLeft<float, S, D, S, D>>();
+    auto kr = std::make_unique<TileRight<float, D, S, D, S>>();
+    auto sa = std::make_unique<TileAcc<float, S, S, S, S>>();
+    auto sc = std::make_unique<SP>();
+    auto cen = std::make_unique<SP>();
+    auto ex = std::make_unique<SP>();
+    auto pr = std::make_unique<SP>();
+    auto rmax = std::make_unique<RR>();
+    auto rsum = std::make_unique<RR>();
+    auto pl = std::make_unique<TileLeft<float, S, S, S, S>>();
+    auto vr = std::make_unique<TileRight<float, S, D, S, D>>();
+    auto oa = std::make_unique<TileAcc<float, S, D, S, D>>();
+    GmND<float, S, D> gq(const_cast<float *>(q)), gk(const_cast<float *>(k)), gv(const_cast<float *>(v)), go(out);
+    const float scale = 1.0f / std::sqrt(static_cast<float>(D));
+    TLOAD(*qt, gq);
+    TLOAD(*kt, gk);
+    TLOAD(*vt, gv);
+    TMOV(*ql, *qt);
+    TTRANS(*ktt, *kt, *kt);
+    TMOV(*kr, *ktt);
+    TMATMUL(*sa, *ql, *kr);
+    TMOV(*sc, *sa);
+    TMULS(*sc, *sc, scale);
+    TROWMAX(*rmax, *sc, *sc);
+    TROWEXPANDSUB(*cen, *sc, *rmax);
+    TEXP(*ex, *cen);
+    TROWSUM(*rsum, *ex, *ex);
+    TROWEXPANDDIV(*pr, *ex, *rsum);
+    TMOV(*pl, *pr);
+    TMOV(*vr, *vt);
+    TMATMUL(*oa, *pl, *vr);
+    TSTORE(go, *oa);
+}
+
+} // namespace
+
+extern "C" {
+
+#define REF_GEMM(M, K, N, KS)                                                          \
+    void ref_gemm_##M##x##K##x##N##_ks##KS(float *c, const uint16_t *a, const uint16_t *b) \
+    {                                                                                  \
+        gemm_tile<M, K, N, KS>(c, a, b);                                               \
+    }
+REF_GEMM(128, 64, 256, 64)
+REF_GEMM(128, 256, 256, 64)
+REF_GEMM(128, 512, 128, 64)
+REF_GEMM(256, 256, 256, 256)
+REF_GEMM(1536, 1536, 1536, 1536)
+REF_GEMM(1536, 1536, 1536, 64)
+
+void ref_matmul_f16_40x50x60(float *o, const uint16_t *a, const uint16_t *b)
+{
+    matmul_valid<float, half, 40, 50, 60, false>(o, reinterpret_cast<const half *>(a),
+                                                 reinterpret_cast<const half *>(b), nullptr);
+}
+void ref_matmul_s8_6x7x8(int32_t *o, const int8_t *a, const int8_t *b)
+{
+    matmul_valid<int32_t, int8_t, 6, 7, 8, false>(o, a, b, nullptr);
+}
+void ref_matmul_f32_120x110x50(float *o, const float *a, const float *b)
+{
+    matmul_valid<float, float, 120, 110, 50, false>(o, a, b, nullptr);
+}
+void ref_matmul_bias_f16_26x100x94(float *o, const uint16_t *a, const uint16_t *b, const float *bias)
+{
+    matmul_valid<float, half, 26, 100, 94, true>(o, reinterpret_cast<const half *>(a),
+                                                 reinterpret_cast<const half *>(b), bias);
+}
+
+// fp32 -> fp16 over n elements, n a multiple of 4096 (64 x 64 tiles)
+void ref_tcvt_f32_f16(uint16_t *dst, const float *src, size_t n)
+{
+    for (size_t i = 0; i + 4096 <= n; i += 4096)
+        cvt_tile<half, float, 64, 64>(reinterpret_cast<half *>(dst) + i, src + i);
+}
+void ref_tcvt_f16_f32(float *dst, const uint16_t *src, size_t n)
+{
+    for (size_t i = 0; i + 4096 <= n; i += 4096)
+        cvt_tile<float, half, 64, 64>(dst + i, reinterpret_cast<const half *>(src) + i);
+}
+
+void ref_tgather_index_f16_16x1024_16x128(uint16_t *dst, const uint16_t *src0, const int32_t *idx)
+{
+    gather_index<half, 16, 1024, 16, 128>(reinterpret_cast<half *>(dst), reinterpret_cast<const half *>(src0), idx);
+}
+void ref_tgather_index_f32_32x64_32x64(float *dst, const float *src0, const int32_t *idx)
+{
+    gather_index<float, 32, 64, 32, 64>(dst, src0, idx);
+}
+void ref_tgather_mask_f16_16x64_p0101(uint16_t *dst, const uint16_t *src)
+{
+    gather_mask<half, 16, 64, MaskPattern::P0101, 2>(reinterpret_cast<half *>(dst),
+                                                     reinterpret_cast<const half *>(src));
+}
+void ref_tgather_mask_f32_8x64_p1000(float *dst, const float *src)
+{
+    gather_mask<float, 8, 64, MaskPattern::P1000, 4>(dst, src);
+}
+void ref_tgather_mask_f32_8x64_p1111(float *dst, const float *src)
+{
+    gather_mask<float, 8, 64, MaskPattern::P1111, 1>(dst, src);
+}
+void ref_mgather_f16_8x128(uint16_t *dst, const uint16_t *gm, const int32_t *idx)
+{
+    mgather<half, 8, 128, 65536>(reinterpret_cast<half *>(dst), reinterpret_cast<const half *>(gm), idx);
+}
+
+void ref_textract_suffix_64x64_16_32(uint16_t *out, const uint16_t *in) { extract_suffix<64, 64, 16, 32>(out, in); }
+void ref_textract_suffix_128x256_0_192(uint16_t *out, const uint16_t *in) { extract_suffix<128, 256, 0, 192>(out, in); }
+
+// raw tile images (element order in tile storage)
+void ref_image_nz_f16_32x48(uint16_t *image, const uint16_t *gm)
+{
+    using T = Tile<TileType::Mat, half, 32, 48, BLayout::ColMajor, 32, 48, SLayout::RowMajor>;
+    load_image<T, GmND<half, 32, 48>>(reinterpret_cast<half *>(image), reinterpret_cast<half *>(const_cast<uint16_t *>(gm)));
+}
+void ref_image_zn_f16_48x32(uint16_t *image, const uint16_t *gm)
+{ // gm stored [32][48] (column-major 48 x 32)
+    using T = Tile<TileType::Mat, half, 48, 32, BLayout::RowMajor, 48, 32, SLayout::ColMajor>;
+    load_image<T, GmDN<half, 48, 32>>(reinterpret_cast<half *>(image), reinterpret_cast<half *>(const_cast<uint16_t *>(gm)));
+}
+void ref_image_nz_f32_32x16(float *image, const float *gm)
+{
+    using T = Tile<TileType::Mat, float, 32, 16, BLayout::ColMajor, 32, 16, SLayout::RowMajor>;
+    load_image<T, GmND<float, 32, 16>>(image, const_cast<float *>(gm));
+}
+void ref_image_pad_f32_16x32_valid_10x20(float *image, const float *gm)
+{ // PadValue::Max fills everything outside the 10 x 20 valid region with +inf
+    using T = Tile<TileType::Vec, float, 16, 32, BLayout::RowMajor, 10, 20, SLayout::NoneBox, 512, PadValue::Max>;
+    using G = GlobalTensor<float, Shape<1, 1, 1, 10, 20>, Stride<200, 200, 200, 20, 1>>;
+    load_image<T, G>(image, const_cast<float *>(gm));
+}
+void ref_image_5d_f32_2x3x4x8(float *image, const float *gm)
+{ // 5-D GM [1,2,3,4,8] with padded strides -> plain [24, 8] tile
+    using T = Tile<TileType::Vec, float, 24, 8, BLayout::RowMajor>;
+    using G = GlobalTensor<float, Shape<1, 2, 3, 4, 8>, Stride<1000, 400, 100, 10, 1>>;
+    load_image<T, G>(image, const_cast<float *>(gm));
+}
+
+void ref_fa_auto_64x32(float *out, const float *q, const float *k, const float *v) { fa_auto<64, 32>(out, q, k, v); }
+void ref_fa_auto_128x64(float *out, const float *q, const float *k, const float *v) { fa_auto<128, 64>(out, q, k, v); }
+
+} // extern "C"

@@ -1,0 +1,66 @@
+"""Writes tests/golden/ref_vectors.npz: outputs of the COMPILED REFERENCE (oracle/_ref, built from the
+reference's CPU-simulation headers) on seeded inputs.  Run in the build container, where the reference
+tree is mounted; the fixture lets the oracle be checked against the reference where the tree is absent.
+
+    python tests/golden/make_golden.py
+
+Inputs are regenerated from seeds by the tests (pto_amd.datagen / numpy default_rng), only the
+reference's outputs are stored.
+"""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path[:0] = [ROOT, os.path.join(ROOT, "pto-isa_amd")]
+
+from oracle import oracle  # noqa: E402
+from pto_amd import datagen  # noqa: E402
+
+
+def p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def cases(ref):
+    out = {}
+    a, b = datagen.gemm_inputs(128, 128, 512)
+    c = np.zeros((128, 128), dtype=np.float32)
+    ref.ref_gemm_128x512x128_ks64(p(c), p(a), p(b))
+    out["gemm_128x512x128_ks64"] = c
+    a, b = datagen.gemm_inputs(128, 256, 64)
+    c = np.zeros((128, 256), dtype=np.float32)
+    ref.ref_gemm_128x64x256_ks64(p(c), p(a), p(b))
+    out["gemm_128x64x256_ks64"] = c
+    x = datagen.tcvt_input(64, 256, inject=0.05).reshape(-1)
+    h = np.zeros(x.size, dtype=np.uint16)
+    ref.ref_tcvt_f32_f16(p(h), p(x), C.c_size_t(x.size))
+    out["tcvt_f32_f16_64x256"] = h
+    rng = np.random.default_rng(9)
+    src = rng.integers(0, 2**16, size=(16, 1024), dtype=np.uint16)
+    idx = rng.integers(-50, 16 * 1024 + 50, size=(16, 128), dtype=np.int32)
+    g = np.zeros((16, 128), dtype=np.uint16)
+    ref.ref_tgather_index_f16_16x1024_16x128(p(g), p(src), p(idx))
+    out["tgather_index_f16_16x1024_16x128"] = g
+    rng = np.random.default_rng(20251220)
+    q, k, v = (rng.standard_normal((64, 32), dtype=np.float32) for _ in range(3))
+    o = np.zeros((64, 32), dtype=np.float32)
+    ref.ref_fa_auto_64x32(p(o), p(q), p(k), p(v))
+    out["fa_auto_64x32"] = o
+    x = np.arange(128 * 256, dtype=np.uint16).reshape(128, 256)
+    e = np.zeros((128, 64), dtype=np.uint16)
+    ref.ref_textract_suffix_128x256_0_192(p(e), p(x))
+    out["textract_suffix_128x256_0_192"] = e
+    return out
+
+
+if __name__ == "__main__":
+    oracle.build(ref=True)
+    r = oracle.ref()
+    if r is None:
+        sys.exit("reference tree not present: cannot regenerate the fixture")
+    np.savez_compressed(os.path.join(HERE, "ref_vectors.npz"), **cases(r))
+    print("wrote", os.path.join(HERE, "ref_vectors.npz"))
