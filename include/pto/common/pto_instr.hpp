@@ -1,0 +1,160 @@
+// Front end of the PTO tile instructions: every instruction waits on the events passed after its
+// operands, runs its gfx950 implementation and returns a RecordEvent
+// (the calling convention of the reference's include/pto/common/pto_instr.hpp:20-1511).
+#pragma once
+#include "pto/common/event.hpp"
+#include "pto/gfx950/matmul.hpp"
+#include "pto/gfx950/mem_ops.hpp"
+#include "pto/gfx950/vec_ops.hpp"
+
+namespace pto {
+
+template <typename... Ev>
+PTO_INST void TSYNC(Ev &... ev)
+{
+    WaitAllEvents(ev...);
+}
+template <Op OpCode>
+PTO_INST void TSYNC()
+{
+    pipe_barrier(OpPipe(OpCode));
+}
+
+template <typename T, typename AddrType>
+PTO_INST void TASSIGN(T &obj, AddrType addr)
+{
+    TASSIGN_IMPL(obj, addr);
+}
+template <std::size_t Addr, typename T>
+PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T &obj)
+{
+    if constexpr (T::Loc == TileType::Mat) {
+        static_assert(Addr % 16 == 0, "[PTO][SA] TASSIGN: Mat tiles are 16-byte aligned in LDS");
+        static_assert(Addr + detail::MatGeom<T>::Bytes <= 160 * 1024, "[PTO][SA] TASSIGN: tile exceeds the 160 KiB LDS of a CU");
+    }
+    TASSIGN_IMPL(obj, Addr);
+}
+
+#define PTO_FRONT(NAME, TPARAMS, PARAMS, ARGS)          \
+    template <TPARAMS, typename... Ev>                  \
+    PTO_INST RecordEvent NAME(PARAMS, Ev &... ev)       \
+    {                                                   \
+        TSYNC(ev...);                                   \
+        NAME##_IMPL ARGS;                               \
+        return {};                                      \
+    }
+#define PTO_C ,
+
+PTO_FRONT(TLOAD, typename TileT PTO_C typename G, TileT &dst PTO_C G &src, (dst, src))
+PTO_FRONT(TEXTRACT, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C uint16_t idxRow PTO_C uint16_t idxCol,
+          (dst, src, idxRow, idxCol))
+PTO_FRONT(TMOV, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TMATMUL, typename C PTO_C typename A PTO_C typename B, C &c PTO_C A &a PTO_C B &b, (c, a, b))
+PTO_FRONT(TMATMUL_ACC, typename C PTO_C typename A PTO_C typename B, C &cOut PTO_C C &cIn PTO_C A &a PTO_C B &b,
+          (cOut, cIn, a, b))
+PTO_FRONT(TMATMUL_BIAS, typename C PTO_C typename A PTO_C typename B, C &c PTO_C A &a PTO_C B &b PTO_C BiasRow bias,
+          (c, a, b, bias))
+PTO_FRONT(TCVT, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C RoundMode mode, (dst, src, mode))
+PTO_FRONT(TGATHER, typename D PTO_C typename S0 PTO_C typename I, D &dst PTO_C S0 &src0 PTO_C I &idx, (dst, src0, idx))
+PTO_FRONT(MGATHER, typename D PTO_C typename G PTO_C typename I, D &dst PTO_C G &src PTO_C I &idx, (dst, src, idx))
+PTO_FRONT(MGATHER_ROWS, typename D PTO_C typename G PTO_C typename I, D &dst PTO_C G &table PTO_C I &rowIdx PTO_C int tableRows,
+          (dst, table, rowIdx, tableRows))
+PTO_FRONT(TADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TSUB, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TMUL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TDIV, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TMAX, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TMIN, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TMULS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TADDS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TSUBS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TDIVS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TMAXS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TMINS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TEXP, typename T, T &dst PTO_C T &src, (dst, src))
+PTO_FRONT(TEXPANDS, typename T, T &dst PTO_C typename T::DType k, (dst, k))
+PTO_FRONT(TRESHAPE, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TROWMAX, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
+PTO_FRONT(TROWSUM, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
+PTO_FRONT(TROWEXPANDSUB, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDMUL, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDDIV, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDADD, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDMAX, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDMIN, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+#undef PTO_FRONT
+#undef PTO_C
+
+// forms whose template arguments come first
+template <typename TileT, typename G, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TSTORE_IMPL<TileT, G, AtomicType::AtomicNone>(dst, src);
+    return {};
+}
+template <STPhase Phase, typename TileT, typename G, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
+{ // the unit-flag phase is an Ascend fix-pipe hint; a store is a store here
+    TSYNC(ev...);
+    TSTORE_IMPL<TileT, G, AtomicType::AtomicNone>(dst, src);
+    return {};
+}
+template <typename TileT, typename G, AtomicType atomic, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TSTORE_IMPL<TileT, G, atomic>(dst, src);
+    return {};
+}
+template <typename D, typename S, typename... Ev>
+PTO_INST RecordEvent TEXTRACT(D &dst, S &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TEXTRACT_IMPL(dst, src, 0, 0);
+    return {};
+}
+template <AccPhase Phase, typename C, typename A, typename B, typename... Ev>
+PTO_INST RecordEvent TMATMUL(C &c, A &a, B &b, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_IMPL(c, a, b);
+    return {};
+}
+template <AccPhase Phase, typename C, typename A, typename B, typename... Ev>
+PTO_INST RecordEvent TMATMUL_ACC(C &cOut, C &cIn, A &a, B &b, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_ACC_IMPL(cOut, cIn, a, b);
+    return {};
+}
+template <AccPhase Phase = AccPhase::Unspecified, typename C, typename A, typename B, typename... Ev>
+PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TMATMUL_ACC(C &c, A &a, B &b, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_ACC_IMPL(c, c, a, b);
+    return {};
+}
+template <typename D, typename S, typename... Ev>
+PTO_INST RecordEvent TCVT(D &dst, S &src, RoundMode mode, SaturationMode sat, Ev &... ev)
+{
+    TSYNC(ev...);
+    TCVT_IMPL(dst, src, mode, sat);
+    return {};
+}
+template <typename D, typename S, MaskPattern pattern, typename... Ev>
+PTO_INST RecordEvent TGATHER(D &dst, S &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TGATHER_IMPL<D, S, pattern>(dst, src);
+    return {};
+}
+template <typename TileT, int isUpperOrLower, typename... Ev>
+PTO_INST RecordEvent TTRI(TileT &dst, int diagonal, Ev &... ev)
+{
+    TSYNC(ev...);
+    TTRI_IMPL<TileT, isUpperOrLower>(dst, diagonal);
+    return {};
+}
+
+} // namespace pto

@@ -1,0 +1,202 @@
+// pto::Tile for gfx950: the reference's template signature and static members
+// (include/pto/common/pto_tile.hpp:1201-1410, aliases :1412-1463) over storage that is native to
+// CDNA4 instead of Ascend's L1/L0/UB buffers:
+//
+//   TileType::Mat    a handle (byte offset, set by TASSIGN) to an LDS-resident tile.  Physical layout:
+//                    the contraction dimension is contiguous (columns for an Nz tile, rows for a Zn
+//                    tile) and 16-byte chunks are XOR-swizzled so that the ds_read_b128 fragment
+//                    loads of TEXTRACT are bank-conflict free.  BLayout/SLayout only select which
+//                    logical dimension is the contiguous one.
+//   Left/Right       per-wave MFMA operand fragments in VGPRs: [32-row block][16-wide k step] x 8 halves.
+//   Acc              per-wave MFMA accumulator fragments (AGPRs): [row block][col block] x 16 floats.
+//   Vec              register tile spread over the workgroup in chunks of 8 consecutive elements of
+//                    the tile's linear (BLayout) order: chunk q -> thread q % kBlockThreads, slot q / kBlockThreads.
+//
+// Register tiles are values: pass them by reference.
+#pragma once
+#include "pto/common/types.hpp"
+#include "pto/gfx950/platform.hpp"
+
+namespace pto {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+namespace detail {
+
+constexpr int kMfmaM = 32; // v_mfma_f32_32x32x16: 32 x 32 output block
+constexpr int kMfmaK = 16; // k extent of one MFMA
+constexpr int kVecChunk = 8;
+
+template <typename T>
+struct FragOf {
+    using type = u32x4;
+};
+template <>
+struct FragOf<_Float16> {
+    using type = f16x8;
+};
+template <>
+struct FragOf<__bf16> {
+    using type = bf16x8;
+};
+
+constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
+
+struct Empty {};
+
+template <TileType Loc, typename T, int Rows, int Cols>
+struct TileStorage { // Bias / Scaling / unsupported locations: no storage
+    Empty none;
+};
+
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Mat, T, Rows, Cols> {
+    uint32_t lds = 0; // byte offset into the workgroup's dynamic LDS
+};
+
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Left, T, Rows, Cols> {
+    static_assert(sizeof(T) == 2, "Left tiles: fp16 / bf16 operands");
+    static_assert(Rows % (kMfmaM * kWavesM) == 0, "Left tile rows must be a multiple of 32 x PTO_WAVES_M");
+    static_assert(Cols % kMfmaK == 0, "Left tile cols (K) must be a multiple of 16");
+    static constexpr int MB = Rows / (kMfmaM * kWavesM);
+    static constexpr int KS = Cols / kMfmaK;
+    typename FragOf<T>::type f[MB][KS];
+};
+
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Right, T, Rows, Cols> {
+    static_assert(sizeof(T) == 2, "Right tiles: fp16 / bf16 operands");
+    static_assert(Cols % (kMfmaM * kWavesN) == 0, "Right tile cols must be a multiple of 32 x PTO_WAVES_N");
+    static_assert(Rows % kMfmaK == 0, "Right tile rows (K) must be a multiple of 16");
+    static constexpr int NB = Cols / (kMfmaM * kWavesN);
+    static constexpr int KS = Rows / kMfmaK;
+    typename FragOf<T>::type f[NB][KS];
+};
+
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Acc, T, Rows, Cols> {
+    static_assert(sizeof(T) == 4, "Acc tiles: fp32 accumulators");
+    static_assert(Rows % (kMfmaM * kWavesM) == 0 && Cols % (kMfmaM * kWavesN) == 0,
+                  "Acc tile must be a multiple of (32 x PTO_WAVES_M) x (32 x PTO_WAVES_N)");
+    static constexpr int MB = Rows / (kMfmaM * kWavesM);
+    static constexpr int NB = Cols / (kMfmaM * kWavesN);
+    f32x16 f[MB][NB];
+};
+
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Vec, T, Rows, Cols> {
+    static constexpr int Chunks = cdiv(Rows * Cols, kVecChunk);
+    static constexpr int Slots = cdiv(Chunks, kBlockThreads);
+    T v[Slots][kVecChunk];
+};
+
+} // namespace detail
+
+template <TileType Loc_, typename Element_, const int Rows_, const int Cols_, const BLayout BFractal_ = BLayout::RowMajor,
+          const int RowValid_ = Rows_, const int ColValid_ = Cols_, const SLayout SFractal_ = SLayout::NoneBox,
+          const int SFractalSize_ = TileConfig::fractalABSize, const PadValue PadVal_ = PadValue::Null,
+          const CompactMode Compact_ = CompactMode::Null>
+struct Tile {
+    using DType = Element_;
+    static constexpr TileType Loc = Loc_;
+    static constexpr int Rows = Rows_;
+    static constexpr int Cols = Cols_;
+    static constexpr int ValidRow = RowValid_;
+    static constexpr int ValidCol = ColValid_;
+    static constexpr BLayout BFractal = BFractal_;
+    static constexpr SLayout SFractal = SFractal_;
+    static constexpr int SFractalSize = SFractalSize_;
+    static constexpr PadValue PadVal = PadVal_;
+    static constexpr CompactMode Compact = Compact_;
+    static constexpr int Numel = Rows * Cols;
+    static constexpr bool isRowMajor = BFractal_ == BLayout::RowMajor;
+    static constexpr int RowStride = isRowMajor ? Cols : 1;
+    static constexpr int ColStride = isRowMajor ? 1 : Rows;
+    static constexpr bool isBoxedLayout = SFractal_ != SLayout::NoneBox;
+    static constexpr bool isInnerRowMajor = SFractal_ == SLayout::RowMajor;
+    static constexpr bool isInnerColMajor = SFractal_ == SLayout::ColMajor;
+    // box geometry of the reference layouts (16 x 32 B, 32 B x 16, or 16 x 16 for the 1 KiB accumulator box)
+    static constexpr int InnerRows =
+        SFractalSize_ == TileConfig::fractalCSize ?
+            TileConfig::fixedRowSize :
+            (isBoxedLayout ? (isInnerRowMajor ? TileConfig::fixedRowSize : TileConfig::alignedSize / (int)sizeof(DType)) : 1);
+    static constexpr int InnerCols =
+        SFractalSize_ == TileConfig::fractalCSize ?
+            TileConfig::fixedColSize :
+            (isBoxedLayout ? (isInnerRowMajor ? TileConfig::alignedSize / (int)sizeof(DType) : TileConfig::fixedColSize) : 1);
+    static constexpr int InnerNumel = InnerRows * InnerCols;
+
+    static_assert(Rows > 0 && Cols > 0 && ValidRow <= Rows && ValidCol <= Cols, "[PTO][SA] invalid tile extents");
+    static_assert(Loc_ == TileType::Vec || Rows_ == 1 || Rows % InnerRows == 0,
+                  "[PTO][SA] tile rows must be a multiple of the inner box rows");
+    static_assert(Cols % InnerCols == 0, "[PTO][SA] tile cols must be a multiple of the inner box cols");
+    static_assert(isBoxedLayout || (isRowMajor ? (Cols * sizeof(DType)) % TileConfig::alignedSize == 0 :
+                                                 (Rows * sizeof(DType)) % TileConfig::alignedSize == 0),
+                  "[PTO][SA] unboxed tiles need a 32-byte aligned contiguous extent");
+
+    // The logical dimension that is contiguous in a Mat tile's LDS image: columns unless the tile
+    // is a Zn (row-major boxes, column-major inside) or plain column-major tile.
+    static constexpr bool colsContiguous = isBoxedLayout ? isInnerRowMajor : isRowMajor;
+
+    using Storage = detail::TileStorage<Loc_, Element_, Rows_, Cols_>;
+    Storage st;
+    int RowMaskInternal = RowValid_;
+    int ColMaskInternal = ColValid_;
+
+    PTO_HD Tile() {}
+    template <int RM = ValidRow, int CM = ValidCol, std::enable_if_t<RM == DYNAMIC && CM == DYNAMIC, int> = 0>
+    PTO_HD Tile(size_t vr, size_t vc) : RowMaskInternal((int)vr), ColMaskInternal((int)vc)
+    {}
+    template <int RM = ValidRow, int CM = ValidCol, std::enable_if_t<(RM == DYNAMIC) != (CM == DYNAMIC), int> = 0>
+    PTO_HD Tile(size_t v)
+    {
+        if constexpr (RM == DYNAMIC)
+            RowMaskInternal = (int)v;
+        else
+            ColMaskInternal = (int)v;
+    }
+
+    PTO_HD constexpr int GetValidRow() const { return ValidRow == DYNAMIC ? RowMaskInternal : ValidRow; }
+    PTO_HD constexpr int GetValidCol() const { return ValidCol == DYNAMIC ? ColMaskInternal : ValidCol; }
+
+    // Mat tiles: pointer to the LDS image (swizzled, see mem_ops.hpp).  Register tiles: their fragments.
+    PTO_DEV auto data()
+    {
+        if constexpr (Loc_ == TileType::Mat)
+            return reinterpret_cast<DType *>(hw::lds_base() + st.lds);
+        else
+            return &st;
+    }
+};
+
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileLeft = Tile<TileType::Left, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor, TileConfig::fractalABSize>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileLeftCompact = Tile<TileType::Left, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor,
+                             TileConfig::fractalABSize, PadValue::Null, CompactMode::Normal>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileRight = Tile<TileType::Right, E, R, C, BLayout::RowMajor, RV, CV, SLayout::ColMajor, TileConfig::fractalABSize>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileRightCompact = Tile<TileType::Right, E, R, C, BLayout::RowMajor, RV, CV, SLayout::ColMajor,
+                              TileConfig::fractalABSize, PadValue::Null, CompactMode::Normal>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileAcc = Tile<TileType::Acc, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor, TileConfig::fractalCSize>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileAccCompact = Tile<TileType::Acc, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor,
+                            TileConfig::fractalCSize, PadValue::Null, CompactMode::Normal>;
+
+template <typename T>
+struct is_tile : std::false_type {};
+template <TileType L, typename E, int R, int C, BLayout B, int RV, int CV, SLayout S, int F, PadValue P, CompactMode M>
+struct is_tile<Tile<L, E, R, C, B, RV, CV, S, F, P, M>> : std::true_type {};
+template <typename T>
+constexpr bool is_tile_data_v = is_tile<std::remove_cv_t<std::remove_reference_t<T>>>::value;
+
+} // namespace pto

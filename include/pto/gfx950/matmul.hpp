@@ -1,0 +1,98 @@
+// TMATMUL / TMATMUL_ACC / TMATMUL_BIAS for gfx950: chains of v_mfma_f32_32x32x16_{f16,bf16}.
+//
+// Reference semantics (include/pto/cpu/TMatmul.hpp:73-116):
+//   C[i,j] = (acc ? acc[i,j] : 0) + sum_k (float)A[i,k] * (float)B[k,j],  M,K,N = a.validRow, a.validCol, b.validCol
+// Each wave owns the (Rows/PTO_WAVES_M) x (Cols/PTO_WAVES_N) sub-block of C selected by its
+// position in the wave grid and holds the matching rows of A / columns of B as fragments.
+// Products are exact in fp32; the order of the fp32 additions inside an MFMA differs from the
+// reference's sequential k loop, which is what the 2e-3 relative tolerance covers.
+#pragma once
+#include "pto/common/tile.hpp"
+
+namespace pto {
+namespace detail {
+
+PTO_DEV f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+PTO_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+
+template <typename AccT, typename LeftT, typename RightT>
+PTO_DEV constexpr void check_mad()
+{
+    using A = typename LeftT::DType;
+    using B = typename RightT::DType;
+    static_assert(std::is_same_v<A, B> && (std::is_same_v<A, half> || std::is_same_v<A, bfloat16_t>) &&
+                      std::is_same_v<typename AccT::DType, float>,
+                  "[PTO][SA] TMATMUL on gfx950: fp16 x fp16 -> fp32 or bf16 x bf16 -> fp32");
+    static_assert(LeftT::Loc == TileType::Left && RightT::Loc == TileType::Right && AccT::Loc == TileType::Acc,
+                  "[PTO][SA] TMATMUL: operands must be Left, Right and Acc tiles");
+    static_assert(LeftT::Rows == AccT::Rows && LeftT::Cols == RightT::Rows && RightT::Cols == AccT::Cols,
+                  "[PTO][SA] TMATMUL: inconsistent m, k, n");
+    static_assert(LeftT::ValidRow == LeftT::Rows && LeftT::ValidCol == LeftT::Cols && RightT::ValidCol == RightT::Cols,
+                  "[PTO][SA] TMATMUL on gfx950: operands must be fully valid (pad the tile instead)");
+}
+
+template <bool kZeroInit, typename AccT, typename LeftT, typename RightT>
+PTO_DEV void mad(AccT &out, const AccT &in, const LeftT &a, const RightT &b)
+{
+    using SA = typename AccT::Storage;
+    using SL = typename LeftT::Storage;
+#pragma unroll
+    for (int mb = 0; mb < SA::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < SA::NB; ++nb) {
+            f32x16 c;
+            if constexpr (kZeroInit) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    c[i] = 0.0f;
+            } else {
+                c = in.st.f[mb][nb];
+            }
+#pragma unroll
+            for (int ks = 0; ks < SL::KS; ++ks)
+                c = mfma32(a.st.f[mb][ks], b.st.f[nb][ks], c);
+            out.st.f[mb][nb] = c;
+        }
+}
+
+} // namespace detail
+
+template <typename AccT, typename LeftT, typename RightT>
+PTO_DEV void TMATMUL_IMPL(AccT &c, LeftT &a, RightT &b)
+{
+    detail::check_mad<AccT, LeftT, RightT>();
+    detail::mad<true>(c, c, a, b);
+}
+
+template <typename AccT, typename LeftT, typename RightT>
+PTO_DEV void TMATMUL_ACC_IMPL(AccT &cOut, AccT &cIn, LeftT &a, RightT &b)
+{
+    detail::check_mad<AccT, LeftT, RightT>();
+    detail::mad<false>(cOut, cIn, a, b);
+}
+
+// bias: a 1 x N fp32 row held as a Vec-distributed tile is not addressable per column from a
+// wave's accumulator lanes, so the bias row is read from memory: BiasT must expose `const float *row`.
+struct BiasRow {
+    const float *row;
+};
+
+template <typename AccT, typename LeftT, typename RightT>
+PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasRow bias)
+{
+    detail::check_mad<AccT, LeftT, RightT>();
+    detail::mad<true>(c, c, a, b);
+    using SA = typename AccT::Storage;
+    const int col0 = hw::wave_n() * (SA::NB * detail::kMfmaM) + (hw::lane() & 31);
+#pragma unroll
+    for (int nb = 0; nb < SA::NB; ++nb) {
+        const float bv = bias.row[col0 + nb * detail::kMfmaM]; // cpu/TMatmul.hpp:109-115: added after the product
+#pragma unroll
+        for (int mb = 0; mb < SA::MB; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                c.st.f[mb][nb][i] += bv;
+    }
+}
+
+} // namespace pto

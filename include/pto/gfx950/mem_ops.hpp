@@ -1,0 +1,415 @@
+// TASSIGN / TLOAD / TSTORE / TEXTRACT / TMOV for gfx950.
+//
+// Reference semantics: include/pto/cpu/TLoad.hpp:143-162, TStore.hpp:121-150, TExtract.hpp:17-50
+// (window form per docs/isa/TEXTRACT.md:14-18), TMov.hpp:20-51, TAssign.hpp:17-29.  A tile's
+// logical content tile(r,c) <-> gm[r*stride3 + c*stride4] is what is preserved; the physical
+// placement is the one described in common/tile.hpp.
+//
+// Mat tile LDS image.  Let `major` index the non-contiguous logical dimension and k the
+// contiguous one (k = column for an Nz tile, row for a Zn tile), RowBytes = extent_k * sizeof(T).
+// Element (major, k) lives at   major*RowBytes + ((chunk ^ swz(major)) << 4) + (k*sizeof(T) & 15),
+// chunk = k*sizeof(T) >> 4.  swz() is chosen so that 16 consecutive `major` values at the same
+// logical chunk fall into 16 different 16-byte bank groups: ds_read_b128 by a half-wave is
+// conflict free, and so is the 1 KiB-contiguous write pattern of global_load_lds_dwordx4.
+#pragma once
+#include "pto/common/global_tensor.hpp"
+#include "pto/common/tile.hpp"
+
+namespace pto {
+namespace detail {
+
+constexpr bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+
+template <int RowBytes>
+PTO_DEV constexpr uint32_t mat_swz(uint32_t major)
+{
+    constexpr int cpr = RowBytes / 16;
+    if constexpr (!is_pow2(cpr) || cpr < 2) {
+        return 0;
+    } else {
+        constexpr int div = cpr >= 16 ? 1 : 16 / cpr;
+        constexpr int mod = cpr >= 16 ? 16 : cpr;
+        return (major / div) % mod;
+    }
+}
+
+template <int RowBytes>
+PTO_DEV constexpr uint32_t mat_chunk_off(uint32_t major, uint32_t chunk)
+{
+    return major * RowBytes + ((chunk ^ mat_swz<RowBytes>(major)) << 4);
+}
+
+// geometry of a Mat tile's LDS image
+template <typename TileT>
+struct MatGeom {
+    using T = typename TileT::DType;
+    static constexpr bool colsK = TileT::colsContiguous;
+    static constexpr int Major = colsK ? TileT::Rows : TileT::Cols;
+    static constexpr int KExt = colsK ? TileT::Cols : TileT::Rows;
+    static constexpr int RowBytes = KExt * (int)sizeof(T);
+    static constexpr int ChunksPerRow = RowBytes / 16;
+    static constexpr int Bytes = Major * RowBytes;
+    static_assert(RowBytes % 16 == 0, "[PTO][SA] Mat tile: contiguous extent must be a multiple of 16 bytes");
+    // byte offset of logical element (r, c)
+    PTO_DEV static uint32_t elem_off(uint32_t r, uint32_t c)
+    {
+        const uint32_t major = colsK ? r : c, k = colsK ? c : r;
+        const uint32_t kb = k * sizeof(T);
+        return mat_chunk_off<RowBytes>(major, kb >> 4) + (kb & 15u);
+    }
+};
+
+#define PTO_GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define PTO_LDS_PTR(p) ((__attribute__((address_space(3))) void *)(p))
+
+// index of the outer (stacked) slab and the in-slab row for a 5-D GlobalTensor whose first four
+// dims are stacked along the tile's rows (TLoad.hpp:74-95)
+template <typename G>
+PTO_DEV int64_t gm_row_offset(const G &g, int64_t r)
+{
+    const int64_t s3 = g.GetShape(3), s2 = g.GetShape(2), s1 = g.GetShape(1);
+    const int64_t rr = r % s3;
+    int64_t slab = r / s3;
+    const int64_t k = slab % s2;
+    slab /= s2;
+    const int64_t j = slab % s1, i = slab / s1;
+    return i * g.GetStride(0) + j * g.GetStride(1) + k * g.GetStride(2) + rr * g.GetStride(3);
+}
+
+template <typename T>
+PTO_DEV T pad_value(PadValue p)
+{
+    if (p == PadValue::Max) {
+        if constexpr (std::is_integral_v<T>)
+            return (T)(~(T)0 ^ (std::is_signed_v<T> ? (T)((T)1 << (sizeof(T) * 8 - 1)) : (T)0));
+        else
+            return (T)__builtin_huge_valf();
+    }
+    if (p == PadValue::Min) {
+        if constexpr (std::is_integral_v<T>)
+            return std::is_signed_v<T> ? (T)((T)1 << (sizeof(T) * 8 - 1)) : (T)0;
+        else
+            return (T)(-__builtin_huge_valf());
+    }
+    return (T)0;
+}
+
+} // namespace detail
+
+// ------------------------------------------------------------------ TASSIGN
+// Mat tiles: `addr` is a byte offset into the workgroup's dynamic LDS (the L1 address space).
+// Register tiles have no address: the call is accepted and ignored, as in the CPU simulation
+// (cpu/TAssign.hpp:20-21).  GlobalTensor: rebinding the base pointer.
+template <typename T, typename AddrType>
+PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
+{
+    if constexpr (is_global_data_v<T>) {
+        obj.SetAddr(reinterpret_cast<typename T::DType *>(addr));
+    } else if constexpr (T::Loc == TileType::Mat) {
+        obj.st.lds = static_cast<uint32_t>((uintptr_t)addr);
+    } else {
+        (void)obj;
+        (void)addr;
+    }
+}
+
+// -------------------------------------------------------------------- TLOAD
+namespace detail {
+
+// GM -> LDS Mat tile.  Fast path: the tile's contiguous dimension is the unit-stride one in
+// memory, the valid region is the whole tile: 16-byte asynchronous global->LDS copies, 1 KiB of
+// LDS per wave instruction; the swizzle is applied on the global-address side.
+template <typename TileT, typename G>
+PTO_DEV void tload_mat(TileT &dst, G &src)
+{
+    using T = typename TileT::DType;
+    using Geo = MatGeom<TileT>;
+    char *lds = hw::lds_base() + dst.st.lds;
+    const T *gm = reinterpret_cast<const T *>(src.data());
+    const int64_t st_r = src.GetStride(3), st_c = src.GetStride(4);
+    constexpr bool fullValid = TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols;
+    constexpr bool staticUnit = Geo::colsK ? (G::staticStride[4] == 1) : (G::staticStride[3] == 1);
+    if constexpr (fullValid && staticUnit) {
+        const int64_t ld = Geo::colsK ? st_r : st_c;
+        constexpr int total = Geo::Major * Geo::ChunksPerRow; // 16-byte chunks
+        constexpr int perWaveInst = kWaveSize;
+        constexpr int nInst = cdiv(total, perWaveInst);
+        const int lane = hw::lane(), wave = hw::wave();
+#pragma unroll
+        for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
+            const int s = s0 + wave;
+            const uint32_t q = (uint32_t)(s * perWaveInst + lane);
+            constexpr bool evenInst = nInst % kBlockWaves == 0, evenTotal = total % perWaveInst == 0;
+            if ((evenInst || s < nInst) && (evenTotal || q < (uint32_t)total)) {
+                const uint32_t major = q / Geo::ChunksPerRow, cpos = q % Geo::ChunksPerRow;
+                const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major);
+                const T *g = gm + (int64_t)major * ld + chunk * (16 / sizeof(T));
+                __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + s * (perWaveInst * 16)), 16, 0, 0);
+            }
+        }
+    } else {
+        // general path: element by element, pad outside the valid region (TLoad.hpp:151-152)
+        const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+        const T pad = pad_value<T>(TileT::PadVal);
+        for (int e = hw::tid(); e < TileT::Numel; e += kBlockThreads) {
+            const int r = e / TileT::Cols, c = e % TileT::Cols;
+            T v = pad;
+            if (r < vr && c < vc)
+                v = gm[(int64_t)r * st_r + (int64_t)c * st_c];
+            *reinterpret_cast<T *>(lds + Geo::elem_off(r, c)) = v;
+        }
+    }
+}
+
+// GM -> Vec register tile.  Chunk q of 8 consecutive elements (in the tile's BLayout order).
+template <typename TileT, typename G>
+PTO_DEV void tload_vec(TileT &dst, G &src)
+{
+    using T = typename TileT::DType;
+    using S = typename TileT::Storage;
+    static_assert(TileT::SFractal == SLayout::NoneBox, "[PTO][SA] Vec tiles are unboxed on gfx950");
+    const T *gm = reinterpret_cast<const T *>(src.data());
+    constexpr int Minor = TileT::isRowMajor ? TileT::Cols : TileT::Rows; // contiguous extent of the tile
+    const int vMajor = TileT::isRowMajor ? dst.GetValidRow() : dst.GetValidCol();
+    const int vMinor = TileT::isRowMajor ? dst.GetValidCol() : dst.GetValidRow();
+    const int64_t stMinor = TileT::isRowMajor ? src.GetStride(4) : src.GetStride(3);
+    const bool stacked = src.GetShape(0) * src.GetShape(1) * src.GetShape(2) != 1;
+    const T pad = pad_value<T>(TileT::PadVal);
+    constexpr bool vecOK = Minor % kVecChunk == 0 && (kVecChunk * sizeof(T)) % 16 == 0 || Minor % kVecChunk == 0;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+        const int e0 = q * kVecChunk;
+        if (S::Chunks % kBlockThreads != 0 && q >= S::Chunks) {
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i)
+                dst.st.v[s][i] = pad;
+            continue;
+        }
+        const int major = e0 / Minor, minor0 = e0 % Minor;
+        int64_t base;
+        if (TileT::isRowMajor)
+            base = stacked ? gm_row_offset(src, major) : (int64_t)major * src.GetStride(3);
+        else
+            base = (int64_t)major * src.GetStride(4);
+        if (vecOK && stMinor == 1 && major < vMajor && minor0 + kVecChunk <= vMinor) {
+            // 8 contiguous elements: one or two 16-byte loads
+            using VT = T __attribute__((ext_vector_type(kVecChunk)));
+            VT v = *reinterpret_cast<const VT *>(gm + base + minor0);
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i)
+                dst.st.v[s][i] = v[i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i) {
+                const int e = e0 + i;
+                const int mj = e / Minor, mn = e % Minor;
+                T v = pad;
+                if (e < TileT::Numel && mj < vMajor && mn < vMinor) {
+                    int64_t b = TileT::isRowMajor ? (stacked ? gm_row_offset(src, mj) : (int64_t)mj * src.GetStride(3)) :
+                                                    (int64_t)mj * src.GetStride(4);
+                    v = gm[b + (int64_t)mn * stMinor];
+                }
+                dst.st.v[s][i] = v;
+            }
+        }
+    }
+}
+
+} // namespace detail
+
+template <typename TileT, typename G>
+PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
+{
+    static_assert(sizeof(typename TileT::DType) == sizeof(typename G::DType), "[PTO][SA] TLOAD: element sizes differ");
+    if constexpr (TileT::Loc == TileType::Mat)
+        detail::tload_mat(dst, src);
+    else if constexpr (TileT::Loc == TileType::Vec)
+        detail::tload_vec(dst, src);
+    else
+        static_assert(TileT::Loc == TileType::Mat, "[PTO][SA] TLOAD: destination must be a Mat or Vec tile");
+}
+
+// ----------------------------------------------------------------- TEXTRACT
+// dst[i,j] = src[idxRow+i, idxCol+j].  Mat -> Left / Right: one ds_read_b128 per 32-row block and
+// 16-wide k step, in the v_mfma_f32_32x32x16 operand layout (lane l: row/col l%32, k = 8*(l/32)..+7).
+// The k offset must be a multiple of 8 elements (16 bytes).
+template <typename DstT, typename SrcT>
+PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t idxCol = 0)
+{
+    static_assert(SrcT::Loc == TileType::Mat, "[PTO][SA] TEXTRACT: source must be a Mat tile");
+    static_assert(sizeof(typename DstT::DType) == sizeof(typename SrcT::DType), "[PTO][SA] TEXTRACT: dtype mismatch");
+    using Geo = detail::MatGeom<SrcT>;
+    using Frag = typename detail::FragOf<typename DstT::DType>::type;
+    const char *lds = hw::lds_base() + src.st.lds;
+    const uint32_t lane = (uint32_t)hw::lane();
+    const uint32_t l32 = lane & 31u, khalf = lane >> 5;
+    if constexpr (DstT::Loc == TileType::Left) {
+        static_assert(Geo::colsK, "[PTO][SA] TEXTRACT to Left: source must be contiguous along columns (Nz / row-major)");
+        using S = typename DstT::Storage;
+        const uint32_t row0 = idxRow + (uint32_t)hw::wave_m() * (S::MB * detail::kMfmaM) + l32;
+        const uint32_t chunk0 = (idxCol >> 3) + khalf;
+#pragma unroll
+        for (int mb = 0; mb < S::MB; ++mb)
+#pragma unroll
+            for (int ks = 0; ks < S::KS; ++ks)
+                dst.st.f[mb][ks] = *reinterpret_cast<const Frag *>(
+                    lds + detail::mat_chunk_off<Geo::RowBytes>(row0 + mb * detail::kMfmaM, chunk0 + ks * 2));
+    } else if constexpr (DstT::Loc == TileType::Right) {
+        static_assert(!Geo::colsK, "[PTO][SA] TEXTRACT to Right: source must be contiguous along rows (Zn / column-major)");
+        using S = typename DstT::Storage;
+        const uint32_t col0 = idxCol + (uint32_t)hw::wave_n() * (S::NB * detail::kMfmaM) + l32;
+        const uint32_t chunk0 = (idxRow >> 3) + khalf;
+#pragma unroll
+        for (int nb = 0; nb < S::NB; ++nb)
+#pragma unroll
+            for (int ks = 0; ks < S::KS; ++ks)
+                dst.st.f[nb][ks] = *reinterpret_cast<const Frag *>(
+                    lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * 2));
+    } else {
+        static_assert(DstT::Loc == TileType::Left, "[PTO][SA] TEXTRACT: destination must be a Left or Right tile");
+    }
+}
+
+// --------------------------------------------------------------------- TMOV
+// Same-shape move between locations.  Mat -> Left/Right is TEXTRACT at (0,0); register tiles of
+// the same location and shape copy their fragments.
+template <typename DstT, typename SrcT>
+PTO_DEV void TMOV_IMPL(DstT &dst, SrcT &src)
+{
+    if constexpr (SrcT::Loc == TileType::Mat && (DstT::Loc == TileType::Left || DstT::Loc == TileType::Right)) {
+        TEXTRACT_IMPL(dst, src, 0, 0);
+    } else if constexpr (SrcT::Loc == DstT::Loc && SrcT::Rows == DstT::Rows && SrcT::Cols == DstT::Cols &&
+                         std::is_same_v<typename SrcT::DType, typename DstT::DType> && SrcT::Loc != TileType::Mat) {
+        dst.st = src.st;
+    } else {
+        static_assert(SrcT::Loc == TileType::Mat && DstT::Loc == TileType::Left,
+                      "[PTO][SA] TMOV: this location pair is not available on gfx950");
+    }
+}
+
+// ------------------------------------------------------------------- TSTORE
+namespace detail {
+
+template <typename D, typename S>
+PTO_DEV D store_cast(S v)
+{
+    if constexpr (std::is_same_v<D, S>)
+        return v;
+    else
+        return static_cast<D>(v); // fp32 -> fp16 / bf16: hardware round-to-nearest-even
+}
+
+// Acc fragments -> GM.  v_mfma_f32_32x32x16 result layout: lane l, register v holds
+// row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32 x 32 block.
+template <typename TileT, typename G, AtomicType atomic>
+PTO_DEV void tstore_acc(G &dst, TileT &src)
+{
+    using S = typename TileT::Storage;
+    using GT = typename G::DType;
+    GT *gm = reinterpret_cast<GT *>(dst.data());
+    const int64_t st_r = dst.GetStride(3), st_c = dst.GetStride(4);
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    const uint32_t lane = (uint32_t)hw::lane();
+    const int rbase = hw::wave_m() * (S::MB * kMfmaM) + (int)(lane >> 5) * 4;
+    const int cbase = hw::wave_n() * (S::NB * kMfmaM) + (int)(lane & 31u);
+    constexpr bool full = TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols;
+#pragma unroll
+    for (int mb = 0; mb < S::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < S::NB; ++nb) {
+            const int c = cbase + nb * kMfmaM;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = rbase + mb * kMfmaM + (v >> 2) * 8 + (v & 3);
+                if (full || (r < vr && c < vc)) {
+                    GT *p = gm + (int64_t)r * st_r + (int64_t)c * st_c;
+                    if constexpr (atomic == AtomicType::AtomicAdd)
+                        atomicAdd(p, store_cast<GT>(src.st.f[mb][nb][v]));
+                    else
+                        *p = store_cast<GT>(src.st.f[mb][nb][v]);
+                }
+            }
+        }
+}
+
+template <typename TileT, typename G>
+PTO_DEV void tstore_vec(G &dst, TileT &src)
+{
+    using T = typename TileT::DType;
+    using S = typename TileT::Storage;
+    T *gm = reinterpret_cast<T *>(dst.data());
+    constexpr int Minor = TileT::isRowMajor ? TileT::Cols : TileT::Rows;
+    const int vMajor = TileT::isRowMajor ? src.GetValidRow() : src.GetValidCol();
+    const int vMinor = TileT::isRowMajor ? src.GetValidCol() : src.GetValidRow();
+    const int64_t stMinor = TileT::isRowMajor ? dst.GetStride(4) : dst.GetStride(3);
+    const bool stacked = dst.GetShape(0) * dst.GetShape(1) * dst.GetShape(2) != 1;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+        if (S::Chunks % kBlockThreads != 0 && q >= S::Chunks)
+            continue;
+        const int e0 = q * kVecChunk;
+        const int major = e0 / Minor, minor0 = e0 % Minor;
+        int64_t base;
+        if (TileT::isRowMajor)
+            base = stacked ? gm_row_offset(dst, major) : (int64_t)major * dst.GetStride(3);
+        else
+            base = (int64_t)major * dst.GetStride(4);
+        if (Minor % kVecChunk == 0 && stMinor == 1 && major < vMajor && minor0 + kVecChunk <= vMinor) {
+            using VT = T __attribute__((ext_vector_type(kVecChunk)));
+            VT v;
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i)
+                v[i] = src.st.v[s][i];
+            *reinterpret_cast<VT *>(gm + base + minor0) = v;
+        } else {
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i) {
+                const int e = e0 + i;
+                const int mj = e / Minor, mn = e % Minor;
+                if (e < TileT::Numel && mj < vMajor && mn < vMinor) {
+                    int64_t b = TileT::isRowMajor ? (stacked ? gm_row_offset(dst, mj) : (int64_t)mj * dst.GetStride(3)) :
+                                                    (int64_t)mj * dst.GetStride(4);
+                    gm[b + (int64_t)mn * stMinor] = src.st.v[s][i];
+                }
+            }
+        }
+    }
+}
+
+// LDS Mat tile -> GM, element by element (not on any hot path)
+template <typename TileT, typename G>
+PTO_DEV void tstore_mat(G &dst, TileT &src)
+{
+    using T = typename TileT::DType;
+    using Geo = MatGeom<TileT>;
+    const char *lds = hw::lds_base() + src.st.lds;
+    T *gm = reinterpret_cast<T *>(dst.data());
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    for (int e = hw::tid(); e < TileT::Numel; e += kBlockThreads) {
+        const int r = e / TileT::Cols, c = e % TileT::Cols;
+        if (r < vr && c < vc)
+            gm[(int64_t)r * dst.GetStride(3) + (int64_t)c * dst.GetStride(4)] =
+                *reinterpret_cast<const T *>(lds + Geo::elem_off(r, c));
+    }
+}
+
+} // namespace detail
+
+template <typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone>
+PTO_DEV void TSTORE_IMPL(G &dst, TileT &src)
+{
+    if constexpr (TileT::Loc == TileType::Acc) {
+        detail::tstore_acc<TileT, G, atomic>(dst, src);
+    } else if constexpr (TileT::Loc == TileType::Vec) {
+        static_assert(sizeof(typename TileT::DType) == sizeof(typename G::DType), "[PTO][SA] TSTORE: element sizes differ");
+        detail::tstore_vec(dst, src);
+    } else if constexpr (TileT::Loc == TileType::Mat) {
+        detail::tstore_mat(dst, src);
+    } else {
+        static_assert(TileT::Loc == TileType::Acc, "[PTO][SA] TSTORE: source must be an Acc, Vec or Mat tile");
+    }
+}
+
+} // namespace pto

@@ -1,0 +1,123 @@
+// gfx950 (MI355X / CDNA4) platform layer of the PTO tile API.
+//
+// Takes the place of the reference's platform shim (include/pto/common/cpu_stub.hpp:29-90 for the
+// CPU simulation, the CCE compiler builtins on Ascend): memory-space qualifiers, pipe and event
+// names, set_flag / wait_flag / pipe_barrier, block indices.
+//
+// Execution model.  One PTO "core" is one HIP workgroup of PTO_WAVES_M x PTO_WAVES_N wavefronts
+// (64 lanes each).  A tile instruction is executed cooperatively by the whole workgroup:
+//   Mat tiles           live in LDS (the role of L1),
+//   Left / Right / Acc  are per-wave MFMA operand / accumulator fragments in VGPRs / AGPRs (L0A/L0B/L0C),
+//   Vec tiles           are distributed over the workgroup's lanes in VGPRs (UB).
+// Ascend pipes become the hardware counters of one instruction stream:
+//   MTE2 (GM->L1)  = asynchronous global->LDS loads, tracked by vmcnt
+//   MTE1 (L1->L0)  = ds_read, tracked by lgkmcnt (the compiler inserts those waits)
+//   M, V, FIX      = MFMA / VALU / global stores on registers: ordered by data dependences
+// so a wait_flag only has to do something where LDS contents cross wavefronts.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+
+#define PTO_HD __host__ __device__ __forceinline__
+#define PTO_DEV __device__ __forceinline__
+#define PTO_INST PTO_DEV
+#define PTO_INTERNAL PTO_DEV
+
+// Qualifiers of the Ascend dialect that kernel sources carry; all memory is reached through
+// generic pointers here.
+#define AICORE
+#define __aicore__
+#define __gm__
+#define __ubuf__
+#define __cbuf__
+#define __ca__
+#define __cb__
+#define __cc__
+#define __fbuf__
+#define __in__
+#define __out__
+#define __tf__
+
+#ifndef PTO_WAVES_M
+#define PTO_WAVES_M 2
+#endif
+#ifndef PTO_WAVES_N
+#define PTO_WAVES_N 2
+#endif
+
+namespace pto {
+constexpr int kWaveSize = 64;
+constexpr int kWavesM = PTO_WAVES_M;
+constexpr int kWavesN = PTO_WAVES_N;
+constexpr int kBlockWaves = kWavesM * kWavesN;
+constexpr int kBlockThreads = kBlockWaves * kWaveSize;
+
+namespace hw {
+PTO_DEV int lane() { return static_cast<int>(threadIdx.x) & (kWaveSize - 1); }
+// wave index as a scalar (SGPR) value
+PTO_DEV int wave() { return __builtin_amdgcn_readfirstlane(static_cast<int>(threadIdx.x) >> 6); }
+PTO_DEV int wave_m() { return wave() / kWavesN; }
+PTO_DEV int wave_n() { return wave() % kWavesN; }
+PTO_DEV int tid() { return static_cast<int>(threadIdx.x); }
+
+// Base of the workgroup's dynamic LDS allocation: address 0 of the "L1" space that TASSIGN names.
+PTO_DEV char *lds_base()
+{
+    extern __shared__ __attribute__((aligned(16))) char pto_dynamic_lds[];
+    return pto_dynamic_lds;
+}
+
+PTO_DEV void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+PTO_DEV void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+// Workgroup barrier that orders LDS traffic only; outstanding global loads keep flying.
+PTO_DEV void lds_barrier()
+{
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+} // namespace hw
+} // namespace pto
+
+// ---- pipes and events (global names, as kernel sources use them unqualified) ----
+enum pipe_t : int { PIPE_S = 0, PIPE_V, PIPE_M, PIPE_MTE1, PIPE_MTE2, PIPE_MTE3, PIPE_ALL, PIPE_FIX };
+enum event_t : int { EVENT_ID0 = 0, EVENT_ID1, EVENT_ID2, EVENT_ID3, EVENT_ID4, EVENT_ID5, EVENT_ID6, EVENT_ID7 };
+constexpr int EVENT_ID_MAX = 8;
+
+// set_flag records "everything issued so far on `src`"; in one instruction stream that is implicit.
+PTO_DEV void set_flag(pipe_t, pipe_t, event_t) {}
+
+// wait_flag(src, dst): later `dst` work may start once earlier `src` work is complete.
+PTO_DEV void wait_flag(pipe_t src, pipe_t dst, event_t)
+{
+    if (src == PIPE_MTE2) {
+        // global->LDS copies of every wave must have landed before anyone reads the tile
+        pto::hw::wait_vm0();
+        pto::hw::lds_barrier();
+    } else if (dst == PIPE_MTE2 && (src == PIPE_MTE1 || src == PIPE_V || src == PIPE_MTE3)) {
+        // every wave must be done reading an LDS tile before a load overwrites it
+        pto::hw::lds_barrier();
+    } else if (src == PIPE_MTE3 && dst != PIPE_S) {
+        pto::hw::wait_vm0();
+    }
+    // MTE1->M, M->MTE1, M->FIX, FIX->M, V<->M ...: register dependences, nothing to do
+}
+
+PTO_DEV void pipe_barrier(pipe_t p)
+{
+    if (p == PIPE_ALL) {
+        pto::hw::wait_vm0();
+        pto::hw::lds_barrier();
+    } else if (p == PIPE_MTE2 || p == PIPE_MTE3) {
+        pto::hw::wait_vm0();
+    }
+}
+
+PTO_DEV int64_t get_block_idx() { return static_cast<int64_t>(blockIdx.x); }
+PTO_DEV int64_t get_block_num() { return static_cast<int64_t>(gridDim.x); }
+PTO_DEV int64_t get_subblockid() { return 0; }
+PTO_DEV int64_t get_subblockdim() { return 1; }
+PTO_DEV int64_t get_coreid() { return static_cast<int64_t>(blockIdx.x); }
+PTO_DEV int64_t get_sys_cnt() { return static_cast<int64_t>(wall_clock64()); }

@@ -1,0 +1,521 @@
+// Vec-tile instructions for gfx950: TCVT, TGATHER (index and mask forms), MGATHER, elementwise
+// and row-broadcast arithmetic, row reductions, TTRI, TRESHAPE.
+//
+// A Vec tile is spread over the workgroup's lanes in chunks of 8 consecutive elements of its
+// linear order (common/tile.hpp), so every elementwise instruction between tiles of equal shape
+// is lane-local VALU work.  Instructions that move data across lanes (row reductions, row
+// broadcasts, gathers) stage through a small statically allocated LDS buffer sized by the tile.
+//
+// Reference semantics: include/pto/cpu/TCvt.hpp:65-92, TGather.hpp:58-129, MGatherScatter.hpp:21-44,
+// TRowMax.hpp:20-59, TRowSum.hpp:17-63, TRowExpandOp.hpp:37-96, TExp.hpp:22-60, TBinSOps.hpp,
+// TAdd/TSub/TMul/TMax.hpp, TTRI.hpp:31-76, TReshape.hpp.
+#pragma once
+#include "pto/common/global_tensor.hpp"
+#include "pto/common/tile.hpp"
+
+namespace pto {
+namespace detail {
+
+// ---- conversions -----------------------------------------------------------------------
+// fp32 -> fp16, round-to-nearest-even: v_cvt_f16_f32 under the default rounding mode.  NaNs are
+// canonicalised in software to sign | 0x7e00 | top 9 payload bits, the result of
+// static_cast<_Float16>(float) on the host, so that the conversion is bit-exact everywhere.
+PTO_DEV uint16_t f32_to_f16_bits_rne(float x)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const _Float16 h = static_cast<_Float16>(x);
+    uint16_t hb = __builtin_bit_cast(uint16_t, h);
+    if ((u & 0x7fffffffu) > 0x7f800000u)
+        hb = (uint16_t)(((u >> 16) & 0x8000u) | 0x7e00u | ((u >> 13) & 0x1ffu));
+    return hb;
+}
+
+// fp32 -> fp16 with an explicit rounding rule, in integer arithmetic (RoundMode values 2..6).
+PTO_DEV uint16_t f32_to_f16_bits_mode(float x, RoundMode mode)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const uint32_t sign = (u >> 16) & 0x8000u, a = u & 0x7fffffffu;
+    if (a > 0x7f800000u)
+        return (uint16_t)(sign | 0x7e00u | ((a >> 13) & 0x1ffu));
+    if (a == 0x7f800000u)
+        return (uint16_t)(sign | 0x7c00u);
+    const uint32_t e = a >> 23;
+    uint32_t h, rem, half_ulp;
+    if (e >= 143u) { // beyond the largest finite half
+        const bool toInf = mode == RoundMode::CAST_ROUND || mode == RoundMode::CAST_RINT ||
+                           (mode == RoundMode::CAST_CEIL && !sign) || (mode == RoundMode::CAST_FLOOR && sign);
+        return (uint16_t)(sign | (toInf ? 0x7c00u : 0x7bffu));
+    }
+    if (e >= 113u) {
+        const uint32_t v = a - (112u << 23);
+        h = v >> 13;
+        rem = v & 0x1fffu;
+        half_ulp = 0x1000u;
+    } else if (e >= 102u) {
+        const uint32_t m = (a & 0x7fffffu) | 0x800000u, shift = 126u - e;
+        h = m >> shift;
+        rem = m & ((1u << shift) - 1u);
+        half_ulp = 1u << (shift - 1u);
+    } else {
+        h = 0;
+        rem = a ? 1u : 0u; // something below half an ulp of the smallest subnormal
+        half_ulp = 2u;
+    }
+    bool up = false;
+    switch (mode) {
+    case RoundMode::CAST_ROUND: up = rem >= half_ulp; break;
+    case RoundMode::CAST_FLOOR: up = sign && rem; break;
+    case RoundMode::CAST_CEIL: up = !sign && rem; break;
+    case RoundMode::CAST_TRUNC: up = false; break;
+    case RoundMode::CAST_ODD: return (uint16_t)(sign | (h | (rem ? 1u : 0u)));
+    default: up = rem > half_ulp || (rem == half_ulp && (h & 1u)); break;
+    }
+    h += up ? 1u : 0u;
+    if (h > 0x7c00u)
+        h = 0x7c00u;
+    return (uint16_t)(sign | h);
+}
+
+// fp32 -> bf16 round-to-nearest-even, integer closed form; NaN -> quiet NaN keeping the top payload bits.
+PTO_DEV uint16_t f32_to_bf16_bits_rne(float x)
+{
+    const uint32_t u = __builtin_bit_cast(uint32_t, x);
+    const uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+    return (uint16_t)(((u & 0x7fffffffu) > 0x7f800000u) ? ((u >> 16) | 0x0040u) : r);
+}
+
+PTO_DEV float round_integral(float v, RoundMode mode)
+{ // cpu/TCvt.hpp:28-63
+    switch (mode) {
+    case RoundMode::CAST_RINT: return __builtin_rintf(v);
+    case RoundMode::CAST_ROUND: return __builtin_roundf(v);
+    case RoundMode::CAST_FLOOR: return __builtin_floorf(v);
+    case RoundMode::CAST_CEIL: return __builtin_ceilf(v);
+    case RoundMode::CAST_TRUNC: return __builtin_truncf(v);
+    case RoundMode::CAST_ODD: {
+        const float f = __builtin_floorf(v), frac = v - f;
+        if (frac > 0.5f)
+            return f + 1.0f;
+        if (frac < 0.5f)
+            return f;
+        return (((long long)f) & 1) ? f : f + 1.0f;
+    }
+    default: return v;
+    }
+}
+
+template <typename D, typename S>
+PTO_DEV D convert(S v, RoundMode mode)
+{
+    if constexpr (std::is_same_v<S, float> && std::is_same_v<D, half>) {
+        const uint16_t b = mode == RoundMode::CAST_RINT || mode == RoundMode::CAST_NONE ? f32_to_f16_bits_rne(v) :
+                                                                                            f32_to_f16_bits_mode(v, mode);
+        return __builtin_bit_cast(half, b);
+    } else if constexpr (std::is_same_v<S, float> && std::is_same_v<D, bfloat16_t>) {
+        return __builtin_bit_cast(bfloat16_t, f32_to_bf16_bits_rne(v));
+    } else if constexpr ((std::is_same_v<S, float> || std::is_same_v<S, half>)&&std::is_integral_v<D>) {
+        return static_cast<D>(round_integral(static_cast<float>(v), mode));
+    } else {
+        return static_cast<D>(v);
+    }
+}
+
+// linear element index -> (row, col) of a tile
+template <typename TileT>
+PTO_DEV void elem_rc(int e, int &r, int &c)
+{
+    if constexpr (TileT::isRowMajor) {
+        r = e / TileT::Cols;
+        c = e % TileT::Cols;
+    } else {
+        c = e / TileT::Rows;
+        r = e % TileT::Rows;
+    }
+}
+template <typename TileT>
+PTO_DEV int elem_index(int r, int c)
+{
+    return TileT::isRowMajor ? r * TileT::Cols + c : c * TileT::Rows + r;
+}
+
+// visit every element this lane owns: fn(slot, i, linear element index)
+template <typename TileT, typename F>
+PTO_DEV void for_each_owned(F &&fn)
+{
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+#pragma unroll
+        for (int i = 0; i < kVecChunk; ++i)
+            fn(s, i, q * kVecChunk + i);
+    }
+}
+
+template <typename A, typename B>
+constexpr bool same_dist = A::Numel == B::Numel && A::Loc == TileType::Vec && B::Loc == TileType::Vec;
+
+// one value per row (a [R,1] / [1,R] / first-column tile) -> LDS array of R floats, visible to all lanes
+template <typename RowT, int R>
+PTO_DEV void stage_row_values(RowT &t, typename RowT::DType *lds)
+{
+    for_each_owned<RowT>([&](int s, int i, int e) {
+        if (e < RowT::Numel) {
+            int r, c;
+            elem_rc<RowT>(e, r, c);
+            // the per-row scalar is element (r,0) of a column tile or (0,r) of a row tile (TRowExpandOp.hpp:20-33)
+            if (RowT::Cols == 1 || (RowT::Rows != 1 && c == 0)) {
+                if (c == 0 && r < R)
+                    lds[r] = t.st.v[s][i];
+            } else if (RowT::Rows == 1 && c < R) {
+                lds[c] = t.st.v[s][i];
+            }
+        }
+    });
+}
+
+} // namespace detail
+
+// --------------------------------------------------------------------- TCVT
+template <typename DstT, typename SrcT>
+PTO_DEV void TCVT_IMPL(DstT &dst, SrcT &src, RoundMode mode)
+{
+    static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] TCVT: Vec tiles with the same number of elements");
+    using S = typename SrcT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = detail::convert<typename DstT::DType>(src.st.v[s][i], mode);
+}
+template <typename DstT, typename SrcT>
+PTO_DEV void TCVT_IMPL(DstT &dst, SrcT &src, RoundMode mode, SaturationMode)
+{
+    TCVT_IMPL(dst, src, mode);
+}
+
+// ------------------------------------------------------------- elementwise
+#define PTO_DEFINE_BINARY(NAME, EXPR)                                                                   \
+    template <typename DstT, typename S0T, typename S1T>                                                \
+    PTO_DEV void NAME##_IMPL(DstT &dst, S0T &src0, S1T &src1)                                           \
+    {                                                                                                   \
+        static_assert(detail::same_dist<DstT, S0T> && detail::same_dist<DstT, S1T>,                     \
+                      "[PTO][SA] " #NAME ": Vec tiles with the same number of elements");              \
+        using T = typename DstT::DType;                                                                 \
+        using S = typename DstT::Storage;                                                               \
+        _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
+        {                                                                                               \
+            const T a = src0.st.v[s][i], b = src1.st.v[s][i];                                           \
+            dst.st.v[s][i] = (EXPR);                                                                    \
+        }                                                                                               \
+    }
+PTO_DEFINE_BINARY(TADD, a + b)
+PTO_DEFINE_BINARY(TSUB, a - b)
+PTO_DEFINE_BINARY(TMUL, a *b)
+PTO_DEFINE_BINARY(TDIV, a / b)
+PTO_DEFINE_BINARY(TMAX, (a < b ? b : a))
+PTO_DEFINE_BINARY(TMIN, (b < a ? b : a))
+#undef PTO_DEFINE_BINARY
+
+#define PTO_DEFINE_SCALAR(NAME, EXPR)                                                                   \
+    template <typename DstT, typename SrcT>                                                             \
+    PTO_DEV void NAME##_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)                              \
+    {                                                                                                   \
+        static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] " #NAME ": Vec tiles of equal size"); \
+        using T = typename DstT::DType;                                                                 \
+        using S = typename DstT::Storage;                                                               \
+        _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
+        {                                                                                               \
+            const T a = src.st.v[s][i];                                                                 \
+            dst.st.v[s][i] = (EXPR);                                                                    \
+        }                                                                                               \
+    }
+PTO_DEFINE_SCALAR(TMULS, a *k)
+PTO_DEFINE_SCALAR(TADDS, a + k)
+PTO_DEFINE_SCALAR(TSUBS, a - k)
+PTO_DEFINE_SCALAR(TDIVS, a / k)
+PTO_DEFINE_SCALAR(TMAXS, (a < k ? k : a))
+PTO_DEFINE_SCALAR(TMINS, (k < a ? k : a))
+#undef PTO_DEFINE_SCALAR
+
+template <typename TileT>
+PTO_DEV void TEXP_IMPL(TileT &dst, TileT &src)
+{
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = (typename TileT::DType)expf((float)src.st.v[s][i]);
+}
+
+template <typename TileT>
+PTO_DEV void TEXPANDS_IMPL(TileT &dst, typename TileT::DType k)
+{
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = k;
+}
+
+// same storage, new logical shape: both tiles have the same element count and so the same
+// lane distribution of their linear order
+template <typename DstT, typename SrcT>
+PTO_DEV void TRESHAPE_IMPL(DstT &dst, SrcT &src)
+{
+    static_assert(detail::same_dist<DstT, SrcT> && sizeof(typename DstT::DType) == sizeof(typename SrcT::DType) &&
+                      DstT::isRowMajor == SrcT::isRowMajor,
+                  "[PTO][SA] TRESHAPE: same element count, element size and major order");
+    using S = typename SrcT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = __builtin_bit_cast(typename DstT::DType, src.st.v[s][i]);
+}
+
+// upper (1) / lower (0) triangular 0/1 mask: TTRI.hpp:31-63
+template <typename TileT, int isUpperOrLower>
+PTO_DEV void TTRI_IMPL(TileT &dst, int diagonal)
+{
+    static_assert(TileT::isRowMajor, "[PTO][SA] TTRI: row-major tiles");
+    using T = typename TileT::DType;
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<TileT>([&](int s, int i, int e) {
+        const int r = e / TileT::Cols, c = e % TileT::Cols;
+        if (r < vr && c < vc) {
+            const bool one = isUpperOrLower ? (c >= diagonal + r) : (c < diagonal + r + 1);
+            dst.st.v[s][i] = one ? (T)1 : (T)0;
+        }
+    });
+}
+
+// --------------------------------------------------------- row reductions
+namespace detail {
+template <bool kMax, typename DstT, typename SrcT>
+PTO_DEV void row_reduce(DstT &dst, SrcT &src)
+{
+    static_assert(SrcT::isRowMajor && SrcT::Loc == TileType::Vec && DstT::Loc == TileType::Vec,
+                  "[PTO][SA] row reduction: row-major Vec source");
+    static_assert(SrcT::Cols % kVecChunk == 0, "[PTO][SA] row reduction: cols must be a multiple of 8");
+    static_assert(SrcT::Rows == DstT::Rows, "[PTO][SA] row reduction: row counts differ");
+    using A = float;
+    using S = typename SrcT::Storage;
+    constexpr int CPR = SrcT::Cols / kVecChunk; // chunks per row
+    __shared__ A part[S::Chunks];
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+        if (q < S::Chunks) {
+            const int c0 = (q % CPR) * kVecChunk;
+            A acc = kMax ? -__builtin_huge_valf() : 0.0f;
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i)
+                if (c0 + i < vc) {
+                    const A v = (A)src.st.v[s][i];
+                    acc = kMax ? (acc < v ? v : acc) : acc + v;
+                }
+            part[q] = acc;
+        }
+    }
+    hw::lds_barrier();
+    for_each_owned<DstT>([&](int s, int i, int e) {
+        if (e < DstT::Numel) {
+            int r, c;
+            elem_rc<DstT>(e, r, c);
+            if (c == 0 && r < vr) {
+                A acc = part[r * CPR];
+                for (int j = 1; j < CPR; ++j) {
+                    const A v = part[r * CPR + j];
+                    acc = kMax ? (acc < v ? v : acc) : acc + v;
+                }
+                dst.st.v[s][i] = (typename DstT::DType)acc;
+            }
+        }
+    });
+    hw::lds_barrier();
+}
+
+enum class RowOp { Sub, Mul, Div, Add, Max, Min };
+
+template <RowOp op, typename DstT, typename RowT>
+PTO_DEV void row_expand(DstT &dst, DstT &src0, RowT &src1)
+{
+    static_assert(DstT::isRowMajor, "[PTO][SA] row broadcast: row-major Vec tile");
+    using T = typename DstT::DType;
+    __shared__ typename RowT::DType rowv[DstT::Rows];
+    stage_row_values<RowT, DstT::Rows>(src1, rowv);
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && r < vr && c < vc) {
+            const T a = src0.st.v[s][i], b = (T)rowv[r];
+            T o;
+            if constexpr (op == RowOp::Sub)
+                o = a - b;
+            else if constexpr (op == RowOp::Mul)
+                o = a * b;
+            else if constexpr (op == RowOp::Div)
+                o = a / b;
+            else if constexpr (op == RowOp::Add)
+                o = a + b;
+            else if constexpr (op == RowOp::Max)
+                o = a < b ? b : a;
+            else
+                o = b < a ? b : a;
+            dst.st.v[s][i] = o;
+        }
+    });
+    hw::lds_barrier();
+}
+} // namespace detail
+
+template <typename DstT, typename SrcT, typename TmpT>
+PTO_DEV void TROWMAX_IMPL(DstT &dst, SrcT &src, TmpT &)
+{
+    detail::row_reduce<true>(dst, src);
+}
+template <typename DstT, typename SrcT, typename TmpT>
+PTO_DEV void TROWSUM_IMPL(DstT &dst, SrcT &src, TmpT &)
+{
+    detail::row_reduce<false>(dst, src);
+}
+#define PTO_DEFINE_ROWEXPAND(NAME, OP)                                \
+    template <typename DstT, typename RowT>                           \
+    PTO_DEV void NAME##_IMPL(DstT &dst, DstT &src0, RowT &src1)       \
+    {                                                                 \
+        detail::row_expand<detail::RowOp::OP>(dst, src0, src1);       \
+    }
+PTO_DEFINE_ROWEXPAND(TROWEXPANDSUB, Sub)
+PTO_DEFINE_ROWEXPAND(TROWEXPANDMUL, Mul)
+PTO_DEFINE_ROWEXPAND(TROWEXPANDDIV, Div)
+PTO_DEFINE_ROWEXPAND(TROWEXPANDADD, Add)
+PTO_DEFINE_ROWEXPAND(TROWEXPANDMAX, Max)
+PTO_DEFINE_ROWEXPAND(TROWEXPANDMIN, Min)
+#undef PTO_DEFINE_ROWEXPAND
+
+// ------------------------------------------------------------------ TGATHER
+// index form: dst[r,c] = src0.flat[idx[r,c]]; out-of-range or negative indices give 0
+// (cpu/TGather.hpp:68-89).  src0 is staged in LDS, then every lane reads its own elements.
+template <typename DstT, typename Src0T, typename IdxT>
+PTO_DEV void TGATHER_IMPL(DstT &dst, Src0T &src0, IdxT &idx)
+{
+    using T = typename DstT::DType;
+    static_assert(sizeof(T) == 2 || sizeof(T) == 4, "[PTO][SA] TGATHER: 16- or 32-bit elements");
+    static_assert(sizeof(typename IdxT::DType) == 4, "[PTO][SA] TGATHER: 32-bit indices");
+    static_assert(std::is_same_v<T, typename Src0T::DType>, "[PTO][SA] TGATHER: dst and src0 types differ");
+    static_assert(DstT::Numel == IdxT::Numel && DstT::isRowMajor == IdxT::isRowMajor,
+                  "[PTO][SA] TGATHER: dst and index tiles must have the same shape");
+    static_assert(Src0T::Numel * sizeof(T) <= 64 * 1024, "[PTO][SA] TGATHER: source tile must fit 64 KiB of LDS");
+    __shared__ T stage[Src0T::Numel]; // in (row, col) row-major order
+    detail::for_each_owned<Src0T>([&](int s, int i, int e) {
+        if (e < Src0T::Numel) {
+            int r, c;
+            detail::elem_rc<Src0T>(e, r, c);
+            stage[r * Src0T::Cols + c] = src0.st.v[s][i];
+        }
+    });
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        int r, c;
+        detail::elem_rc<DstT>(e, r, c);
+        if (e < DstT::Numel && r < vr && c < vc) {
+            const int32_t raw = (int32_t)idx.st.v[s][i];
+            const bool ok = raw >= 0 && raw < Src0T::Numel;
+            dst.st.v[s][i] = ok ? stage[raw] : (T)0;
+        }
+    });
+    hw::lds_barrier();
+}
+
+// mask form: the selected columns of every valid row, packed in row-major running order
+// (cpu/TGather.hpp:102-129).  Staged through LDS because the packed position differs from the source's.
+template <typename DstT, typename SrcT, MaskPattern pattern>
+PTO_DEV void TGATHER_IMPL(DstT &dst, SrcT &src)
+{
+    using T = typename SrcT::DType;
+    static_assert(DstT::isRowMajor && SrcT::isRowMajor, "[PTO][SA] TGATHER(mask): row-major tiles");
+    static_assert(sizeof(typename DstT::DType) == sizeof(T), "[PTO][SA] TGATHER(mask): element sizes differ");
+    constexpr int p = (int)pattern;
+    constexpr int div = p == 7 ? 1 : (p <= 2 ? 2 : 4);
+    constexpr int phase = p == 7 ? 0 : (p <= 2 ? p - 1 : p - 3);
+    __shared__ T stage[DstT::Numel];
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    const int perRow = (vc - phase + div - 1) / div; // selected columns per row
+    detail::for_each_owned<SrcT>([&](int s, int i, int e) {
+        const int r = e / SrcT::Cols, c = e % SrcT::Cols;
+        if (e < SrcT::Numel && r < vr && c < vc && (c % div) == phase) {
+            const int pos = r * perRow + c / div;
+            if (pos < DstT::Numel)
+                stage[pos] = src.st.v[s][i];
+        }
+    });
+    hw::lds_barrier();
+    const int total = vr * perRow;
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        if (e < DstT::Numel && e < total)
+            dst.st.v[s][i] = __builtin_bit_cast(typename DstT::DType, stage[e]);
+    });
+    hw::lds_barrier();
+}
+
+// ------------------------------------------------------------------ MGATHER
+// dst[i,j] = gm[idx[i,j]] (cpu/MGatherScatter.hpp:21-44): one global load per element.
+template <typename DstT, typename G, typename IdxT>
+PTO_DEV void MGATHER_IMPL(DstT &dst, G &src, IdxT &idx)
+{
+    static_assert(sizeof(typename DstT::DType) == sizeof(typename G::DType), "[PTO][SA] MGATHER: element sizes differ");
+    static_assert(DstT::Numel == IdxT::Numel && DstT::isRowMajor == IdxT::isRowMajor,
+                  "[PTO][SA] MGATHER: dst and index tiles must have the same shape");
+    using T = typename DstT::DType;
+    const T *gm = reinterpret_cast<const T *>(src.data());
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        int r, c;
+        detail::elem_rc<DstT>(e, r, c);
+        if (e < DstT::Numel && r < vr && c < vc)
+            dst.st.v[s][i] = gm[(size_t)idx.st.v[s][i]];
+    });
+}
+
+// Row form of MGATHER: dst[i,:] = table[rowIdx[i], :], i.e. MGATHER with idx[i,j] = rowIdx[i]*Cols + j,
+// done with 16-byte loads.  rowIdx is a [Rows,1] int32 tile; rows whose index lies outside
+// [0, tableRows) are zero-filled (the out-of-range rule of TGATHER, cpu/TGather.hpp:78-81).
+template <typename DstT, typename G, typename IdxT>
+PTO_DEV void MGATHER_ROWS_IMPL(DstT &dst, G &table, IdxT &rowIdx, int tableRows)
+{
+    using T = typename DstT::DType;
+    using S = typename DstT::Storage;
+    static_assert(DstT::isRowMajor && DstT::Cols % detail::kVecChunk == 0, "[PTO][SA] MGATHER rows: row-major, cols % 8 == 0");
+    static_assert(IdxT::Rows == DstT::Rows && sizeof(typename IdxT::DType) == 4, "[PTO][SA] MGATHER rows: [Rows,1] int32 indices");
+    __shared__ int32_t rows[DstT::Rows];
+    detail::stage_row_values<IdxT, DstT::Rows>(rowIdx, rows);
+    hw::lds_barrier();
+    const T *gm = reinterpret_cast<const T *>(table.data());
+    const int64_t ld = table.GetStride(3);
+    using VT = T __attribute__((ext_vector_type(detail::kVecChunk)));
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+        const int e0 = q * detail::kVecChunk;
+        const int r = e0 / DstT::Cols, c0 = e0 % DstT::Cols;
+        VT v = {};
+        if (q < S::Chunks && r < vr && c0 + detail::kVecChunk <= vc) {
+            const int32_t ri = rows[r];
+            if (ri >= 0 && ri < tableRows)
+                v = *reinterpret_cast<const VT *>(gm + (int64_t)ri * ld + c0);
+        }
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = v[i];
+    }
+    hw::lds_barrier();
+}
+
+} // namespace pto

@@ -1,0 +1,83 @@
+/*
+ * pto_amd.h -- C ABI of the MI355X (gfx950) back end for the PTO tile compute path.
+ *
+ * Every entry point is stream-ordered and asynchronous, takes raw device pointers owned by the
+ * caller and allocates nothing.  `stream` is a hipStream_t passed as void* (NULL = default stream),
+ * like the `void *stream` of the reference's launch wrappers.  Return value: PTO_OK, or a negative
+ * PTO_ERR_* code; nothing is launched when an error is returned.
+ *
+ * Reference interfaces these replace (cannmirror/pto-isa, file:line):
+ *   pto_gemm_f16f32      LaunchGEMME2E<T>(uint8_t *out, uint8_t *src0, uint8_t *src1, void *stream)
+ *                        kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp:243-264, and the
+ *                        ctypes entry call_kernel(blockDim, stream, out, src0, src1) demos/torch_jit/gemm/gemm_kernel.cpp:259-262
+ *   pto_fa_fwd_f16       LaunchTFA<...>(...) kernels/manual/common/flash_atten/fa_performance_kernel.h:28-41 and
+ *                        call_kernel(...) demos/torch_jit/flash_atten/fa_kernel.cpp:1017-1092
+ *   pto_tcvt_*           runTCVT / launchTCVT tests/cpu/st/testcase/tcvt/tcvt_kernel.cpp:18-66 (TLOAD -> TCVT -> TSTORE)
+ *   pto_gather_rows      MGATHER include/pto/common/pto_instr.hpp:1328-1334 with idx[i,j] = idx[i]*cols + j
+ *                        (test kernels tests/cpu/st/testcase/mgather/, tgather/tgather_kernel.cpp:224-)
+ */
+#ifndef PTO_AMD_H
+#define PTO_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PTO_OK 0
+#define PTO_ERR_BAD_ARG (-1)     /* null pointer, non-positive extent, unknown enum value */
+#define PTO_ERR_UNSUPPORTED (-2) /* shape not a multiple of the tile the kernel is built for */
+#define PTO_ERR_HIP (-3)         /* the HIP runtime refused the launch; see pto_last_hip_error() */
+#define PTO_ERR_WORKSPACE (-4)   /* workspace missing or too small */
+
+/* rounding modes of TCVT: values of pto::RoundMode (include/pto/common/type.hpp:167-176) */
+#define PTO_CAST_RINT 1
+#define PTO_CAST_ROUND 2
+#define PTO_CAST_FLOOR 3
+#define PTO_CAST_CEIL 4
+#define PTO_CAST_TRUNC 5
+#define PTO_CAST_ODD 6
+
+/* Library / device checks: 0 when a gfx950 device is current and usable. */
+int pto_init(void);
+const char *pto_version(void);
+/* hipError_t of the last failing HIP call made by this library on the calling thread (0 = none) */
+int pto_last_hip_error(void);
+
+/* C[m,n] fp32 row-major = A[m,k] fp16 row-major x B, where B is stored [n,k] fp16 (a column-major
+ * k x n operand), fp32 accumulation.  m % 128 == 0, n % 256 == 0, k % 64 == 0 (the 128 x 256 block,
+ * K-step 64 of the reference kernel). */
+int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k);
+
+/* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
+ * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];
+ * lse: NULL or fp32 [batch, heads, seq_q] = max*scale + ln(sum).  scale = 1/sqrt(head_dim) is applied
+ * to (x - max) as in the reference's softmax stage.  causal != 0: key j is visible to query i iff
+ * j <= i + (seq_kv - seq_q).  head_dim in {64, 128}; seq_q % 128 == 0, seq_kv % 64 == 0.
+ * workspace: device scratch of at least pto_fa_fwd_workspace_bytes(...) bytes (holds V transposed). */
+size_t pto_fa_fwd_workspace_bytes(int batch, int heads, int seq_q, int seq_kv, int head_dim);
+int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                   int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int o_fp32,
+                   void *workspace, size_t workspace_bytes);
+
+/* Elementwise conversion of n contiguous fp32 values (TLOAD -> TCVT -> TSTORE over 1 x 8192 tiles).
+ * fp16: any PTO_CAST_* mode (PTO_CAST_RINT = IEEE round-to-nearest-even).  bf16: PTO_CAST_RINT only.
+ * NaN inputs give a quiet NaN that keeps the sign and the top payload bits. */
+int pto_tcvt_f32_f16(void *stream, uint16_t *dst, const float *src, size_t n, int round_mode);
+int pto_tcvt_f32_bf16(void *stream, uint16_t *dst, const float *src, size_t n, int round_mode);
+
+/* out[i, :] = table[idx[i], :] for i < n_idx; rows whose index is outside [0, table_rows) are zero.
+ * elem_bytes in {2, 4}; cols % 8 == 0.  table [table_rows, cols] and out [n_idx, cols] contiguous. */
+int pto_gather_rows(void *stream, void *out, const void *table, const int32_t *idx, size_t n_idx,
+                    size_t table_rows, size_t cols, int elem_bytes);
+
+/* TGATHER index form on one tile pair (tests/cpu/st/testcase/tgather): dst[r,c] = src0.flat[idx[r,c]],
+ * out-of-range -> 0.  src0 [16,1024] fp16, idx and dst [16,128]. */
+int pto_tgather_index_f16_16x1024_16x128(void *stream, uint16_t *dst, const uint16_t *src0, const int32_t *idx);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PTO_AMD_H */

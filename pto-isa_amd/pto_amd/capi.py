@@ -1,0 +1,53 @@
+"""ctypes binding of libpto_amd.so (the C ABI declared in include/pto_amd.h).
+
+Device pointers are passed as integers (e.g. torch.Tensor.data_ptr()); streams as integers
+(torch.cuda.current_stream().cuda_stream) or 0 for the default stream.  The library must have been
+built (python pto-isa_amd/build.py): loading fails loudly otherwise, there is no fallback path.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(_HERE, "libpto_amd.so")
+
+OK, ERR_BAD_ARG, ERR_UNSUPPORTED, ERR_HIP, ERR_WORKSPACE = 0, -1, -2, -3, -4
+CAST_RINT, CAST_ROUND, CAST_FLOOR, CAST_CEIL, CAST_TRUNC, CAST_ODD = 1, 2, 3, 4, 5, 6
+
+SYMBOLS = {
+    "pto_init": (C.c_int, []),
+    "pto_version": (C.c_char_p, []),
+    "pto_last_hip_error": (C.c_int, []),
+    "pto_gemm_f16f32": (C.c_int, [C.c_void_p] * 4 + [C.c_int] * 3),
+    "pto_tcvt_f32_f16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),
+    "pto_tcvt_f32_bf16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),
+    "pto_gather_rows": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t] * 3 + [C.c_int]),
+    "pto_tgather_index_f16_16x1024_16x128": (C.c_int, [C.c_void_p] * 4),
+}
+
+_lib = None
+
+
+def load():
+    """Load the shared library and declare every symbol of include/pto_amd.h."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError("libpto_amd.so is not built: run `python pto-isa_amd/build.py`")
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            fn = getattr(lib, name)          # AttributeError if the library lacks a declared symbol
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+class PtoError(RuntimeError):
+    pass
+
+
+def check(rc, what):
+    if rc != OK:
+        names = {ERR_BAD_ARG: "bad argument", ERR_UNSUPPORTED: "unsupported shape", ERR_HIP: "HIP error",
+                 ERR_WORKSPACE: "workspace too small"}
+        raise PtoError("%s failed: %s (%d), hip=%d" % (what, names.get(rc, "?"), rc, load().pto_last_hip_error()))
