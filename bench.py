@@ -1,0 +1,211 @@
+#!/usr/bin/env python3
+"""Benchmark of the PTO tile compute path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|fa|tcvt|gather]
+
+A step is one pass of the hot path over one batch of synthetic input, resident in HBM before the
+timed region: one fp16 -> fp32 GEMM at m=n=k=6144 (the configuration the headline metric is quoted
+on).  The other workloads of the metric (flash-attention forward, TCVT, gather) are timed the same
+way and reported under "extra".  Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "pto-isa_amd")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_FP16_TFLOPS = 2516.6   # MI355X dense fp16 matrix peak (published)
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
+
+
+def time_launches(torch, fn, steps, warmup):
+    """Average duration in ms of fn() over `steps` launches on torch's current stream (HIP events)."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / steps
+
+
+def bench_gemm(torch, lib, capi, datagen, size, steps, warmup):
+    import numpy as np
+    a, b = datagen.gemm_inputs(size, size, size)
+    ta = torch.from_numpy(a.view(np.int16)).cuda()
+    tb = torch.from_numpy(b.view(np.int16)).cuda()
+    tc = torch.empty((size, size), dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        capi.check(lib.pto_gemm_f16f32(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), size, size, size), "gemm")
+    ms = time_launches(torch, step, steps, warmup)
+    flops = 2.0 * size ** 3
+    return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
+
+
+def bench_fa(torch, lib, capi, datagen, cfg, steps, warmup):
+    import numpy as np
+    B, H, S, D, causal = cfg
+    scale = 1.0 / np.sqrt(D) if not causal else 1.0
+    q, k, v = datagen.fa_inputs(B, H, S, S, D, scale=scale)
+    tq, tk, tv = (torch.from_numpy(t.view(np.int16)).cuda() for t in (q, k, v))
+    to = torch.empty((B, H, S, D), dtype=torch.int16, device="cuda")
+    tl = torch.empty((B, H, S), dtype=torch.float32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        capi.check(lib.pto_fa_fwd_f16(st, to.data_ptr(), tl.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
+                                      B, H, S, S, D, int(causal), 0), "fa")
+    ms = time_launches(torch, step, steps, warmup)
+    flops = 4.0 * B * H * S * S * D      # the reference's convention (flash_atten/main.cpp:650)
+    if causal:
+        flops *= 0.5                     # causal counted as half
+    return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops,
+            "flop_convention": "4*B*H*Sq*Sk*D" + (" / 2 (causal)" if causal else "")}
+
+
+def bench_tcvt(torch, lib, capi, datagen, steps, warmup, kind):
+    rows, cols = 16384, 8192
+    n = rows * cols
+    # two buffer sets, alternated, so that no launch finds its input in cache
+    xs = [torch.randn(n, device="cuda") * 100.0 for _ in range(2)]
+    outs = [torch.empty(n, dtype=torch.int16, device="cuda") for _ in range(2)]
+    fn = lib.pto_tcvt_f32_f16 if kind == "f16" else lib.pto_tcvt_f32_bf16
+    st = torch.cuda.current_stream().cuda_stream
+    i = [0]
+
+    def step():
+        j = i[0] & 1
+        i[0] += 1
+        capi.check(fn(st, outs[j].data_ptr(), xs[j].data_ptr(), n, capi.CAST_RINT), "tcvt")
+    ms = time_launches(torch, step, steps, warmup)
+    nbytes = n * 6.0
+    return {"ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9, "bytes": nbytes}
+
+
+def bench_gather(torch, lib, capi, datagen, steps, warmup):
+    import numpy as np
+    table, idx = datagen.gather_inputs(16384, 1024, 65536)
+    tt = torch.from_numpy(table.view(np.int16)).cuda()
+    ti = torch.from_numpy(idx).cuda()
+    outs = [torch.empty((65536, 1024), dtype=torch.int16, device="cuda") for _ in range(2)]
+    st = torch.cuda.current_stream().cuda_stream
+    i = [0]
+
+    def step():
+        j = i[0] & 1
+        i[0] += 1
+        capi.check(lib.pto_gather_rows(st, outs[j].data_ptr(), tt.data_ptr(), ti.data_ptr(), 65536, 16384, 1024, 2), "gather")
+    ms = time_launches(torch, step, steps, warmup)
+    nbytes = 65536 * 1024 * 2 * 2 + 65536 * 4.0
+    return {"ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9, "bytes": nbytes}
+
+
+def cpu_baseline(datagen, size):
+    """The reference CPU-simulation arithmetic timed on the host cores, on a bounded sample of the
+    6144^3 product: rows [0,64) of C (1/96 of the work) through the oracle's port of the tile path
+    (TLOAD/TEXTRACT/TMATMUL[_ACC] per K-step of 64), threads over rows as the reference does."""
+    from oracle import oracle
+    a, b = datagen.gemm_inputs(size, size, size)
+    rows = 2048
+    cores = oracle.online_cpus()
+    cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else min(cores, int(os.environ["OMP_NUM_THREADS"]))
+    t0 = time.perf_counter()
+    oracle.gemm_f16f32(a, b, base_k=64, row0=0, row1=rows, threads=cores)
+    dt = time.perf_counter() - t0
+    flops = 2.0 * rows * size * size
+    out = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+           "sample": "rows 0..%d of C at m=n=k=%d (%.3g of the flops), %.1f s" % (rows - 1, size, rows / size, dt)}
+    ref = oracle.ref()
+    if ref is not None:
+        import ctypes as C
+        import numpy as np
+        a1, b1 = datagen.gemm_inputs(1536, 1536, 1536)
+        c1 = np.zeros((1536, 1536), dtype=np.float32)
+        t0 = time.perf_counter()
+        ref.ref_gemm_1536x1536x1536_ks1536(c1.ctypes.data_as(C.c_void_p), a1.ctypes.data_as(C.c_void_p),
+                                           b1.ctypes.data_as(C.c_void_p))
+        dt1 = time.perf_counter() - t0
+        out["reference_1536_single_tile"] = {"seconds": dt1, "tflops": 2.0 * 1536 ** 3 / dt1 / 1e12,
+                                             "what": "compiled reference CPU-simulation headers, one TMATMUL 1536^3"}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--only", default="", help="gemm | fa | tcvt | gather: time just that workload")
+    ap.add_argument("--size", type=int, default=6144)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every workload of the metric "
+                 "fits one MI355X, and nothing here uses a second device)" % args.gpus)
+
+    import torch
+    from pto_amd import capi, datagen
+    lib = capi.load()
+    capi.check(lib.pto_init(), "pto_init")
+    torch.cuda.set_device(0)
+
+    extra = {}
+    only = args.only
+    gemm = None
+    if only in ("", "gemm"):
+        gemm = bench_gemm(torch, lib, capi, datagen, args.size, args.steps, args.warmup)
+    if only == "":
+        for s in (3072, 7680):
+            r = bench_gemm(torch, lib, capi, datagen, s, max(args.steps // 2, 1), 2)
+            extra["gemm_%d" % s] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp16_peak": r["tflops"] / PEAK_FP16_TFLOPS}
+    if only in ("", "fa") and hasattr(lib, "pto_fa_fwd_f16"):
+        for name, cfg in (("fa_b1_h16_s4096_d128", (1, 16, 4096, 128, False)),
+                          ("fa_causal_b4_h32_s2048_d64", (4, 32, 2048, 64, True))):
+            r = bench_fa(torch, lib, capi, datagen, cfg, args.steps, args.warmup)
+            extra[name] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp16_peak": r["tflops"] / PEAK_FP16_TFLOPS,
+                           "flop_convention": r["flop_convention"]}
+    if only in ("", "tcvt"):
+        for kind in ("f16", "bf16"):
+            r = bench_tcvt(torch, lib, capi, datagen, args.steps, args.warmup, kind)
+            extra["tcvt_f32_%s_16384x8192" % kind] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS}
+    if only in ("", "gather"):
+        r = bench_gather(torch, lib, capi, datagen, args.steps, args.warmup)
+        extra["gather_rows_65536x1024_f16"] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS}
+
+    line = {
+        "metric": "GEMM TFLOPS & % MFMA peak at m=n=k=6144; flash-attn fwd TFLOPS",
+        "value": gemm["tflops"] if gemm else None,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": gemm["ms"] if gemm else None,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp16 x fp16 -> fp32 accumulate",
+        "data": "synthetic: A [m,k], B [n,k] i.i.d. uniform[-1,1] fp16 from seed 19 / 1019",
+        "config": {"workload": "fp16->fp32 GEMM m=n=k=%d, 128x256 block, K-step 64, full K per output tile" % args.size},
+        "extra": extra,
+    }
+    if gemm:
+        line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
+                            "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": None,
+                            "kernel": "GemmF16F32<128,256,64>", "flops_per_launch": gemm["flops"]}
+    if not args.no_cpu and only in ("", "gemm"):
+        line["cpu_baseline"] = cpu_baseline(datagen, args.size)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
