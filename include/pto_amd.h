@@ -54,13 +54,12 @@ int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];
  * lse: NULL or fp32 [batch, heads, seq_q] = max*scale + ln(sum).  scale = 1/sqrt(head_dim) is applied
- * to (x - max) as in the reference's softmax stage.  causal != 0: key j is visible to query i iff
- * j <= i + (seq_kv - seq_q).  head_dim in {64, 128}; seq_q % 128 == 0, seq_kv % 64 == 0.
- * workspace: device scratch of at least pto_fa_fwd_workspace_bytes(...) bytes (holds V transposed). */
-size_t pto_fa_fwd_workspace_bytes(int batch, int heads, int seq_q, int seq_kv, int head_dim);
+ * to (x - max) as in the reference's softmax stage (pto_macro_fa_softmax.hpp:82-97).  causal != 0:
+ * key j is visible to query i iff j <= i + (seq_kv - seq_q); seq_kv >= seq_q is required then.
+ * head_dim in {64, 128}; seq_q % 128 == 0, seq_kv % 64 == 0.  No workspace: scores and probabilities
+ * never leave the compute unit (the reference's caller-provided GM FIFOs have no counterpart). */
 int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,
-                   int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int o_fp32,
-                   void *workspace, size_t workspace_bytes);
+                   int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int o_fp32);
 
 /* Elementwise conversion of n contiguous fp32 values (TLOAD -> TCVT -> TSTORE over 1 x 8192 tiles).
  * fp16: any PTO_CAST_* mode (PTO_CAST_RINT = IEEE round-to-nearest-even).  bf16: PTO_CAST_RINT only.

@@ -1,0 +1,318 @@
+// Flash-attention forward for MI355X: one fused kernel built from PTO tile instructions.
+//
+// Arithmetic follows the reference's streaming softmax and rescale stages
+// (kernels/manual/common/flash_atten/pto_macro_fa_softmax.hpp:47-215, pto_macro_fa_gu.hpp:33-56):
+//   per key tile X = q k^T (fp32);  M' = max(M, rowmax X);  alpha = exp(s (M - M'));
+//   P = exp(s (X - M'));  S = alpha S + rowsum P;  O = alpha O + half(P) v;  at the end O /= S,
+// s = 1/sqrt(head_dim), causal mask = -3.40282e38 added to the hidden scores.
+//
+// Structure.  The reference runs the four stages on two kinds of cores that hand tiles over
+// through global-memory FIFOs (fa_performance_kernel.cpp:607-963).  A CDNA4 compute unit does
+// matrix and vector work itself, so here a workgroup owns 128 query rows of one head and keeps
+// scores, probabilities and the output accumulator in registers for the whole sweep over the keys:
+//   * wave grid 1 x 4: every wave owns 32 queries and sees every key of the tile,
+//   * the score tile is computed transposed, X^T = K Q^T (TMATMUL with K as the Left operand and
+//     Q^T as the Right operand), so that in the MFMA accumulator layout one lane holds one query
+//     and the per-query quantities (max, sum, alpha) are per-lane scalars: the row reductions of
+//     the softmax are in-register, plus one exchange between the two half-waves for the max,
+//   * P^T in accumulator layout already is a Right (B) operand for O^T = V^T P^T up to a
+//     permutation of the keys inside a 16-key step; V^T is read from the row-major V tile in LDS
+//     with the transposing ds_read_b64_tr_b16 using the same permutation, so P never moves,
+//   * K and V tiles are double-buffered in LDS by asynchronous TLOADs.
+#define PTO_WAVES_M 1
+#define PTO_WAVES_N 4
+#include <pto/pto-inst.hpp>
+
+#include "common.hpp"
+
+using namespace pto;
+
+PTO_DEVICE_CODE_BEGIN
+
+namespace {
+
+constexpr int kBQ = 128; // queries per workgroup (4 waves x 32)
+constexpr int kBKV = 64; // keys per tile
+constexpr float kMaskValue = -3.40282e+38f; // pto_macro_fa_softmax.hpp:67
+
+// exchange a value with the lane 32 positions away
+AICORE inline float SwapHalves(float x) { return __shfl_xor(x, 32); }
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+
+// V^T operand for O^T += V^T P^T: TEXTRACT of the [32 d, kBKV keys] block `db` of the transposed
+// V tile, taken straight from the row-major [keys, D] LDS image with transposing reads.  Key order
+// inside every 16-key MFMA step matches the order in which the accumulator layout holds P^T:
+// k slot j of half-wave h  <->  key 16t + 8(j/4) + 4h + j%4.
+template <typename LeftT, typename MatT>
+AICORE inline void ExtractVT(LeftT &dst, MatT &vMat, int db)
+{
+    using Geo = detail::MatGeom<MatT>;
+    using S = typename LeftT::Storage;
+    static_assert(S::MB == 1 && S::KS == kBKV / 16, "one 32-row block of V^T over the whole key tile");
+    const char *lds = hw::lds_base() + vMat.st.lds;
+    const uint32_t lane = (uint32_t)hw::lane();
+    const uint32_t h = lane >> 5;
+    const uint32_t d0 = (uint32_t)db * 32u + 16u * ((lane >> 4) & 1u) + 4u * (lane & 3u);
+    const uint32_t keyIn = (lane & 15u) >> 2;
+#pragma unroll
+    for (int ks = 0; ks < S::KS; ++ks) {
+        s16x4 part[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const uint32_t key = 16u * ks + 8u * u + 4u * h + keyIn;
+            const uint32_t off = detail::mat_chunk_off<Geo::RowBytes>(key, d0 >> 3) + ((d0 & 7u) << 1);
+            part[u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(lds + off));
+        }
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        s16x8 both = {part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
+        dst.st.f[0][ks] = __builtin_bit_cast(f16x8, both);
+    }
+}
+
+template <int D, bool CAUSAL, bool OUT_F32>
+__global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
+                                                                      __gm__ const half *qAll, __gm__ const half *kAll,
+                                                                      __gm__ const half *vAll, int heads, int seqQ,
+                                                                      int seqKv, int numBH)
+{
+    constexpr int KB = kBKV / 32; // 32-key blocks per tile
+    constexpr int DB = D / 32;    // 32-wide blocks of the head dimension
+    // ---- tiles ----
+    using TileMatQ = Tile<TileType::Mat, half, D, kBQ, BLayout::RowMajor, D, kBQ, SLayout::ColMajor>;   // Q^T, contiguous along d
+    using TileMatK = Tile<TileType::Mat, half, kBKV, D, BLayout::ColMajor, kBKV, D, SLayout::RowMajor>; // K,   contiguous along d
+    using TileMatV = Tile<TileType::Mat, half, kBKV, D, BLayout::ColMajor, kBKV, D, SLayout::RowMajor>; // V,   contiguous along d
+    using RightQ = TileRight<half, D, kBQ, D, kBQ>;        // per wave: 32 queries x D
+    using LeftK = TileLeft<half, 32, D, 32, D>;            // 32 keys x D (every wave holds the same keys)
+    using AccS = TileAcc<float, 32, kBQ, 32, kBQ>;         // X^T block: 32 keys x 32 queries per wave
+    using RightP = TileRight<half, kBKV, kBQ, kBKV, kBQ>;  // P^T: kBKV keys x 32 queries per wave
+    using LeftVT = TileLeft<half, 32, kBKV, 32, kBKV>;     // V^T block: 32 d x kBKV keys
+    using AccO = TileAcc<float, 32, kBQ, 32, kBQ>;         // O^T block: 32 d x 32 queries per wave
+
+    using GlobalQT = GlobalTensor<half, TileShape2D<half, D, kBQ, Layout::DN>, Stride<1, 1, 1, 1, D>, Layout::DN>;
+    using GlobalKV = GlobalTensor<half, TileShape2D<half, kBKV, D, Layout::ND>, Stride<1, 1, 1, D, 1>, Layout::ND>;
+
+    constexpr uint32_t kTileBytes = kBKV * D * sizeof(half);
+    constexpr uint32_t kStageBytes = 2 * kTileBytes;
+    static_assert(D * kBQ * sizeof(half) <= kStageBytes, "Q^T staging reuses the second K/V stage");
+
+    // ---- which (batch*head, query tile) this workgroup owns.  Workgroups are dealt round-robin to
+    // the 8 XCDs: keep a head on one XCD so that its K/V stay in that XCD's L2.  Causal: the query
+    // tiles with the most keys go first.
+    const int numQT = seqQ / kBQ;
+    int bh, qt;
+    {
+        const int bid = (int)get_block_idx();
+        if (numBH % 8 == 0) {
+            const int xcd = bid % 8, slot = bid / 8, perXcd = numBH / 8;
+            bh = xcd + 8 * (slot % perXcd);
+            qt = slot / perXcd;
+        } else {
+            bh = bid % numBH;
+            qt = bid / numBH;
+        }
+        if (CAUSAL)
+            qt = numQT - 1 - qt;
+    }
+    const int q0 = qt * kBQ;
+    __gm__ half *qBase = const_cast<half *>(qAll) + ((int64_t)bh * seqQ + q0) * D;
+    __gm__ half *kBase = const_cast<half *>(kAll) + (int64_t)bh * seqKv * D;
+    __gm__ half *vBase = const_cast<half *>(vAll) + (int64_t)bh * seqKv * D;
+
+    const int causalOff = seqKv - seqQ;
+    int numTiles = seqKv / kBKV;
+    if (CAUSAL) { // tiles wholly above the diagonal are skipped (fa_performance_kernel.cpp:757-758)
+        const int lastKey = q0 + kBQ - 1 + causalOff;
+        const int lim = lastKey / kBKV + 1;
+        numTiles = lim < numTiles ? lim : numTiles;
+    }
+
+    TileMatK kMat[2];
+    TileMatV vMat[2];
+    TileMatQ qMat;
+    TASSIGN(kMat[0], 0u);
+    TASSIGN(vMat[0], kTileBytes);
+    TASSIGN(kMat[1], kStageBytes);
+    TASSIGN(vMat[1], kStageBytes + kTileBytes);
+    TASSIGN(qMat, kStageBytes); // lives in stage 1 until it has been extracted
+
+    RightQ qRight;
+    AccO oAcc[DB];
+    float runMax = 0.0f, runSum = 0.0f; // per lane: this lane's query; runSum is the half-wave partial
+    const int lane = hw::lane();
+    const int myQuery = q0 + hw::wave_n() * 32 + (lane & 31); // row of Q this lane's column holds
+    const uint32_t hHalf = (uint32_t)lane >> 5;
+    // s = 1/sqrt(D) folded with log2(e): exp(s y) = exp2(s log2e y)
+    const float sLog2e = (D == 128 ? 0.08838834764831845f : 0.125f) * 1.4426950408889634f;
+
+    {
+        GlobalQT gmQ(qBase);
+        GlobalKV gmK(kBase), gmV(vBase);
+        TLOAD(qMat, gmQ);
+        TLOAD(kMat[0], gmK);
+        TLOAD(vMat[0], gmV);
+        set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+        wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+        TEXTRACT(qRight, qMat, 0, 0);
+        set_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1);
+        wait_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1); // Q^T is in registers everywhere: stage 1 may be overwritten
+    }
+
+    for (int tile = 0; tile < numTiles; tile += 2) {
+#pragma unroll
+        for (int st = 0; st < 2; ++st) { // unrolled over the two LDS stages
+            const int t = tile + st;
+            if (t >= numTiles)
+                break;
+            if (t > 0)
+                wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
+            if (t + 1 < numTiles) {
+                GlobalKV gmK(kBase + (int64_t)(t + 1) * kBKV * D), gmV(vBase + (int64_t)(t + 1) * kBKV * D);
+                TLOAD(kMat[st ^ 1], gmK);
+                TLOAD(vMat[st ^ 1], gmV);
+                set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+            }
+
+            // ---- X^T = K Q^T ----
+            AccS sAcc[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                LeftK kLeft;
+                TEXTRACT(kLeft, kMat[st], kb * 32, 0);
+                TMATMUL(sAcc[kb], kLeft, qRight);
+            }
+
+            // ---- streaming softmax on the accumulator fragments (one query per lane) ----
+            const int key0 = t * kBKV;
+            if (CAUSAL && key0 + kBKV - 1 > q0 + causalOff) { // the diagonal crosses this tile
+                const int limit = myQuery + causalOff;        // last visible key of this lane's query
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = key0 + kb * 32 + (v >> 2) * 8 + (int)hHalf * 4 + (v & 3);
+                        if (key > limit)
+                            sAcc[kb].st.f[0][0][v] += kMaskValue;
+                    }
+            }
+            float locMax = sAcc[0].st.f[0][0][0];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    locMax = fmaxf(locMax, sAcc[kb].st.f[0][0][v]);
+            locMax = fmaxf(locMax, SwapHalves(locMax));
+            const float newMax = t == 0 ? locMax : fmaxf(runMax, locMax);
+            const float alpha = t == 0 ? 1.0f : __builtin_amdgcn_exp2f((runMax - newMax) * sLog2e);
+            runMax = newMax;
+            const float negMax = -newMax * sLog2e;
+            float locSum = 0.0f;
+            RightP pRight;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int half_ = 0; half_ < 2; ++half_) {
+                    f16x8 pk;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][0][half_ * 8 + j], sLog2e, negMax));
+                        locSum += p; // row sum over the fp32 P, as the reference does
+                        pk[j] = (half)p;
+                    }
+                    pRight.st.f[0][kb * 2 + half_] = pk;
+                }
+            runSum = t == 0 ? locSum : runSum * alpha + locSum;
+
+            // ---- O^T = alpha O^T + V^T P^T ----
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                LeftVT vLeft;
+                ExtractVT(vLeft, vMat[st], db);
+                if (t == 0) {
+                    TMATMUL(oAcc[db], vLeft, pRight);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        oAcc[db].st.f[0][0][v] *= alpha;
+                    TMATMUL_ACC(oAcc[db], oAcc[db], vLeft, pRight);
+                }
+            }
+        }
+    }
+
+    // ---- finish: O /= S, write O (and LSE) ----
+    const float total = runSum + SwapHalves(runSum);
+    const float inv = 1.0f / total;
+    const int64_t row = (int64_t)bh * seqQ + myQuery;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int d = db * 32 + g * 8 + (int)hHalf * 4;
+            float o4[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                o4[r] = oAcc[db].st.f[0][0][g * 4 + r] * inv;
+            if constexpr (OUT_F32) {
+                f32x4 v = {o4[0], o4[1], o4[2], o4[3]};
+                *reinterpret_cast<f32x4 *>(static_cast<float *>(outO) + row * D + d) = v;
+            } else {
+                f16x4 v = {(half)o4[0], (half)o4[1], (half)o4[2], (half)o4[3]};
+                *reinterpret_cast<f16x4 *>(static_cast<half *>(outO) + row * D + d) = v;
+            }
+        }
+    if (outLse != nullptr && hHalf == 0) {
+        const float scale = D == 128 ? 0.08838834764831845f : 0.125f;
+        outLse[row] = runMax * scale + __builtin_logf(total);
+    }
+}
+
+} // namespace
+
+PTO_DEVICE_CODE_END
+
+namespace {
+template <int D, bool CAUSAL, bool OUT_F32>
+int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads,
+              int seqQ, int seqKv)
+{
+    constexpr int lds = 2 * 2 * kBKV * D * (int)sizeof(half);
+    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32>;
+    static const int attr = pto_amd::allow_lds(kernel, lds);
+    if (attr != PTO_OK)
+        return attr;
+    const int numBH = batch * heads;
+    const long long blocks = (long long)numBH * (seqQ / kBQ);
+    if (blocks > 0x7fffffffLL)
+        return PTO_ERR_UNSUPPORTED;
+    kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH);
+    return pto_amd::check_launch();
+}
+} // namespace
+
+extern "C" int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,
+                              int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int o_fp32)
+{
+    if (!o || !q || !k || !v || batch <= 0 || heads <= 0 || seq_q <= 0 || seq_kv <= 0)
+        return PTO_ERR_BAD_ARG;
+    if ((head_dim != 64 && head_dim != 128) || seq_q % kBQ || seq_kv % kBKV)
+        return PTO_ERR_UNSUPPORTED;
+    if (causal && seq_kv < seq_q)
+        return PTO_ERR_UNSUPPORTED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half *hq = reinterpret_cast<const half *>(q), *hk = reinterpret_cast<const half *>(k),
+               *hv = reinterpret_cast<const half *>(v);
+#define PTO_FA_CASE(DD, CC, FF)                                                                      \
+    if (head_dim == DD && (causal != 0) == CC && (o_fp32 != 0) == FF)                                \
+        return launch_fa<DD, CC, FF>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+    PTO_FA_CASE(128, false, false)
+    PTO_FA_CASE(128, false, true)
+    PTO_FA_CASE(128, true, false)
+    PTO_FA_CASE(128, true, true)
+    PTO_FA_CASE(64, false, false)
+    PTO_FA_CASE(64, false, true)
+    PTO_FA_CASE(64, true, false)
+    PTO_FA_CASE(64, true, true)
+#undef PTO_FA_CASE
+    return PTO_ERR_UNSUPPORTED;
+}
