@@ -218,6 +218,15 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
 
 } // namespace detail
 
+// Number of asynchronous global->LDS copy instructions that one TLOAD of a fully valid Mat tile
+// issues per wave (what wait_flag_pending counts).
+template <typename TileT>
+constexpr int TLoadInstrs()
+{
+    using Geo = detail::MatGeom<TileT>;
+    return detail::cdiv(detail::cdiv(Geo::Major * Geo::ChunksPerRow, kWaveSize), kBlockWaves);
+}
+
 template <typename TileT, typename G>
 PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 {

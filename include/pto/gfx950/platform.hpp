@@ -70,6 +70,13 @@ PTO_DEV char *lds_base()
 }
 
 PTO_DEV void wait_vm0() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// wait until at most N of this wave's vector-memory instructions are still outstanding (N <= 63)
+template <int N>
+PTO_DEV void wait_vm()
+{
+    static_assert(N >= 0 && N <= 63, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
 PTO_DEV void wait_lgkm0() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
 // Workgroup barrier that orders LDS traffic only; outstanding global loads keep flying.
 PTO_DEV void lds_barrier()
@@ -103,6 +110,17 @@ PTO_DEV void wait_flag(pipe_t src, pipe_t dst, event_t)
         pto::hw::wait_vm0();
     }
     // MTE1->M, M->MTE1, M->FIX, FIX->M, V<->M ...: register dependences, nothing to do
+}
+
+// Pipelined form of wait_flag(PIPE_MTE2, PIPE_MTE1, id) for software pipelines that keep several
+// TLOADs in flight: returns once all but the `Pending` most recently issued asynchronous copy
+// instructions of every wave have landed in LDS (vmcnt retires in order).  Pending is a count of
+// wave instructions; pto::TLoadInstrs<Tile>() gives the number one TLOAD issues.
+template <int Pending>
+PTO_DEV void wait_flag_pending(pipe_t, pipe_t, event_t)
+{
+    pto::hw::wait_vm<Pending>();
+    pto::hw::lds_barrier();
 }
 
 PTO_DEV void pipe_barrier(pipe_t p)
