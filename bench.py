@@ -112,7 +112,7 @@ def bench_gather(torch, lib, capi, datagen, steps, warmup):
 
 def cpu_baseline(datagen, size):
     """The reference CPU-simulation arithmetic timed on the host cores, on a bounded sample of the
-    6144^3 product: rows [0,64) of C (1/96 of the work) through the oracle's port of the tile path
+    6144^3 product: rows [0,2048) of C (1/3 of the work) through the oracle's port of the tile path
     (TLOAD/TEXTRACT/TMATMUL[_ACC] per K-step of 64), threads over rows as the reference does."""
     from oracle import oracle
     a, b = datagen.gemm_inputs(size, size, size)
@@ -195,13 +195,14 @@ def main():
         "vs_baseline": None,
         "dtype": "fp16 x fp16 -> fp32 accumulate",
         "data": "synthetic: A [m,k], B [n,k] i.i.d. uniform[-1,1] fp16 from seed 19 / 1019",
-        "config": {"workload": "fp16->fp32 GEMM m=n=k=%d, 128x256 block, K-step 64, full K per output tile" % args.size},
+        "config": {"workload": "fp16->fp32 GEMM m=n=k=%d, A row-major, B column-major, full K reduction per output tile "
+                               "(256x256 C tile per workgroup, K-step 32)" % args.size},
         "extra": extra,
     }
     if gemm:
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                             "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": None,
-                            "kernel": "GemmF16F32<128,256,64>", "flops_per_launch": gemm["flops"]}
+                            "kernel": "GemmF16F32Mix<256,256,4,4>", "flops_per_launch": gemm["flops"]}
     if not args.no_cpu and only in ("", "gemm"):
         line["cpu_baseline"] = cpu_baseline(datagen, args.size)
     print(json.dumps(line))

@@ -47,8 +47,8 @@ const char *pto_version(void);
 int pto_last_hip_error(void);
 
 /* C[m,n] fp32 row-major = A[m,k] fp16 row-major x B, where B is stored [n,k] fp16 (a column-major
- * k x n operand), fp32 accumulation.  m % 128 == 0, n % 256 == 0, k % 64 == 0 (the 128 x 256 block,
- * K-step 64 of the reference kernel). */
+ * k x n operand), fp32 accumulation.  m % 128 == 0, n % 256 == 0, k % 32 == 0 (multiples of the
+ * 128 x 256 block of the reference kernel; C is tiled 256 x 256 when m allows it). */
 int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k);
 
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],

@@ -16,20 +16,29 @@ constexpr int kXcds = 8; // MI355X: 8 accelerator dies, workgroups are dealt to 
 // Workgroup id -> C tile.  Consecutive ids land on different XCDs, each with its own L2, so first
 // regroup ids per XCD, then walk the tile grid in bands of GROUP_M tile rows so that the tiles
 // running together on one XCD share A and B panels.
-template <int GROUP_M>
-AICORE inline void TileOfBlock(int block, int tilesM, int tilesN, int &tm, int &tn)
+// ids [0, count) are dealt round-robin to the XCDs; give every XCD a contiguous range instead
+AICORE inline int RegroupXcd(int id, int count)
 {
-    const int total = tilesM * tilesN;
-    int id = block;
-    if (total % kXcds == 0) {
-        const int perXcd = total / kXcds;
-        id = (block % kXcds) * perXcd + block / kXcds;
-    }
+    if (count % kXcds != 0)
+        return id;
+    return (id % kXcds) * (count / kXcds) + id / kXcds;
+}
+
+// linear tile id -> (tile row, tile column), walking bands of GROUP_M tile rows column by column
+template <int GROUP_M>
+AICORE inline void TileOfId(int id, int tilesM, int tilesN, int &tm, int &tn)
+{
     const int band = GROUP_M * tilesN;
     const int g = id / band, inBand = id % band;
     const int rowsHere = (tilesM - g * GROUP_M) < GROUP_M ? (tilesM - g * GROUP_M) : GROUP_M;
     tm = g * GROUP_M + inBand % rowsHere;
     tn = inBand / rowsHere;
+}
+
+template <int GROUP_M>
+AICORE inline void TileOfBlock(int block, int tilesM, int tilesN, int &tm, int &tn)
+{
+    TileOfId<GROUP_M>(RegroupXcd(block, tilesM * tilesN), tilesM, tilesN, tm, tn);
 }
 
 template <int BM, int BN, int BK, int STAGES, int MIN_BLOCKS, int GROUP_M, int MODE = 0>
@@ -173,123 +182,6 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
     }
 }
 
-// Deeper software pipeline for one wave per SIMD (256 x 256 block, 128 x 128 per wave): the
-// TEXTRACTs of K-step i+1 are issued while the TMATMULs of step i execute, so that neither the
-// LDS latency nor the wait for the asynchronous TLOADs is exposed.  Each L1 stage holds BK = 32
-// (two 16-wide MFMA steps); operand fragments are double-buffered per 16-wide step:
-//
-//   TMATMUL_ACC(step i,  k 0..15)   | wait: stage i+1 landed, barrier; TLOAD stage i+STAGES-1;
-//                                   | TEXTRACT(stage i+1, k 0..15)
-//   TMATMUL_ACC(step i,  k 16..31)  | TEXTRACT(stage i+1, k 16..31)
-template <int BM, int BN, int STAGES, int GROUP_M>
-__global__ __launch_bounds__(kBlockThreads, 1) AICORE
-    void GemmF16F32Deep(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k)
-{
-    constexpr int BK = 32, KH = 16;
-    using TileMatA = Tile<TileType::Mat, half, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
-    using TileMatB = Tile<TileType::Mat, half, BK, BN, BLayout::RowMajor, BK, BN, SLayout::ColMajor>;
-    using LeftTile = TileLeft<half, BM, KH, BM, KH>;
-    using RightTile = TileRight<half, KH, BN, KH, BN>;
-    using ResTile = TileAcc<float, BM, BN, BM, BN>;
-    using ShapeA = TileShape2D<half, BM, BK, Layout::ND>;
-    using StrideA = BaseShape2D<half, DYNAMIC, DYNAMIC, Layout::ND>;
-    using GlobalA = GlobalTensor<half, ShapeA, StrideA, Layout::ND>;
-    using ShapeB = TileShape2D<half, BK, BN, Layout::DN>;
-    using StrideB = BaseShape2D<half, DYNAMIC, DYNAMIC, Layout::DN>;
-    using GlobalB = GlobalTensor<half, ShapeB, StrideB, Layout::DN>;
-    using ShapeC = TileShape2D<float, BM, BN, Layout::ND>;
-    using StrideC = BaseShape2D<float, DYNAMIC, DYNAMIC, Layout::ND>;
-    using GlobalC = GlobalTensor<float, ShapeC, StrideC, Layout::ND>;
-
-    constexpr uint32_t kABytes = BM * BK * sizeof(half), kBBytes = BK * BN * sizeof(half);
-    constexpr uint32_t kStage = kABytes + kBBytes;
-    constexpr int kLoadsPerStep = TLoadInstrs<TileMatA>() + TLoadInstrs<TileMatB>();
-
-    int tm, tn;
-    TileOfBlock<GROUP_M>((int)get_block_idx(), m / BM, n / BN, tm, tn);
-    __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)tm * BM * k;
-    __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)tn * BN * k;
-    const StrideA strideA(m, k);
-    const StrideB strideB(k, n);
-
-    TileMatA aMat[STAGES];
-    TileMatB bMat[STAGES];
-#pragma unroll
-    for (int s = 0; s < STAGES; ++s) {
-        TASSIGN(aMat[s], s * kStage);
-        TASSIGN(bMat[s], s * kStage + kABytes);
-    }
-    LeftTile aLo, aHi;   // k 0..15 and k 16..31 of the current stage
-    RightTile bLo, bHi;
-    ResTile cTile;
-
-    const int kLoop = k / BK;
-#pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s)
-        if (s < kLoop) {
-            GlobalA gmA(aPanel + (int64_t)s * BK, ShapeA(), strideA);
-            GlobalB gmB(bPanel + (int64_t)s * BK, ShapeB(), strideB);
-            TLOAD(aMat[s], gmA);
-            TLOAD(bMat[s], gmB);
-        }
-    // stage 0 must be complete before its fragments are read
-    if (STAGES - 2 < kLoop)
-        wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
-    else
-        wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
-    TEXTRACT(aLo, aMat[0], 0, 0);
-    TEXTRACT(bLo, bMat[0], 0, 0);
-    TEXTRACT(aHi, aMat[0], 0, KH);
-    TEXTRACT(bHi, bMat[0], KH, 0);
-    // zero the accumulators through one TMATMUL on zeroed... simpler: explicit clear
-#pragma unroll
-    for (int mb = 0; mb < ResTile::Storage::MB; ++mb)
-#pragma unroll
-        for (int nb = 0; nb < ResTile::Storage::NB; ++nb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i)
-                cTile.st.f[mb][nb][i] = 0.0f;
-
-    for (int kIter = 0; kIter < kLoop; kIter += STAGES) {
-#pragma unroll
-        for (int s = 0; s < STAGES; ++s) {
-            const int it = kIter + s;
-            if (it < kLoop) {
-                TMATMUL_ACC(cTile, cTile, aLo, bLo);
-                __builtin_amdgcn_sched_barrier(0);
-                const bool haveNext = it + 1 < kLoop;
-                if (haveNext) {
-                    // stage it+1 landed everywhere; everyone is past the reads of stage it-1
-                    if (it + STAGES - 2 < kLoop)
-                        wait_flag_pending<(STAGES - 3) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
-                    else
-                        wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
-                    const int nxt = it + STAGES - 1;
-                    if (nxt < kLoop) {
-                        const int ns = (s + STAGES - 1) % STAGES;
-                        GlobalA gmA(aPanel + (int64_t)nxt * BK, ShapeA(), strideA);
-                        GlobalB gmB(bPanel + (int64_t)nxt * BK, ShapeB(), strideB);
-                        TLOAD(aMat[ns], gmA);
-                        TLOAD(bMat[ns], gmB);
-                    }
-                    TEXTRACT(aLo, aMat[(s + 1) % STAGES], 0, 0);
-                    TEXTRACT(bLo, bMat[(s + 1) % STAGES], 0, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-                TMATMUL_ACC(cTile, cTile, aHi, bHi);
-                __builtin_amdgcn_sched_barrier(0);
-                if (haveNext) {
-                    TEXTRACT(aHi, aMat[(s + 1) % STAGES], 0, KH);
-                    TEXTRACT(bHi, bMat[(s + 1) % STAGES], KH, 0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    }
-    GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
-    TSTORE(dstGlobal, cTile);
-}
-
 // One wave per SIMD needs every issue slot: a wave that is stalled issuing its asynchronous copies
 // (the compute unit's single vector-memory front end takes 16 cycles per 1 KiB instruction) cannot
 // issue MFMAs meanwhile.  This kernel therefore (a) keeps the whole steady-state K-step in one
@@ -298,7 +190,8 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
 // one copy instruction per two MFMAs, then one fragment read per two MFMAs.
 template <int BM, int BN, int STAGES, int GROUP_M>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE
-    void GemmF16F32Mix(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k)
+    void GemmF16F32Mix(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
+                       int fullTiles, int splitK)
 {
     constexpr int BK = 32, KH = 16;
     using TileMatA = Tile<TileType::Mat, half, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
@@ -323,10 +216,26 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     constexpr int kReadsPerHalf = LeftTile::Storage::MB + RightTile::Storage::NB;
     static_assert(STAGES >= 3, "needs at least three L1 stages");
 
-    int tm, tn;
-    TileOfBlock<GROUP_M>((int)get_block_idx(), m / BM, n / BN, tm, tn);
-    __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)tm * BM * k;
-    __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)tn * BN * k;
+    // Work split.  The first `fullTiles` workgroups (whole rounds over the compute units) own one C
+    // tile each and the full K range.  The tiles of the last, partial round are cut into `splitK`
+    // K-ranges, one workgroup each, so that the round fills the machine; their partial products are
+    // added into a zeroed C tile with TSTORE<AtomicAdd>.
+    const int tilesM = m / BM, tilesN = n / BN;
+    const int block = (int)get_block_idx();
+    int tm, tn, kFirst = 0, kLoop = k / BK;
+    bool partial = false;
+    if (block < fullTiles) {
+        TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
+    } else {
+        const int tailUnits = (tilesM * tilesN - fullTiles) * splitK;
+        const int u = RegroupXcd(block - fullTiles, tailUnits);
+        TileOfId<GROUP_M>(fullTiles + u / splitK, tilesM, tilesN, tm, tn);
+        kLoop /= splitK;
+        kFirst = (u % splitK) * kLoop;
+        partial = splitK > 1;
+    }
+    __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)tm * BM * k + (int64_t)kFirst * BK;
+    __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)tn * BN * k + (int64_t)kFirst * BK;
     const StrideA strideA(m, k);
     const StrideB strideB(k, n);
 
@@ -348,7 +257,7 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
             for (int i = 0; i < 16; ++i)
                 cTile.st.f[mb][nb][i] = 0.0f;
 
-    const int kLoop = k / BK; // the host guarantees kLoop >= STAGES
+    // the host guarantees kLoop % STAGES == 0 and kLoop >= 2 * STAGES
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) {
         GlobalA gmA(aPanel + (int64_t)s * BK, ShapeA(), strideA);
@@ -399,7 +308,7 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         __builtin_amdgcn_sched_barrier(0);
     };
     using std::integral_constant;
-    for (int it = 0; it < kLoop; it += STAGES) { // the host guarantees kLoop % STAGES == 0
+    for (int it = 0; it < kLoop; it += STAGES) {
         step(integral_constant<int, 0>(), it);
         step(integral_constant<int, 1>(), it + 1);
         step(integral_constant<int, 2>(), it + 2);
@@ -407,7 +316,32 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
             step(integral_constant<int, 3>(), it + 3);
     }
     GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
-    TSTORE(dstGlobal, cTile);
+    if (partial)
+        TSTORE<ResTile, GlobalC, AtomicType::AtomicAdd>(dstGlobal, cTile);
+    else
+        TSTORE(dstGlobal, cTile);
+}
+
+// Clears the C tiles that GemmF16F32Mix accumulates into with atomic adds (tile ids >= fullTiles).
+template <int BM, int BN, int GROUP_M>
+__global__ __launch_bounds__(kBlockThreads, 1) AICORE void GemmZeroTailTiles(__gm__ float *out, int m, int n, int fullTiles)
+{
+    using ResTile = TileAcc<float, BM, BN, BM, BN>;
+    using ShapeC = TileShape2D<float, BM, BN, Layout::ND>;
+    using StrideC = BaseShape2D<float, DYNAMIC, DYNAMIC, Layout::ND>;
+    using GlobalC = GlobalTensor<float, ShapeC, StrideC, Layout::ND>;
+    int tm, tn;
+    TileOfId<GROUP_M>(fullTiles + (int)get_block_idx(), m / BM, n / BN, tm, tn);
+    ResTile zero;
+#pragma unroll
+    for (int mb = 0; mb < ResTile::Storage::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < ResTile::Storage::NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                zero.st.f[mb][nb][i] = 0.0f;
+    GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
+    TSTORE(dstGlobal, zero);
 }
 
 } // namespace
@@ -432,8 +366,44 @@ int launch_gemm(hipStream_t st, float *c, const half *a, const half *b, int m, i
 } // namespace
 
 namespace {
+// Number of K-ranges to cut the tiles of the last partial round into: the candidate that
+// minimises ceil(rem * S / cus) / S, the length of that round in units of one full tile.
+inline int choose_split_k(int rem, int cus, int kLoop, int stages)
+{
+    if (rem == 0)
+        return 1;
+    int best = 1;
+    double bestSpan = (double)((rem + cus - 1) / cus);
+    const int cand[] = {2, 3, 4, 6, 8};
+    for (int s : cand) {
+        if (kLoop % (s * stages) != 0 || kLoop / s < 2 * stages)
+            continue;
+        const double span = (double)((rem * s + cus - 1) / cus) / s;
+        if (span < bestSpan - 1e-9) {
+            bestSpan = span;
+            best = s;
+        }
+    }
+    return best;
+}
+
+inline int compute_units()
+{
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        return n;
+    }();
+    return cus;
+}
+
+// splitMode: 0 = never split K; 1 = split the last partial round when it is short (at most a
+// quarter of the compute units busy) and at least one full round precedes it: the fp32 atomic
+// adds of the split cost more than they save otherwise
 template <int BM, int BN, int STAGES, int GROUP_M>
-int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k)
+int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k, int splitMode = 1)
 {
     static_assert(STAGES == 3 || STAGES == 4, "three or four L1 stages");
     if (m % BM || n % BN || k % (32 * STAGES) || k / 32 < 2 * STAGES)
@@ -443,24 +413,19 @@ int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int 
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
-    const int blocks = (m / BM) * (n / BN);
-    kernel<<<dim3(blocks), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k);
+    const int tiles = (m / BM) * (n / BN), cus = compute_units();
+    int full = tiles / cus * cus;
+    int splitK = 1;
+    if (splitMode == 2 || (splitMode == 1 && full > 0 && (tiles - full) * 4 <= cus))
+        splitK = choose_split_k(tiles - full, cus, k / 32, STAGES);
+    if (splitK == 1)
+        full = tiles;
+    const int tail = tiles - full;
+    if (tail > 0)
+        GemmZeroTailTiles<BM, BN, GROUP_M><<<dim3(tail), dim3(kBlockThreads), 0, st>>>(c, m, n, full);
+    kernel<<<dim3(full + tail * splitK), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k, full, splitK);
     return pto_amd::check_launch();
 }
 
-template <int BM, int BN, int STAGES, int GROUP_M>
-int launch_gemm_deep(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k)
-{
-    if (m % BM || n % BN || k % 32)
-        return PTO_ERR_UNSUPPORTED;
-    constexpr int lds = STAGES * (BM * 32 + 32 * BN) * (int)sizeof(half);
-    auto kernel = GemmF16F32Deep<BM, BN, STAGES, GROUP_M>;
-    static const int attr = pto_amd::allow_lds(kernel, lds);
-    if (attr != PTO_OK)
-        return attr;
-    const int blocks = (m / BM) * (n / BN);
-    kernel<<<dim3(blocks), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k);
-    return pto_amd::check_launch();
-}
 } // namespace
 

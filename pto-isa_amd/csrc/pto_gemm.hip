@@ -32,16 +32,14 @@ extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a
     case 9: return launch_gemm<256, 256, 32, 3, 1, 8>(st, c, ha, hb, m, n, k);
     case 10: return launch_gemm<256, 256, 32, 4, 1, 4>(st, c, ha, hb, m, n, k);
     case 11: return launch_gemm<256, 256, 32, 2, 1, 8>(st, c, ha, hb, m, n, k);
-    case 20: return launch_gemm_deep<256, 256, 4, 8>(st, c, ha, hb, m, n, k);
-    case 21: return launch_gemm_deep<256, 256, 3, 8>(st, c, ha, hb, m, n, k);
-    case 22: return launch_gemm_deep<256, 256, 4, 4>(st, c, ha, hb, m, n, k);
-    case 23: return launch_gemm_deep<128, 256, 4, 8>(st, c, ha, hb, m, n, k);
     case 108: return launch_gemm<256, 256, 64, 2, 1, 8, 3>(st, c, ha, hb, m, n, k); // timestamps
     case 107: return launch_gemm<256, 256, 32, 4, 1, 8, 3>(st, c, ha, hb, m, n, k); // timestamps
     case 109: return launch_gemm<256, 256, 64, 2, 1, 8, 4>(st, c, ha, hb, m, n, k); // per-block stamps
-    case 30: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k);
-    case 31: return launch_gemm_mix<256, 256, 3, 8>(st, c, ha, hb, m, n, k);
-    case 32: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k);
+    case 30: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 2);
+    case 31: return launch_gemm_mix<256, 256, 3, 8>(st, c, ha, hb, m, n, k, 2);
+    case 32: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 2);
+    case 33: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 0);
+    case 34: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 0);
     case 103: return launch_gemm<256, 256, 32, 4, 1, 8, 1>(st, c, ha, hb, m, n, k); // loads only
     case 104: return launch_gemm<256, 256, 32, 4, 1, 8, 2>(st, c, ha, hb, m, n, k); // compute only
     case 101: return launch_gemm<128, 256, 32, 3, 2, 8, 1>(st, c, ha, hb, m, n, k); // loads only
@@ -52,5 +50,17 @@ extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a
 
 extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k)
 {
-    return pto_gemm_f16f32_variant(stream, c, a, b, m, n, k, 2);
+    if (!c || !a || !b || m <= 0 || n <= 0 || k <= 0)
+        return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
+    // Large problems: 256 x 256 C tiles (half the operand traffic per flop of the 128 x 256 block), one
+    // workgroup per compute unit.  Problems with too few such tiles to fill the machine, or with
+    // extents that are not multiples of them: the 128 x 256 block of the reference kernel, two
+    // workgroups per compute unit.
+    const bool big = m % 256 == 0 && n % 256 == 0 && k % 128 == 0 && k / 32 >= 8 &&
+                     (long long)(m / 256) * (n / 256) * 2 >= compute_units();
+    if (big)
+        return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 1);
+    return launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
 }

@@ -16,7 +16,8 @@ def rel_err(got, want):
     return float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
 
 
-@pytest.mark.parametrize("m,n,k", [(128, 256, 64), (128, 256, 128), (256, 512, 256), (384, 256, 1024)])
+@pytest.mark.parametrize("m,n,k", [(128, 256, 32), (128, 256, 64), (128, 256, 96), (256, 512, 256), (384, 256, 1024),
+                                   (4096, 4096, 256), (4096, 4352, 384), (4352, 4096, 128)])
 def test_gemm_small_vs_oracle(oracle, m, n, k):
     from gpu_util import gemm
     a, b = datagen.gemm_inputs(m, n, k)
@@ -26,6 +27,20 @@ def test_gemm_small_vs_oracle(oracle, m, n, k):
     # element-wise relative error where the reference is not tiny
     big = np.abs(want) > 0.05 * np.max(np.abs(want))
     assert np.max(np.abs(got - want)[big] / np.abs(want)[big]) <= TOL
+
+
+def test_gemm_both_kernels_agree_with_integer_reference():
+    """4096 x 4096 selects the 256 x 256-tile kernel (one full round), 4096 x 4352 the same kernel with a
+    K-split last round (atomic adds), 1024 x 1024 the 128 x 256-block kernel: all exact on integer inputs."""
+    from gpu_util import gemm
+    for m, n, k in ((4096, 4096, 512), (4096, 4352, 512), (1024, 1024, 512)):
+        a, b = datagen.gemm_inputs_integer(m, n, k)
+        got = gemm(a, b)
+        rows = np.r_[0:64, m // 2:m // 2 + 64, m - 64:m]
+        want = (a[rows].astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
+        assert np.array_equal(got[rows], want), (m, n, k)
+        colsum = b.astype(np.float64).sum(axis=0)
+        assert np.array_equal(got.astype(np.float64).sum(axis=1), a.astype(np.float64) @ colsum)
 
 
 def test_gemm_integer_inputs_exact(oracle):
@@ -87,6 +102,6 @@ def test_gemm_rejects_bad_shapes():
     t = torch.zeros(16, device="cuda:0")
     p = t.data_ptr()
     assert lib.pto_gemm_f16f32(0, p, p, p, 100, 256, 64) == capi.ERR_UNSUPPORTED
-    assert lib.pto_gemm_f16f32(0, p, p, p, 128, 256, 32) == capi.ERR_UNSUPPORTED
+    assert lib.pto_gemm_f16f32(0, p, p, p, 128, 256, 16) == capi.ERR_UNSUPPORTED
     assert lib.pto_gemm_f16f32(0, 0, p, p, 128, 256, 64) == capi.ERR_BAD_ARG
     assert lib.pto_gemm_f16f32(0, p, p, p, 0, 256, 64) == capi.ERR_BAD_ARG
