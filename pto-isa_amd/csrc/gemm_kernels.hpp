@@ -86,9 +86,6 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
     ResTile cTile;
 
     const int kLoop = k / BK;
-    long long tStart = 0, tLoop = 0, tEnd = 0;
-    if (MODE == 4)
-        tStart = clock64();
     // prologue: STAGES-1 K-steps in flight
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s)
@@ -103,19 +100,13 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
 #pragma unroll
         for (int s = 0; s < STAGES; ++s) { // unrolled over the LDS stages: stage indices are constants
             const int it = kIter + s;
-            auto stamp = [&](int point) {
-                if (MODE == 3 && get_block_idx() == 0 && hw::tid() == 0 && it < 64)
-                    reinterpret_cast<long long *>(out)[4096 + it * 8 + point] = clock64();
-            };
             if (it < kLoop) {
-                stamp(0);
                 // K-step `it` has landed for every wave (the younger steps may still be in flight), and
                 // every wave is done reading the stage that the next TLOAD overwrites.
                 if (it + STAGES - 2 < kLoop)
                     wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, static_cast<event_t>(s));
                 else
                     wait_flag(PIPE_MTE2, PIPE_MTE1, static_cast<event_t>(s));
-                stamp(1);
                 const int nxt = it + STAGES - 1;
                 if (MODE != 2 && nxt < kLoop) {
                     const int ns = (s + STAGES - 1) % STAGES;
@@ -125,17 +116,9 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
                     TLOAD(bMat[ns], gmB);
                     set_flag(PIPE_MTE2, PIPE_MTE1, static_cast<event_t>(ns));
                 }
-                stamp(2);
                 if (MODE != 1 || it == 0) {
                     TEXTRACT(aTile, aMat[s], 0, 0);
                     TEXTRACT(bTile, bMat[s], 0, 0);
-                    if (MODE == 3) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        stamp(3);
-                        hw::wait_lgkm0();
-                        stamp(4);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
                     set_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
                     wait_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
                     if (it == 0)
@@ -143,43 +126,14 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
                     else
                         TMATMUL_ACC(cTile, cTile, aTile, bTile);
                     set_flag(PIPE_M, PIPE_MTE1, EVENT_ID0);
-                    if (MODE == 3) {
-                        __builtin_amdgcn_sched_barrier(0);
-                        stamp(5);
-                    }
                 }
             }
         }
-    }
-    if (MODE == 3)
-        return;
-    if (MODE == 4) {
-        __builtin_amdgcn_sched_barrier(0);
-        tLoop = clock64();
     }
     set_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
     wait_flag(PIPE_M, PIPE_FIX, EVENT_ID0);
     GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
     TSTORE(dstGlobal, cTile);
-    if (MODE == 4) {
-        hw::wait_vm0();
-        __builtin_amdgcn_sched_barrier(0);
-        tEnd = clock64();
-        if (hw::tid() == 0) {
-            long long *dbg = reinterpret_cast<long long *>(out + (int64_t)m * n) + get_block_idx() * 8;
-            dbg[0] = tStart;
-            dbg[1] = tLoop;
-            dbg[2] = tEnd;
-            dbg[3] = (long long)wall_clock64();
-            dbg[4] = tm * 1000 + tn;
-            unsigned xcc = 0;
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-            dbg[5] = xcc;
-            unsigned hwid = 0;
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-            dbg[6] = hwid;
-        }
-    }
 }
 
 // One wave per SIMD needs every issue slot: a wave that is stalled issuing its asynchronous copies
@@ -315,6 +269,7 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         if constexpr (STAGES == 4)
             step(integral_constant<int, 3>(), it + 3);
     }
+    hw::wait_vm0(); // the copies issued past the end of K must not outlive the workgroup's LDS
     GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
     if (partial)
         TSTORE<ResTile, GlobalC, AtomicType::AtomicAdd>(dstGlobal, cTile);

@@ -31,8 +31,8 @@ PTO_DEVICE_CODE_BEGIN
 
 namespace {
 
-constexpr int kBQ = 128; // queries per workgroup (4 waves x 32)
-constexpr int kBKV = 64; // keys per tile
+constexpr int kBQ1 = 128; // queries per workgroup and 32-query block per wave (4 waves x 32)
+constexpr int kBKVDefault = 64; // keys per tile
 constexpr float kMaskValue = -3.40282e+38f; // pto_macro_fa_softmax.hpp:67
 
 // exchange a value with the lane 32 positions away
@@ -44,7 +44,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 // V tile, taken straight from the row-major [keys, D] LDS image with transposing reads.  Key order
 // inside every 16-key MFMA step matches the order in which the accumulator layout holds P^T:
 // k slot j of half-wave h  <->  key 16t + 8(j/4) + 4h + j%4.
-template <typename LeftT, typename MatT>
+template <int kBKV, typename LeftT, typename MatT>
 AICORE inline void ExtractVT(LeftT &dst, MatT &vMat, int db)
 {
     using Geo = detail::MatGeom<MatT>;
@@ -70,13 +70,14 @@ AICORE inline void ExtractVT(LeftT &dst, MatT &vMat, int db)
     }
 }
 
-template <int D, bool CAUSAL, bool OUT_F32>
-__global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
+template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int NQ, int kBKV = kBKVDefault>
+__global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
                                                                       __gm__ const half *qAll, __gm__ const half *kAll,
                                                                       __gm__ const half *vAll, int heads, int seqQ,
                                                                       int seqKv, int numBH)
 {
-    constexpr int KB = kBKV / 32; // 32-key blocks per tile
+    constexpr int kBQ = kBQ1 * NQ; // every wave owns NQ blocks of 32 queries
+    constexpr int KB = kBKV / 32;  // 32-key blocks per tile
     constexpr int DB = D / 32;    // 32-wide blocks of the head dimension
     // ---- tiles ----
     using TileMatQ = Tile<TileType::Mat, half, D, kBQ, BLayout::RowMajor, D, kBQ, SLayout::ColMajor>;   // Q^T, contiguous along d
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void
 
     constexpr uint32_t kTileBytes = kBKV * D * sizeof(half);
     constexpr uint32_t kStageBytes = 2 * kTileBytes;
-    static_assert(D * kBQ * sizeof(half) <= kStageBytes, "Q^T staging reuses the second K/V stage");
+    static_assert(D * kBQ * sizeof(half) <= 2 * kStageBytes, "Q^T is staged in the K/V stages");
 
     // ---- which (batch*head, query tile) this workgroup owns.  Workgroups are dealt round-robin to
     // the 8 XCDs: keep a head on one XCD so that its K/V stay in that XCD's L2.  Causal: the query
@@ -134,28 +135,30 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void
     TASSIGN(vMat[0], kTileBytes);
     TASSIGN(kMat[1], kStageBytes);
     TASSIGN(vMat[1], kStageBytes + kTileBytes);
-    TASSIGN(qMat, kStageBytes); // lives in stage 1 until it has been extracted
+    TASSIGN(qMat, 0u); // staged over both K/V stages until it has been extracted
 
     RightQ qRight;
     AccO oAcc[DB];
-    float runMax = 0.0f, runSum = 0.0f; // per lane: this lane's query; runSum is the half-wave partial
+    float runMax[NQ], runSum[NQ]; // per lane and query block; runSum is the half-wave partial
     const int lane = hw::lane();
-    const int myQuery = q0 + hw::wave_n() * 32 + (lane & 31); // row of Q this lane's column holds
+    // row of Q that this lane's column of query block 0 holds (block nb: + 32 nb)
+    const int myQuery = q0 + hw::wave_n() * (32 * NQ) + (lane & 31);
     const uint32_t hHalf = (uint32_t)lane >> 5;
     // s = 1/sqrt(D) folded with log2(e): exp(s y) = exp2(s log2e y)
     const float sLog2e = (D == 128 ? 0.08838834764831845f : 0.125f) * 1.4426950408889634f;
 
     {
         GlobalQT gmQ(qBase);
-        GlobalKV gmK(kBase), gmV(vBase);
         TLOAD(qMat, gmQ);
-        TLOAD(kMat[0], gmK);
-        TLOAD(vMat[0], gmV);
         set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
         wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
         TEXTRACT(qRight, qMat, 0, 0);
         set_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1);
-        wait_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1); // Q^T is in registers everywhere: stage 1 may be overwritten
+        wait_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1); // Q^T is in registers everywhere: the stages may be filled
+        GlobalKV gmK(kBase), gmV(vBase);
+        TLOAD(kMat[0], gmK);
+        TLOAD(vMat[0], gmV);
+        set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
     }
 
     for (int tile = 0; tile < numTiles; tile += 2) {
@@ -164,15 +167,17 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void
             const int t = tile + st;
             if (t >= numTiles)
                 break;
-            if (t > 0)
-                wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
-            if (t + 1 < numTiles) {
-                GlobalKV gmK(kBase + (int64_t)(t + 1) * kBKV * D), gmV(vBase + (int64_t)(t + 1) * kBKV * D);
+            wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
+            // The next tile is fetched while this tile's score MFMAs issue: one asynchronous copy per
+            // two MFMAs, so that the wave never sits in the vector-memory issue queue.  Past the last
+            // tile the copy re-fetches it into the free stage, which keeps this a straight-line region.
+            {
+                const int tn = t + 1 < numTiles ? t + 1 : t;
+                GlobalKV gmK(kBase + (int64_t)tn * kBKV * D), gmV(vBase + (int64_t)tn * kBKV * D);
                 TLOAD(kMat[st ^ 1], gmK);
                 TLOAD(vMat[st ^ 1], gmV);
                 set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
             }
-
             // ---- X^T = K Q^T ----
             AccS sAcc[KB];
 #pragma unroll
@@ -181,89 +186,122 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void
                 TEXTRACT(kLeft, kMat[st], kb * 32, 0);
                 TMATMUL(sAcc[kb], kLeft, qRight);
             }
+            {
+                constexpr int kCopies = TLoadInstrs<TileMatK>() + TLoadInstrs<TileMatV>();
+                constexpr int kMfma = KB * NQ * (D / 16);
+                constexpr int kPer = kMfma / kCopies > 0 ? kMfma / kCopies : 1;
+#pragma unroll
+                for (int i = 0; i < kCopies; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+                }
+            }
 
-            // ---- streaming softmax on the accumulator fragments (one query per lane) ----
+            // ---- streaming softmax on the accumulator fragments (one query per lane and query block) ----
             const int key0 = t * kBKV;
             if (CAUSAL && key0 + kBKV - 1 > q0 + causalOff) { // the diagonal crosses this tile
-                const int limit = myQuery + causalOff;        // last visible key of this lane's query
+#pragma unroll
+                for (int nb = 0; nb < NQ; ++nb) {
+                    const int limit = myQuery + 32 * nb + causalOff; // last visible key of this lane's query
+#pragma unroll
+                    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = key0 + kb * 32 + (v >> 2) * 8 + (int)hHalf * 4 + (v & 3);
+                            if (key > limit)
+                                sAcc[kb].st.f[0][nb][v] += kMaskValue;
+                        }
+                }
+            }
+            RightP pRight;
+            float alpha[NQ];
+            bool anyRaise = t == 0;
+#pragma unroll
+            for (int nb = 0; nb < NQ; ++nb) {
+                float locMax = sAcc[0].st.f[0][nb][0];
 #pragma unroll
                 for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int key = key0 + kb * 32 + (v >> 2) * 8 + (int)hHalf * 4 + (v & 3);
-                        if (key > limit)
-                            sAcc[kb].st.f[0][0][v] += kMaskValue;
+                    for (int v = 0; v < 16; ++v)
+                        locMax = fmaxf(locMax, sAcc[kb].st.f[0][nb][v]);
+                locMax = fmaxf(locMax, SwapHalves(locMax));
+                // The running max only has to bound the scores well enough to keep exp() in range: it is
+                // raised (and O, S rescaled by alpha) when a tile exceeds it by more than kSlack in the
+                // exponent, i.e. P stays below 2^kSlack.  O / S and max*s + ln(S) do not depend on the choice.
+                constexpr float kSlack = 8.0f;
+                const bool raise = t == 0 || (locMax - runMax[nb]) * sLog2e > kSlack;
+                const float newMax = raise ? locMax : runMax[nb];
+                if (t > 0)
+                    anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
+                alpha[nb] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nb] - newMax) * sLog2e);
+                runMax[nb] = newMax;
+                const float negMax = -newMax * sLog2e;
+                float locSum = 0.0f;
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int half_ = 0; half_ < 2; ++half_) {
+                        f16x8 pk;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const float p =
+                                __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][nb][half_ * 8 + j], sLog2e, negMax));
+                            locSum += p; // row sum over the fp32 P, as the reference does
+                            pk[j] = (half)p;
+                        }
+                        pRight.st.f[nb][kb * 2 + half_] = pk;
                     }
+                runSum[nb] = t == 0 ? locSum : runSum[nb] * alpha[nb] + locSum;
             }
-            float locMax = sAcc[0].st.f[0][0][0];
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    locMax = fmaxf(locMax, sAcc[kb].st.f[0][0][v]);
-            locMax = fmaxf(locMax, SwapHalves(locMax));
-            const float newMax = t == 0 ? locMax : fmaxf(runMax, locMax);
-            const float alpha = t == 0 ? 1.0f : __builtin_amdgcn_exp2f((runMax - newMax) * sLog2e);
-            runMax = newMax;
-            const float negMax = -newMax * sLog2e;
-            float locSum = 0.0f;
-            RightP pRight;
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int half_ = 0; half_ < 2; ++half_) {
-                    f16x8 pk;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][0][half_ * 8 + j], sLog2e, negMax));
-                        locSum += p; // row sum over the fp32 P, as the reference does
-                        pk[j] = (half)p;
-                    }
-                    pRight.st.f[0][kb * 2 + half_] = pk;
-                }
-            runSum = t == 0 ? locSum : runSum * alpha + locSum;
 
             // ---- O^T = alpha O^T + V^T P^T ----
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 LeftVT vLeft;
-                ExtractVT(vLeft, vMat[st], db);
+                ExtractVT<kBKV>(vLeft, vMat[st], db);
                 if (t == 0) {
                     TMATMUL(oAcc[db], vLeft, pRight);
                 } else {
+                    if (anyRaise) { // wave-uniform: some lane's max was raised
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        oAcc[db].st.f[0][0][v] *= alpha;
+                        for (int nb = 0; nb < NQ; ++nb)
+#pragma unroll
+                            for (int v = 0; v < 16; ++v)
+                                oAcc[db].st.f[0][nb][v] *= alpha[nb];
+                    }
                     TMATMUL_ACC(oAcc[db], oAcc[db], vLeft, pRight);
                 }
             }
         }
     }
-
+    hw::wait_vm0(); // the copy issued by the last tile must not outlive the workgroup's LDS
     // ---- finish: O /= S, write O (and LSE) ----
-    const float total = runSum + SwapHalves(runSum);
-    const float inv = 1.0f / total;
-    const int64_t row = (int64_t)bh * seqQ + myQuery;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int nb = 0; nb < NQ; ++nb) {
+        const float total = runSum[nb] + SwapHalves(runSum[nb]);
+        const float inv = 1.0f / total;
+        const int64_t row = (int64_t)bh * seqQ + myQuery + 32 * nb;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int d = db * 32 + g * 8 + (int)hHalf * 4;
-            float o4[4];
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-                o4[r] = oAcc[db].st.f[0][0][g * 4 + r] * inv;
-            if constexpr (OUT_F32) {
-                f32x4 v = {o4[0], o4[1], o4[2], o4[3]};
-                *reinterpret_cast<f32x4 *>(static_cast<float *>(outO) + row * D + d) = v;
-            } else {
-                f16x4 v = {(half)o4[0], (half)o4[1], (half)o4[2], (half)o4[3]};
-                *reinterpret_cast<f16x4 *>(static_cast<half *>(outO) + row * D + d) = v;
+            for (int g = 0; g < 4; ++g) {
+                const int d = db * 32 + g * 8 + (int)hHalf * 4;
+                float o4[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    o4[r] = oAcc[db].st.f[0][nb][g * 4 + r] * inv;
+                if constexpr (OUT_F32) {
+                    f32x4 v = {o4[0], o4[1], o4[2], o4[3]};
+                    *reinterpret_cast<f32x4 *>(static_cast<float *>(outO) + row * D + d) = v;
+                } else {
+                    f16x4 v = {(half)o4[0], (half)o4[1], (half)o4[2], (half)o4[3]};
+                    *reinterpret_cast<f16x4 *>(static_cast<half *>(outO) + row * D + d) = v;
+                }
             }
+        if (outLse != nullptr && hHalf == 0) {
+            const float scale = D == 128 ? 0.08838834764831845f : 0.125f;
+            outLse[row] = runMax[nb] * scale + __builtin_logf(total);
         }
-    if (outLse != nullptr && hHalf == 0) {
-        const float scale = D == 128 ? 0.08838834764831845f : 0.125f;
-        outLse[row] = runMax * scale + __builtin_logf(total);
     }
 }
 
@@ -272,17 +310,20 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void FlashAttnFwd(__gm__ void
 PTO_DEVICE_CODE_END
 
 namespace {
-template <int D, bool CAUSAL, bool OUT_F32>
+template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS = 1, int NQ = 1, int kBKV = kBKVDefault>
 int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads,
               int seqQ, int seqKv)
 {
+    if (seqQ % (kBQ1 * NQ) || seqKv % kBKV)
+        return PTO_ERR_UNSUPPORTED;
+    static_assert(D * kBQ1 * NQ <= 4 * kBKV * D, "Q^T must fit the K/V stages it is staged in");
     constexpr int lds = 2 * 2 * kBKV * D * (int)sizeof(half);
-    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32>;
+    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32, MIN_BLOCKS, NQ, kBKV>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
     const int numBH = batch * heads;
-    const long long blocks = (long long)numBH * (seqQ / kBQ);
+    const long long blocks = (long long)numBH * (seqQ / (kBQ1 * NQ));
     if (blocks > 0x7fffffffLL)
         return PTO_ERR_UNSUPPORTED;
     kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH);
@@ -290,21 +331,49 @@ int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k,
 }
 } // namespace
 
+// Tuning hook (not part of the public header).
+extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k,
+                                      const uint16_t *v, int batch, int heads, int seq_q, int seq_kv, int head_dim,
+                                      int causal, int variant)
+{
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half *hq = reinterpret_cast<const half *>(q), *hk = reinterpret_cast<const half *>(k),
+               *hv = reinterpret_cast<const half *>(v);
+#define PTO_FA_VARIANT(VV, DD, CC, MB, NQ)                       \
+    if (variant == VV && head_dim == DD && (causal != 0) == CC) \
+        return launch_fa<DD, CC, false, MB, NQ>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+    PTO_FA_VARIANT(1, 128, false, 1, 1)
+    PTO_FA_VARIANT(2, 128, false, 2, 1)
+    PTO_FA_VARIANT(3, 128, false, 1, 2)
+    PTO_FA_VARIANT(1, 64, true, 1, 1)
+    PTO_FA_VARIANT(2, 64, true, 2, 1)
+    PTO_FA_VARIANT(3, 64, true, 1, 2)
+    PTO_FA_VARIANT(4, 64, true, 2, 2)
+    PTO_FA_VARIANT(5, 64, true, 3, 1)
+#undef PTO_FA_VARIANT
+    if (variant == 6 && head_dim == 128 && !causal)
+        return launch_fa<128, false, false, 2, 1, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+    if (variant == 6 && head_dim == 64 && causal)
+        return launch_fa<64, true, false, 3, 1, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+    return PTO_ERR_BAD_ARG;
+}
+
 extern "C" int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,
                               int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int o_fp32)
 {
     if (!o || !q || !k || !v || batch <= 0 || heads <= 0 || seq_q <= 0 || seq_kv <= 0)
         return PTO_ERR_BAD_ARG;
-    if ((head_dim != 64 && head_dim != 128) || seq_q % kBQ || seq_kv % kBKV)
+    if ((head_dim != 64 && head_dim != 128) || seq_q % kBQ1 || seq_kv % kBKVDefault)
         return PTO_ERR_UNSUPPORTED;
     if (causal && seq_kv < seq_q)
         return PTO_ERR_UNSUPPORTED;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *hq = reinterpret_cast<const half *>(q), *hk = reinterpret_cast<const half *>(k),
                *hv = reinterpret_cast<const half *>(v);
+    // two workgroups per compute unit at head_dim 128, three at 64 (register budget of the kernel)
 #define PTO_FA_CASE(DD, CC, FF)                                                                      \
     if (head_dim == DD && (causal != 0) == CC && (o_fp32 != 0) == FF)                                \
-        return launch_fa<DD, CC, FF>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+        return launch_fa<DD, CC, FF, (DD == 128 ? 2 : 3)>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
     PTO_FA_CASE(128, false, false)
     PTO_FA_CASE(128, false, true)
     PTO_FA_CASE(128, true, false)

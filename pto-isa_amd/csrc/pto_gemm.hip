@@ -32,9 +32,6 @@ extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a
     case 9: return launch_gemm<256, 256, 32, 3, 1, 8>(st, c, ha, hb, m, n, k);
     case 10: return launch_gemm<256, 256, 32, 4, 1, 4>(st, c, ha, hb, m, n, k);
     case 11: return launch_gemm<256, 256, 32, 2, 1, 8>(st, c, ha, hb, m, n, k);
-    case 108: return launch_gemm<256, 256, 64, 2, 1, 8, 3>(st, c, ha, hb, m, n, k); // timestamps
-    case 107: return launch_gemm<256, 256, 32, 4, 1, 8, 3>(st, c, ha, hb, m, n, k); // timestamps
-    case 109: return launch_gemm<256, 256, 64, 2, 1, 8, 4>(st, c, ha, hb, m, n, k); // per-block stamps
     case 30: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 2);
     case 31: return launch_gemm_mix<256, 256, 3, 8>(st, c, ha, hb, m, n, k, 2);
     case 32: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 2);
