@@ -148,6 +148,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="gemm | fa | tcvt | gather: time just that workload")
     ap.add_argument("--size", type=int, default=6144)
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy a few times (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU; --gpus %d is not supported (every workload of the metric "
@@ -160,6 +162,12 @@ def main():
     torch.cuda.set_device(0)
 
     extra = {}
+    if args.calib_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+        dst = torch.empty_like(src)
+        ms = time_launches(torch, lambda: dst.copy_(src), 5, 2)
+        extra["calib_copy_1GiB"] = {"ms": ms, "gbs": 2.0 * src.numel() * 4 / (ms * 1e-3) / 1e9, "bytes_read": src.numel() * 4,
+                                    "bytes_written": src.numel() * 4}
     only = args.only
     gemm = None
     if only in ("", "gemm"):
