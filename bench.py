@@ -210,7 +210,7 @@ def main():
     if gemm:
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                             "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": None,
-                            "kernel": "GemmF16F32Mix<256,256,4,4>", "flops_per_launch": gemm["flops"]}
+                            "kernel": "GemmF16F32Mix<256,256,4,4> (8 wavefronts per workgroup)", "flops_per_launch": gemm["flops"]}
     if not args.no_cpu and only in ("", "gemm"):
         line["cpu_baseline"] = cpu_baseline(datagen, args.size)
     print(json.dumps(line))

@@ -29,4 +29,7 @@ inline int allow_lds(K kernel, int bytes)
     }
     return PTO_OK;
 }
+
+// defined in pto_gemm_w8.hip (workgroups of eight wavefronts)
+int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
 } // namespace pto_amd

@@ -142,10 +142,10 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
 // straight-line region: TLOAD of stage i+STAGES-1, TMATMUL_ACC on the two 16-wide halves of stage i,
 // TEXTRACT of the halves of stage i+1, and (b) tells the instruction scheduler to interleave them:
 // one copy instruction per two MFMAs, then one fragment read per two MFMAs.
-template <int BM, int BN, int STAGES, int GROUP_M>
-__global__ __launch_bounds__(kBlockThreads, 1) AICORE
-    void GemmF16F32Mix(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
-                       int fullTiles, int splitK)
+// C[row0 : row0+BM, col0 : col0+BN] (+)= A[row0.., kFirst*32 ..] x B[col0.., kFirst*32 ..] over kLoop K-steps of 32.
+template <int BM, int BN, int STAGES>
+AICORE inline void MixTile(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
+                           int row0, int col0, int kFirst, int kLoop, bool partial)
 {
     constexpr int BK = 32, KH = 16;
     using TileMatA = Tile<TileType::Mat, half, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
@@ -170,26 +170,8 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     constexpr int kReadsPerHalf = LeftTile::Storage::MB + RightTile::Storage::NB;
     static_assert(STAGES >= 3, "needs at least three L1 stages");
 
-    // Work split.  The first `fullTiles` workgroups (whole rounds over the compute units) own one C
-    // tile each and the full K range.  The tiles of the last, partial round are cut into `splitK`
-    // K-ranges, one workgroup each, so that the round fills the machine; their partial products are
-    // added into a zeroed C tile with TSTORE<AtomicAdd>.
-    const int tilesM = m / BM, tilesN = n / BN;
-    const int block = (int)get_block_idx();
-    int tm, tn, kFirst = 0, kLoop = k / BK;
-    bool partial = false;
-    if (block < fullTiles) {
-        TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
-    } else {
-        const int tailUnits = (tilesM * tilesN - fullTiles) * splitK;
-        const int u = RegroupXcd(block - fullTiles, tailUnits);
-        TileOfId<GROUP_M>(fullTiles + u / splitK, tilesM, tilesN, tm, tn);
-        kLoop /= splitK;
-        kFirst = (u % splitK) * kLoop;
-        partial = splitK > 1;
-    }
-    __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)tm * BM * k + (int64_t)kFirst * BK;
-    __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)tn * BN * k + (int64_t)kFirst * BK;
+    __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)row0 * k + (int64_t)kFirst * BK;
+    __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)col0 * k + (int64_t)kFirst * BK;
     const StrideA strideA(m, k);
     const StrideB strideB(k, n);
 
@@ -270,11 +252,41 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
             step(integral_constant<int, 3>(), it + 3);
     }
     hw::wait_vm0(); // the copies issued past the end of K must not outlive the workgroup's LDS
-    GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
+    GlobalC dstGlobal(out + (int64_t)row0 * n + col0, ShapeC(), StrideC(m, n));
     if (partial)
         TSTORE<ResTile, GlobalC, AtomicType::AtomicAdd>(dstGlobal, cTile);
     else
         TSTORE(dstGlobal, cTile);
+}
+
+// Work split of the kernel below.  The first `fullTiles` workgroups (whole rounds over the compute
+// units) own one BM x BN C tile each.  The tiles of the last, partial round are divided so that the
+// round fills the machine: tailMode 1 = four (BM/2) x (BN/2) quarter tiles, one workgroup each;
+// tailMode 2 = `splitK` K-ranges per tile whose partial products are added into a zeroed C tile
+// with TSTORE<AtomicAdd> (slow: one atomic per element).
+template <int BM, int BN, int STAGES, int GROUP_M>
+__global__ __launch_bounds__(kBlockThreads, 1) AICORE
+    void GemmF16F32Mix(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
+                       int fullTiles, int tailMode, int splitK)
+{
+    const int tilesM = m / BM, tilesN = n / BN;
+    const int block = (int)get_block_idx();
+    int tm, tn;
+    if (block < fullTiles) {
+        TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
+        MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, 0, k / 32, false);
+    } else if (tailMode == 1) {
+        const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
+        TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
+        const int sub = u % 4;
+        MixTile<BM / 2, BN / 2, STAGES>(out, src0, src1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
+                                        tn * BN + (sub & 1) * (BN / 2), 0, k / 32, false);
+    } else {
+        const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * splitK);
+        TileOfId<GROUP_M>(fullTiles + u / splitK, tilesM, tilesN, tm, tn);
+        const int kLoop = k / 32 / splitK;
+        MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, (u % splitK) * kLoop, kLoop, splitK > 1);
+    }
 }
 
 // Clears the C tiles that GemmF16F32Mix accumulates into with atomic adds (tile ids >= fullTiles).
@@ -354,11 +366,12 @@ inline int compute_units()
     return cus;
 }
 
-// splitMode: 0 = never split K; 1 = split the last partial round when it is short (at most a
-// quarter of the compute units busy) and at least one full round precedes it: the fp32 atomic
-// adds of the split cost more than they save otherwise
+// tailMode: 0 = whole tiles only; 1 = quarter tiles in the last partial round when they fit one round
+// (the quarter tiles move twice the operand bytes per flop, so two rounds of them cost more than the
+// idle compute units of a partial round); 2 = K-split with atomic adds (tuning hook only); 3 = quarter
+// tiles whenever there is a partial round (tuning hook only)
 template <int BM, int BN, int STAGES, int GROUP_M>
-int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k, int splitMode = 1)
+int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k, int tailMode = 1)
 {
     static_assert(STAGES == 3 || STAGES == 4, "three or four L1 stages");
     if (m % BM || n % BN || k % (32 * STAGES) || k / 32 < 2 * STAGES)
@@ -371,14 +384,19 @@ int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int 
     const int tiles = (m / BM) * (n / BN), cus = compute_units();
     int full = tiles / cus * cus;
     int splitK = 1;
-    if (splitMode == 2 || (splitMode == 1 && full > 0 && (tiles - full) * 4 <= cus))
+    if (tailMode == 1 && (full == 0 || (tiles - full) * 4 > cus))
+        tailMode = 0;
+    if (tailMode == 3)
+        tailMode = 1;
+    if (tailMode == 2)
         splitK = choose_split_k(tiles - full, cus, k / 32, STAGES);
-    if (splitK == 1)
+    if (tailMode == 0 || (tailMode == 2 && splitK == 1))
         full = tiles;
     const int tail = tiles - full;
-    if (tail > 0)
+    if (tail > 0 && tailMode == 2)
         GemmZeroTailTiles<BM, BN, GROUP_M><<<dim3(tail), dim3(kBlockThreads), 0, st>>>(c, m, n, full);
-    kernel<<<dim3(full + tail * splitK), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k, full, splitK);
+    const int units = tailMode == 1 ? tail * 4 : tail * splitK;
+    kernel<<<dim3(full + units), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k, full, tailMode, splitK);
     return pto_amd::check_launch();
 }
 

@@ -36,7 +36,10 @@ extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a
     case 31: return launch_gemm_mix<256, 256, 3, 8>(st, c, ha, hb, m, n, k, 2);
     case 32: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 2);
     case 33: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 0);
+    case 35: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 3);
+    case 36: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 3);
     case 34: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 0);
+    case 105: return launch_gemm<256, 256, 64, 2, 1, 8, 1>(st, c, ha, hb, m, n, k); // loads only, 128-byte rows
     case 103: return launch_gemm<256, 256, 32, 4, 1, 8, 1>(st, c, ha, hb, m, n, k); // loads only
     case 104: return launch_gemm<256, 256, 32, 4, 1, 8, 2>(st, c, ha, hb, m, n, k); // compute only
     case 101: return launch_gemm<128, 256, 32, 3, 2, 8, 1>(st, c, ha, hb, m, n, k); // loads only
@@ -51,13 +54,13 @@ extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const 
         return PTO_ERR_BAD_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
-    // Large problems: 256 x 256 C tiles (half the operand traffic per flop of the 128 x 256 block), one
-    // workgroup per compute unit.  Problems with too few such tiles to fill the machine, or with
-    // extents that are not multiples of them: the 128 x 256 block of the reference kernel, two
-    // workgroups per compute unit.
+    // Large problems: 256 x 256 C tiles (two thirds of the operand traffic per flop of the 128 x 256
+    // block), one workgroup of eight wavefronts per compute unit.  Problems with too few such tiles
+    // to fill the machine, or with extents that are not multiples of them: the 128 x 256 block of
+    // the reference kernel, two workgroups of four wavefronts per compute unit.
     const bool big = m % 256 == 0 && n % 256 == 0 && k % 128 == 0 && k / 32 >= 8 &&
                      (long long)(m / 256) * (n / 256) * 2 >= compute_units();
     if (big)
-        return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 1);
+        return pto_amd::gemm_f16f32_tile256_w8(st, c, ha, hb, m, n, k);
     return launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
 }

@@ -4,6 +4,15 @@
 #define PTO_WAVES_N 4
 #include "gemm_kernels.hpp"
 
+namespace pto_amd {
+// 256 x 256 C tiles, eight wavefronts per workgroup (128 x 64 of C per wave): the default for large problems.
+int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k)
+{
+    return launch_gemm_mix<256, 256, 4, 4>(st, c, a, b, m, n, k, 1);
+}
+int gemm_compute_units() { return compute_units(); }
+} // namespace pto_amd
+
 extern "C" int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
                                           int variant)
 {
@@ -18,6 +27,9 @@ extern "C" int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t
     case 3: return launch_gemm<256, 256, 32, 4, 1, 4>(st, c, ha, hb, m, n, k);
     case 4: return launch_gemm<256, 256, 32, 2, 1, 8>(st, c, ha, hb, m, n, k);
     case 5: return launch_gemm<128, 256, 32, 4, 1, 8>(st, c, ha, hb, m, n, k);
+    case 30: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 1);
+    case 31: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 1);
+    case 32: return launch_gemm_mix<256, 256, 3, 4>(st, c, ha, hb, m, n, k, 1);
     default: return PTO_ERR_BAD_ARG;
     }
 }

@@ -31,7 +31,7 @@ def test_gemm_small_vs_oracle(oracle, m, n, k):
 
 def test_gemm_both_kernels_agree_with_integer_reference():
     """4096 x 4096 selects the 256 x 256-tile kernel (one full round), 4096 x 4352 the same kernel with a
-    K-split last round (atomic adds), 1024 x 1024 the 128 x 256-block kernel: all exact on integer inputs."""
+    last round of 128 x 128 quarter tiles, 1024 x 1024 the 128 x 256-block kernel: all exact on integer inputs."""
     from gpu_util import gemm
     for m, n, k in ((4096, 4096, 512), (4096, 4352, 512), (1024, 1024, 512)):
         a, b = datagen.gemm_inputs_integer(m, n, k)
