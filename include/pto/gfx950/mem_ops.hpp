@@ -194,7 +194,8 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
             base = (int64_t)major * src.GetStride(4);
         if (vecOK && stMinor == 1 && major < vMajor && minor0 + kVecChunk <= vMinor) {
             // 8 contiguous elements: one or two 16-byte loads
-            using VT = T __attribute__((ext_vector_type(kVecChunk)));
+            // element-aligned only: rows of a strided view need not start on a 16-byte boundary
+            typedef T VT __attribute__((ext_vector_type(kVecChunk), aligned(sizeof(T))));
             VT v = *reinterpret_cast<const VT *>(gm + base + minor0);
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
@@ -366,7 +367,7 @@ PTO_DEV void tstore_vec(G &dst, TileT &src)
         else
             base = (int64_t)major * dst.GetStride(4);
         if (Minor % kVecChunk == 0 && stMinor == 1 && major < vMajor && minor0 + kVecChunk <= vMinor) {
-            using VT = T __attribute__((ext_vector_type(kVecChunk)));
+            typedef T VT __attribute__((ext_vector_type(kVecChunk), aligned(sizeof(T))));
             VT v;
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)

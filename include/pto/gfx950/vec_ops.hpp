@@ -498,7 +498,7 @@ PTO_DEV void MGATHER_ROWS_IMPL(DstT &dst, G &table, IdxT &rowIdx, int tableRows)
     hw::lds_barrier();
     const T *gm = reinterpret_cast<const T *>(table.data());
     const int64_t ld = table.GetStride(3);
-    using VT = T __attribute__((ext_vector_type(detail::kVecChunk)));
+    typedef T VT __attribute__((ext_vector_type(detail::kVecChunk), aligned(sizeof(T))));
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
 #pragma unroll
     for (int s = 0; s < S::Slots; ++s) {

@@ -76,6 +76,43 @@ int pto_gather_rows(void *stream, void *out, const void *table, const int32_t *i
  * out-of-range -> 0.  src0 [16,1024] fp16, idx and dst [16,128]. */
 int pto_tgather_index_f16_16x1024_16x128(void *stream, uint16_t *dst, const uint16_t *src0, const int32_t *idx);
 
+/* ---- single-tile instruction programs -------------------------------------------------------
+ * One workgroup runs a short PTO program on one or a few tiles: the counterparts of the reference's
+ * per-instruction system-test kernels (tests/cpu/st/testcase/<op>/<op>_kernel.cpp), here so that
+ * every instruction of the path can be driven through the C ABI. */
+
+/* One streaming-softmax step on a [64,256] fp32 score tile (pto_macro_fa_softmax.hpp:82-97, 141-183).
+ * first != 0: max = rowmax(x), p = exp(scale (x - max)), sum = rowsum(p), alpha = 1.
+ * first == 0: max' = max(max_in, rowmax x), alpha = exp(scale (max_in - max')), p = exp(scale (x - max')),
+ *             sum' = alpha sum_in + rowsum(p).   x_exp = fp16(p) under round_mode.  Vectors are [64] fp32. */
+int pto_st_softmax_step_f32_64x256(void *stream, uint16_t *x_exp, float *max_out, float *sum_out, float *alpha_out,
+                                   const float *x, const float *max_in, const float *sum_in, float scale, int first,
+                                   int round_mode);
+/* Rescale-accumulate step on [64,128] fp32 tiles (pto_macro_fa_gu.hpp:33-56): o = o_prev alpha + pv; last: o /= sum. */
+int pto_st_gu_step_f32_64x128(void *stream, float *o_out, const float *o_prev, const float *pv, const float *alpha,
+                              const float *sum, int last);
+/* out = x + tri(diagonal) * value on a [64,128] fp32 tile; upper != 0: TTRI upper form (cpu/TTRI.hpp:31-63). */
+int pto_st_tri_mask_f32_64x128(void *stream, float *out, const float *x, int diagonal, float value, int upper);
+/* TGATHER mask form on a [16,64] tile of 16-bit elements -> [16, 64/div] (tgather_kernel.cpp:18-42); pattern 1..7. */
+int pto_st_tgather_mask_b16_16x64(void *stream, uint16_t *out, const uint16_t *src, int pattern);
+/* MGATHER element form: out[8,128] = gm[idx[8,128]] (tests/cpu/st/testcase/mgather). */
+int pto_st_mgather_b16_8x128(void *stream, uint16_t *out, const uint16_t *gm, const int32_t *idx, int gm_elems);
+/* TLOAD of a [10,20] fp32 region into a [16,32] tile with PadValue::Max; the whole tile image comes back
+ * (tload/main.cpp:138-183, PADMAX case). */
+int pto_st_tload_pad_f32_16x32(void *stream, float *image, const float *gm);
+/* TLOAD of the 5-D view shape [1,2,3,4,8], strides [1000,400,100,10,1] into a [24,8] tile; TSTORE to a dense
+ * [24,8] buffer and back through the same 5-D strides (tload/ and tstore/ 5-D cases). */
+int pto_st_tload_5d_f32(void *stream, float *dense, float *strided, const float *gm);
+/* TEXTRACT windows (docs/isa/TEXTRACT.md:14-18): out_left[128,256] = a[:, col0:col0+64] x eye,
+ * out_right[128,256] = eye x b[row0:row0+64, :].  a [128,256] fp16 row-major; b_t [256][256] (column-major b);
+ * eye_b [256][64] column-major 64 x 256 with eye(k,n) = (k == n); eye_a [128,64] with eye(r,k) = (r == k). */
+int pto_st_textract_windows_f16(void *stream, float *out_left, float *out_right, const uint16_t *a, const uint16_t *b_t,
+                                const uint16_t *eye_b, const uint16_t *eye_a, int col0, int row0);
+/* [128,64] x [64,256] (+ bias[256], may be NULL) with fp16 (bf16 == 0) or bf16 operands, stages ordered by Event
+ * objects (tmatmul_kernel.cpp:26-99 with isBias; docs/coding/Event.md). */
+int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, const float *bias,
+                                  int bf16);
+
 #ifdef __cplusplus
 }
 #endif

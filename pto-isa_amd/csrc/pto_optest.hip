@@ -1,0 +1,376 @@
+// Single-tile instruction kernels: one workgroup runs a short PTO program on one or a few tiles.
+// They are the counterpart of the reference's per-instruction system tests
+// (tests/cpu/st/testcase/<op>/<op>_kernel.cpp) and exist so that every instruction on the path
+// can be checked against the oracle through the C ABI.
+#include <pto/pto-inst.hpp>
+
+#include "common.hpp"
+
+using namespace pto;
+
+PTO_DEVICE_CODE_BEGIN
+
+namespace {
+
+template <typename T, int R, int C>
+using GmND = GlobalTensor<T, Shape<1, 1, 1, R, C>, Stride<R * C, R * C, R * C, C, 1>>;
+template <typename T, int R>
+using GmCol = GlobalTensor<T, Shape<1, 1, 1, R, 1>, Stride<R, R, R, 1, R>, Layout::DN>;
+
+// ---- streaming-softmax step on one [64, 256] fp32 score tile (stage a12 of the attention path) ----
+// first != 0: M = rowmax(X), P = exp(s (X - M)), S = rowsum(P)
+// else:       M' = max(M, rowmax X), alpha = exp(s (M - M')), P = exp(s (X - M')), S' = alpha S + rowsum(P)
+// x_exp = half(P) with RoundMode `mode`.
+constexpr int kSmRows = 64, kSmCols = 256;
+__global__ __launch_bounds__(kBlockThreads) AICORE void SoftmaxStep(__gm__ half *xExpOut, __gm__ float *maxOut,
+                                                                    __gm__ float *sumOut, __gm__ float *alphaOut,
+                                                                    __gm__ const float *xIn, __gm__ const float *maxIn,
+                                                                    __gm__ const float *sumIn, float scale, int first,
+                                                                    int mode)
+{
+    using TileX = Tile<TileType::Vec, float, kSmRows, kSmCols, BLayout::RowMajor>;
+    using TileH = Tile<TileType::Vec, half, kSmRows, kSmCols, BLayout::RowMajor>;
+    using TileR = Tile<TileType::Vec, float, kSmRows, 1, BLayout::ColMajor>;
+    using Tile1F = Tile<TileType::Vec, float, 1, kSmRows * kSmCols, BLayout::RowMajor>;
+    using Tile1H = Tile<TileType::Vec, half, 1, kSmRows * kSmCols, BLayout::RowMajor>;
+    TileX x, p;
+    TileH xExp;
+    TileR localMax, globalMax, expMax, localSum, globalSum;
+    GmND<float, kSmRows, kSmCols> gx(const_cast<float *>(xIn));
+    GmND<half, kSmRows, kSmCols> gxe(xExpOut);
+    GmCol<float, kSmRows> gMaxIn(const_cast<float *>(maxIn)), gSumIn(const_cast<float *>(sumIn)), gMaxOut(maxOut),
+        gSumOut(sumOut), gAlpha(alphaOut);
+    TLOAD(x, gx);
+    if (first) {
+        TROWMAX(globalMax, x, p);
+        TROWEXPANDSUB(p, x, globalMax);
+        TMULS(p, p, scale);
+        TEXP(p, p);
+        TROWSUM(globalSum, p, x);
+        TEXPANDS(expMax, 1.0f);
+    } else {
+        TLOAD(globalMax, gMaxIn);
+        TLOAD(globalSum, gSumIn);
+        TROWMAX(localMax, x, p);
+        TMAX(localMax, localMax, globalMax);   // M'
+        TSUB(expMax, globalMax, localMax);     // M - M'
+        TMULS(globalMax, localMax, 1.0f);      // M <- M'
+        TROWEXPANDSUB(p, x, localMax);
+        TMULS(expMax, expMax, scale);
+        TMULS(p, p, scale);
+        TEXP(expMax, expMax);
+        TEXP(p, p);
+        TMUL(globalSum, expMax, globalSum);
+        TROWSUM(localSum, p, x);
+        TADD(globalSum, globalSum, localSum);
+    }
+    Tile1F p1;
+    Tile1H xe1;
+    TRESHAPE(p1, p);
+    TCVT(xe1, p1, static_cast<RoundMode>(mode));
+    TRESHAPE(xExp, xe1);
+    TSTORE(gxe, xExp);
+    TSTORE(gMaxOut, globalMax);
+    TSTORE(gSumOut, globalSum);
+    TSTORE(gAlpha, expMax);
+}
+
+// ---- rescale-accumulate step (stage a13): O = O alpha + PV; last: O /= S ----
+constexpr int kGuRows = 64, kGuCols = 128;
+__global__ __launch_bounds__(kBlockThreads) AICORE void GuStep(__gm__ float *oOut, __gm__ const float *oPrev,
+                                                               __gm__ const float *pv, __gm__ const float *alpha,
+                                                               __gm__ const float *sum, int last)
+{
+    using TileO = Tile<TileType::Vec, float, kGuRows, kGuCols, BLayout::RowMajor>;
+    using TileR = Tile<TileType::Vec, float, kGuRows, 1, BLayout::ColMajor>;
+    TileO o, est;
+    TileR a, s;
+    GmND<float, kGuRows, kGuCols> gPrev(const_cast<float *>(oPrev)), gPv(const_cast<float *>(pv)), gOut(oOut);
+    GmCol<float, kGuRows> gA(const_cast<float *>(alpha)), gS(const_cast<float *>(sum));
+    TLOAD(o, gPrev);
+    TLOAD(est, gPv);
+    TLOAD(a, gA);
+    TLOAD(s, gS);
+    TROWEXPANDMUL(o, o, a);
+    TADD(o, o, est);
+    if (last)
+        TROWEXPANDDIV(o, o, s);
+    TSTORE(gOut, o);
+}
+
+// ---- TTRI + TADD mask: out = x + triu(diagonal) * value ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void TriMask(__gm__ float *out, __gm__ const float *xIn, int diagonal,
+                                                                float value, int upper)
+{
+    using TileX = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    TileX x, tri;
+    GmND<float, 64, 128> gx(const_cast<float *>(xIn)), go(out);
+    TLOAD(x, gx);
+    if (upper)
+        TTRI<TileX, 1>(tri, diagonal);
+    else
+        TTRI<TileX, 0>(tri, diagonal);
+    TMULS(tri, tri, value);
+    TADD(x, x, tri);
+    TSTORE(go, x);
+}
+
+// ---- mask-form TGATHER on a [16, 64] tile of 16-bit elements ----
+template <MaskPattern P, int DIV>
+AICORE inline void GatherMaskBody(__gm__ uint16_t *out, __gm__ const uint16_t *in)
+{
+    using Src = Tile<TileType::Vec, uint16_t, 16, 64, BLayout::RowMajor>;
+    using Dst = Tile<TileType::Vec, uint16_t, 16, 64 / DIV, BLayout::RowMajor>;
+    Src s;
+    Dst d;
+    GmND<uint16_t, 16, 64> gs(const_cast<uint16_t *>(in));
+    GmND<uint16_t, 16, 64 / DIV> gd(out);
+    TLOAD(s, gs);
+    TGATHER<Dst, Src, P>(d, s);
+    TSTORE(gd, d);
+}
+__global__ __launch_bounds__(kBlockThreads) AICORE void GatherMask(__gm__ uint16_t *out, __gm__ const uint16_t *in, int pattern)
+{
+    switch (pattern) {
+    case 1: GatherMaskBody<MaskPattern::P0101, 2>(out, in); break;
+    case 2: GatherMaskBody<MaskPattern::P1010, 2>(out, in); break;
+    case 3: GatherMaskBody<MaskPattern::P0001, 4>(out, in); break;
+    case 4: GatherMaskBody<MaskPattern::P0010, 4>(out, in); break;
+    case 5: GatherMaskBody<MaskPattern::P0100, 4>(out, in); break;
+    case 6: GatherMaskBody<MaskPattern::P1000, 4>(out, in); break;
+    default: GatherMaskBody<MaskPattern::P1111, 1>(out, in); break;
+    }
+}
+
+// ---- element-form MGATHER: dst[8,128] = gm[idx[8,128]] ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void MGatherElems(__gm__ uint16_t *out, __gm__ const uint16_t *gm,
+                                                                     __gm__ const int32_t *idx, int gmElems)
+{
+    using Dst = Tile<TileType::Vec, uint16_t, 8, 128, BLayout::RowMajor>;
+    using Idx = Tile<TileType::Vec, int32_t, 8, 128, BLayout::RowMajor>;
+    Dst d;
+    Idx ti;
+    GmND<int32_t, 8, 128> gi(const_cast<int32_t *>(idx));
+    GmND<uint16_t, 8, 128> gd(out);
+    GlobalTensor<uint16_t, Shape<1, 1, 1, 1, DYNAMIC>, Stride<1, 1, 1, DYNAMIC, 1>> gsrc(
+        const_cast<uint16_t *>(gm), Shape<1, 1, 1, 1, DYNAMIC>(gmElems), Stride<1, 1, 1, DYNAMIC, 1>(gmElems));
+    TLOAD(ti, gi);
+    MGATHER(d, gsrc, ti);
+    TSTORE(gd, d);
+}
+
+// ---- TLOAD with a valid region and PadValue::Max: the whole [16, 32] tile image comes back ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void LoadPadImage(__gm__ float *image, __gm__ const float *gm)
+{
+    using Padded = Tile<TileType::Vec, float, 16, 32, BLayout::RowMajor, 10, 20, SLayout::NoneBox, 512, PadValue::Max>;
+    using Full = Tile<TileType::Vec, float, 16, 32, BLayout::RowMajor>;
+    Padded t;
+    Full f;
+    GlobalTensor<float, Shape<1, 1, 1, 10, 20>, Stride<200, 200, 200, 20, 1>> g(const_cast<float *>(gm));
+    GmND<float, 16, 32> gi(image);
+    TLOAD(t, g);
+    TRESHAPE(f, t);
+    TSTORE(gi, f);
+}
+
+// ---- 5-D GM [1,2,3,4,8] with padded strides -> [24, 8] tile -> dense [24, 8]; and back out through 5-D strides ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void Load5D(__gm__ float *dense, __gm__ float *strided, __gm__ const float *gm)
+{
+    using T = Tile<TileType::Vec, float, 24, 8, BLayout::RowMajor>;
+    using G5 = GlobalTensor<float, Shape<1, 2, 3, 4, 8>, Stride<1000, 400, 100, 10, 1>>;
+    T t;
+    G5 g(const_cast<float *>(gm)), gOut(strided);
+    GmND<float, 24, 8> gd(dense);
+    TLOAD(t, g);
+    TSTORE(gd, t);
+    TSTORE(gOut, t);
+}
+
+// ---- TEXTRACT windows: C = A[:, col0 : col0+64] (through Left) x I, and C = I x B[row0 : row0+64, :] (through Right) ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void ExtractWindows(__gm__ float *outLeft, __gm__ float *outRight,
+                                                                       __gm__ const half *a, __gm__ const half *bT,
+                                                                       __gm__ const half *eyeB, __gm__ const half *eyeA,
+                                                                       int col0, int row0)
+{
+    // a [128, 256] row-major; bT [256 cols][256 rows] (column-major 256 x 256); eyeB: [256][64] column-major 64 x 256
+    // identity-like (eyeB(k, n) = k == n); eyeA [128, 64] with eyeA(r, k) = r == k
+    using MatA = Tile<TileType::Mat, half, 128, 256, BLayout::ColMajor, 128, 256, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, half, 256, 256, BLayout::RowMajor, 256, 256, SLayout::ColMajor>;
+    using MatEyeB = Tile<TileType::Mat, half, 64, 256, BLayout::RowMajor, 64, 256, SLayout::ColMajor>;
+    using MatEyeA = Tile<TileType::Mat, half, 128, 64, BLayout::ColMajor, 128, 64, SLayout::RowMajor>;
+    MatA am;
+    MatB bm;
+    MatEyeB eb;
+    MatEyeA ea;
+    TASSIGN(am, 0u);
+    TASSIGN(eb, 64u * 1024);
+    TASSIGN(ea, 96u * 1024);
+    TileLeft<half, 128, 64> l;
+    TileRight<half, 64, 256> r;
+    TileAcc<float, 128, 256> c;
+    GmND<half, 128, 256> ga(const_cast<half *>(a));
+    GlobalTensor<half, Shape<1, 1, 1, 64, 256>, Stride<1, 1, 1, 1, 64>, Layout::DN> geb(const_cast<half *>(eyeB));
+    GmND<half, 128, 64> gea(const_cast<half *>(eyeA));
+    GmND<float, 128, 256> gl(outLeft), gr(outRight);
+    TLOAD(am, ga);
+    TLOAD(eb, geb);
+    TLOAD(ea, gea);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    TEXTRACT(l, am, 0, (uint16_t)col0);
+    TMOV(r, eb);
+    TMATMUL(c, l, r);
+    TSTORE(gl, c);
+    // reuse the A region for B once everyone has read it
+    set_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID0);
+    wait_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID0);
+    TASSIGN(bm, 0u);
+    GlobalTensor<half, Shape<1, 1, 1, 256, 256>, Stride<1, 1, 1, 1, 256>, Layout::DN> gb(const_cast<half *>(bT));
+    // the B image spans 128 KiB: it would overwrite the identity tiles, so fetch them again afterwards
+    TLOAD(bm, gb);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID1);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID1);
+    TEXTRACT(r, bm, (uint16_t)row0, 0);
+    set_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1);
+    wait_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1);
+    TASSIGN(ea, 0u);
+    TLOAD(ea, gea);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID2);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID2);
+    TMOV(l, ea);
+    TMATMUL(c, l, r);
+    TSTORE(gr, c);
+}
+
+// ---- one-block matmul [128, K] x [K, 256] with bias, fp16 or bf16, ordered by Event objects ----
+template <typename T, int K>
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulBias(__gm__ float *out, __gm__ const T *a, __gm__ const T *bT,
+                                                                   __gm__ const float *bias)
+{
+    using MatA = Tile<TileType::Mat, T, 128, K, BLayout::ColMajor, 128, K, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, T, K, 256, BLayout::RowMajor, K, 256, SLayout::ColMajor>;
+    MatA am;
+    MatB bm;
+    TASSIGN(am, 0u);
+    TASSIGN(bm, 128u * K * sizeof(T));
+    TileLeft<T, 128, K> l;
+    TileRight<T, K, 256> r;
+    TileAcc<float, 128, 256> c;
+    GmND<T, 128, K> ga(const_cast<T *>(a));
+    GlobalTensor<T, Shape<1, 1, 1, K, 256>, Stride<1, 1, 1, 1, K>, Layout::DN> gb(const_cast<T *>(bT));
+    GmND<float, 128, 256> gc(out);
+    Event<Op::TLOAD, Op::TEXTRACT> loaded;
+    Event<Op::TEXTRACT, Op::TMATMUL> extracted;
+    Event<Op::TMATMUL, Op::TSTORE_ACC> computed;
+    TLOAD(am, ga);
+    loaded = TLOAD(bm, gb);
+    TEXTRACT(l, am, 0, 0, loaded);
+    extracted = TEXTRACT(r, bm, 0, 0);
+    if (bias != nullptr)
+        computed = TMATMUL_BIAS(c, l, r, BiasRow{bias}, extracted);
+    else
+        computed = TMATMUL(c, l, r, extracted);
+    TSTORE(gc, c, computed);
+}
+
+} // namespace
+
+PTO_DEVICE_CODE_END
+
+#define PTO_ST_NONNULL(...)                          \
+    do {                                             \
+        const void *ptrs[] = {__VA_ARGS__};          \
+        for (const void *p : ptrs)                   \
+            if (p == nullptr)                        \
+                return PTO_ERR_BAD_ARG;              \
+    } while (0)
+
+extern "C" int pto_st_softmax_step_f32_64x256(void *stream, uint16_t *x_exp, float *max_out, float *sum_out, float *alpha_out,
+                                              const float *x, const float *max_in, const float *sum_in, float scale,
+                                              int first, int round_mode)
+{
+    PTO_ST_NONNULL(x_exp, max_out, sum_out, alpha_out, x);
+    if (!first)
+        PTO_ST_NONNULL(max_in, sum_in);
+    if (round_mode < PTO_CAST_RINT || round_mode > PTO_CAST_ODD)
+        return PTO_ERR_BAD_ARG;
+    SoftmaxStep<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(
+        reinterpret_cast<half *>(x_exp), max_out, sum_out, alpha_out, x, max_in, sum_in, scale, first, round_mode);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_gu_step_f32_64x128(void *stream, float *o_out, const float *o_prev, const float *pv,
+                                         const float *alpha, const float *sum, int last)
+{
+    PTO_ST_NONNULL(o_out, o_prev, pv, alpha, sum);
+    GuStep<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(o_out, o_prev, pv, alpha, sum, last);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tri_mask_f32_64x128(void *stream, float *out, const float *x, int diagonal, float value, int upper)
+{
+    PTO_ST_NONNULL(out, x);
+    TriMask<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, x, diagonal, value, upper);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tgather_mask_b16_16x64(void *stream, uint16_t *out, const uint16_t *src, int pattern)
+{
+    PTO_ST_NONNULL(out, src);
+    if (pattern < 1 || pattern > 7)
+        return PTO_ERR_BAD_ARG;
+    GatherMask<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, pattern);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_mgather_b16_8x128(void *stream, uint16_t *out, const uint16_t *gm, const int32_t *idx, int gm_elems)
+{
+    PTO_ST_NONNULL(out, gm, idx);
+    MGatherElems<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, gm, idx, gm_elems);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tload_pad_f32_16x32(void *stream, float *image, const float *gm)
+{
+    PTO_ST_NONNULL(image, gm);
+    LoadPadImage<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(image, gm);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tload_5d_f32(void *stream, float *dense, float *strided, const float *gm)
+{
+    PTO_ST_NONNULL(dense, strided, gm);
+    Load5D<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(dense, strided, gm);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_textract_windows_f16(void *stream, float *out_left, float *out_right, const uint16_t *a,
+                                           const uint16_t *b_t, const uint16_t *eye_b, const uint16_t *eye_a, int col0, int row0)
+{
+    PTO_ST_NONNULL(out_left, out_right, a, b_t, eye_b, eye_a);
+    if (col0 < 0 || col0 % 8 || col0 + 64 > 256 || row0 < 0 || row0 % 8 || row0 + 64 > 256)
+        return PTO_ERR_UNSUPPORTED;
+    constexpr int lds = 128 * 1024;
+    static const int attr = pto_amd::allow_lds(ExtractWindows, lds);
+    if (attr != PTO_OK)
+        return attr;
+    ExtractWindows<<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(
+        out_left, out_right, reinterpret_cast<const half *>(a), reinterpret_cast<const half *>(b_t),
+        reinterpret_cast<const half *>(eye_b), reinterpret_cast<const half *>(eye_a), col0, row0);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, const uint16_t *b_t,
+                                             const float *bias, int bf16)
+{
+    PTO_ST_NONNULL(out, a, b_t);
+    constexpr int lds = (128 * 64 + 64 * 256) * 2;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (bf16)
+        MatmulBias<bfloat16_t, 64><<<dim3(1), dim3(kBlockThreads), lds, st>>>(
+            out, reinterpret_cast<const bfloat16_t *>(a), reinterpret_cast<const bfloat16_t *>(b_t), bias);
+    else
+        MatmulBias<half, 64><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const half *>(a),
+                                                                         reinterpret_cast<const half *>(b_t), bias);
+    return pto_amd::check_launch();
+}

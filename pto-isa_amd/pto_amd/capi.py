@@ -23,6 +23,15 @@ SYMBOLS = {
     "pto_tcvt_f32_bf16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),
     "pto_gather_rows": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t] * 3 + [C.c_int]),
     "pto_tgather_index_f16_16x1024_16x128": (C.c_int, [C.c_void_p] * 4),
+    "pto_st_softmax_step_f32_64x256": (C.c_int, [C.c_void_p] * 8 + [C.c_float, C.c_int, C.c_int]),
+    "pto_st_gu_step_f32_64x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int]),
+    "pto_st_tri_mask_f32_64x128": (C.c_int, [C.c_void_p] * 3 + [C.c_int, C.c_float, C.c_int]),
+    "pto_st_tgather_mask_b16_16x64": (C.c_int, [C.c_void_p] * 3 + [C.c_int]),
+    "pto_st_mgather_b16_8x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
+    "pto_st_tload_pad_f32_16x32": (C.c_int, [C.c_void_p] * 3),
+    "pto_st_tload_5d_f32": (C.c_int, [C.c_void_p] * 4),
+    "pto_st_textract_windows_f16": (C.c_int, [C.c_void_p] * 7 + [C.c_int] * 2),
+    "pto_st_matmul_bias_128x64x256": (C.c_int, [C.c_void_p] * 5 + [C.c_int]),
 }
 
 _lib = None
