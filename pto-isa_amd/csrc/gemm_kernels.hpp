@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
 // one copy instruction per two MFMAs, then one fragment read per two MFMAs.
 // C[row0 : row0+BM, col0 : col0+BN] (+)= A[row0.., kFirst*32 ..] x B[col0.., kFirst*32 ..] over kLoop K-steps of 32.
 template <int BM, int BN, int STAGES>
-AICORE inline void MixTile(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
+AICORE inline __attribute__((always_inline)) void MixTile(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
                            int row0, int col0, int kFirst, int kLoop, bool partial)
 {
     constexpr int BK = 32, KH = 16;
@@ -272,21 +272,27 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     const int tilesM = m / BM, tilesN = n / BN;
     const int block = (int)get_block_idx();
     int tm, tn;
-    if (block < fullTiles) {
-        TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
-        MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, 0, k / 32, false);
-    } else if (tailMode == 1) {
+    if (block >= fullTiles && tailMode == 1) {
         const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
         TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
         const int sub = u % 4;
         MixTile<BM / 2, BN / 2, STAGES>(out, src0, src1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
                                         tn * BN + (sub & 1) * (BN / 2), 0, k / 32, false);
+        return;
+    }
+    // whole tiles and K-ranges of whole tiles share one call site, so the tile body is inlined once
+    int kFirst = 0, kLoop = k / 32;
+    bool partial = false;
+    if (block < fullTiles) {
+        TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
     } else {
         const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * splitK);
         TileOfId<GROUP_M>(fullTiles + u / splitK, tilesM, tilesN, tm, tn);
-        const int kLoop = k / 32 / splitK;
-        MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, (u % splitK) * kLoop, kLoop, splitK > 1);
+        kLoop = k / 32 / splitK;
+        kFirst = (u % splitK) * kLoop;
+        partial = splitK > 1;
     }
+    MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, kFirst, kLoop, partial);
 }
 
 // Clears the C tiles that GemmF16F32Mix accumulates into with atomic adds (tile ids >= fullTiles).
