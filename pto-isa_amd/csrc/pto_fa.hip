@@ -40,35 +40,128 @@ AICORE inline float SwapHalves(float x) { return __shfl_xor(x, 32); }
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-// V^T operand for O^T += V^T P^T: TEXTRACT of the [32 d, kBKV keys] block `db` of the transposed
-// V tile, taken straight from the row-major [keys, D] LDS image with transposing reads.  Key order
-// inside every 16-key MFMA step matches the order in which the accumulator layout holds P^T:
-// k slot j of half-wave h  <->  key 16t + 8(j/4) + 4h + j%4.
-template <int kBKV, typename LeftT, typename MatT>
-AICORE inline void ExtractVT(LeftT &dst, MatT &vMat, int db)
+// Row r of the K operand (and so of X^T and P^T) holds key KeyOfRow(r): a permutation inside every
+// group of 16 keys, chosen so that the four keys which one transposing read of V^T gathers (rows
+// 4a .. 4a+3) lie in four different 64-byte bank groups of the swizzled [keys, D] LDS image:
+// the XOR swizzle moves the 16-byte chunk by key % 16 for 256-byte rows (D = 128: the keys differ
+// in bits 2-3) and by (key / 2) % 8 for 128-byte rows, two rows per bank line (D = 64: bits 0 and 3).
+template <int D>
+AICORE inline constexpr uint32_t KeyOfRow(uint32_t r)
+{
+    const uint32_t a = (r >> 2) & 3u, b = r & 3u;
+    if (D == 128)
+        return (r & ~15u) | (b << 2) | a;
+    return (r & ~15u) | (b & 1u) | ((b >> 1) << 3) | (a << 1);
+}
+
+// K operand for X^T = K Q^T: 32 rows x D of the key tile, row r <- key KeyOfRow(r)
+template <int D, typename LeftT, typename MatT>
+AICORE inline void ExtractK(LeftT &dst, MatT &kMat, int kb)
 {
     using Geo = detail::MatGeom<MatT>;
     using S = typename LeftT::Storage;
-    static_assert(S::MB == 1 && S::KS == kBKV / 16, "one 32-row block of V^T over the whole key tile");
-    const char *lds = hw::lds_base() + vMat.st.lds;
+    using Frag = typename detail::FragOf<half>::type;
+    static_assert(S::MB == 1 && S::KS == D / 16, "one 32-key block over the whole head dimension");
+    const char *lds = hw::lds_base() + kMat.st.lds;
     const uint32_t lane = (uint32_t)hw::lane();
-    const uint32_t h = lane >> 5;
-    const uint32_t d0 = (uint32_t)db * 32u + 16u * ((lane >> 4) & 1u) + 4u * (lane & 3u);
-    const uint32_t keyIn = (lane & 15u) >> 2;
+    const uint32_t key = (uint32_t)kb * 32u + KeyOfRow<D>(lane & 31u), khalf = lane >> 5;
 #pragma unroll
-    for (int ks = 0; ks < S::KS; ++ks) {
-        s16x4 part[2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-            const uint32_t key = 16u * ks + 8u * u + 4u * h + keyIn;
-            const uint32_t off = detail::mat_chunk_off<Geo::RowBytes>(key, d0 >> 3) + ((d0 & 7u) << 1);
-            part[u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4 *)(lds + off));
-        }
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-        s16x8 both = {part[0][0], part[0][1], part[0][2], part[0][3], part[1][0], part[1][1], part[1][2], part[1][3]};
-        dst.st.f[0][ks] = __builtin_bit_cast(f16x8, both);
-    }
+    for (int ks = 0; ks < S::KS; ++ks)
+        dst.st.f[0][ks] = *reinterpret_cast<const Frag *>(lds + detail::mat_chunk_off<Geo::RowBytes>(key, khalf + ks * 2));
 }
+
+// One transposing 64-bit LDS read at byte address addr + OFF.
+template <uint32_t OFF>
+AICORE inline s16x4 DsReadTr16(uint32_t addr)
+{
+    static_assert(OFF < 65536u, "the offset field of an LDS instruction has 16 bits");
+    s16x4 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+
+// V^T operand for O^T += V^T P^T: TEXTRACT of the [32 d, kBKV keys] block `db` of the transposed
+// V tile, taken straight from the row-major [keys, D] LDS image with transposing reads.  Key order
+// inside every 16-key MFMA step matches the order in which the accumulator layout holds P^T:
+// k slot j of half-wave h  <->  row 16t + 8(j/4) + 4h + j%4 of X^T, which holds key KeyOfRow(row).
+//
+// The reads are issued as assembly so that they carry no compiler-visible LDS dependency: before a
+// compiler-generated LDS read that may alias an outstanding asynchronous copy into LDS the compiler
+// waits for every outstanding copy, which would make the prefetch of the next tile synchronous.
+// The workgroup barrier at the top of a tile is what orders these reads after the copy that filled
+// the stage.  Wait<N>() is the matching wait on the LDS counter (LDS operations of a wave complete
+// in order: at most N younger ones may still be outstanding); it names the fragment registers as
+// operands so that no use of them can be moved above it.
+template <int D, int kBKV>
+struct VTReader {
+    static constexpr int DB = D / 32, KS = kBKV / 16;
+    static constexpr int kReads = 2 * KS; // reads per 32-row block of V^T
+    static constexpr uint32_t kStepBytes = 16u * D * (uint32_t)sizeof(half);
+    static_assert(KS == 2 || KS == 4, "key tiles of 32 or 64");
+    struct Frag {
+        s16x4 part[KS][2];
+    };
+    uint32_t base[DB][2]; // LDS byte address of (block db, read u) for key step 0 of a tile at LDS offset 0
+
+    template <typename MatT>
+    AICORE inline void Init()
+    {
+        using Geo = detail::MatGeom<MatT>;
+        static_assert(detail::mat_swz<Geo::RowBytes>(16) == detail::mat_swz<Geo::RowBytes>(0), "the swizzle repeats every 16 keys");
+        const uint32_t lane = (uint32_t)hw::lane();
+        const uint32_t h = lane >> 5, keyIn = (lane & 15u) >> 2;
+        const uint32_t ldsBase = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)hw::lds_base();
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const uint32_t d0 = (uint32_t)db * 32u + 16u * ((lane >> 4) & 1u) + 4u * (lane & 3u);
+                const uint32_t key = KeyOfRow<D>(8u * u + 4u * h + keyIn);
+                base[db][u] = ldsBase + detail::mat_chunk_off<Geo::RowBytes>(key, d0 >> 3) + ((d0 & 7u) << 1);
+            }
+    }
+
+    template <uint32_t LDS_OFF, int... KSI>
+    AICORE inline void IssueSteps(Frag &f, int db, std::integer_sequence<int, KSI...>) const
+    {
+        ((f.part[KSI][0] = DsReadTr16<LDS_OFF + KSI * kStepBytes>(base[db][0]),
+          f.part[KSI][1] = DsReadTr16<LDS_OFF + KSI * kStepBytes>(base[db][1])),
+         ...);
+    }
+    // issue the reads of block db of the V tile at LDS offset LDS_OFF
+    template <uint32_t LDS_OFF>
+    AICORE inline void Issue(Frag &f, int db) const
+    {
+        IssueSteps<LDS_OFF>(f, db, std::make_integer_sequence<int, KS>());
+    }
+
+    template <int N>
+    AICORE static inline void Wait(Frag &f)
+    {
+        static_assert(N >= 0 && N <= 15, "the LDS counter has 4 bits");
+        if constexpr (KS == 4)
+            asm volatile("s_waitcnt lgkmcnt(%8)"
+                         : "+v"(f.part[0][0]), "+v"(f.part[0][1]), "+v"(f.part[1][0]), "+v"(f.part[1][1]), "+v"(f.part[2][0]),
+                           "+v"(f.part[2][1]), "+v"(f.part[3][0]), "+v"(f.part[3][1])
+                         : "n"(N));
+        else
+            asm volatile("s_waitcnt lgkmcnt(%4)"
+                         : "+v"(f.part[0][0]), "+v"(f.part[0][1]), "+v"(f.part[1][0]), "+v"(f.part[1][1])
+                         : "n"(N));
+    }
+
+    template <typename LeftT>
+    AICORE static inline void ToLeft(LeftT &dst, const Frag &f)
+    {
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const s16x8 both = {f.part[ks][0][0], f.part[ks][0][1], f.part[ks][0][2], f.part[ks][0][3],
+                                f.part[ks][1][0], f.part[ks][1][1], f.part[ks][1][2], f.part[ks][1][3]};
+            dst.st.f[0][ks] = __builtin_bit_cast(f16x8, both);
+        }
+    }
+};
 
 template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int NQ, int kBKV = kBKVDefault>
 __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
@@ -147,6 +240,114 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
     // s = 1/sqrt(D) folded with log2(e): exp(s y) = exp2(s log2e y)
     const float sLog2e = (D == 128 ? 0.08838834764831845f : 0.125f) * 1.4426950408889634f;
 
+    // ---- the three stages of one key tile ----
+    // X^T = K Q^T for the key tile in LDS stage `stage`
+    auto scoreTile = [&](AccS(&sAcc)[KB], int stage) {
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            LeftK kLeft;
+            ExtractK<D>(kLeft, kMat[stage], kb);
+            TMATMUL(sAcc[kb], kLeft, qRight);
+        }
+    };
+    // streaming softmax on the accumulator fragments of tile t (one query per lane and query block)
+    auto softmaxTile = [&](AccS(&sAcc)[KB], int t, RightP &pRight, float(&alpha)[NQ], bool &anyRaise) {
+        const int key0 = t * kBKV;
+        if (CAUSAL && key0 + kBKV - 1 > q0 + causalOff) { // the diagonal crosses this tile
+#pragma unroll
+            for (int nb = 0; nb < NQ; ++nb) {
+                const int limit = myQuery + 32 * nb + causalOff; // last visible key of this lane's query
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = key0 + kb * 32 + (int)KeyOfRow<D>((v >> 2) * 8 + hHalf * 4 + (v & 3));
+                        if (key > limit)
+                            sAcc[kb].st.f[0][nb][v] += kMaskValue;
+                    }
+            }
+        }
+        anyRaise = t == 0;
+#pragma unroll
+        for (int nb = 0; nb < NQ; ++nb) {
+            float locMax = sAcc[0].st.f[0][nb][0];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    locMax = fmaxf(locMax, sAcc[kb].st.f[0][nb][v]);
+            locMax = fmaxf(locMax, SwapHalves(locMax));
+            // The running max only has to bound the scores well enough to keep exp() in range: it is
+            // raised (and O, S rescaled by alpha) when a tile exceeds it by more than kSlack in the
+            // exponent, i.e. P stays below 2^kSlack.  O / S and max*s + ln(S) do not depend on the choice.
+            constexpr float kSlack = 8.0f;
+            const bool raise = t == 0 || (locMax - runMax[nb]) * sLog2e > kSlack;
+            const float newMax = raise ? locMax : runMax[nb];
+            if (t > 0)
+                anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
+            alpha[nb] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nb] - newMax) * sLog2e);
+            runMax[nb] = newMax;
+            const float negMax = -newMax * sLog2e;
+            float locSum = 0.0f;
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int half_ = 0; half_ < 2; ++half_) {
+                    f16x8 pk;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float p =
+                            __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][nb][half_ * 8 + j], sLog2e, negMax));
+                        locSum += p; // row sum over the fp32 P, as the reference does
+                        pk[j] = (half)p;
+                    }
+                    pRight.st.f[nb][kb * 2 + half_] = pk;
+                }
+            runSum[nb] = t == 0 ? locSum : runSum[nb] * alpha[nb] + locSum;
+        }
+    };
+    // O^T = alpha O^T + V^T P^T.  vFrag holds block 0 of V^T of this tile (issued earlier); the reads
+    // of block db+1 are in flight while the MFMAs of block db run.
+    using VT = VTReader<D, kBKV>;
+    VT vt;
+    vt.template Init<TileMatV>();
+    auto outputTile = [&](auto stageTag, int t, typename VT::Frag &vFirst, RightP &pRight, float(&alpha)[NQ], bool anyRaise) {
+        constexpr uint32_t kVOff = decltype(stageTag)::value * kStageBytes + kTileBytes;
+        typename VT::Frag vOther;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            typename VT::Frag &cur = (db & 1) ? vOther : vFirst;
+            typename VT::Frag &nxt = (db & 1) ? vFirst : vOther;
+            if (db + 1 < DB) {
+                vt.template Issue<kVOff>(nxt, db + 1);
+                VT::template Wait<VT::kReads>(cur);
+            } else {
+                VT::template Wait<0>(cur);
+            }
+            LeftVT vLeft;
+            VT::ToLeft(vLeft, cur);
+            if (t == 0) {
+                TMATMUL(oAcc[db], vLeft, pRight);
+            } else {
+                if (anyRaise) { // wave-uniform: some lane's max was raised
+#pragma unroll
+                    for (int nb = 0; nb < NQ; ++nb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            oAcc[db].st.f[0][nb][v] *= alpha[nb];
+                }
+                TMATMUL_ACC(oAcc[db], oAcc[db], vLeft, pRight);
+            }
+        }
+    };
+    auto keyTile = [&](__gm__ half *base, int t) {
+        const int tc = t < numTiles ? t : numTiles - 1; // past the end: re-fetch the last tile (nobody reads it)
+        return GlobalKV(base + (int64_t)tc * kBKV * D);
+    };
+    constexpr int kCopies = TLoadInstrs<TileMatK>() + TLoadInstrs<TileMatV>();
+    constexpr int kScoreMfma = KB * NQ * (D / 16);
+    constexpr int kKReads = KB * (D / 16);
+
     {
         GlobalQT gmQ(qBase);
         TLOAD(qMat, gmQ);
@@ -161,118 +362,47 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
         set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
     }
 
-    for (int tile = 0; tile < numTiles; tile += 2) {
+    // One key tile in LDS stage st (a compile-time constant: every LDS address is an immediate).
+    auto tileStep = [&](auto stageTag, int t) {
+        constexpr int st = decltype(stageTag)::value;
+        wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
+        // The next tile is fetched while this tile's score MFMAs issue, a few asynchronous copies
+        // between MFMAs, so that the wave never sits in the vector-memory issue queue.  Past the last
+        // tile the copy re-fetches it into the free stage, which keeps this a straight-line region.
+        {
+            GlobalKV gmK = keyTile(kBase, t + 1), gmV = keyTile(vBase, t + 1);
+            TLOAD(kMat[st ^ 1], gmK);
+            TLOAD(vMat[st ^ 1], gmV);
+            set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+        }
+        AccS sAcc[KB];
+        scoreTile(sAcc, st);
+        {
+            // issue order: K fragment reads run kAhead MFMAs ahead of their use; one copy per kPer MFMAs
+            constexpr int kPer = kScoreMfma / kCopies > 0 ? kScoreMfma / kCopies : 1;
+            constexpr int kAhead = 4;
+            __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
 #pragma unroll
-        for (int st = 0; st < 2; ++st) { // unrolled over the two LDS stages
-            const int t = tile + st;
-            if (t >= numTiles)
-                break;
-            wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
-            // The next tile is fetched while this tile's score MFMAs issue: one asynchronous copy per
-            // two MFMAs, so that the wave never sits in the vector-memory issue queue.  Past the last
-            // tile the copy re-fetches it into the free stage, which keeps this a straight-line region.
-            {
-                const int tn = t + 1 < numTiles ? t + 1 : t;
-                GlobalKV gmK(kBase + (int64_t)tn * kBKV * D), gmV(vBase + (int64_t)tn * kBKV * D);
-                TLOAD(kMat[st ^ 1], gmK);
-                TLOAD(vMat[st ^ 1], gmV);
-                set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
-            }
-            // ---- X^T = K Q^T ----
-            AccS sAcc[KB];
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) {
-                LeftK kLeft;
-                TEXTRACT(kLeft, kMat[st], kb * 32, 0);
-                TMATMUL(sAcc[kb], kLeft, qRight);
-            }
-            {
-                constexpr int kCopies = TLoadInstrs<TileMatK>() + TLoadInstrs<TileMatV>();
-                constexpr int kMfma = KB * NQ * (D / 16);
-                constexpr int kPer = kMfma / kCopies > 0 ? kMfma / kCopies : 1;
-#pragma unroll
-                for (int i = 0; i < kCopies; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, kPer, 0);
+            for (int i = 0; i < kScoreMfma; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                if (i + kAhead < kKReads)
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                if (i % kPer == kPer - 1 && i / kPer < kCopies)
                     __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
-                }
-            }
-
-            // ---- streaming softmax on the accumulator fragments (one query per lane and query block) ----
-            const int key0 = t * kBKV;
-            if (CAUSAL && key0 + kBKV - 1 > q0 + causalOff) { // the diagonal crosses this tile
-#pragma unroll
-                for (int nb = 0; nb < NQ; ++nb) {
-                    const int limit = myQuery + 32 * nb + causalOff; // last visible key of this lane's query
-#pragma unroll
-                    for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int key = key0 + kb * 32 + (v >> 2) * 8 + (int)hHalf * 4 + (v & 3);
-                            if (key > limit)
-                                sAcc[kb].st.f[0][nb][v] += kMaskValue;
-                        }
-                }
-            }
-            RightP pRight;
-            float alpha[NQ];
-            bool anyRaise = t == 0;
-#pragma unroll
-            for (int nb = 0; nb < NQ; ++nb) {
-                float locMax = sAcc[0].st.f[0][nb][0];
-#pragma unroll
-                for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        locMax = fmaxf(locMax, sAcc[kb].st.f[0][nb][v]);
-                locMax = fmaxf(locMax, SwapHalves(locMax));
-                // The running max only has to bound the scores well enough to keep exp() in range: it is
-                // raised (and O, S rescaled by alpha) when a tile exceeds it by more than kSlack in the
-                // exponent, i.e. P stays below 2^kSlack.  O / S and max*s + ln(S) do not depend on the choice.
-                constexpr float kSlack = 8.0f;
-                const bool raise = t == 0 || (locMax - runMax[nb]) * sLog2e > kSlack;
-                const float newMax = raise ? locMax : runMax[nb];
-                if (t > 0)
-                    anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
-                alpha[nb] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nb] - newMax) * sLog2e);
-                runMax[nb] = newMax;
-                const float negMax = -newMax * sLog2e;
-                float locSum = 0.0f;
-#pragma unroll
-                for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                    for (int half_ = 0; half_ < 2; ++half_) {
-                        f16x8 pk;
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const float p =
-                                __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][nb][half_ * 8 + j], sLog2e, negMax));
-                            locSum += p; // row sum over the fp32 P, as the reference does
-                            pk[j] = (half)p;
-                        }
-                        pRight.st.f[nb][kb * 2 + half_] = pk;
-                    }
-                runSum[nb] = t == 0 ? locSum : runSum[nb] * alpha[nb] + locSum;
-            }
-
-            // ---- O^T = alpha O^T + V^T P^T ----
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                LeftVT vLeft;
-                ExtractVT<kBKV>(vLeft, vMat[st], db);
-                if (t == 0) {
-                    TMATMUL(oAcc[db], vLeft, pRight);
-                } else {
-                    if (anyRaise) { // wave-uniform: some lane's max was raised
-#pragma unroll
-                        for (int nb = 0; nb < NQ; ++nb)
-#pragma unroll
-                            for (int v = 0; v < 16; ++v)
-                                oAcc[db].st.f[0][nb][v] *= alpha[nb];
-                    }
-                    TMATMUL_ACC(oAcc[db], oAcc[db], vLeft, pRight);
-                }
             }
         }
+        typename VT::Frag vFirst;
+        vt.template Issue<st * kStageBytes + kTileBytes>(vFirst, 0); // lands during the softmax
+        RightP pRight;
+        float alpha[NQ];
+        bool anyRaise;
+        softmaxTile(sAcc, t, pRight, alpha, anyRaise);
+        outputTile(stageTag, t, vFirst, pRight, alpha, anyRaise);
+    };
+    for (int tile = 0; tile < numTiles; tile += 2) {
+        tileStep(std::integral_constant<int, 0>(), tile);
+        if (tile + 1 < numTiles)
+            tileStep(std::integral_constant<int, 1>(), tile + 1);
     }
     hw::wait_vm0(); // the copy issued by the last tile must not outlive the workgroup's LDS
     // ---- finish: O /= S, write O (and LSE) ----
