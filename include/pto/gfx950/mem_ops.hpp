@@ -116,6 +116,15 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
 // -------------------------------------------------------------------- TLOAD
 namespace detail {
 
+// Tells the compiler that p is the same in every lane (it then lives in scalar registers and the
+// access can use the scalar-base + 32-bit lane offset addressing form).
+PTO_DEV const char *uniform_ptr(const char *p)
+{
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const char *>((uintptr_t)(((uint64_t)hi << 32) | lo));
+}
+
 // GM -> LDS Mat tile.  Fast path: the tile's contiguous dimension is the unit-stride one in
 // memory, the valid region is the whole tile: 16-byte asynchronous global->LDS copies, 1 KiB of
 // LDS per wave instruction; the swizzle is applied on the global-address side.
@@ -135,16 +144,35 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
         constexpr int perWaveInst = kWaveSize;
         constexpr int nInst = cdiv(total, perWaveInst);
         const int lane = hw::lane(), wave = hw::wave();
+        constexpr int cpr = Geo::ChunksPerRow;
+        // rows that one wave instruction covers, when a row is at most one instruction long
+        constexpr int rpi = (cpr <= kWaveSize && kWaveSize % cpr == 0) ? kWaveSize / cpr : 0;
+        if constexpr (rpi > 0 && (rpi * kBlockWaves) % 16 == 0 && nInst % kBlockWaves == 0 && total % perWaveInst == 0) {
+            // The swizzle repeats every 16 rows and the instructions of one wave are a multiple of 16
+            // rows apart: every instruction of this wave uses the same per-lane byte offset (32 bits: a
+            // tile spans less than 4 GiB of memory) on top of a wave-uniform base, which the loop
+            // around the TLOAD only has to advance with scalar arithmetic.
+            const uint32_t major0 = (uint32_t)wave * rpi + (uint32_t)lane / cpr, cpos = (uint32_t)lane % cpr;
+            const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major0);
+            const uint32_t laneOff = (major0 * (uint32_t)ld + chunk * (16 / sizeof(T))) * (uint32_t)sizeof(T);
+            const char *base = reinterpret_cast<const char *>(gm);
 #pragma unroll
-        for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
-            const int s = s0 + wave;
-            const uint32_t q = (uint32_t)(s * perWaveInst + lane);
-            constexpr bool evenInst = nInst % kBlockWaves == 0, evenTotal = total % perWaveInst == 0;
-            if ((evenInst || s < nInst) && (evenTotal || q < (uint32_t)total)) {
-                const uint32_t major = q / Geo::ChunksPerRow, cpos = q % Geo::ChunksPerRow;
-                const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major);
-                const T *g = gm + (int64_t)major * ld + chunk * (16 / sizeof(T));
-                __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + s * (perWaveInst * 16)), 16, 0, 0);
+            for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
+                const char *g = uniform_ptr(base + (int64_t)(s0 * rpi) * ld * (int64_t)sizeof(T)) + laneOff;
+                __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + (s0 + wave) * (perWaveInst * 16)), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
+                const int s = s0 + wave;
+                const uint32_t q = (uint32_t)(s * perWaveInst + lane);
+                constexpr bool evenInst = nInst % kBlockWaves == 0, evenTotal = total % perWaveInst == 0;
+                if ((evenInst || s < nInst) && (evenTotal || q < (uint32_t)total)) {
+                    const uint32_t major = q / Geo::ChunksPerRow, cpos = q % Geo::ChunksPerRow;
+                    const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major);
+                    const T *g = gm + (int64_t)major * ld + chunk * (16 / sizeof(T));
+                    __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + s * (perWaveInst * 16)), 16, 0, 0);
+                }
             }
         }
     } else {

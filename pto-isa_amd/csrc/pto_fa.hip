@@ -54,21 +54,50 @@ AICORE inline constexpr uint32_t KeyOfRow(uint32_t r)
     return (r & ~15u) | (b & 1u) | ((b >> 1) << 3) | (a << 1);
 }
 
-// K operand for X^T = K Q^T: 32 rows x D of the key tile, row r <- key KeyOfRow(r)
-template <int D, typename LeftT, typename MatT>
-AICORE inline void ExtractK(LeftT &dst, MatT &kMat, int kb)
+// compile-time loop: f(integral_constant<int, I>) for I = FIRST .. LAST-1
+template <int FIRST, int LAST, typename F>
+AICORE inline void StaticFor(F &&f)
 {
-    using Geo = detail::MatGeom<MatT>;
-    using S = typename LeftT::Storage;
-    using Frag = typename detail::FragOf<half>::type;
-    static_assert(S::MB == 1 && S::KS == D / 16, "one 32-key block over the whole head dimension");
-    const char *lds = hw::lds_base() + kMat.st.lds;
-    const uint32_t lane = (uint32_t)hw::lane();
-    const uint32_t key = (uint32_t)kb * 32u + KeyOfRow<D>(lane & 31u), khalf = lane >> 5;
-#pragma unroll
-    for (int ks = 0; ks < S::KS; ++ks)
-        dst.st.f[0][ks] = *reinterpret_cast<const Frag *>(lds + detail::mat_chunk_off<Geo::RowBytes>(key, khalf + ks * 2));
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>());
+        StaticFor<FIRST + 1, LAST>(f);
+    }
 }
+
+// K operand for X^T = K Q^T, one 16-wide step of the head dimension at a time: fragment (kb, ks) =
+// rows kb*32 .. +31 (row r <- key KeyOfRow(r)) x d = 16 ks .. +15 of the key tile.  Issued as
+// assembly, like the V^T reads below, so that the order of issue and the lookahead are what the
+// source says: fragment i+kAhead is requested before the MFMA on fragment i.
+template <int D>
+struct KReader {
+    static constexpr int KS = D / 16;
+    static constexpr uint32_t kRowBytes = D * (uint32_t)sizeof(half);
+    uint32_t base[KS]; // LDS byte address of this lane's 16 bytes of step ks, block 0, tile at LDS offset 0
+
+    AICORE inline void Init()
+    {
+        const uint32_t lane = (uint32_t)hw::lane();
+        const uint32_t key = KeyOfRow<D>(lane & 31u), khalf = lane >> 5;
+        const uint32_t ldsBase = (uint32_t)(size_t)(__attribute__((address_space(3))) char *)hw::lds_base();
+        static_assert(detail::mat_swz<kRowBytes>(32) == detail::mat_swz<kRowBytes>(0), "the swizzle repeats every 32 keys");
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+            base[ks] = ldsBase + detail::mat_chunk_off<kRowBytes>(key, khalf + 2u * ks);
+    }
+    template <uint32_t LDS_OFF, int KB_, int KS_>
+    AICORE inline void Issue(f16x8 &f) const
+    {
+        constexpr uint32_t off = LDS_OFF + KB_ * 32u * kRowBytes;
+        static_assert(off < 65536u, "the offset field of an LDS instruction has 16 bits");
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(f) : "v"(base[KS_]), "n"(off));
+    }
+    template <int N>
+    AICORE static inline void Wait(f16x8 &f)
+    {
+        static_assert(N >= 0 && N <= 15, "the LDS counter has 4 bits");
+        asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(f) : "n"(N));
+    }
+};
 
 // One transposing 64-bit LDS read at byte address addr + OFF.
 template <uint32_t OFF>
@@ -241,14 +270,40 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
     const float sLog2e = (D == 128 ? 0.08838834764831845f : 0.125f) * 1.4426950408889634f;
 
     // ---- the three stages of one key tile ----
-    // X^T = K Q^T for the key tile in LDS stage `stage`
-    auto scoreTile = [&](AccS(&sAcc)[KB], int stage) {
+    // X^T = K Q^T for the key tile in LDS stage st: one MFMA per K fragment, fragments requested kAhead MFMAs ahead
+    KReader<D> kr;
+    kr.Init();
+    // `between(i)` runs before the MFMA on fragment i (the caller issues its asynchronous copies there).
+    // A scheduling barrier after every MFMA keeps the issue order exactly as written.
+    auto scoreTile = [&](AccS(&sAcc)[KB], auto stageTag, auto &&between) {
+        constexpr uint32_t kOff = decltype(stageTag)::value * kStageBytes;
+        constexpr int KSTEPS = D / 16, kTotal = KB * KSTEPS, kAhead = 4;
+        using LeftStep = TileLeft<half, 32, 16, 32, 16>;
+        using RightStep = TileRight<half, 16, kBQ, 16, kBQ>;
+        f16x8 frag[kAhead + 1];
+        StaticFor<0, kAhead>([&](auto i) {
+            constexpr int I = decltype(i)::value;
+            kr.template Issue<kOff, I / KSTEPS, I % KSTEPS>(frag[I % (kAhead + 1)]);
+        });
+        StaticFor<0, kTotal>([&](auto i) {
+            constexpr int I = decltype(i)::value, J = I + kAhead;
+            if constexpr (J < kTotal)
+                kr.template Issue<kOff, J / KSTEPS, J % KSTEPS>(frag[J % (kAhead + 1)]);
+            between(i);
+            KReader<D>::template Wait<(kTotal - 1 - I < kAhead ? kTotal - 1 - I : kAhead)>(frag[I % (kAhead + 1)]);
+            constexpr int kb = I / KSTEPS, ks = I % KSTEPS;
+            LeftStep a;
+            RightStep b;
+            a.st.f[0][0] = frag[I % (kAhead + 1)];
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb) {
-            LeftK kLeft;
-            ExtractK<D>(kLeft, kMat[stage], kb);
-            TMATMUL(sAcc[kb], kLeft, qRight);
-        }
+            for (int nb = 0; nb < NQ; ++nb)
+                b.st.f[nb][0] = qRight.st.f[nb][ks];
+            if constexpr (ks == 0)
+                TMATMUL(sAcc[kb], a, b);
+            else
+                TMATMUL_ACC(sAcc[kb], sAcc[kb], a, b);
+            __builtin_amdgcn_sched_barrier(0);
+        });
     };
     // streaming softmax on the accumulator fragments of tile t (one query per lane and query block)
     auto softmaxTile = [&](AccS(&sAcc)[KB], int t, RightP &pRight, float(&alpha)[NQ], bool &anyRaise) {
@@ -344,9 +399,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
         const int tc = t < numTiles ? t : numTiles - 1; // past the end: re-fetch the last tile (nobody reads it)
         return GlobalKV(base + (int64_t)tc * kBKV * D);
     };
-    constexpr int kCopies = TLoadInstrs<TileMatK>() + TLoadInstrs<TileMatV>();
     constexpr int kScoreMfma = KB * NQ * (D / 16);
-    constexpr int kKReads = KB * (D / 16);
 
     {
         GlobalQT gmQ(qBase);
@@ -366,31 +419,23 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
     auto tileStep = [&](auto stageTag, int t) {
         constexpr int st = decltype(stageTag)::value;
         wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
-        // The next tile is fetched while this tile's score MFMAs issue, a few asynchronous copies
-        // between MFMAs, so that the wave never sits in the vector-memory issue queue.  Past the last
-        // tile the copy re-fetches it into the free stage, which keeps this a straight-line region.
-        {
-            GlobalKV gmK = keyTile(kBase, t + 1), gmV = keyTile(vBase, t + 1);
-            TLOAD(kMat[st ^ 1], gmK);
-            TLOAD(vMat[st ^ 1], gmV);
-            set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
-        }
+        // The next tile is fetched while this tile's score MFMAs issue: the K copies before the second
+        // MFMA, the V copies halfway, so that the wave never sits long in the vector-memory issue queue.
+        // Past the last tile the copies re-fetch it into the free stage, which keeps this a straight-line region.
         AccS sAcc[KB];
-        scoreTile(sAcc, st);
-        {
-            // issue order: K fragment reads run kAhead MFMAs ahead of their use; one copy per kPer MFMAs
-            constexpr int kPer = kScoreMfma / kCopies > 0 ? kScoreMfma / kCopies : 1;
-            constexpr int kAhead = 4;
-            __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
-#pragma unroll
-            for (int i = 0; i < kScoreMfma; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                if (i + kAhead < kKReads)
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-                if (i % kPer == kPer - 1 && i / kPer < kCopies)
-                    __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        scoreTile(sAcc, stageTag, [&](auto i) {
+            constexpr int I = decltype(i)::value;
+            if constexpr (I == 1) {
+                GlobalKV gmK = keyTile(kBase, t + 1);
+                TLOAD(kMat[st ^ 1], gmK);
             }
-        }
+            if constexpr (I == kScoreMfma / 2 + 1) {
+                GlobalKV gmV = keyTile(vBase, t + 1);
+                TLOAD(vMat[st ^ 1], gmV);
+                set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+            }
+        });
         typename VT::Frag vFirst;
         vt.template Issue<st * kStageBytes + kTileBytes>(vFirst, 0); // lands during the softmax
         RightP pRight;
