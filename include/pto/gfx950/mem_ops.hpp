@@ -128,7 +128,8 @@ PTO_DEV const char *uniform_ptr(const char *p)
 // GM -> LDS Mat tile.  Fast path: the tile's contiguous dimension is the unit-stride one in
 // memory, the valid region is the whole tile: 16-byte asynchronous global->LDS copies, 1 KiB of
 // LDS per wave instruction; the swizzle is applied on the global-address side.
-template <typename TileT, typename G>
+// SLICE >= 0: only the SLICE-th group of kBlockWaves copy instructions (one per wave).
+template <int SLICE = -1, typename TileT, typename G>
 PTO_DEV void tload_mat(TileT &dst, G &src)
 {
     using T = typename TileT::DType;
@@ -156,12 +157,15 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major0);
             const uint32_t laneOff = (major0 * (uint32_t)ld + chunk * (16 / sizeof(T))) * (uint32_t)sizeof(T);
             const char *base = reinterpret_cast<const char *>(gm);
+            constexpr int first = SLICE < 0 ? 0 : SLICE * kBlockWaves, last = SLICE < 0 ? nInst : first + kBlockWaves;
+            static_assert(last <= nInst, "[PTO][SA] TLOAD slice: the tile has fewer copy instructions");
 #pragma unroll
-            for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
+            for (int s0 = first; s0 < last; s0 += kBlockWaves) {
                 const char *g = uniform_ptr(base + (int64_t)(s0 * rpi) * ld * (int64_t)sizeof(T)) + laneOff;
                 __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + (s0 + wave) * (perWaveInst * 16)), 16, 0, 0);
             }
         } else {
+            static_assert(SLICE < 0, "[PTO][SA] TLOAD slice: this tile geometry has no per-wave slices");
 #pragma unroll
             for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
                 const int s = s0 + wave;
@@ -176,6 +180,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             }
         }
     } else {
+        static_assert(SLICE < 0, "[PTO][SA] TLOAD slice: only for fully valid, unit-stride Mat tiles");
         // general path: element by element, pad outside the valid region (TLoad.hpp:151-152)
         const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
         const T pad = pad_value<T>(TileT::PadVal);
@@ -249,6 +254,17 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
 
 // Number of asynchronous global->LDS copy instructions that one TLOAD of a fully valid Mat tile
 // issues per wave (what wait_flag_pending counts).
+// One slice of a Mat tile's TLOAD: the SLICE-th of TLoadInstrs<TileT>() asynchronous copy instructions
+// of every wave (TLOAD == all slices).  Lets a kernel spread the copies of a tile over its
+// instruction stream, and lets the waves of a workgroup issue theirs at different points, so that
+// they do not queue up behind each other at the compute unit's one vector-memory address unit.
+template <int SLICE, typename TileT, typename G>
+PTO_DEV void TLOAD_SLICE(TileT &dst, G &src)
+{
+    static_assert(TileT::Loc == TileType::Mat, "[PTO][SA] TLOAD_SLICE: destination must be a Mat tile");
+    detail::tload_mat<SLICE>(dst, src);
+}
+
 template <typename TileT>
 constexpr int TLoadInstrs()
 {

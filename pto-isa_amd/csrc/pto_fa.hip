@@ -283,15 +283,15 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
         f16x8 frag[kAhead + 1];
         StaticFor<0, kAhead>([&](auto i) {
             constexpr int I = decltype(i)::value;
-            kr.template Issue<kOff, I / KSTEPS, I % KSTEPS>(frag[I % (kAhead + 1)]);
+            kr.template Issue<kOff, I % KB, I / KB>(frag[I % (kAhead + 1)]);
         });
         StaticFor<0, kTotal>([&](auto i) {
             constexpr int I = decltype(i)::value, J = I + kAhead;
             if constexpr (J < kTotal)
-                kr.template Issue<kOff, J / KSTEPS, J % KSTEPS>(frag[J % (kAhead + 1)]);
+                kr.template Issue<kOff, J % KB, J / KB>(frag[J % (kAhead + 1)]);
             between(i);
             KReader<D>::template Wait<(kTotal - 1 - I < kAhead ? kTotal - 1 - I : kAhead)>(frag[I % (kAhead + 1)]);
-            constexpr int kb = I / KSTEPS, ks = I % KSTEPS;
+            constexpr int kb = I % KB, ks = I / KB; // the KB accumulator chains alternate
             LeftStep a;
             RightStep b;
             a.st.f[0][0] = frag[I % (kAhead + 1)];
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
             alpha[nb] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nb] - newMax) * sLog2e);
             runMax[nb] = newMax;
             const float negMax = -newMax * sLog2e;
-            float locSum = 0.0f;
+            float part[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // four partial sums: no long chain of dependent additions
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -353,11 +353,12 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
                     for (int j = 0; j < 8; ++j) {
                         const float p =
                             __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][nb][half_ * 8 + j], sLog2e, negMax));
-                        locSum += p; // row sum over the fp32 P, as the reference does
+                        part[j & 3] += p; // row sum over the fp32 P, as the reference does
                         pk[j] = (half)p;
                     }
                     pRight.st.f[nb][kb * 2 + half_] = pk;
                 }
+            const float locSum = (part[0] + part[1]) + (part[2] + part[3]);
             runSum[nb] = t == 0 ? locSum : runSum[nb] * alpha[nb] + locSum;
         }
     };
@@ -420,8 +421,8 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
         constexpr int st = decltype(stageTag)::value;
         wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // tile t has landed; everyone left tile t-1
         // The next tile is fetched while this tile's score MFMAs issue: the K copies before the second
-        // MFMA, the V copies halfway, so that the wave never sits long in the vector-memory issue queue.
-        // Past the last tile the copies re-fetch it into the free stage, which keeps this a straight-line region.
+        // MFMA, the V copies halfway.  Past the last tile the copies re-fetch it into the free stage,
+        // which keeps the loop free of special cases.
         AccS sAcc[KB];
         __builtin_amdgcn_sched_barrier(0);
         scoreTile(sAcc, stageTag, [&](auto i) {
