@@ -22,6 +22,14 @@ for p in (ROOT, os.path.join(ROOT, "pto-isa_amd")):
 PEAK_FP16_TFLOPS = 2516.6   # MI355X dense fp16 matrix peak (published)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 
+# HBM-side traffic of one 6144^3 GEMM launch, from two rocprofv3 --pmc runs of this script
+# (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch of the GEMM kernel), each scaled by what the same
+# counter reads for a plain 1 GiB device copy in the same run (--calib-copy): FETCH_SIZE reads
+# 524,300 KiB for 1,048,576 KiB actually read (factor 2.0), WRITE_SIZE reads 1,048,576 KiB for
+# 1,048,576 KiB written (factor 1.0).
+GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369415.0, 2.0
+GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 147456.0, 1.0
+
 
 def time_launches(torch, fn, steps, warmup):
     """Average duration in ms of fn() over `steps` launches on torch's current stream (HIP events)."""
@@ -112,11 +120,11 @@ def bench_gather(torch, lib, capi, datagen, steps, warmup):
 
 def cpu_baseline(datagen, size):
     """The reference CPU-simulation arithmetic timed on the host cores, on a bounded sample of the
-    6144^3 product: rows [0,2048) of C (1/3 of the work) through the oracle's port of the tile path
+    6144^3 product: rows [0,4096) of C (2/3 of the work) through the oracle's port of the tile path
     (TLOAD/TEXTRACT/TMATMUL[_ACC] per K-step of 64), threads over rows as the reference does."""
     from oracle import oracle
     a, b = datagen.gemm_inputs(size, size, size)
-    rows = 2048
+    rows = 4096
     cores = oracle.online_cpus()
     cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else min(cores, int(os.environ["OMP_NUM_THREADS"]))
     t0 = time.perf_counter()
@@ -143,8 +151,8 @@ def cpu_baseline(datagen, size):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="gemm | fa | tcvt | gather: time just that workload")
     ap.add_argument("--size", type=int, default=6144)
@@ -207,10 +215,17 @@ def main():
                                "(256x256 C tile per workgroup, K-step 32)" % args.size},
         "extra": extra,
     }
+    traffic = None
+    if gemm and args.size == 6144:
+        rd = GEMM_6144_FETCH_KIB * GEMM_6144_FETCH_SCALE * 1024.0
+        wr = GEMM_6144_WRITE_KIB * GEMM_6144_WRITE_SCALE * 1024.0
+        traffic = rd + wr
     if gemm:
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
-                            "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": None,
-                            "kernel": "GemmF16F32Mix<256,256,4,4> (8 wavefronts per workgroup)", "flops_per_launch": gemm["flops"]}
+                            "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": traffic,
+                            "kernel": "GemmF16F32Mix<256,256,4,4> (8 wavefronts per workgroup)", "flops_per_launch": gemm["flops"],
+                            "traffic_unit": "bytes per launch (read + write at the L2 <-> fabric boundary)",
+                            "algorithmic_bytes": 2.0 * 2 * args.size ** 2 + 4.0 * args.size ** 2}
     if not args.no_cpu and only in ("", "gemm"):
         line["cpu_baseline"] = cpu_baseline(datagen, args.size)
     print(json.dumps(line))
