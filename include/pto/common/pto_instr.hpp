@@ -6,6 +6,7 @@
 #include "pto/gfx950/matmul.hpp"
 #include "pto/gfx950/mem_ops.hpp"
 #include "pto/gfx950/vec_ops.hpp"
+#include "pto/gfx950/vec_ops_ext.hpp"
 
 namespace pto {
 
@@ -48,7 +49,6 @@ PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T &obj)
 PTO_FRONT(TLOAD, typename TileT PTO_C typename G, TileT &dst PTO_C G &src, (dst, src))
 PTO_FRONT(TEXTRACT, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C uint16_t idxRow PTO_C uint16_t idxCol,
           (dst, src, idxRow, idxCol))
-PTO_FRONT(TMOV, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TMATMUL, typename C PTO_C typename A PTO_C typename B, C &c PTO_C A &a PTO_C B &b, (c, a, b))
 PTO_FRONT(TMATMUL_ACC, typename C PTO_C typename A PTO_C typename B, C &cOut PTO_C C &cIn PTO_C A &a PTO_C B &b,
           (cOut, cIn, a, b))
@@ -82,8 +82,56 @@ PTO_FRONT(TROWEXPANDDIV, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C
 PTO_FRONT(TROWEXPANDADD, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
 PTO_FRONT(TROWEXPANDMAX, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
 PTO_FRONT(TROWEXPANDMIN, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDEXPDIF, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPAND, typename D PTO_C typename R, D &dst PTO_C R &src, (dst, src))
+PTO_FRONT(TROWMIN, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
+PTO_FRONT(TCOLMAX, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TCOLMIN, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TCOLSUM, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TCOLEXPAND, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TCOLEXPANDSUB, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TCOLEXPANDMUL, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TCOLEXPANDDIV, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TCOLEXPANDADD, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TCOLEXPANDMAX, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TCOLEXPANDMIN, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TABS, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TNEG, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TRELU, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TSQRT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TRSQRT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TLOG, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TRECIP, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TPRELU, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TLRELU, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TCMP, typename T, T &dst PTO_C T &src0 PTO_C T &src1 PTO_C CmpMode mode, (dst, src0, src1, mode))
+PTO_FRONT(TCMPS, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src0 PTO_C T src1 PTO_C CmpMode mode,
+          (dst, src0, src1, mode))
+PTO_FRONT(TSEL, typename T PTO_C typename M, T &dst PTO_C M &selMask PTO_C T &src0 PTO_C T &src1, (dst, selMask, src0, src1))
+PTO_FRONT(TSELS, typename T, T &dst PTO_C T &src0 PTO_C T &src1 PTO_C uint8_t selectMode, (dst, src0, src1, selectMode))
+PTO_FRONT(TFILLPAD, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 #undef PTO_FRONT
 #undef PTO_C
+
+// TMOV (pto_instr.hpp:881-940): Mat -> Left / Right, register tile copies, and accumulator -> Vec with an
+// optional clamp at zero; the split mode over Vec cores is an Ascend hint
+template <typename D, typename S, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    if constexpr (S::Loc == TileType::Acc && D::Loc == TileType::Vec)
+        TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    else
+        TMOV_IMPL(dst, src);
+    return {};
+}
+template <typename D, typename S, AccToVecMode mode, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    return {};
+}
 
 // forms whose template arguments come first
 template <typename TileT, typename G, typename... Ev>

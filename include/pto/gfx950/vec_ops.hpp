@@ -246,7 +246,7 @@ PTO_DEV void TEXP_IMPL(TileT &dst, TileT &src)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = (typename TileT::DType)expf((float)src.st.v[s][i]);
+            dst.st.v[s][i] = (typename TileT::DType)::exp((double)src.st.v[s][i]); // evaluated in double: TExp.hpp:36
 }
 
 template <typename TileT>
@@ -294,7 +294,8 @@ PTO_DEV void TTRI_IMPL(TileT &dst, int diagonal)
 
 // --------------------------------------------------------- row reductions
 namespace detail {
-template <bool kMax, typename DstT, typename SrcT>
+// KIND: 0 sum, 1 maximum, 2 minimum
+template <int KIND, typename DstT, typename SrcT>
 PTO_DEV void row_reduce(DstT &dst, SrcT &src)
 {
     static_assert(SrcT::isRowMajor && SrcT::Loc == TileType::Vec && DstT::Loc == TileType::Vec,
@@ -311,12 +312,12 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
         const int q = s * kBlockThreads + hw::tid();
         if (q < S::Chunks) {
             const int c0 = (q % CPR) * kVecChunk;
-            A acc = kMax ? -__builtin_huge_valf() : 0.0f;
+            A acc = KIND == 1 ? -__builtin_huge_valf() : KIND == 2 ? __builtin_huge_valf() : 0.0f;
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
                 if (c0 + i < vc) {
                     const A v = (A)src.st.v[s][i];
-                    acc = kMax ? (acc < v ? v : acc) : acc + v;
+                    acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : acc + v;
                 }
             part[q] = acc;
         }
@@ -330,7 +331,7 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
                 A acc = part[r * CPR];
                 for (int j = 1; j < CPR; ++j) {
                     const A v = part[r * CPR + j];
-                    acc = kMax ? (acc < v ? v : acc) : acc + v;
+                    acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : acc + v;
                 }
                 dst.st.v[s][i] = (typename DstT::DType)acc;
             }
@@ -377,12 +378,12 @@ PTO_DEV void row_expand(DstT &dst, DstT &src0, RowT &src1)
 template <typename DstT, typename SrcT, typename TmpT>
 PTO_DEV void TROWMAX_IMPL(DstT &dst, SrcT &src, TmpT &)
 {
-    detail::row_reduce<true>(dst, src);
+    detail::row_reduce<1>(dst, src);
 }
 template <typename DstT, typename SrcT, typename TmpT>
 PTO_DEV void TROWSUM_IMPL(DstT &dst, SrcT &src, TmpT &)
 {
-    detail::row_reduce<false>(dst, src);
+    detail::row_reduce<0>(dst, src);
 }
 #define PTO_DEFINE_ROWEXPAND(NAME, OP)                                \
     template <typename DstT, typename RowT>                           \

@@ -1,0 +1,417 @@
+// Further Vec-tile instructions for gfx950: unary math, ReLU family, compare / select, column
+// reductions and broadcasts, row minimum / broadcast, TFILLPAD, and TMOV from an accumulator tile.
+// Semantics follow the reference's CPU simulation (file:line at each op).  Vec tiles are distributed
+// over the workgroup as in vec_ops.hpp; ops that cross lanes stage through small static LDS arrays.
+#pragma once
+#include "pto/gfx950/vec_ops.hpp"
+
+namespace pto {
+
+// ------------------------------------------------------------------ unary
+// The CPU simulation evaluates sqrt / log / exp in double and casts (ElementOp.h:265-340, TSqrt.hpp:23,
+// TRSqrt.hpp:30): the same is done here, these are not hot-loop ops.
+#define PTO_DEFINE_UNARY(NAME, EXPR)                                                                    \
+    template <typename DstT, typename SrcT>                                                             \
+    PTO_DEV void NAME##_IMPL(DstT &dst, SrcT &src)                                                      \
+    {                                                                                                   \
+        static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] " #NAME ": Vec tiles of equal size"); \
+        using T = typename DstT::DType;                                                                 \
+        using S = typename DstT::Storage;                                                               \
+        _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
+        {                                                                                               \
+            const T a = src.st.v[s][i];                                                                 \
+            dst.st.v[s][i] = (EXPR);                                                                    \
+        }                                                                                               \
+    }
+PTO_DEFINE_UNARY(TABS, (a < (T)0 ? -a : a))                                // TAbs.hpp:24
+PTO_DEFINE_UNARY(TNEG, -a)                                                 // ElementOp.h:297-302
+PTO_DEFINE_UNARY(TRELU, (a < (T)0 ? (T)0 : a))                             // ElementOp.h:345-350 (max(a, 0))
+PTO_DEFINE_UNARY(TSQRT, (T)::sqrt((double)a))                      // TSqrt.hpp:23
+PTO_DEFINE_UNARY(TRSQRT, (T)(1.0 / ::sqrt((double)a)))             // TRSqrt.hpp:29-31
+PTO_DEFINE_UNARY(TLOG, (T)::log((double)a))                        // ElementOp.h:289-294
+PTO_DEFINE_UNARY(TRECIP, (T)((T)1 / a))                                    // ElementOp.h:321-330
+#undef PTO_DEFINE_UNARY
+
+// dst = src0 > 0 ? src0 : src0 * src1  (ElementOp.h:257-262)
+template <typename DstT, typename S0T, typename S1T>
+PTO_DEV void TPRELU_IMPL(DstT &dst, S0T &src0, S1T &src1)
+{
+    static_assert(detail::same_dist<DstT, S0T> && detail::same_dist<DstT, S1T>, "[PTO][SA] TPRELU: Vec tiles of equal size");
+    using T = typename DstT::DType;
+    using S = typename DstT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i) {
+            const T a = src0.st.v[s][i], b = src1.st.v[s][i];
+            dst.st.v[s][i] = a > (T)0 ? a : (T)(a * b);
+        }
+}
+// dst = src > 0 ? src : src * k  (ElementOp.h:503-508)
+template <typename DstT, typename SrcT>
+PTO_DEV void TLRELU_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)
+{
+    static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] TLRELU: Vec tiles of equal size");
+    using T = typename DstT::DType;
+    using S = typename DstT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i) {
+            const T a = src.st.v[s][i];
+            dst.st.v[s][i] = a > (T)0 ? a : (T)(a * k);
+        }
+}
+
+// ------------------------------------------------------------ compare / select
+namespace detail {
+template <typename T>
+PTO_DEV bool cmp_exact(T a, T b, CmpMode mode)
+{
+    switch (mode) {
+    case CmpMode::EQ: return a == b;
+    case CmpMode::NE: return a != b;
+    case CmpMode::LT: return a < b;
+    case CmpMode::LE: return a <= b;
+    case CmpMode::GT: return a > b;
+    case CmpMode::GE: return a >= b;
+    }
+    return a == b;
+}
+// TCMPS compares with a tolerance for EQ / NE: |a - b| < 1e-9 in double (TCmps.hpp:28-37)
+template <typename T>
+PTO_DEV bool cmp_scalar(T a, T b, CmpMode mode)
+{
+    const double diff = (double)a - (double)b;
+    const double ad = diff < 0 ? -diff : diff;
+    switch (mode) {
+    case CmpMode::EQ: return ad < 1e-9;
+    case CmpMode::NE: return ad > 1e-9;
+    case CmpMode::LT: return a < b;
+    case CmpMode::GT: return a > b;
+    case CmpMode::GE: return a >= b;
+    case CmpMode::LE: return a <= b;
+    }
+    return ad < 1e-9;
+}
+} // namespace detail
+
+// dst = (src0 <mode> src1) as 0 / 1 in the tiles' own type (ElementTileOp.h:178-184, ElementOp.h:227-253)
+template <typename TileT>
+PTO_DEV void TCMP_IMPL(TileT &dst, TileT &src0, TileT &src1, CmpMode mode)
+{
+    using T = typename TileT::DType;
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = detail::cmp_exact<T>(src0.st.v[s][i], src1.st.v[s][i], mode) ? (T)1 : (T)0;
+}
+
+// Packed form: bit (c % 8) of byte c / 8 of row r of dst = (src0[r,c] <mode> scalar); dst is a
+// uint8 tile with the source's rows whose first Cols/8 columns receive the bytes (TCmps.hpp:50-90 with
+// dst valid columns = Cols / 8, the shape its test uses).  A chunk of 8 elements is one byte.
+template <typename DstT, typename SrcT, typename T>
+PTO_DEV void TCMPS_IMPL(DstT &dst, SrcT &src0, T scalar, CmpMode mode)
+{
+    static_assert(sizeof(typename DstT::DType) == 1 && SrcT::isRowMajor && DstT::isRowMajor && SrcT::Cols % 8 == 0 &&
+                      DstT::Rows == SrcT::Rows && DstT::Cols >= SrcT::Cols / 8,
+                  "[PTO][SA] TCMPS: uint8 destination with the source's rows, source columns a multiple of 8");
+    using S = typename SrcT::Storage;
+    constexpr int kBytes = SrcT::Rows * (SrcT::Cols / 8);
+    __shared__ uint8_t packed[kBytes];
+    const int vr = src0.GetValidRow(), vc = src0.GetValidCol();
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+        if (q < S::Chunks) {
+            const int r = (q * 8) / SrcT::Cols, c0 = (q * 8) % SrcT::Cols;
+            uint32_t byte = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (r < vr && c0 + i < vc && detail::cmp_scalar<typename SrcT::DType>(src0.st.v[s][i], (typename SrcT::DType)scalar, mode))
+                    byte |= 1u << i;
+            packed[q] = (uint8_t)byte;
+        }
+    }
+    hw::lds_barrier();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && c < SrcT::Cols / 8)
+            dst.st.v[s][i] = packed[r * (SrcT::Cols / 8) + c];
+    });
+    hw::lds_barrier();
+}
+
+// dst[i,j] = bit ? src0[i,j] : src1[i,j]; the bits are consumed in running order over the valid
+// region, byte after byte along the mask tile's valid columns, then its next row (TSel.hpp:22-49).
+template <typename TileT, typename MaskT>
+PTO_DEV void TSEL_IMPL(TileT &dst, MaskT &selMask, TileT &src0, TileT &src1)
+{
+    static_assert(sizeof(typename MaskT::DType) == 1 && TileT::isRowMajor && MaskT::isRowMajor,
+                  "[PTO][SA] TSEL: row-major tiles, byte mask");
+    __shared__ uint8_t bits[MaskT::Numel];
+    detail::for_each_owned<MaskT>([&](int s, int i, int e) {
+        if (e < MaskT::Numel)
+            bits[e] = (uint8_t)selMask.st.v[s][i];
+    });
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol(), vmc = selMask.GetValidCol();
+    detail::for_each_owned<TileT>([&](int s, int i, int e) {
+        const int r = e / TileT::Cols, c = e % TileT::Cols;
+        if (e < TileT::Numel && r < vr && c < vc) {
+            const int k = r * vc + c, b = k >> 3;
+            const uint32_t byte = bits[(b / vmc) * MaskT::Cols + (b % vmc)];
+            dst.st.v[s][i] = ((byte >> (k & 7)) & 1u) ? src0.st.v[s][i] : src1.st.v[s][i];
+        }
+    });
+    hw::lds_barrier();
+}
+
+// dst = selectMode == 1 ? src0 : src1 for the whole tile (TSelS.hpp:20-41)
+template <typename TileT>
+PTO_DEV void TSELS_IMPL(TileT &dst, TileT &src0, TileT &src1, uint8_t selectMode)
+{
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = selectMode == 1 ? src0.st.v[s][i] : src1.st.v[s][i];
+}
+
+// ------------------------------------------------------------------ TFILLPAD
+// dst = src inside the source's valid region, the destination's pad value elsewhere, over the whole
+// tile (TFillPad.hpp:22-49; Max / Min pad = +/- infinity for floating types).
+template <typename DstT, typename SrcT>
+PTO_DEV void TFILLPAD_IMPL(DstT &dst, SrcT &src)
+{
+    static_assert(DstT::Rows == SrcT::Rows && DstT::Cols == SrcT::Cols && sizeof(typename DstT::DType) == sizeof(typename SrcT::DType),
+                  "[PTO][SA] TFILLPAD: same shape and element size");
+    static_assert(DstT::PadVal != PadValue::Null, "[PTO][SA] TFILLPAD: the destination tile needs a pad value");
+    using T = typename DstT::DType;
+    const T pad = detail::pad_value<T>(DstT::PadVal);
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        int r, c;
+        detail::elem_rc<DstT>(e, r, c);
+        if (e < DstT::Numel)
+            dst.st.v[s][i] = (r < vr && c < vc) ? __builtin_bit_cast(T, src.st.v[s][i]) : pad;
+    });
+}
+
+// ------------------------------------------------------- column reductions
+namespace detail {
+enum class Red { Max, Min, Sum };
+// One value per column into a [1, Cols] tile.  A lane owns the same 8 columns in every slot (the
+// number of chunks per row divides the workgroup size); its rows are g, g + G, g + 2G, ... for its
+// group g of G = threads / chunks-per-row.  Per-lane partials over its rows, then the G partials of a
+// column are combined in order of g.  Max / min are exact; the sum adds in this order, the CPU
+// simulation in row order (TColSum.hpp:22-30).
+template <Red red, typename DstT, typename SrcT>
+PTO_DEV void col_reduce(DstT &dst, SrcT &src)
+{
+    static_assert(SrcT::isRowMajor && SrcT::Cols % kVecChunk == 0 && DstT::Rows == 1 && DstT::Cols == SrcT::Cols,
+                  "[PTO][SA] column reduction: row-major source, [1, Cols] destination");
+    constexpr int CPR = SrcT::Cols / kVecChunk;
+    static_assert(CPR <= kBlockThreads && kBlockThreads % CPR == 0, "[PTO][SA] column reduction: chunks per row must divide the workgroup size");
+    constexpr int G = kBlockThreads / CPR;
+    using S = typename SrcT::Storage;
+    using A = float;
+    __shared__ A part[G][SrcT::Cols];
+    const int vr = src.GetValidRow();
+    const int g = hw::tid() / CPR, c0 = (hw::tid() % CPR) * kVecChunk;
+    A acc[kVecChunk];
+    bool any = false;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int r = s * G + g;
+        if (r < vr && r < SrcT::Rows) {
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i) {
+                const A v = (A)src.st.v[s][i];
+                if (!any)
+                    acc[i] = v;
+                else if (red == Red::Max)
+                    acc[i] = acc[i] < v ? v : acc[i];
+                else if (red == Red::Min)
+                    acc[i] = v < acc[i] ? v : acc[i];
+                else
+                    acc[i] += v;
+            }
+            any = true;
+        }
+    }
+    __shared__ int has[G];
+    if (hw::tid() % CPR == 0)
+        has[g] = any ? 1 : 0;
+    if (any) {
+#pragma unroll
+        for (int i = 0; i < kVecChunk; ++i)
+            part[g][c0 + i] = acc[i];
+    }
+    hw::lds_barrier();
+    const int vc = src.GetValidCol();
+    for_each_owned<DstT>([&](int s, int i, int e) {
+        if (e < DstT::Numel && e < vc && vr > 0) {
+            A a = part[0][e];
+            for (int k = 1; k < G; ++k)
+                if (has[k]) {
+                    const A v = part[k][e];
+                    a = red == Red::Max ? (a < v ? v : a) : red == Red::Min ? (v < a ? v : a) : a + v;
+                }
+            dst.st.v[s][i] = (typename DstT::DType)a;
+        }
+    });
+    hw::lds_barrier();
+}
+
+enum class ColOp { Copy, Sub, Mul, Div, Add, Max, Min };
+// dst[i,j] = src0[i,j] <op> src1[0,j]  (TColExpand.hpp:22-33, TColExpandOp.hpp)
+template <ColOp op, typename DstT, typename ColT>
+PTO_DEV void col_expand(DstT &dst, DstT &src0, ColT &src1)
+{
+    static_assert(DstT::isRowMajor && ColT::Rows == 1 && ColT::Cols == DstT::Cols, "[PTO][SA] column broadcast: [1, Cols] source");
+    using T = typename DstT::DType;
+    __shared__ typename ColT::DType colv[DstT::Cols];
+    for_each_owned<ColT>([&](int s, int i, int e) {
+        if (e < ColT::Numel)
+            colv[e] = src1.st.v[s][i];
+    });
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && r < vr && c < vc) {
+            const T a = src0.st.v[s][i], b = (T)colv[c];
+            T o;
+            if constexpr (op == ColOp::Copy)
+                o = b;
+            else if constexpr (op == ColOp::Sub)
+                o = a - b;
+            else if constexpr (op == ColOp::Mul)
+                o = a * b;
+            else if constexpr (op == ColOp::Div)
+                o = a / b;
+            else if constexpr (op == ColOp::Add)
+                o = a + b;
+            else if constexpr (op == ColOp::Max)
+                o = a < b ? b : a;
+            else
+                o = b < a ? b : a;
+            dst.st.v[s][i] = o;
+        }
+    });
+    hw::lds_barrier();
+}
+} // namespace detail
+
+template <typename DstT, typename SrcT>
+PTO_DEV void TCOLMAX_IMPL(DstT &dst, SrcT &src) { detail::col_reduce<detail::Red::Max>(dst, src); } // TColMax.hpp:22-35
+template <typename DstT, typename SrcT>
+PTO_DEV void TCOLMIN_IMPL(DstT &dst, SrcT &src) { detail::col_reduce<detail::Red::Min>(dst, src); } // TColMin.hpp
+template <typename DstT, typename SrcT>
+PTO_DEV void TCOLSUM_IMPL(DstT &dst, SrcT &src) { detail::col_reduce<detail::Red::Sum>(dst, src); } // TColSum.hpp:22-31
+template <typename DstT, typename SrcT, typename TmpT>
+PTO_DEV void TCOLSUM_IMPL(DstT &dst, SrcT &src, TmpT &, bool) { detail::col_reduce<detail::Red::Sum>(dst, src); }
+
+template <typename DstT, typename ColT>
+PTO_DEV void TCOLEXPAND_IMPL(DstT &dst, ColT &src) { detail::col_expand<detail::ColOp::Copy>(dst, dst, src); }
+#define PTO_DEFINE_COLEXPAND(NAME, OP)                                \
+    template <typename DstT, typename ColT>                           \
+    PTO_DEV void NAME##_IMPL(DstT &dst, DstT &src0, ColT &src1)       \
+    {                                                                 \
+        detail::col_expand<detail::ColOp::OP>(dst, src0, src1);       \
+    }
+PTO_DEFINE_COLEXPAND(TCOLEXPANDSUB, Sub)
+PTO_DEFINE_COLEXPAND(TCOLEXPANDMUL, Mul)
+PTO_DEFINE_COLEXPAND(TCOLEXPANDDIV, Div)
+PTO_DEFINE_COLEXPAND(TCOLEXPANDADD, Add)
+PTO_DEFINE_COLEXPAND(TCOLEXPANDMAX, Max)
+PTO_DEFINE_COLEXPAND(TCOLEXPANDMIN, Min)
+#undef PTO_DEFINE_COLEXPAND
+
+// ------------------------------------------------ more row reductions / broadcasts
+// row minimum (TRowMin.hpp:22-58); exact
+template <typename DstT, typename SrcT, typename TmpT>
+PTO_DEV void TROWMIN_IMPL(DstT &dst, SrcT &src, TmpT &)
+{
+    detail::row_reduce<2>(dst, src);
+}
+
+// dst[i,j] = src[i]  (TRowExpand.hpp) and dst[i,j] = exp(src0[i,j] - src1[i]) with the exponential
+// evaluated in double (TRowExpandOp.hpp:93-96, ElementOp.h:265-270)
+template <typename DstT, typename RowT>
+PTO_DEV void TROWEXPAND_IMPL(DstT &dst, RowT &src)
+{
+    static_assert(DstT::isRowMajor, "[PTO][SA] TROWEXPAND: row-major destination");
+    __shared__ typename RowT::DType rowv[DstT::Rows];
+    detail::stage_row_values<RowT, DstT::Rows>(src, rowv);
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && r < vr && c < vc)
+            dst.st.v[s][i] = (typename DstT::DType)rowv[r];
+    });
+    hw::lds_barrier();
+}
+template <typename DstT, typename RowT>
+PTO_DEV void TROWEXPANDEXPDIF_IMPL(DstT &dst, DstT &src0, RowT &src1)
+{
+    static_assert(DstT::isRowMajor, "[PTO][SA] TROWEXPANDEXPDIF: row-major tiles");
+    using T = typename DstT::DType;
+    __shared__ typename RowT::DType rowv[DstT::Rows];
+    detail::stage_row_values<RowT, DstT::Rows>(src1, rowv);
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && r < vr && c < vc) {
+            const T d = src0.st.v[s][i] - (T)rowv[r];
+            dst.st.v[s][i] = (T)::exp((double)d);
+        }
+    });
+    hw::lds_barrier();
+}
+
+// ------------------------------------------------------- TMOV Acc -> Vec
+// Same-shape copy of an accumulator tile into a Vec tile, optionally clamped at zero
+// (TMov.hpp:20-69).  The accumulator's per-wave MFMA layout is redistributed through LDS.
+template <ReluPreMode relu = ReluPreMode::NoRelu, typename DstT, typename AccT>
+PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
+{
+    static_assert(AccT::Loc == TileType::Acc && DstT::Loc == TileType::Vec && DstT::isRowMajor && DstT::Rows == AccT::Rows &&
+                      DstT::Cols == AccT::Cols && sizeof(typename DstT::DType) == 4 && sizeof(typename AccT::DType) == 4,
+                  "[PTO][SA] TMOV Acc->Vec: row-major fp32 Vec tile of the accumulator's shape");
+    using S = typename AccT::Storage;
+    using T = typename DstT::DType;
+    __shared__ T stage[AccT::Rows * AccT::Cols];
+    const uint32_t lane = (uint32_t)hw::lane();
+    const int rbase = hw::wave_m() * (S::MB * detail::kMfmaM) + (int)(lane >> 5) * 4;
+    const int cbase = hw::wave_n() * (S::NB * detail::kMfmaM) + (int)(lane & 31u);
+#pragma unroll
+    for (int mb = 0; mb < S::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < S::NB; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int r = rbase + mb * detail::kMfmaM + (v >> 2) * 8 + (v & 3), c = cbase + nb * detail::kMfmaM;
+                stage[r * AccT::Cols + c] = (T)src.st.f[mb][nb][v];
+            }
+    hw::lds_barrier();
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && r < vr && c < vc) {
+            T v = stage[e];
+            if (relu == ReluPreMode::NormalRelu && v < (T)0)
+                v = (T)0;
+            dst.st.v[s][i] = v;
+        }
+    });
+    hw::lds_barrier();
+}
+
+} // namespace pto

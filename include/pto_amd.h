@@ -113,6 +113,37 @@ int pto_st_textract_windows_f16(void *stream, float *out_left, float *out_right,
 int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, const float *bias,
                                   int bf16);
 
+/* One Vec instruction on [64,128] fp32 tiles: out = OP(a [, b | scalar | vec]).  vec is a per-row [64] operand for
+ * the TROWEXPAND* ops and a per-column [128] operand for the TCOLEXPAND* ops.  op codes (PTO_VOP_*): unary
+ * (cpu/TAbs.hpp, TSqrt.hpp, TRSqrt.hpp, ElementOp.h:273-350), binary incl. TPRELU and TCMP with 0/1 results
+ * (ElementTileOp.h:170-238), scalar incl. TLRELU (ElementTileScalarOp.h), TSELS (scalar = select mode, TSelS.hpp),
+ * row broadcasts (TRowExpand.hpp, TRowExpandOp.hpp:57-96), column broadcasts (TColExpand.hpp, TColExpandOp.hpp). */
+enum {
+    PTO_VOP_ABS = 0, PTO_VOP_NEG, PTO_VOP_RELU, PTO_VOP_SQRT, PTO_VOP_RSQRT, PTO_VOP_LOG, PTO_VOP_RECIP, PTO_VOP_EXP,
+    PTO_VOP_ADD = 20, PTO_VOP_SUB, PTO_VOP_MUL, PTO_VOP_DIV, PTO_VOP_MAX, PTO_VOP_MIN, PTO_VOP_PRELU,
+    PTO_VOP_CMP_EQ, PTO_VOP_CMP_NE, PTO_VOP_CMP_LT, PTO_VOP_CMP_LE, PTO_VOP_CMP_GT, PTO_VOP_CMP_GE, PTO_VOP_SELS,
+    PTO_VOP_ADDS = 40, PTO_VOP_SUBS, PTO_VOP_MULS, PTO_VOP_DIVS, PTO_VOP_MAXS, PTO_VOP_MINS, PTO_VOP_LRELU,
+    PTO_VOP_ROWEXPAND = 60, PTO_VOP_ROWEXPANDSUB, PTO_VOP_ROWEXPANDMUL, PTO_VOP_ROWEXPANDDIV, PTO_VOP_ROWEXPANDADD,
+    PTO_VOP_ROWEXPANDMAX, PTO_VOP_ROWEXPANDMIN, PTO_VOP_ROWEXPANDEXPDIF,
+    PTO_VOP_COLEXPAND = 80, PTO_VOP_COLEXPANDSUB, PTO_VOP_COLEXPANDMUL, PTO_VOP_COLEXPANDDIV, PTO_VOP_COLEXPANDADD,
+    PTO_VOP_COLEXPANDMAX, PTO_VOP_COLEXPANDMIN
+};
+int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const float *b, const float *vec, float scalar, int op);
+/* Reductions over the valid region [valid_rows, valid_cols] of a [64,128] fp32 tile (row stride 128 in memory):
+ * op 0 TROWMAX, 1 TROWMIN, 2 TROWSUM -> out[valid_rows]; 3 TCOLMAX, 4 TCOLMIN, 5 TCOLSUM -> out[valid_cols]
+ * (cpu/TRowMax.hpp, TRowMin.hpp, TRowSum.hpp, TColMax.hpp, TColMin.hpp, TColSum.hpp). */
+int pto_st_reduce_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int op);
+/* TCMPS then TSEL on [64,128] fp32 tiles: bits[64][16] = packed (a <cmp_mode> scalar), bit c%8 of byte c/8
+ * (cpu/TCmps.hpp:50-90; EQ / NE within 1e-9); sel = bit ? a : b (cpu/TSel.hpp:22-49).  cmp_mode 0..5 = EQ NE LT LE GT GE. */
+int pto_st_cmps_sel_f32_64x128(void *stream, float *sel, uint8_t *bits, const float *a, const float *b, float scalar,
+                               int cmp_mode);
+/* TFILLPAD: out[64,128] = a inside [valid_rows, valid_cols], the pad value elsewhere; pad_kind 1 zero, 2 +inf, 3 -inf
+ * (cpu/TFillPad.hpp:22-49). */
+int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int pad_kind);
+/* out[64,128] = scale * (relu ? max(a b, 0) : a b): fp16 matmul [64,64] x [64,128] (b_t stored [128][64]), TMOV of
+ * the accumulator into a Vec tile with ReluPreMode (cpu/TMov.hpp:53-69), TMULS, TSTORE. */
+int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, int relu, float scale);
+
 #ifdef __cplusplus
 }
 #endif

@@ -70,6 +70,18 @@ def lib():
         L.po_result_cmp_f32.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.POINTER(C.c_double),
                                         C.POINTER(C.c_size_t)]
         L.po_result_cmp_f32.restype = C.c_int
+        L.po_vec_op.argtypes = [C.c_void_p] * 4 + [C.c_float] + [C.c_int] * 4
+        L.po_vec_op.restype = None
+        L.po_reduce.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 4
+        L.po_reduce.restype = None
+        L.po_tcmps_packed.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int]
+        L.po_tcmps_packed.restype = None
+        L.po_tsel_packed.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p] + [C.c_int] * 3
+        L.po_tsel_packed.restype = None
+        L.po_tfillpad.argtypes = [C.c_void_p, C.c_void_p] + [C.c_int] * 6
+        L.po_tfillpad.restype = None
+        L.po_tmov_relu.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+        L.po_tmov_relu.restype = None
         _lib = L
     return _lib
 
@@ -252,3 +264,65 @@ def result_cmp(expect, actual, eps):
     nb = C.c_size_t()
     ok = lib().po_result_cmp_f32(_p(e), _p(a), e.size, eps, C.byref(md), C.byref(nb))
     return bool(ok), md.value, nb.value
+
+
+# ------------------------------------------------- further Vec instructions
+VOP = dict(ABS=0, NEG=1, RELU=2, SQRT=3, RSQRT=4, LOG=5, RECIP=6, EXP=7,
+           ADD=20, SUB=21, MUL=22, DIV=23, MAX=24, MIN=25, PRELU=26, CMP_EQ=27, CMP_NE=28, CMP_LT=29, CMP_LE=30, CMP_GT=31,
+           CMP_GE=32, SELS=33, ADDS=40, SUBS=41, MULS=42, DIVS=43, MAXS=44, MINS=45, LRELU=46,
+           ROWEXPAND=60, ROWEXPANDSUB=61, ROWEXPANDMUL=62, ROWEXPANDDIV=63, ROWEXPANDADD=64, ROWEXPANDMAX=65, ROWEXPANDMIN=66,
+           ROWEXPANDEXPDIF=67, COLEXPAND=80, COLEXPANDSUB=81, COLEXPANDMUL=82, COLEXPANDDIV=83, COLEXPANDADD=84,
+           COLEXPANDMAX=85, COLEXPANDMIN=86)
+
+
+def vec_op(op, a, b=None, vec=None, scalar=0.0):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    rows, cols = a.shape
+    out = np.empty_like(a)
+    b = None if b is None else np.ascontiguousarray(b, dtype=np.float32)
+    vec = None if vec is None else np.ascontiguousarray(vec, dtype=np.float32)
+    lib().po_vec_op(_p(out), _p(a), None if b is None else _p(b), None if vec is None else _p(vec), float(scalar),
+                    VOP[op] if isinstance(op, str) else int(op), cols, rows, cols)
+    return out
+
+
+def reduce(op, a):
+    """op 0 TROWMAX, 1 TROWMIN, 2 TROWSUM, 3 TCOLMAX, 4 TCOLMIN, 5 TCOLSUM over the whole array."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    rows, cols = a.shape
+    out = np.empty(rows if op < 3 else cols, dtype=np.float32)
+    lib().po_reduce(_p(out), _p(a), cols, rows, cols, op)
+    return out
+
+
+def tcmps_packed(a, scalar, mode):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    rows, cols = a.shape
+    out = np.zeros((rows, cols // 8), dtype=np.uint8)
+    lib().po_tcmps_packed(_p(out), cols // 8, _p(a), cols, rows, cols, float(scalar), mode)
+    return out
+
+
+def tsel_packed(mask, mask_valid_cols, a, b):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    mask = np.ascontiguousarray(mask, dtype=np.uint8)
+    rows, cols = a.shape
+    out = np.empty_like(a)
+    lib().po_tsel_packed(_p(out), _p(mask), mask.shape[1], mask_valid_cols, _p(a), _p(b), cols, rows, cols)
+    return out
+
+
+def tfillpad(a, vr, vc, pad_kind):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    rows, cols = a.shape
+    out = np.empty_like(a)
+    lib().po_tfillpad(_p(out), _p(a), cols, rows, cols, vr, vc, pad_kind)
+    return out
+
+
+def tmov_relu(x, relu):
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    lib().po_tmov_relu(_p(out), _p(x), x.size, int(relu))
+    return out

@@ -797,3 +797,151 @@ int po_result_cmp_f32(const float *expect, const float *actual, size_t n, float 
         *n_bad = bad;
     return bad <= (size_t)((double)n * eps) && zero <= 1000;
 }
+
+/* ------------------------------------------------- further Vec instructions */
+static int po_cmp(float a, float b, int mode)
+{ /* ElementOp.h:227-253; CmpMode EQ NE LT LE GT GE = 0..5 (common/type.hpp:131-139) */
+    switch (mode) {
+    case 0: return a == b;
+    case 1: return a != b;
+    case 2: return a < b;
+    case 3: return a <= b;
+    case 4: return a > b;
+    case 5: return a >= b;
+    default: return a == b;
+    }
+}
+
+void po_vec_op(float *dst, const float *a, const float *b, const float *vec, float k, int op, int ld, int rows, int cols)
+{
+    for (int r = 0; r < rows; r++)
+        for (int c = 0; c < cols; c++) {
+            size_t x = (size_t)r * (size_t)ld + (size_t)c;
+            float v = a[x], w = (op >= 20 && op < 40) ? b[x] : 0.0f, o;
+            float rv = (op >= 60 && op < 80) ? vec[r] : 0.0f, cv = op >= 80 ? vec[c] : 0.0f;
+            switch (op) {
+            case 0: o = v < 0 ? -v : v; break;                          /* TAbs.hpp:24 */
+            case 1: o = -v; break;                                      /* ElementOp.h:297-302 */
+            case 2: o = v < 0.0f ? 0.0f : v; break;                     /* std::max(src, 0): ElementOp.h:345-350 */
+            case 3: o = (float)sqrt((double)v); break;                  /* TSqrt.hpp:23 */
+            case 4: o = (float)(1.0 / sqrt((double)v)); break;          /* TRSqrt.hpp:29-31 */
+            case 5: o = (float)log((double)v); break;                   /* ElementOp.h:289-294 */
+            case 6: o = 1.0f / v; break;                                /* TRECIP = TDIVS(dst, 1, src): pto_instr.hpp:296-304 */
+            case 7: o = (float)exp((double)v); break;                   /* TExp.hpp:36 */
+            case 20: o = v + w; break;
+            case 21: o = v - w; break;
+            case 22: o = v * w; break;
+            case 23: o = v / w; break;
+            case 24: o = v < w ? w : v; break;                          /* std::max */
+            case 25: o = w < v ? w : v; break;                          /* std::min */
+            case 26: o = v > 0.0f ? v : v * w; break;                   /* ElementOp.h:257-262 */
+            case 27: case 28: case 29: case 30: case 31: case 32: o = (float)po_cmp(v, w, op - 27); break;
+            case 33: o = (k == 1.0f) ? v : w; break;                    /* TSelS.hpp:20-31 */
+            case 40: o = v + k; break;
+            case 41: o = v - k; break;
+            case 42: o = v * k; break;
+            case 43: o = v / k; break;
+            case 44: o = v < k ? k : v; break;
+            case 45: o = k < v ? k : v; break;
+            case 46: o = v > 0.0f ? v : v * k; break;                   /* ElementOp.h:503-508 */
+            case 60: o = rv; break;                                     /* TRowExpand.hpp */
+            case 61: o = v - rv; break;
+            case 62: o = v * rv; break;
+            case 63: o = v / rv; break;
+            case 64: o = v + rv; break;
+            case 65: o = v < rv ? rv : v; break;
+            case 66: o = rv < v ? rv : v; break;
+            case 67: o = (float)exp((double)(v - rv)); break;           /* ElementOp.h:265-270 */
+            case 80: o = cv; break;                                     /* TColExpand.hpp:22-33 */
+            case 81: o = v - cv; break;
+            case 82: o = v * cv; break;
+            case 83: o = v / cv; break;
+            case 84: o = v + cv; break;
+            case 85: o = v < cv ? cv : v; break;
+            case 86: o = cv < v ? cv : v; break;
+            default: o = 0.0f; break;
+            }
+            dst[x] = o;
+        }
+}
+
+void po_reduce(float *dst, const float *a, int ld, int rows, int cols, int op)
+{
+    if (op < 3) {
+        for (int i = 0; i < rows; i++) {
+            float acc = op == 2 ? 0.0f : a[(size_t)i * (size_t)ld];
+            for (int j = (op == 2 ? 0 : 1); j < cols; j++) {
+                float v = a[(size_t)i * (size_t)ld + (size_t)j];
+                acc = op == 0 ? (acc < v ? v : acc) : op == 1 ? (v < acc ? v : acc) : acc + v;
+            }
+            dst[i] = acc;
+        }
+    } else {
+        for (int j = 0; j < cols; j++) {
+            float acc = op == 5 ? 0.0f : a[j];
+            for (int i = (op == 5 ? 0 : 1); i < rows; i++) {
+                float v = a[(size_t)i * (size_t)ld + (size_t)j];
+                acc = op == 3 ? (v > acc ? v : acc) : op == 4 ? (v < acc ? v : acc) : acc + v; /* TColMax.hpp:27-33, TColSum.hpp:25-28 */
+            }
+            dst[j] = acc;
+        }
+    }
+}
+
+void po_tcmps_packed(uint8_t *dst, int dst_ld, const float *a, int ld, int rows, int cols, float scalar, int mode)
+{
+    for (int r = 0; r < rows; r++)
+        for (int cb = 0; cb < cols / 8; cb++) {
+            unsigned byte = 0;
+            for (int bit = 0; bit < 8; bit++) {
+                float v = a[(size_t)r * (size_t)ld + (size_t)(cb * 8 + bit)];
+                double diff = (double)v - (double)scalar; /* TCmps.hpp:28 */
+                int res;
+                switch (mode) {
+                case 0: res = fabs(diff) < 1e-9; break;
+                case 1: res = fabs(diff) > 1e-9; break;
+                case 2: res = v < scalar; break;
+                case 3: res = v <= scalar; break;
+                case 4: res = v > scalar; break;
+                case 5: res = v >= scalar; break;
+                default: res = fabs(diff) < 1e-9; break;
+                }
+                byte |= (unsigned)res << bit; /* TCmps.hpp:71-76 */
+            }
+            dst[(size_t)r * (size_t)dst_ld + (size_t)cb] = (uint8_t)byte;
+        }
+}
+
+void po_tsel_packed(float *dst, const uint8_t *mask, int mask_ld, int mask_valid_cols, const float *a, const float *b, int ld,
+                    int rows, int cols)
+{
+    size_t mr = 0, mc = 0;
+    unsigned bit = 0;
+    for (int i = 0; i < rows; i++)
+        for (int j = 0; j < cols; j++) { /* TSel.hpp:27-47 */
+            size_t x = (size_t)i * (size_t)ld + (size_t)j;
+            unsigned sel = (mask[mr * (size_t)mask_ld + mc] >> bit) & 1u;
+            if (++bit == 8) {
+                bit = 0;
+                if (++mc == (size_t)mask_valid_cols) {
+                    mr++;
+                    mc = 0;
+                }
+            }
+            dst[x] = sel ? a[x] : b[x];
+        }
+}
+
+void po_tfillpad(float *dst, const float *a, int ld, int rows, int cols, int vr, int vc, int pad_kind)
+{
+    float pad = pad_kind == 2 ? INFINITY : pad_kind == 3 ? -INFINITY : 0.0f; /* TFillPad.hpp:26-38 */
+    for (int i = 0; i < rows; i++)
+        for (int j = 0; j < cols; j++)
+            dst[(size_t)i * (size_t)ld + (size_t)j] = (i < vr && j < vc) ? a[(size_t)i * (size_t)ld + (size_t)j] : pad;
+}
+
+void po_tmov_relu(float *dst, const float *src, size_t n, int relu)
+{
+    for (size_t i = 0; i < n; i++)
+        dst[i] = (relu && src[i] < 0.0f) ? 0.0f : src[i]; /* TMov.hpp:57-67 */
+}

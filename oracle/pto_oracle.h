@@ -147,6 +147,24 @@ int po_result_cmp_f32(const float *expect, const float *actual, size_t n, float 
 
 int po_online_cpus(void);
 
+
+/* ---- further Vec instructions (plain row-major fp32 arrays, leading dimension ld) ----
+ * Parity: pinned against the compiled reference (oracle/_ref, tests/test_oracle_vec_ext.py) and against numpy
+ * closed forms.  op codes are the PTO_VOP_* values of include/pto_amd.h. */
+void po_vec_op(float *dst, const float *a, const float *b, const float *vec, float scalar, int op, int ld, int rows,
+               int cols); /* cpu/ElementOp.h:77-535, TAbs.hpp, TSqrt.hpp, TRSqrt.hpp, TRowExpandOp.hpp:36-96, TColExpandOp.hpp, TSelS.hpp */
+/* op 0 TROWMAX, 1 TROWMIN, 2 TROWSUM (dst[rows]); 3 TCOLMAX, 4 TCOLMIN, 5 TCOLSUM (dst[cols]); sequential order */
+void po_reduce(float *dst, const float *a, int ld, int rows, int cols, int op); /* cpu/TRowMax.hpp, TRowMin.hpp, TRowSum.hpp, TColMax.hpp:22-35, TColMin.hpp, TColSum.hpp:22-31 */
+/* packed compare with a scalar: bit c%8 of dst[r*dst_ld + c/8]; mode 0..5 = EQ NE LT LE GT GE; EQ / NE within 1e-9 */
+void po_tcmps_packed(uint8_t *dst, int dst_ld, const float *a, int ld, int rows, int cols, float scalar, int mode); /* cpu/TCmps.hpp:24-90 */
+/* dst = bit ? a : b, bits consumed in running order over [rows, cols], bytes along mask_valid_cols then the next mask row */
+void po_tsel_packed(float *dst, const uint8_t *mask, int mask_ld, int mask_valid_cols, const float *a, const float *b,
+                    int ld, int rows, int cols); /* cpu/TSel.hpp:22-49 */
+/* dst[rows, cols] = a inside [vr, vc], pad elsewhere; pad_kind 1 zero, 2 +inf, 3 -inf */
+void po_tfillpad(float *dst, const float *a, int ld, int rows, int cols, int vr, int vc, int pad_kind); /* cpu/TFillPad.hpp:22-49 */
+/* same-shape move with optional clamp at zero */
+void po_tmov_relu(float *dst, const float *src, size_t n, int relu); /* cpu/TMov.hpp:53-69 */
+
 #ifdef __cplusplus
 }
 #endif

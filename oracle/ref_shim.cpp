@@ -232,6 +232,114 @@ void fa_auto(float *out, const float *q, const float *k, const float *v)
     TSTORE(go, *oa);
 }
 
+
+// ---- further Vec instructions on [64,128] fp32 tiles (op codes: PTO_VOP_* of include/pto_amd.h) ----
+using VX = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+using VRow = Tile<TileType::Vec, float, 64, 1, BLayout::ColMajor>;   // one value per row
+using VCol = Tile<TileType::Vec, float, 1, 128, BLayout::RowMajor>;  // one value per column
+
+void vec_op_64x128(float *out, const float *a, const float *b, const float *vec, float k, int op)
+{
+    auto ta = std::make_unique<VX>(), tb = std::make_unique<VX>(), to = std::make_unique<VX>();
+    auto rv = std::make_unique<VRow>();
+    auto cv = std::make_unique<VCol>();
+    GmND<float, 64, 128> ga(const_cast<float *>(a)), go(out);
+    TLOAD(*ta, ga);
+    if (b) {
+        GmND<float, 64, 128> gb(const_cast<float *>(b));
+        TLOAD(*tb, gb);
+    }
+    if (op >= 60 && op < 80) {
+        GmDN<float, 64, 1> gr(const_cast<float *>(vec));
+        TLOAD(*rv, gr);
+    }
+    if (op >= 80) {
+        GmND<float, 1, 128> gc(const_cast<float *>(vec));
+        TLOAD(*cv, gc);
+    }
+    switch (op) {
+    case 0: TABS(*to, *ta); break;
+    case 1: TNEG(*to, *ta); break;
+    case 2: TRELU(*to, *ta); break;
+    case 3: TSQRT(*to, *ta); break;
+    case 4: TRSQRT(*to, *ta); break;
+    case 5: TLOG(*to, *ta); break;
+    case 6: TRECIP(*to, *ta); break;
+    case 7: TEXP(*to, *ta); break;
+    case 20: TADD(*to, *ta, *tb); break;
+    case 21: TSUB(*to, *ta, *tb); break;
+    case 22: TMUL(*to, *ta, *tb); break;
+    case 23: TDIV(*to, *ta, *tb); break;
+    case 24: TMAX(*to, *ta, *tb); break;
+    case 25: TMIN(*to, *ta, *tb); break;
+    case 26: TPRELU_IMPL(*to, *ta, *tb); break; // the front end of TPRELU takes a scratch tile and returns nothing
+    case 27: TCMP(*to, *ta, *tb, CmpMode::EQ); break;
+    case 28: TCMP(*to, *ta, *tb, CmpMode::NE); break;
+    case 29: TCMP(*to, *ta, *tb, CmpMode::LT); break;
+    case 30: TCMP(*to, *ta, *tb, CmpMode::LE); break;
+    case 31: TCMP(*to, *ta, *tb, CmpMode::GT); break;
+    case 32: TCMP(*to, *ta, *tb, CmpMode::GE); break;
+    case 33: TSELS(*to, *ta, *tb, k); break;
+    case 40: TADDS(*to, *ta, k); break;
+    case 41: TSUBS(*to, *ta, k); break;
+    case 42: TMULS(*to, *ta, k); break;
+    case 43: TDIVS(*to, *ta, k); break;
+    case 44: TMAXS(*to, *ta, k); break;
+    case 45: TMINS(*to, *ta, k); break;
+    case 46: TLRELU(*to, *ta, k); break;
+    case 60: TROWEXPAND(*to, *rv); break;
+    case 61: TROWEXPANDSUB(*to, *ta, *rv); break;
+    case 62: TROWEXPANDMUL(*to, *ta, *rv); break;
+    case 63: TROWEXPANDDIV(*to, *ta, *rv); break;
+    case 64: TROWEXPANDADD(*to, *ta, *rv); break;
+    case 65: TROWEXPANDMAX(*to, *ta, *rv); break;
+    case 66: TROWEXPANDMIN(*to, *ta, *rv); break;
+    case 67: TROWEXPANDEXPDIF(*to, *ta, *rv); break;
+    case 80: TCOLEXPAND(*to, *cv); break;
+    case 81: TCOLEXPANDSUB(*to, *ta, *cv); break;
+    case 82: TCOLEXPANDMUL(*to, *ta, *cv); break;
+    case 83: TCOLEXPANDDIV(*to, *ta, *cv); break;
+    case 84: TCOLEXPANDADD(*to, *ta, *cv); break;
+    case 85: TCOLEXPANDMAX(*to, *ta, *cv); break;
+    case 86: TCOLEXPANDMIN(*to, *ta, *cv); break;
+    default: return;
+    }
+    TSTORE(go, *to);
+}
+
+// reductions of the valid region [vr, vc]; out holds vr (row ops) or vc (column ops) values
+void reduce_64x128(float *out, const float *a, int vr, int vc, int op)
+{
+    using VD = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, -1, -1>;
+    using RD = Tile<TileType::Vec, float, 64, 1, BLayout::ColMajor, -1, 1>;
+    using CD = Tile<TileType::Vec, float, 1, 128, BLayout::RowMajor, 1, -1>;
+    auto ta = std::make_unique<VD>(vr, vc), tmp = std::make_unique<VD>(vr, vc);
+    for (int r = 0; r < vr; ++r)
+        for (int c = 0; c < vc; ++c)
+            ta->data()[r * 128 + c] = a[r * 128 + c];
+    if (op < 3) {
+        auto r = std::make_unique<RD>(vr);
+        if (op == 0)
+            TROWMAX(*r, *ta, *tmp);
+        else if (op == 1)
+            TROWMIN(*r, *ta, *tmp);
+        else
+            TROWSUM(*r, *ta, *tmp);
+        for (int i = 0; i < vr; ++i)
+            out[i] = r->data()[i];
+    } else {
+        auto c = std::make_unique<CD>(vc);
+        if (op == 3)
+            TCOLMAX(*c, *ta);
+        else if (op == 4)
+            TCOLMIN(*c, *ta);
+        else
+            TCOLSUM(*c, *ta);
+        for (int j = 0; j < vc; ++j)
+            out[j] = c->data()[j];
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -339,5 +447,70 @@ void ref_image_5d_f32_2x3x4x8(float *image, const float *gm)
 
 void ref_fa_auto_64x32(float *out, const float *q, const float *k, const float *v) { fa_auto<64, 32>(out, q, k, v); }
 void ref_fa_auto_128x64(float *out, const float *q, const float *k, const float *v) { fa_auto<128, 64>(out, q, k, v); }
+
+
+void ref_vec_op_f32_64x128(float *out, const float *a, const float *b, const float *vec, float k, int op)
+{
+    vec_op_64x128(out, a, b, vec, k, op);
+}
+void ref_reduce_f32_64x128(float *out, const float *a, int vr, int vc, int op) { reduce_64x128(out, a, vr, vc, op); }
+// TCMPS into a [64,128] uint8 tile whose first 16 valid columns take the packed bits, then TSEL with that mask
+void ref_cmps_sel_f32_64x128(float *sel, uint8_t *bits, const float *a, const float *b, float scalar, int mode)
+{
+    using MB = Tile<TileType::Vec, uint8_t, 64, 128, BLayout::RowMajor, 64, 16>;
+    using MS = Tile<TileType::Vec, uint8_t, 64, 32, BLayout::RowMajor, 64, 16>;
+    auto ta = std::make_unique<VX>(), tb = std::make_unique<VX>(), to = std::make_unique<VX>();
+    auto m = std::make_unique<MB>();
+    auto ms = std::make_unique<MS>();
+    GmND<float, 64, 128> ga(const_cast<float *>(a)), gb(const_cast<float *>(b)), go(sel);
+    TLOAD(*ta, ga);
+    TLOAD(*tb, gb);
+    TCMPS(*m, *ta, scalar, static_cast<CmpMode>(mode));
+    for (int r = 0; r < 64; ++r)
+        for (int c = 0; c < 16; ++c) {
+            bits[r * 16 + c] = m->data()[r * 128 + c];
+            ms->data()[r * 32 + c] = m->data()[r * 128 + c];
+        }
+    TSEL(*to, *ms, *ta, *tb);
+    TSTORE(go, *to);
+}
+void ref_fillpad_f32_64x128(float *out, const float *a, int vr, int vc, int pad_kind)
+{
+    using VS = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, -1, -1>;
+    auto ts = std::make_unique<VS>(vr, vc);
+    for (int r = 0; r < vr; ++r)
+        for (int c = 0; c < vc; ++c)
+            ts->data()[r * 128 + c] = a[r * 128 + c];
+    GmND<float, 64, 128> go(out);
+    if (pad_kind == 1) {
+        auto td = std::make_unique<Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, 64, 128, SLayout::NoneBox, 512, PadValue::Zero>>();
+        TFILLPAD(*td, *ts);
+        TSTORE(go, *td);
+    } else if (pad_kind == 2) {
+        auto td = std::make_unique<Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, 64, 128, SLayout::NoneBox, 512, PadValue::Max>>();
+        TFILLPAD(*td, *ts);
+        TSTORE(go, *td);
+    } else {
+        auto td = std::make_unique<Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, 64, 128, SLayout::NoneBox, 512, PadValue::Min>>();
+        TFILLPAD(*td, *ts);
+        TSTORE(go, *td);
+    }
+}
+// accumulator tile -> Vec tile with ReluPreMode
+void ref_tmov_acc_vec_f32_64x128(float *out, const float *acc_rowmajor, int relu)
+{
+    using Acc = TileAcc<float, 64, 128, 64, 128>;
+    auto c = std::make_unique<Acc>();
+    auto v = std::make_unique<VX>();
+    for (int r = 0; r < 64; ++r)
+        for (int col = 0; col < 128; ++col)
+            c->data()[GetTileElementOffset<Acc>(r, col)] = acc_rowmajor[r * 128 + col];
+    if (relu)
+        TMOV<VX, Acc, ReluPreMode::NormalRelu>(*v, *c);
+    else
+        TMOV(*v, *c);
+    GmND<float, 64, 128> go(out);
+    TSTORE(go, *v);
+}
 
 } // extern "C"

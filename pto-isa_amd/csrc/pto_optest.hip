@@ -273,6 +273,186 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulBias(__gm__ float 
     TSTORE(gc, c, computed);
 }
 
+
+// ---- one Vec instruction on [64, 128] fp32 tiles; `vec` is a per-row ([64]) or per-column ([128]) operand ----
+enum VecOp : int {
+    kAbs = 0, kNeg, kRelu, kSqrt, kRsqrt, kLog, kRecip, kExp,
+    kAdd = 20, kSub, kMul, kDiv, kMax, kMin, kPrelu, kCmpEq, kCmpNe, kCmpLt, kCmpLe, kCmpGt, kCmpGe, kSels,
+    kAdds = 40, kSubs, kMuls, kDivs, kMaxs, kMins, kLrelu,
+    kRowExpand = 60, kRowSub, kRowMul, kRowDiv, kRowAdd, kRowMax, kRowMin, kRowExpDif,
+    kColExpand = 80, kColSub, kColMul, kColDiv, kColAdd, kColMax, kColMin,
+};
+__global__ __launch_bounds__(kBlockThreads) AICORE void VecOpKernel(__gm__ float *out, __gm__ const float *aIn, __gm__ const float *bIn,
+                                                                    __gm__ const float *vecIn, float k, int op)
+{
+    using TileX = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    using TileR = Tile<TileType::Vec, float, 64, 1, BLayout::ColMajor>;
+    using TileC = Tile<TileType::Vec, float, 1, 128, BLayout::RowMajor>;
+    TileX a, b, o;
+    TileR rv;
+    TileC cv;
+    GmND<float, 64, 128> ga(const_cast<float *>(aIn)), gb(const_cast<float *>(bIn)), go(out);
+    TLOAD(a, ga);
+    if (op >= kAdd && op < kAdds)
+        TLOAD(b, gb);
+    if (op >= kRowExpand && op < kColExpand) {
+        GmCol<float, 64> gr(const_cast<float *>(vecIn));
+        TLOAD(rv, gr);
+    }
+    if (op >= kColExpand) {
+        GmND<float, 1, 128> gc(const_cast<float *>(vecIn));
+        TLOAD(cv, gc);
+    }
+    switch (op) {
+    case kAbs: TABS(o, a); break;
+    case kNeg: TNEG(o, a); break;
+    case kRelu: TRELU(o, a); break;
+    case kSqrt: TSQRT(o, a); break;
+    case kRsqrt: TRSQRT(o, a); break;
+    case kLog: TLOG(o, a); break;
+    case kRecip: TRECIP(o, a); break;
+    case kExp: TEXP(o, a); break;
+    case kAdd: TADD(o, a, b); break;
+    case kSub: TSUB(o, a, b); break;
+    case kMul: TMUL(o, a, b); break;
+    case kDiv: TDIV(o, a, b); break;
+    case kMax: TMAX(o, a, b); break;
+    case kMin: TMIN(o, a, b); break;
+    case kPrelu: TPRELU(o, a, b); break;
+    case kCmpEq: TCMP(o, a, b, CmpMode::EQ); break;
+    case kCmpNe: TCMP(o, a, b, CmpMode::NE); break;
+    case kCmpLt: TCMP(o, a, b, CmpMode::LT); break;
+    case kCmpLe: TCMP(o, a, b, CmpMode::LE); break;
+    case kCmpGt: TCMP(o, a, b, CmpMode::GT); break;
+    case kCmpGe: TCMP(o, a, b, CmpMode::GE); break;
+    case kSels: TSELS(o, a, b, (uint8_t)k); break;
+    case kAdds: TADDS(o, a, k); break;
+    case kSubs: TSUBS(o, a, k); break;
+    case kMuls: TMULS(o, a, k); break;
+    case kDivs: TDIVS(o, a, k); break;
+    case kMaxs: TMAXS(o, a, k); break;
+    case kMins: TMINS(o, a, k); break;
+    case kLrelu: TLRELU(o, a, k); break;
+    case kRowExpand: TROWEXPAND(o, rv); break;
+    case kRowSub: TROWEXPANDSUB(o, a, rv); break;
+    case kRowMul: TROWEXPANDMUL(o, a, rv); break;
+    case kRowDiv: TROWEXPANDDIV(o, a, rv); break;
+    case kRowAdd: TROWEXPANDADD(o, a, rv); break;
+    case kRowMax: TROWEXPANDMAX(o, a, rv); break;
+    case kRowMin: TROWEXPANDMIN(o, a, rv); break;
+    case kRowExpDif: TROWEXPANDEXPDIF(o, a, rv); break;
+    case kColExpand: TCOLEXPAND(o, cv); break;
+    case kColSub: TCOLEXPANDSUB(o, a, cv); break;
+    case kColMul: TCOLEXPANDMUL(o, a, cv); break;
+    case kColDiv: TCOLEXPANDDIV(o, a, cv); break;
+    case kColAdd: TCOLEXPANDADD(o, a, cv); break;
+    case kColMax: TCOLEXPANDMAX(o, a, cv); break;
+    case kColMin: TCOLEXPANDMIN(o, a, cv); break;
+    default: TMULS(o, a, 0.0f); break;
+    }
+    TSTORE(go, o);
+}
+
+// ---- row / column reductions of the valid region [vr, vc] of a [64, 128] fp32 tile ----
+// op 0..2: TROWMAX / TROWMIN / TROWSUM -> out[64]; 3..5: TCOLMAX / TCOLMIN / TCOLSUM -> out[128].
+// Entries outside the valid region are left as the caller set them.
+__global__ __launch_bounds__(kBlockThreads) AICORE void ReduceKernel(__gm__ float *out, __gm__ const float *aIn, int vr, int vc, int op)
+{
+    using TileX = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    using TileR = Tile<TileType::Vec, float, 64, 1, BLayout::ColMajor, DYNAMIC, 1>;
+    using TileC = Tile<TileType::Vec, float, 1, 128, BLayout::RowMajor, 1, DYNAMIC>;
+    TileX a(vr, vc), tmp(vr, vc);
+    GlobalTensor<float, Shape<1, 1, 1, DYNAMIC, DYNAMIC>, Stride<1, 1, 1, 128, 1>> ga(const_cast<float *>(aIn), Shape<1, 1, 1, DYNAMIC, DYNAMIC>(vr, vc));
+    TLOAD(a, ga);
+    if (op < 3) {
+        TileR r(vr);
+        if (op == 0)
+            TROWMAX(r, a, tmp);
+        else if (op == 1)
+            TROWMIN(r, a, tmp);
+        else
+            TROWSUM(r, a, tmp);
+        GlobalTensor<float, Shape<1, 1, 1, DYNAMIC, 1>, Stride<1, 1, 1, 1, 64>, Layout::DN> gr(out, Shape<1, 1, 1, DYNAMIC, 1>(vr));
+        TSTORE(gr, r);
+    } else {
+        TileC c(vc);
+        if (op == 3)
+            TCOLMAX(c, a);
+        else if (op == 4)
+            TCOLMIN(c, a);
+        else
+            TCOLSUM(c, a);
+        GlobalTensor<float, Shape<1, 1, 1, 1, DYNAMIC>, Stride<1, 1, 1, 128, 1>> gc(out, Shape<1, 1, 1, 1, DYNAMIC>(vc));
+        TSTORE(gc, c);
+    }
+}
+
+// ---- TCMPS into a packed bit mask, then TSEL with that mask: bits[64][16] and sel = bit ? a : b ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void CmpsSelKernel(__gm__ float *sel, __gm__ uint8_t *bits, __gm__ const float *aIn,
+                                                                      __gm__ const float *bIn, float scalar, int mode)
+{
+    using TileX = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    using TileM = Tile<TileType::Vec, uint8_t, 64, 32, BLayout::RowMajor, 64, 16>;
+    TileX a, b, o;
+    TileM m;
+    GmND<float, 64, 128> ga(const_cast<float *>(aIn)), gb(const_cast<float *>(bIn)), go(sel);
+    GlobalTensor<uint8_t, Shape<1, 1, 1, 64, 16>, Stride<1024, 1024, 1024, 16, 1>> gm(bits);
+    TLOAD(a, ga);
+    TLOAD(b, gb);
+    TCMPS(m, a, scalar, static_cast<CmpMode>(mode));
+    TSEL(o, m, a, b);
+    TSTORE(gm, m);
+    TSTORE(go, o);
+}
+
+// ---- TFILLPAD: [64, 128] tile whose valid region [vr, vc] comes from GM, the rest is the pad value ----
+template <PadValue PAD>
+__global__ __launch_bounds__(kBlockThreads) AICORE void FillPadKernel(__gm__ float *out, __gm__ const float *aIn, int vr, int vc)
+{
+    using TileS = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    using TileD = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, 64, 128, SLayout::NoneBox, 512, PAD>;
+    TileS a(vr, vc);
+    TileD d;
+    GlobalTensor<float, Shape<1, 1, 1, DYNAMIC, DYNAMIC>, Stride<1, 1, 1, 128, 1>> ga(const_cast<float *>(aIn), Shape<1, 1, 1, DYNAMIC, DYNAMIC>(vr, vc));
+    GmND<float, 64, 128> go(out);
+    TLOAD(a, ga);
+    TFILLPAD(d, a);
+    TSTORE(go, d);
+}
+
+// ---- [64, 64] x [64, 128] fp16 matmul, accumulator moved to a Vec tile (optionally clamped at zero), scaled, stored ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMovKernel(__gm__ float *out, __gm__ const half *a, __gm__ const half *bT,
+                                                                        int relu, float scale)
+{
+    using MatA = Tile<TileType::Mat, half, 64, 64, BLayout::ColMajor, 64, 64, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, half, 64, 128, BLayout::RowMajor, 64, 128, SLayout::ColMajor>;
+    using TileV = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    MatA am;
+    MatB bm;
+    TASSIGN(am, 0u);
+    TASSIGN(bm, 64u * 64u * sizeof(half));
+    TileLeft<half, 64, 64> l;
+    TileRight<half, 64, 128> r;
+    TileAcc<float, 64, 128> c;
+    TileV v;
+    GmND<half, 64, 64> ga(const_cast<half *>(a));
+    GlobalTensor<half, Shape<1, 1, 1, 64, 128>, Stride<1, 1, 1, 1, 64>, Layout::DN> gb(const_cast<half *>(bT));
+    GmND<float, 64, 128> go(out);
+    TLOAD(am, ga);
+    TLOAD(bm, gb);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    TMOV(l, am);
+    TMOV(r, bm);
+    TMATMUL(c, l, r);
+    if (relu)
+        TMOV<TileV, TileAcc<float, 64, 128>, ReluPreMode::NormalRelu>(v, c);
+    else
+        TMOV(v, c);
+    TMULS(v, v, scale);
+    TSTORE(go, v);
+}
+
 } // namespace
 
 PTO_DEVICE_CODE_END
@@ -372,5 +552,61 @@ extern "C" int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uin
     else
         MatmulBias<half, 64><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const half *>(a),
                                                                          reinterpret_cast<const half *>(b_t), bias);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const float *b, const float *vec, float scalar, int op)
+{
+    PTO_ST_NONNULL(out, a);
+    const bool known = (op >= kAbs && op <= kExp) || (op >= kAdd && op <= kSels) || (op >= kAdds && op <= kLrelu) ||
+                       (op >= kRowExpand && op <= kRowExpDif) || (op >= kColExpand && op <= kColMin);
+    if (!known)
+        return PTO_ERR_BAD_ARG;
+    if (op >= kAdd && op <= kSels)
+        PTO_ST_NONNULL(b);
+    if (op >= kRowExpand)
+        PTO_ST_NONNULL(vec);
+    VecOpKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, a, b, vec, scalar, op);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_reduce_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int op)
+{
+    PTO_ST_NONNULL(out, a);
+    if (valid_rows < 1 || valid_rows > 64 || valid_cols < 1 || valid_cols > 128 || op < 0 || op > 5)
+        return PTO_ERR_BAD_ARG;
+    ReduceKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, a, valid_rows, valid_cols, op);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_cmps_sel_f32_64x128(void *stream, float *sel, uint8_t *bits, const float *a, const float *b, float scalar, int cmp_mode)
+{
+    PTO_ST_NONNULL(sel, bits, a, b);
+    if (cmp_mode < 0 || cmp_mode > 5)
+        return PTO_ERR_BAD_ARG;
+    CmpsSelKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(sel, bits, a, b, scalar, cmp_mode);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int pad_kind)
+{
+    PTO_ST_NONNULL(out, a);
+    if (valid_rows < 1 || valid_rows > 64 || valid_cols < 1 || valid_cols > 128 || pad_kind < 1 || pad_kind > 3)
+        return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (pad_kind == 1)
+        FillPadKernel<PadValue::Zero><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, a, valid_rows, valid_cols);
+    else if (pad_kind == 2)
+        FillPadKernel<PadValue::Max><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, a, valid_rows, valid_cols);
+    else
+        FillPadKernel<PadValue::Min><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, a, valid_rows, valid_cols);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, int relu, float scale)
+{
+    PTO_ST_NONNULL(out, a, b_t);
+    MatmulMovKernel<<<dim3(1), dim3(kBlockThreads), (64 * 64 + 64 * 128) * sizeof(half), static_cast<hipStream_t>(stream)>>>(
+        out, reinterpret_cast<const half *>(a), reinterpret_cast<const half *>(b_t), relu, scale);
     return pto_amd::check_launch();
 }

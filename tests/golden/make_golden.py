@@ -57,6 +57,19 @@ def cases(ref):
     return out
 
 
+def vec_ext_cases(ref):
+    """Outputs of the compiled reference for the further Vec instructions -> ref_vec_ext.npz."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from vec_ext_cases import ALL_OPS, vec_inputs
+    out = {}
+    for op in ALL_OPS:
+        a, b, vec, k = vec_inputs(op)
+        o = np.zeros((64, 128), dtype=np.float32)
+        ref.ref_vec_op_f32_64x128(p(o), p(a), p(b), None if vec is None else p(vec), C.c_float(float(k)), oracle.VOP[op])
+        out["vec_" + op] = o[::4].copy()  # every fourth row keeps the fixture small
+    return out
+
+
 if __name__ == "__main__":
     oracle.build(ref=True)
     r = oracle.ref()
@@ -64,3 +77,5 @@ if __name__ == "__main__":
         sys.exit("reference tree not present: cannot regenerate the fixture")
     np.savez_compressed(os.path.join(HERE, "ref_vectors.npz"), **cases(r))
     print("wrote", os.path.join(HERE, "ref_vectors.npz"))
+    np.savez_compressed(os.path.join(HERE, "ref_vec_ext.npz"), **vec_ext_cases(r))
+    print("wrote", os.path.join(HERE, "ref_vec_ext.npz"))

@@ -1,0 +1,121 @@
+"""GPU parity of the further Vec instructions (unary math, ReLU family, compare / select, row and column
+broadcasts and reductions, TFILLPAD, TMOV accumulator -> Vec) through the C ABI, against the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from pto_amd import capi
+from vec_ext_cases import ALL_OPS, REDUCE_SHAPES, reduce_inputs, vec_inputs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+# device results that may differ from the host's in the last place: library log / exp in double then cast
+ULP_OPS = {"LOG": 1, "EXP": 1, "ROWEXPANDEXPDIF": 1}
+
+
+def dev(a):
+    a = np.ascontiguousarray(a)
+    if a.dtype in (np.uint16, np.float16):
+        return torch.from_numpy(a.view(np.int16)).to(DEV)
+    return torch.from_numpy(a).to(DEV)
+
+
+def st():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def ulp_diff(a, b):
+    ia, ib = a.view(np.int32).astype(np.int64), b.view(np.int32).astype(np.int64)
+    return np.abs(ia - ib)
+
+
+@pytest.mark.parametrize("op", ALL_OPS)
+def test_vec_op(oracle, op):
+    lib = capi.load()
+    a, b, vec, k = vec_inputs(op)
+    ta, tb = dev(a), dev(b)
+    tv = dev(vec) if vec is not None else None
+    out = torch.full((64, 128), float("nan"), device=DEV)
+    capi.check(lib.pto_st_vec_op_f32_64x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tv.data_ptr() if tv is not None else 0,
+                                            float(k), oracle.VOP[op]), op)
+    torch.cuda.synchronize()
+    got, want = out.cpu().numpy(), oracle.vec_op(op, a, b, vec, k)
+    if op in ULP_OPS:
+        assert ulp_diff(got, want).max() <= ULP_OPS[op], op
+        assert (ulp_diff(got, want) > 0).mean() < 0.01, op       # and almost all results are identical
+    else:
+        assert np.array_equal(got, want, equal_nan=True), op      # bit-exact
+
+
+def test_vec_op_bad_code():
+    lib = capi.load()
+    out = torch.zeros((64, 128), device=DEV)
+    assert lib.pto_st_vec_op_f32_64x128(st(), out.data_ptr(), out.data_ptr(), out.data_ptr(), 0, 0.0, 999) == capi.ERR_BAD_ARG
+
+
+@pytest.mark.parametrize("op", range(6))
+@pytest.mark.parametrize("shape", REDUCE_SHAPES)
+def test_reduce(oracle, op, shape):
+    lib = capi.load()
+    vr, vc = shape
+    full = reduce_inputs()
+    ta = dev(full)
+    out = torch.full((128,), -777.0, device=DEV)
+    capi.check(lib.pto_st_reduce_f32_64x128(st(), out.data_ptr(), ta.data_ptr(), vr, vc, op), "reduce")
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    n = vr if op < 3 else vc
+    want = oracle.reduce(op, full[:vr, :vc])
+    if op % 3 == 2:       # sums add in another order than the sequential oracle: fp32 rounding only
+        mag = np.abs(full[:vr, :vc]).sum(axis=1 if op < 3 else 0)
+        assert np.all(np.abs(got[:n] - want) <= 2.0 ** -20 * mag)
+    else:
+        assert np.array_equal(got[:n], want)
+    assert np.all(got[n:] == -777.0)                               # nothing outside the valid region is written
+
+
+@pytest.mark.parametrize("mode", range(6))
+def test_cmps_sel(oracle, mode):
+    lib = capi.load()
+    a, b, _, _ = vec_inputs("CMP_EQ", seed=mode)
+    scalar = np.float32(a[3, 5])
+    a[::7, ::3] = scalar
+    a[1, 1] = scalar + np.float32(1e-6)
+    ta, tb = dev(a), dev(b)
+    sel = torch.zeros((64, 128), device=DEV)
+    bits = torch.zeros((64, 16), dtype=torch.uint8, device=DEV)
+    capi.check(lib.pto_st_cmps_sel_f32_64x128(st(), sel.data_ptr(), bits.data_ptr(), ta.data_ptr(), tb.data_ptr(), float(scalar), mode), "cmps")
+    torch.cuda.synchronize()
+    obits = oracle.tcmps_packed(a, scalar, mode)
+    assert np.array_equal(bits.cpu().numpy(), obits)
+    mask = np.zeros((64, 32), dtype=np.uint8)
+    mask[:, :16] = obits
+    assert np.array_equal(sel.cpu().numpy(), oracle.tsel_packed(mask, 16, a, b))
+
+
+@pytest.mark.parametrize("pad_kind", [1, 2, 3])
+@pytest.mark.parametrize("shape", [(64, 128), (10, 20), (64, 5), (1, 1)])
+def test_fillpad(oracle, pad_kind, shape):
+    lib = capi.load()
+    vr, vc = shape
+    a = reduce_inputs(3)
+    ta = dev(a)
+    out = torch.full((64, 128), 5.0, device=DEV)
+    capi.check(lib.pto_st_fillpad_f32_64x128(st(), out.data_ptr(), ta.data_ptr(), vr, vc, pad_kind), "fillpad")
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(), oracle.tfillpad(a, vr, vc, pad_kind))
+
+
+@pytest.mark.parametrize("relu", [0, 1])
+def test_matmul_tmov_acc_to_vec(oracle, relu):
+    lib = capi.load()
+    rng = np.random.default_rng(21)
+    a = rng.integers(-4, 5, size=(64, 64)).astype(np.float32)     # integer values: the fp32 products and sums are exact
+    b = rng.integers(-4, 5, size=(64, 128)).astype(np.float32)
+    ta, tb = dev(a.astype(np.float16)), dev(np.ascontiguousarray(b.T).astype(np.float16))
+    out = torch.zeros((64, 128), device=DEV)
+    capi.check(lib.pto_st_matmul_tmov_f16_64x64x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), relu, 0.5), "tmov")
+    torch.cuda.synchronize()
+    want = oracle.tmov_relu((a @ b).astype(np.float32), relu) * np.float32(0.5)
+    assert np.array_equal(out.cpu().numpy(), want)
