@@ -7,6 +7,7 @@
 #include "pto/gfx950/mem_ops.hpp"
 #include "pto/gfx950/vec_ops.hpp"
 #include "pto/gfx950/vec_ops_ext.hpp"
+#include "pto/gfx950/fifo_ops.hpp"
 
 namespace pto {
 
@@ -110,6 +111,8 @@ PTO_FRONT(TCMPS, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &s
 PTO_FRONT(TSEL, typename T PTO_C typename M, T &dst PTO_C M &selMask PTO_C T &src0 PTO_C T &src1, (dst, selMask, src0, src1))
 PTO_FRONT(TSELS, typename T, T &dst PTO_C T &src0 PTO_C T &src1 PTO_C uint8_t selectMode, (dst, src0, src1, selectMode))
 PTO_FRONT(TFILLPAD, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TPUSH, typename P PTO_C typename T PTO_C typename F, P &prod PTO_C T &tile PTO_C F &fifo, (prod, tile, fifo))
+PTO_FRONT(TPOP, typename P PTO_C typename T PTO_C typename F, P &cons PTO_C T &tile PTO_C F &fifo, (cons, tile, fifo))
 #undef PTO_FRONT
 #undef PTO_C
 

@@ -144,6 +144,15 @@ int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int vali
  * the accumulator into a Vec tile with ReluPreMode (cpu/TMov.hpp:53-69), TMULS, TSTORE. */
 int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, int relu, float scale);
 
+/* Two-stage pipeline through TPUSH / TPOP FIFOs (common/fifo.hpp, cpu/TPush.hpp, cpu/TPop.hpp; the hand-offs of
+ * fa_performance_kernel.cpp:346-583): out[64,64] = sum_t fp16(0.25 (a b[t])) v[t], t in {0,1}.  a [64,64] fp16;
+ * b_t [2][128][64] (each b[t] column-major 64 x 128); v_t [2][64][128] (each v[t] column-major 128 x 64).
+ * The score tile goes accumulator -> FIFO -> Vec tile through qk_fifo (2 x 64 x 128 fp32 of global memory) or, with
+ * lds_fifo != 0, through an LDS FIFO (qk_fifo unused); the probability tile goes Vec -> FIFO -> Mat tile through
+ * p_fifo (2 x 64 x 128 fp16 of global memory). */
+int pto_st_pushpop_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, const uint16_t *v_t,
+                                 float *qk_fifo, uint16_t *p_fifo, int lds_fifo);
+
 #ifdef __cplusplus
 }
 #endif

@@ -453,6 +453,84 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMovKernel(__gm__ f
     TSTORE(go, v);
 }
 
+
+// ---- two-stage pipeline through FIFOs, the shape of the attention kernel's Cube -> Vec -> Cube hand-offs
+// (fa_performance_kernel.cpp:346-583): for t in {0, 1}
+//   S = a x b[t]                       [64,64] x [64,128] fp16 -> fp32 accumulator
+//   TPUSH(S)  ->  TPOP as a Vec tile   (global-memory FIFO, or an LDS FIFO when LDS_FIFO)
+//   P = fp16(0.25 S)                   TMULS, TCVT
+//   TPUSH(P)  ->  TPOP as a Mat tile   (global-memory FIFO)
+//   O (+)= P x v[t]                    [64,128] x [128,64]
+template <bool LDS_FIFO>
+__global__ __launch_bounds__(kBlockThreads) AICORE void PushPopKernel(__gm__ float *out, __gm__ const half *a, __gm__ const half *bT,
+                                                                      __gm__ const half *vT, __gm__ float *qkFifoMem, __gm__ half *pFifoMem)
+{
+    using MatA = Tile<TileType::Mat, half, 64, 64, BLayout::ColMajor, 64, 64, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, half, 64, 128, BLayout::RowMajor, 64, 128, SLayout::ColMajor>;
+    using MatP = Tile<TileType::Mat, half, 64, 128, BLayout::ColMajor, 64, 128, SLayout::RowMajor>;
+    using MatV = Tile<TileType::Mat, half, 128, 64, BLayout::RowMajor, 128, 64, SLayout::ColMajor>;
+    using VecS = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    using VecP = Tile<TileType::Vec, half, 64, 128, BLayout::RowMajor>;
+    using AccS = TileAcc<float, 64, 128>;
+    using AccO = TileAcc<float, 64, 64>;
+    constexpr uint32_t kA = 0, kB = 8192, kP = kB + 16384, kV = kP + 16384, kFifo = kV + 16384;
+    MatA am;
+    MatB bm;
+    MatP pm;
+    MatV vm;
+    TASSIGN(am, kA);
+    TASSIGN(bm, kB);
+    TASSIGN(pm, kP);
+    TASSIGN(vm, kV);
+    using QkFifo = DataFIFO<float, LDS_FIFO ? FIFOType::VEC_FIFO : FIFOType::GM_FIFO, 2, 1>;
+    using PFifo = DataFIFO<half, FIFOType::GM_FIFO, 2, 1>;
+    using QkSync = TFIFOSync<0, QkFifo, TSyncOpType::TSTORE_C2GM, TSyncOpType::TLOAD>;
+    using PSync = TFIFOSync<2, PFifo, TSyncOpType::TSTORE_V2GM, TSyncOpType::TLOAD>;
+    QkFifo qkFifo = LDS_FIFO ? QkFifo(kFifo, 0) : QkFifo(qkFifoMem);
+    PFifo pFifo(pFifoMem);
+    typename QkSync::Producer qkProd;
+    typename QkSync::Consumer qkCons;
+    typename PSync::Producer pProd;
+    typename PSync::Consumer pCons;
+
+    TileLeft<half, 64, 64> aLeft;
+    TileRight<half, 64, 128> bRight;
+    TileLeft<half, 64, 128> pLeft;
+    TileRight<half, 128, 64> vRight;
+    AccS sAcc;
+    AccO oAcc;
+    VecS sVec;
+    VecP pVec;
+    GmND<half, 64, 64> ga(const_cast<half *>(a));
+    TLOAD(am, ga);
+    for (int t = 0; t < 2; ++t) {
+        GlobalTensor<half, Shape<1, 1, 1, 64, 128>, Stride<1, 1, 1, 1, 64>, Layout::DN> gb(const_cast<half *>(bT) + t * 128 * 64);
+        GlobalTensor<half, Shape<1, 1, 1, 128, 64>, Stride<1, 1, 1, 1, 128>, Layout::DN> gv(const_cast<half *>(vT) + t * 64 * 128);
+        pipe_barrier(PIPE_ALL); // everyone has left the Mat tiles of the previous step
+        TLOAD(bm, gb);
+        TLOAD(vm, gv);
+        set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+        wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+        TMOV(aLeft, am);
+        TMOV(bRight, bm);
+        TMATMUL(sAcc, aLeft, bRight);
+        TPUSH(qkProd, sAcc, qkFifo);
+        TPOP(qkCons, sVec, qkFifo);
+        TMULS(sVec, sVec, 0.25f);
+        TCVT(pVec, sVec, RoundMode::CAST_RINT);
+        TPUSH(pProd, pVec, pFifo);
+        TPOP(pCons, pm, pFifo);
+        TMOV(pLeft, pm);
+        TMOV(vRight, vm);
+        if (t == 0)
+            TMATMUL(oAcc, pLeft, vRight);
+        else
+            TMATMUL_ACC(oAcc, oAcc, pLeft, vRight);
+    }
+    GmND<float, 64, 64> go(out);
+    TSTORE(go, oAcc);
+}
+
 } // namespace
 
 PTO_DEVICE_CODE_END
@@ -608,5 +686,26 @@ extern "C" int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const 
     PTO_ST_NONNULL(out, a, b_t);
     MatmulMovKernel<<<dim3(1), dim3(kBlockThreads), (64 * 64 + 64 * 128) * sizeof(half), static_cast<hipStream_t>(stream)>>>(
         out, reinterpret_cast<const half *>(a), reinterpret_cast<const half *>(b_t), relu, scale);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_pushpop_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, const uint16_t *v_t,
+                                            float *qk_fifo, uint16_t *p_fifo, int lds_fifo)
+{
+    PTO_ST_NONNULL(out, a, b_t, v_t, p_fifo);
+    if (!lds_fifo)
+        PTO_ST_NONNULL(qk_fifo);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    constexpr int ldsPlain = 8192 + 3 * 16384, ldsFifo = ldsPlain + 2 * 64 * 128 * 4;
+    const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b_t), *hv = reinterpret_cast<const half *>(v_t);
+    half *hp = reinterpret_cast<half *>(p_fifo);
+    if (lds_fifo) {
+        static const int attr = pto_amd::allow_lds(PushPopKernel<true>, ldsFifo);
+        if (attr != PTO_OK)
+            return attr;
+        PushPopKernel<true><<<dim3(1), dim3(kBlockThreads), ldsFifo, st>>>(out, ha, hb, hv, qk_fifo, hp);
+    } else {
+        PushPopKernel<false><<<dim3(1), dim3(kBlockThreads), ldsPlain, st>>>(out, ha, hb, hv, qk_fifo, hp);
+    }
     return pto_amd::check_launch();
 }

@@ -37,6 +37,7 @@ SYMBOLS = {
     "pto_st_cmps_sel_f32_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int]),
     "pto_st_fillpad_f32_64x128": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 3),
     "pto_st_matmul_tmov_f16_64x64x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int, C.c_float]),
+    "pto_st_pushpop_f16_64x64x128": (C.c_int, [C.c_void_p] * 7 + [C.c_int]),
 }
 
 _lib = None

@@ -221,3 +221,36 @@ def test_matmul_bias_and_bf16(oracle, bf16, with_bias):
         ref = np.zeros((128, 256), dtype=np.float32)
         o.tstore(ref, [1, 1, 1, 128, 256], [0, 0, 0, 256, 1], acc, Lc)
         assert np.array_equal(out.cpu().numpy(), ref)
+
+
+@pytest.mark.parametrize("lds_fifo", [0, 1])
+def test_tpush_tpop_pipeline(lds_fifo):
+    """Accumulator -> FIFO -> Vec tile and Vec -> FIFO -> Mat tile hand-offs; integer-valued data, so every
+    product, sum and the fp16 cast are exact and the result must equal numpy's."""
+    lib = capi.load()
+    rng = np.random.default_rng(31 + lds_fifo)
+    a = rng.integers(-2, 3, size=(64, 64)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(2, 64, 128)).astype(np.float32)
+    v = rng.integers(-2, 3, size=(2, 128, 64)).astype(np.float32)
+    ta = dev(a.astype(np.float16))
+    tb = dev(np.ascontiguousarray(b.transpose(0, 2, 1)).astype(np.float16))    # [t][n][k]
+    tv = dev(np.ascontiguousarray(v.transpose(0, 2, 1)).astype(np.float16))    # [t][n][k]
+    qk = torch.zeros(2 * 64 * 128, device=DEV)
+    pf = torch.zeros(2 * 64 * 128, dtype=torch.int16, device=DEV)
+    out = torch.zeros((64, 64), device=DEV)
+    capi.check(lib.pto_st_pushpop_f16_64x64x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tv.data_ptr(),
+                                                0 if lds_fifo else qk.data_ptr(), pf.data_ptr(), lds_fifo), "pushpop")
+    torch.cuda.synchronize()
+    want = np.zeros((64, 64), dtype=np.float32)
+    for t in range(2):
+        p = ((a @ b[t]) * np.float32(0.25)).astype(np.float16).astype(np.float32)
+        want += p @ v[t]
+    assert np.array_equal(out.cpu().numpy(), want)
+    # the FIFO slots hold what was pushed: slot t = tile t (depth 2)
+    pslots = pf.cpu().numpy().view(np.float16).reshape(2, 64, 128).astype(np.float32)
+    for t in range(2):
+        assert np.array_equal(pslots[t], ((a @ b[t]) * np.float32(0.25)))
+    if not lds_fifo:
+        qslots = qk.cpu().numpy().reshape(2, 64, 128)
+        for t in range(2):
+            assert np.array_equal(qslots[t], a @ b[t])
