@@ -40,7 +40,27 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", OUT)
+    build_host(verbose)
     return OUT
+
+
+def build_host(verbose=True):
+    """The `call_kernel` libraries of the two demos and the GEMM host program; plain host C++ on top of libpto_amd.so."""
+    inc = ["-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__"]
+    link = ["-L" + HERE, "-lpto_amd", "-Wl,-rpath,$ORIGIN"]
+    jobs = [
+        (["-shared", "-fPIC", os.path.join(CSRC, "call_kernel_gemm.cpp")], os.path.join(HERE, "libpto_call_gemm.so"), link),
+        (["-shared", "-fPIC", os.path.join(CSRC, "call_kernel_fa.cpp")], os.path.join(HERE, "libpto_call_fa.so"), link),
+        ([os.path.join(HERE, "host", "gemm_main.cpp")], os.path.join(HERE, "host", "gemm_main"),
+         ["-L" + HERE, "-lpto_amd", "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"]),
+    ]
+    for srcs, out, libs in jobs:
+        cmd = ["g++", "-O2", "-std=c++17"] + inc + srcs + ["-o", out] + libs
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host build failed for %s:\n%s" % (out, r.stderr))
+        if verbose:
+            print("built", out)
 
 
 if __name__ == "__main__":

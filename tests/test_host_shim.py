@@ -1,0 +1,104 @@
+"""The reference-shaped host boundary: `call_kernel` libraries of the two demos, the GEMM host program with the
+reference's file protocol, and its data generator."""
+import ctypes as C
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "pto-isa_amd")
+
+
+def _lib(name):
+    path = os.path.join(PKG, name)
+    if not os.path.exists(path):
+        pytest.fail("%s is not built: run python pto-isa_amd/build.py" % name)
+    return C.CDLL(path)
+
+
+def test_call_kernel_libraries_export_the_entry_point():
+    for name in ("libpto_call_gemm.so", "libpto_call_fa.so"):
+        assert hasattr(_lib(name), "call_kernel")
+    assert os.access(os.path.join(PKG, "host", "gemm_main"), os.X_OK)
+
+
+def test_gen_data_file_protocol(tmp_path):
+    subprocess.run([sys.executable, os.path.join(PKG, "host", "gen_data.py"), str(tmp_path), "128", "64", "256"], check=True)
+    a = np.fromfile(tmp_path / "input" / "x1_gm.bin", dtype=np.float16).reshape(128, 64)
+    bt = np.fromfile(tmp_path / "input" / "x2_gm.bin", dtype=np.float16).reshape(256, 64)     # stored [n, k]
+    g = np.fromfile(tmp_path / "output" / "golden.bin", dtype=np.float32).reshape(128, 256)
+    assert np.array_equal(g, a.astype(np.float32) @ bt.astype(np.float32).T)
+    assert np.abs(a).max() <= 5 and np.abs(bt).max() <= 5
+
+
+@pytest.mark.gpu
+def test_gemm_main_runs_the_file_protocol(tmp_path):
+    subprocess.run([sys.executable, os.path.join(PKG, "host", "gen_data.py"), str(tmp_path), "512", "768", "512"], check=True)
+    r = subprocess.run([os.path.join(PKG, "host", "gemm_main"), str(tmp_path), "512", "768", "512"], capture_output=True, text=True, timeout=120)
+    assert "test success" in r.stdout, r.stdout + r.stderr
+    out = np.fromfile(tmp_path / "output" / "output_z.bin", dtype=np.float32)
+    gold = np.fromfile(tmp_path / "output" / "golden.bin", dtype=np.float32)
+    assert np.max(np.abs(out - gold) / np.maximum(np.abs(gold), 1.0)) < 2e-3
+
+
+@pytest.mark.gpu
+def test_gemm_main_reports_failure_on_wrong_golden(tmp_path):
+    subprocess.run([sys.executable, os.path.join(PKG, "host", "gen_data.py"), str(tmp_path), "256", "256", "256"], check=True)
+    g = np.fromfile(tmp_path / "output" / "golden.bin", dtype=np.float32)
+    (g + 1000.0).astype(np.float32).tofile(tmp_path / "output" / "golden.bin")
+    r = subprocess.run([os.path.join(PKG, "host", "gemm_main"), str(tmp_path), "256", "256", "256"], capture_output=True, text=True, timeout=120)
+    assert "test failed" in r.stdout and r.returncode == 1
+
+
+@pytest.mark.gpu
+def test_call_kernel_gemm_6144(oracle):
+    import torch
+    from pto_amd import datagen
+    lib = _lib("libpto_call_gemm.so")
+    lib.call_kernel.argtypes = [C.c_uint32] + [C.c_void_p] * 4
+    lib.call_kernel.restype = None
+    a, b = datagen.gemm_inputs(6144, 6144, 6144)
+    ta, tb = torch.from_numpy(a.view(np.int16)).cuda(), torch.from_numpy(b.view(np.int16)).cuda()
+    tc = torch.zeros((6144, 6144), dtype=torch.float32, device="cuda")
+    lib.call_kernel(24, torch.cuda.current_stream().cuda_stream, tc.data_ptr(), ta.data_ptr(), tb.data_ptr())
+    torch.cuda.synchronize()
+    rows = [0, 1, 255, 256, 3071, 4097, 6143]
+    want = oracle.gemm_f16f32(a, b, base_k=64, row0=0, row1=2)[:2]
+    got = tc[:2].cpu().numpy()
+    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 2e-3
+    af, bf = a.view(np.float16).astype(np.float32), b.view(np.float16).astype(np.float32)
+    ref = af[rows] @ bf.T
+    assert np.max(np.abs(tc[rows].cpu().numpy() - ref)) / np.max(np.abs(ref)) < 2e-3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("causal", [False, True])
+def test_call_kernel_flash_attention(causal):
+    import torch
+    lib = _lib("libpto_call_fa.so")
+    lib.call_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_bool] + [C.c_void_p] * 11
+    lib.call_kernel.restype = None
+    s0, s1, d = 256, 256 if causal else 512, 128
+    rng = np.random.default_rng(7)
+    q = (rng.standard_normal((s0, d)) * 1.5).astype(np.float16)
+    k = (rng.standard_normal((s1, d)) * 1.2).astype(np.float16)
+    v = rng.standard_normal((s1, d)).astype(np.float16)
+    tq, tk, tv = (torch.from_numpy(t.view(np.int16)).cuda() for t in (q, k, v))
+    o = torch.zeros((s0, d), dtype=torch.float32, device="cuda")
+    lib.call_kernel(torch.cuda.current_stream().cuda_stream, d, s0, s1, causal, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(),
+                    0, 0, 0, 0, 0, 0, 0)
+    torch.cuda.synchronize()
+    assert lib.pto_last_status_fa() == 0
+    s = q.astype(np.float64) @ k.astype(np.float64).T / np.sqrt(d)
+    if causal:
+        s = np.where(np.triu(np.ones((s0, s1), dtype=bool), 1), -np.inf, s)
+    p = np.exp(s - s.max(axis=1, keepdims=True))
+    want = (p / p.sum(axis=1, keepdims=True)) @ v.astype(np.float64)
+    assert np.max(np.abs(o.cpu().numpy() - want)) / np.max(np.abs(want)) < 2e-3
+    # unsupported head size: nothing is launched and the status says so
+    lib.call_kernel(torch.cuda.current_stream().cuda_stream, 64, s0, s1, causal, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(),
+                    0, 0, 0, 0, 0, 0, 0)
+    assert lib.pto_last_status_fa() != 0
