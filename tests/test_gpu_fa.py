@@ -108,6 +108,20 @@ def test_fa_config3_noncausal_b1_h16_s4096_d128():
     assert np.all(o.min(axis=2) >= v.astype(np.float32).min(axis=2) - 1e-3)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_fa_d128_workgroups_of_256_queries(causal):
+    """Enough (batch, head, 256-query) units for every compute unit: the eight-wavefront kernel runs; fp32 output + LSE."""
+    B, H, S, D = 2, 16, 2048, 128
+    q, k, v = datagen.fa_inputs(B, H, S, S, D, scale=1.0)
+    o, lse = fa_gpu(q, k, v, causal=causal, o_fp32=True)
+    for b, h in ((0, 0), (1, 13)):
+        want, want_lse = dense_fp64(q[b, h], k[b, h], v[b, h], causal=causal)
+        assert rel(o[b, h], want) <= TOL
+        assert np.max(np.abs(lse[b, h] - want_lse)) <= 1e-3
+    if causal:
+        assert np.allclose(o[:, :, 0, :], v[:, :, 0, :].astype(np.float32), atol=1e-6)
+
+
 def test_fa_config4_causal_b4_h32_s2048_d64():
     """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row."""
     B, H, S, D = 4, 32, 2048, 64
