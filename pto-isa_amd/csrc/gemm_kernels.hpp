@@ -17,11 +17,11 @@ constexpr int kXcds = 8; // MI355X: 8 accelerator dies, workgroups are dealt to 
 // regroup ids per XCD, then walk the tile grid in bands of GROUP_M tile rows so that the tiles
 // running together on one XCD share A and B panels.
 // ids [0, count) are dealt round-robin to the XCDs; give every XCD a contiguous range instead
+// (XCD x gets ids x, x + 8, ...: count / 8 of them, one more for x < count % 8)
 AICORE inline int RegroupXcd(int id, int count)
 {
-    if (count % kXcds != 0)
-        return id;
-    return (id % kXcds) * (count / kXcds) + id / kXcds;
+    const int xcd = id % kXcds, pos = id / kXcds, base = count / kXcds, extra = count % kXcds;
+    return xcd * base + (xcd < extra ? xcd : extra) + pos;
 }
 
 // linear tile id -> (tile row, tile column), walking bands of GROUP_M tile rows column by column
