@@ -120,11 +120,11 @@ def bench_gather(torch, lib, capi, datagen, steps, warmup):
 
 def cpu_baseline(datagen, size):
     """The reference CPU-simulation arithmetic timed on the host cores, on a bounded sample of the
-    6144^3 product: rows [0,4096) of C (2/3 of the work) through the oracle's port of the tile path
+    6144^3 product (all of it: 5-15 s on 16 cores) through the oracle's port of the tile path
     (TLOAD/TEXTRACT/TMATMUL[_ACC] per K-step of 64), threads over rows as the reference does."""
     from oracle import oracle
     a, b = datagen.gemm_inputs(size, size, size)
-    rows = 4096
+    rows = size
     cores = oracle.online_cpus()
     cores = min(cores, 16) if os.environ.get("OMP_NUM_THREADS") is None else min(cores, int(os.environ["OMP_NUM_THREADS"]))
     t0 = time.perf_counter()
@@ -132,7 +132,7 @@ def cpu_baseline(datagen, size):
     dt = time.perf_counter() - t0
     flops = 2.0 * rows * size * size
     out = {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
-           "sample": "rows 0..%d of C at m=n=k=%d (%.3g of the flops), %.1f s" % (rows - 1, size, rows / size, dt)}
+           "sample": "the whole m=n=k=%d product (rows 0..%d of C), %.1f s" % (size, rows - 1, dt)}
     ref = oracle.ref()
     if ref is not None:
         import ctypes as C
@@ -145,6 +145,35 @@ def cpu_baseline(datagen, size):
         dt1 = time.perf_counter() - t0
         out["reference_1536_single_tile"] = {"seconds": dt1, "tflops": 2.0 * 1536 ** 3 / dt1 / 1e12,
                                              "what": "compiled reference CPU-simulation headers, one TMATMUL 1536^3"}
+    return out
+
+
+def cpu_baselines_extra(datagen, cores):
+    """The oracle timed on bounded samples of the other workloads (reported beside the GPU figures, nothing more):
+    attention = the first 2048 query rows of one head of each configuration; TCVT = 2^24 elements; gather = 8192 rows."""
+    import numpy as np
+    from oracle import oracle
+    out = {}
+    for name, (B, H, S, D, causal) in (("fa_b1_h16_s4096_d128", (1, 16, 4096, 128, False)),
+                                       ("fa_causal_b4_h32_s2048_d64", (4, 32, 2048, 64, True))):
+        q, k, v = datagen.fa_inputs(1, 1, S, S, D, scale=1.0 / np.sqrt(D) if not causal else 1.0)
+        rows = min(S, 2048)
+        keys = S if not causal else rows             # causal: the first `rows` queries see the first `rows` keys
+        t0 = time.perf_counter()
+        oracle.fa_stream_f16(q[0, 0, :rows], k[0, 0, :keys], v[0, 0, :keys], tile_s1=128, causal=causal, threads=cores)
+        dt = time.perf_counter() - t0
+        flops = 4.0 * rows * keys * D * (0.5 if causal else 1.0)
+        out[name] = {"tflops": flops / dt / 1e12, "cores": cores, "kind": "port", "sample": "%d query rows x %d keys of one head, %.2f s" % (rows, keys, dt)}
+    x = datagen.tcvt_input(2048, 8192, inject=0.001).reshape(-1)
+    t0 = time.perf_counter()
+    oracle.tcvt_f32_f16(x)
+    dt = time.perf_counter() - t0
+    out["tcvt_f32_f16"] = {"gbs": x.size * 6.0 / dt / 1e9, "cores": 1, "kind": "port", "sample": "%d elements, %.2f s" % (x.size, dt)}
+    table, idx = datagen.gather_inputs(16384, 1024, 8192)
+    t0 = time.perf_counter()
+    oracle.gather_rows(table, idx)
+    dt = time.perf_counter() - t0
+    out["gather_rows"] = {"gbs": (8192 * 1024 * 2 * 2 + 8192 * 4.0) / dt / 1e9, "cores": 1, "kind": "port", "sample": "8192 rows of 1024 fp16, %.3f s" % dt}
     return out
 
 
@@ -228,6 +257,8 @@ def main():
                             "algorithmic_bytes": 2.0 * 2 * args.size ** 2 + 4.0 * args.size ** 2}
     if not args.no_cpu and only in ("", "gemm"):
         line["cpu_baseline"] = cpu_baseline(datagen, args.size)
+        if only == "":
+            line["extra"]["cpu_baselines"] = cpu_baselines_extra(datagen, line["cpu_baseline"]["cores"])
     print(json.dumps(line))
 
 
