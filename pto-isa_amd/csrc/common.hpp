@@ -32,7 +32,8 @@ inline int allow_lds(K kernel, int bytes)
 
 // defined in pto_gemm_w8.hip (workgroups of eight wavefronts)
 int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
-// defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries)
+// defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries, two groups of four waves in
+// opposite MFMA / softmax phases)
 int fa_fwd_d128_w8(hipStream_t st, void *o, float *lse, const _Float16 *q, const _Float16 *k, const _Float16 *v, int batch, int heads,
                    int seqQ, int seqKv, bool causal, bool oFp32);
 } // namespace pto_amd

@@ -14,8 +14,20 @@ constexpr int kBQ1 = 32 * PTO_WAVES_N; // queries per workgroup: one 32-query bl
 constexpr int kBKVDefault = 64; // keys per tile
 constexpr float kMaskValue = -3.40282e+38f; // pto_macro_fa_softmax.hpp:67
 
-// exchange a value with the lane 32 positions away
-AICORE inline float SwapHalves(float x) { return __shfl_xor(x, 32); }
+// max of x and of the value that the lane 32 positions away holds: one cross-half register swap
+// (after it `a` holds the lower half-wave's values in both halves, `b` the upper half-wave's)
+AICORE inline float MaxOverHalves(float x)
+{
+    float a = x, b = x;
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return fmaxf(a, b);
+}
+AICORE inline float SumOverHalves(float x)
+{
+    float a = x, b = x;
+    asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    return a + b;
+}
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 
@@ -88,27 +100,23 @@ AICORE inline s16x4 DsReadTr16(uint32_t addr)
     return v;
 }
 
-// V^T operand for O^T += V^T P^T: TEXTRACT of the [32 d, kBKV keys] block `db` of the transposed
-// V tile, taken straight from the row-major [keys, D] LDS image with transposing reads.  Key order
-// inside every 16-key MFMA step matches the order in which the accumulator layout holds P^T:
+// V^T operand for O^T += V^T P^T: TEXTRACT of [32 d, 16 keys] pieces of the transposed V tile, taken
+// straight from the row-major [keys, D] LDS image with transposing reads.  Key order inside every
+// 16-key MFMA step matches the order in which the accumulator layout holds P^T:
 // k slot j of half-wave h  <->  row 16t + 8(j/4) + 4h + j%4 of X^T, which holds key KeyOfRow(row).
 //
 // The reads are issued as assembly so that they carry no compiler-visible LDS dependency: before a
 // compiler-generated LDS read that may alias an outstanding asynchronous copy into LDS the compiler
 // waits for every outstanding copy, which would make the prefetch of the next tile synchronous.
 // The workgroup barrier at the top of a tile is what orders these reads after the copy that filled
-// the stage.  Wait<N>() is the matching wait on the LDS counter (LDS operations of a wave complete
-// in order: at most N younger ones may still be outstanding); it names the fragment registers as
-// operands so that no use of them can be moved above it.
+// the stage.  The matching wait on the LDS counter (LDS operations of a wave complete in order: at
+// most N younger ones may still be outstanding) names the fragment registers as operands so that
+// no use of them can be moved above it.
 template <int D, int kBKV>
 struct VTReader {
-    static constexpr int DB = D / 32, KS = kBKV / 16;
-    static constexpr int kReads = 2 * KS; // reads per 32-row block of V^T
+    static constexpr int DB = D / 32;
     static constexpr uint32_t kStepBytes = 16u * D * (uint32_t)sizeof(half);
-    static_assert(KS == 2 || KS == 4, "key tiles of 32 or 64");
-    struct Frag {
-        s16x4 part[KS][2];
-    };
+    static_assert(kBKV == 32 || kBKV == 64, "key tiles of 32 or 64");
     uint32_t base[DB][2]; // LDS byte address of (block db, read u) for key step 0 of a tile at LDS offset 0
 
     template <typename MatT>
@@ -128,56 +136,16 @@ struct VTReader {
                 base[db][u] = ldsBase + detail::mat_chunk_off<Geo::RowBytes>(key, d0 >> 3) + ((d0 & 7u) << 1);
             }
     }
-
-    template <uint32_t LDS_OFF, int... KSI>
-    AICORE inline void IssueSteps(Frag &f, int db, std::integer_sequence<int, KSI...>) const
-    {
-        ((f.part[KSI][0] = DsReadTr16<LDS_OFF + KSI * kStepBytes>(base[db][0]),
-          f.part[KSI][1] = DsReadTr16<LDS_OFF + KSI * kStepBytes>(base[db][1])),
-         ...);
-    }
-    // issue the reads of block db of the V tile at LDS offset LDS_OFF
-    template <uint32_t LDS_OFF>
-    AICORE inline void Issue(Frag &f, int db) const
-    {
-        IssueSteps<LDS_OFF>(f, db, std::make_integer_sequence<int, KS>());
-    }
-
-    template <int N>
-    AICORE static inline void Wait(Frag &f)
-    {
-        static_assert(N >= 0 && N <= 15, "the LDS counter has 4 bits");
-        if constexpr (KS == 4)
-            asm volatile("s_waitcnt lgkmcnt(%8)"
-                         : "+v"(f.part[0][0]), "+v"(f.part[0][1]), "+v"(f.part[1][0]), "+v"(f.part[1][1]), "+v"(f.part[2][0]),
-                           "+v"(f.part[2][1]), "+v"(f.part[3][0]), "+v"(f.part[3][1])
-                         : "n"(N));
-        else
-            asm volatile("s_waitcnt lgkmcnt(%4)"
-                         : "+v"(f.part[0][0]), "+v"(f.part[0][1]), "+v"(f.part[1][0]), "+v"(f.part[1][1])
-                         : "n"(N));
-    }
-
-    template <typename LeftT>
-    AICORE static inline void ToLeft(LeftT &dst, const Frag &f)
-    {
-        typedef short s16x8 __attribute__((ext_vector_type(8)));
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            const s16x8 both = {f.part[ks][0][0], f.part[ks][0][1], f.part[ks][0][2], f.part[ks][0][3],
-                                f.part[ks][1][0], f.part[ks][1][1], f.part[ks][1][2], f.part[ks][1][3]};
-            dst.st.f[0][ks] = __builtin_bit_cast(f16x8, both);
-        }
-    }
 };
 
-template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int NQ, int kBKV = kBKVDefault>
+template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int kBKV = kBKVDefault, bool PP = false>
 __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
                                                                       __gm__ const half *qAll, __gm__ const half *kAll,
                                                                       __gm__ const half *vAll, int heads, int seqQ,
                                                                       int seqKv, int numBH)
 {
-    constexpr int kBQ = kBQ1 * NQ; // every wave owns NQ blocks of 32 queries
+    constexpr int NQ = 1;          // 32-query blocks per wave
+    constexpr int kBQ = kBQ1 * NQ; // queries per workgroup
     constexpr int KB = kBKV / 32;  // 32-key blocks per tile
     constexpr int DB = D / 32;    // 32-wide blocks of the head dimension
     // ---- tiles ----
@@ -254,9 +222,11 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
     kr.Init();
     // `between(i)` runs before the MFMA on fragment i (the caller issues its asynchronous copies there).
     // A scheduling barrier after every MFMA keeps the issue order exactly as written.
-    auto scoreTile = [&](AccS(&sAcc)[KB], auto stageTag, auto &&between) {
+    // `extraTag`: number of LDS reads that between(kTotal - kAhead) issues itself (they are younger than every K read).
+    constexpr int kAheadK = 4, kTailHook = KB * (D / 16) - kAheadK;
+    auto scoreTile = [&](AccS(&sAcc)[KB], auto stageTag, auto &&between, auto extraTag) {
         constexpr uint32_t kOff = decltype(stageTag)::value * kStageBytes;
-        constexpr int KSTEPS = D / 16, kTotal = KB * KSTEPS, kAhead = 4;
+        constexpr int KSTEPS = D / 16, kTotal = KB * KSTEPS, kAhead = kAheadK, kExtra = decltype(extraTag)::value;
         using LeftStep = TileLeft<half, 32, 16, 32, 16>;
         using RightStep = TileRight<half, 16, kBQ, 16, kBQ>;
         f16x8 frag[kAhead + 1];
@@ -269,7 +239,8 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
             if constexpr (J < kTotal)
                 kr.template Issue<kOff, J % KB, J / KB>(frag[J % (kAhead + 1)]);
             between(i);
-            KReader<D>::template Wait<(kTotal - 1 - I < kAhead ? kTotal - 1 - I : kAhead)>(frag[I % (kAhead + 1)]);
+            KReader<D>::template Wait<(kTotal - 1 - I < kAhead ? kTotal - 1 - I : kAhead) + (I >= kTailHook ? kExtra : 0)>(
+                frag[I % (kAhead + 1)]);
             constexpr int kb = I % KB, ks = I / KB; // the KB accumulator chains alternate
             LeftStep a;
             RightStep b;
@@ -310,7 +281,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
                     locMax = fmaxf(locMax, sAcc[kb].st.f[0][nb][v]);
-            locMax = fmaxf(locMax, SwapHalves(locMax));
+            locMax = MaxOverHalves(locMax);
             // The running max only has to bound the scores well enough to keep exp() in range: it is
             // raised (and O, S rescaled by alpha) when a tile exceeds it by more than kSlack in the
             // exponent, i.e. P stays below 2^kSlack.  O / S and max*s + ln(S) do not depend on the choice.
@@ -341,39 +312,80 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
             runSum[nb] = t == 0 ? locSum : runSum[nb] * alpha[nb] + locSum;
         }
     };
-    // O^T = alpha O^T + V^T P^T.  vFrag holds block 0 of V^T of this tile (issued earlier); the reads
-    // of block db+1 are in flight while the MFMAs of block db run.
     using VT = VTReader<D, kBKV>;
     VT vt;
     vt.template Init<TileMatV>();
-    auto outputTile = [&](auto stageTag, int t, typename VT::Frag &vFirst, RightP &pRight, float(&alpha)[NQ], bool anyRaise) {
-        constexpr uint32_t kVOff = decltype(stageTag)::value * kStageBytes + kTileBytes;
-        typename VT::Frag vOther;
+    // O^T += V^T P^T with the 16-key step as the outer loop: consecutive MFMAs go to different accumulator
+    // blocks.  (An MFMA that needs the result of the one before it can only issue in the very cycle that one
+    // ends; when another wave of the SIMD issues vector instructions meanwhile, every such issue slips and the
+    // matrix pipe idles.  Independent MFMAs queue up behind each other and absorb the slips.)
+    // One step = the V^T fragments of all DB blocks for 16 keys; the step after it is in flight.
+    struct VStep {
+        s16x4 part[DB][2];
+    };
+    constexpr int kStepReads = 2 * DB;
+    auto issueVStep = [&](auto offTag, auto ksTag, VStep &f) {
+        constexpr uint32_t off = decltype(offTag)::value + decltype(ksTag)::value * VT::kStepBytes;
+        StaticFor<0, DB>([&](auto dbTag) {
+            constexpr int db = decltype(dbTag)::value;
+            f.part[db][0] = DsReadTr16<off>(vt.base[db][0]);
+            f.part[db][1] = DsReadTr16<off>(vt.base[db][1]);
+        });
+    };
+    auto waitVStep = [&](auto nTag, VStep &f) {
+        constexpr int N = decltype(nTag)::value;
+        static_assert(N >= 0 && N <= 15, "the LDS counter has 4 bits");
+        if constexpr (DB == 4)
+            asm volatile("s_waitcnt lgkmcnt(%8)"
+                         : "+v"(f.part[0][0]), "+v"(f.part[0][1]), "+v"(f.part[1][0]), "+v"(f.part[1][1]), "+v"(f.part[2][0]),
+                           "+v"(f.part[2][1]), "+v"(f.part[3][0]), "+v"(f.part[3][1])
+                         : "n"(N));
+        else
+            asm volatile("s_waitcnt lgkmcnt(%4)"
+                         : "+v"(f.part[0][0]), "+v"(f.part[0][1]), "+v"(f.part[1][0]), "+v"(f.part[1][1])
+                         : "n"(N));
+    };
+    // `first` holds step 0 (requested earlier); oAcc must have been initialised (this always accumulates)
+    auto outputTileWide = [&](auto stageTag, VStep &first, RightP &pRight, float(&alpha)[NQ], bool anyRaise) {
+        using VOff = std::integral_constant<uint32_t, decltype(stageTag)::value * kStageBytes + kTileBytes>;
+        using LeftStep = TileLeft<half, 32, 16, 32, 16>;
+        using RightStep = TileRight<half, 16, kBQ, 16, kBQ>;
+        typedef short s16x8 __attribute__((ext_vector_type(8)));
+        constexpr int KS = kBKV / 16;
+        VStep other;
+        if (anyRaise) { // wave-uniform: some lane's max was raised
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            typename VT::Frag &cur = (db & 1) ? vOther : vFirst;
-            typename VT::Frag &nxt = (db & 1) ? vFirst : vOther;
-            if (db + 1 < DB) {
-                vt.template Issue<kVOff>(nxt, db + 1);
-                VT::template Wait<VT::kReads>(cur);
-            } else {
-                VT::template Wait<0>(cur);
-            }
-            LeftVT vLeft;
-            VT::ToLeft(vLeft, cur);
-            if (t == 0) {
-                TMATMUL(oAcc[db], vLeft, pRight);
-            } else {
-                if (anyRaise) { // wave-uniform: some lane's max was raised
+            for (int db = 0; db < DB; ++db)
 #pragma unroll
-                    for (int nb = 0; nb < NQ; ++nb)
+                for (int nb = 0; nb < NQ; ++nb)
 #pragma unroll
-                        for (int v = 0; v < 16; ++v)
-                            oAcc[db].st.f[0][nb][v] *= alpha[nb];
-                }
-                TMATMUL_ACC(oAcc[db], oAcc[db], vLeft, pRight);
-            }
+                    for (int v = 0; v < 16; ++v)
+                        oAcc[db].st.f[0][nb][v] *= alpha[nb];
         }
+        StaticFor<0, KS>([&](auto ksTag) {
+            constexpr int ks = decltype(ksTag)::value;
+            VStep &cur = (ks & 1) ? other : first;
+            VStep &nxt = (ks & 1) ? first : other;
+            if constexpr (ks + 1 < KS) {
+                issueVStep(VOff(), std::integral_constant<int, ks + 1>(), nxt);
+                waitVStep(std::integral_constant<int, kStepReads>(), cur);
+            } else {
+                waitVStep(std::integral_constant<int, 0>(), cur);
+            }
+            RightStep b;
+#pragma unroll
+            for (int nb = 0; nb < NQ; ++nb)
+                b.st.f[nb][0] = pRight.st.f[nb][ks];
+            StaticFor<0, DB>([&](auto dbTag) {
+                constexpr int db = decltype(dbTag)::value;
+                const s16x8 both = {cur.part[db][0][0], cur.part[db][0][1], cur.part[db][0][2], cur.part[db][0][3],
+                                    cur.part[db][1][0], cur.part[db][1][1], cur.part[db][1][2], cur.part[db][1][3]};
+                LeftStep a;
+                a.st.f[0][0] = __builtin_bit_cast(f16x8, both);
+                TMATMUL_ACC(oAcc[db], oAcc[db], a, b);
+                __builtin_amdgcn_sched_barrier(0);
+            });
+        });
     };
     auto keyTile = [&](__gm__ half *base, int t) {
         const int tc = t < numTiles ? t : numTiles - 1; // past the end: re-fetch the last tile (nobody reads it)
@@ -381,6 +393,13 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
     };
     constexpr int kScoreMfma = KB * NQ * (D / 16);
 
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int nb = 0; nb < NQ; ++nb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                oAcc[db].st.f[0][nb][v] = 0.0f;
     {
         GlobalQT gmQ(qBase);
         TLOAD(qMat, gmQ);
@@ -391,10 +410,88 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
         wait_flag(PIPE_MTE1, PIPE_MTE2, EVENT_ID1); // Q^T is in registers everywhere: the stages may be filled
         GlobalKV gmK(kBase), gmV(vBase);
         TLOAD(kMat[0], gmK);
-        TLOAD(vMat[0], gmV);
+        if constexpr (!PP)
+            TLOAD(vMat[0], gmV);
         set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
     }
 
+    if constexpr (PP) {
+        // ---- two groups of four waves in opposite phases ----
+        // A SIMD issues one matrix or vector instruction per slot, and inside one wave an MFMA and the vector
+        // instructions after it do not overlap: the softmax of one wave can only hide under the MFMAs of ANOTHER
+        // wave of its SIMD.  Waves w and w+4 share a SIMD.  Time is cut into phases by workgroup barriers; in every
+        // phase one group (waves 0-3 in even phases, waves 4-7 in odd ones) runs the MFMAs of O^T += V^T P^T for its
+        // tile t-1 and of X^T = K Q^T for its tile t, while the other group runs the softmax of its tile and
+        // issues its share of the copies for the coming phases.
+        //   bundle b = {K tile b, V tile b-1} lives in stage b % 2 and is read in phases 2b (first group) and
+        //   2b+1 (second group); it is copied during phases 2b-2 (second group's share) and 2b-1 (first group's),
+        //   i.e. in its softmax phase of step t a wave of group g copies its share of bundle t+1+g.
+        // The wave in its MFMA phase runs at raised priority.
+        static_assert(kBlockWaves == 8 && NQ == 1, "two groups of four waves");
+        const int group = hw::wave_n() >> 2;
+        AccS sAcc[KB];
+        RightP pRight;
+        float alpha[NQ];
+        bool anyRaise = false;
+        auto phaseEnd = [&]() { // own copies landed, own LDS reads done, everyone arrived
+            set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+            wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+        };
+        auto loadBundle = [&](int b) { // this wave's share of bundle b
+            TileMatK kDst;
+            TileMatV vDst;
+            const uint32_t off = (uint32_t)(b & 1) * kStageBytes;
+            TASSIGN(kDst, off);
+            TASSIGN(vDst, off + kTileBytes);
+            GlobalKV gmK = keyTile(kBase, b), gmV = keyTile(vBase, b - 1);
+            TLOAD(kDst, gmK);
+            TLOAD(vDst, gmV);
+        };
+        // Step t of a wave: MFMA phase = scores of tile t, then output of tile t-1; softmax phase = tile t.
+        // The first V^T step is requested right after the last K fragment so that the output MFMAs follow the
+        // score MFMAs without a gap.  The copies are issued at the start of the softmax phase, which is the
+        // shorter of the two (measured: a copy instruction holds its wave for 30-100 cycles wherever it sits).
+        auto ppStep = [&](auto stageTag, int t) {
+            constexpr int st = decltype(stageTag)::value;
+            using VOff = std::integral_constant<uint32_t, st * kStageBytes + kTileBytes>;
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_setprio(3); // the wave that feeds the matrix pipe issues first
+            VStep vFirst;
+            if (t < numTiles) {
+                scoreTile(sAcc, stageTag, [&](auto i) {
+                    constexpr int I = decltype(i)::value;
+                    if constexpr (I == kTailHook) // at t == 0 nobody uses what these reads return
+                        issueVStep(VOff(), std::integral_constant<int, 0>(), vFirst);
+                }, std::integral_constant<int, kStepReads>());
+            } else {
+                issueVStep(VOff(), std::integral_constant<int, 0>(), vFirst);
+            }
+            if (t > 0)
+                outputTileWide(stageTag, vFirst, pRight, alpha, anyRaise);
+            __builtin_amdgcn_sched_barrier(0);
+            phaseEnd();
+            __builtin_amdgcn_sched_barrier(0);
+            if (t < numTiles) {
+                __builtin_amdgcn_s_setprio(0);
+                loadBundle(t + 1 + group);
+                softmaxTile(sAcc, t, pRight, alpha, anyRaise);
+                __builtin_amdgcn_sched_barrier(0);
+                phaseEnd();
+            }
+        };
+        phaseEnd(); // K tile 0 has landed
+        if (group == 1) { // phase 0: the second group has no scores yet
+            loadBundle(1);
+            phaseEnd();
+        }
+        for (int tile = 0; tile <= numTiles; tile += 2) {
+            ppStep(std::integral_constant<int, 0>(), tile);
+            if (tile + 1 <= numTiles)
+                ppStep(std::integral_constant<int, 1>(), tile + 1);
+        }
+        if (group == 0) // pairs with the barrier that ends the second group's last phase
+            phaseEnd();
+    } else {
     // One key tile in LDS stage st (a compile-time constant: every LDS address is an immediate).
     auto tileStep = [&](auto stageTag, int t) {
         constexpr int st = decltype(stageTag)::value;
@@ -415,25 +512,26 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
                 TLOAD(vMat[st ^ 1], gmV);
                 set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
             }
-        });
-        typename VT::Frag vFirst;
-        vt.template Issue<st * kStageBytes + kTileBytes>(vFirst, 0); // lands during the softmax
+        }, std::integral_constant<int, 0>());
+        VStep vFirst; // lands during the softmax
+        issueVStep(std::integral_constant<uint32_t, st * kStageBytes + kTileBytes>(), std::integral_constant<int, 0>(), vFirst);
         RightP pRight;
         float alpha[NQ];
         bool anyRaise;
         softmaxTile(sAcc, t, pRight, alpha, anyRaise);
-        outputTile(stageTag, t, vFirst, pRight, alpha, anyRaise);
+        outputTileWide(stageTag, vFirst, pRight, alpha, anyRaise);
     };
     for (int tile = 0; tile < numTiles; tile += 2) {
         tileStep(std::integral_constant<int, 0>(), tile);
         if (tile + 1 < numTiles)
             tileStep(std::integral_constant<int, 1>(), tile + 1);
     }
+    }
     hw::wait_vm0(); // the copy issued by the last tile must not outlive the workgroup's LDS
     // ---- finish: O /= S, write O (and LSE) ----
 #pragma unroll
     for (int nb = 0; nb < NQ; ++nb) {
-        const float total = runSum[nb] + SwapHalves(runSum[nb]);
+        const float total = SumOverHalves(runSum[nb]);
         const float inv = 1.0f / total;
         const int64_t row = (int64_t)bh * seqQ + myQuery + 32 * nb;
 #pragma unroll
@@ -465,20 +563,20 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
 PTO_DEVICE_CODE_END
 
 namespace {
-template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS = 1, int NQ = 1, int kBKV = kBKVDefault>
+template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS = 1, int kBKV = kBKVDefault, bool PP = false>
 int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads,
               int seqQ, int seqKv)
 {
-    if (seqQ % (kBQ1 * NQ) || seqKv % kBKV)
+    if (seqQ % kBQ1 || seqKv % kBKV)
         return PTO_ERR_UNSUPPORTED;
-    static_assert(D * kBQ1 * NQ <= 4 * kBKV * D, "Q^T must fit the K/V stages it is staged in");
+    static_assert(D * kBQ1 <= 4 * kBKV * D, "Q^T must fit the K/V stages it is staged in");
     constexpr int lds = 2 * 2 * kBKV * D * (int)sizeof(half);
-    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32, MIN_BLOCKS, NQ, kBKV>;
+    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32, MIN_BLOCKS, kBKV, PP>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
     const int numBH = batch * heads;
-    const long long blocks = (long long)numBH * (seqQ / (kBQ1 * NQ));
+    const long long blocks = (long long)numBH * (seqQ / kBQ1);
     if (blocks > 0x7fffffffLL)
         return PTO_ERR_UNSUPPORTED;
     kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH);

@@ -122,6 +122,22 @@ def test_fa_d128_workgroups_of_256_queries(causal):
         assert np.allclose(o[:, :, 0, :], v[:, :, 0, :].astype(np.float32), atol=1e-6)
 
 
+@pytest.mark.parametrize("Skv,causal", [(64, False), (320, False), (320, True), (256, True), (384, False)])
+def test_fa_d128_eight_wave_kernel_tile_counts(Skv, causal):
+    """The eight-wavefront kernel (two wave groups in opposite phases) on one, odd and even numbers of key tiles,
+    seq_kv != seq_q, causal with an offset diagonal; fp16 output and fp32 output agree."""
+    B, H, Sq, D = 16, 16, 256, 128     # 256 workgroups of 256 queries: the dispatch picks the eight-wavefront kernel
+    q, k, v = datagen.fa_inputs(B, H, Sq, Skv, D, scale=1.0)
+    o, lse = fa_gpu(q, k, v, causal=causal, o_fp32=True)
+    assert np.all(np.isfinite(o)) and np.all(np.isfinite(lse))
+    for b, h in ((0, 0), (7, 3), (15, 15)):
+        want, want_lse = dense_fp64(q[b, h], k[b, h], v[b, h], causal=causal)
+        assert rel(o[b, h], want) <= TOL
+        assert np.max(np.abs(lse[b, h] - want_lse)) <= 1e-3
+    o16, _ = fa_gpu(q, k, v, causal=causal, o_fp32=False, want_lse=False)
+    assert np.array_equal(o16, o.astype(np.float16).astype(np.float32))
+
+
 def test_fa_config4_causal_b4_h32_s2048_d64():
     """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row."""
     B, H, S, D = 4, 32, 2048, 64
