@@ -7,8 +7,9 @@
 //                    tile) and 16-byte chunks are XOR-swizzled so that the ds_read_b128 fragment
 //                    loads of TEXTRACT are bank-conflict free.  BLayout/SLayout only select which
 //                    logical dimension is the contiguous one.
-//   Left/Right       per-wave MFMA operand fragments in VGPRs: [32-row block][16-wide k step] x 8 halves.
-//   Acc              per-wave MFMA accumulator fragments (AGPRs): [row block][col block] x 16 floats.
+//   Left/Right       per-wave MFMA operand fragments in VGPRs: [row block][k step] x 8 halves; a block is
+//                    PTO_MFMA_M rows, a k step 512 / PTO_MFMA_M columns (32 x 16 or 16 x 32).
+//   Acc              per-wave MFMA accumulator fragments: [row block][col block] x (16 or 4) floats.
 //   Vec              register tile spread over the workgroup in chunks of 8 consecutive elements of
 //                    the tile's linear (BLayout) order: chunk q -> thread q % kBlockThreads, slot q / kBlockThreads.
 //
@@ -29,9 +30,21 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 namespace detail {
 
-constexpr int kMfmaM = 32; // v_mfma_f32_32x32x16: 32 x 32 output block
-constexpr int kMfmaK = 16; // k extent of one MFMA
+static_assert(PTO_MFMA_M == 32 || PTO_MFMA_M == 16, "v_mfma_f32_32x32x16 or v_mfma_f32_16x16x32");
+constexpr int kMfmaM = PTO_MFMA_M;                     // the MFMA's output block is kMfmaM x kMfmaM
+constexpr int kMfmaK = 512 / kMfmaM;                   // k extent of one MFMA
+constexpr int kAccElems = kMfmaM * kMfmaM / kWaveSize; // accumulator values per lane and block
 constexpr int kVecChunk = 8;
+typedef float AccFrag __attribute__((ext_vector_type(kAccElems)));
+
+// Operand layout (both shapes): lane l holds row (column) l % kMfmaM of the block and the eight k values
+// 8 * (l / kMfmaM) .. +7 of the step.  Result layout: lane l holds column l % kMfmaM and, in register v,
+// row acc_elem_row(v) + acc_lane_row(l) of the block.
+PTO_DEV uint32_t frag_lane_major(uint32_t lane) { return lane % kMfmaM; }
+PTO_DEV uint32_t frag_lane_kgroup(uint32_t lane) { return lane / kMfmaM; }
+PTO_DEV int acc_lane_col(uint32_t lane) { return (int)(lane % kMfmaM); }
+PTO_DEV int acc_lane_row(uint32_t lane) { return (int)(lane / kMfmaM) * 4; }
+constexpr int acc_elem_row(int v) { return (v >> 2) * (4 * (kWaveSize / kMfmaM)) + (v & 3); }
 
 template <typename T>
 struct FragOf {
@@ -63,8 +76,8 @@ struct TileStorage<TileType::Mat, T, Rows, Cols> {
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Left, T, Rows, Cols> {
     static_assert(sizeof(T) == 2, "Left tiles: fp16 / bf16 operands");
-    static_assert(Rows % (kMfmaM * kWavesM) == 0, "Left tile rows must be a multiple of 32 x PTO_WAVES_M");
-    static_assert(Cols % kMfmaK == 0, "Left tile cols (K) must be a multiple of 16");
+    static_assert(Rows % (kMfmaM * kWavesM) == 0, "Left tile rows must be a multiple of PTO_MFMA_M x PTO_WAVES_M");
+    static_assert(Cols % kMfmaK == 0, "Left tile cols (K) must be a multiple of the MFMA's k extent");
     static constexpr int MB = Rows / (kMfmaM * kWavesM);
     static constexpr int KS = Cols / kMfmaK;
     typename FragOf<T>::type f[MB][KS];
@@ -73,8 +86,8 @@ struct TileStorage<TileType::Left, T, Rows, Cols> {
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Right, T, Rows, Cols> {
     static_assert(sizeof(T) == 2, "Right tiles: fp16 / bf16 operands");
-    static_assert(Cols % (kMfmaM * kWavesN) == 0, "Right tile cols must be a multiple of 32 x PTO_WAVES_N");
-    static_assert(Rows % kMfmaK == 0, "Right tile rows (K) must be a multiple of 16");
+    static_assert(Cols % (kMfmaM * kWavesN) == 0, "Right tile cols must be a multiple of PTO_MFMA_M x PTO_WAVES_N");
+    static_assert(Rows % kMfmaK == 0, "Right tile rows (K) must be a multiple of the MFMA's k extent");
     static constexpr int NB = Cols / (kMfmaM * kWavesN);
     static constexpr int KS = Rows / kMfmaK;
     typename FragOf<T>::type f[NB][KS];
@@ -84,10 +97,10 @@ template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Acc, T, Rows, Cols> {
     static_assert(sizeof(T) == 4, "Acc tiles: fp32 accumulators");
     static_assert(Rows % (kMfmaM * kWavesM) == 0 && Cols % (kMfmaM * kWavesN) == 0,
-                  "Acc tile must be a multiple of (32 x PTO_WAVES_M) x (32 x PTO_WAVES_N)");
+                  "Acc tile must be a multiple of (PTO_MFMA_M x PTO_WAVES_M) x (PTO_MFMA_M x PTO_WAVES_N)");
     static constexpr int MB = Rows / (kMfmaM * kWavesM);
     static constexpr int NB = Cols / (kMfmaM * kWavesN);
-    f32x16 f[MB][NB];
+    AccFrag f[MB][NB];
 };
 
 template <typename T, int Rows, int Cols>

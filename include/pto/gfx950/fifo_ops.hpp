@@ -74,15 +74,15 @@ PTO_DEV void lds_image_store(uint32_t off, TileT &tile)
     if constexpr (TileT::Loc == TileType::Acc) {
         using S = typename TileT::Storage;
         const uint32_t lane = (uint32_t)hw::lane();
-        const int rbase = hw::wave_m() * (S::MB * kMfmaM) + (int)(lane >> 5) * 4;
-        const int cbase = hw::wave_n() * (S::NB * kMfmaM) + (int)(lane & 31u);
+        const int rbase = hw::wave_m() * (S::MB * kMfmaM) + acc_lane_row(lane);
+        const int cbase = hw::wave_n() * (S::NB * kMfmaM) + acc_lane_col(lane);
 #pragma unroll
         for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
             for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int r = rbase + mb * kMfmaM + (v >> 2) * 8 + (v & 3), c = cbase + nb * kMfmaM;
+                for (int v = 0; v < kAccElems; ++v) {
+                    const int r = rbase + mb * kMfmaM + acc_elem_row(v), c = cbase + nb * kMfmaM;
                     img[r * TileT::Cols + c] = store_cast<T>(tile.st.f[mb][nb][v]);
                 }
     } else {

@@ -1,4 +1,5 @@
-// TMATMUL / TMATMUL_ACC / TMATMUL_BIAS for gfx950: chains of v_mfma_f32_32x32x16_{f16,bf16}.
+// TMATMUL / TMATMUL_ACC / TMATMUL_BIAS for gfx950: chains of v_mfma_f32_32x32x16_{f16,bf16} (or, with
+// PTO_MFMA_M 16, v_mfma_f32_16x16x32_{f16,bf16}).
 //
 // Reference semantics (include/pto/cpu/TMatmul.hpp:73-116):
 //   C[i,j] = (acc ? acc[i,j] : 0) + sum_k (float)A[i,k] * (float)B[k,j],  M,K,N = a.validRow, a.validCol, b.validCol
@@ -12,8 +13,26 @@
 namespace pto {
 namespace detail {
 
-PTO_DEV f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-PTO_DEV f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+// (the accumulator type is a template parameter only so that the branch for the other MFMA shape is discarded
+// instead of type-checked)
+template <typename C>
+PTO_DEV C mfma32(f16x8 a, f16x8 b, C c)
+{
+    static_assert(std::is_same_v<C, AccFrag>, "accumulator fragment of the configured MFMA shape");
+    if constexpr (sizeof(C) == 64)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+template <typename C>
+PTO_DEV C mfma32(bf16x8 a, bf16x8 b, C c)
+{
+    static_assert(std::is_same_v<C, AccFrag>, "accumulator fragment of the configured MFMA shape");
+    if constexpr (sizeof(C) == 64)
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
 
 template <typename AccT, typename LeftT, typename RightT>
 PTO_DEV constexpr void check_mad()
@@ -40,10 +59,10 @@ PTO_DEV void mad(AccT &out, const AccT &in, const LeftT &a, const RightT &b)
     for (int mb = 0; mb < SA::MB; ++mb)
 #pragma unroll
         for (int nb = 0; nb < SA::NB; ++nb) {
-            f32x16 c;
+            AccFrag c;
             if constexpr (kZeroInit) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i)
+                for (int i = 0; i < kAccElems; ++i)
                     c[i] = 0.0f;
             } else {
                 c = in.st.f[mb][nb];
@@ -83,14 +102,14 @@ PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasRow bias)
     detail::check_mad<AccT, LeftT, RightT>();
     detail::mad<true>(c, c, a, b);
     using SA = typename AccT::Storage;
-    const int col0 = hw::wave_n() * (SA::NB * detail::kMfmaM) + (hw::lane() & 31);
+    const int col0 = hw::wave_n() * (SA::NB * detail::kMfmaM) + detail::acc_lane_col((uint32_t)hw::lane());
 #pragma unroll
     for (int nb = 0; nb < SA::NB; ++nb) {
         const float bv = bias.row[col0 + nb * detail::kMfmaM]; // cpu/TMatmul.hpp:109-115: added after the product
 #pragma unroll
         for (int mb = 0; mb < SA::MB; ++mb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
+            for (int i = 0; i < detail::kAccElems; ++i)
                 c.st.f[mb][nb][i] += bv;
     }
 }

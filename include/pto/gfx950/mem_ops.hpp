@@ -285,8 +285,8 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 }
 
 // ----------------------------------------------------------------- TEXTRACT
-// dst[i,j] = src[idxRow+i, idxCol+j].  Mat -> Left / Right: one ds_read_b128 per 32-row block and
-// 16-wide k step, in the v_mfma_f32_32x32x16 operand layout (lane l: row/col l%32, k = 8*(l/32)..+7).
+// dst[i,j] = src[idxRow+i, idxCol+j].  Mat -> Left / Right: one ds_read_b128 per row block and k step, in the
+// MFMA operand layout (lane l: row/col l % kMfmaM, k = 8*(l / kMfmaM)..+7).
 // The k offset must be a multiple of 8 elements (16 bytes).
 template <typename DstT, typename SrcT>
 PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t idxCol = 0)
@@ -297,7 +297,8 @@ PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t i
     using Frag = typename detail::FragOf<typename DstT::DType>::type;
     const char *lds = hw::lds_base() + src.st.lds;
     const uint32_t lane = (uint32_t)hw::lane();
-    const uint32_t l32 = lane & 31u, khalf = lane >> 5;
+    const uint32_t l32 = detail::frag_lane_major(lane), khalf = detail::frag_lane_kgroup(lane);
+    constexpr uint32_t kStepChunks = detail::kMfmaK / 8; // 16-byte chunks per k step
     if constexpr (DstT::Loc == TileType::Left) {
         static_assert(Geo::colsK, "[PTO][SA] TEXTRACT to Left: source must be contiguous along columns (Nz / row-major)");
         using S = typename DstT::Storage;
@@ -308,7 +309,7 @@ PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t i
 #pragma unroll
             for (int ks = 0; ks < S::KS; ++ks)
                 dst.st.f[mb][ks] = *reinterpret_cast<const Frag *>(
-                    lds + detail::mat_chunk_off<Geo::RowBytes>(row0 + mb * detail::kMfmaM, chunk0 + ks * 2));
+                    lds + detail::mat_chunk_off<Geo::RowBytes>(row0 + mb * detail::kMfmaM, chunk0 + ks * kStepChunks));
     } else if constexpr (DstT::Loc == TileType::Right) {
         static_assert(!Geo::colsK, "[PTO][SA] TEXTRACT to Right: source must be contiguous along rows (Zn / column-major)");
         using S = typename DstT::Storage;
@@ -319,7 +320,7 @@ PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t i
 #pragma unroll
             for (int ks = 0; ks < S::KS; ++ks)
                 dst.st.f[nb][ks] = *reinterpret_cast<const Frag *>(
-                    lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * 2));
+                    lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * kStepChunks));
     } else {
         static_assert(DstT::Loc == TileType::Left, "[PTO][SA] TEXTRACT: destination must be a Left or Right tile");
     }
@@ -354,8 +355,8 @@ PTO_DEV D store_cast(S v)
         return static_cast<D>(v); // fp32 -> fp16 / bf16: hardware round-to-nearest-even
 }
 
-// Acc fragments -> GM.  v_mfma_f32_32x32x16 result layout: lane l, register v holds
-// row 8*(v/4) + 4*(l/32) + v%4, column l%32 of the 32 x 32 block.
+// Acc fragments -> GM.  MFMA result layout: lane l, register v holds row acc_elem_row(v) + acc_lane_row(l),
+// column l % kMfmaM of the block (32 x 32: row 8*(v/4) + 4*(l/32) + v%4).
 template <typename TileT, typename G, AtomicType atomic>
 PTO_DEV void tstore_acc(G &dst, TileT &src)
 {
@@ -365,8 +366,8 @@ PTO_DEV void tstore_acc(G &dst, TileT &src)
     const int64_t st_r = dst.GetStride(3), st_c = dst.GetStride(4);
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     const uint32_t lane = (uint32_t)hw::lane();
-    const int rbase = hw::wave_m() * (S::MB * kMfmaM) + (int)(lane >> 5) * 4;
-    const int cbase = hw::wave_n() * (S::NB * kMfmaM) + (int)(lane & 31u);
+    const int rbase = hw::wave_m() * (S::MB * kMfmaM) + acc_lane_row(lane);
+    const int cbase = hw::wave_n() * (S::NB * kMfmaM) + acc_lane_col(lane);
     constexpr bool full = TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols;
 #pragma unroll
     for (int mb = 0; mb < S::MB; ++mb)
@@ -374,8 +375,8 @@ PTO_DEV void tstore_acc(G &dst, TileT &src)
         for (int nb = 0; nb < S::NB; ++nb) {
             const int c = cbase + nb * kMfmaM;
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = rbase + mb * kMfmaM + (v >> 2) * 8 + (v & 3);
+            for (int v = 0; v < kAccElems; ++v) {
+                const int r = rbase + mb * kMfmaM + acc_elem_row(v);
                 if (full || (r < vr && c < vc)) {
                     GT *p = gm + (int64_t)r * st_r + (int64_t)c * st_c;
                     if constexpr (atomic == AtomicType::AtomicAdd)

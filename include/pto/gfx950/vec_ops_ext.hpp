@@ -389,15 +389,15 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
     using T = typename DstT::DType;
     __shared__ T stage[AccT::Rows * AccT::Cols];
     const uint32_t lane = (uint32_t)hw::lane();
-    const int rbase = hw::wave_m() * (S::MB * detail::kMfmaM) + (int)(lane >> 5) * 4;
-    const int cbase = hw::wave_n() * (S::NB * detail::kMfmaM) + (int)(lane & 31u);
+    const int rbase = hw::wave_m() * (S::MB * detail::kMfmaM) + detail::acc_lane_row(lane);
+    const int cbase = hw::wave_n() * (S::NB * detail::kMfmaM) + detail::acc_lane_col(lane);
 #pragma unroll
     for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
         for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = rbase + mb * detail::kMfmaM + (v >> 2) * 8 + (v & 3), c = cbase + nb * detail::kMfmaM;
+            for (int v = 0; v < detail::kAccElems; ++v) {
+                const int r = rbase + mb * detail::kMfmaM + detail::acc_elem_row(v), c = cbase + nb * detail::kMfmaM;
                 stage[r * AccT::Cols + c] = (T)src.st.f[mb][nb][v];
             }
     hw::lds_barrier();

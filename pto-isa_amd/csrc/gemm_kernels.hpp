@@ -190,7 +190,7 @@ AICORE inline __attribute__((always_inline)) void MixTile(__gm__ float *out, __g
 #pragma unroll
         for (int nb = 0; nb < ResTile::Storage::NB; ++nb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
+            for (int i = 0; i < detail::kAccElems; ++i)
                 cTile.st.f[mb][nb][i] = 0.0f;
 
     // the host guarantees kLoop % STAGES == 0 and kLoop >= 2 * STAGES
@@ -259,12 +259,129 @@ AICORE inline __attribute__((always_inline)) void MixTile(__gm__ float *out, __g
         TSTORE(dstGlobal, cTile);
 }
 
+// The same K-step pipeline with the two halves of a step taken along M instead of K: the wave multiplies the
+// upper half of its rows (first half), then the lower half, by the whole [32, BN] B panel of the step.  Works with
+// either MFMA shape (a 16 x 16 x 32 MFMA covers the whole 32-wide K-step, so the step cannot be halved along K).
+// Row halves are halves of the WORKGROUP tile: wave row wm owns rows wm*BM/4 .. of each half.
+template <int BM, int BN, int STAGES>
+AICORE inline __attribute__((always_inline)) void MixTileRows(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m,
+                                                              int n, int k, int row0, int col0, int kLoop)
+{
+    constexpr int BK = 32, HM = BM / 2;
+    using TileMatA = Tile<TileType::Mat, half, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
+    using TileMatB = Tile<TileType::Mat, half, BK, BN, BLayout::RowMajor, BK, BN, SLayout::ColMajor>;
+    using LeftHalf = TileLeft<half, HM, BK, HM, BK>;
+    using RightTile = TileRight<half, BK, BN, BK, BN>;
+    using AccHalf = TileAcc<float, HM, BN, HM, BN>;
+    using ShapeA = TileShape2D<half, BM, BK, Layout::ND>;
+    using StrideA = BaseShape2D<half, DYNAMIC, DYNAMIC, Layout::ND>;
+    using GlobalA = GlobalTensor<half, ShapeA, StrideA, Layout::ND>;
+    using ShapeB = TileShape2D<half, BK, BN, Layout::DN>;
+    using StrideB = BaseShape2D<half, DYNAMIC, DYNAMIC, Layout::DN>;
+    using GlobalB = GlobalTensor<half, ShapeB, StrideB, Layout::DN>;
+    using ShapeC = TileShape2D<float, HM, BN, Layout::ND>;
+    using StrideC = BaseShape2D<float, DYNAMIC, DYNAMIC, Layout::ND>;
+    using GlobalC = GlobalTensor<float, ShapeC, StrideC, Layout::ND>;
+
+    constexpr uint32_t kABytes = BM * BK * sizeof(half), kBBytes = BK * BN * sizeof(half);
+    constexpr uint32_t kStage = kABytes + kBBytes;
+    constexpr int kLoadsPerStep = TLoadInstrs<TileMatA>() + TLoadInstrs<TileMatB>();
+    constexpr int kMfmaPerHalf = AccHalf::Storage::MB * AccHalf::Storage::NB * LeftHalf::Storage::KS;
+    constexpr int kReadsA = LeftHalf::Storage::MB * LeftHalf::Storage::KS, kReadsB = RightTile::Storage::NB * RightTile::Storage::KS;
+    static_assert(STAGES >= 3, "needs at least three L1 stages");
+    static_assert(kMfmaPerHalf % kLoadsPerStep == 0 && kMfmaPerHalf >= kReadsA, "issue pattern below");
+
+    __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)row0 * k;
+    __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)col0 * k;
+    const StrideA strideA(m, k);
+    const StrideB strideB(k, n);
+
+    TileMatA aMat[STAGES];
+    TileMatB bMat[STAGES];
+#pragma unroll
+    for (int s = 0; s < STAGES; ++s) {
+        TASSIGN(aMat[s], s * kStage);
+        TASSIGN(bMat[s], s * kStage + kABytes);
+    }
+    LeftHalf aUp, aDn;
+    RightTile bAll;
+    AccHalf cUp, cDn;
+#pragma unroll
+    for (int mb = 0; mb < AccHalf::Storage::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < AccHalf::Storage::NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < detail::kAccElems; ++i) {
+                cUp.st.f[mb][nb][i] = 0.0f;
+                cDn.st.f[mb][nb][i] = 0.0f;
+            }
+
+    // the host guarantees kLoop % STAGES == 0 and kLoop >= 2 * STAGES
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+        GlobalA gmA(aPanel + (int64_t)s * BK, ShapeA(), strideA);
+        GlobalB gmB(bPanel + (int64_t)s * BK, ShapeB(), strideB);
+        TLOAD(aMat[s], gmA);
+        TLOAD(bMat[s], gmB);
+    }
+    wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // stage 0 is complete
+    TEXTRACT(aUp, aMat[0], 0, 0);
+    TEXTRACT(aDn, aMat[0], HM, 0);
+    TEXTRACT(bAll, bMat[0], 0, 0);
+
+    auto step = [&](auto stageTag, int it) {
+        constexpr int s = decltype(stageTag)::value;
+        constexpr int sNext = (s + 1) % STAGES, sLoad = (s + STAGES - 1) % STAGES;
+        hw::wait_vm<(STAGES - 3) * kLoadsPerStep>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const int fetch = it + STAGES - 1 < kLoop ? it + STAGES - 1 : kLoop - 1;
+        GlobalA gmA(aPanel + (int64_t)fetch * BK, ShapeA(), strideA);
+        GlobalB gmB(bPanel + (int64_t)fetch * BK, ShapeB(), strideB);
+        TLOAD(aMat[sLoad], gmA);
+        TLOAD(bMat[sLoad], gmB);
+        TMATMUL_ACC(cUp, cUp, aUp, bAll);
+        TEXTRACT(aUp, aMat[sNext], 0, 0);
+        TMATMUL_ACC(cDn, cDn, aDn, bAll);
+        TEXTRACT(aDn, aMat[sNext], HM, 0);
+        TEXTRACT(bAll, bMat[sNext], 0, 0);
+        // issue order: MFMAs of the upper half with the copies between them, then the fragment reads for the
+        // next step's upper half one per MFMA of the lower half, then the remaining reads
+#pragma unroll
+        for (int i = 0; i < kLoadsPerStep; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerHalf / kLoadsPerStep, 0);
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < kReadsA; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerHalf / kReadsA, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, kReadsA + kReadsB, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::integral_constant;
+    for (int it = 0; it < kLoop; it += STAGES) {
+        step(integral_constant<int, 0>(), it);
+        step(integral_constant<int, 1>(), it + 1);
+        step(integral_constant<int, 2>(), it + 2);
+        if constexpr (STAGES == 4)
+            step(integral_constant<int, 3>(), it + 3);
+    }
+    hw::wait_vm0(); // the copies issued past the end of K must not outlive the workgroup's LDS
+    GlobalC dstUp(out + (int64_t)row0 * n + col0, ShapeC(), StrideC(m, n));
+    GlobalC dstDn(out + (int64_t)(row0 + HM) * n + col0, ShapeC(), StrideC(m, n));
+    TSTORE(dstUp, cUp);
+    TSTORE(dstDn, cDn);
+}
+
 // Work split of the kernel below.  The first `fullTiles` workgroups (whole rounds over the compute
 // units) own one BM x BN C tile each.  The tiles of the last, partial round are divided so that the
 // round fills the machine: tailMode 1 = four (BM/2) x (BN/2) quarter tiles, one workgroup each;
 // tailMode 2 = `splitK` K-ranges per tile whose partial products are added into a zeroed C tile
 // with TSTORE<AtomicAdd> (slow: one atomic per element).
-template <int BM, int BN, int STAGES, int GROUP_M>
+// ROWS: the halves of a K-step are taken along M (MixTileRows; needed for the 16 x 16 x 32 MFMA) instead of along K.
+template <int BM, int BN, int STAGES, int GROUP_M, bool ROWS = false>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     void GemmF16F32Mix(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k,
                        int fullTiles, int tailMode, int splitK)
@@ -276,8 +393,12 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
         TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
         const int sub = u % 4;
-        MixTile<BM / 2, BN / 2, STAGES>(out, src0, src1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
-                                        tn * BN + (sub & 1) * (BN / 2), 0, k / 32, false);
+        if constexpr (ROWS)
+            MixTileRows<BM / 2, BN / 2, STAGES>(out, src0, src1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
+                                                tn * BN + (sub & 1) * (BN / 2), k / 32);
+        else
+            MixTile<BM / 2, BN / 2, STAGES>(out, src0, src1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
+                                            tn * BN + (sub & 1) * (BN / 2), 0, k / 32, false);
         return;
     }
     // whole tiles and K-ranges of whole tiles share one call site, so the tile body is inlined once
@@ -292,7 +413,10 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         kFirst = (u % splitK) * kLoop;
         partial = splitK > 1;
     }
-    MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, kFirst, kLoop, partial);
+    if constexpr (ROWS)
+        MixTileRows<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, kLoop); // the launcher rejects K-splits
+    else
+        MixTile<BM, BN, STAGES>(out, src0, src1, m, n, k, tm * BM, tn * BN, kFirst, kLoop, partial);
 }
 
 // Clears the C tiles that GemmF16F32Mix accumulates into with atomic adds (tile ids >= fullTiles).
@@ -311,7 +435,7 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE void GemmZeroTailTiles(__g
 #pragma unroll
         for (int nb = 0; nb < ResTile::Storage::NB; ++nb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i)
+            for (int i = 0; i < detail::kAccElems; ++i)
                 zero.st.f[mb][nb][i] = 0.0f;
     GlobalC dstGlobal(out + (int64_t)tm * BM * n + (int64_t)tn * BN, ShapeC(), StrideC(m, n));
     TSTORE(dstGlobal, zero);
@@ -376,14 +500,16 @@ inline int compute_units()
 // (the quarter tiles move twice the operand bytes per flop, so two rounds of them cost more than the
 // idle compute units of a partial round); 2 = K-split with atomic adds (tuning hook only); 3 = quarter
 // tiles whenever there is a partial round (tuning hook only)
-template <int BM, int BN, int STAGES, int GROUP_M>
+template <int BM, int BN, int STAGES, int GROUP_M, bool ROWS = false>
 int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k, int tailMode = 1)
 {
     static_assert(STAGES == 3 || STAGES == 4, "three or four L1 stages");
     if (m % BM || n % BN || k % (32 * STAGES) || k / 32 < 2 * STAGES)
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = STAGES * (BM * 32 + 32 * BN) * (int)sizeof(half);
-    auto kernel = GemmF16F32Mix<BM, BN, STAGES, GROUP_M>;
+    if (ROWS && tailMode == 2)
+        return PTO_ERR_UNSUPPORTED;
+    auto kernel = GemmF16F32Mix<BM, BN, STAGES, GROUP_M, ROWS>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;

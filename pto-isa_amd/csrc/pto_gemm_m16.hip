@@ -1,0 +1,32 @@
+// The 256 x 256 GEMM tile for workgroups of 8 wavefronts (wave grid 2 x 4) on v_mfma_f32_16x16x32_f16: same flops
+// per cycle as the 32 x 32 x 16 form, half the accumulator register traffic per flop, and a higher sustained clock
+// under the chip's power limit.
+#define PTO_WAVES_M 2
+#define PTO_WAVES_N 4
+#define PTO_MFMA_M 16
+#include "gemm_kernels.hpp"
+
+namespace pto_amd {
+// 256 x 256 C tiles, eight wavefronts per workgroup (128 x 64 of C per wave), 16 x 16 x 32 MFMAs: the default for
+// large problems.
+int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k)
+{
+    return launch_gemm_mix<256, 256, 4, 4, true>(st, c, a, b, m, n, k, 1);
+}
+} // namespace pto_amd
+
+extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
+                                           int variant)
+{
+    if (!c || !a || !b || m <= 0 || n <= 0 || k <= 0)
+        return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
+    switch (variant) {
+    case 0: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 1);
+    case 1: return launch_gemm_mix<256, 256, 3, 4, true>(st, c, ha, hb, m, n, k, 1);
+    case 2: return launch_gemm_mix<256, 256, 4, 8, true>(st, c, ha, hb, m, n, k, 1);
+    case 3: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
+    default: return PTO_ERR_BAD_ARG;
+    }
+}

@@ -5,11 +5,6 @@
 #include "gemm_kernels.hpp"
 
 namespace pto_amd {
-// 256 x 256 C tiles, eight wavefronts per workgroup (128 x 64 of C per wave): the default for large problems.
-int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k)
-{
-    return launch_gemm_mix<256, 256, 4, 4>(st, c, a, b, m, n, k, 1);
-}
 int gemm_compute_units() { return compute_units(); }
 } // namespace pto_amd
 
@@ -30,6 +25,7 @@ extern "C" int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t
     case 30: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 1);
     case 31: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 1);
     case 32: return launch_gemm_mix<256, 256, 3, 4>(st, c, ha, hb, m, n, k, 1);
+    case 50: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 1);
     default: return PTO_ERR_BAD_ARG;
     }
 }
