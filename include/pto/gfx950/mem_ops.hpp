@@ -8,9 +8,10 @@
 // Mat tile LDS image.  Let `major` index the non-contiguous logical dimension and k the
 // contiguous one (k = column for an Nz tile, row for a Zn tile), RowBytes = extent_k * sizeof(T).
 // Element (major, k) lives at   major*RowBytes + ((chunk ^ swz(major)) << 4) + (k*sizeof(T) & 15),
-// chunk = k*sizeof(T) >> 4.  swz() is chosen so that 16 consecutive `major` values at the same
-// logical chunk fall into 16 different 16-byte bank groups: ds_read_b128 by a half-wave is
-// conflict free, and so is the 1 KiB-contiguous write pattern of global_load_lds_dwordx4.
+// chunk = k*sizeof(T) >> 4.  swz() spreads consecutive `major` values at the same logical chunk over the
+// 16-byte bank groups so that the ds_read_b128 fragment reads are conflict free (checked with the LDS
+// bank-conflict counter and with read-rate probes), and the 1 KiB-contiguous write pattern of
+// global_load_lds_dwordx4 is conflict free by construction.
 #pragma once
 #include "pto/common/global_tensor.hpp"
 #include "pto/common/tile.hpp"
@@ -27,7 +28,10 @@ PTO_DEV constexpr uint32_t mat_swz(uint32_t major)
     if constexpr (!is_pow2(cpr) || cpr < 2) {
         return 0;
     } else {
-        constexpr int div = cpr >= 16 ? 1 : 16 / cpr;
+        // rows per swizzle step.  64-byte rows: 2 (measured conflict-free for ds_read_b128 fragment reads of both
+        // MFMA shapes: lanes read 32 rows x 1 chunk or 16 rows x 1 chunk per half / quarter wave; a step of 4 rows
+        // costs 7 % of the LDS read rate with 16-row blocks)
+        constexpr int div = cpr >= 16 ? 1 : (cpr == 4 ? 2 : 16 / cpr);
         constexpr int mod = cpr >= 16 ? 16 : cpr;
         return (major / div) % mod;
     }
