@@ -152,7 +152,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
         constexpr int cpr = Geo::ChunksPerRow;
         // rows that one wave instruction covers, when a row is at most one instruction long
         constexpr int rpi = (cpr <= kWaveSize && kWaveSize % cpr == 0) ? kWaveSize / cpr : 0;
-        if constexpr (rpi > 0 && (rpi * kBlockWaves) % 16 == 0 && nInst % kBlockWaves == 0 && total % perWaveInst == 0) {
+        if constexpr (rpi > 0 && (rpi * kBlockWaves) % 16 == 0 && total % perWaveInst == 0 && (nInst % kBlockWaves == 0 || SLICE < 0)) {
             // The swizzle repeats every 16 rows and the instructions of one wave are a multiple of 16
             // rows apart: every instruction of this wave uses the same per-lane byte offset (32 bits: a
             // tile spans less than 4 GiB of memory) on top of a wave-uniform base, which the loop
@@ -163,10 +163,15 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             const char *base = reinterpret_cast<const char *>(gm);
             constexpr int first = SLICE < 0 ? 0 : SLICE * kBlockWaves, last = SLICE < 0 ? nInst : first + kBlockWaves;
             static_assert(last <= nInst, "[PTO][SA] TLOAD slice: the tile has fewer copy instructions");
+            static_assert(nInst % kBlockWaves == 0 || nInst > kBlockWaves, "[PTO][SA] TLOAD: fewer copy instructions than waves");
 #pragma unroll
             for (int s0 = first; s0 < last; s0 += kBlockWaves) {
-                const char *g = uniform_ptr(base + (int64_t)(s0 * rpi) * ld * (int64_t)sizeof(T)) + laneOff;
-                __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + (s0 + wave) * (perWaveInst * 16)), 16, 0, 0);
+                // When the last round of instructions is not full, the waves past its end repeat their instruction
+                // of the round before (same data to the same place): every wave then issues TLoadInstrs<TileT>()
+                // copies, which keeps the vmcnt bookkeeping of software pipelines uniform and the code branch-free.
+                const int s0e = (nInst % kBlockWaves != 0 && s0 + wave >= nInst) ? s0 - kBlockWaves : s0;
+                const char *g = uniform_ptr(base + (int64_t)(s0e * rpi) * ld * (int64_t)sizeof(T)) + laneOff;
+                __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + (s0e + wave) * (perWaveInst * 16)), 16, 0, 0);
             }
         } else {
             static_assert(SLICE < 0, "[PTO][SA] TLOAD slice: this tile geometry has no per-wave slices");
@@ -275,7 +280,6 @@ constexpr int TLoadInstrs()
     using Geo = detail::MatGeom<TileT>;
     return detail::cdiv(detail::cdiv(Geo::Major * Geo::ChunksPerRow, kWaveSize), kBlockWaves);
 }
-
 template <typename TileT, typename G>
 PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 {

@@ -393,7 +393,9 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
         TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
         const int sub = u % 4;
-        if constexpr (ROWS)
+        if constexpr (ROWS && (BN / 2) % (detail::kMfmaM * kWavesN) != 0)
+            ; // this tile shape has no quarter tiles: the launcher never asks for them
+        else if constexpr (ROWS)
             MixTileRows<BM / 2, BN / 2, STAGES>(out, src0, src1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
                                                 tn * BN + (sub & 1) * (BN / 2), k / 32);
         else
@@ -509,6 +511,8 @@ int launch_gemm_mix(hipStream_t st, float *c, const half *a, const half *b, int 
     constexpr int lds = STAGES * (BM * 32 + 32 * BN) * (int)sizeof(half);
     if (ROWS && tailMode == 2)
         return PTO_ERR_UNSUPPORTED;
+    if (ROWS && (BN / 2) % (detail::kMfmaM * kWavesN) != 0) // no quarter tiles for this shape
+        tailMode = 0;
     auto kernel = GemmF16F32Mix<BM, BN, STAGES, GROUP_M, ROWS>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)

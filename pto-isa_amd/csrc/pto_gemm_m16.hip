@@ -11,6 +11,12 @@ namespace pto_amd {
 // large problems.
 int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k)
 {
+    // A problem whose 256 x 256 tiles do not even fill one round: 256 x 192 tiles put more compute units to work
+    // (3072^3: 192 instead of 144 workgroups, measured +12 %).  With several rounds the square tile wins (less operand
+    // traffic per flop) even where the narrower one would divide the rounds evenly (6144^3: -4 %, 7680^3: -9 %).
+    const int cus = compute_units();
+    if (n % 192 == 0 && (m / 256) * (n / 256) < cus && (m / 256) * (n / 192) <= cus)
+        return launch_gemm_mix<256, 192, 4, 4, true>(st, c, a, b, m, n, k, 0);
     return launch_gemm_mix<256, 256, 4, 4, true>(st, c, a, b, m, n, k, 1);
 }
 } // namespace pto_amd
@@ -27,6 +33,8 @@ extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_
     case 1: return launch_gemm_mix<256, 256, 3, 4, true>(st, c, ha, hb, m, n, k, 1);
     case 2: return launch_gemm_mix<256, 256, 4, 8, true>(st, c, ha, hb, m, n, k, 1);
     case 3: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
+    case 10: return launch_gemm_mix<256, 192, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
+    case 11: return launch_gemm_mix<256, 192, 4, 8, true>(st, c, ha, hb, m, n, k, 0);
     default: return PTO_ERR_BAD_ARG;
     }
 }
