@@ -13,6 +13,16 @@ namespace {
 
 constexpr int kXcds = 8; // MI355X: 8 accelerator dies, workgroups are dealt to them round-robin
 
+// compile-time loop: f(integral_constant<int, I>) for I = FIRST .. LAST-1
+template <int FIRST, int LAST, typename F>
+AICORE inline void StaticFor(F &&f)
+{
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>());
+        StaticFor<FIRST + 1, LAST>(f);
+    }
+}
+
 // Workgroup id -> C tile.  Consecutive ids land on different XCDs, each with its own L2, so first
 // regroup ids per XCD, then walk the tile grid in bands of GROUP_M tile rows so that the tiles
 // running together on one XCD share A and B panels.
@@ -288,8 +298,15 @@ AICORE inline __attribute__((always_inline)) void MixTileRows(__gm__ float *out,
     constexpr int kLoadsPerStep = TLoadInstrs<TileMatA>() + TLoadInstrs<TileMatB>();
     constexpr int kMfmaPerHalf = AccHalf::Storage::MB * AccHalf::Storage::NB * LeftHalf::Storage::KS;
     constexpr int kReadsA = LeftHalf::Storage::MB * LeftHalf::Storage::KS, kReadsB = RightTile::Storage::NB * RightTile::Storage::KS;
-    static_assert(STAGES >= 3, "needs at least three L1 stages");
-    static_assert(kMfmaPerHalf % kLoadsPerStep == 0 && kMfmaPerHalf >= kReadsA, "issue pattern below");
+    constexpr int kReads = 2 * kReadsA + kReadsB, kMfma = 2 * kMfmaPerHalf;
+    // Issue pattern of a step: the copies first, kMfmaPerCopy MFMAs before each (the LDS reads may not be moved above
+    // an asynchronous copy into LDS); then the fragment reads spread over the MFMAs that follow; the last kMfmaTail
+    // MFMAs of the step have no read after them.
+    constexpr int kMfmaPerCopy = kMfma / 4 / kLoadsPerStep > 0 ? kMfma / 4 / kLoadsPerStep : 1;
+    constexpr int kMfmaTail = kMfma / 8 > 0 ? kMfma / 8 : 1;
+    constexpr int kMfmaForReads = kMfma - kMfmaPerCopy * kLoadsPerStep - kMfmaTail;
+    static_assert(STAGES == 4, "two fragment sets alternate with the stage index");
+    static_assert(kMfmaForReads > 0, "issue pattern below");
 
     __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)row0 * k;
     __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)col0 * k;
@@ -303,8 +320,11 @@ AICORE inline __attribute__((always_inline)) void MixTileRows(__gm__ float *out,
         TASSIGN(aMat[s], s * kStage);
         TASSIGN(bMat[s], s * kStage + kABytes);
     }
-    LeftHalf aUp, aDn;
-    RightTile bAll;
+    // Two sets of operand fragments: the MFMAs of step it read set it % 2 while the fragments of step it+1 arrive in the
+    // other one, every read interleaved with the MFMAs and none left for the end of the step - the wait for the LDS
+    // queue that follows the barrier then finds it empty.
+    LeftHalf aUp[2], aDn[2];
+    RightTile bAll[2];
     AccHalf cUp, cDn;
 #pragma unroll
     for (int mb = 0; mb < AccHalf::Storage::MB; ++mb)
@@ -325,9 +345,9 @@ AICORE inline __attribute__((always_inline)) void MixTileRows(__gm__ float *out,
         TLOAD(bMat[s], gmB);
     }
     wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // stage 0 is complete
-    TEXTRACT(aUp, aMat[0], 0, 0);
-    TEXTRACT(aDn, aMat[0], HM, 0);
-    TEXTRACT(bAll, bMat[0], 0, 0);
+    TEXTRACT(aUp[0], aMat[0], 0, 0);
+    TEXTRACT(aDn[0], aMat[0], HM, 0);
+    TEXTRACT(bAll[0], bMat[0], 0, 0);
 
     auto step = [&](auto stageTag, int it) {
         constexpr int s = decltype(stageTag)::value;
@@ -340,24 +360,26 @@ AICORE inline __attribute__((always_inline)) void MixTileRows(__gm__ float *out,
         GlobalB gmB(bPanel + (int64_t)fetch * BK, ShapeB(), strideB);
         TLOAD(aMat[sLoad], gmA);
         TLOAD(bMat[sLoad], gmB);
-        TMATMUL_ACC(cUp, cUp, aUp, bAll);
-        TEXTRACT(aUp, aMat[sNext], 0, 0);
-        TMATMUL_ACC(cDn, cDn, aDn, bAll);
-        TEXTRACT(aDn, aMat[sNext], HM, 0);
-        TEXTRACT(bAll, bMat[sNext], 0, 0);
-        // issue order: MFMAs of the upper half with the copies between them, then the fragment reads for the
-        // next step's upper half one per MFMA of the lower half, then the remaining reads
+        constexpr int p = s & 1, q = p ^ 1;
+        TMATMUL_ACC(cUp, cUp, aUp[p], bAll[p]);
+        TMATMUL_ACC(cDn, cDn, aDn[p], bAll[p]);
+        TEXTRACT(aUp[q], aMat[sNext], 0, 0);
+        TEXTRACT(bAll[q], bMat[sNext], 0, 0);
+        TEXTRACT(aDn[q], aMat[sNext], HM, 0);
 #pragma unroll
         for (int i = 0; i < kLoadsPerStep; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerHalf / kLoadsPerStep, 0);
+            __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerCopy, 0);
             __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
         }
-#pragma unroll
-        for (int i = 0; i < kReadsA; ++i) {
+        StaticFor<0, kReads>([](auto iTag) {
+            // read i follows its share of the MFMAs: floor((i+1) N / R) - floor(i N / R)
+            constexpr int i = decltype(iTag)::value;
+            constexpr int n = (i + 1) * kMfmaForReads / kReads - i * kMfmaForReads / kReads;
+            if constexpr (n > 0)
+                __builtin_amdgcn_sched_group_barrier(0x008, n, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerHalf / kReadsA, 0);
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, kReadsA + kReadsB, 0);
+        });
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaTail, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
     using std::integral_constant;

@@ -30,7 +30,6 @@ extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_
     const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
     switch (variant) {
     case 0: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 1);
-    case 1: return launch_gemm_mix<256, 256, 3, 4, true>(st, c, ha, hb, m, n, k, 1);
     case 2: return launch_gemm_mix<256, 256, 4, 8, true>(st, c, ha, hb, m, n, k, 1);
     case 3: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
     case 10: return launch_gemm_mix<256, 192, 4, 4, true>(st, c, ha, hb, m, n, k, 0);

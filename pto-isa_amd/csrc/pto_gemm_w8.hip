@@ -25,7 +25,6 @@ extern "C" int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t
     case 30: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 1);
     case 31: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 1);
     case 32: return launch_gemm_mix<256, 256, 3, 4>(st, c, ha, hb, m, n, k, 1);
-    case 50: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 1);
     default: return PTO_ERR_BAD_ARG;
     }
 }
