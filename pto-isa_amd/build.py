@@ -45,13 +45,15 @@ def build(verbose=True):
 
 
 def build_host(verbose=True):
-    """The `call_kernel` libraries of the two demos and the GEMM host program; plain host C++ on top of libpto_amd.so."""
+    """The `call_kernel` libraries of the two demos and the GEMM and flash-attention host programs; plain host C++ on top of libpto_amd.so."""
     inc = ["-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__"]
     link = ["-L" + HERE, "-lpto_amd", "-Wl,-rpath,$ORIGIN"]
     jobs = [
         (["-shared", "-fPIC", os.path.join(CSRC, "call_kernel_gemm.cpp")], os.path.join(HERE, "libpto_call_gemm.so"), link),
         (["-shared", "-fPIC", os.path.join(CSRC, "call_kernel_fa.cpp")], os.path.join(HERE, "libpto_call_fa.so"), link),
         ([os.path.join(HERE, "host", "gemm_main.cpp")], os.path.join(HERE, "host", "gemm_main"),
+         ["-L" + HERE, "-lpto_amd", "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"]),
+        ([os.path.join(HERE, "host", "fa_main.cpp")], os.path.join(HERE, "host", "fa_main"),
          ["-L" + HERE, "-lpto_amd", "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"]),
     ]
     for srcs, out, libs in jobs:

@@ -53,6 +53,43 @@ def test_gemm_main_reports_failure_on_wrong_golden(tmp_path):
     assert "test failed" in r.stdout and r.returncode == 1
 
 
+def test_gen_data_fa_file_protocol(tmp_path):
+    """Files and golden of the flash-attention host program: the streamed recipe equals a dense fp64 softmax up to the
+    fp16 rounding of the probabilities."""
+    subprocess.run([sys.executable, os.path.join(PKG, "host", "gen_data_fa.py"), str(tmp_path), "128", "128", "512"], check=True)
+    q = np.fromfile(tmp_path / "q.bin", dtype=np.float16).reshape(128, 128)
+    kt = np.fromfile(tmp_path / "kt.bin", dtype=np.float16).reshape(512, 128)                   # stored [s1, head]
+    v = np.fromfile(tmp_path / "v.bin", dtype=np.float16).reshape(512, 128)
+    o = np.fromfile(tmp_path / "o.bin", dtype=np.float32).reshape(128, 128)
+    s = q.astype(np.float64) @ kt.astype(np.float64).T / np.sqrt(128.0)
+    p = np.exp(s - s.max(axis=1, keepdims=True))
+    want = (p / p.sum(axis=1, keepdims=True)) @ v.astype(np.float64)
+    assert np.max(np.abs(o - want)) / np.max(np.abs(want)) < 2e-3
+    assert os.access(os.path.join(PKG, "host", "fa_main"), os.X_OK)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("head,s0,s1,causal", [(128, 128, 1024, 0), (128, 512, 512, 1), (64, 256, 768, 0)])
+def test_fa_main_runs_the_file_protocol(tmp_path, head, s0, s1, causal):
+    subprocess.run([sys.executable, os.path.join(PKG, "host", "gen_data_fa.py"), str(tmp_path), str(head), str(s0), str(s1), str(causal)],
+                   check=True)
+    r = subprocess.run([os.path.join(PKG, "host", "fa_main"), str(tmp_path), str(head), str(s0), str(s1), str(causal)],
+                       capture_output=True, text=True, timeout=120)
+    assert "test success" in r.stdout, r.stdout + r.stderr
+    out = np.fromfile(tmp_path / "o_out.bin", dtype=np.float32)
+    gold = np.fromfile(tmp_path / "o.bin", dtype=np.float32)
+    assert np.max(np.abs(out - gold)) / np.max(np.abs(gold)) < 2e-3
+
+
+@pytest.mark.gpu
+def test_fa_main_reports_failure_on_wrong_golden(tmp_path):
+    subprocess.run([sys.executable, os.path.join(PKG, "host", "gen_data_fa.py"), str(tmp_path), "128", "128", "256"], check=True)
+    g = np.fromfile(tmp_path / "o.bin", dtype=np.float32)
+    (g + 10.0).astype(np.float32).tofile(tmp_path / "o.bin")
+    r = subprocess.run([os.path.join(PKG, "host", "fa_main"), str(tmp_path), "128", "128", "256"], capture_output=True, text=True, timeout=120)
+    assert "test failed" in r.stdout and r.returncode == 1
+
+
 @pytest.mark.gpu
 def test_call_kernel_gemm_6144(oracle):
     import torch
