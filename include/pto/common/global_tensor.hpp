@@ -85,6 +85,16 @@ struct BaseShape2D<T, rows, cols, Layout::DN>
     PTO_HD constexpr BaseShape2D(int64_t r, int64_t c) : Parent(r * c, r * c, r * c, 1, r) {}
 };
 
+// block-scale matrices of MX operands (pto_tile.hpp:651-680, 776-805): dense, the k-block index contiguous
+template <typename T, int64_t rows, int64_t cols>
+struct BaseShape2D<T, rows, cols, Layout::MX_A_ND> : BaseShape2D<T, rows, cols, Layout::ND> {
+    using BaseShape2D<T, rows, cols, Layout::ND>::BaseShape2D;
+};
+template <typename T, int64_t rows, int64_t cols>
+struct BaseShape2D<T, rows, cols, Layout::MX_B_DN> : BaseShape2D<T, rows, cols, Layout::DN> {
+    using BaseShape2D<T, rows, cols, Layout::DN>::BaseShape2D;
+};
+
 template <typename Element_, typename Shape_, typename Stride_, Layout Layout_ = Layout::ND>
 struct GlobalTensor {
     using Shape = Shape_;

@@ -186,6 +186,22 @@ PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TMATMUL_ACC(C &
     TMATMUL_ACC_IMPL(c, c, a, b);
     return {};
 }
+// TMATMUL_MX(c, a, aScale, b, bScale) and the accumulating form (cOut, cIn, a, aScale, b, bScale)  (pto_instr.hpp:403-440)
+template <typename C, typename A, typename AS, typename B, typename BS, typename... Ev>
+PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TMATMUL_MX(C &c, A &a, AS &aScale, B &b, BS &bScale, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_MX_IMPL(c, a, aScale, b, bScale);
+    return {};
+}
+template <typename C, typename A, typename AS, typename B, typename BS, typename... Ev>
+PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TMATMUL_MX(C &cOut, C &cIn, A &a, AS &aScale, B &b, BS &bScale,
+                                                                             Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_MX_IMPL(cOut, cIn, a, aScale, b, bScale);
+    return {};
+}
 template <typename D, typename S, typename... Ev>
 PTO_INST RecordEvent TCVT(D &dst, S &src, RoundMode mode, SaturationMode sat, Ev &... ev)
 {

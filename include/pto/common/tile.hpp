@@ -27,6 +27,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
 
 namespace detail {
 
@@ -71,6 +72,54 @@ struct TileStorage { // Bias / Scaling / unsupported locations: no storage
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Mat, T, Rows, Cols> {
     uint32_t lds = 0; // byte offset into the workgroup's dynamic LDS
+};
+
+// 8-bit MX operands (v_mfma_scale_f32_32x32x64_f8f6f4): a fragment is 32 rows x 64 k; lane l holds row l % 32 and the
+// bytes k = 16 (l / 32) .. +15 (first four registers) and k = 32 + 16 (l / 32) .. +15 (last four).
+template <typename T>
+constexpr bool is_mx8_v = std::is_same_v<T, float8_e4m3_t> || std::is_same_v<T, float8_e5m2_t>;
+constexpr int kMxM = 32, kMxK = 64, kMxBlock = 32;
+
+template <int Rows, int Cols>
+struct TileStorage<TileType::Left, float8_e4m3_t, Rows, Cols> {
+    static_assert(kMfmaM == kMxM, "MX operand tiles need PTO_MFMA_M 32 (accumulator layout of the 32 x 32 MFMA)");
+    static_assert(Rows % (kMxM * kWavesM) == 0 && Cols % kMxK == 0, "MX Left tile: multiples of 32 x PTO_WAVES_M rows, 64 columns");
+    static constexpr int MB = Rows / (kMxM * kWavesM), Blocks = MB;
+    static constexpr int KS = Cols / kMxK;
+    i32x8 f[MB][KS];
+};
+template <int Rows, int Cols>
+struct TileStorage<TileType::Left, float8_e5m2_t, Rows, Cols> : TileStorage<TileType::Left, float8_e4m3_t, Rows, Cols> {};
+template <int Rows, int Cols>
+struct TileStorage<TileType::Right, float8_e4m3_t, Rows, Cols> {
+    static_assert(kMfmaM == kMxM, "MX operand tiles need PTO_MFMA_M 32 (accumulator layout of the 32 x 32 MFMA)");
+    static_assert(Cols % (kMxM * kWavesN) == 0 && Rows % kMxK == 0, "MX Right tile: multiples of 32 x PTO_WAVES_N columns, 64 rows");
+    static constexpr int NB = Cols / (kMxM * kWavesN), Blocks = NB;
+    static constexpr int KS = Rows / kMxK;
+    i32x8 f[NB][KS];
+};
+template <int Rows, int Cols>
+struct TileStorage<TileType::Right, float8_e5m2_t, Rows, Cols> : TileStorage<TileType::Right, float8_e4m3_t, Rows, Cols> {};
+
+// Block scales of an MX operand tile: one e8m0 value per row (column) and 32-wide k block, KB blocks per row.
+// Per 32-row block of its part of the operand a wave holds the scales of the lane's row, four k blocks to a
+// register, each register shifted right by 8 bits in lanes 32-63: the MFMA of 64-wide k step s takes the scale of
+// k block 2 s (lanes 0-31) / 2 s + 1 (lanes 32-63), which then is byte 0 (s even) or byte 2 (s odd) of register s / 2.
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::ScaleLeft, T, Rows, Cols> {
+    static_assert(sizeof(T) == 1 && Cols % 2 == 0 && (Cols == 2 || Cols % 4 == 0) && Rows % (kMxM * kWavesM) == 0,
+                  "scale tile: 2 or a multiple of 4 k blocks per row");
+    static constexpr int MB = Rows / (kMxM * kWavesM), Blocks = MB;
+    static constexpr int KB = Cols, Regs = (Cols + 3) / 4;
+    uint32_t s[MB][Regs];
+};
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::ScaleRight, T, Rows, Cols> {
+    static_assert(sizeof(T) == 1 && Rows % 2 == 0 && (Rows == 2 || Rows % 4 == 0) && Cols % (kMxM * kWavesN) == 0,
+                  "scale tile: 2 or a multiple of 4 k blocks per column");
+    static constexpr int NB = Cols / (kMxM * kWavesN), Blocks = NB;
+    static constexpr int KB = Rows, Regs = (Rows + 3) / 4;
+    uint32_t s[NB][Regs];
 };
 
 template <typename T, int Rows, int Cols>
@@ -150,8 +199,10 @@ struct Tile {
     static_assert(Loc_ == TileType::Vec || Rows_ == 1 || Rows % InnerRows == 0,
                   "[PTO][SA] tile rows must be a multiple of the inner box rows");
     static_assert(Cols % InnerCols == 0, "[PTO][SA] tile cols must be a multiple of the inner box cols");
-    static_assert(isBoxedLayout || (isRowMajor ? (Cols * sizeof(DType)) % TileConfig::alignedSize == 0 :
-                                                 (Rows * sizeof(DType)) % TileConfig::alignedSize == 0),
+    // (scale tiles are register tiles of a few bytes per row; a Mat tile of 1-byte block scales has 16-byte rows)
+    static_assert(isBoxedLayout || Loc_ == TileType::ScaleLeft || Loc_ == TileType::ScaleRight ||
+                      (isRowMajor ? (Cols * sizeof(DType)) : (Rows * sizeof(DType))) %
+                              (Loc_ == TileType::Mat && sizeof(DType) == 1 ? 16 : TileConfig::alignedSize) == 0,
                   "[PTO][SA] unboxed tiles need a 32-byte aligned contiguous extent");
 
     // The logical dimension that is contiguous in a Mat tile's LDS image: columns unless the tile
@@ -201,6 +252,11 @@ using TileRightCompact = Tile<TileType::Right, E, R, C, BLayout::RowMajor, RV, C
                               TileConfig::fractalABSize, PadValue::Null, CompactMode::Normal>;
 template <typename E, int R, int C, int RV = R, int CV = C>
 using TileAcc = Tile<TileType::Acc, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor, TileConfig::fractalCSize>;
+// block scales of MX operands (pto_tile.hpp:1441-1456): [rows, k / 32] for the left operand, [k / 32, cols] for the right
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileLeftScale = Tile<TileType::ScaleLeft, E, R, C, BLayout::RowMajor, RV, CV, SLayout::NoneBox>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileRightScale = Tile<TileType::ScaleRight, E, R, C, BLayout::ColMajor, RV, CV, SLayout::NoneBox>;
 template <typename E, int R, int C, int RV = R, int CV = C>
 using TileAccCompact = Tile<TileType::Acc, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor,
                             TileConfig::fractalCSize, PadValue::Null, CompactMode::Normal>;

@@ -12,6 +12,10 @@ namespace pto {
 using half = _Float16;
 using aclFloat16 = _Float16;
 using bfloat16_t = __bf16;
+// 8-bit storage types of the MX formats (element types of `TMATMUL_MX` operands and their block scales)
+struct float8_e4m3_t { uint8_t bits; };
+struct float8_e5m2_t { uint8_t bits; };
+struct float8_e8m0_t { uint8_t bits; }; // a power of two: 2^(bits - 127)
 
 constexpr int DYNAMIC = -1;
 
@@ -19,7 +23,9 @@ enum class TileType { Vec, Mat, Left, Right, Acc, Bias, Scaling, ScaleLeft, Scal
 enum class BLayout { RowMajor = 0, ColMajor = 1 };
 enum class SLayout { NoneBox = 0, RowMajor = 1, ColMajor = 2 };
 
-enum class Layout { ND, DN, NZ };
+// MX_A_ND / MX_B_DN: block scales of an MX matmul in memory, [rows, k / 32] row-major for the left operand and
+// [k / 32, cols] column-major for the right one (type.hpp:114-119)
+enum class Layout { ND, DN, NZ, MX_A_ND, MX_B_DN };
 
 enum class MaskPattern : uint8_t { P0101 = 1, P1010 = 2, P0001 = 3, P0010 = 4, P0100 = 5, P1000 = 6, P1111 = 7 };
 enum class CmpMode : uint8_t { EQ = 0, NE = 1, LT = 2, LE = 3, GT = 4, GE = 5 };

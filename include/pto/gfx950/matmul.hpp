@@ -90,6 +90,68 @@ PTO_DEV void TMATMUL_ACC_IMPL(AccT &cOut, AccT &cIn, LeftT &a, RightT &b)
     detail::mad<false>(cOut, cIn, a, b);
 }
 
+// TMATMUL_MX: C (+)= (A * scaleA) x (B * scaleB) on 8-bit MX operands, one e8m0 scale per row (column) and 32-wide
+// k block (reference semantics: the data generators of tests/npu/a5/src/st/testcase/tmatmul_mx and
+// kernels/manual/a5/matmul_mxfp8_performance/scripts/gen_data.py:24-50: operand element x 2^(scale - 127), products
+// accumulated in fp32).  v_mfma_scale_f32_32x32x64_f8f6f4 applies the scales inside the MFMA.
+namespace detail {
+template <typename T>
+constexpr int mx_format = std::is_same_v<T, float8_e5m2_t> ? 1 : 0; // the MFMA's cbsz / blgp operand-format code
+
+template <bool kZeroInit, typename AccT, typename LeftT, typename LeftScaleT, typename RightT, typename RightScaleT>
+PTO_DEV void mad_mx(AccT &out, const AccT &in, const LeftT &a, const LeftScaleT &sa, const RightT &b, const RightScaleT &sb)
+{
+    static_assert(is_mx8_v<typename LeftT::DType> && is_mx8_v<typename RightT::DType> && std::is_same_v<typename AccT::DType, float>,
+                  "[PTO][SA] TMATMUL_MX on gfx950: fp8 (e4m3 / e5m2) operands, fp32 accumulator");
+    static_assert(LeftT::Loc == TileType::Left && RightT::Loc == TileType::Right && AccT::Loc == TileType::Acc &&
+                      LeftScaleT::Loc == TileType::ScaleLeft && RightScaleT::Loc == TileType::ScaleRight,
+                  "[PTO][SA] TMATMUL_MX: operands must be Left, ScaleLeft, Right, ScaleRight and Acc tiles");
+    static_assert(LeftT::Rows == AccT::Rows && LeftT::Cols == RightT::Rows && RightT::Cols == AccT::Cols,
+                  "[PTO][SA] TMATMUL_MX: inconsistent m, k, n");
+    static_assert(LeftScaleT::Rows == LeftT::Rows && LeftScaleT::Cols * kMxBlock == LeftT::Cols &&
+                      RightScaleT::Cols == RightT::Cols && RightScaleT::Rows * kMxBlock == RightT::Rows,
+                  "[PTO][SA] TMATMUL_MX: one scale per row (column) and 32 k values");
+    using SA = typename AccT::Storage;
+    using SL = typename LeftT::Storage;
+    constexpr int fa = mx_format<typename LeftT::DType>, fb = mx_format<typename RightT::DType>;
+#pragma unroll
+    for (int mb = 0; mb < SA::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < SA::NB; ++nb) {
+            AccFrag c;
+            if constexpr (kZeroInit) {
+#pragma unroll
+                for (int i = 0; i < kAccElems; ++i)
+                    c[i] = 0.0f;
+            } else {
+                c = in.st.f[mb][nb];
+            }
+#pragma unroll
+            for (int ks = 0; ks < SL::KS; ++ks) {
+                // k step ks: scale byte 0 (even step) or 2 (odd step) of register ks / 2
+                if (ks % 2 == 0)
+                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a.st.f[mb][ks], b.st.f[nb][ks], c, fa, fb, 0,
+                                                                        (int)sa.st.s[mb][ks / 2], 0, (int)sb.st.s[nb][ks / 2]);
+                else
+                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a.st.f[mb][ks], b.st.f[nb][ks], c, fa, fb, 2,
+                                                                        (int)sa.st.s[mb][ks / 2], 2, (int)sb.st.s[nb][ks / 2]);
+            }
+            out.st.f[mb][nb] = c;
+        }
+}
+} // namespace detail
+
+template <typename AccT, typename LeftT, typename LeftScaleT, typename RightT, typename RightScaleT>
+PTO_DEV void TMATMUL_MX_IMPL(AccT &c, LeftT &a, LeftScaleT &sa, RightT &b, RightScaleT &sb)
+{
+    detail::mad_mx<true>(c, c, a, sa, b, sb);
+}
+template <typename AccT, typename LeftT, typename LeftScaleT, typename RightT, typename RightScaleT>
+PTO_DEV void TMATMUL_MX_IMPL(AccT &cOut, AccT &cIn, LeftT &a, LeftScaleT &sa, RightT &b, RightScaleT &sb)
+{
+    detail::mad_mx<false>(cOut, cIn, a, sa, b, sb);
+}
+
 // bias: a 1 x N fp32 row held as a Vec-distributed tile is not addressable per column from a
 // wave's accumulator lanes, so the bias row is read from memory: BiasT must expose `const float *row`.
 struct BiasRow {

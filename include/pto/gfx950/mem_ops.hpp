@@ -280,6 +280,44 @@ constexpr int TLoadInstrs()
     using Geo = detail::MatGeom<TileT>;
     return detail::cdiv(detail::cdiv(Geo::Major * Geo::ChunksPerRow, kWaveSize), kBlockWaves);
 }
+namespace detail {
+// GM -> block-scale register tile (the reference stages scales in L1 and TEXTRACTs them; a scale tile here is a few
+// registers per lane, so it is loaded straight from memory: one 4-byte load per four k blocks and 32-row block).
+// The k-block index must be the unit-stride dimension and the tile's first k block 4-byte aligned in memory.
+template <typename TileT, typename G>
+PTO_DEV void tload_scale(TileT &dst, G &src)
+{
+    using S = typename TileT::Storage;
+    constexpr bool left = TileT::Loc == TileType::ScaleLeft;
+    static_assert(left ? G::staticStride[4] == 1 : G::staticStride[3] == 1, "[PTO][SA] TLOAD of a scale tile: k blocks must be contiguous");
+    const char *gm = reinterpret_cast<const char *>(src.data());
+    const int64_t ld = left ? src.GetStride(3) : src.GetStride(4);
+    const uint32_t lane = (uint32_t)hw::lane();
+    const uint32_t shift = (lane / kMxM) * 8;
+    constexpr int blocks = S::Blocks;
+    const uint32_t major0 = (uint32_t)(left ? hw::wave_m() : hw::wave_n()) * (blocks * kMxM) + lane % kMxM;
+#pragma unroll
+    for (int b = 0; b < blocks; ++b) {
+        const char *p = gm + (int64_t)(major0 + b * kMxM) * ld;
+        if constexpr (S::KB == 2) {
+            dst.st.s[b][0] = (uint32_t)*reinterpret_cast<const uint16_t *>(p) >> shift;
+        } else if constexpr (S::Regs % 4 == 0) {
+#pragma unroll
+            for (int r = 0; r < S::Regs; r += 4) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(p + 4 * r);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    dst.st.s[b][r + i] = v[i] >> shift;
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < S::Regs; ++r)
+                dst.st.s[b][r] = *reinterpret_cast<const uint32_t *>(p + 4 * r) >> shift;
+        }
+    }
+}
+} // namespace detail
+
 template <typename TileT, typename G>
 PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 {
@@ -288,6 +326,8 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
         detail::tload_mat(dst, src);
     else if constexpr (TileT::Loc == TileType::Vec)
         detail::tload_vec(dst, src);
+    else if constexpr (TileT::Loc == TileType::ScaleLeft || TileT::Loc == TileType::ScaleRight)
+        detail::tload_scale(dst, src);
     else
         static_assert(TileT::Loc == TileType::Mat, "[PTO][SA] TLOAD: destination must be a Mat or Vec tile");
 }
@@ -296,8 +336,90 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 // dst[i,j] = src[idxRow+i, idxCol+j].  Mat -> Left / Right: one ds_read_b128 per row block and k step, in the
 // MFMA operand layout (lane l: row/col l % kMfmaM, k = 8*(l / kMfmaM)..+7).
 // The k offset must be a multiple of 8 elements (16 bytes).
+namespace detail {
+// Mat -> Left / Right of an 8-bit MX operand: two ds_read_b128 per 32-row block and 64-wide k step (lane l: row
+// l % 32, bytes 16 (l / 32) .. +15 and 32 + 16 (l / 32) .. +15 of the step).  The k offset must be a multiple of 64.
 template <typename DstT, typename SrcT>
-PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t idxCol = 0)
+PTO_DEV void textract_mx(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol)
+{
+    using Geo = MatGeom<SrcT>;
+    using S = typename DstT::Storage;
+    constexpr bool left = DstT::Loc == TileType::Left;
+    static_assert(left ? Geo::colsK : !Geo::colsK, "[PTO][SA] TEXTRACT: the source must be contiguous along k");
+    const char *lds = hw::lds_base() + src.st.lds;
+    const uint32_t lane = (uint32_t)hw::lane();
+    constexpr int blocks = S::Blocks;
+    const uint32_t major0 = (left ? idxRow : idxCol) + (uint32_t)(left ? hw::wave_m() : hw::wave_n()) * (blocks * kMxM) + lane % kMxM;
+    const uint32_t chunk0 = ((left ? idxCol : idxRow) >> 4) + lane / kMxM;
+#pragma unroll
+    for (int b = 0; b < blocks; ++b)
+#pragma unroll
+        for (int ks = 0; ks < S::KS; ++ks) {
+            const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4));
+            const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4 + 2));
+            dst.st.f[b][ks] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        }
+}
+
+// Mat tile of scales in LDS (one row of k-block scales per operand row / column, unboxed) -> scale register tile:
+// k blocks [kb, kb + dst.KB) of rows [idx, idx + extent); kb a multiple of 4 (of 2 for a tile of one k step: one
+// ds_read_u8 per 32-row block, lanes 32-63 read the step's second block)
+template <typename DstT, typename SrcT>
+PTO_DEV void textract_scale_mat(DstT &dst, SrcT &src, uint32_t idxMajor, uint32_t kb)
+{
+    using Geo = MatGeom<SrcT>;
+    using D = typename DstT::Storage;
+    constexpr bool left = DstT::Loc == TileType::ScaleLeft;
+    static_assert(sizeof(typename SrcT::DType) == 1 && !SrcT::isBoxedLayout && (left ? Geo::colsK : !Geo::colsK) && Geo::ChunksPerRow == 1,
+                  "[PTO][SA] TEXTRACT of scales: unboxed Mat tile, 16 k blocks per row, contiguous along k");
+    const char *lds = hw::lds_base() + src.st.lds;
+    const uint32_t lane = (uint32_t)hw::lane();
+    const uint32_t shift = (lane / kMxM) * 8;
+    constexpr int blocks = D::Blocks;
+    const uint32_t major0 = idxMajor + (uint32_t)(left ? hw::wave_m() : hw::wave_n()) * (blocks * kMxM) + lane % kMxM;
+#pragma unroll
+    for (int b = 0; b < blocks; ++b) {
+        const char *p = lds + (major0 + b * kMxM) * Geo::RowBytes + kb;
+        if constexpr (D::KB == 2) {
+            dst.st.s[b][0] = *reinterpret_cast<const uint8_t *>(p + lane / kMxM);
+        } else if constexpr (D::Regs == 4) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(p);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                dst.st.s[b][i] = v[i] >> shift;
+        } else {
+#pragma unroll
+            for (int r = 0; r < D::Regs; ++r)
+                dst.st.s[b][r] = *reinterpret_cast<const uint32_t *>(p + 4 * r) >> shift;
+        }
+    }
+}
+
+// scale tile -> scale tile window (registers only): k blocks [kb, kb + dst.KB) of the source; kb a multiple of 2,
+// and of 4 unless the destination holds a single k step (2 blocks)
+template <typename DstT, typename SrcT>
+PTO_DEV void textract_scale(DstT &dst, const SrcT &src, uint32_t kb)
+{
+    using D = typename DstT::Storage;
+    using S = typename SrcT::Storage;
+    constexpr bool left = DstT::Loc == TileType::ScaleLeft;
+    static_assert(left ? DstT::Rows == SrcT::Rows : DstT::Cols == SrcT::Cols, "[PTO][SA] TEXTRACT of scales: windows along k only");
+    constexpr int blocks = D::Blocks;
+#pragma unroll
+    for (int b = 0; b < blocks; ++b) {
+        if constexpr (D::KB == 2) {
+            dst.st.s[b][0] = src.st.s[b][kb / 4] >> ((kb % 4) * 8);
+        } else {
+#pragma unroll
+            for (int r = 0; r < D::Regs; ++r)
+                dst.st.s[b][r] = src.st.s[b][kb / 4 + r];
+        }
+    }
+}
+} // namespace detail
+
+template <typename DstT, typename SrcT>
+PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol)
 {
     static_assert(SrcT::Loc == TileType::Mat, "[PTO][SA] TEXTRACT: source must be a Mat tile");
     static_assert(sizeof(typename DstT::DType) == sizeof(typename SrcT::DType), "[PTO][SA] TEXTRACT: dtype mismatch");
@@ -331,6 +453,27 @@ PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t i
                     lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * kStepChunks));
     } else {
         static_assert(DstT::Loc == TileType::Left, "[PTO][SA] TEXTRACT: destination must be a Left or Right tile");
+    }
+}
+
+template <typename DstT, typename SrcT>
+PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t idxCol = 0)
+{
+    if constexpr (DstT::Loc == TileType::ScaleLeft || DstT::Loc == TileType::ScaleRight) {
+        constexpr bool left = DstT::Loc == TileType::ScaleLeft;
+        if constexpr (SrcT::Loc == TileType::Mat) {
+            detail::textract_scale_mat(dst, src, left ? idxRow : idxCol, left ? idxCol : idxRow);
+        } else {
+            static_assert(SrcT::Loc == DstT::Loc, "[PTO][SA] TEXTRACT of scales: from a Mat tile or a scale tile of the same kind");
+            detail::textract_scale(dst, src, left ? idxCol : idxRow);
+        }
+        return;
+    } else if constexpr (detail::is_mx8_v<typename DstT::DType>) {
+        static_assert(SrcT::Loc == TileType::Mat && sizeof(typename SrcT::DType) == 1, "[PTO][SA] TEXTRACT: 8-bit Mat source");
+        detail::textract_mx(dst, src, idxRow, idxCol);
+        return;
+    } else {
+        textract_frag(dst, src, idxRow, idxCol);
     }
 }
 

@@ -10,6 +10,8 @@
  *   pto_gemm_f16f32      LaunchGEMME2E<T>(uint8_t *out, uint8_t *src0, uint8_t *src1, void *stream)
  *                        kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp:243-264, and the
  *                        ctypes entry call_kernel(blockDim, stream, out, src0, src1) demos/torch_jit/gemm/gemm_kernel.cpp:259-262
+ *   pto_gemm_mxfp8       LaunchMxMatmul(uint8_t *out, uint8_t *src0, uint8_t *src1, uint8_t *src2, uint8_t *src3, void *stream)
+ *                        kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:344-364
  *   pto_fa_fwd_f16       LaunchTFA<...>(...) kernels/manual/common/flash_atten/fa_performance_kernel.h:28-41 and
  *                        call_kernel(...) demos/torch_jit/flash_atten/fa_kernel.cpp:1017-1092
  *   pto_tcvt_*           runTCVT / launchTCVT tests/cpu/st/testcase/tcvt/tcvt_kernel.cpp:18-66 (TLOAD -> TCVT -> TSTORE)
@@ -50,6 +52,14 @@ int pto_last_hip_error(void);
  * k x n operand), fp32 accumulation.  m % 128 == 0, n % 256 == 0, k % 32 == 0 (multiples of the
  * 128 x 256 block of the reference kernel; C is tiled 256 x 256 when m allows it). */
 int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k);
+
+/* MXFP8 GEMM: C[m,n] row-major = (A .* 2^(scale_a - 127)) x (B .* 2^(scale_b - 127)) with fp32 accumulation.
+ * a [m,k] and b stored [n,k] (a column-major k x n operand) hold 8-bit floats: format 0 = e4m3 (OCP, no infinities),
+ * 1 = e5m2, the same for both operands.  scale_a [m,k/32] and scale_b stored [n,k/32] hold one e8m0 exponent per row
+ * (column) and 32 consecutive k (the reference's x1_gm / x2_gm / x1_scale_gm / x2_scale_gm files).  c: bf16
+ * (c_fp32 == 0, round-to-nearest-even of the fp32 sum) or fp32.  m % 256 == 0, n % 256 == 0, k % 512 == 0. */
+int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
+                   int m, int n, int k, int format, int c_fp32);
 
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];

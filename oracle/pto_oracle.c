@@ -502,6 +502,76 @@ void po_gemm_f16f32(float *C, const uint16_t *A, const uint16_t *B, int m, int n
     free(Bf);
 }
 
+/* ------------------------------------------------------------------ MX GEMM */
+/* float8_e4m3fn: 1-4-3, bias 7, no infinities, S.1111.111 = NaN; float8_e5m2: 1-5-2, bias 15, IEEE-style inf / NaN */
+float po_fp8_e4m3fn_to_f32(uint8_t v)
+{
+    const int s = v >> 7, e = (v >> 3) & 0xf, f = v & 7;
+    float r;
+    if (e == 0xf && f == 7)
+        r = NAN;
+    else if (e == 0)
+        r = ldexpf((float)f, -9); /* subnormal: f/8 * 2^-6 */
+    else
+        r = ldexpf((float)(8 + f), e - 10);
+    return s ? -r : r;
+}
+
+float po_fp8_e5m2_to_f32(uint8_t v)
+{
+    const int s = v >> 7, e = (v >> 2) & 0x1f, f = v & 3;
+    float r;
+    if (e == 0x1f)
+        r = f ? NAN : INFINITY;
+    else if (e == 0)
+        r = ldexpf((float)f, -16); /* subnormal: f/4 * 2^-14 */
+    else
+        r = ldexpf((float)(4 + f), e - 17);
+    return s ? -r : r;
+}
+
+typedef struct {
+    float *C;
+    const double *A, *B; /* dequantised operands, A [m,k], B [n,k] */
+    int n, k;
+} po_mx_ctx;
+
+static void po_mx_rows(size_t r0, size_t r1, void *ctx)
+{
+    const po_mx_ctx *g = (const po_mx_ctx *)ctx;
+    for (size_t i = r0; i < r1; i++)
+        for (int j = 0; j < g->n; j++) {
+            const double *a = g->A + i * (size_t)g->k, *b = g->B + (size_t)j * (size_t)g->k;
+            double acc = 0.0;
+            for (int kk = 0; kk < g->k; kk++)
+                acc += a[kk] * b[kk];
+            g->C[i * (size_t)g->n + (size_t)j] = (float)acc;
+        }
+}
+
+static double *po_mx_dequant(const uint8_t *X, const uint8_t *S, int rows, int k, int format)
+{
+    double *out = (double *)malloc(sizeof(double) * (size_t)rows * (size_t)k);
+    const int kb = k / 32;
+    for (int r = 0; r < rows; r++)
+        for (int kk = 0; kk < k; kk++) {
+            const uint8_t v = X[(size_t)r * (size_t)k + (size_t)kk];
+            const double e = format ? (double)po_fp8_e5m2_to_f32(v) : (double)po_fp8_e4m3fn_to_f32(v);
+            out[(size_t)r * (size_t)k + (size_t)kk] = e * ldexp(1.0, (int)S[(size_t)r * (size_t)kb + (size_t)(kk / 32)] - 127);
+        }
+    return out;
+}
+
+void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, int m, int n, int k,
+                int format_a, int format_b, int threads)
+{
+    double *Ad = po_mx_dequant(A, SA, m, k, format_a), *Bd = po_mx_dequant(B, SB, n, k, format_b);
+    po_mx_ctx c = {C, Ad, Bd, n, k};
+    po_parallel_rows((size_t)m, threads, po_mx_rows, &c);
+    free(Ad);
+    free(Bd);
+}
+
 /* ------------------------------------------------------------------- gather */
 void po_tgather_index(void *dst, const po_layout *Ld, const void *src0, const po_layout *L0, const int32_t *idx,
                       const po_layout *L1, int esz, int valid_row, int valid_col)

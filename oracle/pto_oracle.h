@@ -90,6 +90,16 @@ void po_tmatmul_bias_f16(float *dst, const po_layout *Lc, const uint16_t *a, con
 void po_gemm_f16f32(float *C, const uint16_t *A, const uint16_t *B, int m, int n, int k, int base_k, int row0,
                     int row1, int threads);
 
+/* MX matmul (TMATMUL_MX over a whole problem), as the reference's data generators define it
+ * (tests/npu/a5/src/st/testcase/tmatmul_mx/gen_data.py:130-171, kernels/manual/a5/matmul_mxfp8_performance/scripts/gen_data.py:31-50):
+ * x1[i,kk] = fp8(A[i,kk]) * 2^(SA[i,kk/32] - 127), x2[kk,j] = fp8(B[j,kk]) * 2^(SB[j,kk/32] - 127),
+ * C = matmul in float64 -> float32.  A [m,k], B stored [n,k], SA [m,k/32], SB stored [n,k/32] (the generator's
+ * transposed x2 / x2_scale files).  format: 0 = float8_e4m3fn, 1 = float8_e5m2 (ml_dtypes' names). */
+float po_fp8_e4m3fn_to_f32(uint8_t v);
+float po_fp8_e5m2_to_f32(uint8_t v);
+void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, int m, int n, int k,
+                int format_a, int format_b, int threads);
+
 /* ---- conversion: cpu/TCvt.hpp:65-84 ---- */
 uint16_t po_f32_to_f16_rne(uint32_t bits); /* == static_cast<_Float16>(float) */
 uint16_t po_f32_to_bf16_rne(uint32_t bits);

@@ -1,0 +1,289 @@
+// MXFP8 GEMM for MI355X: C[m,n] = (A .* 2^(scaleA-127)) x (B .* 2^(scaleB-127)), fp8 (e4m3 / e5m2) operands with one
+// e8m0 scale per row (column) and 32-wide k block, fp32 accumulation, bf16 or fp32 result.
+//
+// Mirrors the reference kernel kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:149-241
+// (TLOAD of operand and scale panels -> TEXTRACT -> TMATMUL_MX -> TSTORE): A [m,k], B stored [n,k], scaleA [m,k/32],
+// scaleB stored [n,k/32] (scripts/gen_data.py:31-66).
+//
+// Structure: the fp16 GEMM's K-step pipeline (workgroup tile 256 x 256, 8 waves in a 2 x 4 grid, four LDS stages of
+// one 64-byte K-step filled by asynchronous copies, copies / fragment reads / MFMAs interleaved by the scheduler
+// directives).  A K-step is 64 fp8 values = the same 64 bytes per row as 32 fp16 values, and one
+// v_mfma_scale_f32_32x32x64_f8f6f4 (16 passes) takes the place of two v_mfma_f32_32x32x16_f16 (8 passes each), so
+// bytes moved per MFMA cycle are those of the fp16 kernel at twice the flops.  The scales of 512 k (16 blocks = 16
+// bytes per row) are copied into LDS once per eight K-steps (two buffers) and the two scales a lane needs for a K-step
+// are read with the step's fragments (one ds_read_u8 per 32-row block); the MFMA applies them.
+#define PTO_WAVES_M 2
+#define PTO_WAVES_N 4
+#include "gemm_kernels.hpp"
+
+PTO_DEVICE_CODE_BEGIN
+
+namespace {
+
+constexpr int kMxGroupSteps = 8; // K-steps (of 64) per scale group: 16 k blocks = one 16-byte scale row
+
+// One asynchronous copy instruction per wave: the 16-byte scale rows of the workgroup's BM rows of A and BN columns
+// of B for one scale group -> LDS [BM + BN][16 bytes] (the images of an unboxed [BM, 16] row-major and a [16, BN]
+// column-major Mat tile, back to back).  Instruction i covers 64 rows; wave w issues instruction
+// w % ((BM + BN) / 64) (with fewer instructions than waves some waves repeat one: same data to the same place).
+template <int BM, int BN>
+AICORE inline void LoadScaleGroup(uint32_t ldsOff, __gm__ const uint8_t *sa, __gm__ const uint8_t *sb, int64_t ld)
+{
+    constexpr int nA = BM / 64, nB = BN / 64;
+    static_assert(BM % 64 == 0 && BN % 64 == 0 && nA + nB <= kBlockWaves, "one scale copy instruction per wave");
+    const int inst = hw::wave() % (nA + nB), lane = hw::lane();
+    const bool isA = inst < nA;
+    const char *base = reinterpret_cast<const char *>(isA ? sa : sb);
+    const int row = (isA ? inst : inst - nA) * 64;
+    const char *g = detail::uniform_ptr(base + (int64_t)row * ld) + (uint32_t)lane * (uint32_t)ld;
+    __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(hw::lds_base() + ldsOff + inst * 1024), 16, 0, 0);
+}
+
+template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES>
+AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, __gm__ const FA *src0, __gm__ const FB *src1,
+                                                             __gm__ const uint8_t *scale0, __gm__ const uint8_t *scale1, int m,
+                                                             int n, int k, int row0, int col0)
+{
+    constexpr int BK = 64, HM = BM / 2, KB = 2 * kMxGroupSteps;
+    using X = float8_e8m0_t;
+    using TileMatA = Tile<TileType::Mat, FA, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
+    using TileMatB = Tile<TileType::Mat, FB, BK, BN, BLayout::RowMajor, BK, BN, SLayout::ColMajor>;
+    using TileScaleA = Tile<TileType::Mat, X, BM, KB, BLayout::RowMajor, BM, KB, SLayout::NoneBox>;
+    using TileScaleB = Tile<TileType::Mat, X, KB, BN, BLayout::ColMajor, KB, BN, SLayout::NoneBox>;
+    using LeftHalf = TileLeft<FA, HM, BK, HM, BK>;
+    using RightTile = TileRight<FB, BK, BN, BK, BN>;
+    using LeftScaleStep = TileLeftScale<X, HM, 2>;
+    using RightScaleStep = TileRightScale<X, 2, BN>;
+    using AccHalf = TileAcc<float, HM, BN, HM, BN>;
+    using ShapeA = TileShape2D<FA, BM, BK, Layout::ND>;
+    using StrideA = BaseShape2D<FA, DYNAMIC, DYNAMIC, Layout::ND>;
+    using GlobalA = GlobalTensor<FA, ShapeA, StrideA, Layout::ND>;
+    using ShapeB = TileShape2D<FB, BK, BN, Layout::DN>;
+    using StrideB = BaseShape2D<FB, DYNAMIC, DYNAMIC, Layout::DN>;
+    using GlobalB = GlobalTensor<FB, ShapeB, StrideB, Layout::DN>;
+    using ShapeC = TileShape2D<OutT, HM, BN, Layout::ND>;
+    using StrideC = BaseShape2D<OutT, DYNAMIC, DYNAMIC, Layout::ND>;
+    using GlobalC = GlobalTensor<OutT, ShapeC, StrideC, Layout::ND>;
+
+    constexpr uint32_t kABytes = BM * BK, kBBytes = BK * BN;
+    constexpr uint32_t kStage = kABytes + kBBytes;
+    constexpr uint32_t kScaleOff = STAGES * kStage, kScaleBytes = (BM + BN) * 16; // two buffers of [BM + BN][16] scale rows
+    constexpr int kLoadsPerStep = TLoadInstrs<TileMatA>() + TLoadInstrs<TileMatB>();
+    constexpr int kMfma = 2 * AccHalf::Storage::MB * AccHalf::Storage::NB;
+    constexpr int kReadsA = 2 * LeftHalf::Storage::MB, kReadsB = 2 * RightTile::Storage::NB; // two ds_read_b128 per fragment
+    constexpr int kReads = 2 * kReadsA + kReadsB + (2 * LeftHalf::Storage::MB + RightTile::Storage::NB); // + the scale reads
+    // issue pattern of a step: the copies first, one MFMA before each; the fragment reads spread over the next MFMAs;
+    // the last MFMA has no read after it
+    constexpr int kMfmaCopies = kMfma >= 8 ? kLoadsPerStep : 1, kMfmaTail = 1;
+    constexpr int kMfmaForReads = kMfma - kMfmaCopies - kMfmaTail;
+    static_assert(STAGES == 4, "two fragment sets alternate with the stage index");
+    static_assert(kMfmaForReads >= 0, "issue pattern below");
+
+    __gm__ FA *aPanel = const_cast<FA *>(src0) + (int64_t)row0 * k;
+    __gm__ FB *bPanel = const_cast<FB *>(src1) + (int64_t)col0 * k;
+    const int64_t ldScale = k / 32;
+    __gm__ const uint8_t *saPanel = scale0 + (int64_t)row0 * ldScale;
+    __gm__ const uint8_t *sbPanel = scale1 + (int64_t)col0 * ldScale;
+    const StrideA strideA(m, k);
+    const StrideB strideB(k, n);
+    const int kLoop = k / BK, groups = kLoop / kMxGroupSteps;
+
+    TileMatA aMat[STAGES];
+    TileMatB bMat[STAGES];
+#pragma unroll
+    for (int s = 0; s < STAGES; ++s) {
+        TASSIGN(aMat[s], s * kStage);
+        TASSIGN(bMat[s], s * kStage + kABytes);
+    }
+    TileScaleA aScaleMat;
+    TileScaleB bScaleMat;
+    TASSIGN(aScaleMat, kScaleOff);
+    TASSIGN(bScaleMat, kScaleOff + BM * 16);
+
+    // Operand fragments and their scales.  The lower row half and B have two sets: the MFMAs of step it read set it % 2
+    // while the other arrives.  The upper row half, whose MFMAs come first in a step, has one (the register file of two
+    // waves per SIMD does not hold a second): its reads for the next step follow its last MFMA and have half a step to land.
+    LeftHalf aUp, aDn[2];
+    RightTile bAll[2];
+    LeftScaleStep saUp, saDn[2];
+    RightScaleStep sbAll[2];
+    AccHalf cUp, cDn;
+#pragma unroll
+    for (int mb = 0; mb < AccHalf::Storage::MB; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < AccHalf::Storage::NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < detail::kAccElems; ++i) {
+                cUp.st.f[mb][nb][i] = 0.0f;
+                cDn.st.f[mb][nb][i] = 0.0f;
+            }
+
+    // prologue: the scales of group 0, then STAGES-1 K-steps in flight
+    LoadScaleGroup<BM, BN>(kScaleOff, saPanel, sbPanel, ldScale);
+#pragma unroll
+    for (int s = 0; s < STAGES - 1; ++s) {
+        GlobalA gmA(aPanel + (int64_t)s * BK, ShapeA(), strideA);
+        GlobalB gmB(bPanel + (int64_t)s * BK, ShapeB(), strideB);
+        TLOAD(aMat[s], gmA);
+        TLOAD(bMat[s], gmB);
+    }
+    wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // scales and stage 0 are complete
+    TEXTRACT(saUp, aScaleMat, 0, 0);
+    TEXTRACT(saDn[0], aScaleMat, HM, 0);
+    TEXTRACT(sbAll[0], bScaleMat, 0, 0);
+    TEXTRACT(aUp, aMat[0], 0, 0);
+    TEXTRACT(aDn[0], aMat[0], HM, 0);
+    TEXTRACT(bAll[0], bMat[0], 0, 0);
+
+    // K-step j of a scale group (compile-time: LDS stage j % 4, fragment set j % 2, scales of k blocks 2j, 2j+1 of the
+    // group).  Scale buffer group % 2 holds the group's scales.  Past the end of K the copies re-fetch the last K-step /
+    // scale group and the reads fetch values nobody uses.
+    auto step = [&](auto jTag, int it, int group) {
+        constexpr int j = decltype(jTag)::value;
+        constexpr int s = j % STAGES, sNext = (s + 1) % STAGES, sLoad = (s + STAGES - 1) % STAGES;
+        // the copies of K-step it+1 (issued two steps ago) have landed; only those of the previous step (plus its scale
+        // copy, if it had one) may still be in flight
+        hw::wait_vm<(STAGES - 3) * kLoadsPerStep + (j == 2 ? 1 : 0)>();
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        const uint32_t otherBuf = kScaleOff + (uint32_t)((group + 1) & 1) * kScaleBytes;
+        if constexpr (j == 1) {
+            // scales of the next group into the other buffer: last read in step 6 of the previous group, and those
+            // values have fed MFMAs since
+            const int g = group + 1 < groups ? group + 1 : groups - 1;
+            LoadScaleGroup<BM, BN>(otherBuf, saPanel + g * 16, sbPanel + g * 16, ldScale);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (j == kMxGroupSteps - 1) { // the next step is the first of the next group
+            TASSIGN(aScaleMat, otherBuf);
+            TASSIGN(bScaleMat, otherBuf + BM * 16);
+        }
+        const int fetch = it + STAGES - 1 < kLoop ? it + STAGES - 1 : kLoop - 1;
+        GlobalA gmA(aPanel + (int64_t)fetch * BK, ShapeA(), strideA);
+        GlobalB gmB(bPanel + (int64_t)fetch * BK, ShapeB(), strideB);
+        TLOAD(aMat[sLoad], gmA);
+        TLOAD(bMat[sLoad], gmB);
+        constexpr int p = j & 1, q = p ^ 1, kbNext = 2 * ((j + 1) % kMxGroupSteps);
+        TMATMUL_MX(cUp, cUp, aUp, saUp, bAll[p], sbAll[p]);
+        TEXTRACT(aUp, aMat[sNext], 0, 0);
+        TEXTRACT(saUp, aScaleMat, 0, +kbNext);
+        TMATMUL_MX(cDn, cDn, aDn[p], saDn[p], bAll[p], sbAll[p]);
+        TEXTRACT(bAll[q], bMat[sNext], 0, 0);
+        TEXTRACT(sbAll[q], bScaleMat, +kbNext, 0);
+        TEXTRACT(aDn[q], aMat[sNext], HM, 0);
+        TEXTRACT(saDn[q], aScaleMat, +HM, +kbNext);
+#pragma unroll
+        for (int i = 0; i < kLoadsPerStep; ++i) {
+            if (i < kMfmaCopies)
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
+        }
+        StaticFor<0, kReads>([](auto iTag) {
+            constexpr int i = decltype(iTag)::value;
+            constexpr int cnt = (i + 1) * kMfmaForReads / kReads - i * kMfmaForReads / kReads;
+            if constexpr (cnt > 0)
+                __builtin_amdgcn_sched_group_barrier(0x008, cnt, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        });
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaTail, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    using std::integral_constant;
+    for (int group = 0; group < groups; ++group) {
+        const int it = group * kMxGroupSteps;
+        step(integral_constant<int, 0>(), it, group);
+        step(integral_constant<int, 1>(), it + 1, group);
+        step(integral_constant<int, 2>(), it + 2, group);
+        step(integral_constant<int, 3>(), it + 3, group);
+        step(integral_constant<int, 4>(), it + 4, group);
+        step(integral_constant<int, 5>(), it + 5, group);
+        step(integral_constant<int, 6>(), it + 6, group);
+        step(integral_constant<int, 7>(), it + 7, group);
+    }
+    hw::wait_vm0(); // the copies issued past the end of K must not outlive the workgroup's LDS
+    GlobalC dstUp(out + (int64_t)row0 * n + col0, ShapeC(), StrideC(m, n));
+    GlobalC dstDn(out + (int64_t)(row0 + HM) * n + col0, ShapeC(), StrideC(m, n));
+    TSTORE(dstUp, cUp);
+    TSTORE(dstDn, cDn);
+}
+
+// The first `fullTiles` workgroups (whole rounds over the compute units) own one BM x BN C tile each; with quarter != 0
+// the tiles of the last, partial round are cut into four (BM/2) x (BN/2) tiles, one workgroup each.
+template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES, int GROUP_M>
+__global__ __launch_bounds__(kBlockThreads, 1) AICORE
+    void GemmMx(__gm__ OutT *out, __gm__ const FA *src0, __gm__ const FB *src1, __gm__ const uint8_t *scale0,
+                __gm__ const uint8_t *scale1, int m, int n, int k, int fullTiles)
+{
+    const int tilesM = m / BM, tilesN = n / BN;
+    const int block = (int)get_block_idx();
+    int tm, tn;
+    if (block >= fullTiles) {
+        const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
+        TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
+        const int sub = u % 4;
+        MxTileRows<FA, FB, OutT, BM / 2, BN / 2, STAGES>(out, src0, src1, scale0, scale1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
+                                                        tn * BN + (sub & 1) * (BN / 2));
+        return;
+    }
+    TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
+    MxTileRows<FA, FB, OutT, BM, BN, STAGES>(out, src0, src1, scale0, scale1, m, n, k, tm * BM, tn * BN);
+}
+
+} // namespace
+
+PTO_DEVICE_CODE_END
+
+namespace {
+
+template <typename FA, typename FB, typename OutT>
+int launch_gemm_mx(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n,
+                   int k, int tailMode)
+{
+    constexpr int BM = 256, BN = 256, STAGES = 4, GROUP_M = 4;
+    if (m % BM || n % BN || k % (64 * kMxGroupSteps))
+        return PTO_ERR_UNSUPPORTED;
+    constexpr int lds = STAGES * (BM + BN) * 64 + 2 * (BM + BN) * 16;
+    auto kernel = GemmMx<FA, FB, OutT, BM, BN, STAGES, GROUP_M>;
+    static const int attr = pto_amd::allow_lds(kernel, lds);
+    if (attr != PTO_OK)
+        return attr;
+    const int tiles = (m / BM) * (n / BN), cus = compute_units();
+    int full = tiles / cus * cus;
+    // quarter tiles move twice the operand bytes per flop: only when they fit one round
+    if (tailMode == 0 || full == 0 || (tiles - full) * 4 > cus)
+        full = tiles;
+    kernel<<<dim3(full + (tiles - full) * 4), dim3(kBlockThreads), lds, st>>>(
+        reinterpret_cast<OutT *>(c), reinterpret_cast<const FA *>(a), reinterpret_cast<const FB *>(b), sa, sb, m, n, k, full);
+    return pto_amd::check_launch();
+}
+
+int gemm_mx_dispatch(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n,
+                     int k, int format, int c_fp32, int tailMode)
+{
+    if (format == 0)
+        return c_fp32 ? launch_gemm_mx<float8_e4m3_t, float8_e4m3_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float8_e4m3_t, float8_e4m3_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
+    if (format == 1)
+        return c_fp32 ? launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
+    return PTO_ERR_UNSUPPORTED;
+}
+
+} // namespace
+
+extern "C" int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
+                              const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32)
+{
+    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0)
+        return PTO_ERR_BAD_ARG;
+    return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 1);
+}
+
+// Tuning hook (not part of the public header): variant 0 = whole tiles only, 1 = quarter tiles in the last round.
+extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
+                                      const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant)
+{
+    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0 || variant < 0 || variant > 1)
+        return PTO_ERR_BAD_ARG;
+    return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, variant);
+}

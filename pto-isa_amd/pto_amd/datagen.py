@@ -14,6 +14,7 @@ SEED_TCVT = 3001
 SEED_TCVT_INJECT = 3002
 SEED_GATHER_TABLE = 4001
 SEED_GATHER_IDX = 4002
+SEED_MX_A, SEED_MX_B, SEED_MX_SA, SEED_MX_SB = 19, 2019, 3019, 4019
 
 
 def _rng(seed):
@@ -66,6 +67,57 @@ def tcvt_input(rows, cols, inject=0.001):
         rnd = r.integers(0, 2**32, size=cnt // 4 + 1, dtype=np.uint64).astype(np.uint32)
         xv[r.integers(0, n, size=rnd.size)] = rnd
     return x.reshape(rows, cols)
+
+
+def fp8_values(fmt):
+    """The 256 values of float8_e4m3fn (fmt 0: 1-4-3, bias 7, no infinities, 0x7f / 0xff NaN) or float8_e5m2
+    (fmt 1: 1-5-2, bias 15, IEEE-style infinities and NaNs) as float64, indexed by the byte."""
+    v = np.arange(256)
+    s = np.where(v & 0x80, -1.0, 1.0)
+    if fmt == 0:
+        e, f = (v >> 3) & 0xF, (v & 7).astype(np.float64)
+        mag = np.where(e == 0, f * 2.0 ** -9, (8 + f) * 2.0 ** (e.astype(np.float64) - 10))
+        mag = np.where((e == 0xF) & (f == 7), np.nan, mag)
+    else:
+        e, f = (v >> 2) & 0x1F, (v & 3).astype(np.float64)
+        mag = np.where(e == 0, f * 2.0 ** -16, (4 + f) * 2.0 ** (e.astype(np.float64) - 17))
+        mag = np.where(e == 0x1F, np.where(f == 0, np.inf, np.nan), mag)
+    return s * mag
+
+
+def fp8_encode(x, fmt):
+    """float array -> fp8 bytes, nearest finite value (saturating); a tie takes the value with the lower byte."""
+    tab = fp8_values(fmt)
+    finite = np.flatnonzero(np.isfinite(tab) & ~((np.arange(256) == 0x80)))      # one zero: +0
+    order = finite[np.argsort(tab[finite], kind="stable")]
+    vals = tab[order]
+    x = np.asarray(x, dtype=np.float64)
+    hi = np.clip(np.searchsorted(vals, x), 1, vals.size - 1)
+    lo = hi - 1
+    pick = np.where(np.abs(x - vals[lo]) <= np.abs(vals[hi] - x), lo, hi)
+    return order[pick].astype(np.uint8)
+
+
+def mx_inputs(m, n, k, fmt, dist="uniform", scale_lo=127, scale_hi=130):
+    """Operands of the MXFP8 GEMM: A [m,k], B [n,k] fp8 bytes, SA [m,k/32], SB [n,k/32] e8m0 bytes.
+
+    dist "uniform": uniform(-5, 5) rounded to fp8 and scales in [127, 130), the distribution of
+    kernels/manual/a5/matmul_mxfp8_performance/scripts/gen_data.py:31-38; "integer": integers in [-10, 10) as in
+    tests/npu/a5/src/st/testcase/tmatmul_mx/gen_data.py:113-120; "bytes": every finite encoding, subnormals included."""
+    ra, rb = _rng(SEED_MX_A), _rng(SEED_MX_B)
+    if dist == "uniform":
+        a = fp8_encode(ra.uniform(-5.0, 5.0, size=(m, k)), fmt)
+        b = fp8_encode(rb.uniform(-5.0, 5.0, size=(n, k)), fmt)
+    elif dist == "integer":
+        a = fp8_encode(ra.integers(-10, 10, size=(m, k)), fmt)
+        b = fp8_encode(rb.integers(-10, 10, size=(n, k)), fmt)
+    else:
+        finite = np.flatnonzero(np.isfinite(fp8_values(fmt))).astype(np.uint8)
+        a = finite[ra.integers(0, finite.size, size=(m, k))]
+        b = finite[rb.integers(0, finite.size, size=(n, k))]
+    sa = _rng(SEED_MX_SA).integers(scale_lo, scale_hi, size=(m, k // 32)).astype(np.uint8)
+    sb = _rng(SEED_MX_SB).integers(scale_lo, scale_hi, size=(n, k // 32)).astype(np.uint8)
+    return a, b, sa, sb
 
 
 def gather_inputs(table_rows, cols, n_idx):

@@ -457,3 +457,70 @@ def test_result_cmp_semantics(oracle):
     a[1] = 1.01
     ok, _, nbad = oracle.result_cmp(e, a, 1e-3)
     assert not ok and nbad == 2
+
+
+# ------------------------------------------------------------------ MX GEMM
+def _torch_fp8_table(fmt):
+    import torch
+    dt = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
+    return torch.arange(256, dtype=torch.int32).to(torch.uint8).view(dt).to(torch.float32).numpy()
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_fp8_decode_matches_an_independent_implementation(oracle, fmt):
+    """The oracle's and the data generator's fp8 decoders against torch's float8_e4m3fn / float8_e5m2 (all 256 bytes)."""
+    from pto_amd import datagen
+    want = _torch_fp8_table(fmt)
+    got = oracle.fp8_table(fmt)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(got[ok].view(np.uint32), want[ok].view(np.uint32))      # signed zeros and infinities included
+    gen = datagen.fp8_values(fmt).astype(np.float32)
+    assert np.array_equal(np.isnan(gen), np.isnan(want)) and np.array_equal(gen[ok], want[ok])
+    # known values: largest finite, smallest subnormal, one
+    if fmt == 0:
+        assert got[0x7E] == 448.0 and got[0x01] == 2.0 ** -9 and got[0x38] == 1.0
+    else:
+        assert got[0x7B] == 57344.0 and got[0x01] == 2.0 ** -16 and got[0x3C] == 1.0 and np.isinf(got[0x7C])
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_fp8_encode_round_trips_and_rounds_to_nearest(fmt):
+    import torch
+    from pto_amd import datagen
+    tab = datagen.fp8_values(fmt)
+    finite = np.flatnonzero(np.isfinite(tab) & (np.arange(256) != 0x80))
+    assert np.array_equal(datagen.fp8_encode(tab[finite], fmt), finite.astype(np.uint8))
+    x = np.random.Generator(np.random.Philox(key=5)).uniform(-5, 5, size=4096)
+    got = tab[datagen.fp8_encode(x, fmt)]
+    dt = torch.float8_e5m2 if fmt else torch.float8_e4m3fn
+    want = torch.from_numpy(x).to(dt).to(torch.float64).numpy()
+    # nearest value either way; only exact ties may differ (torch rounds them to even)
+    assert np.all(np.abs(got - x) <= np.abs(want - x) + 1e-12)
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_mx_gemm_oracle_closed_forms(oracle, fmt):
+    from pto_amd import datagen
+    m, n, k = 24, 40, 128
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt, dist="integer")
+    tab = _torch_fp8_table(fmt).astype(np.float64)          # decoded independently of the oracle
+    ad = tab[a] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
+    bd = tab[b] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
+    got = oracle.mx_gemm(a, b, sa, sb, fmt)
+    assert np.array_equal(got, (ad @ bd.T).astype(np.float32))                   # integers: exact
+    # raising every scale of A by one doubles C; of one k block of B: adds that block's contribution once more
+    assert np.array_equal(oracle.mx_gemm(a, b, sa + 1, sb, fmt), 2 * got)
+    sb2 = sb.copy()
+    sb2[:, 2] += 1
+    extra = ad[:, 64:96] @ bd[:, 64:96].T
+    assert np.array_equal(oracle.mx_gemm(a, b, sa, sb2, fmt), (ad @ bd.T + extra).astype(np.float32))
+    # mixed operand formats
+    a1, _, _, _ = datagen.mx_inputs(m, n, k, 1 - fmt, dist="integer")
+    ad1 = _torch_fp8_table(1 - fmt).astype(np.float64)[a1] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
+    assert np.array_equal(oracle.mx_gemm(a1, b, sa, sb, 1 - fmt, fmt), (ad1 @ bd.T).astype(np.float32))
+    # the generator's distribution, against a float64 matmul
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt)
+    ad = tab[a] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
+    bd = tab[b] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
+    assert np.allclose(oracle.mx_gemm(a, b, sa, sb, fmt), ad @ bd.T, rtol=1e-6, atol=1e-4)
