@@ -1,11 +1,11 @@
 #!/usr/bin/env python3
 """Benchmark of the PTO tile compute path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|fa|tcvt|gather]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|mx|fa|tcvt|gather]
 
 A step is one pass of the hot path over one batch of synthetic input, resident in HBM before the
 timed region: one fp16 -> fp32 GEMM at m=n=k=6144 (the configuration the headline metric is quoted
-on).  The other workloads of the metric (flash-attention forward, TCVT, gather) are timed the same
+on).  The other workloads of the metric (flash-attention forward, TCVT, gather) and the MXFP8 GEMM are timed the same
 way and reported under "extra".  Prints ONE JSON line.
 """
 import argparse
@@ -20,6 +20,7 @@ for p in (ROOT, os.path.join(ROOT, "pto-isa_amd")):
         sys.path.insert(0, p)
 
 PEAK_FP16_TFLOPS = 2516.6   # MI355X dense fp16 matrix peak (published)
+PEAK_FP8_TFLOPS = 5033.2    # dense fp8 matrix peak (published)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 
 # HBM-side traffic of one 6144^3 GEMM launch, from two rocprofv3 --pmc runs of this script
@@ -55,6 +56,21 @@ def bench_gemm(torch, lib, capi, datagen, size, steps, warmup):
 
     def step():
         capi.check(lib.pto_gemm_f16f32(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), size, size, size), "gemm")
+    ms = time_launches(torch, step, steps, warmup)
+    flops = 2.0 * size ** 3
+    return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
+
+
+def bench_gemm_mx(torch, lib, capi, datagen, size, steps, warmup):
+    """MXFP8 GEMM of the reference's matmul_mxfp8_performance case: e5m2 operands, e8m0 block scales, bf16 result."""
+    a, b, sa, sb = datagen.mx_inputs(size, size, size, 1)
+    ta, tb, tsa, tsb = (torch.from_numpy(x).cuda() for x in (a, b, sa, sb))
+    tc = torch.empty((size, size), dtype=torch.bfloat16, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        capi.check(lib.pto_gemm_mxfp8(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                      size, size, size, 1, 0), "gemm_mxfp8")
     ms = time_launches(torch, step, steps, warmup)
     flops = 2.0 * size ** 3
     return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
@@ -183,7 +199,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="gemm | fa | tcvt | gather: time just that workload")
+    ap.add_argument("--only", default="", help="gemm | mx | fa | tcvt | gather: time just that workload")
     ap.add_argument("--size", type=int, default=6144)
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -213,6 +229,9 @@ def main():
         for s in (3072, 7680):
             r = bench_gemm(torch, lib, capi, datagen, s, max(args.steps // 2, 1), 2)
             extra["gemm_%d" % s] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp16_peak": r["tflops"] / PEAK_FP16_TFLOPS}
+    if only in ("", "mx"):
+        r = bench_gemm_mx(torch, lib, capi, datagen, 6144, args.steps, args.warmup)
+        extra["gemm_mxfp8_e5m2_bf16_6144"] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp8_peak": r["tflops"] / PEAK_FP8_TFLOPS}
     if only in ("", "fa") and hasattr(lib, "pto_fa_fwd_f16"):
         for name, cfg in (("fa_b1_h16_s4096_d128", (1, 16, 4096, 128, False)),
                           ("fa_causal_b4_h32_s2048_d64", (4, 32, 2048, 64, True))):
