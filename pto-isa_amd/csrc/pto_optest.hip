@@ -273,6 +273,52 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulBias(__gm__ float 
     TSTORE(gc, c, computed);
 }
 
+// ---- one-block MX matmul [128, 256] x [256, 128], fp8 operands (formats may differ) with e8m0 block scales ----
+// (tests/npu/a5/src/st/testcase/tmatmul_mx/tmatmul_mx_kernel.cpp: TLOAD -> TEXTRACT -> TMATMUL_MX -> TSTORE).  K is taken
+// in two halves of 128: TMATMUL_MX on the first, the accumulating form on the second; the scale tiles are loaded whole
+// from memory (MX_A_ND / MX_B_DN) and windowed per half.
+template <typename FA, typename FB>
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMx(__gm__ float *out, __gm__ const FA *a, __gm__ const FB *bT,
+                                                                 __gm__ const float8_e8m0_t *sa, __gm__ const float8_e8m0_t *sbT)
+{
+    constexpr int M = 128, N = 128, K = 256, KH = 128, KB = K / 32;
+    using X = float8_e8m0_t;
+    using MatA = Tile<TileType::Mat, FA, M, K, BLayout::ColMajor, M, K, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, FB, K, N, BLayout::RowMajor, K, N, SLayout::ColMajor>;
+    MatA am;
+    MatB bm;
+    TASSIGN(am, 0u);
+    TASSIGN(bm, (uint32_t)(M * K));
+    TileLeft<FA, M, KH> l;
+    TileRight<FB, KH, N> r;
+    TileLeftScale<X, M, KB> lsAll;
+    TileRightScale<X, KB, N> rsAll;
+    TileLeftScale<X, M, KH / 32> ls;
+    TileRightScale<X, KH / 32, N> rs;
+    TileAcc<float, M, N> c;
+    GmND<FA, M, K> ga(const_cast<FA *>(a));
+    GlobalTensor<FB, Shape<1, 1, 1, K, N>, Stride<1, 1, 1, 1, K>, Layout::DN> gb(const_cast<FB *>(bT));
+    GlobalTensor<X, TileShape2D<X, M, KB, Layout::MX_A_ND>, BaseShape2D<X, M, KB, Layout::MX_A_ND>, Layout::MX_A_ND> gsa(const_cast<X *>(sa));
+    GlobalTensor<X, TileShape2D<X, KB, N, Layout::MX_B_DN>, BaseShape2D<X, KB, N, Layout::MX_B_DN>, Layout::MX_B_DN> gsb(const_cast<X *>(sbT));
+    GmND<float, M, N> gc(out);
+    TLOAD(am, ga);
+    TLOAD(bm, gb);
+    TLOAD(lsAll, gsa);
+    TLOAD(rsAll, gsb);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    TEXTRACT(l, am, 0, 0);
+    TEXTRACT(r, bm, 0, 0);
+    TEXTRACT(ls, lsAll, 0, 0);
+    TEXTRACT(rs, rsAll, 0, 0);
+    TMATMUL_MX(c, l, ls, r, rs);
+    TEXTRACT(l, am, 0, KH);
+    TEXTRACT(r, bm, KH, 0);
+    TEXTRACT(ls, lsAll, 0, KH / 32);
+    TEXTRACT(rs, rsAll, KH / 32, 0);
+    TMATMUL_MX(c, c, l, ls, r, rs);
+    TSTORE(gc, c);
+}
 
 // ---- one Vec instruction on [64, 128] fp32 tiles; `vec` is a per-row ([64]) or per-column ([128]) operand ----
 enum VecOp : int {
@@ -615,6 +661,35 @@ extern "C" int pto_st_textract_windows_f16(void *stream, float *out_left, float 
     ExtractWindows<<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(
         out_left, out_right, reinterpret_cast<const half *>(a), reinterpret_cast<const half *>(b_t),
         reinterpret_cast<const half *>(eye_b), reinterpret_cast<const half *>(eye_a), col0, row0);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
+                                            const uint8_t *scale_b_t, int format_a, int format_b)
+{
+    PTO_ST_NONNULL(out, a, b_t, scale_a, scale_b_t);
+    if (format_a < 0 || format_a > 1 || format_b < 0 || format_b > 1)
+        return PTO_ERR_BAD_ARG;
+    constexpr int lds = 128 * 256 + 256 * 128;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const float8_e8m0_t *sa = reinterpret_cast<const float8_e8m0_t *>(scale_a), *sb = reinterpret_cast<const float8_e8m0_t *>(scale_b_t);
+#define PTO_ST_MX(FA, FB)                                                                                                     \
+    do {                                                                                                                      \
+        static const int attr = pto_amd::allow_lds(MatmulMx<FA, FB>, lds);                                                    \
+        if (attr != PTO_OK)                                                                                                   \
+            return attr;                                                                                                      \
+        MatmulMx<FA, FB><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const FA *>(a),                     \
+                                                                    reinterpret_cast<const FB *>(b_t), sa, sb);              \
+    } while (0)
+    if (format_a == 0 && format_b == 0)
+        PTO_ST_MX(float8_e4m3_t, float8_e4m3_t);
+    else if (format_a == 0)
+        PTO_ST_MX(float8_e4m3_t, float8_e5m2_t);
+    else if (format_b == 0)
+        PTO_ST_MX(float8_e5m2_t, float8_e4m3_t);
+    else
+        PTO_ST_MX(float8_e5m2_t, float8_e5m2_t);
+#undef PTO_ST_MX
     return pto_amd::check_launch();
 }
 

@@ -254,3 +254,25 @@ def test_tpush_tpop_pipeline(lds_fifo):
         qslots = qk.cpu().numpy().reshape(2, 64, 128)
         for t in range(2):
             assert np.array_equal(qslots[t], a @ b[t])
+
+
+@pytest.mark.parametrize("fmt_a,fmt_b", [(0, 0), (1, 1), (0, 1), (1, 0)])
+def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b):
+    """TMATMUL_MX and its accumulating form on two 128-wide k halves (two MFMA k steps each), mixed operand formats,
+    scale tiles loaded from memory (MX_A_ND / MX_B_DN) and windowed: exact on integer operands, <= 2e-3 on random ones."""
+    from pto_amd import datagen
+    lib = capi.load()
+    for dist, lo, hi in (("integer", 125, 130), ("uniform", 120, 135), ("bytes", 110, 140)):
+        a, _, sa, _ = datagen.mx_inputs(128, 128, 256, fmt_a, dist=dist, scale_lo=lo, scale_hi=hi)
+        _, b, _, sb = datagen.mx_inputs(128, 128, 256, fmt_b, dist=dist, scale_lo=lo, scale_hi=hi)
+        out = torch.full((128, 128), float("nan"), device=DEV)
+        ta, tb, tsa, tsb = (torch.from_numpy(x).to(DEV) for x in (a, b, sa, sb))
+        capi.check(lib.pto_st_matmul_mx_128x256x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(),
+                                                    tsb.data_ptr(), fmt_a, fmt_b), "matmul mx")
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        want = oracle.mx_gemm(a, b, sa, sb, fmt_a, fmt_b)
+        if dist == "integer":
+            assert np.array_equal(got, want), (dist, fmt_a, fmt_b)
+        else:
+            assert np.max(np.abs(got - want)) <= 2e-3 * np.max(np.abs(want)), (dist, fmt_a, fmt_b)
