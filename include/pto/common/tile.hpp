@@ -78,6 +78,13 @@ struct TileStorage<TileType::Mat, T, Rows, Cols> {
 // bytes k = 16 (l / 32) .. +15 (first four registers) and k = 32 + 16 (l / 32) .. +15 (last four).
 template <typename T>
 constexpr bool is_mx8_v = std::is_same_v<T, float8_e4m3_t> || std::is_same_v<T, float8_e5m2_t>;
+template <typename T>
+constexpr bool is_mx4_v = std::is_same_v<T, float4_e2m1x2_t>;
+template <typename T>
+constexpr bool is_mx_operand_v = is_mx8_v<T> || is_mx4_v<T>;
+// bits per logical element (extents of 4-bit types count elements, their storage type holds two)
+template <typename T>
+constexpr int elem_bits = is_mx4_v<T> ? 4 : 8 * (int)sizeof(T);
 constexpr int kMxM = 32, kMxK = 64, kMxBlock = 32;
 
 template <int Rows, int Cols>
@@ -100,6 +107,25 @@ struct TileStorage<TileType::Right, float8_e4m3_t, Rows, Cols> {
 };
 template <int Rows, int Cols>
 struct TileStorage<TileType::Right, float8_e5m2_t, Rows, Cols> : TileStorage<TileType::Right, float8_e4m3_t, Rows, Cols> {};
+
+// 4-bit MX operands: a fragment is 32 rows x 64 k = 32 bytes per row; lane l holds row l % 32 and the 16 bytes
+// k = 32 (l / 32) .. +31 (four registers).
+template <int Rows, int Cols>
+struct TileStorage<TileType::Left, float4_e2m1x2_t, Rows, Cols> {
+    static_assert(kMfmaM == kMxM, "MX operand tiles need PTO_MFMA_M 32 (accumulator layout of the 32 x 32 MFMA)");
+    static_assert(Rows % (kMxM * kWavesM) == 0 && Cols % kMxK == 0, "MX Left tile: multiples of 32 x PTO_WAVES_M rows, 64 columns");
+    static constexpr int MB = Rows / (kMxM * kWavesM), Blocks = MB;
+    static constexpr int KS = Cols / kMxK;
+    u32x4 f[MB][KS];
+};
+template <int Rows, int Cols>
+struct TileStorage<TileType::Right, float4_e2m1x2_t, Rows, Cols> {
+    static_assert(kMfmaM == kMxM, "MX operand tiles need PTO_MFMA_M 32 (accumulator layout of the 32 x 32 MFMA)");
+    static_assert(Cols % (kMxM * kWavesN) == 0 && Rows % kMxK == 0, "MX Right tile: multiples of 32 x PTO_WAVES_N columns, 64 rows");
+    static constexpr int NB = Cols / (kMxM * kWavesN), Blocks = NB;
+    static constexpr int KS = Rows / kMxK;
+    u32x4 f[NB][KS];
+};
 
 // Block scales of an MX operand tile: one e8m0 value per row (column) and 32-wide k block, KB blocks per row.
 // Per 32-row block of its part of the operand a wave holds the scales of the lane's row, four k blocks to a

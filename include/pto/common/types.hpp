@@ -16,6 +16,9 @@ using bfloat16_t = __bf16;
 struct float8_e4m3_t { uint8_t bits; };
 struct float8_e5m2_t { uint8_t bits; };
 struct float8_e8m0_t { uint8_t bits; }; // a power of two: 2^(bits - 127)
+// two 4-bit e2m1 values (0, 0.5, 1, 1.5, 2, 3, 4, 6 and their negatives): element 2i in bits 0-3, element 2i+1 in bits 4-7.
+// Tile and GlobalTensor extents of this type count 4-bit elements; pointers to it advance by two elements.
+struct float4_e2m1x2_t { uint8_t bits; };
 
 constexpr int DYNAMIC = -1;
 

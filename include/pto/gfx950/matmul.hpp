@@ -91,18 +91,23 @@ PTO_DEV void TMATMUL_ACC_IMPL(AccT &cOut, AccT &cIn, LeftT &a, RightT &b)
 }
 
 // TMATMUL_MX: C (+)= (A * scaleA) x (B * scaleB) on 8-bit MX operands, one e8m0 scale per row (column) and 32-wide
-// k block (reference semantics: the data generators of tests/npu/a5/src/st/testcase/tmatmul_mx and
+// k block; operands may also be 4-bit e2m1 pairs (reference semantics: the data generators of tests/npu/a5/src/st/testcase/tmatmul_mx and
 // kernels/manual/a5/matmul_mxfp8_performance/scripts/gen_data.py:24-50: operand element x 2^(scale - 127), products
 // accumulated in fp32).  v_mfma_scale_f32_32x32x64_f8f6f4 applies the scales inside the MFMA.
 namespace detail {
 template <typename T>
-constexpr int mx_format = std::is_same_v<T, float8_e5m2_t> ? 1 : 0; // the MFMA's cbsz / blgp operand-format code
+constexpr int mx_format = is_mx4_v<T> ? 4 : std::is_same_v<T, float8_e5m2_t> ? 1 : 0; // the MFMA's cbsz / blgp operand-format code
+
+// the MFMA's operand type is eight registers whatever the format; 4-bit operands occupy the first four
+PTO_DEV i32x8 mx_operand(i32x8 f) { return f; }
+PTO_DEV i32x8 mx_operand(u32x4 f) { return i32x8{(int)f[0], (int)f[1], (int)f[2], (int)f[3], 0, 0, 0, 0}; }
 
 template <bool kZeroInit, typename AccT, typename LeftT, typename LeftScaleT, typename RightT, typename RightScaleT>
 PTO_DEV void mad_mx(AccT &out, const AccT &in, const LeftT &a, const LeftScaleT &sa, const RightT &b, const RightScaleT &sb)
 {
-    static_assert(is_mx8_v<typename LeftT::DType> && is_mx8_v<typename RightT::DType> && std::is_same_v<typename AccT::DType, float>,
-                  "[PTO][SA] TMATMUL_MX on gfx950: fp8 (e4m3 / e5m2) operands, fp32 accumulator");
+    static_assert(is_mx_operand_v<typename LeftT::DType> && is_mx_operand_v<typename RightT::DType> &&
+                      std::is_same_v<typename AccT::DType, float>,
+                  "[PTO][SA] TMATMUL_MX on gfx950: fp8 (e4m3 / e5m2) or fp4 (e2m1) operands, fp32 accumulator");
     static_assert(LeftT::Loc == TileType::Left && RightT::Loc == TileType::Right && AccT::Loc == TileType::Acc &&
                       LeftScaleT::Loc == TileType::ScaleLeft && RightScaleT::Loc == TileType::ScaleRight,
                   "[PTO][SA] TMATMUL_MX: operands must be Left, ScaleLeft, Right, ScaleRight and Acc tiles");
@@ -130,11 +135,11 @@ PTO_DEV void mad_mx(AccT &out, const AccT &in, const LeftT &a, const LeftScaleT 
             for (int ks = 0; ks < SL::KS; ++ks) {
                 // k step ks: scale byte 0 (even step) or 2 (odd step) of register ks / 2
                 if (ks % 2 == 0)
-                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a.st.f[mb][ks], b.st.f[nb][ks], c, fa, fb, 0,
-                                                                        (int)sa.st.s[mb][ks / 2], 0, (int)sb.st.s[nb][ks / 2]);
+                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(mx_operand(a.st.f[mb][ks]), mx_operand(b.st.f[nb][ks]), c, fa, fb,
+                                                                        0, (int)sa.st.s[mb][ks / 2], 0, (int)sb.st.s[nb][ks / 2]);
                 else
-                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a.st.f[mb][ks], b.st.f[nb][ks], c, fa, fb, 2,
-                                                                        (int)sa.st.s[mb][ks / 2], 2, (int)sb.st.s[nb][ks / 2]);
+                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(mx_operand(a.st.f[mb][ks]), mx_operand(b.st.f[nb][ks]), c, fa, fb,
+                                                                        2, (int)sa.st.s[mb][ks / 2], 2, (int)sb.st.s[nb][ks / 2]);
             }
             out.st.f[mb][nb] = c;
         }

@@ -6,7 +6,7 @@
 // placement is the one described in common/tile.hpp.
 //
 // Mat tile LDS image.  Let `major` index the non-contiguous logical dimension and k the
-// contiguous one (k = column for an Nz tile, row for a Zn tile), RowBytes = extent_k * sizeof(T).
+// contiguous one (k = column for an Nz tile, row for a Zn tile), RowBytes = extent_k * sizeof(T) (extent_k / 2 for 4-bit elements).
 // Element (major, k) lives at   major*RowBytes + ((chunk ^ swz(major)) << 4) + (k*sizeof(T) & 15),
 // chunk = k*sizeof(T) >> 4.  swz() spreads consecutive `major` values at the same logical chunk over the
 // 16-byte bank groups so that the ds_read_b128 fragment reads are conflict free (checked with the LDS
@@ -50,7 +50,7 @@ struct MatGeom {
     static constexpr bool colsK = TileT::colsContiguous;
     static constexpr int Major = colsK ? TileT::Rows : TileT::Cols;
     static constexpr int KExt = colsK ? TileT::Cols : TileT::Rows;
-    static constexpr int RowBytes = KExt * (int)sizeof(T);
+    static constexpr int RowBytes = KExt * elem_bits<T> / 8;
     static constexpr int ChunksPerRow = RowBytes / 16;
     static constexpr int Bytes = Major * RowBytes;
     static_assert(RowBytes % 16 == 0, "[PTO][SA] Mat tile: contiguous extent must be a multiple of 16 bytes");
@@ -58,7 +58,7 @@ struct MatGeom {
     PTO_DEV static uint32_t elem_off(uint32_t r, uint32_t c)
     {
         const uint32_t major = colsK ? r : c, k = colsK ? c : r;
-        const uint32_t kb = k * sizeof(T);
+        const uint32_t kb = k * elem_bits<T> / 8;
         return mat_chunk_off<RowBytes>(major, kb >> 4) + (kb & 15u);
     }
 };
@@ -144,7 +144,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
     constexpr bool fullValid = TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols;
     constexpr bool staticUnit = Geo::colsK ? (G::staticStride[4] == 1) : (G::staticStride[3] == 1);
     if constexpr (fullValid && staticUnit) {
-        const int64_t ld = Geo::colsK ? st_r : st_c;
+        const int64_t ld = (Geo::colsK ? st_r : st_c) * elem_bits<T> / 8; // bytes between consecutive rows (columns) in memory
         constexpr int total = Geo::Major * Geo::ChunksPerRow; // 16-byte chunks
         constexpr int perWaveInst = kWaveSize;
         constexpr int nInst = cdiv(total, perWaveInst);
@@ -159,7 +159,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             // around the TLOAD only has to advance with scalar arithmetic.
             const uint32_t major0 = (uint32_t)wave * rpi + (uint32_t)lane / cpr, cpos = (uint32_t)lane % cpr;
             const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major0);
-            const uint32_t laneOff = (major0 * (uint32_t)ld + chunk * (16 / sizeof(T))) * (uint32_t)sizeof(T);
+            const uint32_t laneOff = major0 * (uint32_t)ld + chunk * 16;
             const char *base = reinterpret_cast<const char *>(gm);
             constexpr int first = SLICE < 0 ? 0 : SLICE * kBlockWaves, last = SLICE < 0 ? nInst : first + kBlockWaves;
             static_assert(last <= nInst, "[PTO][SA] TLOAD slice: the tile has fewer copy instructions");
@@ -170,7 +170,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
                 // of the round before (same data to the same place): every wave then issues TLoadInstrs<TileT>()
                 // copies, which keeps the vmcnt bookkeeping of software pipelines uniform and the code branch-free.
                 const int s0e = (nInst % kBlockWaves != 0 && s0 + wave >= nInst) ? s0 - kBlockWaves : s0;
-                const char *g = uniform_ptr(base + (int64_t)(s0e * rpi) * ld * (int64_t)sizeof(T)) + laneOff;
+                const char *g = uniform_ptr(base + (int64_t)(s0e * rpi) * ld) + laneOff;
                 __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + (s0e + wave) * (perWaveInst * 16)), 16, 0, 0);
             }
         } else {
@@ -183,13 +183,14 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
                 if ((evenInst || s < nInst) && (evenTotal || q < (uint32_t)total)) {
                     const uint32_t major = q / Geo::ChunksPerRow, cpos = q % Geo::ChunksPerRow;
                     const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major);
-                    const T *g = gm + (int64_t)major * ld + chunk * (16 / sizeof(T));
+                    const char *g = reinterpret_cast<const char *>(gm) + (int64_t)major * ld + chunk * 16;
                     __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + s * (perWaveInst * 16)), 16, 0, 0);
                 }
             }
         }
     } else {
         static_assert(SLICE < 0, "[PTO][SA] TLOAD slice: only for fully valid, unit-stride Mat tiles");
+        static_assert(elem_bits<T> >= 8, "[PTO][SA] TLOAD of 4-bit elements: fully valid, unit-stride Mat tiles only");
         // general path: element by element, pad outside the valid region (TLoad.hpp:151-152)
         const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
         const T pad = pad_value<T>(TileT::PadVal);
@@ -337,8 +338,9 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 // MFMA operand layout (lane l: row/col l % kMfmaM, k = 8*(l / kMfmaM)..+7).
 // The k offset must be a multiple of 8 elements (16 bytes).
 namespace detail {
-// Mat -> Left / Right of an 8-bit MX operand: two ds_read_b128 per 32-row block and 64-wide k step (lane l: row
-// l % 32, bytes 16 (l / 32) .. +15 and 32 + 16 (l / 32) .. +15 of the step).  The k offset must be a multiple of 64.
+// Mat -> Left / Right of an MX operand.  8-bit: two ds_read_b128 per 32-row block and 64-wide k step (lane l: row
+// l % 32, bytes 16 (l / 32) .. +15 and 32 + 16 (l / 32) .. +15 of the step).  4-bit: one ds_read_b128 (bytes
+// 16 (l / 32) .. +15 of the step's 32).  The k offset must be a multiple of 64.
 template <typename DstT, typename SrcT>
 PTO_DEV void textract_mx(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol)
 {
@@ -350,14 +352,19 @@ PTO_DEV void textract_mx(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol)
     const uint32_t lane = (uint32_t)hw::lane();
     constexpr int blocks = S::Blocks;
     const uint32_t major0 = (left ? idxRow : idxCol) + (uint32_t)(left ? hw::wave_m() : hw::wave_n()) * (blocks * kMxM) + lane % kMxM;
-    const uint32_t chunk0 = ((left ? idxCol : idxRow) >> 4) + lane / kMxM;
+    using T = typename DstT::DType;
+    const uint32_t chunk0 = (((left ? idxCol : idxRow) * elem_bits<T> / 8) >> 4) + lane / kMxM;
 #pragma unroll
     for (int b = 0; b < blocks; ++b)
 #pragma unroll
         for (int ks = 0; ks < S::KS; ++ks) {
-            const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4));
-            const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4 + 2));
-            dst.st.f[b][ks] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            if constexpr (is_mx4_v<T>) {
+                dst.st.f[b][ks] = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 2));
+            } else {
+                const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4));
+                const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4 + 2));
+                dst.st.f[b][ks] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            }
         }
 }
 
@@ -468,8 +475,9 @@ PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t i
             detail::textract_scale(dst, src, left ? idxCol : idxRow);
         }
         return;
-    } else if constexpr (detail::is_mx8_v<typename DstT::DType>) {
-        static_assert(SrcT::Loc == TileType::Mat && sizeof(typename SrcT::DType) == 1, "[PTO][SA] TEXTRACT: 8-bit Mat source");
+    } else if constexpr (detail::is_mx_operand_v<typename DstT::DType>) {
+        static_assert(SrcT::Loc == TileType::Mat && std::is_same_v<typename SrcT::DType, typename DstT::DType>,
+                      "[PTO][SA] TEXTRACT: Mat source of the same element type");
         detail::textract_mx(dst, src, idxRow, idxCol);
         return;
     } else {

@@ -57,9 +57,16 @@ int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b
  * a [m,k] and b stored [n,k] (a column-major k x n operand) hold 8-bit floats: format 0 = e4m3 (OCP, no infinities),
  * 1 = e5m2, the same for both operands.  scale_a [m,k/32] and scale_b stored [n,k/32] hold one e8m0 exponent per row
  * (column) and 32 consecutive k (the reference's x1_gm / x2_gm / x1_scale_gm / x2_scale_gm files).  c: bf16
- * (c_fp32 == 0, round-to-nearest-even of the fp32 sum) or fp32.  m % 256 == 0, n % 256 == 0, k % 512 == 0. */
+ * (c_fp32 == 0, round-to-nearest-even of the fp32 sum) or fp32.  m >= 256, n >= 256 (any value: the last tile row /
+ * column is moved back to end at m / n and recomputes what it overlaps), k % 512 == 0. */
 int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
                    int m, int n, int k, int format, int c_fp32);
+
+/* MXFP4 GEMM: as pto_gemm_mxfp8 with 4-bit e2m1 operands packed two per byte, element 2i in bits 0-3 (the reference's
+ * pack_two_fp4): a [m,k/2] bytes, b stored [n,k/2] bytes (LaunchMxMatmul of
+ * kernels/manual/a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp).  Same limits. */
+int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
+                   int m, int n, int k, int c_fp32);
 
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];

@@ -69,6 +69,8 @@ def lib():
         L.po_fp8_e4m3fn_to_f32.restype = C.c_float
         L.po_fp8_e5m2_to_f32.argtypes = [C.c_uint8]
         L.po_fp8_e5m2_to_f32.restype = C.c_float
+        L.po_fp4_e2m1_to_f32.argtypes = [C.c_uint8]
+        L.po_fp4_e2m1_to_f32.restype = C.c_float
         L.po_fa_auto_f32.argtypes = [C.c_void_p] * 4 + [C.c_int] * 3
         L.po_fa_auto_f32.restype = None
         L.po_fa_stream_f16.argtypes = [C.c_void_p] * 6 + [C.c_int] * 8
@@ -182,19 +184,23 @@ def gemm_f16f32(A, B, base_k=64, row0=0, row1=0, threads=0):
 
 
 def fp8_table(fmt):
-    """All 256 values of float8_e4m3fn (fmt 0) or float8_e5m2 (fmt 1) as float32."""
+    """All 256 values of float8_e4m3fn (fmt 0) or float8_e5m2 (fmt 1), or the 16 of float4_e2m1 (fmt 4), as float32."""
+    if fmt == 4:
+        return np.array([lib().po_fp4_e2m1_to_f32(v) for v in range(16)], dtype=np.float32)
     f = lib().po_fp8_e5m2_to_f32 if fmt else lib().po_fp8_e4m3fn_to_f32
     return np.array([f(v) for v in range(256)], dtype=np.float32)
 
 
 def mx_gemm(A, B, SA, SB, fmt_a=0, fmt_b=None, threads=0):
-    """A [m,k] uint8 fp8, B [n,k] uint8 fp8, SA [m,k/32], SB [n,k/32] uint8 e8m0 -> C [m,n] fp32 (float64 accumulation)."""
+    """A [m,k] uint8 fp8 (or [m,k/2] packed fp4, fmt 4), B [n,k] likewise, SA [m,k/32], SB [n,k/32] uint8 e8m0
+    -> C [m,n] fp32 (float64 accumulation)."""
     A, B, SA, SB = (np.ascontiguousarray(x, dtype=np.uint8) for x in (A, B, SA, SB))
-    m, k = A.shape
+    fmt_b = fmt_a if fmt_b is None else fmt_b
+    m, k = A.shape[0], A.shape[1] * (2 if fmt_a == 4 else 1)
     n = B.shape[0]
-    assert B.shape[1] == k and k % 32 == 0 and SA.shape == (m, k // 32) and SB.shape == (n, k // 32)
+    assert B.shape[1] * (2 if fmt_b == 4 else 1) == k and k % 32 == 0 and SA.shape == (m, k // 32) and SB.shape == (n, k // 32)
     Cm = np.empty((m, n), dtype=np.float32)
-    lib().po_mx_gemm(_p(Cm), _p(A), _p(B), _p(SA), _p(SB), m, n, k, fmt_a, fmt_a if fmt_b is None else fmt_b, threads)
+    lib().po_mx_gemm(_p(Cm), _p(A), _p(B), _p(SA), _p(SB), m, n, k, fmt_a, fmt_b, threads)
     return Cm
 
 

@@ -530,6 +530,14 @@ float po_fp8_e5m2_to_f32(uint8_t v)
     return s ? -r : r;
 }
 
+/* float4_e2m1: 1-2-1, bias 1, no infinities or NaNs: 0, 0.5 (subnormal), 1, 1.5, 2, 3, 4, 6 */
+float po_fp4_e2m1_to_f32(uint8_t nibble)
+{
+    const int s = (nibble >> 3) & 1, e = (nibble >> 1) & 3, f = nibble & 1;
+    const float r = e == 0 ? 0.5f * (float)f : ldexpf((float)(2 + f), e - 2);
+    return s ? -r : r;
+}
+
 typedef struct {
     float *C;
     const double *A, *B; /* dequantised operands, A [m,k], B [n,k] */
@@ -555,8 +563,14 @@ static double *po_mx_dequant(const uint8_t *X, const uint8_t *S, int rows, int k
     const int kb = k / 32;
     for (int r = 0; r < rows; r++)
         for (int kk = 0; kk < k; kk++) {
-            const uint8_t v = X[(size_t)r * (size_t)k + (size_t)kk];
-            const double e = format ? (double)po_fp8_e5m2_to_f32(v) : (double)po_fp8_e4m3fn_to_f32(v);
+            double e;
+            if (format == 4) {
+                const uint8_t pair = X[((size_t)r * (size_t)k + (size_t)kk) / 2];
+                e = (double)po_fp4_e2m1_to_f32((uint8_t)((kk & 1) ? pair >> 4 : pair & 15));
+            } else {
+                const uint8_t v = X[(size_t)r * (size_t)k + (size_t)kk];
+                e = format ? (double)po_fp8_e5m2_to_f32(v) : (double)po_fp8_e4m3fn_to_f32(v);
+            }
             out[(size_t)r * (size_t)k + (size_t)kk] = e * ldexp(1.0, (int)S[(size_t)r * (size_t)kb + (size_t)(kk / 32)] - 127);
         }
     return out;

@@ -94,9 +94,12 @@ void po_gemm_f16f32(float *C, const uint16_t *A, const uint16_t *B, int m, int n
  * (tests/npu/a5/src/st/testcase/tmatmul_mx/gen_data.py:130-171, kernels/manual/a5/matmul_mxfp8_performance/scripts/gen_data.py:31-50):
  * x1[i,kk] = fp8(A[i,kk]) * 2^(SA[i,kk/32] - 127), x2[kk,j] = fp8(B[j,kk]) * 2^(SB[j,kk/32] - 127),
  * C = matmul in float64 -> float32.  A [m,k], B stored [n,k], SA [m,k/32], SB stored [n,k/32] (the generator's
- * transposed x2 / x2_scale files).  format: 0 = float8_e4m3fn, 1 = float8_e5m2 (ml_dtypes' names). */
+ * transposed x2 / x2_scale files).  format: 0 = float8_e4m3fn, 1 = float8_e5m2 (ml_dtypes' names), 4 = float4_e2m1
+ * packed two per byte, element 2i in the low nibble (pack_two_fp4, tmatmul_mx/gen_data.py:74-84; the operand then has
+ * k/2 bytes per row). */
 float po_fp8_e4m3fn_to_f32(uint8_t v);
 float po_fp8_e5m2_to_f32(uint8_t v);
+float po_fp4_e2m1_to_f32(uint8_t nibble);
 void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, int m, int n, int k,
                 int format_a, int format_b, int threads);
 

@@ -1,9 +1,11 @@
-// MXFP8 GEMM for MI355X: C[m,n] = (A .* 2^(scaleA-127)) x (B .* 2^(scaleB-127)), fp8 (e4m3 / e5m2) operands with one
-// e8m0 scale per row (column) and 32-wide k block, fp32 accumulation, bf16 or fp32 result.
+// MXFP8 / MXFP4 GEMM for MI355X: C[m,n] = (A .* 2^(scaleA-127)) x (B .* 2^(scaleB-127)), fp8 (e4m3 / e5m2) or fp4
+// (e2m1, two per byte) operands with one e8m0 scale per row (column) and 32-wide k block, fp32 accumulation, bf16 or
+// fp32 result.
 //
-// Mirrors the reference kernel kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:149-241
-// (TLOAD of operand and scale panels -> TEXTRACT -> TMATMUL_MX -> TSTORE): A [m,k], B stored [n,k], scaleA [m,k/32],
-// scaleB stored [n,k/32] (scripts/gen_data.py:31-66).
+// Mirrors the reference kernels kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:149-241 and
+// kernels/manual/a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp (TLOAD of operand and scale panels ->
+// TEXTRACT -> TMATMUL_MX -> TSTORE): A [m,k], B stored [n,k], scaleA [m,k/32], scaleB stored [n,k/32]
+// (scripts/gen_data.py:31-66).
 //
 // Structure: the fp16 GEMM's K-step pipeline (workgroup tile 256 x 256, 8 waves in a 2 x 4 grid, four LDS stages of
 // one 64-byte K-step filled by asynchronous copies, copies / fragment reads / MFMAs interleaved by the scheduler
@@ -12,6 +14,10 @@
 // bytes moved per MFMA cycle are those of the fp16 kernel at twice the flops.  The scales of 512 k (16 blocks = 16
 // bytes per row) are copied into LDS once per eight K-steps (two buffers) and the two scales a lane needs for a K-step
 // are read with the step's fragments (one ds_read_u8 per 32-row block); the MFMA applies them.
+// fp4: a 64-byte K-step holds 128 k = two MFMAs (8 passes each) per fragment pair and four scale blocks (one ds_read_b32
+// per 32-row block); a scale group is four K-steps.  Same bytes per step again, at four times the fp16 flops.
+// m and n need not be multiples of the tile: the last tile row / column is moved back to end at m / n and recomputes
+// what it overlaps (m, n >= 256).
 #define PTO_WAVES_M 2
 #define PTO_WAVES_N 4
 #include "gemm_kernels.hpp"
@@ -20,7 +26,10 @@ PTO_DEVICE_CODE_BEGIN
 
 namespace {
 
-constexpr int kMxGroupSteps = 8; // K-steps (of 64) per scale group: 16 k blocks = one 16-byte scale row
+constexpr int kMxStepBytes = 64; // one K-step per operand row in LDS
+// K-steps per scale group (16 k blocks = one 16-byte scale row): 8 steps of 64 k (8-bit) or 4 steps of 128 k (4-bit)
+template <typename T>
+constexpr int kMxGroupSteps = 16 / (kMxStepBytes * 8 / detail::elem_bits<T> / 32);
 
 // One asynchronous copy instruction per wave: the 16-byte scale rows of the workgroup's BM rows of A and BN columns
 // of B for one scale group -> LDS [BM + BN][16 bytes] (the images of an unboxed [BM, 16] row-major and a [16, BN]
@@ -44,7 +53,10 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
                                                              __gm__ const uint8_t *scale0, __gm__ const uint8_t *scale1, int m,
                                                              int n, int k, int row0, int col0)
 {
-    constexpr int BK = 64, HM = BM / 2, KB = 2 * kMxGroupSteps;
+    static_assert(detail::elem_bits<FA> == detail::elem_bits<FB>, "operands of one width");
+    constexpr int BK = kMxStepBytes * 8 / detail::elem_bits<FA>; // k per K-step
+    constexpr int kGroupSteps = kMxGroupSteps<FA>, kStepBlocks = BK / 32;
+    constexpr int HM = BM / 2, KB = 16;
     using X = float8_e8m0_t;
     using TileMatA = Tile<TileType::Mat, FA, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
     using TileMatB = Tile<TileType::Mat, FB, BK, BN, BLayout::RowMajor, BK, BN, SLayout::ColMajor>;
@@ -52,8 +64,8 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
     using TileScaleB = Tile<TileType::Mat, X, KB, BN, BLayout::ColMajor, KB, BN, SLayout::NoneBox>;
     using LeftHalf = TileLeft<FA, HM, BK, HM, BK>;
     using RightTile = TileRight<FB, BK, BN, BK, BN>;
-    using LeftScaleStep = TileLeftScale<X, HM, 2>;
-    using RightScaleStep = TileRightScale<X, 2, BN>;
+    using LeftScaleStep = TileLeftScale<X, HM, kStepBlocks>;
+    using RightScaleStep = TileRightScale<X, kStepBlocks, BN>;
     using AccHalf = TileAcc<float, HM, BN, HM, BN>;
     using ShapeA = TileShape2D<FA, BM, BK, Layout::ND>;
     using StrideA = BaseShape2D<FA, DYNAMIC, DYNAMIC, Layout::ND>;
@@ -65,11 +77,11 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
     using StrideC = BaseShape2D<OutT, DYNAMIC, DYNAMIC, Layout::ND>;
     using GlobalC = GlobalTensor<OutT, ShapeC, StrideC, Layout::ND>;
 
-    constexpr uint32_t kABytes = BM * BK, kBBytes = BK * BN;
+    constexpr uint32_t kABytes = BM * kMxStepBytes, kBBytes = kMxStepBytes * BN;
     constexpr uint32_t kStage = kABytes + kBBytes;
     constexpr uint32_t kScaleOff = STAGES * kStage, kScaleBytes = (BM + BN) * 16; // two buffers of [BM + BN][16] scale rows
     constexpr int kLoadsPerStep = TLoadInstrs<TileMatA>() + TLoadInstrs<TileMatB>();
-    constexpr int kMfma = 2 * AccHalf::Storage::MB * AccHalf::Storage::NB;
+    constexpr int kMfma = 2 * AccHalf::Storage::MB * AccHalf::Storage::NB * LeftHalf::Storage::KS;
     constexpr int kReadsA = 2 * LeftHalf::Storage::MB, kReadsB = 2 * RightTile::Storage::NB; // two ds_read_b128 per fragment
     constexpr int kReads = 2 * kReadsA + kReadsB + (2 * LeftHalf::Storage::MB + RightTile::Storage::NB); // + the scale reads
     // issue pattern of a step: the copies first, one MFMA before each; the fragment reads spread over the next MFMAs;
@@ -79,14 +91,15 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
     static_assert(STAGES == 4, "two fragment sets alternate with the stage index");
     static_assert(kMfmaForReads >= 0, "issue pattern below");
 
-    __gm__ FA *aPanel = const_cast<FA *>(src0) + (int64_t)row0 * k;
-    __gm__ FB *bPanel = const_cast<FB *>(src1) + (int64_t)col0 * k;
+    // (operand pointers advance in bytes: one byte per 8-bit element, two 4-bit elements per byte)
+    __gm__ FA *aPanel = const_cast<FA *>(src0) + (int64_t)row0 * k * detail::elem_bits<FA> / 8;
+    __gm__ FB *bPanel = const_cast<FB *>(src1) + (int64_t)col0 * k * detail::elem_bits<FB> / 8;
     const int64_t ldScale = k / 32;
     __gm__ const uint8_t *saPanel = scale0 + (int64_t)row0 * ldScale;
     __gm__ const uint8_t *sbPanel = scale1 + (int64_t)col0 * ldScale;
     const StrideA strideA(m, k);
     const StrideB strideB(k, n);
-    const int kLoop = k / BK, groups = kLoop / kMxGroupSteps;
+    const int kLoop = k / BK, groups = kLoop / kGroupSteps;
 
     TileMatA aMat[STAGES];
     TileMatB bMat[STAGES];
@@ -122,8 +135,8 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
     LoadScaleGroup<BM, BN>(kScaleOff, saPanel, sbPanel, ldScale);
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) {
-        GlobalA gmA(aPanel + (int64_t)s * BK, ShapeA(), strideA);
-        GlobalB gmB(bPanel + (int64_t)s * BK, ShapeB(), strideB);
+        GlobalA gmA(aPanel + (int64_t)s * kMxStepBytes, ShapeA(), strideA);
+        GlobalB gmB(bPanel + (int64_t)s * kMxStepBytes, ShapeB(), strideB);
         TLOAD(aMat[s], gmA);
         TLOAD(bMat[s], gmB);
     }
@@ -154,16 +167,16 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
             LoadScaleGroup<BM, BN>(otherBuf, saPanel + g * 16, sbPanel + g * 16, ldScale);
             __builtin_amdgcn_sched_barrier(0);
         }
-        if constexpr (j == kMxGroupSteps - 1) { // the next step is the first of the next group
+        if constexpr (j == kGroupSteps - 1) { // the next step is the first of the next group
             TASSIGN(aScaleMat, otherBuf);
             TASSIGN(bScaleMat, otherBuf + BM * 16);
         }
         const int fetch = it + STAGES - 1 < kLoop ? it + STAGES - 1 : kLoop - 1;
-        GlobalA gmA(aPanel + (int64_t)fetch * BK, ShapeA(), strideA);
-        GlobalB gmB(bPanel + (int64_t)fetch * BK, ShapeB(), strideB);
+        GlobalA gmA(aPanel + (int64_t)fetch * kMxStepBytes, ShapeA(), strideA);
+        GlobalB gmB(bPanel + (int64_t)fetch * kMxStepBytes, ShapeB(), strideB);
         TLOAD(aMat[sLoad], gmA);
         TLOAD(bMat[sLoad], gmB);
-        constexpr int p = j & 1, q = p ^ 1, kbNext = 2 * ((j + 1) % kMxGroupSteps);
+        constexpr int p = j & 1, q = p ^ 1, kbNext = kStepBlocks * ((j + 1) % kGroupSteps);
         TMATMUL_MX(cUp, cUp, aUp, saUp, bAll[p], sbAll[p]);
         TEXTRACT(aUp, aMat[sNext], 0, 0);
         TEXTRACT(saUp, aScaleMat, 0, +kbNext);
@@ -188,17 +201,10 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
         __builtin_amdgcn_sched_group_barrier(0x008, kMfmaTail, 0);
         __builtin_amdgcn_sched_barrier(0);
     };
-    using std::integral_constant;
+    static_assert(kGroupSteps % STAGES == 0, "the LDS stage of a step is a compile-time constant");
     for (int group = 0; group < groups; ++group) {
-        const int it = group * kMxGroupSteps;
-        step(integral_constant<int, 0>(), it, group);
-        step(integral_constant<int, 1>(), it + 1, group);
-        step(integral_constant<int, 2>(), it + 2, group);
-        step(integral_constant<int, 3>(), it + 3, group);
-        step(integral_constant<int, 4>(), it + 4, group);
-        step(integral_constant<int, 5>(), it + 5, group);
-        step(integral_constant<int, 6>(), it + 6, group);
-        step(integral_constant<int, 7>(), it + 7, group);
+        const int it = group * kGroupSteps;
+        StaticFor<0, kGroupSteps>([&](auto jTag) { step(jTag, it + decltype(jTag)::value, group); });
     }
     hw::wait_vm0(); // the copies issued past the end of K must not outlive the workgroup's LDS
     GlobalC dstUp(out + (int64_t)row0 * n + col0, ShapeC(), StrideC(m, n));
@@ -214,10 +220,10 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     void GemmMx(__gm__ OutT *out, __gm__ const FA *src0, __gm__ const FB *src1, __gm__ const uint8_t *scale0,
                 __gm__ const uint8_t *scale1, int m, int n, int k, int fullTiles)
 {
-    const int tilesM = m / BM, tilesN = n / BN;
+    const int tilesM = (m + BM - 1) / BM, tilesN = (n + BN - 1) / BN;
     const int block = (int)get_block_idx();
     int tm, tn;
-    if (block >= fullTiles) {
+    if (block >= fullTiles) { // (only when m and n are multiples of the tile)
         const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
         TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
         const int sub = u % 4;
@@ -226,7 +232,9 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         return;
     }
     TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
-    MxTileRows<FA, FB, OutT, BM, BN, STAGES>(out, src0, src1, scale0, scale1, m, n, k, tm * BM, tn * BN);
+    // the last tile row / column ends at m / n: it recomputes the rows / columns it shares with its neighbour
+    const int row0 = tm * BM + BM <= m ? tm * BM : m - BM, col0 = tn * BN + BN <= n ? tn * BN : n - BN;
+    MxTileRows<FA, FB, OutT, BM, BN, STAGES>(out, src0, src1, scale0, scale1, m, n, k, row0, col0);
 }
 
 } // namespace
@@ -240,17 +248,17 @@ int launch_gemm_mx(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, 
                    int k, int tailMode)
 {
     constexpr int BM = 256, BN = 256, STAGES = 4, GROUP_M = 4;
-    if (m % BM || n % BN || k % (64 * kMxGroupSteps))
+    if (m < BM || n < BN || k % 512) // 512 k = one 16-byte scale row in either operand width
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = STAGES * (BM + BN) * 64 + 2 * (BM + BN) * 16;
     auto kernel = GemmMx<FA, FB, OutT, BM, BN, STAGES, GROUP_M>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
-    const int tiles = (m / BM) * (n / BN), cus = compute_units();
+    const int tiles = ((m + BM - 1) / BM) * ((n + BN - 1) / BN), cus = compute_units();
     int full = tiles / cus * cus;
     // quarter tiles move twice the operand bytes per flop: only when they fit one round
-    if (tailMode == 0 || full == 0 || (tiles - full) * 4 > cus)
+    if (tailMode == 0 || full == 0 || (tiles - full) * 4 > cus || m % BM || n % BN)
         full = tiles;
     kernel<<<dim3(full + (tiles - full) * 4), dim3(kBlockThreads), lds, st>>>(
         reinterpret_cast<OutT *>(c), reinterpret_cast<const FA *>(a), reinterpret_cast<const FB *>(b), sa, sb, m, n, k, full);
@@ -266,6 +274,9 @@ int gemm_mx_dispatch(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b
     if (format == 1)
         return c_fp32 ? launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
                         launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
+    if (format == 4)
+        return c_fp32 ? launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
     return PTO_ERR_UNSUPPORTED;
 }
 
@@ -276,10 +287,21 @@ extern "C" int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uin
 {
     if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0)
         return PTO_ERR_BAD_ARG;
+    if (format != 0 && format != 1)
+        return PTO_ERR_UNSUPPORTED;
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 1);
 }
 
-// Tuning hook (not part of the public header): variant 0 = whole tiles only, 1 = quarter tiles in the last round.
+extern "C" int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
+                              const uint8_t *scale_b, int m, int n, int k, int c_fp32)
+{
+    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0)
+        return PTO_ERR_BAD_ARG;
+    return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, 4, c_fp32, 1);
+}
+
+// Tuning hook (not part of the public header): variant 0 = whole tiles only, 1 = quarter tiles in the last round;
+// format 0 / 1 = fp8 e4m3 / e5m2, 4 = fp4 e2m1.
 extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                                       const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant)
 {

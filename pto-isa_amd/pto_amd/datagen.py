@@ -85,10 +85,31 @@ def fp8_values(fmt):
     return s * mag
 
 
+def fp4_values():
+    """The 16 values of float4_e2m1 (1-2-1, bias 1: 0, 0.5, 1, 1.5, 2, 3, 4, 6 and their negatives) indexed by the nibble."""
+    mag = np.array([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+    return np.concatenate([mag, -mag])
+
+
+def fp4_pack(nibbles):
+    """[rows, k] nibbles -> [rows, k/2] bytes, element 2i in the low half (pack_two_fp4, tmatmul_mx/gen_data.py:74-84)."""
+    nib = np.asarray(nibbles, dtype=np.uint8)
+    return (nib[:, 0::2] & 15) | ((nib[:, 1::2] & 15) << 4)
+
+
+def fp4_unpack(packed):
+    p = np.asarray(packed, dtype=np.uint8)
+    out = np.empty((p.shape[0], p.shape[1] * 2), dtype=np.uint8)
+    out[:, 0::2] = p & 15
+    out[:, 1::2] = p >> 4
+    return out
+
+
 def fp8_encode(x, fmt):
-    """float array -> fp8 bytes, nearest finite value (saturating); a tie takes the value with the lower byte."""
-    tab = fp8_values(fmt)
-    finite = np.flatnonzero(np.isfinite(tab) & ~((np.arange(256) == 0x80)))      # one zero: +0
+    """float array -> fp8 bytes (fmt 0 / 1) or fp4 nibbles (fmt 4), nearest finite value (saturating); a tie takes the
+    lower value."""
+    tab = fp4_values() if fmt == 4 else fp8_values(fmt)
+    finite = np.flatnonzero(np.isfinite(tab) & ~((np.arange(tab.size) == tab.size // 2)))      # one zero: +0
     order = finite[np.argsort(tab[finite], kind="stable")]
     vals = tab[order]
     x = np.asarray(x, dtype=np.float64)
@@ -99,13 +120,21 @@ def fp8_encode(x, fmt):
 
 
 def mx_inputs(m, n, k, fmt, dist="uniform", scale_lo=127, scale_hi=130):
-    """Operands of the MXFP8 GEMM: A [m,k], B [n,k] fp8 bytes, SA [m,k/32], SB [n,k/32] e8m0 bytes.
+    """Operands of the MX GEMMs: A [m,k], B [n,k] fp8 bytes (fmt 0 e4m3, 1 e5m2) or [m,k/2], [n,k/2] packed fp4 (fmt 4),
+    SA [m,k/32], SB [n,k/32] e8m0 bytes.  For fp4 "uniform" and "integer" draw integers in [-6, 6) as the reference's
+    generators do (matmul_mxfp4_performance/scripts/gen_data.py, tmatmul_mx/gen_data.py:108-111).
 
     dist "uniform": uniform(-5, 5) rounded to fp8 and scales in [127, 130), the distribution of
     kernels/manual/a5/matmul_mxfp8_performance/scripts/gen_data.py:31-38; "integer": integers in [-10, 10) as in
     tests/npu/a5/src/st/testcase/tmatmul_mx/gen_data.py:113-120; "bytes": every finite encoding, subnormals included."""
     ra, rb = _rng(SEED_MX_A), _rng(SEED_MX_B)
-    if dist == "uniform":
+    if fmt == 4:
+        if dist == "bytes":
+            a, b = ra.integers(0, 16, size=(m, k)), rb.integers(0, 16, size=(n, k))
+        else:
+            a, b = fp8_encode(ra.integers(-6, 6, size=(m, k)), 4), fp8_encode(rb.integers(-6, 6, size=(n, k)), 4)
+        a, b = fp4_pack(a), fp4_pack(b)
+    elif dist == "uniform":
         a = fp8_encode(ra.uniform(-5.0, 5.0, size=(m, k)), fmt)
         b = fp8_encode(rb.uniform(-5.0, 5.0, size=(n, k)), fmt)
     elif dist == "integer":

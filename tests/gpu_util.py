@@ -33,18 +33,22 @@ def gemm(a, b):
 
 
 def gemm_mx(a, b, sa, sb, fmt, c_fp32=True):
-    """a [m,k], b [n,k] fp8 bytes, sa [m,k/32], sb [n,k/32] e8m0 bytes -> C [m,n] through pto_gemm_mxfp8:
-    fp32 values (c_fp32) or the bf16 bit patterns as uint16."""
+    """a [m,k], b [n,k] fp8 bytes (fmt 0 / 1) or [m,k/2], [n,k/2] packed fp4 (fmt 4), sa [m,k/32], sb [n,k/32] e8m0 bytes
+    -> C [m,n] through pto_gemm_mxfp8 / pto_gemm_mxfp4: fp32 values (c_fp32) or the bf16 bit patterns as uint16."""
     lib = capi.load()
-    m, k = a.shape
+    m, k = a.shape[0], a.shape[1] * (2 if fmt == 4 else 1)
     n = b.shape[0]
     ta, tb, tsa, tsb = (to_dev(x) for x in (a, b, sa, sb))
     if c_fp32:
         tc = torch.full((m, n), float("nan"), dtype=torch.float32, device=DEV)
     else:
         tc = torch.full((m, n), -1, dtype=torch.int16, device=DEV)
-    capi.check(lib.pto_gemm_mxfp8(stream(), tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
-                                  m, n, k, fmt, int(c_fp32)), "pto_gemm_mxfp8")
+    if fmt == 4:
+        capi.check(lib.pto_gemm_mxfp4(stream(), tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                      m, n, k, int(c_fp32)), "pto_gemm_mxfp4")
+    else:
+        capi.check(lib.pto_gemm_mxfp8(stream(), tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                      m, n, k, fmt, int(c_fp32)), "pto_gemm_mxfp8")
     torch.cuda.synchronize()
     out = tc.cpu().numpy()
     return out if c_fp32 else out.view(np.uint16)

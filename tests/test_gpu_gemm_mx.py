@@ -1,4 +1,4 @@
-"""GPU parity of the MXFP8 GEMM (TLOAD -> TEXTRACT -> TMATMUL_MX -> TSTORE) through the C ABI.
+"""GPU parity of the MXFP8 / MXFP4 GEMMs (TLOAD -> TEXTRACT -> TMATMUL_MX -> TSTORE) through the C ABI.
 
 Reference: the oracle's float64 matmul of the dequantised operands (the golden of the reference's tmatmul_mx test
 and of its matmul_mxfp8_performance kernel).  Products of two scaled fp8 values are exact in fp32; the GPU adds them in
@@ -24,7 +24,7 @@ def bf16_rne(x):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 4])
 @pytest.mark.parametrize("m,n,k", [(256, 256, 512), (256, 512, 1024), (512, 256, 1536), (768, 768, 2048)])
 def test_mx_gemm_small_vs_oracle(oracle, m, n, k, fmt):
     from gpu_util import gemm_mx
@@ -37,7 +37,7 @@ def test_mx_gemm_small_vs_oracle(oracle, m, n, k, fmt):
     assert np.array_equal(got16, bf16_rne(got))
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 4])
 def test_mx_gemm_integer_operands_exact(oracle, fmt):
     """Integers in [-10, 10) (those fp8 can hold) and scales 2^0 .. 2^2: every partial sum is an integer below 2^24,
     exact in fp32 in any order, so a wrong fragment byte order, k-block / scale pairing or dropped step cannot hide."""
@@ -48,7 +48,7 @@ def test_mx_gemm_integer_operands_exact(oracle, fmt):
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 4])
 def test_mx_gemm_scale_of_every_block_is_applied(oracle, fmt):
     """Operands of all ones: C[i,j] = 32 * sum_kb 2^(sa[i,kb] + sb[j,kb] - 254), scales drawn from a wide range, so the
     result identifies which scale byte met which k block of which row and column."""
@@ -57,6 +57,8 @@ def test_mx_gemm_scale_of_every_block_is_applied(oracle, fmt):
     one = datagen.fp8_encode(np.ones(1), fmt)[0]
     a = np.full((m, k), one, dtype=np.uint8)
     b = np.full((n, k), one, dtype=np.uint8)
+    if fmt == 4:
+        a, b = datagen.fp4_pack(a), datagen.fp4_pack(b)
     _, _, sa, sb = datagen.mx_inputs(m, n, k, fmt, scale_lo=123, scale_hi=131)
     got = gemm_mx(a, b, sa, sb, fmt)
     want = 32.0 * (np.exp2(sa.astype(np.float64) - 127) @ np.exp2(sb.astype(np.float64) - 127).T)
@@ -69,7 +71,7 @@ def test_mx_gemm_scale_of_every_block_is_applied(oracle, fmt):
     assert np.max(np.abs(got - want) / want) <= 1e-5
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 4])
 def test_mx_gemm_every_encoding(oracle, fmt):
     """Random finite bytes (subnormals, both zeros, the largest values) and a wide range of scales."""
     from gpu_util import gemm_mx
@@ -92,6 +94,36 @@ def test_mx_gemm_quarter_tile_round(oracle):
     tab = datagen.fp8_values(1)
     bd = tab[b] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
     ad = tab[a] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
+    assert np.array_equal(got.astype(np.float64).sum(axis=1), ad @ bd.sum(axis=0))
+
+
+@pytest.mark.parametrize("fmt,m,n,k", [(1, 300, 700, 1024), (0, 257, 511, 512), (4, 1000, 260, 1024)])
+def test_mx_gemm_ragged_m_n(oracle, fmt, m, n, k):
+    """m, n that are not multiples of the 256 x 256 tile: the last tile row / column overlaps its neighbour."""
+    from gpu_util import gemm_mx
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt, dist="integer")
+    got = gemm_mx(a, b, sa, sb, fmt)
+    assert np.array_equal(got, oracle.mx_gemm(a, b, sa, sb, fmt))
+    got16 = gemm_mx(a, b, sa, sb, fmt, c_fp32=False)
+    assert np.array_equal(got16, bf16_rne(got))
+
+
+def test_mxfp4_gemm_reference_config_2040_8192_8100(oracle):
+    """The reference's matmul_mxfp4_performance case: e2m1 operands, m, k, n = 2040, 8192, 8100, bf16 result, its generator's
+    integer distribution in [-6, 6) and scales 2^0 .. 2^2: partial sums stay below 2^24, so the fp32 result is exact."""
+    from gpu_util import gemm_mx
+    m, k, n = 2040, 8192, 8100
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 4)
+    got = gemm_mx(a, b, sa, sb, 4)
+    rows = np.r_[0:24, 1000:1024, m - 24:m]
+    want = oracle.mx_gemm(a[rows], b, sa[rows], sb, 4)
+    assert np.array_equal(got[rows], want)
+    got16 = gemm_mx(a, b, sa, sb, 4, c_fp32=False)
+    assert np.array_equal(got16, bf16_rne(got))
+    # every row: row sums against (A dequantised) @ (column sums of B dequantised), exact in float64
+    tab = datagen.fp4_values()
+    bd = tab[datagen.fp4_unpack(b)] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
+    ad = tab[datagen.fp4_unpack(a)] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
     assert np.array_equal(got.astype(np.float64).sum(axis=1), ad @ bd.sum(axis=0))
 
 
@@ -132,7 +164,10 @@ def test_mx_gemm_rejects_bad_arguments():
     t = torch.zeros(16, device="cuda:0")
     p = t.data_ptr()
     assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 256, 256, 0, 1) == capi.ERR_UNSUPPORTED   # k % 512
-    assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 128, 256, 512, 0, 1) == capi.ERR_UNSUPPORTED   # m % 256
+    assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 128, 256, 512, 0, 1) == capi.ERR_UNSUPPORTED   # m < 256
+    assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 256, 512, 4, 1) == capi.ERR_UNSUPPORTED   # fp4 has its own entry point
+    assert lib.pto_gemm_mxfp4(0, p, p, p, p, p, 256, 256, 768, 1) == capi.ERR_UNSUPPORTED      # k % 512
+    assert lib.pto_gemm_mxfp4(0, p, 0, p, p, p, 256, 256, 512, 1) == capi.ERR_BAD_ARG
     assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 256, 512, 2, 1) == capi.ERR_UNSUPPORTED   # unknown format
     assert lib.pto_gemm_mxfp8(0, p, p, p, 0, p, 256, 256, 512, 0, 1) == capi.ERR_BAD_ARG
     assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 0, 512, 0, 1) == capi.ERR_BAD_ARG

@@ -524,3 +524,33 @@ def test_mx_gemm_oracle_closed_forms(oracle, fmt):
     ad = tab[a] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
     bd = tab[b] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
     assert np.allclose(oracle.mx_gemm(a, b, sa, sb, fmt), ad @ bd.T, rtol=1e-6, atol=1e-4)
+
+
+def test_fp4_decode_and_mx_gemm_oracle_fp4(oracle):
+    """float4_e2m1: the published value set (OCP MX: 0, 0.5, 1, 1.5, 2, 3, 4, 6), the bit-field formula, packing order, and
+    the oracle's fp4 GEMM against a float64 matmul of independently decoded operands."""
+    from pto_amd import datagen
+    want = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6, -0.0, -0.5, -1, -1.5, -2, -3, -4, -6], dtype=np.float32)
+    got = oracle.fp8_table(4)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    assert np.array_equal(datagen.fp4_values().astype(np.float32), want)
+    # formula: sign | 2-bit exponent (bias 1) | 1-bit mantissa, e = 0 subnormal
+    for v in range(16):
+        e, f = (v >> 1) & 3, v & 1
+        mag = 0.5 * f if e == 0 else (1 + f / 2) * 2.0 ** (e - 1)
+        assert abs(got[v]) == mag
+    nib = np.arange(64, dtype=np.uint8).reshape(2, 32) % 16
+    packed = datagen.fp4_pack(nib)
+    assert packed[0, 0] == (nib[0, 0] | (nib[0, 1] << 4)) and np.array_equal(datagen.fp4_unpack(packed), nib)
+    assert np.array_equal(datagen.fp8_encode(np.array([-6, -5, -1.2, 0, 0.2, 0.3, 2.4, 2.6, 5, 9]), 4),
+                          np.array([15, 15, 10, 0, 0, 1, 4, 5, 6, 7], dtype=np.uint8))
+    m, n, k = 16, 24, 128
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 4, dist="bytes", scale_lo=120, scale_hi=135)
+    assert a.shape == (m, k // 2)
+    ad = want.astype(np.float64)[datagen.fp4_unpack(a)] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
+    bd = want.astype(np.float64)[datagen.fp4_unpack(b)] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
+    assert np.allclose(oracle.mx_gemm(a, b, sa, sb, 4), ad @ bd.T, rtol=1e-6, atol=0)
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 4, dist="integer")
+    ad = want.astype(np.float64)[datagen.fp4_unpack(a)] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
+    bd = want.astype(np.float64)[datagen.fp4_unpack(b)] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
+    assert np.array_equal(oracle.mx_gemm(a, b, sa, sb, 4), (ad @ bd.T).astype(np.float32))
