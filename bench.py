@@ -21,6 +21,7 @@ for p in (ROOT, os.path.join(ROOT, "pto-isa_amd")):
 
 PEAK_FP16_TFLOPS = 2516.6   # MI355X dense fp16 matrix peak (published)
 PEAK_FP8_TFLOPS = 5033.2    # dense fp8 matrix peak (published)
+PEAK_FP4_TFLOPS = 10066.3   # dense fp4 matrix peak (published)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 
 # HBM-side traffic of one 6144^3 GEMM launch, from two rocprofv3 --pmc runs of this script
@@ -61,18 +62,23 @@ def bench_gemm(torch, lib, capi, datagen, size, steps, warmup):
     return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
 
 
-def bench_gemm_mx(torch, lib, capi, datagen, size, steps, warmup):
-    """MXFP8 GEMM of the reference's matmul_mxfp8_performance case: e5m2 operands, e8m0 block scales, bf16 result."""
-    a, b, sa, sb = datagen.mx_inputs(size, size, size, 1)
+def bench_gemm_mx(torch, lib, capi, datagen, m, n, k, fmt, steps, warmup):
+    """MX GEMMs of the reference's matmul_mxfp8_performance (fmt 1: e5m2) and matmul_mxfp4_performance (fmt 4: e2m1)
+    cases: e8m0 block scales, bf16 result."""
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt)
     ta, tb, tsa, tsb = (torch.from_numpy(x).cuda() for x in (a, b, sa, sb))
-    tc = torch.empty((size, size), dtype=torch.bfloat16, device="cuda")
+    tc = torch.empty((m, n), dtype=torch.bfloat16, device="cuda")
     st = torch.cuda.current_stream().cuda_stream
 
     def step():
-        capi.check(lib.pto_gemm_mxfp8(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
-                                      size, size, size, 1, 0), "gemm_mxfp8")
+        if fmt == 4:
+            capi.check(lib.pto_gemm_mxfp4(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                          m, n, k, 0), "gemm_mxfp4")
+        else:
+            capi.check(lib.pto_gemm_mxfp8(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                          m, n, k, fmt, 0), "gemm_mxfp8")
     ms = time_launches(torch, step, steps, warmup)
-    flops = 2.0 * size ** 3
+    flops = 2.0 * m * n * k
     return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
 
 
@@ -230,8 +236,13 @@ def main():
             r = bench_gemm(torch, lib, capi, datagen, s, max(args.steps // 2, 1), 2)
             extra["gemm_%d" % s] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp16_peak": r["tflops"] / PEAK_FP16_TFLOPS}
     if only in ("", "mx"):
-        r = bench_gemm_mx(torch, lib, capi, datagen, 6144, args.steps, args.warmup)
+        r = bench_gemm_mx(torch, lib, capi, datagen, 6144, 6144, 6144, 1, args.steps, args.warmup)
         extra["gemm_mxfp8_e5m2_bf16_6144"] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp8_peak": r["tflops"] / PEAK_FP8_TFLOPS}
+        r = bench_gemm_mx(torch, lib, capi, datagen, 2040, 8100, 8192, 4, args.steps, args.warmup)
+        extra["gemm_mxfp4_e2m1_bf16_m2040_k8192_n8100"] = {"ms": r["ms"], "tflops": r["tflops"],
+                                                           "frac_fp4_peak": r["tflops"] / PEAK_FP4_TFLOPS}
+        r = bench_gemm_mx(torch, lib, capi, datagen, 6144, 6144, 6144, 4, args.steps, args.warmup)
+        extra["gemm_mxfp4_e2m1_bf16_6144"] = {"ms": r["ms"], "tflops": r["tflops"], "frac_fp4_peak": r["tflops"] / PEAK_FP4_TFLOPS}
     if only in ("", "fa") and hasattr(lib, "pto_fa_fwd_f16"):
         for name, cfg in (("fa_b1_h16_s4096_d128", (1, 16, 4096, 128, False)),
                           ("fa_causal_b4_h32_s2048_d64", (4, 32, 2048, 64, True))):
