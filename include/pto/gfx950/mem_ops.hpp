@@ -275,13 +275,45 @@ PTO_DEV void TLOAD_SLICE(TileT &dst, G &src)
     detail::tload_mat<SLICE>(dst, src);
 }
 
-template <typename TileT>
-constexpr int TLoadInstrs()
-{
-    using Geo = detail::MatGeom<TileT>;
-    return detail::cdiv(detail::cdiv(Geo::Major * Geo::ChunksPerRow, kWaveSize), kBlockWaves);
-}
 namespace detail {
+template <typename TileT>
+constexpr bool is_scale_mat_v = TileT::Loc == TileType::Mat && std::is_same_v<typename TileT::DType, float8_e8m0_t>;
+
+// GM -> Mat tile of block scales ([rows, k blocks] row-major for a left operand, [k blocks, columns] column-major for a
+// right one; k blocks contiguous in memory).  LDS image: [k block / 4][row (column)][4 k blocks], so that the scales
+// of one k step of 32 consecutive rows are 32 consecutive words (fragment reads without bank conflicts).  One 4-byte
+// asynchronous copy instruction per 64 rows and 4 k blocks.
+template <typename TileT>
+struct ScaleMatGeom {
+    static constexpr bool left = TileT::isRowMajor;
+    static constexpr int Major = left ? TileT::Rows : TileT::Cols, KB = left ? TileT::Cols : TileT::Rows;
+    static_assert(!TileT::isBoxedLayout && KB % 4 == 0 && Major % kWaveSize == 0,
+                  "[PTO][SA] Mat tile of block scales: unboxed, multiples of 64 rows (columns) and of 4 k blocks");
+    static constexpr int nInst = (Major / kWaveSize) * (KB / 4);
+    PTO_DEV static uint32_t off(uint32_t major, uint32_t kb) { return ((kb / 4) * Major + major) * 4 + kb % 4; }
+};
+template <typename TileT, typename G>
+PTO_DEV void tload_scale_mat(TileT &dst, G &src)
+{
+    using Geo = ScaleMatGeom<TileT>;
+    static_assert(Geo::left ? G::staticStride[4] == 1 : G::staticStride[3] == 1, "[PTO][SA] TLOAD of block scales: k blocks must be contiguous");
+    static_assert(TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols, "[PTO][SA] TLOAD of block scales: fully valid tiles");
+    char *lds = hw::lds_base() + dst.st.lds;
+    const char *gm = reinterpret_cast<const char *>(src.data());
+    const int64_t ld = Geo::left ? src.GetStride(3) : src.GetStride(4);
+    const int lane = hw::lane(), wave = hw::wave();
+    const uint32_t laneOff = (uint32_t)lane * (uint32_t)ld;
+    static_assert(Geo::nInst % kBlockWaves == 0 || Geo::nInst > kBlockWaves, "[PTO][SA] TLOAD: fewer copy instructions than waves");
+#pragma unroll
+    for (int s0 = 0; s0 < Geo::nInst; s0 += kBlockWaves) {
+        // (waves past the end of an incomplete last round repeat their previous instruction, as for operand tiles)
+        const int s = ((Geo::nInst % kBlockWaves != 0 && s0 + wave >= Geo::nInst) ? s0 - kBlockWaves : s0) + wave;
+        const int q = s / (Geo::Major / kWaveSize), g = s % (Geo::Major / kWaveSize);
+        const char *p = uniform_ptr(gm + (int64_t)(g * kWaveSize) * ld + 4 * q) + laneOff;
+        __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(p), PTO_LDS_PTR(lds + s * (kWaveSize * 4)), 4, 0, 0);
+    }
+}
+
 // GM -> block-scale register tile (the reference stages scales in L1 and TEXTRACTs them; a scale tile here is a few
 // registers per lane, so it is loaded straight from memory: one 4-byte load per four k blocks and 32-row block).
 // The k-block index must be the unit-stride dimension and the tile's first k block 4-byte aligned in memory.
@@ -319,11 +351,23 @@ PTO_DEV void tload_scale(TileT &dst, G &src)
 }
 } // namespace detail
 
+template <typename TileT>
+constexpr int TLoadInstrs()
+{
+    if constexpr (detail::is_scale_mat_v<TileT>) {
+        return detail::cdiv(detail::ScaleMatGeom<TileT>::nInst, kBlockWaves);
+    } else {
+        using Geo = detail::MatGeom<TileT>;
+        return detail::cdiv(detail::cdiv(Geo::Major * Geo::ChunksPerRow, kWaveSize), kBlockWaves);
+    }
+}
 template <typename TileT, typename G>
 PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 {
     static_assert(sizeof(typename TileT::DType) == sizeof(typename G::DType), "[PTO][SA] TLOAD: element sizes differ");
-    if constexpr (TileT::Loc == TileType::Mat)
+    if constexpr (detail::is_scale_mat_v<TileT>)
+        detail::tload_scale_mat(dst, src);
+    else if constexpr (TileT::Loc == TileType::Mat)
         detail::tload_mat(dst, src);
     else if constexpr (TileT::Loc == TileType::Vec)
         detail::tload_vec(dst, src);
@@ -368,17 +412,16 @@ PTO_DEV void textract_mx(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol)
         }
 }
 
-// Mat tile of scales in LDS (one row of k-block scales per operand row / column, unboxed) -> scale register tile:
+// Mat tile of scales in LDS (image [k block / 4][row][4 k blocks], see tload_scale_mat) -> scale register tile:
 // k blocks [kb, kb + dst.KB) of rows [idx, idx + extent); kb a multiple of 4 (of 2 for a tile of one k step: one
 // ds_read_u8 per 32-row block, lanes 32-63 read the step's second block)
 template <typename DstT, typename SrcT>
 PTO_DEV void textract_scale_mat(DstT &dst, SrcT &src, uint32_t idxMajor, uint32_t kb)
 {
-    using Geo = MatGeom<SrcT>;
+    using Geo = ScaleMatGeom<SrcT>;
     using D = typename DstT::Storage;
     constexpr bool left = DstT::Loc == TileType::ScaleLeft;
-    static_assert(sizeof(typename SrcT::DType) == 1 && !SrcT::isBoxedLayout && (left ? Geo::colsK : !Geo::colsK) && Geo::ChunksPerRow == 1,
-                  "[PTO][SA] TEXTRACT of scales: unboxed Mat tile, 16 k blocks per row, contiguous along k");
+    static_assert(is_scale_mat_v<SrcT> && left == Geo::left, "[PTO][SA] TEXTRACT of scales: from a Mat tile of block scales of the same side");
     const char *lds = hw::lds_base() + src.st.lds;
     const uint32_t lane = (uint32_t)hw::lane();
     const uint32_t shift = (lane / kMxM) * 8;
@@ -386,18 +429,13 @@ PTO_DEV void textract_scale_mat(DstT &dst, SrcT &src, uint32_t idxMajor, uint32_
     const uint32_t major0 = idxMajor + (uint32_t)(left ? hw::wave_m() : hw::wave_n()) * (blocks * kMxM) + lane % kMxM;
 #pragma unroll
     for (int b = 0; b < blocks; ++b) {
-        const char *p = lds + (major0 + b * kMxM) * Geo::RowBytes + kb;
+        const char *p = lds + Geo::off(major0 + b * kMxM, kb);
         if constexpr (D::KB == 2) {
             dst.st.s[b][0] = *reinterpret_cast<const uint8_t *>(p + lane / kMxM);
-        } else if constexpr (D::Regs == 4) {
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(p);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                dst.st.s[b][i] = v[i] >> shift;
         } else {
 #pragma unroll
             for (int r = 0; r < D::Regs; ++r)
-                dst.st.s[b][r] = *reinterpret_cast<const uint32_t *>(p + 4 * r) >> shift;
+                dst.st.s[b][r] = *reinterpret_cast<const uint32_t *>(p + r * (Geo::Major * 4)) >> shift;
         }
     }
 }

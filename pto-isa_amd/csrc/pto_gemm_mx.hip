@@ -12,8 +12,10 @@
 // directives).  A K-step is 64 fp8 values = the same 64 bytes per row as 32 fp16 values, and one
 // v_mfma_scale_f32_32x32x64_f8f6f4 (16 passes) takes the place of two v_mfma_f32_32x32x16_f16 (8 passes each), so
 // bytes moved per MFMA cycle are those of the fp16 kernel at twice the flops.  The scales of 512 k (16 blocks = 16
-// bytes per row) are copied into LDS once per eight K-steps (two buffers) and the two scales a lane needs for a K-step
-// are read with the step's fragments (one ds_read_u8 per 32-row block); the MFMA applies them.
+// bytes per row) come into LDS once per eight K-steps with one 16-byte asynchronous copy instruction per wave, are
+// rearranged there into the image of a Mat tile of block scales (the scales of one step of consecutive rows in
+// consecutive words: a 64-lane read of words 16 bytes apart costs 6 LDS cycles instead of 2), and the two scales a lane
+// needs for a K-step are read with the step's fragments (one ds_read_u8 per 32-row block); the MFMA applies them.
 // fp4: a 64-byte K-step holds 128 k = two MFMAs (8 passes each) per fragment pair and four scale blocks (one ds_read_b32
 // per 32-row block); a scale group is four K-steps.  Same bytes per step again, at four times the fp16 flops.
 // m and n need not be multiples of the tile: the last tile row / column is moved back to end at m / n and recomputes
@@ -31,21 +33,43 @@ constexpr int kMxStepBytes = 64; // one K-step per operand row in LDS
 template <typename T>
 constexpr int kMxGroupSteps = 16 / (kMxStepBytes * 8 / detail::elem_bits<T> / 32);
 
-// One asynchronous copy instruction per wave: the 16-byte scale rows of the workgroup's BM rows of A and BN columns
-// of B for one scale group -> LDS [BM + BN][16 bytes] (the images of an unboxed [BM, 16] row-major and a [16, BN]
-// column-major Mat tile, back to back).  Instruction i covers 64 rows; wave w issues instruction
+// One asynchronous copy instruction per wave: the 16-byte scale rows (16 k blocks = one scale group) of the workgroup's
+// BM rows of A and BN columns of B -> LDS [BM + BN][16 bytes].  Instruction i covers 64 rows; wave w issues instruction
 // w % ((BM + BN) / 64) (with fewer instructions than waves some waves repeat one: same data to the same place).
 template <int BM, int BN>
-AICORE inline void LoadScaleGroup(uint32_t ldsOff, __gm__ const uint8_t *sa, __gm__ const uint8_t *sb, int64_t ld)
+AICORE inline void LoadScaleRows(uint32_t ldsOff, __gm__ const uint8_t *sa, __gm__ const uint8_t *sb, int64_t ld)
 {
     constexpr int nA = BM / 64, nB = BN / 64;
     static_assert(BM % 64 == 0 && BN % 64 == 0 && nA + nB <= kBlockWaves, "one scale copy instruction per wave");
-    const int inst = hw::wave() % (nA + nB), lane = hw::lane();
+    int lane = hw::lane();
+    // (used once per eight K-steps: keeps the address arithmetic from being hoisted into registers that live across the loop)
+    asm volatile("" : "+v"(lane));
+    const int inst = hw::wave() % (nA + nB);
     const bool isA = inst < nA;
     const char *base = reinterpret_cast<const char *>(isA ? sa : sb);
     const int row = (isA ? inst : inst - nA) * 64;
     const char *g = detail::uniform_ptr(base + (int64_t)row * ld) + (uint32_t)lane * (uint32_t)ld;
     __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(hw::lds_base() + ldsOff + inst * 1024), 16, 0, 0);
+}
+
+// [BM + BN][16 bytes] scale rows at `rawOff` -> the LDS images of a [BM, 16] left and a [16, BN] right Mat tile of block
+// scales at `dstOff` and `dstOff + BM * 16` ([k block / 4][row][4 k blocks], see detail::ScaleMatGeom): one row per thread
+// (with more threads than rows some rows are done twice: same data to the same place, no branch).
+template <int BM, int BN>
+AICORE inline void RearrangeScaleRows(uint32_t dstOff, uint32_t rawOff)
+{
+    static_assert(kBlockThreads % (BM + BN) == 0, "one scale row per thread");
+    int t = hw::tid();
+    asm volatile("" : "+v"(t)); // (as in LoadScaleRows: recompute the addresses rather than keep them in registers)
+    t %= BM + BN;
+    char *lds = hw::lds_base();
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(lds + rawOff + t * 16);
+    const bool isA = t < BM;
+    char *dst = lds + dstOff + (isA ? 0 : BM * 16) + (isA ? t : t - BM) * 4;
+    const int major = isA ? BM : BN;
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<uint32_t *>(dst + q * major * 4) = v[q];
 }
 
 template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES>
@@ -54,6 +78,10 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
                                                              int n, int k, int row0, int col0)
 {
     static_assert(detail::elem_bits<FA> == detail::elem_bits<FB>, "operands of one width");
+    // the tile origin comes out of integer divisions, which run on the vector unit: move it (and with it every panel
+    // pointer below) into scalar registers
+    row0 = __builtin_amdgcn_readfirstlane(row0);
+    col0 = __builtin_amdgcn_readfirstlane(col0);
     constexpr int BK = kMxStepBytes * 8 / detail::elem_bits<FA>; // k per K-step
     constexpr int kGroupSteps = kMxGroupSteps<FA>, kStepBlocks = BK / 32;
     constexpr int HM = BM / 2, KB = 16;
@@ -79,8 +107,10 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
 
     constexpr uint32_t kABytes = BM * kMxStepBytes, kBBytes = kMxStepBytes * BN;
     constexpr uint32_t kStage = kABytes + kBBytes;
-    constexpr uint32_t kScaleOff = STAGES * kStage, kScaleBytes = (BM + BN) * 16; // two buffers of [BM + BN][16] scale rows
+    // scale rows as copied, then two buffers of rearranged scales (the current group's and the next one's)
+    constexpr uint32_t kScaleBytes = (BM + BN) * 16, kRawOff = STAGES * kStage, kScaleOff = kRawOff + kScaleBytes;
     constexpr int kLoadsPerStep = TLoadInstrs<TileMatA>() + TLoadInstrs<TileMatB>();
+    constexpr int kScaleLoads = 1; // copy instructions per wave and scale group
     constexpr int kMfma = 2 * AccHalf::Storage::MB * AccHalf::Storage::NB * LeftHalf::Storage::KS;
     constexpr int kReadsA = 2 * LeftHalf::Storage::MB, kReadsB = 2 * RightTile::Storage::NB; // two ds_read_b128 per fragment
     constexpr int kReads = 2 * kReadsA + kReadsB + (2 * LeftHalf::Storage::MB + RightTile::Storage::NB); // + the scale reads
@@ -132,7 +162,7 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
             }
 
     // prologue: the scales of group 0, then STAGES-1 K-steps in flight
-    LoadScaleGroup<BM, BN>(kScaleOff, saPanel, sbPanel, ldScale);
+    LoadScaleRows<BM, BN>(kRawOff, saPanel, sbPanel, ldScale);
 #pragma unroll
     for (int s = 0; s < STAGES - 1; ++s) {
         GlobalA gmA(aPanel + (int64_t)s * kMxStepBytes, ShapeA(), strideA);
@@ -141,6 +171,8 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
         TLOAD(bMat[s], gmB);
     }
     wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // scales and stage 0 are complete
+    RearrangeScaleRows<BM, BN>(kScaleOff, kRawOff);
+    hw::lds_barrier();
     TEXTRACT(saUp, aScaleMat, 0, 0);
     TEXTRACT(saDn[0], aScaleMat, HM, 0);
     TEXTRACT(sbAll[0], bScaleMat, 0, 0);
@@ -155,16 +187,21 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
         constexpr int j = decltype(jTag)::value;
         constexpr int s = j % STAGES, sNext = (s + 1) % STAGES, sLoad = (s + STAGES - 1) % STAGES;
         // the copies of K-step it+1 (issued two steps ago) have landed; only those of the previous step (plus its scale
-        // copy, if it had one) may still be in flight
-        hw::wait_vm<(STAGES - 3) * kLoadsPerStep + (j == 2 ? 1 : 0)>();
+        // copies, if it had any) may still be in flight
+        hw::wait_vm<(STAGES - 3) * kLoadsPerStep + (j == 1 ? kScaleLoads : 0)>();
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t otherBuf = kScaleOff + (uint32_t)((group + 1) & 1) * kScaleBytes;
-        if constexpr (j == 1) {
-            // scales of the next group into the other buffer: last read in step 6 of the previous group, and those
-            // values have fed MFMAs since
+        if constexpr (j == 0) {
+            // scale rows of the next group (every wave rearranged the previous ones two steps into the previous group)
             const int g = group + 1 < groups ? group + 1 : groups - 1;
-            LoadScaleGroup<BM, BN>(otherBuf, saPanel + g * 16, sbPanel + g * 16, ldScale);
+            LoadScaleRows<BM, BN>(kRawOff, saPanel + g * 16, sbPanel + g * 16, ldScale);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (j == 2) {
+            // they have landed (the wait above covers every copy older than the previous step's): into the other buffer,
+            // whose scales were last read in the previous group; first read in this group's last step, a barrier later
+            RearrangeScaleRows<BM, BN>(otherBuf, kRawOff);
             __builtin_amdgcn_sched_barrier(0);
         }
         if constexpr (j == kGroupSteps - 1) { // the next step is the first of the next group
@@ -250,7 +287,7 @@ int launch_gemm_mx(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, 
     constexpr int BM = 256, BN = 256, STAGES = 4, GROUP_M = 4;
     if (m < BM || n < BN || k % 512) // 512 k = one 16-byte scale row in either operand width
         return PTO_ERR_UNSUPPORTED;
-    constexpr int lds = STAGES * (BM + BN) * 64 + 2 * (BM + BN) * 16;
+    constexpr int lds = STAGES * (BM + BN) * 64 + 3 * (BM + BN) * 16;
     auto kernel = GemmMx<FA, FB, OutT, BM, BN, STAGES, GROUP_M>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
