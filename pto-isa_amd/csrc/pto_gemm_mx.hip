@@ -72,7 +72,7 @@ AICORE inline void RearrangeScaleRows(uint32_t dstOff, uint32_t rawOff)
         *reinterpret_cast<uint32_t *>(dst + q * major * 4) = v[q];
 }
 
-template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES>
+template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES, bool DEEP>
 AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, __gm__ const FA *src0, __gm__ const FB *src1,
                                                              __gm__ const uint8_t *scale0, __gm__ const uint8_t *scale1, int m,
                                                              int n, int k, int row0, int col0)
@@ -161,18 +161,25 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
                 cDn.st.f[mb][nb][i] = 0.0f;
             }
 
-    // prologue: the scales of group 0, then STAGES-1 K-steps in flight
+    // prologue: the scales of group 0, then kAhead K-steps in flight.  DEEP: a step's copies are issued STAGES steps
+    // ahead, into the stage whose fragments were read one step earlier (every wave drains its LDS reads before the step's
+    // barrier), instead of STAGES-1 steps ahead: they have three K-steps to land instead of two.
+    constexpr int kAhead = DEEP ? STAGES : STAGES - 1;
     LoadScaleRows<BM, BN>(kRawOff, saPanel, sbPanel, ldScale);
 #pragma unroll
-    for (int s = 0; s < STAGES - 1; ++s) {
+    for (int s = 0; s < kAhead; ++s) {
         GlobalA gmA(aPanel + (int64_t)s * kMxStepBytes, ShapeA(), strideA);
         GlobalB gmB(bPanel + (int64_t)s * kMxStepBytes, ShapeB(), strideB);
         TLOAD(aMat[s], gmA);
         TLOAD(bMat[s], gmB);
     }
-    wait_flag_pending<(STAGES - 2) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // scales and stage 0 are complete
+    wait_flag_pending<(kAhead - 1) * kLoadsPerStep>(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); // scales and stage 0 are complete
     RearrangeScaleRows<BM, BN>(kScaleOff, kRawOff);
     hw::lds_barrier();
+    {   // scale rows of group 1: rearranged two steps into group 0
+        const int g = 1 < groups ? 1 : groups - 1;
+        LoadScaleRows<BM, BN>(kRawOff, saPanel + g * 16, sbPanel + g * 16, ldScale);
+    }
     TEXTRACT(saUp, aScaleMat, 0, 0);
     TEXTRACT(saDn[0], aScaleMat, HM, 0);
     TEXTRACT(sbAll[0], bScaleMat, 0, 0);
@@ -185,22 +192,20 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
     // scale group and the reads fetch values nobody uses.
     auto step = [&](auto jTag, int it, int group) {
         constexpr int j = decltype(jTag)::value;
-        constexpr int s = j % STAGES, sNext = (s + 1) % STAGES, sLoad = (s + STAGES - 1) % STAGES;
-        // the copies of K-step it+1 (issued two steps ago) have landed; only those of the previous step (plus its scale
-        // copies, if it had any) may still be in flight
-        hw::wait_vm<(STAGES - 3) * kLoadsPerStep + (j == 1 ? kScaleLoads : 0)>();
+        constexpr int s = j % STAGES, sNext = (s + 1) % STAGES, sLoad = (s + kAhead) % STAGES;
+        // the copies of K-step it+1 have landed; only those of the kAhead-2 steps after it may still be in flight, and the
+        // scale copy that follows the copies of a group's last step while that step is among them
+        hw::wait_vm<(kAhead - 2) * kLoadsPerStep + (j <= kAhead - 3 ? kScaleLoads : 0)>();
+        if constexpr (DEEP)
+            hw::wait_lgkm0(); // this wave's reads of the stage that the copies below overwrite (issued last step) are done
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
         const uint32_t otherBuf = kScaleOff + (uint32_t)((group + 1) & 1) * kScaleBytes;
-        if constexpr (j == 0) {
-            // scale rows of the next group (every wave rearranged the previous ones two steps into the previous group)
-            const int g = group + 1 < groups ? group + 1 : groups - 1;
-            LoadScaleRows<BM, BN>(kRawOff, saPanel + g * 16, sbPanel + g * 16, ldScale);
-            __builtin_amdgcn_sched_barrier(0);
-        }
         if constexpr (j == 2) {
-            // they have landed (the wait above covers every copy older than the previous step's): into the other buffer,
-            // whose scales were last read in the previous group; first read in this group's last step, a barrier later
+            // The scale rows of the next group, copied during the previous group's last step (in the prologue for
+            // group 1), have landed: the wait above covers every copy older than step 0's.  Into the other buffer, whose
+            // scales were last read in the previous group; first read in this group's last step, a barrier later.
+            static_assert(kAhead - 3 < 2 && kGroupSteps > 3, "the scale copy is older than every copy that may be in flight here");
             RearrangeScaleRows<BM, BN>(otherBuf, kRawOff);
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -208,11 +213,16 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
             TASSIGN(aScaleMat, otherBuf);
             TASSIGN(bScaleMat, otherBuf + BM * 16);
         }
-        const int fetch = it + STAGES - 1 < kLoop ? it + STAGES - 1 : kLoop - 1;
+        const int fetch = it + kAhead < kLoop ? it + kAhead : kLoop - 1;
         GlobalA gmA(aPanel + (int64_t)fetch * kMxStepBytes, ShapeA(), strideA);
         GlobalB gmB(bPanel + (int64_t)fetch * kMxStepBytes, ShapeB(), strideB);
         TLOAD(aMat[sLoad], gmA);
         TLOAD(bMat[sLoad], gmB);
+        if constexpr (j == kGroupSteps - 1) {
+            // scale rows of the group after the next one (every wave rearranged the next group's earlier in this group)
+            const int g = group + 2 < groups ? group + 2 : groups - 1;
+            LoadScaleRows<BM, BN>(kRawOff, saPanel + g * 16, sbPanel + g * 16, ldScale);
+        }
         constexpr int p = j & 1, q = p ^ 1, kbNext = kStepBlocks * ((j + 1) % kGroupSteps);
         TMATMUL_MX(cUp, cUp, aUp, saUp, bAll[p], sbAll[p]);
         TEXTRACT(aUp, aMat[sNext], 0, 0);
@@ -223,7 +233,7 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
         TEXTRACT(aDn[q], aMat[sNext], HM, 0);
         TEXTRACT(saDn[q], aScaleMat, +HM, +kbNext);
 #pragma unroll
-        for (int i = 0; i < kLoadsPerStep; ++i) {
+        for (int i = 0; i < kLoadsPerStep + (j == kGroupSteps - 1 ? kScaleLoads : 0); ++i) {
             if (i < kMfmaCopies)
                 __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
@@ -252,7 +262,7 @@ AICORE inline __attribute__((always_inline)) void MxTileRows(__gm__ OutT *out, _
 
 // The first `fullTiles` workgroups (whole rounds over the compute units) own one BM x BN C tile each; with quarter != 0
 // the tiles of the last, partial round are cut into four (BM/2) x (BN/2) tiles, one workgroup each.
-template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES, int GROUP_M>
+template <typename FA, typename FB, typename OutT, int BM, int BN, int STAGES, int GROUP_M, bool DEEP>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     void GemmMx(__gm__ OutT *out, __gm__ const FA *src0, __gm__ const FB *src1, __gm__ const uint8_t *scale0,
                 __gm__ const uint8_t *scale1, int m, int n, int k, int fullTiles)
@@ -264,14 +274,14 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
         const int u = RegroupXcd(block - fullTiles, (tilesM * tilesN - fullTiles) * 4);
         TileOfId<GROUP_M>(fullTiles + u / 4, tilesM, tilesN, tm, tn);
         const int sub = u % 4;
-        MxTileRows<FA, FB, OutT, BM / 2, BN / 2, STAGES>(out, src0, src1, scale0, scale1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
+        MxTileRows<FA, FB, OutT, BM / 2, BN / 2, STAGES, DEEP>(out, src0, src1, scale0, scale1, m, n, k, tm * BM + (sub >> 1) * (BM / 2),
                                                         tn * BN + (sub & 1) * (BN / 2));
         return;
     }
     TileOfId<GROUP_M>(RegroupXcd(block, fullTiles), tilesM, tilesN, tm, tn);
     // the last tile row / column ends at m / n: it recomputes the rows / columns it shares with its neighbour
     const int row0 = tm * BM + BM <= m ? tm * BM : m - BM, col0 = tn * BN + BN <= n ? tn * BN : n - BN;
-    MxTileRows<FA, FB, OutT, BM, BN, STAGES>(out, src0, src1, scale0, scale1, m, n, k, row0, col0);
+    MxTileRows<FA, FB, OutT, BM, BN, STAGES, DEEP>(out, src0, src1, scale0, scale1, m, n, k, row0, col0);
 }
 
 } // namespace
@@ -280,7 +290,7 @@ PTO_DEVICE_CODE_END
 
 namespace {
 
-template <typename FA, typename FB, typename OutT>
+template <typename FA, typename FB, typename OutT, bool DEEP = true>
 int launch_gemm_mx(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n,
                    int k, int tailMode)
 {
@@ -288,7 +298,7 @@ int launch_gemm_mx(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, 
     if (m < BM || n < BN || k % 512) // 512 k = one 16-byte scale row in either operand width
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = STAGES * (BM + BN) * 64 + 3 * (BM + BN) * 16;
-    auto kernel = GemmMx<FA, FB, OutT, BM, BN, STAGES, GROUP_M>;
+    auto kernel = GemmMx<FA, FB, OutT, BM, BN, STAGES, GROUP_M, DEEP>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
@@ -302,19 +312,28 @@ int launch_gemm_mx(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, 
     return pto_amd::check_launch();
 }
 
-int gemm_mx_dispatch(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n,
-                     int k, int format, int c_fp32, int tailMode)
+template <bool DEEP>
+int gemm_mx_dispatch_fmt(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m,
+                         int n, int k, int format, int c_fp32, int tailMode)
 {
     if (format == 0)
-        return c_fp32 ? launch_gemm_mx<float8_e4m3_t, float8_e4m3_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
-                        launch_gemm_mx<float8_e4m3_t, float8_e4m3_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
+        return c_fp32 ? launch_gemm_mx<float8_e4m3_t, float8_e4m3_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float8_e4m3_t, float8_e4m3_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
     if (format == 1)
-        return c_fp32 ? launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
-                        launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
+        return c_fp32 ? launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
     if (format == 4)
-        return c_fp32 ? launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, float>(st, c, a, b, sa, sb, m, n, k, tailMode) :
-                        launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, bfloat16_t>(st, c, a, b, sa, sb, m, n, k, tailMode);
+        return c_fp32 ? launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
     return PTO_ERR_UNSUPPORTED;
+}
+
+// variant: bit 0 = quarter tiles in the last round, bit 1 = copies issued STAGES-1 instead of STAGES steps ahead
+int gemm_mx_dispatch(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n,
+                     int k, int format, int c_fp32, int variant)
+{
+    return (variant & 2) ? gemm_mx_dispatch_fmt<false>(st, c, a, b, sa, sb, m, n, k, format, c_fp32, variant & 1) :
+                           gemm_mx_dispatch_fmt<true>(st, c, a, b, sa, sb, m, n, k, format, c_fp32, variant & 1);
 }
 
 } // namespace
@@ -337,12 +356,12 @@ extern "C" int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uin
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, 4, c_fp32, 1);
 }
 
-// Tuning hook (not part of the public header): variant 0 = whole tiles only, 1 = quarter tiles in the last round;
-// format 0 / 1 = fp8 e4m3 / e5m2, 4 = fp4 e2m1.
+// Tuning hook (not part of the public header): variant bit 0 = quarter tiles in the last round, bit 1 = the shallower copy
+// pipeline; format 0 / 1 = fp8 e4m3 / e5m2, 4 = fp4 e2m1.
 extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                                       const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant)
 {
-    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0 || variant < 0 || variant > 1)
+    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0 || variant < 0 || variant > 3)
         return PTO_ERR_BAD_ARG;
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, variant);
 }
