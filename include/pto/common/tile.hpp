@@ -225,10 +225,10 @@ struct Tile {
     static_assert(Loc_ == TileType::Vec || Rows_ == 1 || Rows % InnerRows == 0,
                   "[PTO][SA] tile rows must be a multiple of the inner box rows");
     static_assert(Cols % InnerCols == 0, "[PTO][SA] tile cols must be a multiple of the inner box cols");
-    // (scale tiles are register tiles of a few bytes per row; a Mat tile of 1-byte block scales has 16-byte rows)
+    // (scale tiles are register tiles of a few bytes per row; a Mat tile of block scales holds multiples of 4 per row)
     static_assert(isBoxedLayout || Loc_ == TileType::ScaleLeft || Loc_ == TileType::ScaleRight ||
                       (isRowMajor ? (Cols * sizeof(DType)) : (Rows * sizeof(DType))) %
-                              (Loc_ == TileType::Mat && sizeof(DType) == 1 ? 16 : TileConfig::alignedSize) == 0,
+                              (Loc_ == TileType::Mat && std::is_same_v<DType, float8_e8m0_t> ? 4 : TileConfig::alignedSize) == 0,
                   "[PTO][SA] unboxed tiles need a 32-byte aligned contiguous extent");
 
     // The logical dimension that is contiguous in a Mat tile's LDS image: columns unless the tile

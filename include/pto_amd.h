@@ -132,9 +132,11 @@ int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, c
 
 /* MX matmul [128,256] x [256,128] -> fp32 [128,128]: a [128,256] and b_t [128][256] (column-major b) fp8 bytes in
  * format_a / format_b (0 = e4m3, 1 = e5m2; they may differ), scale_a [128,8] and scale_b_t [128][8] e8m0 bytes; K in two
- * halves, TMATMUL_MX then its accumulating form (tests/npu/a5/src/st/testcase/tmatmul_mx/tmatmul_mx_kernel.cpp). */
+ * halves, TMATMUL_MX then its accumulating form (tests/npu/a5/src/st/testcase/tmatmul_mx/tmatmul_mx_kernel.cpp).
+ * scales_via_lds != 0: the scales are TLOADed into Mat tiles and TEXTRACTed from there (as the reference stages them in
+ * L1) instead of being loaded from memory into scale tiles directly. */
 int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
-                                 const uint8_t *scale_b_t, int format_a, int format_b);
+                                 const uint8_t *scale_b_t, int format_a, int format_b, int scales_via_lds);
 
 /* One Vec instruction on [64,128] fp32 tiles: out = OP(a [, b | scalar | vec]).  vec is a per-row [64] operand for
  * the TROWEXPAND* ops and a per-column [128] operand for the TCOLEXPAND* ops.  op codes (PTO_VOP_*): unary

@@ -275,9 +275,10 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulBias(__gm__ float 
 
 // ---- one-block MX matmul [128, 256] x [256, 128], fp8 operands (formats may differ) with e8m0 block scales ----
 // (tests/npu/a5/src/st/testcase/tmatmul_mx/tmatmul_mx_kernel.cpp: TLOAD -> TEXTRACT -> TMATMUL_MX -> TSTORE).  K is taken
-// in two halves of 128: TMATMUL_MX on the first, the accumulating form on the second; the scale tiles are loaded whole
-// from memory (MX_A_ND / MX_B_DN) and windowed per half.
-template <typename FA, typename FB>
+// in two halves of 128: TMATMUL_MX on the first, the accumulating form on the second.  VIA_MAT == false: the scale tiles
+// are loaded whole from memory (MX_A_ND / MX_B_DN) into registers and windowed per half; true: the scales are TLOADed
+// into Mat tiles (as the reference kernels stage them in L1) and each half's scale tiles TEXTRACTed from there.
+template <typename FA, typename FB, bool VIA_MAT>
 __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMx(__gm__ float *out, __gm__ const FA *a, __gm__ const FB *bT,
                                                                  __gm__ const float8_e8m0_t *sa, __gm__ const float8_e8m0_t *sbT)
 {
@@ -301,21 +302,40 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMx(__gm__ float *o
     GlobalTensor<X, TileShape2D<X, M, KB, Layout::MX_A_ND>, BaseShape2D<X, M, KB, Layout::MX_A_ND>, Layout::MX_A_ND> gsa(const_cast<X *>(sa));
     GlobalTensor<X, TileShape2D<X, KB, N, Layout::MX_B_DN>, BaseShape2D<X, KB, N, Layout::MX_B_DN>, Layout::MX_B_DN> gsb(const_cast<X *>(sbT));
     GmND<float, M, N> gc(out);
+    Tile<TileType::Mat, X, M, KB, BLayout::RowMajor, M, KB, SLayout::NoneBox> lsMat;
+    Tile<TileType::Mat, X, KB, N, BLayout::ColMajor, KB, N, SLayout::NoneBox> rsMat;
+    TASSIGN(lsMat, (uint32_t)(M * K + K * N));
+    TASSIGN(rsMat, (uint32_t)(M * K + K * N + M * KB));
     TLOAD(am, ga);
     TLOAD(bm, gb);
-    TLOAD(lsAll, gsa);
-    TLOAD(rsAll, gsb);
+    if constexpr (VIA_MAT) {
+        TLOAD(lsMat, gsa);
+        TLOAD(rsMat, gsb);
+    } else {
+        TLOAD(lsAll, gsa);
+        TLOAD(rsAll, gsb);
+    }
     set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
     wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
     TEXTRACT(l, am, 0, 0);
     TEXTRACT(r, bm, 0, 0);
-    TEXTRACT(ls, lsAll, 0, 0);
-    TEXTRACT(rs, rsAll, 0, 0);
+    if constexpr (VIA_MAT) {
+        TEXTRACT(ls, lsMat, 0, 0);
+        TEXTRACT(rs, rsMat, 0, 0);
+    } else {
+        TEXTRACT(ls, lsAll, 0, 0);
+        TEXTRACT(rs, rsAll, 0, 0);
+    }
     TMATMUL_MX(c, l, ls, r, rs);
     TEXTRACT(l, am, 0, KH);
     TEXTRACT(r, bm, KH, 0);
-    TEXTRACT(ls, lsAll, 0, KH / 32);
-    TEXTRACT(rs, rsAll, KH / 32, 0);
+    if constexpr (VIA_MAT) {
+        TEXTRACT(ls, lsMat, 0, KH / 32);
+        TEXTRACT(rs, rsMat, KH / 32, 0);
+    } else {
+        TEXTRACT(ls, lsAll, 0, KH / 32);
+        TEXTRACT(rs, rsAll, KH / 32, 0);
+    }
     TMATMUL_MX(c, c, l, ls, r, rs);
     TSTORE(gc, c);
 }
@@ -665,21 +685,26 @@ extern "C" int pto_st_textract_windows_f16(void *stream, float *out_left, float 
 }
 
 extern "C" int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
-                                            const uint8_t *scale_b_t, int format_a, int format_b)
+                                            const uint8_t *scale_b_t, int format_a, int format_b, int scales_via_lds)
 {
     PTO_ST_NONNULL(out, a, b_t, scale_a, scale_b_t);
     if (format_a < 0 || format_a > 1 || format_b < 0 || format_b > 1)
         return PTO_ERR_BAD_ARG;
-    constexpr int lds = 128 * 256 + 256 * 128;
+    constexpr int lds = 128 * 256 + 256 * 128 + 2 * 128 * 8;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const float8_e8m0_t *sa = reinterpret_cast<const float8_e8m0_t *>(scale_a), *sb = reinterpret_cast<const float8_e8m0_t *>(scale_b_t);
 #define PTO_ST_MX(FA, FB)                                                                                                     \
     do {                                                                                                                      \
-        static const int attr = pto_amd::allow_lds(MatmulMx<FA, FB>, lds);                                                    \
-        if (attr != PTO_OK)                                                                                                   \
-            return attr;                                                                                                      \
-        MatmulMx<FA, FB><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const FA *>(a),                     \
-                                                                    reinterpret_cast<const FB *>(b_t), sa, sb);              \
+        static const int attr0 = pto_amd::allow_lds(MatmulMx<FA, FB, false>, lds);                                            \
+        static const int attr1 = pto_amd::allow_lds(MatmulMx<FA, FB, true>, lds);                                             \
+        if (attr0 != PTO_OK || attr1 != PTO_OK)                                                                               \
+            return attr0 != PTO_OK ? attr0 : attr1;                                                                           \
+        if (scales_via_lds)                                                                                                   \
+            MatmulMx<FA, FB, true><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const FA *>(a),           \
+                                                                              reinterpret_cast<const FB *>(b_t), sa, sb);    \
+        else                                                                                                                  \
+            MatmulMx<FA, FB, false><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const FA *>(a),          \
+                                                                               reinterpret_cast<const FB *>(b_t), sa, sb);   \
     } while (0)
     if (format_a == 0 && format_b == 0)
         PTO_ST_MX(float8_e4m3_t, float8_e4m3_t);

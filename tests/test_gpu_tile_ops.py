@@ -256,10 +256,12 @@ def test_tpush_tpop_pipeline(lds_fifo):
             assert np.array_equal(qslots[t], a @ b[t])
 
 
+@pytest.mark.parametrize("via_lds", [0, 1])
 @pytest.mark.parametrize("fmt_a,fmt_b", [(0, 0), (1, 1), (0, 1), (1, 0)])
-def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b):
+def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b, via_lds):
     """TMATMUL_MX and its accumulating form on two 128-wide k halves (two MFMA k steps each), mixed operand formats,
-    scale tiles loaded from memory (MX_A_ND / MX_B_DN) and windowed: exact on integer operands, <= 2e-3 on random ones."""
+    scale tiles loaded from memory (MX_A_ND / MX_B_DN) and windowed, or staged in Mat tiles of block scales and
+    TEXTRACTed: exact on integer operands, <= 2e-3 on random ones."""
     from pto_amd import datagen
     lib = capi.load()
     for dist, lo, hi in (("integer", 125, 130), ("uniform", 120, 135), ("bytes", 110, 140)):
@@ -268,7 +270,7 @@ def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b):
         out = torch.full((128, 128), float("nan"), device=DEV)
         ta, tb, tsa, tsb = (torch.from_numpy(x).to(DEV) for x in (a, b, sa, sb))
         capi.check(lib.pto_st_matmul_mx_128x256x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(),
-                                                    tsb.data_ptr(), fmt_a, fmt_b), "matmul mx")
+                                                    tsb.data_ptr(), fmt_a, fmt_b, via_lds), "matmul mx")
         torch.cuda.synchronize()
         got = out.cpu().numpy()
         want = oracle.mx_gemm(a, b, sa, sb, fmt_a, fmt_b)
