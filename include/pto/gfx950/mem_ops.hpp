@@ -28,10 +28,12 @@ PTO_DEV constexpr uint32_t mat_swz(uint32_t major)
     if constexpr (!is_pow2(cpr) || cpr < 2) {
         return 0;
     } else {
-        // rows per swizzle step.  64-byte rows: 2 (measured conflict-free for ds_read_b128 fragment reads of both
-        // MFMA shapes: lanes read 32 rows x 1 chunk or 16 rows x 1 chunk per half / quarter wave; a step of 4 rows
-        // costs 7 % of the LDS read rate with 16-row blocks)
-        constexpr int div = cpr >= 16 ? 1 : (cpr == 4 ? 2 : 16 / cpr);
+        // rows per swizzle step.  64-byte rows: the 16 lanes that a ds_read_b128 serves together read 16 consecutive rows
+        // at one logical chunk; rows 4 apart share their banks, so the chunk position has to differ among them: a step
+        // of 4 rows for the 32-row blocks of the 32 x 32 MFMAs, of 2 rows for the 16-row blocks of the 16 x 16 ones
+        // (where 16 lanes are 16 rows x 1 chunk but the next 16 lanes the same rows at the next chunk).  The LDS
+        // bank-conflict counter reads 0 for either pairing and about one conflict cycle per read cycle for the other.
+        constexpr int div = cpr >= 16 ? 1 : (cpr == 4 ? (kMfmaM == 32 ? 4 : 2) : 16 / cpr);
         constexpr int mod = cpr >= 16 ? 16 : cpr;
         return (major / div) % mod;
     }
