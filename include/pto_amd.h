@@ -12,6 +12,8 @@
  *                        ctypes entry call_kernel(blockDim, stream, out, src0, src1) demos/torch_jit/gemm/gemm_kernel.cpp:259-262
  *   pto_gemm_mxfp8       LaunchMxMatmul(uint8_t *out, uint8_t *src0, uint8_t *src1, uint8_t *src2, uint8_t *src3, void *stream)
  *                        kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:344-364
+ *   pto_topk_f32         launchTopk<float>(uint8_t *out, uint8_t *index, uint8_t *src, uint8_t *inIdx, void *stream)
+ *                        kernels/manual/a2a3/topk/topk_kernel.cpp:334-345
  *   pto_fa_fwd_f16       LaunchTFA<...>(...) kernels/manual/common/flash_atten/fa_performance_kernel.h:28-41 and
  *                        call_kernel(...) demos/torch_jit/flash_atten/fa_kernel.cpp:1017-1092
  *   pto_tcvt_*           runTCVT / launchTCVT tests/cpu/st/testcase/tcvt/tcvt_kernel.cpp:18-66 (TLOAD -> TCVT -> TSTORE)
@@ -67,6 +69,14 @@ int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, co
  * kernels/manual/a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp).  Same limits. */
 int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
                    int m, int n, int k, int c_fp32);
+
+/* Row-wise top-k.  src [rows, ld] fp32, the first valid_cols columns of every row are scored; in_idx [valid_cols] uint32
+ * gives the index reported for a column (the reference passes 0, 1, 2, ...).  Per row the (score, index) pairs are put in
+ * descending order of score, equal scores (-0 == +0) in ascending order of index, and the first topk are written:
+ * out_score [rows, topk] fp32 (the source bit patterns), out_index [rows, topk] uint32.  valid_cols <= 4096,
+ * topk <= valid_cols <= ld.  NaN scores are ordered by their bit patterns (positive NaNs first, negative ones last). */
+int pto_topk_f32(void *stream, float *out_score, uint32_t *out_index, const float *src, const uint32_t *in_idx, int rows,
+                 int valid_cols, int ld, int topk);
 
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];

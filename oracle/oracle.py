@@ -63,6 +63,8 @@ def lib():
         L.po_gather_rows.restype = None
         L.po_gemm_f16f32.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_int] * 7
         L.po_gemm_f16f32.restype = None
+        L.po_topk_f32.argtypes = [C.c_void_p] * 4 + [C.c_int] * 4
+        L.po_topk_f32.restype = None
         L.po_mx_gemm.argtypes = [C.c_void_p] * 5 + [C.c_int] * 6
         L.po_mx_gemm.restype = None
         L.po_fp8_e4m3fn_to_f32.argtypes = [C.c_uint8]
@@ -181,6 +183,17 @@ def gemm_f16f32(A, B, base_k=64, row0=0, row1=0, threads=0):
     Cm = np.zeros((m, n), dtype=np.float32)
     lib().po_gemm_f16f32(_p(Cm), _p(A), _p(B), m, n, k, base_k, row0, row1, threads)
     return Cm
+
+
+def topk_f32(src, in_idx, valid_cols, topk):
+    """src [rows, ld] fp32, in_idx [>= valid_cols] uint32 -> (scores [rows, topk] fp32, indices [rows, topk] uint32)."""
+    src = np.ascontiguousarray(src, dtype=np.float32)
+    in_idx = np.ascontiguousarray(in_idx, dtype=np.uint32)
+    rows, ld = src.shape
+    out_s = np.empty((rows, topk), dtype=np.float32)
+    out_i = np.empty((rows, topk), dtype=np.uint32)
+    lib().po_topk_f32(_p(out_s), _p(out_i), _p(src), _p(in_idx), rows, valid_cols, ld, topk)
+    return out_s, out_i
 
 
 def fp8_table(fmt):

@@ -586,6 +586,42 @@ void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA,
     free(Bd);
 }
 
+/* -------------------------------------------------------------------- top-k */
+typedef struct {
+    float score;
+    uint32_t index;
+    int pos;
+} po_score_index;
+
+static int po_score_index_cmp(const void *pa, const void *pb)
+{ /* cpu/TSort32.hpp:64-72; the position keeps the sort stable */
+    const po_score_index *a = (const po_score_index *)pa, *b = (const po_score_index *)pb;
+    if (a->score != b->score)
+        return a->score > b->score ? -1 : 1;
+    if (a->index != b->index)
+        return a->index < b->index ? -1 : 1;
+    return a->pos < b->pos ? -1 : (a->pos > b->pos ? 1 : 0);
+}
+
+void po_topk_f32(float *out_score, uint32_t *out_index, const float *src, const uint32_t *in_idx, int rows, int valid_cols,
+                 int ld, int topk)
+{
+    po_score_index *buf = (po_score_index *)malloc(sizeof(po_score_index) * (size_t)valid_cols);
+    for (int r = 0; r < rows; r++) {
+        for (int c = 0; c < valid_cols; c++) {
+            buf[c].score = src[(size_t)r * (size_t)ld + (size_t)c];
+            buf[c].index = in_idx[c];
+            buf[c].pos = c;
+        }
+        qsort(buf, (size_t)valid_cols, sizeof(po_score_index), po_score_index_cmp);
+        for (int c = 0; c < topk; c++) {
+            out_score[(size_t)r * (size_t)topk + (size_t)c] = buf[c].score;
+            out_index[(size_t)r * (size_t)topk + (size_t)c] = buf[c].index;
+        }
+    }
+    free(buf);
+}
+
 /* ------------------------------------------------------------------- gather */
 void po_tgather_index(void *dst, const po_layout *Ld, const void *src0, const po_layout *L0, const int32_t *idx,
                       const po_layout *L1, int esz, int valid_row, int valid_col)

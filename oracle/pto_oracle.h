@@ -103,6 +103,13 @@ float po_fp4_e2m1_to_f32(uint8_t nibble);
 void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, int m, int n, int k,
                 int format_a, int format_b, int threads);
 
+/* Row-wise top-k as kernels/manual/a2a3/topk computes it: per row the (score, index) pairs (index = in_idx[column]) in
+ * the order of the TSORT32 / TMRGSORT comparator (cpu/TSort32.hpp:32-41, 64-72: score descending, equal scores by
+ * ascending index; stable), the first topk scores and indices written (golden: scripts/gen_data.py:55-64,
+ * np.lexsort((idx, -row))[:topk]).  src [rows, ld] with valid_cols <= ld used per row. */
+void po_topk_f32(float *out_score, uint32_t *out_index, const float *src, const uint32_t *in_idx, int rows, int valid_cols,
+                 int ld, int topk);
+
 /* ---- conversion: cpu/TCvt.hpp:65-84 ---- */
 uint16_t po_f32_to_f16_rne(uint32_t bits); /* == static_cast<_Float16>(float) */
 uint16_t po_f32_to_bf16_rne(uint32_t bits);

@@ -15,6 +15,7 @@ SEED_TCVT_INJECT = 3002
 SEED_GATHER_TABLE = 4001
 SEED_GATHER_IDX = 4002
 SEED_MX_A, SEED_MX_B, SEED_MX_SA, SEED_MX_SB = 19, 2019, 3019, 4019
+SEED_TOPK = 5019
 
 
 def _rng(seed):
@@ -147,6 +148,20 @@ def mx_inputs(m, n, k, fmt, dist="uniform", scale_lo=127, scale_hi=130):
     sa = _rng(SEED_MX_SA).integers(scale_lo, scale_hi, size=(m, k // 32)).astype(np.uint8)
     sb = _rng(SEED_MX_SB).integers(scale_lo, scale_hi, size=(n, k // 32)).astype(np.uint8)
     return a, b, sa, sb
+
+
+def topk_inputs(rows, valid_cols, ld, distinct=0):
+    """src [rows, ld] fp32: row i holds uniform(i, i + valid_cols) in its first valid_cols columns and zeros after, as
+    kernels/manual/a2a3/topk/scripts/gen_data.py:37-41; distinct > 0: only that many different scores (many ties);
+    in_idx = 0 .. valid_cols-1."""
+    r = _rng(SEED_TOPK)
+    src = np.zeros((rows, ld), dtype=np.float32)
+    if distinct:
+        src[:, :valid_cols] = r.integers(0, distinct, size=(rows, valid_cols)).astype(np.float32) - distinct // 2
+    else:
+        src[:, :valid_cols] = (r.uniform(0.0, float(valid_cols), size=(rows, valid_cols)) +
+                               np.arange(rows, dtype=np.float64)[:, None]).astype(np.float32)
+    return src, np.arange(valid_cols, dtype=np.uint32)
 
 
 def gather_inputs(table_rows, cols, n_idx):

@@ -554,3 +554,27 @@ def test_fp4_decode_and_mx_gemm_oracle_fp4(oracle):
     ad = want.astype(np.float64)[datagen.fp4_unpack(a)] * np.repeat(np.exp2(sa.astype(np.float64) - 127), 32, axis=1)
     bd = want.astype(np.float64)[datagen.fp4_unpack(b)] * np.repeat(np.exp2(sb.astype(np.float64) - 127), 32, axis=1)
     assert np.array_equal(oracle.mx_gemm(a, b, sa, sb, 4), (ad @ bd.T).astype(np.float32))
+
+
+# -------------------------------------------------------------------- top-k
+def test_topk_oracle_matches_the_reference_golden_recipe(oracle):
+    """np.lexsort((idx, -row))[:k], the recipe of kernels/manual/a2a3/topk/scripts/gen_data.py:55-64, on its distribution, on
+    rows with many ties, signed zeros and infinities, and with indices that are not the column numbers."""
+    from pto_amd import datagen
+    rows, cols, ld, k = 12, 300, 320, 123
+    for distinct in (0, 5):
+        src, idx = datagen.topk_inputs(rows, cols, ld, distinct=distinct)
+        src[1, ::7] = -0.0
+        src[2, ::5] = np.inf
+        src[3, 1::6] = -np.inf
+        r = np.random.Generator(np.random.Philox(key=3))
+        for index in (idx, r.permutation(5000)[:cols].astype(np.uint32)):
+            s, i = oracle.topk_f32(src, index, cols, k)
+            for row in range(rows):
+                v = src[row, :cols]
+                order = np.lexsort((index, -v))[:k]
+                assert np.array_equal(i[row], index[order])
+                assert np.array_equal(s[row].view(np.uint32), v[order].view(np.uint32))
+    # known answer
+    s, i = oracle.topk_f32(np.array([[1.0, 3.0, 2.0, 3.0, -1.0, 9.0]], dtype=np.float32), np.arange(5, dtype=np.uint32), 5, 3)
+    assert s.tolist() == [[3.0, 3.0, 2.0]] and i.tolist() == [[1, 3, 2]]
