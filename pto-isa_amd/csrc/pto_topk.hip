@@ -7,10 +7,14 @@
 // (include/pto/cpu/TSort32.hpp:32-41: score descending, then index ascending, -0 == +0).
 //
 // The reference builds the order from 32-element hardware sorts and 4-way merges in its unified buffer, re-viewing one
-// buffer through differently shaped tiles.  On a CDNA4 compute unit the natural form is one workgroup per row and a
-// bitonic network over 64-bit keys in LDS: key = (order-preserving image of the score) << 32 | ~index, so that one
-// unsigned comparison implements the comparator.  Each of the four waves owns a quarter of the row: the stages whose
-// partners lie inside a quarter need no workgroup barrier (a wave's LDS operations execute in order).
+// buffer through differently shaped tiles.  On a CDNA4 compute unit the natural form is one workgroup (four waves) per
+// row and a bitonic network over 64-bit keys whose unsigned order is the comparator:
+//   key = (order-preserving image of the score) << 32 | low word that decides among equal scores.
+// * Indices that increase with the column (the reference passes 0, 1, 2, ...): low word = ~column, and a thread keeps
+//   its N/256 consecutive keys in registers.  Partners inside a thread are compared in registers, partners inside a
+//   wave are fetched with lane swizzles, and only the two or three strides that cross waves go through LDS.
+// * Any other index vector: low word = ~index, keys and columns in LDS, every stage a pass over LDS; each wave owns a
+//   quarter of the row and the stages whose partners lie inside a quarter need no workgroup barrier.
 #include <hip/hip_runtime.h>
 
 #include "common.hpp"
@@ -19,28 +23,93 @@ namespace {
 
 constexpr int kTopkThreads = 256, kTopkWaves = 4;
 
-// N: padded row length, a power of two in [256, 4096]
-template <int N>
-__global__ __launch_bounds__(kTopkThreads) void TopkRows(float *outScore, uint32_t *outIndex, const float *src, const uint32_t *inIdx,
-                                                         int validCols, int ld, int topk)
+__device__ inline uint32_t ScoreOrder(uint32_t bits) { return (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u); }
+__device__ inline uint32_t ScoreBits(uint32_t ord) { return (ord & 0x80000000u) ? (ord & 0x7fffffffu) : ~ord; }
+
+// value of lane ^ M of the wave, M a power of two below 64
+template <int M>
+__device__ inline uint32_t LaneXor(uint32_t v, int lane)
 {
-    __shared__ uint64_t key[N];
-    __shared__ uint16_t pos[N];
-    const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
-    const float *row = src + (size_t)blockIdx.x * (size_t)ld;
-    for (int i = tid; i < N; i += kTopkThreads) {
-        uint64_t kv = 0; // padding: below every real key
-        if (i < validCols) {
-            uint32_t b = __float_as_uint(row[i]);
-            if (b == 0x80000000u)
-                b = 0; // -0 and +0 compare equal
-            const uint32_t ord = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
-            kv = ((uint64_t)ord << 32) | (uint32_t)~inIdx[i];
-        }
-        key[i] = kv;
-        pos[i] = (uint16_t)i;
+    if constexpr (M == 1)
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false); // quad_perm [1,0,3,2]
+    else if constexpr (M == 2)
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false); // quad_perm [2,3,0,1]
+    else if constexpr (M == 8)
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false); // row_ror:8 (rows of 16 lanes)
+    else if constexpr (M < 32)
+        return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (M << 10) | 0x1f); // bit mode: lane ^ M within 32 lanes
+    else
+        return (uint32_t)__builtin_amdgcn_ds_bpermute(((lane ^ 32) << 2), (int)v);
+}
+template <int M>
+__device__ inline uint64_t LaneXor64(uint64_t v, int lane)
+{
+    return ((uint64_t)LaneXor<M>((uint32_t)(v >> 32), lane) << 32) | LaneXor<M>((uint32_t)v, lane);
+}
+
+template <int FIRST, int LAST, typename F>
+__device__ inline void StaticFor(F &&f)
+{
+    if constexpr (FIRST < LAST) {
+        f(std::integral_constant<int, FIRST>());
+        StaticFor<FIRST + 1, LAST>(f);
     }
-    __syncthreads();
+}
+
+// Bitonic sort, descending, of the 256 E keys of a workgroup; thread t holds the keys of ranks t E .. t E + E - 1.
+template <int E>
+__device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
+{
+    constexpr int N = kTopkThreads * E, kLogN = __builtin_ctz(N);
+    const int lane = tid & 63;
+    StaticFor<1, kLogN + 1>([&](auto sizeTag) {
+        constexpr int kk = 1 << decltype(sizeTag)::value; // the network sorts runs of kk keys, alternating direction
+        StaticFor<0, decltype(sizeTag)::value>([&](auto strideTag) {
+            constexpr int j = kk >> (decltype(strideTag)::value + 1); // distance between partners
+            if constexpr (j < E) {
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+                    if ((e & j) == 0) {
+                        const bool descending = ((tid * E + e) & kk) == 0;
+                        const uint64_t a = k[e], b = k[e | j];
+                        const bool swap = descending ? a < b : a > b;
+                        k[e] = swap ? b : a;
+                        k[e | j] = swap ? a : b;
+                    }
+            } else {
+                uint64_t other[E];
+                if constexpr (j < 64 * E) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        other[e] = LaneXor64<j / E>(k[e], lane);
+                } else {
+                    __syncthreads(); // everyone is done reading the previous exchange
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        lds[tid * E + e] = k[e];
+                    __syncthreads();
+#pragma unroll
+                    for (int e = 0; e < E; ++e)
+                        other[e] = lds[(tid * E + e) ^ j];
+                }
+                // the lower rank of a pair keeps the larger key where the run is descending
+                const bool lower = ((tid * E) & j) == 0, descending = ((tid * E) & kk) == 0;
+                const bool keepMax = lower == descending;
+#pragma unroll
+                for (int e = 0; e < E; ++e) {
+                    const bool otherLarger = other[e] > k[e];
+                    k[e] = (otherLarger == keepMax) ? other[e] : k[e];
+                }
+            }
+        });
+    });
+}
+
+// Any index vector: keys and columns in LDS, one pass over LDS per stage.
+template <int N>
+__device__ inline void SortInLds(uint64_t *key, uint16_t *pos, int tid)
+{
+    const int wave = tid / 64, lane = tid % 64;
     constexpr int kChunk = N / kTopkWaves, kPairsPerWave = kChunk / 2;
     for (int k = 2; k <= N; k <<= 1)
         for (int j = k >> 1; j > 0; j >>= 1) {
@@ -66,10 +135,73 @@ __global__ __launch_bounds__(kTopkThreads) void TopkRows(float *outScore, uint32
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // this wave's exchanges are done before its next stage reads them
         }
     __syncthreads();
+}
+
+// E: keys per thread; the row is padded to N = 256 E keys (padding keys are 0, below every real key).
+template <int E>
+__global__ __launch_bounds__(kTopkThreads) void TopkRows(float *outScore, uint32_t *outIndex, const float *src, const uint32_t *inIdx,
+                                                         int validCols, int ld, int topk)
+{
+    constexpr int N = kTopkThreads * E;
+    __shared__ uint64_t key[N];
+    __shared__ uint16_t pos[N];
+    const int tid = threadIdx.x;
+    const float *row = src + (size_t)blockIdx.x * (size_t)ld;
+    float *rowScore = outScore + (size_t)blockIdx.x * (size_t)topk;
+    uint32_t *rowIndex = outIndex + (size_t)blockIdx.x * (size_t)topk;
+
+    // do the indices increase with the column?  (then the column decides among equal scores, as the index would)
+    bool increasing = true;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int i = tid * E + e;
+        if (i + 1 < validCols)
+            increasing = increasing && inIdx[i] < inIdx[i + 1];
+    }
+    bool inRegisters = false;
+    if constexpr (E <= 8)
+        inRegisters = __syncthreads_and(increasing) != 0;
+    if constexpr (E <= 8) if (inRegisters) {
+        uint64_t k[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int i = tid * E + e;
+            k[e] = 0;
+            if (i < validCols) {
+                const uint32_t b = __float_as_uint(row[i]);
+                const bool negZero = b == 0x80000000u; // compares equal to +0: same key, remembered below the column bits
+                k[e] = ((uint64_t)ScoreOrder(negZero ? 0u : b) << 32) | ((uint32_t)(4095 - i) << 20) | (negZero ? 1u : 0u);
+            }
+        }
+        SortInRegisters<E>(k, key, tid);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int i = tid * E + e;
+            if (i < topk) {
+                const uint32_t low = (uint32_t)k[e];
+                rowScore[i] = __uint_as_float((low & 1u) ? 0x80000000u : ScoreBits((uint32_t)(k[e] >> 32)));
+                rowIndex[i] = inIdx[4095 - (int)(low >> 20)];
+            }
+        }
+        return;
+    }
+    for (int i = tid; i < N; i += kTopkThreads) {
+        uint64_t kv = 0;
+        if (i < validCols) {
+            uint32_t b = __float_as_uint(row[i]);
+            if (b == 0x80000000u)
+                b = 0; // -0 and +0 compare equal
+            kv = ((uint64_t)ScoreOrder(b) << 32) | (uint32_t)~inIdx[i];
+        }
+        key[i] = kv;
+        pos[i] = (uint16_t)i;
+    }
+    __syncthreads();
+    SortInLds<N>(key, pos, tid);
     for (int i = tid; i < topk; i += kTopkThreads) {
         const int p = pos[i];
-        outScore[(size_t)blockIdx.x * (size_t)topk + i] = row[p];
-        outIndex[(size_t)blockIdx.x * (size_t)topk + i] = inIdx[p];
+        rowScore[i] = row[p];
+        rowIndex[i] = inIdx[p];
     }
 }
 
@@ -83,16 +215,16 @@ extern "C" int pto_topk_f32(void *stream, float *out_score, uint32_t *out_index,
     if (ld < valid_cols || topk > valid_cols || valid_cols > 4096)
         return PTO_ERR_UNSUPPORTED;
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define PTO_TOPK_CASE(NN)                                                                                              \
-    if (valid_cols <= NN) {                                                                                            \
-        TopkRows<NN><<<dim3(rows), dim3(kTopkThreads), 0, st>>>(out_score, out_index, src, in_idx, valid_cols, ld, topk); \
+#define PTO_TOPK_CASE(EE)                                                                                              \
+    if (valid_cols <= kTopkThreads * EE) {                                                                             \
+        TopkRows<EE><<<dim3(rows), dim3(kTopkThreads), 0, st>>>(out_score, out_index, src, in_idx, valid_cols, ld, topk); \
         return pto_amd::check_launch();                                                                                \
     }
-    PTO_TOPK_CASE(256)
-    PTO_TOPK_CASE(512)
-    PTO_TOPK_CASE(1024)
-    PTO_TOPK_CASE(2048)
-    PTO_TOPK_CASE(4096)
+    PTO_TOPK_CASE(1)
+    PTO_TOPK_CASE(2)
+    PTO_TOPK_CASE(4)
+    PTO_TOPK_CASE(8)
+    PTO_TOPK_CASE(16)
 #undef PTO_TOPK_CASE
     return PTO_ERR_UNSUPPORTED;
 }

@@ -47,8 +47,16 @@ def test_topk_ties_signed_zeros_infinities_and_arbitrary_indices(oracle):
     idx[0] = 0xFFFFFFFF
     for k in (1, 100, cols):
         assert same(topk_gpu(src, idx, cols, k), oracle.topk_f32(src, idx, cols, k))
-    mono = np.arange(cols, dtype=np.uint32)
-    assert same(topk_gpu(src, mono, cols, cols), oracle.topk_f32(src, mono, cols, cols))
+    # indices that increase with the column (the register-resident network; the rows above went through LDS)
+    for mono in (np.arange(cols, dtype=np.uint32), (np.arange(cols, dtype=np.uint32) * 3 + 7) ** 2):
+        for k in (1, 100, cols):
+            assert same(topk_gpu(src, mono, cols, k), oracle.topk_f32(src, mono, cols, k))
+    # and with other row lengths (1, 2, 8 keys per thread; padded rows)
+    for c in (200, 512, 1900):
+        s2, _ = datagen.topk_inputs(4, c, c + 8, distinct=5)
+        s2[1, ::9] = -0.0
+        for mono in (np.arange(c, dtype=np.uint32), r.permutation(1 << 16)[:c].astype(np.uint32)):
+            assert same(topk_gpu(s2, mono, c, c), oracle.topk_f32(s2, mono, c, c))
 
 
 def test_topk_reference_config_4800x1024_top1000(oracle):
