@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the PTO tile compute path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|mx|fa|tcvt|gather]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|mx|fa|tcvt|gather|topk]
 
 A step is one pass of the hot path over one batch of synthetic input, resident in HBM before the
 timed region: one fp16 -> fp32 GEMM at m=n=k=6144 (the configuration the headline metric is quoted
@@ -80,6 +80,23 @@ def bench_gemm_mx(torch, lib, capi, datagen, m, n, k, fmt, steps, warmup):
     ms = time_launches(torch, step, steps, warmup)
     flops = 2.0 * m * n * k
     return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
+
+
+def bench_topk(torch, lib, capi, datagen, steps, warmup):
+    """Row-wise top-k of the reference's topk kernel: 4800 rows of 1024 scores (row stride 1280), top 1000."""
+    import numpy as np
+    rows, cols, ld, k = 4800, 1024, 1280, 1000
+    src, idx = datagen.topk_inputs(rows, cols, ld)
+    ts, ti = torch.from_numpy(src).cuda(), torch.from_numpy(idx.view(np.int32)).cuda()
+    out_s = torch.empty((rows, k), dtype=torch.float32, device="cuda")
+    out_i = torch.empty((rows, k), dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        capi.check(lib.pto_topk_f32(st, out_s.data_ptr(), out_i.data_ptr(), ts.data_ptr(), ti.data_ptr(), rows, cols, ld, k), "topk")
+    ms = time_launches(torch, step, steps, warmup)
+    nbytes = rows * cols * 4 + rows * k * 8      # scores read once, scores + indices written
+    return {"ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9, "rows_per_s": rows / (ms * 1e-3)}
 
 
 def bench_fa(torch, lib, capi, datagen, cfg, steps, warmup):
@@ -172,7 +189,8 @@ def cpu_baseline(datagen, size):
 
 def cpu_baselines_extra(datagen, cores):
     """The oracle timed on bounded samples of the other workloads (reported beside the GPU figures, nothing more):
-    attention = the first 2048 query rows of one head of each configuration; TCVT = 2^24 elements; gather = 8192 rows."""
+    attention = the first 2048 query rows of one head of each configuration; TCVT = 2^24 elements; gather = 8192 rows;
+    top-k = 480 rows; MX GEMMs = a 64 x 2048 x 6144 block."""
     import numpy as np
     from oracle import oracle
     out = {}
@@ -196,6 +214,18 @@ def cpu_baselines_extra(datagen, cores):
     oracle.gather_rows(table, idx)
     dt = time.perf_counter() - t0
     out["gather_rows"] = {"gbs": (8192 * 1024 * 2 * 2 + 8192 * 4.0) / dt / 1e9, "cores": 1, "kind": "port", "sample": "8192 rows of 1024 fp16, %.3f s" % dt}
+    src, tidx = datagen.topk_inputs(480, 1024, 1280)
+    t0 = time.perf_counter()
+    oracle.topk_f32(src, tidx, 1024, 1000)
+    dt = time.perf_counter() - t0
+    out["topk_1024_top1000"] = {"rows_per_s": 480 / dt, "cores": 1, "kind": "port", "sample": "480 rows, %.3f s" % dt}
+    for name, fmt in (("gemm_mxfp8_e5m2", 1), ("gemm_mxfp4_e2m1", 4)):
+        a, b, sa, sb = datagen.mx_inputs(64, 2048, 6144, fmt)
+        t0 = time.perf_counter()
+        oracle.mx_gemm(a, b, sa, sb, fmt, threads=cores)
+        dt = time.perf_counter() - t0
+        out[name] = {"tflops": 2.0 * 64 * 2048 * 6144 / dt / 1e12, "cores": cores, "kind": "port",
+                     "sample": "64 x 2048 x 6144 (float64 accumulation), %.2f s" % dt}
     return out
 
 
@@ -205,7 +235,7 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="gemm | mx | fa | tcvt | gather: time just that workload")
+    ap.add_argument("--only", default="", help="gemm | mx | fa | tcvt | gather | topk: time just that workload")
     ap.add_argument("--size", type=int, default=6144)
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -253,6 +283,10 @@ def main():
         for kind in ("f16", "bf16"):
             r = bench_tcvt(torch, lib, capi, datagen, args.steps, args.warmup, kind)
             extra["tcvt_f32_%s_16384x8192" % kind] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS}
+    if only in ("", "topk"):
+        r = bench_topk(torch, lib, capi, datagen, args.steps, args.warmup)
+        extra["topk_4800x1024_top1000_f32"] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS,
+                                               "rows_per_s": r["rows_per_s"]}
     if only in ("", "gather"):
         r = bench_gather(torch, lib, capi, datagen, args.steps, args.warmup)
         extra["gather_rows_65536x1024_f16"] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS}
