@@ -33,11 +33,22 @@ GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369559.0, 2.0
 GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 147901.0, 1.0
 
 
-def time_launches(torch, fn, steps, warmup):
-    """Average duration in ms of fn() over `steps` launches on torch's current stream (HIP events)."""
+SETTLE_S = 0.0   # set from --settle-ms: the workloads under "extra" keep warming up until this much time has passed
+
+
+def time_launches(torch, fn, steps, warmup, settle_s=None):
+    """Average duration in ms of fn() over `steps` launches on torch's current stream (HIP events), after `warmup`
+    untimed launches and, where settle_s is set, further untimed launches until that much wall time has passed (a
+    launch of 0.1 ms repeated 30 times does not bring the GPU out of its idle clocks)."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
+    settle_s = SETTLE_S if settle_s is None else settle_s
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < settle_s:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
     start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(steps):
@@ -47,7 +58,7 @@ def time_launches(torch, fn, steps, warmup):
     return start.elapsed_time(end) / steps
 
 
-def bench_gemm(torch, lib, capi, datagen, size, steps, warmup):
+def bench_gemm(torch, lib, capi, datagen, size, steps, warmup, settle_s=None):
     import numpy as np
     a, b = datagen.gemm_inputs(size, size, size)
     ta = torch.from_numpy(a.view(np.int16)).cuda()
@@ -57,7 +68,7 @@ def bench_gemm(torch, lib, capi, datagen, size, steps, warmup):
 
     def step():
         capi.check(lib.pto_gemm_f16f32(st, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), size, size, size), "gemm")
-    ms = time_launches(torch, step, steps, warmup)
+    ms = time_launches(torch, step, steps, warmup, settle_s)
     flops = 2.0 * size ** 3
     return {"ms": ms, "tflops": flops / (ms * 1e-3) / 1e12, "flops": flops}
 
@@ -233,7 +244,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--settle-ms", type=float, default=300.0,
+                    help="workloads under \"extra\": after the warm-up launches keep launching untimed until this much time has passed")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--only", default="", help="gemm | mx | fa | tcvt | gather | topk: time just that workload")
     ap.add_argument("--size", type=int, default=6144)
@@ -246,6 +259,8 @@ def main():
 
     import torch
     from pto_amd import capi, datagen
+    global SETTLE_S
+    SETTLE_S = max(args.settle_ms, 0.0) * 1e-3
     lib = capi.load()
     capi.check(lib.pto_init(), "pto_init")
     torch.cuda.set_device(0)
@@ -254,13 +269,13 @@ def main():
     if args.calib_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
         dst = torch.empty_like(src)
-        ms = time_launches(torch, lambda: dst.copy_(src), 5, 2)
+        ms = time_launches(torch, lambda: dst.copy_(src), 5, 2, settle_s=0.0)
         extra["calib_copy_1GiB"] = {"ms": ms, "gbs": 2.0 * src.numel() * 4 / (ms * 1e-3) / 1e9, "bytes_read": src.numel() * 4,
                                     "bytes_written": src.numel() * 4}
     only = args.only
     gemm = None
     if only in ("", "gemm"):
-        gemm = bench_gemm(torch, lib, capi, datagen, args.size, args.steps, args.warmup)
+        gemm = bench_gemm(torch, lib, capi, datagen, args.size, args.steps, args.warmup, settle_s=0.0)   # exactly W warm-ups
     if only == "":
         for s in (3072, 7680):
             r = bench_gemm(torch, lib, capi, datagen, s, max(args.steps // 2, 1), 2)
@@ -308,6 +323,8 @@ def main():
                                "(256x256 C tile per workgroup, K-step 32)" % args.size},
         "extra": extra,
     }
+    extra["warmup_policy"] = ("headline: exactly %d untimed launches; workloads under extra: %d launches, then untimed launches "
+                              "until %.0f ms have passed" % (args.warmup, args.warmup, args.settle_ms))
     traffic = None
     if gemm and args.size == 6144:
         rd = GEMM_6144_FETCH_KIB * GEMM_6144_FETCH_SCALE * 1024.0
