@@ -29,8 +29,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 # counter reads for a plain 1 GiB device copy in the same run (--calib-copy): FETCH_SIZE reads
 # 524,300 KiB for 1,048,576 KiB actually read (factor 2.0), WRITE_SIZE reads 1,048,576 KiB for
 # 1,048,576 KiB written (factor 1.0).
-GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369559.0, 2.0
-GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 147901.0, 1.0
+GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369647.0, 2.0
+GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 147905.0, 1.0
 
 
 SETTLE_S = 0.0   # set from --settle-ms: the workloads under "extra" keep warming up until this much time has passed
