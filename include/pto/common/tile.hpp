@@ -28,6 +28,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 namespace detail {
 
@@ -37,6 +38,15 @@ constexpr int kMfmaK = 512 / kMfmaM;                   // k extent of one MFMA
 constexpr int kAccElems = kMfmaM * kMfmaM / kWaveSize; // accumulator values per lane and block
 constexpr int kVecChunk = 8;
 typedef float AccFrag __attribute__((ext_vector_type(kAccElems)));
+typedef int AccFragI32 __attribute__((ext_vector_type(kAccElems)));
+template <typename T>
+struct AccFragOf {
+    using type = AccFrag;
+};
+template <>
+struct AccFragOf<int32_t> {
+    using type = AccFragI32;
+};
 
 // Operand layout (both shapes): lane l holds row (column) l % kMfmaM of the block and the eight k values
 // 8 * (l / kMfmaM) .. +7 of the step.  Result layout: lane l holds column l % kMfmaM and, in register v,
@@ -59,6 +69,23 @@ template <>
 struct FragOf<__bf16> {
     using type = bf16x8;
 };
+template <>
+struct FragOf<int8_t> {
+    using type = i32x4;
+};
+template <>
+struct FragOf<float> {
+    using type = f32x4;
+};
+// Operand element types of the plain (unscaled) MFMAs.  Whatever the type, a lane holds 16 bytes of its row per
+// fragment: 8 fp16 / bf16, 16 int8 or 4 fp32 values; the lanes of a row cover 64 / PTO_MFMA_M such chunks, which is the
+// k extent of one fragment (fp16: one MFMA; int8: one MFMA of twice the k; fp32: four MFMAs, MFMA s taking value s of
+// every lane's chunk - the same assignment of k to MFMAs on both operands, so the sum over k is unchanged).
+template <typename T>
+constexpr bool is_mfma_operand_v = std::is_same_v<T, _Float16> || std::is_same_v<T, __bf16> || std::is_same_v<T, int8_t> ||
+                                   std::is_same_v<T, float>;
+template <typename T>
+constexpr int kFragK = (16 / (int)sizeof(T)) * (kWaveSize / kMfmaM);
 
 constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 
@@ -150,32 +177,32 @@ struct TileStorage<TileType::ScaleRight, T, Rows, Cols> {
 
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Left, T, Rows, Cols> {
-    static_assert(sizeof(T) == 2, "Left tiles: fp16 / bf16 operands");
+    static_assert(is_mfma_operand_v<T>, "Left tiles: fp16, bf16, int8 or fp32 operands (fp8 / fp4 for TMATMUL_MX)");
     static_assert(Rows % (kMfmaM * kWavesM) == 0, "Left tile rows must be a multiple of PTO_MFMA_M x PTO_WAVES_M");
-    static_assert(Cols % kMfmaK == 0, "Left tile cols (K) must be a multiple of the MFMA's k extent");
+    static_assert(Cols % kFragK<T> == 0, "Left tile cols (K) must be a multiple of the k extent of a fragment");
     static constexpr int MB = Rows / (kMfmaM * kWavesM);
-    static constexpr int KS = Cols / kMfmaK;
+    static constexpr int KS = Cols / kFragK<T>;
     typename FragOf<T>::type f[MB][KS];
 };
 
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Right, T, Rows, Cols> {
-    static_assert(sizeof(T) == 2, "Right tiles: fp16 / bf16 operands");
+    static_assert(is_mfma_operand_v<T>, "Right tiles: fp16, bf16, int8 or fp32 operands (fp8 / fp4 for TMATMUL_MX)");
     static_assert(Cols % (kMfmaM * kWavesN) == 0, "Right tile cols must be a multiple of PTO_MFMA_M x PTO_WAVES_N");
-    static_assert(Rows % kMfmaK == 0, "Right tile rows (K) must be a multiple of the MFMA's k extent");
+    static_assert(Rows % kFragK<T> == 0, "Right tile rows (K) must be a multiple of the k extent of a fragment");
     static constexpr int NB = Cols / (kMfmaM * kWavesN);
-    static constexpr int KS = Rows / kMfmaK;
+    static constexpr int KS = Rows / kFragK<T>;
     typename FragOf<T>::type f[NB][KS];
 };
 
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Acc, T, Rows, Cols> {
-    static_assert(sizeof(T) == 4, "Acc tiles: fp32 accumulators");
+    static_assert(std::is_same_v<T, float> || std::is_same_v<T, int32_t>, "Acc tiles: fp32 or int32 accumulators");
     static_assert(Rows % (kMfmaM * kWavesM) == 0 && Cols % (kMfmaM * kWavesN) == 0,
                   "Acc tile must be a multiple of (PTO_MFMA_M x PTO_WAVES_M) x (PTO_MFMA_M x PTO_WAVES_N)");
     static constexpr int MB = Rows / (kMfmaM * kWavesM);
     static constexpr int NB = Cols / (kMfmaM * kWavesN);
-    AccFrag f[MB][NB];
+    typename AccFragOf<T>::type f[MB][NB];
 };
 
 template <typename T, int Rows, int Cols>

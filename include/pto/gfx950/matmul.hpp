@@ -1,8 +1,9 @@
 // TMATMUL / TMATMUL_ACC / TMATMUL_BIAS for gfx950: chains of v_mfma_f32_32x32x16_{f16,bf16} (or, with
-// PTO_MFMA_M 16, v_mfma_f32_16x16x32_{f16,bf16}).
+// PTO_MFMA_M 16, v_mfma_f32_16x16x32_{f16,bf16}); int8 x int8 -> int32 on v_mfma_i32_32x32x32_i8 / 16x16x64 and
+// fp32 x fp32 -> fp32 on v_mfma_f32_32x32x2_f32 / 16x16x4 (the type triples of include/pto/cpu/TMatmul.hpp:46-51).
 //
 // Reference semantics (include/pto/cpu/TMatmul.hpp:73-116):
-//   C[i,j] = (acc ? acc[i,j] : 0) + sum_k (float)A[i,k] * (float)B[k,j],  M,K,N = a.validRow, a.validCol, b.validCol
+//   C[i,j] = (acc ? acc[i,j] : 0) + sum_k (CT)A[i,k] * (CT)B[k,j],  M,K,N = a.validRow, a.validCol, b.validCol
 // Each wave owns the (Rows/PTO_WAVES_M) x (Cols/PTO_WAVES_N) sub-block of C selected by its
 // position in the wave grid and holds the matching rows of A / columns of B as fragments.
 // Products are exact in fp32; the order of the fp32 additions inside an MFMA differs from the
@@ -34,14 +35,41 @@ PTO_DEV C mfma32(bf16x8 a, bf16x8 b, C c)
         return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
 }
 
+// one 16-byte chunk per lane of each operand: 16 int8 values, one MFMA of twice the fp16 k extent
+template <typename C>
+PTO_DEV C mfma32(i32x4 a, i32x4 b, C c)
+{
+    static_assert(std::is_same_v<C, AccFragI32>, "int32 accumulator fragment of the configured MFMA shape");
+    if constexpr (sizeof(C) == 64)
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+}
+// 4 fp32 values per lane: four MFMAs, MFMA s takes value s of every lane's chunk
+template <typename C>
+PTO_DEV C mfma32(f32x4 a, f32x4 b, C c)
+{
+    static_assert(std::is_same_v<C, AccFrag>, "accumulator fragment of the configured MFMA shape");
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        if constexpr (sizeof(C) == 64)
+            c = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], c, 0, 0, 0);
+        else
+            c = __builtin_amdgcn_mfma_f32_16x16x4f32(a[s], b[s], c, 0, 0, 0);
+    }
+    return c;
+}
+
 template <typename AccT, typename LeftT, typename RightT>
 PTO_DEV constexpr void check_mad()
 {
     using A = typename LeftT::DType;
     using B = typename RightT::DType;
-    static_assert(std::is_same_v<A, B> && (std::is_same_v<A, half> || std::is_same_v<A, bfloat16_t>) &&
-                      std::is_same_v<typename AccT::DType, float>,
-                  "[PTO][SA] TMATMUL on gfx950: fp16 x fp16 -> fp32 or bf16 x bf16 -> fp32");
+    using CT = typename AccT::DType;
+    static_assert(std::is_same_v<A, B> &&
+                      (((std::is_same_v<A, half> || std::is_same_v<A, bfloat16_t> || std::is_same_v<A, float>) && std::is_same_v<CT, float>) ||
+                       (std::is_same_v<A, int8_t> && std::is_same_v<CT, int32_t>)),
+                  "[PTO][SA] TMATMUL on gfx950: fp16 / bf16 / fp32 operands -> fp32, or int8 x int8 -> int32");
     static_assert(LeftT::Loc == TileType::Left && RightT::Loc == TileType::Right && AccT::Loc == TileType::Acc,
                   "[PTO][SA] TMATMUL: operands must be Left, Right and Acc tiles");
     static_assert(LeftT::Rows == AccT::Rows && LeftT::Cols == RightT::Rows && RightT::Cols == AccT::Cols,
@@ -55,15 +83,16 @@ PTO_DEV void mad(AccT &out, const AccT &in, const LeftT &a, const RightT &b)
 {
     using SA = typename AccT::Storage;
     using SL = typename LeftT::Storage;
+    using CFrag = typename AccFragOf<typename AccT::DType>::type;
 #pragma unroll
     for (int mb = 0; mb < SA::MB; ++mb)
 #pragma unroll
         for (int nb = 0; nb < SA::NB; ++nb) {
-            AccFrag c;
+            CFrag c;
             if constexpr (kZeroInit) {
 #pragma unroll
                 for (int i = 0; i < kAccElems; ++i)
-                    c[i] = 0.0f;
+                    c[i] = 0;
             } else {
                 c = in.st.f[mb][nb];
             }

@@ -381,8 +381,8 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
 
 // ----------------------------------------------------------------- TEXTRACT
 // dst[i,j] = src[idxRow+i, idxCol+j].  Mat -> Left / Right: one ds_read_b128 per row block and k step, in the
-// MFMA operand layout (lane l: row/col l % kMfmaM, k = 8*(l / kMfmaM)..+7).
-// The k offset must be a multiple of 8 elements (16 bytes).
+// MFMA operand layout (lane l: row/col l % kMfmaM, the 16-byte chunk l / kMfmaM of the step: 8 fp16 / bf16, 16 int8 or
+// 4 fp32 values).  The k offset must be a multiple of 16 bytes.
 namespace detail {
 // Mat -> Left / Right of an MX operand.  8-bit: two ds_read_b128 per 32-row block and 64-wide k step (lane l: row
 // l % 32, bytes 16 (l / 32) .. +15 and 32 + 16 (l / 32) .. +15 of the step).  4-bit: one ds_read_b128 (bytes
@@ -475,12 +475,14 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
     const char *lds = hw::lds_base() + src.st.lds;
     const uint32_t lane = (uint32_t)hw::lane();
     const uint32_t l32 = detail::frag_lane_major(lane), khalf = detail::frag_lane_kgroup(lane);
-    constexpr uint32_t kStepChunks = detail::kMfmaK / 8; // 16-byte chunks per k step
+    using ElemT = typename DstT::DType;
+    constexpr uint32_t kStepChunks = kWaveSize / detail::kMfmaM; // 16-byte chunks per fragment (one per lane group)
+    constexpr uint32_t kChunkElems = 16 / sizeof(ElemT);
     if constexpr (DstT::Loc == TileType::Left) {
         static_assert(Geo::colsK, "[PTO][SA] TEXTRACT to Left: source must be contiguous along columns (Nz / row-major)");
         using S = typename DstT::Storage;
         const uint32_t row0 = idxRow + (uint32_t)hw::wave_m() * (S::MB * detail::kMfmaM) + l32;
-        const uint32_t chunk0 = (idxCol >> 3) + khalf;
+        const uint32_t chunk0 = idxCol / kChunkElems + khalf;
 #pragma unroll
         for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
@@ -491,7 +493,7 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
         static_assert(!Geo::colsK, "[PTO][SA] TEXTRACT to Right: source must be contiguous along rows (Zn / column-major)");
         using S = typename DstT::Storage;
         const uint32_t col0 = idxCol + (uint32_t)hw::wave_n() * (S::NB * detail::kMfmaM) + l32;
-        const uint32_t chunk0 = (idxRow >> 3) + khalf;
+        const uint32_t chunk0 = idxRow / kChunkElems + khalf;
 #pragma unroll
         for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll

@@ -273,6 +273,38 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulBias(__gm__ float 
     TSTORE(gc, c, computed);
 }
 
+// ---- one-block matmul [128, K] x [K, 256] for the other operand types of TMATMUL: int8 -> int32, fp32 -> fp32 ----
+// (tests/cpu/st/testcase/tmatmul/tmatmul_kernel.cpp with the int8 and float cases of its gen_data.py:92-99).  K is taken
+// in two halves: TMATMUL on the first, TMATMUL_ACC on the second.
+template <typename T, typename CT, int K>
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulTyped(__gm__ CT *out, __gm__ const T *a, __gm__ const T *bT)
+{
+    constexpr int KH = K / 2;
+    using MatA = Tile<TileType::Mat, T, 128, K, BLayout::ColMajor, 128, K, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, T, K, 256, BLayout::RowMajor, K, 256, SLayout::ColMajor>;
+    MatA am;
+    MatB bm;
+    TASSIGN(am, 0u);
+    TASSIGN(bm, 128u * K * sizeof(T));
+    TileLeft<T, 128, KH> l;
+    TileRight<T, KH, 256> r;
+    TileAcc<CT, 128, 256> c;
+    GmND<T, 128, K> ga(const_cast<T *>(a));
+    GlobalTensor<T, Shape<1, 1, 1, K, 256>, Stride<1, 1, 1, 1, K>, Layout::DN> gb(const_cast<T *>(bT));
+    GmND<CT, 128, 256> gc(out);
+    TLOAD(am, ga);
+    TLOAD(bm, gb);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    TEXTRACT(l, am, 0, 0);
+    TEXTRACT(r, bm, 0, 0);
+    TMATMUL(c, l, r);
+    TEXTRACT(l, am, 0, KH);
+    TEXTRACT(r, bm, KH, 0);
+    TMATMUL_ACC(c, c, l, r);
+    TSTORE(gc, c);
+}
+
 // ---- one-block MX matmul [128, 256] x [256, 128], fp8 operands (formats may differ) with e8m0 block scales ----
 // (tests/npu/a5/src/st/testcase/tmatmul_mx/tmatmul_mx_kernel.cpp: TLOAD -> TEXTRACT -> TMATMUL_MX -> TSTORE).  K is taken
 // in two halves of 128: TMATMUL_MX on the first, the accumulating form on the second.  VIA_MAT == false: the scale tiles
@@ -681,6 +713,22 @@ extern "C" int pto_st_textract_windows_f16(void *stream, float *out_left, float 
     ExtractWindows<<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(
         out_left, out_right, reinterpret_cast<const half *>(a), reinterpret_cast<const half *>(b_t),
         reinterpret_cast<const half *>(eye_b), reinterpret_cast<const half *>(eye_a), col0, row0);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_matmul_s8_128x128x256(void *stream, int32_t *out, const int8_t *a, const int8_t *b_t)
+{
+    PTO_ST_NONNULL(out, a, b_t);
+    constexpr int lds = 128 * 128 + 128 * 256;
+    MatmulTyped<int8_t, int32_t, 128><<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(out, a, b_t);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_matmul_f32_128x32x256(void *stream, float *out, const float *a, const float *b_t)
+{
+    PTO_ST_NONNULL(out, a, b_t);
+    constexpr int lds = (128 * 32 + 32 * 256) * 4;
+    MatmulTyped<float, float, 32><<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(out, a, b_t);
     return pto_amd::check_launch();
 }
 

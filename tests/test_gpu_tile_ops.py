@@ -278,3 +278,60 @@ def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b, via_lds):
             assert np.array_equal(got, want), (dist, fmt_a, fmt_b)
         else:
             assert np.max(np.abs(got - want)) <= 2e-3 * np.max(np.abs(want)), (dist, fmt_a, fmt_b)
+
+
+def test_tmatmul_int8_to_int32(oracle):
+    """int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), TMATMUL then TMATMUL_ACC over two k halves: exact."""
+    lib = capi.load()
+    rng = np.random.default_rng(23)
+    a = rng.integers(-128, 128, size=(128, 128), dtype=np.int8)
+    b = rng.integers(-128, 128, size=(128, 256), dtype=np.int8)
+    a[0, :] = -128
+    b[:, 0] = -128                                               # the extreme product, 128 times
+    out = torch.full((128, 256), -1, dtype=torch.int32, device=DEV)
+    ta, tb = torch.from_numpy(a).to(DEV), torch.from_numpy(np.ascontiguousarray(b.T)).to(DEV)
+    capi.check(lib.pto_st_matmul_s8_128x128x256(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr()), "matmul s8")
+    torch.cuda.synchronize()
+    want = a.astype(np.int32) @ b.astype(np.int32)
+    assert np.array_equal(out.cpu().numpy(), want)
+    o = oracle
+    La, Lb = o.make_layout(128, 128, o.BL_COL, o.SL_ROW, 1), o.make_layout(128, 256, o.BL_ROW, o.SL_COL, 1)
+    Lc = o.make_layout(128, 256, o.BL_COL, o.SL_ROW, 4, 1024)
+    tA = o.tload(La, np.int8, a, [1, 1, 1, 128, 128], [0, 0, 0, 128, 1])
+    tB = o.tload(Lb, np.int8, b, [1, 1, 1, 128, 256], [0, 0, 0, 256, 1])
+    acc = o.tmatmul(tA, La, tB, Lb, Lc, 128, 256, 128)
+    ref = np.zeros((128, 256), dtype=np.int32)
+    o.tstore(ref, [1, 1, 1, 128, 256], [0, 0, 0, 256, 1], acc, Lc)
+    assert np.array_equal(out.cpu().numpy(), ref)
+
+
+def test_tmatmul_fp32(oracle):
+    """fp32 x fp32 -> fp32 (v_mfma_f32_32x32x2_f32): exact on integers, fp32 rounding only otherwise."""
+    lib = capi.load()
+    rng = np.random.default_rng(29)
+    for integer in (True, False):
+        if integer:
+            a = rng.integers(-9, 10, size=(128, 32)).astype(np.float32)
+            b = rng.integers(-9, 10, size=(32, 256)).astype(np.float32)
+        else:
+            a = rng.standard_normal((128, 32)).astype(np.float32)
+            b = rng.standard_normal((32, 256)).astype(np.float32)
+        out = torch.full((128, 256), float("nan"), device=DEV)
+        ta, tb = dev(a), dev(np.ascontiguousarray(b.T))
+        capi.check(lib.pto_st_matmul_f32_128x32x256(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr()), "matmul f32")
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        if integer:
+            assert np.array_equal(got, want.astype(np.float32))
+        else:
+            assert np.max(np.abs(got - want)) <= 1e-5 * np.max(np.abs(want))
+            o = oracle
+            La, Lb = o.make_layout(128, 32, o.BL_COL, o.SL_ROW, 4), o.make_layout(32, 256, o.BL_ROW, o.SL_COL, 4)
+            Lc = o.make_layout(128, 256, o.BL_COL, o.SL_ROW, 4, 1024)
+            tA = o.tload(La, np.float32, a, [1, 1, 1, 128, 32], [0, 0, 0, 32, 1])
+            tB = o.tload(Lb, np.float32, b, [1, 1, 1, 32, 256], [0, 0, 0, 256, 1])
+            acc = o.tmatmul(tA, La, tB, Lb, Lc, 128, 256, 32)
+            ref = np.zeros((128, 256), dtype=np.float32)
+            o.tstore(ref, [1, 1, 1, 128, 256], [0, 0, 0, 256, 1], acc, Lc)
+            assert np.max(np.abs(got - ref)) <= 1e-5 * np.max(np.abs(ref))
