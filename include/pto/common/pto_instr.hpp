@@ -158,6 +158,28 @@ PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
     TSTORE_IMPL<TileT, G, atomic>(dst, src);
     return {};
 }
+// (pto_instr.hpp:183-207 of the reference: atomic type + unit-flag phase, atomic type + ReLU, all three)
+template <typename TileT, typename G, AtomicType atomic, STPhase Phase, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TSTORE_IMPL<TileT, G, atomic>(dst, src);
+    return {};
+}
+template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TSTORE_IMPL<TileT, G, atomic, relu>(dst, src);
+    return {};
+}
+template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu, STPhase Phase, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TSTORE_IMPL<TileT, G, atomic, relu>(dst, src);
+    return {};
+}
 template <typename D, typename S, typename... Ev>
 PTO_INST RecordEvent TEXTRACT(D &dst, S &src, Ev &... ev)
 {

@@ -558,7 +558,7 @@ PTO_DEV D store_cast(S v)
 
 // Acc fragments -> GM.  MFMA result layout: lane l, register v holds row acc_elem_row(v) + acc_lane_row(l),
 // column l % kMfmaM of the block (32 x 32: row 8*(v/4) + 4*(l/32) + v%4).
-template <typename TileT, typename G, AtomicType atomic>
+template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu = ReluPreMode::NoRelu>
 PTO_DEV void tstore_acc(G &dst, TileT &src)
 {
     using S = typename TileT::Storage;
@@ -580,10 +580,13 @@ PTO_DEV void tstore_acc(G &dst, TileT &src)
                 const int r = rbase + mb * kMfmaM + acc_elem_row(v);
                 if (full || (r < vr && c < vc)) {
                     GT *p = gm + (int64_t)r * st_r + (int64_t)c * st_c;
+                    auto x = src.st.f[mb][nb][v];
+                    if constexpr (relu == ReluPreMode::NormalRelu)
+                        x = x < 0 ? 0 : x; // before the conversion, as the fix pipe does (a2a3/TStore.hpp:328)
                     if constexpr (atomic == AtomicType::AtomicAdd)
-                        atomicAdd(p, store_cast<GT>(src.st.f[mb][nb][v]));
+                        atomicAdd(p, store_cast<GT>(x));
                     else
-                        *p = store_cast<GT>(src.st.f[mb][nb][v]);
+                        *p = store_cast<GT>(x);
                 }
             }
         }
@@ -653,11 +656,12 @@ PTO_DEV void tstore_mat(G &dst, TileT &src)
 
 } // namespace detail
 
-template <typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone>
+template <typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone, ReluPreMode relu = ReluPreMode::NoRelu>
 PTO_DEV void TSTORE_IMPL(G &dst, TileT &src)
 {
+    static_assert(relu == ReluPreMode::NoRelu || TileT::Loc == TileType::Acc, "[PTO][SA] TSTORE: ReLU applies to Acc tiles");
     if constexpr (TileT::Loc == TileType::Acc) {
-        detail::tstore_acc<TileT, G, atomic>(dst, src);
+        detail::tstore_acc<TileT, G, atomic, relu>(dst, src);
     } else if constexpr (TileT::Loc == TileType::Vec) {
         static_assert(sizeof(typename TileT::DType) == sizeof(typename G::DType), "[PTO][SA] TSTORE: element sizes differ");
         detail::tstore_vec(dst, src);

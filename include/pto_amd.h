@@ -142,9 +142,10 @@ int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, c
 
 /* [128,128] x [128,256] int8 -> int32 and [128,32] x [32,256] fp32 -> fp32 (the other operand types of TMATMUL,
  * include/pto/cpu/TMatmul.hpp:46-51; tests/cpu/st/testcase/tmatmul/gen_data.py:92-99): a row-major, b_t = b stored
- * [256][K] (column-major b); K in two halves, TMATMUL then TMATMUL_ACC. */
-int pto_st_matmul_s8_128x128x256(void *stream, int32_t *out, const int8_t *a, const int8_t *b_t);
-int pto_st_matmul_f32_128x32x256(void *stream, float *out, const float *a, const float *b_t);
+ * [256][K] (column-major b); K in two halves, TMATMUL then TMATMUL_ACC.  relu != 0: stored with
+ * TSTORE<..., ReluPreMode::NormalRelu, STPhase::Final> (negative results become 0). */
+int pto_st_matmul_s8_128x128x256(void *stream, int32_t *out, const int8_t *a, const int8_t *b_t, int relu);
+int pto_st_matmul_f32_128x32x256(void *stream, float *out, const float *a, const float *b_t, int relu);
 
 /* MX matmul [128,256] x [256,128] -> fp32 [128,128]: a [128,256] and b_t [128][256] (column-major b) fp8 bytes in
  * format_a / format_b (0 = e4m3, 1 = e5m2; they may differ), scale_a [128,8] and scale_b_t [128][8] e8m0 bytes; K in two

@@ -275,9 +275,10 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulBias(__gm__ float 
 
 // ---- one-block matmul [128, K] x [K, 256] for the other operand types of TMATMUL: int8 -> int32, fp32 -> fp32 ----
 // (tests/cpu/st/testcase/tmatmul/tmatmul_kernel.cpp with the int8 and float cases of its gen_data.py:92-99).  K is taken
-// in two halves: TMATMUL on the first, TMATMUL_ACC on the second.
+// in two halves: TMATMUL on the first, TMATMUL_ACC on the second.  relu: the store clamps negative results to zero
+// (TSTORE<..., AtomicType::AtomicNone, ReluPreMode::NormalRelu, STPhase::Final>).
 template <typename T, typename CT, int K>
-__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulTyped(__gm__ CT *out, __gm__ const T *a, __gm__ const T *bT)
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulTyped(__gm__ CT *out, __gm__ const T *a, __gm__ const T *bT, int relu)
 {
     constexpr int KH = K / 2;
     using MatA = Tile<TileType::Mat, T, 128, K, BLayout::ColMajor, 128, K, SLayout::RowMajor>;
@@ -302,7 +303,12 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulTyped(__gm__ CT *o
     TEXTRACT(l, am, 0, KH);
     TEXTRACT(r, bm, KH, 0);
     TMATMUL_ACC(c, c, l, r);
-    TSTORE(gc, c);
+    using AccT = TileAcc<CT, 128, 256>;
+    using GmC = GmND<CT, 128, 256>;
+    if (relu)
+        TSTORE<AccT, GmC, AtomicType::AtomicNone, ReluPreMode::NormalRelu, STPhase::Final>(gc, c);
+    else
+        TSTORE<AccT, GmC, AtomicType::AtomicNone, STPhase::Final>(gc, c);
 }
 
 // ---- one-block MX matmul [128, 256] x [256, 128], fp8 operands (formats may differ) with e8m0 block scales ----
@@ -716,19 +722,19 @@ extern "C" int pto_st_textract_windows_f16(void *stream, float *out_left, float 
     return pto_amd::check_launch();
 }
 
-extern "C" int pto_st_matmul_s8_128x128x256(void *stream, int32_t *out, const int8_t *a, const int8_t *b_t)
+extern "C" int pto_st_matmul_s8_128x128x256(void *stream, int32_t *out, const int8_t *a, const int8_t *b_t, int relu)
 {
     PTO_ST_NONNULL(out, a, b_t);
     constexpr int lds = 128 * 128 + 128 * 256;
-    MatmulTyped<int8_t, int32_t, 128><<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(out, a, b_t);
+    MatmulTyped<int8_t, int32_t, 128><<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(out, a, b_t, relu);
     return pto_amd::check_launch();
 }
 
-extern "C" int pto_st_matmul_f32_128x32x256(void *stream, float *out, const float *a, const float *b_t)
+extern "C" int pto_st_matmul_f32_128x32x256(void *stream, float *out, const float *a, const float *b_t, int relu)
 {
     PTO_ST_NONNULL(out, a, b_t);
     constexpr int lds = (128 * 32 + 32 * 256) * 4;
-    MatmulTyped<float, float, 32><<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(out, a, b_t);
+    MatmulTyped<float, float, 32><<<dim3(1), dim3(kBlockThreads), lds, static_cast<hipStream_t>(stream)>>>(out, a, b_t, relu);
     return pto_amd::check_launch();
 }
 

@@ -290,10 +290,14 @@ def test_tmatmul_int8_to_int32(oracle):
     b[:, 0] = -128                                               # the extreme product, 128 times
     out = torch.full((128, 256), -1, dtype=torch.int32, device=DEV)
     ta, tb = torch.from_numpy(a).to(DEV), torch.from_numpy(np.ascontiguousarray(b.T)).to(DEV)
-    capi.check(lib.pto_st_matmul_s8_128x128x256(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr()), "matmul s8")
+    capi.check(lib.pto_st_matmul_s8_128x128x256(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), 0), "matmul s8")
     torch.cuda.synchronize()
     want = a.astype(np.int32) @ b.astype(np.int32)
     assert np.array_equal(out.cpu().numpy(), want)
+    out_relu = torch.full((128, 256), -1, dtype=torch.int32, device=DEV)
+    capi.check(lib.pto_st_matmul_s8_128x128x256(st(), out_relu.data_ptr(), ta.data_ptr(), tb.data_ptr(), 1), "matmul s8 relu")
+    torch.cuda.synchronize()
+    assert np.array_equal(out_relu.cpu().numpy(), np.maximum(want, 0)) and (want < 0).any()
     o = oracle
     La, Lb = o.make_layout(128, 128, o.BL_COL, o.SL_ROW, 1), o.make_layout(128, 256, o.BL_ROW, o.SL_COL, 1)
     Lc = o.make_layout(128, 256, o.BL_COL, o.SL_ROW, 4, 1024)
@@ -318,9 +322,12 @@ def test_tmatmul_fp32(oracle):
             b = rng.standard_normal((32, 256)).astype(np.float32)
         out = torch.full((128, 256), float("nan"), device=DEV)
         ta, tb = dev(a), dev(np.ascontiguousarray(b.T))
-        capi.check(lib.pto_st_matmul_f32_128x32x256(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr()), "matmul f32")
+        capi.check(lib.pto_st_matmul_f32_128x32x256(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), 0), "matmul f32")
+        out_relu = torch.full((128, 256), float("nan"), device=DEV)
+        capi.check(lib.pto_st_matmul_f32_128x32x256(st(), out_relu.data_ptr(), ta.data_ptr(), tb.data_ptr(), 1), "matmul f32 relu")
         torch.cuda.synchronize()
         got = out.cpu().numpy()
+        assert np.array_equal(out_relu.cpu().numpy(), np.maximum(got, 0))
         want = a.astype(np.float64) @ b.astype(np.float64)
         if integer:
             assert np.array_equal(got, want.astype(np.float32))
