@@ -171,6 +171,10 @@ enum {
     PTO_VOP_COLEXPANDMAX, PTO_VOP_COLEXPANDMIN
 };
 int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const float *b, const float *vec, float scalar, int op);
+/* The arithmetic subset of the same (ABS NEG RELU, ADD SUB MUL MAX MIN, ADDS SUBS MULS MAXS MINS, the row / column
+ * expand forms without the divisions) on [64,128] fp16 (dtype 0) or int32 (dtype 1) tiles; same operation codes. */
+int pto_st_vec_op_typed_64x128(void *stream, void *out, const void *a, const void *b, const void *vec, float scalar, int op,
+                               int dtype);
 /* Reductions over the valid region [valid_rows, valid_cols] of a [64,128] fp32 tile (row stride 128 in memory):
  * op 0 TROWMAX, 1 TROWMIN, 2 TROWSUM -> out[valid_rows]; 3 TCOLMAX, 4 TCOLMIN, 5 TCOLSUM -> out[valid_cols]
  * (cpu/TRowMax.hpp, TRowMin.hpp, TRowSum.hpp, TColMax.hpp, TColMin.hpp, TColSum.hpp). */

@@ -787,6 +787,86 @@ extern "C" int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uin
     return pto_amd::check_launch();
 }
 
+// The arithmetic subset of the Vec instructions on fp16 and int32 tiles (the reference's per-instruction tests run
+// them on half, float, int32 and int16: e.g. tests/cpu/st/testcase/tadd/main.cpp).
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) AICORE void VecOpTyped(__gm__ T *out, __gm__ const T *aIn, __gm__ const T *bIn,
+                                                                   __gm__ const T *vecIn, T k, int op)
+{
+    using TileX = Tile<TileType::Vec, T, 64, 128, BLayout::RowMajor>;
+    using TileR = Tile<TileType::Vec, T, 64, 1, BLayout::ColMajor>;
+    using TileC = Tile<TileType::Vec, T, 1, 128, BLayout::RowMajor>;
+    TileX a, b, o;
+    TileR rv;
+    TileC cv;
+    GmND<T, 64, 128> ga(const_cast<T *>(aIn)), gb(const_cast<T *>(bIn)), go(out);
+    TLOAD(a, ga);
+    if (op >= kAdd && op < kAdds)
+        TLOAD(b, gb);
+    if (op >= kRowExpand && op < kColExpand) {
+        GmCol<T, 64> gr(const_cast<T *>(vecIn));
+        TLOAD(rv, gr);
+    }
+    if (op >= kColExpand) {
+        GmND<T, 1, 128> gc(const_cast<T *>(vecIn));
+        TLOAD(cv, gc);
+    }
+    switch (op) {
+    case kAbs: TABS(o, a); break;
+    case kNeg: TNEG(o, a); break;
+    case kRelu: TRELU(o, a); break;
+    case kAdd: TADD(o, a, b); break;
+    case kSub: TSUB(o, a, b); break;
+    case kMul: TMUL(o, a, b); break;
+    case kMax: TMAX(o, a, b); break;
+    case kMin: TMIN(o, a, b); break;
+    case kAdds: TADDS(o, a, k); break;
+    case kSubs: TSUBS(o, a, k); break;
+    case kMuls: TMULS(o, a, k); break;
+    case kMaxs: TMAXS(o, a, k); break;
+    case kMins: TMINS(o, a, k); break;
+    case kRowExpand: TROWEXPAND(o, rv); break;
+    case kRowSub: TROWEXPANDSUB(o, a, rv); break;
+    case kRowMul: TROWEXPANDMUL(o, a, rv); break;
+    case kRowAdd: TROWEXPANDADD(o, a, rv); break;
+    case kRowMax: TROWEXPANDMAX(o, a, rv); break;
+    case kRowMin: TROWEXPANDMIN(o, a, rv); break;
+    case kColExpand: TCOLEXPAND(o, cv); break;
+    case kColSub: TCOLEXPANDSUB(o, a, cv); break;
+    case kColMul: TCOLEXPANDMUL(o, a, cv); break;
+    case kColAdd: TCOLEXPANDADD(o, a, cv); break;
+    case kColMax: TCOLEXPANDMAX(o, a, cv); break;
+    case kColMin: TCOLEXPANDMIN(o, a, cv); break;
+    default: TSUB(o, a, a); break;
+    }
+    TSTORE(go, o);
+}
+
+extern "C" int pto_st_vec_op_typed_64x128(void *stream, void *out, const void *a, const void *b, const void *vec, float scalar, int op,
+                                          int dtype)
+{
+    PTO_ST_NONNULL(out, a);
+    const bool known = (op >= kAbs && op <= kRelu) || (op >= kAdd && op <= kMin && op != kDiv) ||
+                       (op >= kAdds && op <= kMins && op != kDivs) || (op >= kRowExpand && op <= kRowMin && op != kRowDiv) ||
+                       (op >= kColExpand && op <= kColMin && op != kColDiv);
+    if (!known || dtype < 0 || dtype > 1)
+        return PTO_ERR_BAD_ARG;
+    if (op >= kAdd && op <= kMin)
+        PTO_ST_NONNULL(b);
+    if (op >= kRowExpand)
+        PTO_ST_NONNULL(vec);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        VecOpTyped<half><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<half *>(out), static_cast<const half *>(a),
+                                                                  static_cast<const half *>(b), static_cast<const half *>(vec),
+                                                                  (half)scalar, op);
+    else
+        VecOpTyped<int32_t><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<int32_t *>(out), static_cast<const int32_t *>(a),
+                                                                     static_cast<const int32_t *>(b), static_cast<const int32_t *>(vec),
+                                                                     (int32_t)scalar, op);
+    return pto_amd::check_launch();
+}
+
 extern "C" int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const float *b, const float *vec, float scalar, int op)
 {
     PTO_ST_NONNULL(out, a);

@@ -119,3 +119,54 @@ def test_matmul_tmov_acc_to_vec(oracle, relu):
     torch.cuda.synchronize()
     want = oracle.tmov_relu((a @ b).astype(np.float32), relu) * np.float32(0.5)
     assert np.array_equal(out.cpu().numpy(), want)
+
+
+TYPED_OPS = {
+    "ABS": lambda a, b, v, k: np.abs(a), "NEG": lambda a, b, v, k: -a, "RELU": lambda a, b, v, k: np.maximum(a, 0),
+    "ADD": lambda a, b, v, k: a + b, "SUB": lambda a, b, v, k: a - b, "MUL": lambda a, b, v, k: a * b,
+    "MAX": lambda a, b, v, k: np.maximum(a, b), "MIN": lambda a, b, v, k: np.minimum(a, b),
+    "ADDS": lambda a, b, v, k: a + k, "SUBS": lambda a, b, v, k: a - k, "MULS": lambda a, b, v, k: a * k,
+    "MAXS": lambda a, b, v, k: np.maximum(a, k), "MINS": lambda a, b, v, k: np.minimum(a, k),
+    "ROWEXPAND": lambda a, b, v, k: np.broadcast_to(v[:, None], a.shape), "ROWEXPANDSUB": lambda a, b, v, k: a - v[:, None],
+    "ROWEXPANDMUL": lambda a, b, v, k: a * v[:, None], "ROWEXPANDADD": lambda a, b, v, k: a + v[:, None],
+    "ROWEXPANDMAX": lambda a, b, v, k: np.maximum(a, v[:, None]), "ROWEXPANDMIN": lambda a, b, v, k: np.minimum(a, v[:, None]),
+    "COLEXPAND": lambda a, b, v, k: np.broadcast_to(v[None, :], a.shape), "COLEXPANDSUB": lambda a, b, v, k: a - v[None, :],
+    "COLEXPANDMUL": lambda a, b, v, k: a * v[None, :], "COLEXPANDADD": lambda a, b, v, k: a + v[None, :],
+    "COLEXPANDMAX": lambda a, b, v, k: np.maximum(a, v[None, :]), "COLEXPANDMIN": lambda a, b, v, k: np.minimum(a, v[None, :]),
+}
+
+
+@pytest.mark.parametrize("dtype", ["f16", "s32"])
+@pytest.mark.parametrize("op", sorted(TYPED_OPS))
+def test_vec_op_fp16_and_int32(oracle, op, dtype):
+    """The arithmetic Vec instructions on fp16 tiles (one IEEE rounding per operation, as numpy's float16) and on int32
+    tiles (wrap-around arithmetic): bit-exact."""
+    lib = capi.load()
+    rng = np.random.default_rng(101 + len(op))
+    if dtype == "f16":
+        a = (rng.standard_normal((64, 128)) * 8).astype(np.float16)
+        b = (rng.standard_normal((64, 128)) * 8).astype(np.float16)
+        k = np.float16(1.75)
+        mk = lambda n: (rng.standard_normal(n) * 4).astype(np.float16)
+    else:
+        a = rng.integers(-2**31, 2**31, size=(64, 128), dtype=np.int64).astype(np.int32)
+        b = rng.integers(-2**31, 2**31, size=(64, 128), dtype=np.int64).astype(np.int32)
+        a[0, 0] = -2**31                                        # abs / neg of the most negative value wrap
+        k = np.int32(37)
+        mk = lambda n: rng.integers(-2**20, 2**20, size=n).astype(np.int32)
+    vec = mk(64) if op.startswith("ROW") else (mk(128) if op.startswith("COL") else None)
+    with np.errstate(over="ignore", invalid="ignore"):
+        want = np.ascontiguousarray(TYPED_OPS[op](a, b, vec, k)).astype(a.dtype)
+    ta, tb = dev(a), dev(b)
+    tv = dev(vec) if vec is not None else None
+    out = torch.zeros((64, 128), dtype=torch.int16 if dtype == "f16" else torch.int32, device=DEV)
+    capi.check(lib.pto_st_vec_op_typed_64x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tv.data_ptr() if tv is not None else 0,
+                                              float(k), oracle.VOP[op], 0 if dtype == "f16" else 1), op)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(a.dtype)
+    if dtype == "f16":
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got), nan)
+        assert np.array_equal(got[~nan].view(np.uint16), want[~nan].view(np.uint16)), op
+    else:
+        assert np.array_equal(got, want), op
