@@ -104,6 +104,37 @@ PTO_FRONT(TRSQRT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TLOG, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TRECIP, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TPRELU, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+// bitwise / shift / remainder / three-operand forms (pto_instr.hpp:72-86, 246-333, 1137, 1215-1300, 1418 of the reference;
+// the forms that take a scratch tile accept and ignore it)
+PTO_FRONT(TAND, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TOR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TSHL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TSHR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TREM, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TNOT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TANDS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TORS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TSHLS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TSHRS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TREMS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TADDC, typename T, T &dst PTO_C T &a PTO_C T &b PTO_C T &c, (dst, a, b, c))
+PTO_FRONT(TSUBC, typename T, T &dst PTO_C T &a PTO_C T &b PTO_C T &c, (dst, a, b, c))
+PTO_FRONT(TADDSC, typename T, T &dst PTO_C T &a PTO_C typename T::DType k PTO_C T &b, (dst, a, k, b))
+PTO_FRONT(TSUBSC, typename T, T &dst PTO_C T &a PTO_C typename T::DType k PTO_C T &b, (dst, a, k, b))
+template <typename D, typename A, typename B, typename Tmp, typename... Ev>
+PTO_INST std::enable_if_t<is_tile_data_v<Tmp>, RecordEvent> TXOR(D &dst, A &a, B &b, Tmp &, Ev &... ev)
+{
+    TSYNC(ev...);
+    TXOR_IMPL(dst, a, b);
+    return {};
+}
+template <typename D, typename S, typename Tmp, typename... Ev>
+PTO_INST std::enable_if_t<is_tile_data_v<Tmp>, RecordEvent> TXORS(D &dst, S &src, typename S::DType k, Tmp &, Ev &... ev)
+{
+    TSYNC(ev...);
+    TXORS_IMPL(dst, src, k);
+    return {};
+}
 PTO_FRONT(TLRELU, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TCMP, typename T, T &dst PTO_C T &src0 PTO_C T &src1 PTO_C CmpMode mode, (dst, src0, src1, mode))
 PTO_FRONT(TCMPS, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src0 PTO_C T src1 PTO_C CmpMode mode,

@@ -414,4 +414,110 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
     hw::lds_barrier();
 }
 
+// ------------------------------------------------ bitwise, shift, remainder and three-operand forms
+// (cpu/ElementOp.h:145-198, 305-310, 365-378, 425-470; ElementTileOp.h:108-166, 203, 287; ElementTileScalarOp.h:113-):
+// integer tiles for the bitwise and shift ops; TREM is `%` on integers and fmod (evaluated in double) on floats, a
+// zero divisor is the caller's error as in the reference; TADDC = a + b + c, TSUBC = a - b + c.
+namespace detail {
+template <typename T>
+PTO_DEV T elem_rem(T a, T b)
+{
+    if constexpr (std::is_integral_v<T>)
+        return (T)(a % b);
+    else
+        return (T)::fmod((double)a, (double)b);
+}
+} // namespace detail
+
+#define PTO_DEFINE_BINARY_EXT(NAME, INT_ONLY, EXPR)                                                     \
+    template <typename DstT, typename S0T, typename S1T>                                                \
+    PTO_DEV void NAME##_IMPL(DstT &dst, S0T &src0, S1T &src1)                                           \
+    {                                                                                                   \
+        static_assert(detail::same_dist<DstT, S0T> && detail::same_dist<DstT, S1T>,                     \
+                      "[PTO][SA] " #NAME ": Vec tiles with the same number of elements");              \
+        using T = typename DstT::DType;                                                                 \
+        static_assert(!(INT_ONLY) || std::is_integral_v<T>, "[PTO][SA] " #NAME ": integer tiles");      \
+        using S = typename DstT::Storage;                                                               \
+        _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
+        {                                                                                               \
+            const T a = src0.st.v[s][i], b = src1.st.v[s][i];                                           \
+            dst.st.v[s][i] = (T)(EXPR);                                                                 \
+        }                                                                                               \
+    }
+PTO_DEFINE_BINARY_EXT(TAND, true, a & b)
+PTO_DEFINE_BINARY_EXT(TOR, true, a | b)
+PTO_DEFINE_BINARY_EXT(TXOR, true, a ^ b)
+PTO_DEFINE_BINARY_EXT(TSHL, true, a << b)
+PTO_DEFINE_BINARY_EXT(TSHR, true, a >> b)
+PTO_DEFINE_BINARY_EXT(TREM, false, detail::elem_rem<T>(a, b))
+#undef PTO_DEFINE_BINARY_EXT
+
+#define PTO_DEFINE_SCALAR_EXT(NAME, INT_ONLY, EXPR)                                                     \
+    template <typename DstT, typename SrcT>                                                             \
+    PTO_DEV void NAME##_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)                              \
+    {                                                                                                   \
+        static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] " #NAME ": Vec tiles of equal size"); \
+        using T = typename DstT::DType;                                                                 \
+        static_assert(!(INT_ONLY) || std::is_integral_v<T>, "[PTO][SA] " #NAME ": integer tiles");      \
+        using S = typename DstT::Storage;                                                               \
+        _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
+        {                                                                                               \
+            const T a = src.st.v[s][i];                                                                 \
+            dst.st.v[s][i] = (T)(EXPR);                                                                 \
+        }                                                                                               \
+    }
+PTO_DEFINE_SCALAR_EXT(TANDS, true, a & k)
+PTO_DEFINE_SCALAR_EXT(TORS, true, a | k)
+PTO_DEFINE_SCALAR_EXT(TXORS, true, a ^ k)
+PTO_DEFINE_SCALAR_EXT(TSHLS, true, a << k)
+PTO_DEFINE_SCALAR_EXT(TSHRS, true, a >> k)
+PTO_DEFINE_SCALAR_EXT(TREMS, false, detail::elem_rem<T>(a, k))
+#undef PTO_DEFINE_SCALAR_EXT
+
+template <typename DstT, typename SrcT>
+PTO_DEV void TNOT_IMPL(DstT &dst, SrcT &src)
+{
+    static_assert(detail::same_dist<DstT, SrcT> && std::is_integral_v<typename DstT::DType>, "[PTO][SA] TNOT: integer Vec tiles of equal size");
+    using S = typename DstT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.st.v[s][i] = (typename DstT::DType)~src.st.v[s][i];
+}
+
+// dst = src0 +/- src1 + src2; the scalar forms take the scalar as the second operand
+template <bool kSub, typename TileT>
+PTO_DEV void vec_addc(TileT &dst, TileT &src0, TileT &src1, TileT &src2)
+{
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i) {
+            const auto a = src0.st.v[s][i], b = src1.st.v[s][i], c = src2.st.v[s][i];
+            dst.st.v[s][i] = kSub ? a - b + c : a + b + c;
+        }
+}
+template <typename TileT>
+PTO_DEV void TADDC_IMPL(TileT &dst, TileT &src0, TileT &src1, TileT &src2) { vec_addc<false>(dst, src0, src1, src2); }
+template <typename TileT>
+PTO_DEV void TSUBC_IMPL(TileT &dst, TileT &src0, TileT &src1, TileT &src2) { vec_addc<true>(dst, src0, src1, src2); }
+template <bool kSub, typename TileT>
+PTO_DEV void vec_addsc(TileT &dst, TileT &src0, typename TileT::DType k, TileT &src1)
+{
+    using S = typename TileT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i) {
+            const auto a = src0.st.v[s][i], c = src1.st.v[s][i];
+            dst.st.v[s][i] = kSub ? a - k + c : a + k + c;
+        }
+}
+template <typename TileT>
+PTO_DEV void TADDSC_IMPL(TileT &dst, TileT &src0, typename TileT::DType k, TileT &src1) { vec_addsc<false>(dst, src0, k, src1); }
+template <typename TileT>
+PTO_DEV void TSUBSC_IMPL(TileT &dst, TileT &src0, typename TileT::DType k, TileT &src1) { vec_addsc<true>(dst, src0, k, src1); }
+
 } // namespace pto

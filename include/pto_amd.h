@@ -175,6 +175,14 @@ int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const flo
  * expand forms without the divisions) on [64,128] fp16 (dtype 0) or int32 (dtype 1) tiles; same operation codes. */
 int pto_st_vec_op_typed_64x128(void *stream, void *out, const void *a, const void *b, const void *vec, float scalar, int op,
                                int dtype);
+/* Bitwise, shift, remainder and three-operand Vec instructions on [64,128] tiles (pto_instr.hpp TAND TOR TXOR TSHL TSHR
+ * TREM TNOT, TANDS TORS TXORS TSHLS TSHRS TREMS, TADDC TSUBC TADDSC TSUBSC; element rules cpu/ElementOp.h:145-198,
+ * 305-310, 365-378, 425-470).  op: 0 AND, 1 OR, 2 XOR, 3 SHL, 4 SHR, 5 REM, 6 NOT, 7..12 the scalar forms of 0..5,
+ * 13 ADDC (a + b + c), 14 SUBC (a - b + c), 15 ADDSC (a + scalar + c), 16 SUBSC (a - scalar + c).
+ * dtype 1: int32 tiles, scalar_i (every op); dtype 0: fp32 tiles, scalar_f (REM, REMS and the three-operand ops).
+ * a, b and c are always read. */
+int pto_st_vec_bitop_64x128(void *stream, void *out, const void *a, const void *b, const void *c, float scalar_f, int scalar_i,
+                            int op, int dtype);
 /* Reductions over the valid region [valid_rows, valid_cols] of a [64,128] fp32 tile (row stride 128 in memory):
  * op 0 TROWMAX, 1 TROWMIN, 2 TROWSUM -> out[valid_rows]; 3 TCOLMAX, 4 TCOLMIN, 5 TCOLSUM -> out[valid_cols]
  * (cpu/TRowMax.hpp, TRowMin.hpp, TRowSum.hpp, TColMax.hpp, TColMin.hpp, TColSum.hpp). */

@@ -867,6 +867,72 @@ extern "C" int pto_st_vec_op_typed_64x128(void *stream, void *out, const void *a
     return pto_amd::check_launch();
 }
 
+// Bitwise, shift, remainder and three-operand Vec instructions (the reference tests them per instruction:
+// tests/cpu/st/testcase/{tand,tor,txor,tnot,tshl,tshr,trem,taddc,tsubc,tands,...}/): int32 tiles run every op, fp32 tiles
+// the remainder and three-operand ones.
+enum BitOp : int {
+    kBitAnd = 0, kBitOr, kBitXor, kBitShl, kBitShr, kBitRem, kBitNot, kBitAnds, kBitOrs, kBitXors, kBitShls, kBitShrs, kBitRems,
+    kBitAddc, kBitSubc, kBitAddsc, kBitSubsc, kBitOpCount
+};
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) AICORE void VecBitOp(__gm__ T *out, __gm__ const T *aIn, __gm__ const T *bIn,
+                                                                 __gm__ const T *cIn, T k, int op)
+{
+    using TileX = Tile<TileType::Vec, T, 64, 128, BLayout::RowMajor>;
+    TileX a, b, c, o, tmp;
+    GmND<T, 64, 128> ga(const_cast<T *>(aIn)), gb(const_cast<T *>(bIn)), gc(const_cast<T *>(cIn)), go(out);
+    TLOAD(a, ga);
+    TLOAD(b, gb);
+    TLOAD(c, gc);
+    if constexpr (std::is_integral_v<T>) {
+        switch (op) {
+        case kBitAnd: TAND(o, a, b); break;
+        case kBitOr: TOR(o, a, b); break;
+        case kBitXor: TXOR(o, a, b, tmp); break;
+        case kBitShl: TSHL(o, a, b); break;
+        case kBitShr: TSHR(o, a, b); break;
+        case kBitNot: TNOT(o, a); break;
+        case kBitAnds: TANDS(o, a, k); break;
+        case kBitOrs: TORS(o, a, k); break;
+        case kBitXors: TXORS(o, a, k, tmp); break;
+        case kBitShls: TSHLS(o, a, k); break;
+        case kBitShrs: TSHRS(o, a, k); break;
+        default: break;
+        }
+    }
+    switch (op) {
+    case kBitRem: TREM(o, a, b); break;
+    case kBitRems: TREMS(o, a, k); break;
+    case kBitAddc: TADDC(o, a, b, c); break;
+    case kBitSubc: TSUBC(o, a, b, c); break;
+    case kBitAddsc: TADDSC(o, a, k, c); break;
+    case kBitSubsc: TSUBSC(o, a, k, c); break;
+    default: break;
+    }
+    TSTORE(go, o);
+}
+
+// dtype 0: fp32 (scalar_f), 1: int32 (scalar_i); a, b and c are all read
+extern "C" int pto_st_vec_bitop_64x128(void *stream, void *out, const void *a, const void *b, const void *c, float scalar_f,
+                                       int scalar_i, int op, int dtype)
+{
+    PTO_ST_NONNULL(out, a, b, c);
+    if (op < 0 || op >= kBitOpCount || dtype < 0 || dtype > 1)
+        return PTO_ERR_BAD_ARG;
+    const bool forFloat = op == kBitRem || op == kBitRems || op >= kBitAddc;
+    if (dtype == 0 && !forFloat)
+        return PTO_ERR_UNSUPPORTED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        VecBitOp<float><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<float *>(out), static_cast<const float *>(a),
+                                                                 static_cast<const float *>(b), static_cast<const float *>(c), scalar_f, op);
+    else
+        VecBitOp<int32_t><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<int32_t *>(out), static_cast<const int32_t *>(a),
+                                                                   static_cast<const int32_t *>(b), static_cast<const int32_t *>(c),
+                                                                   scalar_i, op);
+    return pto_amd::check_launch();
+}
+
 extern "C" int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const float *b, const float *vec, float scalar, int op)
 {
     PTO_ST_NONNULL(out, a);

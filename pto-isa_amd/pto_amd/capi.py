@@ -39,6 +39,7 @@ SYMBOLS = {
     "pto_st_matmul_f32_128x32x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_mx_128x256x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 3),
     "pto_st_vec_op_typed_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int]),
+    "pto_st_vec_bitop_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int, C.c_int]),
     "pto_st_vec_op_f32_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int]),
     "pto_st_reduce_f32_64x128": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 3),
     "pto_st_cmps_sel_f32_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int]),

@@ -170,3 +170,66 @@ def test_vec_op_fp16_and_int32(oracle, op, dtype):
         assert np.array_equal(got[~nan].view(np.uint16), want[~nan].view(np.uint16)), op
     else:
         assert np.array_equal(got, want), op
+
+
+BIT_OPS = ["AND", "OR", "XOR", "SHL", "SHR", "REM", "NOT", "ANDS", "ORS", "XORS", "SHLS", "SHRS", "REMS", "ADDC", "SUBC", "ADDSC", "SUBSC"]
+FLOAT_BIT_OPS = ["REM", "REMS", "ADDC", "SUBC", "ADDSC", "SUBSC"]
+
+
+def c_rem(a, b):
+    """C's remainder (sign of the dividend), the rule of the reference's element operation, for integers and floats."""
+    if a.dtype.kind == "i":
+        a64, b64 = a.astype(np.int64), np.broadcast_to(b, a.shape).astype(np.int64)
+        return (a64 - np.trunc(a64 / b64).astype(np.int64) * b64).astype(a.dtype)
+    return np.fmod(a.astype(np.float64), np.float64(b) if np.ndim(b) == 0 else b.astype(np.float64)).astype(a.dtype)
+
+
+@pytest.mark.parametrize("op,dtype", [(op, "s32") for op in BIT_OPS] + [(op, "f32") for op in FLOAT_BIT_OPS])
+def test_vec_bitwise_shift_rem_carry(op, dtype):
+    """TAND .. TSUBSC against numpy's integer / float rules (wrap-around int32; shifts by 0..31, arithmetic right
+    shift; remainder with the dividend's sign; a + b + c evaluated left to right in the element type): bit-exact."""
+    lib = capi.load()
+    rng = np.random.default_rng(300 + BIT_OPS.index(op))
+    if dtype == "s32":
+        a = rng.integers(-2**31, 2**31, size=(64, 128), dtype=np.int64).astype(np.int32)
+        b = rng.integers(-2**31, 2**31, size=(64, 128), dtype=np.int64).astype(np.int32)
+        c = rng.integers(-2**31, 2**31, size=(64, 128), dtype=np.int64).astype(np.int32)
+        k = np.int32(-1234577 if op in ("ANDS", "ORS", "XORS", "ADDSC", "SUBSC") else 11)
+        if op in ("SHL", "SHR"):
+            b = rng.integers(0, 32, size=(64, 128)).astype(np.int32)
+        if op == "REM":
+            b = rng.integers(1, 2**20, size=(64, 128)).astype(np.int32) * rng.choice(np.array([-1, 1], dtype=np.int32), size=(64, 128))
+            a[0, :4] = [-2**31, 2**31 - 1, 0, -1]
+        if op == "SHL":                                         # a left shift of a negative value: the bits move, as on the device
+            want = ((a.astype(np.int64) << b) & 0xffffffff).astype(np.uint32).view(np.int32)
+        elif op == "SHLS":
+            want = ((a.astype(np.int64) << int(k)) & 0xffffffff).astype(np.uint32).view(np.int32)
+    else:
+        a = (rng.standard_normal((64, 128)) * 100).astype(np.float32)
+        b = (rng.standard_normal((64, 128)) * 7).astype(np.float32)
+        b[b == 0] = 1
+        c = (rng.standard_normal((64, 128)) * 50).astype(np.float32)
+        k = np.float32(3.7)
+    with np.errstate(over="ignore"):
+        table = {"AND": lambda: a & b, "OR": lambda: a | b, "XOR": lambda: a ^ b, "SHR": lambda: a >> b, "REM": lambda: c_rem(a, b),
+                 "NOT": lambda: ~a, "ANDS": lambda: a & k, "ORS": lambda: a | k, "XORS": lambda: a ^ k, "SHRS": lambda: a >> k,
+                 "REMS": lambda: c_rem(a, k), "ADDC": lambda: a + b + c, "SUBC": lambda: a - b + c, "ADDSC": lambda: a + k + c,
+                 "SUBSC": lambda: a - k + c}
+        if op not in ("SHL", "SHLS"):
+            want = table[op]().astype(a.dtype)
+    ta, tb, tc = dev(a), dev(b), dev(c)
+    out = torch.zeros((64, 128), dtype=torch.int32, device=DEV)
+    capi.check(lib.pto_st_vec_bitop_64x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), float(k), int(k) if dtype == "s32" else 0,
+                                           BIT_OPS.index(op), 1 if dtype == "s32" else 0), op)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(a.dtype)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), op
+
+
+def test_vec_bitop_rejects_bad_arguments():
+    lib = capi.load()
+    t = torch.zeros((64, 128), dtype=torch.int32, device=DEV)
+    p = t.data_ptr()
+    assert lib.pto_st_vec_bitop_64x128(st(), p, p, p, p, 0.0, 0, 17, 1) == capi.ERR_BAD_ARG
+    assert lib.pto_st_vec_bitop_64x128(st(), p, p, p, p, 0.0, 0, 0, 0) == capi.ERR_UNSUPPORTED   # TAND on fp32
+    assert lib.pto_st_vec_bitop_64x128(st(), p, p, 0, p, 0.0, 0, 0, 1) == capi.ERR_BAD_ARG
