@@ -155,8 +155,18 @@ PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
     TSYNC(ev...);
     if constexpr (S::Loc == TileType::Acc && D::Loc == TileType::Vec)
         TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    else if constexpr ((S::Loc == TileType::Acc || S::Loc == TileType::Vec) && (D::Loc == TileType::Left || D::Loc == TileType::Right))
+        TMOV_TO_OPERAND_IMPL(dst, src); // the chained matmuls of the Auto-mode programs
     else
         TMOV_IMPL(dst, src);
+    return {};
+}
+// TTRANS (pto_instr.hpp:1032 of the reference): the scratch tile is accepted and ignored
+template <typename D, typename S, typename Tmp, typename... Ev>
+PTO_INST RecordEvent TTRANS(D &dst, S &src, Tmp &, Ev &... ev)
+{
+    TSYNC(ev...);
+    TTRANS_IMPL(dst, src);
     return {};
 }
 template <typename D, typename S, AccToVecMode mode, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>

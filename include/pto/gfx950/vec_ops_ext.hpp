@@ -414,6 +414,115 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
     hw::lds_barrier();
 }
 
+// ------------------------------------- TMOV Vec / Acc -> Left / Right, TTRANS
+// Same-shape moves from a register tile that the whole workgroup holds (Vec) or that the waves hold as MFMA
+// results (Acc) into the per-wave operand fragments of TMATMUL, and the transpose of a Vec tile (the reference's
+// Auto-mode programs chain matmuls this way: demos/cpu/mla_attention_demo/mla_attention_demo.cpp:300-395; element
+// rules cpu/TMov.hpp, cpu/TTrans.hpp).  All of them redistribute through an LDS staging array that holds the
+// destination's element type: k-contiguous per row for a Left destination, per column for a Right destination, so
+// that a fragment is one 16-byte read.
+namespace detail {
+constexpr int stage_bytes(int n)
+{
+    int b = 1024;
+    while (b < n)
+        b *= 2;
+    return b;
+}
+// staging arrays are shared by all moves of a size class
+template <int Bytes>
+PTO_DEV char *stage_buffer()
+{
+    __shared__ __attribute__((aligned(16))) char buf[Bytes];
+    return buf;
+}
+// every element (r, c) of a Vec or Acc tile -> stage[index(r, c)]
+template <typename T, typename SrcT, typename IndexF>
+PTO_DEV void stage_write(SrcT &src, T *stage, IndexF &&index)
+{
+    if constexpr (SrcT::Loc == TileType::Acc) {
+        using S = typename SrcT::Storage;
+        const uint32_t lane = (uint32_t)hw::lane();
+        const int rbase = hw::wave_m() * (S::MB * kMfmaM) + acc_lane_row(lane);
+        const int cbase = hw::wave_n() * (S::NB * kMfmaM) + acc_lane_col(lane);
+#pragma unroll
+        for (int mb = 0; mb < S::MB; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < S::NB; ++nb)
+#pragma unroll
+                for (int v = 0; v < kAccElems; ++v)
+                    stage[index(rbase + mb * kMfmaM + acc_elem_row(v), cbase + nb * kMfmaM)] = (T)src.st.f[mb][nb][v];
+    } else {
+        static_assert(SrcT::Loc == TileType::Vec, "[PTO][SA] TMOV / TTRANS: Vec or Acc source");
+        for_each_owned<SrcT>([&](int s, int i, int e) {
+            if (e < SrcT::Numel) {
+                int r, c;
+                elem_rc<SrcT>(e, r, c);
+                stage[index(r, c)] = (T)src.st.v[s][i];
+            }
+        });
+    }
+}
+} // namespace detail
+
+template <typename DstT, typename SrcT>
+PTO_DEV void TMOV_TO_OPERAND_IMPL(DstT &dst, SrcT &src)
+{
+    static_assert((DstT::Loc == TileType::Left || DstT::Loc == TileType::Right) && DstT::Rows == SrcT::Rows && DstT::Cols == SrcT::Cols,
+                  "[PTO][SA] TMOV to a matmul operand: Left or Right destination of the source's shape");
+    using T = typename DstT::DType;
+    static_assert(!detail::is_mx_operand_v<T>, "[PTO][SA] TMOV to a matmul operand: fp16, bf16, int8 or fp32 elements");
+    using S = typename DstT::Storage;
+    using Frag = typename detail::FragOf<T>::type;
+    constexpr bool left = DstT::Loc == TileType::Left;
+    constexpr int K = left ? DstT::Cols : DstT::Rows; // extent along k; a row (column) of the operand is K contiguous elements
+    constexpr int kChunkElems = 16 / (int)sizeof(T), kStepChunks = kWaveSize / detail::kMfmaM;
+    T *stage = reinterpret_cast<T *>(detail::stage_buffer<detail::stage_bytes(DstT::Numel * (int)sizeof(T))>());
+    detail::stage_write<T>(src, stage, [&](int r, int c) { return left ? r * K + c : c * K + r; });
+    hw::lds_barrier();
+    const uint32_t lane = (uint32_t)hw::lane();
+    const int major = (int)detail::frag_lane_major(lane), kgroup = (int)detail::frag_lane_kgroup(lane);
+    if constexpr (left) {
+        const int row0 = hw::wave_m() * (S::MB * detail::kMfmaM) + major;
+#pragma unroll
+        for (int mb = 0; mb < S::MB; ++mb)
+#pragma unroll
+            for (int ks = 0; ks < S::KS; ++ks)
+                dst.st.f[mb][ks] =
+                    *reinterpret_cast<const Frag *>(stage + (row0 + mb * detail::kMfmaM) * K + (kgroup + ks * kStepChunks) * kChunkElems);
+    } else {
+        const int col0 = hw::wave_n() * (S::NB * detail::kMfmaM) + major;
+#pragma unroll
+        for (int nb = 0; nb < S::NB; ++nb)
+#pragma unroll
+            for (int ks = 0; ks < S::KS; ++ks)
+                dst.st.f[nb][ks] =
+                    *reinterpret_cast<const Frag *>(stage + (col0 + nb * detail::kMfmaM) * K + (kgroup + ks * kStepChunks) * kChunkElems);
+    }
+    hw::lds_barrier();
+}
+
+// dst[c][r] = src[r][c] (cpu/TTrans.hpp); the scratch tile of the reference's form is not needed
+template <typename DstT, typename SrcT>
+PTO_DEV void TTRANS_IMPL(DstT &dst, SrcT &src)
+{
+    static_assert(DstT::Loc == TileType::Vec && SrcT::Loc == TileType::Vec && DstT::Rows == SrcT::Cols && DstT::Cols == SrcT::Rows &&
+                      sizeof(typename DstT::DType) == sizeof(typename SrcT::DType),
+                  "[PTO][SA] TTRANS: Vec tiles, destination of the transposed shape, same element size");
+    using T = typename DstT::DType;
+    T *stage = reinterpret_cast<T *>(detail::stage_buffer<detail::stage_bytes(DstT::Numel * (int)sizeof(T))>());
+    detail::stage_write<T>(src, stage, [&](int r, int c) { return c * SrcT::Rows + r; }); // row-major image of the transpose
+    hw::lds_barrier();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        if (e < DstT::Numel) {
+            int r, c;
+            detail::elem_rc<DstT>(e, r, c);
+            dst.st.v[s][i] = stage[r * DstT::Cols + c];
+        }
+    });
+    hw::lds_barrier();
+}
+
 // ------------------------------------------------ bitwise, shift, remainder and three-operand forms
 // (cpu/ElementOp.h:145-198, 305-310, 365-378, 425-470; ElementTileOp.h:108-166, 203, 287; ElementTileScalarOp.h:113-):
 // integer tiles for the bitwise and shift ops; TREM is `%` on integers and fmod (evaluated in double) on floats, a

@@ -14,6 +14,7 @@
  *                        kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:344-364
  *   pto_topk_f32         launchTopk<float>(uint8_t *out, uint8_t *index, uint8_t *src, uint8_t *inIdx, void *stream)
  *                        kernels/manual/a2a3/topk/topk_kernel.cpp:334-345
+ *   pto_mla_attention_*  mla_pto(q, k, v, wq, wk, wv, wo, out) demos/cpu/mla_attention_demo/mla_attention_demo.cpp:227-397
  *   pto_fa_fwd_f16       LaunchTFA<...>(...) kernels/manual/common/flash_atten/fa_performance_kernel.h:28-41 and
  *                        call_kernel(...) demos/torch_jit/flash_atten/fa_kernel.cpp:1017-1092
  *   pto_tcvt_*           runTCVT / launchTCVT tests/cpu/st/testcase/tcvt/tcvt_kernel.cpp:18-66 (TLOAD -> TCVT -> TSTORE)
@@ -77,6 +78,13 @@ int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, co
  * topk <= valid_cols <= ld.  NaN scores are ordered by their bit patterns (positive NaNs first, negative ones last). */
 int pto_topk_f32(void *stream, float *out_score, uint32_t *out_index, const float *src, const uint32_t *in_idx, int rows,
                  int valid_cols, int ld, int topk);
+
+/* Multi-latent attention of the reference's Auto-mode demo (demos/cpu/mla_attention_demo/mla_attention_demo.cpp:227-397,
+ * mla_pto(q, k, v, wq, wk, wv, wo, out)) at the demo's sizes: 64 positions, head dim 32, latent dim 16, fp32.
+ * q, k, v, out [batch, heads, 64, 32]; wq, wk, wv [32, 16]; wo [16, 32], all contiguous.  Per (batch, head):
+ * out = (softmax((q wq) (k wk)^T / 4) (v wv)) wo, one workgroup each, every intermediate a tile. */
+int pto_mla_attention_f32_s64_d32_r16(void *stream, float *out, const float *q, const float *k, const float *v, const float *wq,
+                                      const float *wk, const float *wv, const float *wo, int batch, int heads);
 
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];
@@ -196,6 +204,12 @@ int pto_st_cmps_sel_f32_64x128(void *stream, float *sel, uint8_t *bits, const fl
 int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int pad_kind);
 /* out[64,128] = scale * (relu ? max(a b, 0) : a b): fp16 matmul [64,64] x [64,128] (b_t stored [128][64]), TMOV of
  * the accumulator into a Vec tile with ReluPreMode (cpu/TMov.hpp:53-69), TMULS, TSTORE. */
+/* TMOV Vec -> Left / Right, Acc -> Left and TTRANS (the operand moves of the Auto-mode programs, cpu/TMov.hpp,
+ * cpu/TTrans.hpp): a [64,64], b [64,128] fp16 row-major are loaded as Vec tiles and moved into operand tiles;
+ * mid [64,128] = a b (fp32); out [64,64] = half(mid) b^T, with b^T made by TTRANS and half(mid) by the Acc -> Left move. */
+int pto_st_matmul_vec_operands_f16_64x64x128(void *stream, float *out, float *mid, const uint16_t *a, const uint16_t *b);
+/* TTRANS on fp32: out [128,64] = in [64,128] transposed. */
+int pto_st_ttrans_f32_64x128(void *stream, float *out, const float *in);
 int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, int relu, float scale);
 
 /* Two-stage pipeline through TPUSH / TPOP FIFOs (common/fifo.hpp, cpu/TPush.hpp, cpu/TPop.hpp; the hand-offs of

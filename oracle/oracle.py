@@ -286,6 +286,36 @@ def fa_auto_f32(q, k, v, threads=0):
     return out
 
 
+def mla_attention(q, k, v, wq, wk, wv, wo):
+    """Multi-latent attention in float64, the reference's check of its Auto-mode demo
+    (demos/cpu/mla_attention_demo/mla_attention_demo.cpp:113-225, mla_reference): per (batch, head)
+    Q_lat = Q Wq, K_lat = K Wk, V_lat = V Wv ([S,D] x [D,R]), P = softmax(Q_lat K_lat^T / sqrt(R)) over every row,
+    out = (P V_lat) Wo.  q, k, v [B,H,S,D]; wq, wk, wv [D,R]; wo [R,D]; returns float32 [B,H,S,D] (the cast of the
+    float64 result, as the demo stores it).  numpy only: the sizes are tiny."""
+    q, k, v, wq, wk, wv, wo = (np.asarray(t, dtype=np.float64) for t in (q, k, v, wq, wk, wv, wo))
+    R = wq.shape[1]
+    out = np.empty(q.shape, dtype=np.float32)
+    for b in range(q.shape[0]):
+        for h in range(q.shape[1]):
+            ql, kl, vl = q[b, h] @ wq, k[b, h] @ wk, v[b, h] @ wv
+            sc = (ql @ kl.T) * (1.0 / np.sqrt(float(R)))
+            e = np.exp(sc - sc.max(axis=1, keepdims=True))
+            denom = e.sum(axis=1, keepdims=True)
+            p = e * np.where(denom > 0.0, 1.0 / denom, 0.0)
+            out[b, h] = ((p @ vl) @ wo).astype(np.float32)
+    return out
+
+
+def mla_verify_allclose(actual, ref, abs_tol=2e-4, rel_tol=2e-4):
+    """The demo's acceptance test (mla_attention_demo.cpp:69-111, 45-47): number of elements with
+    |a - r| > abs_tol + rel_tol |r| or a non-finite value."""
+    a, r = np.asarray(actual, dtype=np.float32).ravel(), np.asarray(ref, dtype=np.float32).ravel()
+    finite = np.isfinite(a) & np.isfinite(r)
+    bad = ~finite
+    bad[finite] = ~(np.abs(a[finite] - r[finite]) <= np.float32(abs_tol) + np.float32(rel_tol) * np.abs(r[finite]))
+    return int(bad.sum())
+
+
 def fa_stream_f16(q, k, v, tile_s1=128, causal=False, q_offset=0, round_away=True, threads=0):
     """One head: q [S0,D], k,v [S1,D] fp16 -> (o fp32 [S0,D], row_max [S0], row_sum [S0])."""
     q, k, v = (np.ascontiguousarray(t).view(np.uint16) for t in (q, k, v))

@@ -233,6 +233,75 @@ void fa_auto(float *out, const float *q, const float *k, const float *v)
 }
 
 
+// ---- multi-latent attention on one head, the instruction sequence of the reference's Auto-mode demo
+// (demos/cpu/mla_attention_demo), at its sizes S = 64, D = 32, R = 16 ----
+template <int S, int D, int R>
+void mla_auto(float *out, const float *q, const float *k, const float *v, const float *wq, const float *wk, const float *wv,
+              const float *wo)
+{
+    using XP = Tile<TileType::Vec, float, S, D, BLayout::RowMajor, S, D, SLayout::NoneBox>;
+    using WP = Tile<TileType::Vec, float, D, R, BLayout::RowMajor, D, R, SLayout::NoneBox>;
+    using WOP = Tile<TileType::Vec, float, R, D, BLayout::RowMajor, R, D, SLayout::NoneBox>;
+    using LP = Tile<TileType::Vec, float, S, R, BLayout::RowMajor, S, R, SLayout::NoneBox>;
+    using LTP = Tile<TileType::Vec, float, R, S, BLayout::RowMajor, R, S, SLayout::NoneBox>;
+    using SP = Tile<TileType::Vec, float, S, S, BLayout::RowMajor, S, S, SLayout::NoneBox>;
+    using RR = Tile<TileType::Vec, float, S, S, BLayout::ColMajor, S, S, SLayout::NoneBox>;
+    using AccL = TileAcc<float, S, R, S, R>;
+    auto x = std::make_unique<XP>();
+    auto w = std::make_unique<WP>();
+    auto w2 = std::make_unique<WOP>();
+    auto xl = std::make_unique<TileLeft<float, S, D, S, D>>();
+    auto wr = std::make_unique<TileRight<float, D, R, D, R>>();
+    auto wor = std::make_unique<TileRight<float, R, D, R, D>>();
+    std::unique_ptr<AccL> lat[3] = {std::make_unique<AccL>(), std::make_unique<AccL>(), std::make_unique<AccL>()};
+    const float *xs[3] = {q, k, v}, *ws[3] = {wq, wk, wv};
+    for (int i = 0; i < 3; ++i) {
+        GmND<float, S, D> gx(const_cast<float *>(xs[i]));
+        GmND<float, D, R> gw(const_cast<float *>(ws[i]));
+        TLOAD(*x, gx);
+        TLOAD(*w, gw);
+        TMOV(*xl, *x);
+        TMOV(*wr, *w);
+        TMATMUL(*lat[i], *xl, *wr);
+    }
+    auto ql = std::make_unique<TileLeft<float, S, R, S, R>>();
+    auto kp = std::make_unique<LP>();
+    auto kt = std::make_unique<LTP>();
+    auto ktr = std::make_unique<TileRight<float, R, S, R, S>>();
+    auto sa = std::make_unique<TileAcc<float, S, S, S, S>>();
+    auto sc = std::make_unique<SP>();
+    auto pr = std::make_unique<SP>();
+    auto rmax = std::make_unique<RR>();
+    auto rsum = std::make_unique<RR>();
+    TMOV(*ql, *lat[0]);
+    TMOV(*kp, *lat[1]);
+    TTRANS(*kt, *kp, *kp);
+    TMOV(*ktr, *kt);
+    TMATMUL(*sa, *ql, *ktr);
+    TMOV(*sc, *sa);
+    TMULS(*sc, *sc, 1.0f / std::sqrt(static_cast<float>(R)));
+    TROWMAX(*rmax, *sc, *sc);
+    TROWEXPANDSUB(*pr, *sc, *rmax);
+    TEXP(*pr, *pr);
+    TROWSUM(*rsum, *pr, *pr);
+    TROWEXPANDDIV(*pr, *pr, *rsum);
+    auto pl = std::make_unique<TileLeft<float, S, S, S, S>>();
+    auto vr = std::make_unique<TileRight<float, S, R, S, R>>();
+    auto ctx = std::make_unique<AccL>();
+    auto cl = std::make_unique<TileLeft<float, S, R, S, R>>();
+    auto oa = std::make_unique<TileAcc<float, S, D, S, D>>();
+    TMOV(*pl, *pr);
+    TMOV(*vr, *lat[2]);
+    TMATMUL(*ctx, *pl, *vr);
+    TMOV(*cl, *ctx);
+    GmND<float, R, D> gwo(const_cast<float *>(wo));
+    TLOAD(*w2, gwo);
+    TMOV(*wor, *w2);
+    TMATMUL(*oa, *cl, *wor);
+    GmND<float, S, D> go(out);
+    TSTORE(go, *oa);
+}
+
 // ---- further Vec instructions on [64,128] fp32 tiles (op codes: PTO_VOP_* of include/pto_amd.h) ----
 using VX = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
 using VRow = Tile<TileType::Vec, float, 64, 1, BLayout::ColMajor>;   // one value per row
@@ -446,6 +515,11 @@ void ref_image_5d_f32_2x3x4x8(float *image, const float *gm)
 }
 
 void ref_fa_auto_64x32(float *out, const float *q, const float *k, const float *v) { fa_auto<64, 32>(out, q, k, v); }
+void ref_mla_auto_64x32x16(float *out, const float *q, const float *k, const float *v, const float *wq, const float *wk,
+                           const float *wv, const float *wo)
+{
+    mla_auto<64, 32, 16>(out, q, k, v, wq, wk, wv, wo);
+}
 void ref_fa_auto_128x64(float *out, const float *q, const float *k, const float *v) { fa_auto<128, 64>(out, q, k, v); }
 
 

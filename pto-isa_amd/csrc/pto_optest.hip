@@ -981,6 +981,69 @@ extern "C" int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *
     return pto_amd::check_launch();
 }
 
+// Matmul whose operands arrive as Vec tiles and are moved into Left / Right with TMOV (the operand path of the Auto-mode
+// programs: cpu/TMov.hpp Vec -> Left / Right), the result moved Acc -> Left and multiplied once more, and TTRANS:
+//   out = (A B) B2 with A [64,64], B [64,128], B2 = B^T [128,64] made by TTRANS; fp16 operands, fp32 accumulators;
+//   the intermediate A B is cast to fp16 by the Acc -> Left move.
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatmulVecOperands(__gm__ float *out, __gm__ float *mid, __gm__ const half *a,
+                                                                          __gm__ const half *b)
+{
+    using VA = Tile<TileType::Vec, half, 64, 64, BLayout::RowMajor>;
+    using VB = Tile<TileType::Vec, half, 64, 128, BLayout::RowMajor>;
+    using VBT = Tile<TileType::Vec, half, 128, 64, BLayout::RowMajor>;
+    VA va;
+    VB vb;
+    VBT vbt;
+    GmND<half, 64, 64> ga(const_cast<half *>(a));
+    GmND<half, 64, 128> gb(const_cast<half *>(b));
+    TLOAD(va, ga);
+    TLOAD(vb, gb);
+    TileLeft<half, 64, 64> l;
+    TileRight<half, 64, 128> r;
+    TMOV(l, va);
+    TMOV(r, vb);
+    TileAcc<float, 64, 128> c;
+    TMATMUL(c, l, r);
+    GmND<float, 64, 128> gmid(mid);
+    TSTORE(gmid, c);
+    TTRANS(vbt, vb, vb);
+    TileLeft<half, 64, 128> l2;
+    TileRight<half, 128, 64> r2;
+    TMOV(l2, c);
+    TMOV(r2, vbt);
+    TileAcc<float, 64, 64> c2;
+    TMATMUL(c2, l2, r2);
+    GmND<float, 64, 64> go(out);
+    TSTORE(go, c2);
+}
+
+// TTRANS alone on fp32: out [128,64] = in [64,128] transposed
+__global__ __launch_bounds__(kBlockThreads) AICORE void TransKernel(__gm__ float *out, __gm__ const float *in)
+{
+    Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor> x;
+    Tile<TileType::Vec, float, 128, 64, BLayout::RowMajor> y;
+    GmND<float, 64, 128> gi(const_cast<float *>(in));
+    GmND<float, 128, 64> go(out);
+    TLOAD(x, gi);
+    TTRANS(y, x, x);
+    TSTORE(go, y);
+}
+
+extern "C" int pto_st_matmul_vec_operands_f16_64x64x128(void *stream, float *out, float *mid, const uint16_t *a, const uint16_t *b)
+{
+    PTO_ST_NONNULL(out, mid, a, b);
+    MatmulVecOperands<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, mid, reinterpret_cast<const half *>(a),
+                                                                                            reinterpret_cast<const half *>(b));
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_ttrans_f32_64x128(void *stream, float *out, const float *in)
+{
+    PTO_ST_NONNULL(out, in);
+    TransKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, in);
+    return pto_amd::check_launch();
+}
+
 extern "C" int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, int relu, float scale)
 {
     PTO_ST_NONNULL(out, a, b_t);

@@ -21,6 +21,7 @@ SYMBOLS = {
     "pto_gemm_mxfp8": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 5),
     "pto_gemm_mxfp4": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 4),
     "pto_topk_f32": (C.c_int, [C.c_void_p] * 5 + [C.c_int] * 4),
+    "pto_mla_attention_f32_s64_d32_r16": (C.c_int, [C.c_void_p] * 9 + [C.c_int] * 2),
     "pto_fa_fwd_f16": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 7),
     "pto_tcvt_f32_f16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),
     "pto_tcvt_f32_bf16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),
@@ -39,6 +40,8 @@ SYMBOLS = {
     "pto_st_matmul_f32_128x32x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_mx_128x256x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 3),
     "pto_st_vec_op_typed_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int]),
+    "pto_st_matmul_vec_operands_f16_64x64x128": (C.c_int, [C.c_void_p] * 5),
+    "pto_st_ttrans_f32_64x128": (C.c_int, [C.c_void_p] * 3),
     "pto_st_vec_bitop_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int, C.c_int]),
     "pto_st_vec_op_f32_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int]),
     "pto_st_reduce_f32_64x128": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 3),

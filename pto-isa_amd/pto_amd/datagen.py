@@ -164,6 +164,17 @@ def topk_inputs(rows, valid_cols, ld, distinct=0):
     return src, np.arange(valid_cols, dtype=np.uint32)
 
 
+def mla_inputs(batch, heads, x_scale=0.02, w_scale=0.02, seed=20251220):
+    """q, k, v [batch, heads, 64, 32] and wq, wk, wv [32, 16], wo [16, 32] fp32 for the multi-latent attention demo:
+    normal values times a scale (the reference demo uses 0.02 for everything, which makes the softmax almost uniform;
+    x_scale 1, w_scale 0.5 gives scores of a few units and a peaked softmax)."""
+    rng = np.random.default_rng(seed)
+    q, k, v = ((rng.standard_normal((batch, heads, 64, 32)) * x_scale).astype(np.float32) for _ in range(3))
+    wq, wk, wv = ((rng.standard_normal((32, 16)) * w_scale).astype(np.float32) for _ in range(3))
+    wo = (rng.standard_normal((16, 32)) * w_scale).astype(np.float32)
+    return q, k, v, wq, wk, wv, wo
+
+
 def gather_inputs(table_rows, cols, n_idx):
     """fp16 table of random bit patterns (NaNs included: the gather is a bit copy) and int32 row indices."""
     table = _rng(SEED_GATHER_TABLE).integers(0, 2**16, size=(table_rows, cols), dtype=np.uint16)

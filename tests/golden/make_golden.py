@@ -1,4 +1,4 @@
-"""Writes tests/golden/ref_vectors.npz: outputs of the COMPILED REFERENCE (oracle/_ref, built from the
+"""Writes tests/golden/ref_vectors.npz, ref_vec_ext.npz and ref_mla.npz: outputs of the COMPILED REFERENCE (oracle/_ref, built from the
 reference's CPU-simulation headers) on seeded inputs.  Run in the build container, where the reference
 tree is mounted; the fixture lets the oracle be checked against the reference where the tree is absent.
 
@@ -70,6 +70,24 @@ def vec_ext_cases(ref):
     return out
 
 
+MLA_CASES = {"demo_scale": (0.02, 0.02), "peaked": (1.0, 0.5)}
+
+
+def mla_cases(ref):
+    """The reference's CPU simulation running the multi-latent attention program on two heads -> ref_mla.npz."""
+    out = {}
+    for name, (xs, ws) in MLA_CASES.items():
+        q, k, v, wq, wk, wv, wo = datagen.mla_inputs(1, 2, xs, ws)
+        o = np.zeros_like(q)
+        for h in range(2):
+            oh = np.zeros((64, 32), dtype=np.float32)
+            ref.ref_mla_auto_64x32x16(p(oh), p(np.ascontiguousarray(q[0, h])), p(np.ascontiguousarray(k[0, h])),
+                                      p(np.ascontiguousarray(v[0, h])), p(wq), p(wk), p(wv), p(wo))
+            o[0, h] = oh
+        out["mla_" + name] = o
+    return out
+
+
 if __name__ == "__main__":
     oracle.build(ref=True)
     r = oracle.ref()
@@ -79,3 +97,5 @@ if __name__ == "__main__":
     print("wrote", os.path.join(HERE, "ref_vectors.npz"))
     np.savez_compressed(os.path.join(HERE, "ref_vec_ext.npz"), **vec_ext_cases(r))
     print("wrote", os.path.join(HERE, "ref_vec_ext.npz"))
+    np.savez_compressed(os.path.join(HERE, "ref_mla.npz"), **mla_cases(r))
+    print("wrote", os.path.join(HERE, "ref_mla.npz"))

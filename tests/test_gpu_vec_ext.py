@@ -233,3 +233,27 @@ def test_vec_bitop_rejects_bad_arguments():
     assert lib.pto_st_vec_bitop_64x128(st(), p, p, p, p, 0.0, 0, 17, 1) == capi.ERR_BAD_ARG
     assert lib.pto_st_vec_bitop_64x128(st(), p, p, p, p, 0.0, 0, 0, 0) == capi.ERR_UNSUPPORTED   # TAND on fp32
     assert lib.pto_st_vec_bitop_64x128(st(), p, p, 0, p, 0.0, 0, 0, 1) == capi.ERR_BAD_ARG
+
+
+def test_ttrans_and_tmov_to_operands():
+    """TTRANS is a permutation (bit-exact); TMOV Vec -> Left / Right and Acc -> Left feed matmuls whose small-integer
+    inputs make every product and sum exact in fp16 / fp32."""
+    lib = capi.load()
+    rng = np.random.default_rng(55)
+    x = rng.standard_normal((64, 128)).astype(np.float32)
+    x[0, :3] = [np.nan, np.inf, -0.0]
+    tx = dev(x)
+    ty = torch.zeros((128, 64), device=DEV)
+    capi.check(lib.pto_st_ttrans_f32_64x128(st(), ty.data_ptr(), tx.data_ptr()), "ttrans")
+    torch.cuda.synchronize()
+    assert np.array_equal(ty.cpu().numpy().view(np.uint32), np.ascontiguousarray(x.T).view(np.uint32))
+    a = rng.integers(-2, 3, size=(64, 64)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(64, 128)).astype(np.float32)
+    ta, tb = dev(a.astype(np.float16)), dev(b.astype(np.float16))
+    mid = torch.zeros((64, 128), device=DEV)
+    out = torch.zeros((64, 64), device=DEV)
+    capi.check(lib.pto_st_matmul_vec_operands_f16_64x64x128(st(), out.data_ptr(), mid.data_ptr(), ta.data_ptr(), tb.data_ptr()), "vec operands")
+    torch.cuda.synchronize()
+    want_mid = a @ b                                            # |values| <= 256: exact in fp16 as well
+    assert np.array_equal(mid.cpu().numpy(), want_mid)
+    assert np.array_equal(out.cpu().numpy(), want_mid @ b.T)

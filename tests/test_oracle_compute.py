@@ -578,3 +578,56 @@ def test_topk_oracle_matches_the_reference_golden_recipe(oracle):
     # known answer
     s, i = oracle.topk_f32(np.array([[1.0, 3.0, 2.0, 3.0, -1.0, 9.0]], dtype=np.float32), np.arange(5, dtype=np.uint32), 5, 3)
     assert s.tolist() == [[3.0, 3.0, 2.0]] and i.tolist() == [[1, 3, 2]]
+
+
+# ------------------------------------------------------------ multi-latent attention (the Auto-mode demo)
+MLA_GOLD = os.path.join(os.path.dirname(__file__), "golden", "ref_mla.npz")
+
+
+def _rel_to_max(got, want):
+    return float(np.max(np.abs(got.astype(np.float64) - want)) / np.max(np.abs(want)))
+
+
+@pytest.mark.parametrize("case,scales", [("demo_scale", (0.02, 0.02)), ("peaked", (1.0, 0.5))])
+def test_mla_oracle_vs_reference_outputs(oracle, case, scales):
+    """The float64 restatement against what the reference's CPU simulation produced for the same program (committed
+    outputs; also the compiled reference itself where it is built): an fp32 chain of five matmuls and a softmax
+    agrees with float64 to ~1e-6 of the largest output; a wrong scale, transposed weight or missing stage does not."""
+    args = datagen.mla_inputs(1, 2, *scales)
+    want = oracle.mla_attention(*args)
+    gold = np.load(MLA_GOLD)["mla_" + case]
+    assert _rel_to_max(gold, want.astype(np.float64)) < 5e-6
+    assert oracle.mla_verify_allclose(gold, want) == 0          # the demo's own acceptance test
+    r = oracle.ref()
+    if r is not None:
+        q, k, v, wq, wk, wv, wo = args
+        for h in range(2):
+            o = np.zeros((64, 32), dtype=np.float32)
+            r.ref_mla_auto_64x32x16(_p(o), _p(np.ascontiguousarray(q[0, h])), _p(np.ascontiguousarray(k[0, h])),
+                                    _p(np.ascontiguousarray(v[0, h])), _p(wq), _p(wk), _p(wv), _p(wo))
+            assert np.array_equal(o, gold[0, h])
+
+
+def test_mla_oracle_closed_forms(oracle):
+    from scipy.special import softmax
+    q, k, v, wq, wk, wv, wo = datagen.mla_inputs(2, 3, 1.0, 0.5, seed=5)
+    # no key projection: all scores are zero, the softmax is uniform, every position gets mean(V) Wv Wo
+    out = oracle.mla_attention(q, k, v, wq, np.zeros_like(wk), wv, wo)
+    want = (v.astype(np.float64).mean(axis=2, keepdims=True) @ wv.astype(np.float64)) @ wo.astype(np.float64)
+    assert np.max(np.abs(out - np.broadcast_to(want, out.shape))) < 1e-6
+    # associativity: P (V (Wv Wo)) with a library softmax of Q (Wq Wk^T) K^T / sqrt(R)
+    out = oracle.mla_attention(q, k, v, wq, wk, wv, wo)
+    q64, k64, v64 = (t.astype(np.float64) for t in (q, k, v))
+    sc = q64 @ (wq.astype(np.float64) @ wk.astype(np.float64).T) @ np.swapaxes(k64, 2, 3) / 4.0
+    want = softmax(sc, axis=-1) @ (v64 @ (wv.astype(np.float64) @ wo.astype(np.float64)))
+    assert np.max(np.abs(out - want)) < 1e-6 * np.max(np.abs(want))
+    # one key far ahead of the others: the output row is that key's value row projected
+    q1, k1 = np.zeros_like(q), np.zeros_like(k)
+    q1[..., 0], k1[:, :, 17, 0] = 40.0, 40.0
+    w1 = np.zeros_like(wq)
+    w1[0, 0] = 1.0
+    out = oracle.mla_attention(q1, k1, v, w1, w1, wv, wo)
+    want = (v64[:, :, 17:18] @ wv.astype(np.float64)) @ wo.astype(np.float64)
+    assert np.max(np.abs(out - np.broadcast_to(want, out.shape))) < 1e-6
+    # the acceptance test counts what it should
+    assert oracle.mla_verify_allclose(np.array([1.0, 2.0, np.nan, 0.0]), np.array([1.0001, 2.1, 0.0, 0.0])) == 2
