@@ -376,6 +376,25 @@ PTO_DEV void TROWEXPANDEXPDIF_IMPL(DstT &dst, DstT &src0, RowT &src1)
     hw::lds_barrier();
 }
 
+// LDS staging arrays of the moves that redistribute a tile over the workgroup (Acc -> Vec, Vec / Acc -> Left / Right,
+// TTRANS): one array per power-of-two size class, shared by every move of that class in a kernel.
+namespace detail {
+constexpr int stage_bytes(int n)
+{
+    int b = 1024;
+    while (b < n)
+        b *= 2;
+    return b;
+}
+// staging arrays are shared by all moves of a size class
+template <int Bytes>
+PTO_DEV char *stage_buffer()
+{
+    __shared__ __attribute__((aligned(16))) char buf[Bytes];
+    return buf;
+}
+} // namespace detail
+
 // ------------------------------------------------------- TMOV Acc -> Vec
 // Same-shape copy of an accumulator tile into a Vec tile, optionally clamped at zero
 // (TMov.hpp:20-69).  The accumulator's per-wave MFMA layout is redistributed through LDS.
@@ -387,7 +406,7 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
                   "[PTO][SA] TMOV Acc->Vec: row-major fp32 Vec tile of the accumulator's shape");
     using S = typename AccT::Storage;
     using T = typename DstT::DType;
-    __shared__ T stage[AccT::Rows * AccT::Cols];
+    T *stage = reinterpret_cast<T *>(detail::stage_buffer<detail::stage_bytes(AccT::Rows * AccT::Cols * (int)sizeof(T))>());
     const uint32_t lane = (uint32_t)hw::lane();
     const int rbase = hw::wave_m() * (S::MB * detail::kMfmaM) + detail::acc_lane_row(lane);
     const int cbase = hw::wave_n() * (S::NB * detail::kMfmaM) + detail::acc_lane_col(lane);
@@ -422,20 +441,6 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
 // destination's element type: k-contiguous per row for a Left destination, per column for a Right destination, so
 // that a fragment is one 16-byte read.
 namespace detail {
-constexpr int stage_bytes(int n)
-{
-    int b = 1024;
-    while (b < n)
-        b *= 2;
-    return b;
-}
-// staging arrays are shared by all moves of a size class
-template <int Bytes>
-PTO_DEV char *stage_buffer()
-{
-    __shared__ __attribute__((aligned(16))) char buf[Bytes];
-    return buf;
-}
 // every element (r, c) of a Vec or Acc tile -> stage[index(r, c)]
 template <typename T, typename SrcT, typename IndexF>
 PTO_DEV void stage_write(SrcT &src, T *stage, IndexF &&index)

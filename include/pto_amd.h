@@ -86,6 +86,13 @@ int pto_topk_f32(void *stream, float *out_score, uint32_t *out_index, const floa
 int pto_mla_attention_f32_s64_d32_r16(void *stream, float *out, const float *q, const float *k, const float *v, const float *wq,
                                       const float *wk, const float *wv, const float *wo, int batch, int heads);
 
+/* Whole-tile attention of the reference's Auto-mode demo and tflashattn system test
+ * (demos/cpu/flash_attention_demo/flash_attention_demo.cpp:169-258, flash_attention_pto(q, k, v, out)): fp32,
+ * out = softmax(q k^T / sqrt(head_dim)) v per (batch, head), scores as one [seq, seq] tile, one workgroup per head.
+ * q, k, v, out [batch, heads, seq, head_dim] contiguous; (seq, head_dim) = (64, 32) (the demo's) or (128, 64). */
+int pto_attention_auto_f32(void *stream, float *out, const float *q, const float *k, const float *v, int batch, int heads, int seq,
+                           int head_dim);
+
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];
  * lse: NULL or fp32 [batch, heads, seq_q] = max*scale + ln(sum).  scale = 1/sqrt(head_dim) is applied

@@ -114,6 +114,53 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MlaAttention(__gm__ floa
     TSTORE(gOut, oAcc);
 }
 
+// The reference's other Auto-mode attention program (demos/cpu/flash_attention_demo/flash_attention_demo.cpp:169-258,
+// flash_attention_pto; the same sequence is its tflashattn system test): O = softmax(Q K^T / sqrt(D)) V on one
+// [S, D] fp32 head per workgroup, scores and probabilities as whole [S, S] tiles.
+template <int S, int D>
+__global__ __launch_bounds__(kBlockThreads) AICORE void AttentionAuto(__gm__ float *out, __gm__ const float *q, __gm__ const float *k,
+                                                                      __gm__ const float *v)
+{
+    const size_t head = (size_t)get_block_idx() * S * D;
+    using RowStat = Tile<TileType::Vec, float, S, S, BLayout::ColMajor, S, S, SLayout::NoneBox>;
+    Gm<S, D> gq(const_cast<float *>(q) + head), gk(const_cast<float *>(k) + head), gv(const_cast<float *>(v) + head), go(out + head);
+    TileAcc<float, S, S> sAcc;
+    {
+        Plain<S, D> x;
+        Plain<D, S> kT;
+        TileLeft<float, S, D> qL;
+        TileRight<float, D, S> kR;
+        TLOAD(x, gq);
+        TMOV(qL, x);
+        TLOAD(x, gk);
+        TTRANS(kT, x, x);
+        TMOV(kR, kT);
+        TMATMUL(sAcc, qL, kR);
+    }
+    Plain<S, S> p;
+    TMOV(p, sAcc);
+    TMULS(p, p, 1.0f / __builtin_sqrtf((float)D));
+    {
+        RowStat rowMax, rowSum;
+        TROWMAX(rowMax, p, p);
+        TROWEXPANDSUB(p, p, rowMax);
+        TEXP(p, p);
+        TROWSUM(rowSum, p, p);
+        TROWEXPANDDIV(p, p, rowSum);
+    }
+    TileLeft<float, S, S> pL;
+    TMOV(pL, p);
+    TileRight<float, S, D> vR;
+    {
+        Plain<S, D> x;
+        TLOAD(x, gv);
+        TMOV(vR, x);
+    }
+    TileAcc<float, S, D> oAcc;
+    TMATMUL(oAcc, pL, vR);
+    TSTORE(go, oAcc);
+}
+
 } // namespace
 
 PTO_DEVICE_CODE_END
@@ -127,5 +174,23 @@ extern "C" int pto_mla_attention_f32_s64_d32_r16(void *stream, float *out, const
     if (blocks > 0x7fffffffLL)
         return PTO_ERR_UNSUPPORTED;
     MlaAttention<<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, q, k, v, wq, wk, wv, wo);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_attention_auto_f32(void *stream, float *out, const float *q, const float *k, const float *v, int batch, int heads,
+                                      int seq, int head_dim)
+{
+    if (!out || !q || !k || !v || batch <= 0 || heads <= 0)
+        return PTO_ERR_BAD_ARG;
+    const long long blocks = (long long)batch * heads;
+    if (blocks > 0x7fffffffLL)
+        return PTO_ERR_UNSUPPORTED;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (seq == 64 && head_dim == 32)
+        AttentionAuto<64, 32><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, st>>>(out, q, k, v);
+    else if (seq == 128 && head_dim == 64)
+        AttentionAuto<128, 64><<<dim3((unsigned)blocks), dim3(kBlockThreads), 0, st>>>(out, q, k, v);
+    else
+        return PTO_ERR_UNSUPPORTED;
     return pto_amd::check_launch();
 }

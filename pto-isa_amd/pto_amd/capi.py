@@ -21,6 +21,7 @@ SYMBOLS = {
     "pto_gemm_mxfp8": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 5),
     "pto_gemm_mxfp4": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 4),
     "pto_topk_f32": (C.c_int, [C.c_void_p] * 5 + [C.c_int] * 4),
+    "pto_attention_auto_f32": (C.c_int, [C.c_void_p] * 5 + [C.c_int] * 4),
     "pto_mla_attention_f32_s64_d32_r16": (C.c_int, [C.c_void_p] * 9 + [C.c_int] * 2),
     "pto_fa_fwd_f16": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 7),
     "pto_tcvt_f32_f16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),

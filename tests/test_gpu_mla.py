@@ -55,6 +55,33 @@ def test_mla_many_heads_and_limits(oracle):
     assert np.all(np.isfinite(got)) and rel(got, oracle.mla_attention(*args)) <= 1e-4
 
 
+@pytest.mark.parametrize("S,D", [(64, 32), (128, 64)])
+def test_attention_auto_vs_oracle_and_reference_output(oracle, S, D):
+    """The whole-tile fp32 attention program against the oracle's restatement of the same instruction sequence
+    (rounding-level agreement) and, at the demo's size and seed, against the committed output of the reference's CPU
+    simulation."""
+    from gpu_util import to_dev, stream
+    lib = capi.load()
+    rng = np.random.default_rng(20251220)
+    q, k, v = (rng.standard_normal((S, D), dtype=np.float32) for _ in range(3))   # the inputs of the committed output
+    extra = np.random.default_rng(8)
+    qs = np.stack([q] + [extra.standard_normal((S, D), dtype=np.float32) * 2 for _ in range(4)]).reshape(1, 5, S, D)
+    ks = np.stack([k] + [extra.standard_normal((S, D), dtype=np.float32) * 2 for _ in range(4)]).reshape(1, 5, S, D)
+    vs = np.stack([v] + [extra.standard_normal((S, D), dtype=np.float32) for _ in range(4)]).reshape(1, 5, S, D)
+    tq, tk, tv = to_dev(qs), to_dev(ks), to_dev(vs)
+    out = torch.full((1, 5, S, D), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(lib.pto_attention_auto_f32(stream(), out.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), 1, 5, S, D), "attention_auto")
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    for h in range(5):
+        want = oracle.fa_auto_f32(qs[0, h], ks[0, h], vs[0, h])
+        assert rel(got[0, h], want) <= TOL
+    if (S, D) == (64, 32):
+        gold = np.load(os.path.join(os.path.dirname(GOLD), "ref_vectors.npz"))["fa_auto_64x32"]
+        assert rel(got[0, 0], gold) <= TOL
+    assert lib.pto_attention_auto_f32(0, out.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), 1, 5, 96, 32) == capi.ERR_UNSUPPORTED
+
+
 def test_mla_rejects_bad_arguments():
     lib = capi.load()
     p = torch.zeros(64 * 32, device="cuda:0").data_ptr()
