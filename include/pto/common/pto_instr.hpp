@@ -8,6 +8,7 @@
 #include "pto/gfx950/vec_ops.hpp"
 #include "pto/gfx950/vec_ops_ext.hpp"
 #include "pto/gfx950/fifo_ops.hpp"
+#include "pto/gfx950/sort_ops.hpp"
 
 namespace pto {
 
@@ -174,6 +175,48 @@ PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
 {
     TSYNC(ev...);
     TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    return {};
+}
+
+// TSORT32 (pto_instr.hpp:786-798 of the reference; it takes no events) and TMRGSORT (pto_instr.hpp:582-622)
+template <typename D, typename S, typename I>
+PTO_INST RecordEvent TSORT32(D &dst, S &src, I &idx)
+{
+    TSORT32_IMPL(dst, src, idx);
+    return {};
+}
+template <typename D, typename S, typename I, typename Tmp>
+PTO_INST RecordEvent TSORT32(D &dst, S &src, I &idx, Tmp &tmp)
+{
+    TSORT32_IMPL(dst, src, idx, tmp);
+    return {};
+}
+template <typename D, typename Tmp, typename S0, typename S1, typename S2, typename S3, bool exhausted, typename... Ev>
+PTO_INST RecordEvent TMRGSORT(D &dst, MrgSortExecutedNumList &executed, Tmp &tmp, S0 &src0, S1 &src1, S2 &src2, S3 &src3, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMRGSORT_IMPL<D, Tmp, S0, S1, S2, S3, exhausted>(dst, executed, tmp, src0, src1, src2, src3);
+    return {};
+}
+template <typename D, typename Tmp, typename S0, typename S1, typename S2, bool exhausted, typename... Ev>
+PTO_INST RecordEvent TMRGSORT(D &dst, MrgSortExecutedNumList &executed, Tmp &tmp, S0 &src0, S1 &src1, S2 &src2, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMRGSORT_IMPL<D, Tmp, S0, S1, S2, exhausted>(dst, executed, tmp, src0, src1, src2);
+    return {};
+}
+template <typename D, typename Tmp, typename S0, typename S1, bool exhausted, typename... Ev>
+PTO_INST RecordEvent TMRGSORT(D &dst, MrgSortExecutedNumList &executed, Tmp &tmp, S0 &src0, S1 &src1, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMRGSORT_IMPL<D, Tmp, S0, S1, exhausted>(dst, executed, tmp, src0, src1);
+    return {};
+}
+template <typename D, typename S, typename... Ev>
+PTO_INST RecordEvent TMRGSORT(D &dst, S &src, uint32_t blockLen, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMRGSORT_IMPL(dst, src, blockLen);
     return {};
 }
 

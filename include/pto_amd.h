@@ -211,6 +211,20 @@ int pto_st_cmps_sel_f32_64x128(void *stream, float *sel, uint8_t *bits, const fl
 int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int pad_kind);
 /* out[64,128] = scale * (relu ? max(a b, 0) : a b): fp16 matmul [64,64] x [64,128] (b_t stored [128][64]), TMOV of
  * the accumulator into a Vec tile with ReluPreMode (cpu/TMov.hpp:53-69), TMULS, TSTORE. */
+/* TSORT32 (pto_instr.hpp:786-798, cpu/TSort32.hpp) on an [8,128] tile of fp32 (dtype 0) or int32 (dtype 1) scores with
+ * uint32 indices and the valid region [valid_rows, valid_cols]: out [8,256] is read, every group of 32 valid columns
+ * of a row is written back as (score, index bit pattern) structures in descending order of score, equal scores in
+ * ascending order of index, and the rest of out is left as it was. */
+int pto_st_tsort32_8x128(void *stream, void *out, const void *src, const uint32_t *idx, int valid_rows, int valid_cols, int dtype);
+/* TMRGSORT with one source (pto_instr.hpp:616-622, cpu/TMrgSort.hpp:181-230) on [1,1024] fp32 tiles: every complete
+ * group of four sorted blocks of block_len elements (block_len / 2 structures) inside the first valid_cols columns is
+ * merged; out is read first and keeps its other elements. */
+int pto_st_tmrgsort_blocks_f32_1x1024(void *stream, float *out, const float *src, int valid_cols, int block_len);
+/* TMRGSORT with 2..4 lists (pto_instr.hpp:582-614, cpu/TMrgSort.hpp:118-178): src_i [256] fp32 hold cols_i / 2 sorted
+ * (score, index) structures; the merge fills the first out_cols columns of out [1024] (read first), stops early when
+ * exhausted != 0 and a list runs empty, and reports in executed[4] how many structures of each list it took. */
+int pto_st_tmrgsort_lists_f32(void *stream, float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2,
+                              const float *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted);
 /* TMOV Vec -> Left / Right, Acc -> Left and TTRANS (the operand moves of the Auto-mode programs, cpu/TMov.hpp,
  * cpu/TTrans.hpp): a [64,64], b [64,128] fp16 row-major are loaded as Vec tiles and moved into operand tiles;
  * mid [64,128] = a b (fp32); out [64,64] = half(mid) b^T, with b^T made by TTRANS and half(mid) by the Acc -> Left move. */

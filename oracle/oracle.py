@@ -196,6 +196,76 @@ def topk_f32(src, in_idx, valid_cols, topk):
     return out_s, out_i
 
 
+def tsort32(dst, src, idx, valid_row, valid_col, index_as_value=False):
+    """TSORT32 (cpu/TSort32.hpp:44-88): in every row, every group of 32 valid columns is put in descending order of
+    score, equal scores in ascending order of index (a stable sort, so equal pairs keep their order), and written as
+    (score, index) structures at columns 2 j, 2 j + 1 of dst [rows, >= 2 cols] (the rest of dst is left as it is).
+    The index is stored as its bit pattern (the NPU form) or, index_as_value, converted to the element type by value
+    (what the CPU simulation's assignment does).  Pure Python: single tiles only."""
+    dst = np.array(dst, copy=True)
+    for r in range(valid_row):
+        for j in range(0, valid_col, 32):
+            n = min(32, valid_col - j)
+            order = sorted(range(n), key=lambda t: (-_sort_key(src[r, j + t]), int(idx[r, j + t]), t))
+            for m, t in enumerate(order):
+                dst[r, 2 * (j + m)] = src[r, j + t]
+                if index_as_value:
+                    dst[r, 2 * (j + m) + 1] = dst.dtype.type(idx[r, j + t])
+                else:
+                    dst[r, 2 * (j + m) + 1:2 * (j + m) + 2] = np.array([idx[r, j + t]], dtype=np.uint32).view(dst.dtype)
+    return dst
+
+
+def _sort_key(x):
+    return float(x) if isinstance(x, (np.floating, float)) else int(x)
+
+
+def _merge(lists, out_max, exhausted):
+    """The sequential merge of cpu/TMrgSort.hpp:118-178: take the head with the largest score, the lowest list
+    number on ties; stop at out_max structures, when everything is taken, or (exhausted) right after the structure
+    that empties a list.  lists: arrays [n_i, 2].  Returns (merged [m, 2], taken counts)."""
+    pos = [0] * len(lists)
+    out = []
+    while len(out) < out_max:
+        pick = -1
+        for b, l in enumerate(lists):
+            if pos[b] < len(l) and (pick < 0 or l[pos[b], 0] > lists[pick][pos[pick], 0]):
+                pick = b
+        if pick < 0:
+            break
+        out.append(lists[pick][pos[pick]])
+        pos[pick] += 1
+        if exhausted and any(pos[b] == len(l) for b, l in enumerate(lists)):
+            break
+    dt = lists[0].dtype
+    return (np.array(out, dtype=dt).reshape(-1, 2), pos)
+
+
+def tmrgsort_blocks(dst, src, valid_cols, block_len):
+    """TMRGSORT with one source (cpu/TMrgSort.hpp:181-230): every complete group of four blocks of block_len
+    elements inside the first valid_cols columns is merged; the rest of dst is left as it is."""
+    dst = np.array(dst, copy=True).reshape(-1)
+    src = np.asarray(src).reshape(-1)
+    if block_len == 0 or block_len % 2:
+        return dst
+    group = 4 * block_len
+    for c in range(0, valid_cols - group + 1, group):
+        lists = [src[c + b * block_len:c + (b + 1) * block_len].reshape(-1, 2) for b in range(4)]
+        merged, _ = _merge(lists, 2 * block_len, False)
+        dst[c:c + group] = merged.reshape(-1)
+    return dst
+
+
+def tmrgsort_lists(dst, lists, cols, out_cols, exhausted):
+    """TMRGSORT with two to four lists (cpu/TMrgSort.hpp:232-297): lists[i][:cols[i]] are (score, index) structures
+    in descending order of score; returns (dst with the merged structures in front, executed counts [4])."""
+    dst = np.array(dst, copy=True).reshape(-1)
+    ls = [np.asarray(l).reshape(-1)[:c // 2 * 2].reshape(-1, 2) for l, c in zip(lists, cols)]
+    merged, pos = _merge(ls, out_cols // 2, exhausted)
+    dst[:merged.size] = merged.reshape(-1)
+    return dst, np.array(pos + [0] * (4 - len(pos)), dtype=np.uint32)
+
+
 def fp8_table(fmt):
     """All 256 values of float8_e4m3fn (fmt 0) or float8_e5m2 (fmt 1), or the 16 of float4_e2m1 (fmt 4), as float32."""
     if fmt == 4:

@@ -520,6 +520,81 @@ void ref_mla_auto_64x32x16(float *out, const float *q, const float *k, const flo
 {
     mla_auto<64, 32, 16>(out, q, k, v, wq, wk, wv, wo);
 }
+// ---- TSORT32 / TMRGSORT on the tiles of the single-tile programs: [8,128] sources with a run-time valid region,
+// [1,1024] one-source merges, two to four [1,256] lists into [1,1024] ----
+extern "C++" {
+template <typename T>
+void sort32_8x128(T *out, const T *src, const uint32_t *idx, int vr, int vc)
+{
+    using S = Tile<TileType::Vec, T, 8, 128, BLayout::RowMajor, -1, -1>;
+    using I = Tile<TileType::Vec, uint32_t, 8, 128, BLayout::RowMajor, -1, -1>;
+    using D = Tile<TileType::Vec, T, 8, 256, BLayout::RowMajor>;
+    auto s = std::make_unique<S>(vr, vc);
+    auto x = std::make_unique<I>(vr, vc);
+    auto d = std::make_unique<D>();
+    std::memcpy(s->data(), src, sizeof(T) * 8 * 128);
+    std::memcpy(x->data(), idx, sizeof(uint32_t) * 8 * 128);
+    std::memcpy(d->data(), out, sizeof(T) * 8 * 256);
+    TSORT32(*d, *s, *x);
+    std::memcpy(out, d->data(), sizeof(T) * 8 * 256);
+}
+} // extern "C++"
+void ref_tsort32_f32_8x128(float *out, const float *src, const uint32_t *idx, int vr, int vc) { sort32_8x128<float>(out, src, idx, vr, vc); }
+void ref_tsort32_s32_8x128(int32_t *out, const int32_t *src, const uint32_t *idx, int vr, int vc)
+{
+    sort32_8x128<int32_t>(out, src, idx, vr, vc);
+}
+void ref_tmrgsort_blocks_f32_1x1024(float *out, const float *src, int valid_cols, int block_len)
+{
+    using S = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
+    using D = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, -1>;
+    auto s = std::make_unique<S>();
+    auto d = std::make_unique<D>(valid_cols);
+    std::memcpy(s->data(), src, sizeof(float) * 1024);
+    std::memcpy(d->data(), out, sizeof(float) * 1024);
+    TMRGSORT(*d, *s, static_cast<uint32_t>(block_len));
+    std::memcpy(out, d->data(), sizeof(float) * 1024);
+}
+extern "C++" {
+template <bool EXH>
+void mrgsort_lists(float *out, uint32_t *executed, const float *const *src, const int *cols, int out_cols, int lists)
+{
+    using L = Tile<TileType::Vec, float, 1, 256, BLayout::RowMajor, 1, -1>;
+    using D = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, -1>;
+    using Tmp = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
+    std::unique_ptr<L> l[4];
+    for (int i = 0; i < 4; ++i) {
+        l[i] = std::make_unique<L>(i < lists ? cols[i] : 0);
+        if (i < lists)
+            std::memcpy(l[i]->data(), src[i], sizeof(float) * 256);
+    }
+    auto d = std::make_unique<D>(out_cols);
+    auto tmp = std::make_unique<Tmp>();
+    std::memcpy(d->data(), out, sizeof(float) * 1024);
+    MrgSortExecutedNumList ex = {};
+    if (lists == 4)
+        TMRGSORT<D, Tmp, L, L, L, L, EXH>(*d, ex, *tmp, *l[0], *l[1], *l[2], *l[3]);
+    else if (lists == 3)
+        TMRGSORT<D, Tmp, L, L, L, EXH>(*d, ex, *tmp, *l[0], *l[1], *l[2]);
+    else
+        TMRGSORT<D, Tmp, L, L, EXH>(*d, ex, *tmp, *l[0], *l[1]);
+    std::memcpy(out, d->data(), sizeof(float) * 1024);
+    executed[0] = ex.mrgSortList0;
+    executed[1] = ex.mrgSortList1;
+    executed[2] = ex.mrgSortList2;
+    executed[3] = ex.mrgSortList3;
+}
+} // extern "C++"
+void ref_tmrgsort_lists_f32(float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2, const float *src3,
+                            int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
+{
+    const float *src[4] = {src0, src1, src2, src3};
+    const int cols[4] = {cols0, cols1, cols2, cols3};
+    if (exhausted)
+        mrgsort_lists<true>(out, executed, src, cols, out_cols, lists);
+    else
+        mrgsort_lists<false>(out, executed, src, cols, out_cols, lists);
+}
 void ref_fa_auto_128x64(float *out, const float *q, const float *k, const float *v) { fa_auto<128, 64>(out, q, k, v); }
 
 

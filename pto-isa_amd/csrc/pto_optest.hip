@@ -1029,6 +1029,147 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void TransKernel(__gm__ float
     TSTORE(go, y);
 }
 
+// ---- TSORT32 on an [8, 128] tile with valid region [vr, vc]; out [8, 256] is loaded first so that the elements the
+// instruction leaves alone keep what the caller put there ----
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) AICORE void Sort32Kernel(__gm__ T *out, __gm__ const T *srcIn, __gm__ const uint32_t *idxIn,
+                                                                    int vr, int vc)
+{
+    using Full = Tile<TileType::Vec, T, 8, 128, BLayout::RowMajor>;
+    using FullI = Tile<TileType::Vec, uint32_t, 8, 128, BLayout::RowMajor>;
+    using Src = Tile<TileType::Vec, T, 8, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    using Idx = Tile<TileType::Vec, uint32_t, 8, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    using Dst = Tile<TileType::Vec, T, 8, 256, BLayout::RowMajor>;
+    Full sf;
+    FullI xf;
+    Dst d;
+    GmND<T, 8, 128> gs(const_cast<T *>(srcIn));
+    GmND<uint32_t, 8, 128> gi(const_cast<uint32_t *>(idxIn));
+    GmND<T, 8, 256> go(out);
+    TLOAD(sf, gs);
+    TLOAD(xf, gi);
+    TLOAD(d, go);
+    Src s(vr, vc);
+    Idx x(vr, vc);
+    s.st = sf.st;
+    x.st = xf.st;
+    TSORT32(d, s, x);
+    TSTORE(go, d);
+}
+
+// ---- TMRGSORT, one source: [1, 1024] tile, the destination's valid columns and the block length at run time ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void MergeBlocksKernel(__gm__ float *out, __gm__ const float *srcIn, int validCols,
+                                                                          int blockLen)
+{
+    using Full = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
+    using Dst = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, DYNAMIC>;
+    Full s, d0;
+    GmND<float, 1, 1024> gs(const_cast<float *>(srcIn)), go(out);
+    TLOAD(s, gs);
+    TLOAD(d0, go);
+    Dst d(validCols);
+    d.st = d0.st;
+    TMRGSORT(d, s, (uint32_t)blockLen);
+    d0.st = d.st;
+    TSTORE(go, d0);
+}
+
+// ---- TMRGSORT, two to four lists of up to 128 structures each into a destination of up to 512 ----
+template <int LISTS, bool EXHAUSTED>
+__global__ __launch_bounds__(kBlockThreads) AICORE void MergeListsKernel(__gm__ float *out, __gm__ uint32_t *executedOut,
+                                                                         __gm__ const float *in0, __gm__ const float *in1,
+                                                                         __gm__ const float *in2, __gm__ const float *in3, int c0, int c1,
+                                                                         int c2, int c3, int outCols)
+{
+    using Full = Tile<TileType::Vec, float, 1, 256, BLayout::RowMajor>;
+    using List = Tile<TileType::Vec, float, 1, 256, BLayout::RowMajor, 1, DYNAMIC>;
+    using FullD = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
+    using Dst = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, DYNAMIC>;
+    Full f;
+    FullD d0, tmp;
+    List l0(c0), l1(c1), l2(c2), l3(c3);
+    GmND<float, 1, 1024> go(out);
+    const float *ins[4] = {in0, in1, in2, in3};
+    List *lists[4] = {&l0, &l1, &l2, &l3};
+#pragma unroll
+    for (int i = 0; i < LISTS; ++i) {
+        GmND<float, 1, 256> g(const_cast<float *>(ins[i]));
+        TLOAD(f, g);
+        lists[i]->st = f.st;
+    }
+    TLOAD(d0, go);
+    Dst d(outCols);
+    d.st = d0.st;
+    MrgSortExecutedNumList executed = {};
+    if constexpr (LISTS == 4)
+        TMRGSORT<Dst, FullD, List, List, List, List, EXHAUSTED>(d, executed, tmp, l0, l1, l2, l3);
+    else if constexpr (LISTS == 3)
+        TMRGSORT<Dst, FullD, List, List, List, EXHAUSTED>(d, executed, tmp, l0, l1, l2);
+    else
+        TMRGSORT<Dst, FullD, List, List, EXHAUSTED>(d, executed, tmp, l0, l1);
+    d0.st = d.st;
+    TSTORE(go, d0);
+    if (hw::tid() == 0) {
+        executedOut[0] = executed.mrgSortList0;
+        executedOut[1] = executed.mrgSortList1;
+        executedOut[2] = executed.mrgSortList2;
+        executedOut[3] = executed.mrgSortList3;
+    }
+}
+
+extern "C" int pto_st_tsort32_8x128(void *stream, void *out, const void *src, const uint32_t *idx, int valid_rows, int valid_cols, int dtype)
+{
+    PTO_ST_NONNULL(out, src, idx);
+    if (valid_rows < 0 || valid_rows > 8 || valid_cols < 0 || valid_cols > 128 || dtype < 0 || dtype > 1)
+        return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == 0)
+        Sort32Kernel<float><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<float *>(out), static_cast<const float *>(src), idx, valid_rows,
+                                                                    valid_cols);
+    else
+        Sort32Kernel<int32_t><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<int32_t *>(out), static_cast<const int32_t *>(src), idx,
+                                                                      valid_rows, valid_cols);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tmrgsort_blocks_f32_1x1024(void *stream, float *out, const float *src, int valid_cols, int block_len)
+{
+    PTO_ST_NONNULL(out, src);
+    if (valid_cols < 0 || valid_cols > 1024 || block_len < 0 || block_len > 256)
+        return PTO_ERR_BAD_ARG;
+    MergeBlocksKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, valid_cols, block_len);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tmrgsort_lists_f32(void *stream, float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2,
+                                         const float *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
+{
+    PTO_ST_NONNULL(out, executed, src0, src1);
+    if (lists < 2 || lists > 4 || (lists > 2 && !src2) || (lists > 3 && !src3) || out_cols < 0 || out_cols > 1024)
+        return PTO_ERR_BAD_ARG;
+    const int cols[4] = {cols0, cols1, cols2, cols3};
+    for (int i = 0; i < lists; ++i)
+        if (cols[i] < 0 || cols[i] > 256 || cols[i] % 2)
+            return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PTO_ST_MERGE(L, E) \
+    MergeListsKernel<L, E><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols)
+    if (lists == 4 && exhausted)
+        PTO_ST_MERGE(4, true);
+    else if (lists == 4)
+        PTO_ST_MERGE(4, false);
+    else if (lists == 3 && exhausted)
+        PTO_ST_MERGE(3, true);
+    else if (lists == 3)
+        PTO_ST_MERGE(3, false);
+    else if (exhausted)
+        PTO_ST_MERGE(2, true);
+    else
+        PTO_ST_MERGE(2, false);
+#undef PTO_ST_MERGE
+    return pto_amd::check_launch();
+}
+
 extern "C" int pto_st_matmul_vec_operands_f16_64x64x128(void *stream, float *out, float *mid, const uint16_t *a, const uint16_t *b)
 {
     PTO_ST_NONNULL(out, mid, a, b);

@@ -1,4 +1,4 @@
-"""Writes tests/golden/ref_vectors.npz, ref_vec_ext.npz and ref_mla.npz: outputs of the COMPILED REFERENCE (oracle/_ref, built from the
+"""Writes tests/golden/ref_vectors.npz, ref_vec_ext.npz, ref_mla.npz and ref_sort.npz: outputs of the COMPILED REFERENCE (oracle/_ref, built from the
 reference's CPU-simulation headers) on seeded inputs.  Run in the build container, where the reference
 tree is mounted; the fixture lets the oracle be checked against the reference where the tree is absent.
 
@@ -88,6 +88,30 @@ def mla_cases(ref):
     return out
 
 
+def sort_cases(ref):
+    """TSORT32 / TMRGSORT outputs of the reference's CPU simulation for the seeded cases of tests/sort_cases.py -> ref_sort.npz."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import sort_cases as sc
+    out = {}
+    for dtype, vr, vc, seed in sc.SORT32_CASES:
+        src, idx, o = sc.sort32_inputs(dtype, vr, vc, seed)
+        (ref.ref_tsort32_f32_8x128 if dtype == "f32" else ref.ref_tsort32_s32_8x128)(p(o), p(src), p(idx), vr, vc)
+        out["sort32_%d" % seed] = o
+    for valid_cols, block_len, seed in sc.BLOCK_CASES:
+        src, o = sc.block_inputs(valid_cols, block_len, seed)
+        ref.ref_tmrgsort_blocks_f32_1x1024(p(o), p(src), valid_cols, block_len)
+        out["blocks_%d" % seed] = o.view(np.uint32)
+    for counts, out_structs, exhausted, seed in sc.LIST_CASES:
+        lists, o = sc.list_inputs(counts, seed)
+        ex = np.zeros(4, dtype=np.uint32)
+        ptrs = [p(l) for l in lists] + [None] * (4 - len(lists))
+        cols = [2 * n for n in counts] + [0] * (4 - len(counts))
+        ref.ref_tmrgsort_lists_f32(p(o), p(ex), *ptrs, *cols, 2 * out_structs, len(counts), exhausted)
+        out["lists_%d" % seed] = o.view(np.uint32)
+        out["lists_%d_executed" % seed] = ex
+    return out
+
+
 if __name__ == "__main__":
     oracle.build(ref=True)
     r = oracle.ref()
@@ -99,3 +123,5 @@ if __name__ == "__main__":
     print("wrote", os.path.join(HERE, "ref_vec_ext.npz"))
     np.savez_compressed(os.path.join(HERE, "ref_mla.npz"), **mla_cases(r))
     print("wrote", os.path.join(HERE, "ref_mla.npz"))
+    np.savez_compressed(os.path.join(HERE, "ref_sort.npz"), **sort_cases(r))
+    print("wrote", os.path.join(HERE, "ref_sort.npz"))

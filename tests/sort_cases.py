@@ -1,0 +1,62 @@
+"""Seeded inputs for the TSORT32 / TMRGSORT tests (shared by the oracle tests, the GPU tests and tests/golden/make_golden.py)."""
+import numpy as np
+
+SORT32_CASES = [("f32", 8, 128, 0), ("f32", 8, 32, 1), ("f32", 5, 77, 2), ("s32", 7, 32, 3), ("s32", 8, 100, 4), ("f32", 1, 5, 5),
+                ("f32", 8, 128, 6)]
+
+
+def sort32_inputs(dtype, vr, vc, seed):
+    """src [8,128], idx [8,128] uint32, out0 [8,256] (what the destination holds before).  Scores are quantised so
+    that equal scores are frequent, indices repeat, and signed zeros appear."""
+    rng = np.random.default_rng(500 + seed)
+    if dtype == "f32":
+        src = (rng.integers(-12, 13, size=(8, 128)) * 0.25).astype(np.float32)
+        if seed == 6:
+            src = rng.standard_normal((8, 128)).astype(np.float32)      # distinct scores
+        src[0, 3], src[0, 9] = -0.0, 0.0
+        out0 = np.full((8, 256), -777.0, dtype=np.float32)
+    else:
+        src = rng.integers(-6, 7, size=(8, 128)).astype(np.int32)
+        src[1, :4] = [2**31 - 1, -2**31, 0, -1]
+        out0 = np.full((8, 256), -777, dtype=np.int32)
+    idx = rng.integers(0, 40, size=(8, 128)).astype(np.uint32)
+    idx[2, :] = np.arange(128, dtype=np.uint32) + 3000000000           # indices above 2^31 (and above 2^24)
+    return src, idx, out0
+
+
+def sorted_list(rng, n, lo=-8, hi=9, tag=0):
+    """n (score, index) structures in descending order of score, with ties; the index records list and position."""
+    scores = np.sort(rng.integers(lo, hi, size=n).astype(np.float32) * 0.5)[::-1]
+    out = np.empty((n, 2), dtype=np.float32)
+    out[:, 0] = scores
+    out[:, 1] = (np.arange(n, dtype=np.uint32) + np.uint32(1000 * tag)).view(np.float32)
+    return out
+
+
+BLOCK_CASES = [(1024, 64, 0), (1024, 256, 1), (700, 64, 2), (512, 8, 3), (1000, 128, 4), (100, 64, 5)]
+
+
+def block_inputs(valid_cols, block_len, seed):
+    rng = np.random.default_rng(600 + seed)
+    src = np.zeros(1024, dtype=np.float32)
+    per = block_len // 2
+    for b in range(1024 // block_len):
+        src[b * block_len:(b + 1) * block_len] = sorted_list(rng, per, tag=b).reshape(-1)
+    return src, np.full(1024, -555.0, dtype=np.float32)
+
+
+# (structures per list, out structures, exhausted, seed)
+LIST_CASES = [((128, 128, 128, 128), 512, 0, 0), ((128, 128, 128, 128), 512, 1, 1), ((100, 7, 64, 33), 204, 0, 2),
+              ((100, 7, 64, 33), 204, 1, 3), ((128, 90, 50), 268, 0, 4), ((128, 90, 50), 200, 1, 5), ((64, 128), 192, 0, 6),
+              ((64, 128), 100, 0, 7), ((64, 128), 192, 1, 8), ((5, 0, 9, 3), 17, 1, 9), ((5, 0, 9, 3), 17, 0, 10),
+              ((0, 0), 4, 1, 11), ((128, 128, 128, 128), 40, 1, 12)]
+
+
+def list_inputs(counts, seed):
+    rng = np.random.default_rng(700 + seed)
+    lists = []
+    for b, n in enumerate(counts):
+        l = np.full(256, 123.0, dtype=np.float32)
+        l[:2 * n] = sorted_list(rng, n, tag=b).reshape(-1)
+        lists.append(l)
+    return lists, np.full(1024, -555.0, dtype=np.float32)

@@ -1,0 +1,85 @@
+"""Pins the oracle's TSORT32 / TMRGSORT restatements (CPU only) against the committed outputs of the reference's CPU
+simulation (tests/golden/ref_sort.npz; the compiled reference itself where it is built) and against numpy's sorts."""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import sort_cases as sc
+
+GOLD = np.load(os.path.join(os.path.dirname(__file__), "golden", "ref_sort.npz"))
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+@pytest.mark.parametrize("dtype,vr,vc,seed", sc.SORT32_CASES)
+def test_tsort32_vs_reference_and_lexsort(oracle, dtype, vr, vc, seed):
+    src, idx, out0 = sc.sort32_inputs(dtype, vr, vc, seed)
+    # the CPU simulation stores the index converted by value
+    got = oracle.tsort32(out0, src, idx, vr, vc, index_as_value=True)
+    assert np.array_equal(got.view(np.uint32), GOLD["sort32_%d" % seed].view(np.uint32))
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        (r.ref_tsort32_f32_8x128 if dtype == "f32" else r.ref_tsort32_s32_8x128)(_p(o), _p(src), _p(idx), vr, vc)
+        assert np.array_equal(o.view(np.uint32), got.view(np.uint32))
+    # the bit-pattern form against numpy: per group, lexsort by (-score, index), position last
+    bits = oracle.tsort32(out0, src, idx, vr, vc)
+    for row in range(vr):
+        for j in range(0, vc, 32):
+            n = min(32, vc - j)
+            s = src[row, j:j + n].astype(np.float64)
+            order = np.lexsort((np.arange(n), idx[row, j:j + n], -s))
+            assert np.array_equal(bits[row, 2 * j:2 * (j + n):2], src[row, j + order])      # values (-0 == +0 may swap bits)
+            assert np.array_equal(bits[row, 2 * j + 1:2 * (j + n):2].view(np.uint32), idx[row, j + order])
+    # untouched: rows beyond the valid ones and columns beyond twice the valid ones
+    assert np.array_equal(bits[vr:], out0[vr:]) and np.array_equal(bits[:, 2 * vc:], out0[:, 2 * vc:])
+
+
+@pytest.mark.parametrize("valid_cols,block_len,seed", sc.BLOCK_CASES)
+def test_tmrgsort_blocks_vs_reference_and_stable_sort(oracle, valid_cols, block_len, seed):
+    src, out0 = sc.block_inputs(valid_cols, block_len, seed)
+    got = oracle.tmrgsort_blocks(out0, src, valid_cols, block_len)
+    assert np.array_equal(got.view(np.uint32), GOLD["blocks_%d" % seed])
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        r.ref_tmrgsort_blocks_f32_1x1024(_p(o), _p(src), valid_cols, block_len)
+        assert np.array_equal(o.view(np.uint32), got.view(np.uint32))
+    # merging sorted blocks = a stable sort of their concatenation by descending score
+    group = 4 * block_len
+    done = valid_cols // group * group
+    for c in range(0, done, group):
+        st = src[c:c + group].reshape(-1, 2)
+        order = np.argsort(-st[:, 0], kind="stable")
+        assert np.array_equal(got[c:c + group].view(np.uint32), st[order].reshape(-1).view(np.uint32))
+    assert np.array_equal(got[done:], out0[done:])
+
+
+@pytest.mark.parametrize("counts,out_structs,exhausted,seed", sc.LIST_CASES)
+def test_tmrgsort_lists_vs_reference_and_stable_sort(oracle, counts, out_structs, exhausted, seed):
+    lists, out0 = sc.list_inputs(counts, seed)
+    got, ex = oracle.tmrgsort_lists(out0, lists, [2 * n for n in counts], 2 * out_structs, exhausted)
+    assert np.array_equal(got.view(np.uint32), GOLD["lists_%d" % seed])
+    assert np.array_equal(ex, GOLD["lists_%d_executed" % seed])
+    r = oracle.ref()
+    if r is not None:
+        o, e = out0.copy(), np.zeros(4, dtype=np.uint32)
+        ptrs = [_p(l) for l in lists] + [None] * (4 - len(lists))
+        cols = [2 * n for n in counts] + [0] * (4 - len(counts))
+        r.ref_tmrgsort_lists_f32(_p(o), _p(e), *ptrs, *cols, 2 * out_structs, len(counts), exhausted)
+        assert np.array_equal(o.view(np.uint32), got.view(np.uint32)) and np.array_equal(e, ex)
+    # the merged prefix is a prefix of the stable sort of the concatenation; the counts say where it stops
+    cat = np.concatenate([l[:2 * n].reshape(-1, 2) for l, n in zip(lists, counts)])
+    full = cat[np.argsort(-cat[:, 0], kind="stable")] if len(cat) else cat
+    taken = int(ex.sum())
+    assert taken <= min(out_structs, len(cat))
+    assert np.array_equal(got[:2 * taken].view(np.uint32), full[:taken].reshape(-1).view(np.uint32))
+    assert np.array_equal(got[2 * taken:], out0[2 * taken:])
+    if not exhausted:
+        assert taken == min(out_structs, len(cat))
+    elif taken < min(out_structs, len(cat)):
+        assert any(int(ex[b]) == n for b, n in enumerate(counts))        # it stopped because a list ran empty
