@@ -29,8 +29,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 # counter reads for a plain 1 GiB device copy in the same run (--calib-copy): FETCH_SIZE reads
 # 524,300 KiB for 1,048,576 KiB actually read (factor 2.0), WRITE_SIZE reads 1,048,576 KiB for
 # 1,048,576 KiB written (factor 1.0).
-GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369647.0, 2.0
-GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 147905.0, 1.0
+GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369195.0, 2.0
+GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 151607.0, 1.0
 
 
 SETTLE_S = 0.0   # set from --settle-ms: the workloads under "extra" keep warming up until this much time has passed
@@ -333,7 +333,7 @@ def main():
     if gemm:
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                             "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": traffic,
-                            "kernel": "GemmF16F32Mix<256,256,4,4> (8 wavefronts per workgroup)", "flops_per_launch": gemm["flops"],
+                            "kernel": "GemmF16F32Fine<256,256,4> (4 wavefronts per workgroup)", "flops_per_launch": gemm["flops"],
                             "traffic_unit": "bytes per launch (read + write at the L2 <-> fabric boundary)",
                             "algorithmic_bytes": 2.0 * 2 * args.size ** 2 + 4.0 * args.size ** 2}
     if not args.no_cpu and only in ("", "gemm"):

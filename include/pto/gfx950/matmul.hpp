@@ -20,6 +20,16 @@ template <typename C>
 PTO_DEV C mfma32(f16x8 a, f16x8 b, C c)
 {
     static_assert(std::is_same_v<C, AccFrag>, "accumulator fragment of the configured MFMA shape");
+#ifdef PTO_MFMA_F16_ACC_IN_AGPRS
+    // The accumulator is pinned to the accumulation registers and the instruction keeps its place in the program: for
+    // kernels of one wave per SIMD that use all 256 accumulation registers, where the compiler's own choice between
+    // the two register files moves accumulators back and forth.  The caller leaves the wait states that the hardware
+    // needs between the last MFMA and the first ordinary read of an accumulator (s_nop) to this header's user.
+    if constexpr (sizeof(C) == 16) {
+        asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+        return c;
+    }
+#endif
     if constexpr (sizeof(C) == 64)
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     else

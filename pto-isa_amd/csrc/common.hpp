@@ -30,7 +30,10 @@ inline int allow_lds(K kernel, int bytes)
     return PTO_OK;
 }
 
-// defined in pto_gemm_w8.hip (workgroups of eight wavefronts)
+// defined in pto_gemm_m16w4.hip (workgroups of four wavefronts, one per SIMD); PTO_ERR_UNSUPPORTED = no tile shape of
+// that kernel fits the problem
+int gemm_f16f32_tile256_w4(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
+// defined in pto_gemm_m16.hip (workgroups of eight wavefronts)
 int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
 // defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries, two groups of four waves in
 // opposite MFMA / softmax phases)

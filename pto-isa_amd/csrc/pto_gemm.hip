@@ -60,7 +60,13 @@ extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const 
     // the reference kernel, two workgroups of four wavefronts per compute unit.
     const bool big = m % 256 == 0 && n % 256 == 0 && k % 128 == 0 && k / 32 >= 8 &&
                      (long long)(m / 256) * (n / 256) * 2 >= compute_units();
-    if (big)
+    if (big) {
+        // four wavefronts with the K-step written fragment by fragment where that kernel has a tile shape for the
+        // problem and is the faster one (uneven rounds, or 192 x 192 tiles for a single round), else eight wavefronts
+        const int rc = pto_amd::gemm_f16f32_tile256_w4(st, c, ha, hb, m, n, k);
+        if (rc != PTO_ERR_UNSUPPORTED)
+            return rc;
         return pto_amd::gemm_f16f32_tile256_w8(st, c, ha, hb, m, n, k);
+    }
     return launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
 }

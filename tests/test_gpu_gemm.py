@@ -30,7 +30,7 @@ def test_gemm_small_vs_oracle(oracle, m, n, k):
 
 
 def test_gemm_both_kernels_agree_with_integer_reference():
-    """4096 x 4096 selects the 256 x 256-tile kernel (one full round), 4096 x 4352 the same kernel with a
+    """4096 x 4096 selects the eight-wave 256 x 256-tile kernel (one full round), 4096 x 4352 the four-wave kernel with a
     last round of 128 x 128 quarter tiles, 1024 x 1024 the 128 x 256-block kernel: all exact on integer inputs."""
     from gpu_util import gemm
     for m, n, k in ((4096, 4096, 512), (4096, 4352, 512), (1024, 1024, 512)):
@@ -41,6 +41,29 @@ def test_gemm_both_kernels_agree_with_integer_reference():
         assert np.array_equal(got[rows], want), (m, n, k)
         colsum = b.astype(np.float64).sum(axis=0)
         assert np.array_equal(got.astype(np.float64).sum(axis=1), a.astype(np.float64) @ colsum)
+
+
+def test_gemm_four_wave_tile_shapes_exact():
+    """Every tile shape of the four-wave kernel (tuning hook: 256 x 256 with and without quarter tiles for the last
+    round, 192 x 256, 256 x 192, 192 x 192) on integer inputs: exact, whatever the tiling."""
+    import ctypes as C
+    import torch
+    from gpu_util import to_dev
+    lib = capi.load()
+    fn = lib.pto_gemm_f16f32_m16w4_variant
+    fn.restype, fn.argtypes = C.c_int, [C.c_void_p] * 4 + [C.c_int] * 4
+    for m, n, k in ((768, 1536, 512), (4352, 4096, 256)):
+        a, b = datagen.gemm_inputs_integer(m, n, k)
+        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
+        ta, tb = to_dev(a), to_dev(b)
+        for variant in (0, 1, 2, 3, 4):
+            if (m % 192 or n % 192) and variant >= 2:
+                assert fn(0, ta.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant) == capi.ERR_UNSUPPORTED
+                continue
+            tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "four-wave GEMM variant %d" % variant)
+            torch.cuda.synchronize()
+            assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
 
 
 def test_gemm_integer_inputs_exact(oracle):
