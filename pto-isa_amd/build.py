@@ -13,7 +13,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libpto_amd.so")
-SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_mx.hip", "pto_elementwise.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_optest.hip"]
+SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_mx.hip", "pto_elementwise.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_fa_w8m16.hip", "pto_optest.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
          # packed-fp32 VALU forms are kept off for every device function

@@ -45,6 +45,10 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
 #undef PTO_FA_VARIANT
     if (variant == 10 && head_dim == 128)
         return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false);
+    if (variant == 20 && head_dim == 128)
+        return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false);
+    if (variant == 21 && head_dim == 128) // fp32 output and LSE
+        return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, true);
     if (variant == 6 && head_dim == 128 && !causal)
         return launch_fa<128, false, false, 2, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
     if (variant == 6 && head_dim == 64 && causal)
@@ -74,8 +78,13 @@ extern "C" int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t 
                 n = 256;
             return n;
         }();
-        if ((long long)batch * heads * (seq_q / 256) >= cus)
+        if ((long long)batch * heads * (seq_q / 256) >= cus) {
+            // the same schedule on 16 x 16 x 32 MFMAs: +1.5 .. 3.6 % without a mask and for long causal sequences
+            // (interleaved runs; B2 H16 S2048 causal is 6 % slower on it and stays on the 32 x 32 x 16 kernel)
+            if (!causal || seq_kv >= 4096)
+                return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, o_fp32 != 0);
             return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, o_fp32 != 0);
+        }
     }
     // otherwise workgroups of four wavefronts (128 queries): two per compute unit at head_dim 128, three at 64
 #define PTO_FA_CASE(DD, CC, FF)                                                                      \

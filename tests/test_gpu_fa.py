@@ -138,6 +138,33 @@ def test_fa_d128_eight_wave_kernel_tile_counts(Skv, causal):
     assert np.array_equal(o16, o.astype(np.float16).astype(np.float32))
 
 
+@pytest.mark.parametrize("Sq,Skv", [(4096, 4096), (256, 4160)])
+def test_fa_d128_eight_wave_kernel_on_16x16x32_causal(Sq, Skv):
+    """Long causal sequences at head_dim 128 run the eight-wavefront kernel on 16 x 16 x 32 MFMAs (as every unmasked
+    problem of that size does): diagonal inside the tiles, an offset diagonal (seq_kv > seq_q), fp32 output + LSE."""
+    B, H, D = (1, 16, 128) if Sq == 4096 else (16, 16, 128)
+    q, k, v = datagen.fa_inputs(B, H, Sq, Skv, D, scale=1.0)
+    o, lse = fa_gpu(q, k, v, causal=True, o_fp32=True)
+    assert np.all(np.isfinite(o)) and np.all(np.isfinite(lse))
+    for b, h in ((0, 0), (B - 1, 13)):
+        want, want_lse = dense_fp64(q[b, h], k[b, h], v[b, h], causal=True)
+        assert rel(o[b, h], want) <= TOL
+        assert np.max(np.abs(lse[b, h] - want_lse)) <= 1e-3
+    if Sq == Skv:
+        assert np.allclose(o[:, :, 0, :], v[:, :, 0, :].astype(np.float32), atol=1e-6)
+
+
+def test_fa_d128_eight_wave_kernel_on_16x16x32_vs_streaming_oracle(oracle):
+    """The same kernel against the oracle's streaming recurrence with its key tile (64) and fp16 P: rounding only."""
+    B, H, Sq, Skv, D = 16, 16, 256, 192, 128
+    q, k, v = datagen.fa_inputs(B, H, Sq, Skv, D, scale=1.0)
+    o, lse = fa_gpu(q, k, v, causal=False, o_fp32=True)
+    for b, h in ((0, 0), (9, 5)):
+        oo, m, l = oracle.fa_stream_f16(q[b, h], k[b, h], v[b, h], tile_s1=64, causal=False, q_offset=0, round_away=False)
+        assert rel(o[b, h], oo) <= 5e-4
+        assert np.max(np.abs(lse[b, h] - (m / np.sqrt(D) + np.log(l)))) <= 1e-4
+
+
 def test_fa_config4_causal_b4_h32_s2048_d64():
     """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row."""
     B, H, S, D = 4, 32, 2048, 64
