@@ -113,6 +113,9 @@ PTO_FRONT(TSHL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a 
 PTO_FRONT(TSHR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TREM, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TNOT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TPARTADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TPARTMAX, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TPARTMIN, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TANDS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TORS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TSHLS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))

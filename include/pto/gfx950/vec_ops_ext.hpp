@@ -634,4 +634,40 @@ PTO_DEV void TADDSC_IMPL(TileT &dst, TileT &src0, typename TileT::DType k, TileT
 template <typename TileT>
 PTO_DEV void TSUBSC_IMPL(TileT &dst, TileT &src0, typename TileT::DType k, TileT &src1) { vec_addsc<true>(dst, src0, k, src1); }
 
+// ------------------------------------------------------ TPARTADD / TPARTMAX / TPARTMIN
+// Elementwise over the destination's valid region where the sources' valid regions may be smaller (cpu/TPartOp.hpp:19-45):
+// both sources valid -> op(src0, src1); one valid -> that source's element; none -> 0.  Tiles of one shape.
+namespace detail {
+template <int KIND, typename DstT, typename S0T, typename S1T> // KIND: 0 add, 1 max, 2 min
+PTO_DEV void part_op(DstT &dst, S0T &src0, S1T &src1)
+{
+    using T = typename DstT::DType;
+    static_assert(DstT::Loc == TileType::Vec && S0T::Loc == TileType::Vec && S1T::Loc == TileType::Vec && DstT::Rows == S0T::Rows &&
+                      DstT::Cols == S0T::Cols && DstT::Rows == S1T::Rows && DstT::Cols == S1T::Cols && DstT::isRowMajor == S0T::isRowMajor &&
+                      DstT::isRowMajor == S1T::isRowMajor,
+                  "[PTO][SA] TPART*: Vec tiles of one shape and layout");
+    static_assert(std::is_same_v<typename S0T::DType, T> && std::is_same_v<typename S1T::DType, T>, "[PTO][SA] TPART*: one element type");
+    const int dvr = dst.GetValidRow(), dvc = dst.GetValidCol(), avr = src0.GetValidRow(), avc = src0.GetValidCol(),
+              bvr = src1.GetValidRow(), bvc = src1.GetValidCol();
+    for_each_owned<DstT>([&](int s, int i, int e) {
+        if (e < DstT::Numel) {
+            int r, c;
+            elem_rc<DstT>(e, r, c);
+            if (r < dvr && c < dvc) {
+                const bool in0 = r < avr && c < avc, in1 = r < bvr && c < bvc;
+                const T a = src0.st.v[s][i], b = src1.st.v[s][i];
+                const T both = KIND == 0 ? (T)(a + b) : KIND == 1 ? (a < b ? b : a) : (b < a ? b : a);
+                dst.st.v[s][i] = in0 && in1 ? both : in0 ? a : in1 ? b : (T)0;
+            }
+        }
+    });
+}
+} // namespace detail
+template <typename DstT, typename S0T, typename S1T>
+PTO_DEV void TPARTADD_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<0>(dst, src0, src1); }
+template <typename DstT, typename S0T, typename S1T>
+PTO_DEV void TPARTMAX_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<1>(dst, src0, src1); }
+template <typename DstT, typename S0T, typename S1T>
+PTO_DEV void TPARTMIN_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<2>(dst, src0, src1); }
+
 } // namespace pto

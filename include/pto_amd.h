@@ -211,6 +211,11 @@ int pto_st_cmps_sel_f32_64x128(void *stream, float *sel, uint8_t *bits, const fl
 int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int valid_rows, int valid_cols, int pad_kind);
 /* out[64,128] = scale * (relu ? max(a b, 0) : a b): fp16 matmul [64,64] x [64,128] (b_t stored [128][64]), TMOV of
  * the accumulator into a Vec tile with ReluPreMode (cpu/TMov.hpp:53-69), TMULS, TSTORE. */
+/* TPARTADD (op 0), TPARTMAX (1), TPARTMIN (2) on [64,128] fp32 tiles (cpu/TPartOp.hpp:19-45): over the destination's valid
+ * region, op(a, b) where both sources are valid, the valid source's element where one is, 0 where none is; out is read
+ * first and keeps its elements outside the destination's valid region. */
+int pto_st_tpart_f32_64x128(void *stream, float *out, const float *a, const float *b, int op, int dst_valid_rows, int dst_valid_cols,
+                            int a_valid_rows, int a_valid_cols, int b_valid_rows, int b_valid_cols);
 /* TSORT32 (pto_instr.hpp:786-798, cpu/TSort32.hpp) on an [8,128] tile of fp32 (dtype 0) or int32 (dtype 1) scores with
  * uint32 indices and the valid region [valid_rows, valid_cols]: out [8,256] is read, every group of 32 valid columns
  * of a row is written back as (score, index bit pattern) structures in descending order of score, equal scores in

@@ -196,6 +196,20 @@ def topk_f32(src, in_idx, valid_cols, topk):
     return out_s, out_i
 
 
+def tpart(dst, a, b, op, dvalid, avalid, bvalid):
+    """TPARTADD (op 0) / TPARTMAX (1) / TPARTMIN (2), cpu/TPartOp.hpp:19-45: over dst's valid region [dvr, dvc]: op(a, b)
+    where both sources are inside their valid regions, the element of the one that is where only one is, 0 where none
+    is; the rest of dst is left as it is."""
+    dst = np.array(dst, copy=True)
+    (dvr, dvc), (avr, avc), (bvr, bvc) = dvalid, avalid, bvalid
+    r, c = np.meshgrid(np.arange(dst.shape[0]), np.arange(dst.shape[1]), indexing="ij")
+    in_a, in_b, in_d = (r < avr) & (c < avc), (r < bvr) & (c < bvc), (r < dvr) & (c < dvc)
+    both = a + b if op == 0 else np.maximum(a, b) if op == 1 else np.minimum(a, b)
+    val = np.where(in_a & in_b, both, np.where(in_a, a, np.where(in_b, b, 0))).astype(dst.dtype)
+    dst[in_d] = val[in_d]
+    return dst
+
+
 def tsort32(dst, src, idx, valid_row, valid_col, index_as_value=False):
     """TSORT32 (cpu/TSort32.hpp:44-88): in every row, every group of 32 valid columns is put in descending order of
     score, equal scores in ascending order of index (a stable sort, so equal pairs keep their order), and written as

@@ -544,6 +544,21 @@ void ref_tsort32_s32_8x128(int32_t *out, const int32_t *src, const uint32_t *idx
 {
     sort32_8x128<int32_t>(out, src, idx, vr, vc);
 }
+void ref_tpart_f32_64x128(float *out, const float *a, const float *b, int op, int dvr, int dvc, int avr, int avc, int bvr, int bvc)
+{
+    using Dyn = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, -1, -1>;
+    auto ta = std::make_unique<Dyn>(avr, avc), tb = std::make_unique<Dyn>(bvr, bvc), td = std::make_unique<Dyn>(dvr, dvc);
+    std::memcpy(ta->data(), a, sizeof(float) * 64 * 128);
+    std::memcpy(tb->data(), b, sizeof(float) * 64 * 128);
+    std::memcpy(td->data(), out, sizeof(float) * 64 * 128);
+    if (op == 0)
+        TPARTADD(*td, *ta, *tb);
+    else if (op == 1)
+        TPARTMAX(*td, *ta, *tb);
+    else
+        TPARTMIN(*td, *ta, *tb);
+    std::memcpy(out, td->data(), sizeof(float) * 64 * 128);
+}
 void ref_tmrgsort_blocks_f32_1x1024(float *out, const float *src, int valid_cols, int block_len)
 {
     using S = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;

@@ -1117,6 +1117,46 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MergeListsKernel(__gm__ 
     }
 }
 
+// ---- TPARTADD / TPARTMAX / TPARTMIN on [64, 128] fp32 tiles whose three valid regions come at run time; out is loaded
+// first so that the elements outside the destination's valid region keep what the caller put there ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void PartOpKernel(__gm__ float *out, __gm__ const float *aIn, __gm__ const float *bIn,
+                                                                     int op, int dvr, int dvc, int avr, int avc, int bvr, int bvc)
+{
+    using Full = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    using Dyn = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    Full fa, fb, fo;
+    GmND<float, 64, 128> ga(const_cast<float *>(aIn)), gb(const_cast<float *>(bIn)), go(out);
+    TLOAD(fa, ga);
+    TLOAD(fb, gb);
+    TLOAD(fo, go);
+    Dyn a(avr, avc), b(bvr, bvc), d(dvr, dvc);
+    a.st = fa.st;
+    b.st = fb.st;
+    d.st = fo.st;
+    if (op == 0)
+        TPARTADD(d, a, b);
+    else if (op == 1)
+        TPARTMAX(d, a, b);
+    else
+        TPARTMIN(d, a, b);
+    fo.st = d.st;
+    TSTORE(go, fo);
+}
+
+extern "C" int pto_st_tpart_f32_64x128(void *stream, float *out, const float *a, const float *b, int op, int dst_valid_rows,
+                                       int dst_valid_cols, int a_valid_rows, int a_valid_cols, int b_valid_rows, int b_valid_cols)
+{
+    PTO_ST_NONNULL(out, a, b);
+    const int v[6] = {dst_valid_rows, dst_valid_cols, a_valid_rows, a_valid_cols, b_valid_rows, b_valid_cols};
+    for (int i = 0; i < 6; ++i)
+        if (v[i] < 0 || v[i] > (i % 2 ? 128 : 64))
+            return PTO_ERR_BAD_ARG;
+    if (op < 0 || op > 2)
+        return PTO_ERR_BAD_ARG;
+    PartOpKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, a, b, op, v[0], v[1], v[2], v[3], v[4], v[5]);
+    return pto_amd::check_launch();
+}
+
 extern "C" int pto_st_tsort32_8x128(void *stream, void *out, const void *src, const uint32_t *idx, int valid_rows, int valid_cols, int dtype)
 {
     PTO_ST_NONNULL(out, src, idx);

@@ -109,6 +109,10 @@ def sort_cases(ref):
         ref.ref_tmrgsort_lists_f32(p(o), p(ex), *ptrs, *cols, 2 * out_structs, len(counts), exhausted)
         out["lists_%d" % seed] = o.view(np.uint32)
         out["lists_%d_executed" % seed] = ex
+    for n, (op, dv, av, bv) in enumerate(sc.PART_CASES):
+        a, b, o = sc.part_inputs(n)
+        ref.ref_tpart_f32_64x128(p(o), p(a), p(b), op, *dv, *av, *bv)
+        out["part_%d" % n] = o[::3].copy()      # every third row keeps the fixture small
     return out
 
 

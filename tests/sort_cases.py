@@ -60,3 +60,16 @@ def list_inputs(counts, seed):
         l[:2 * n] = sorted_list(rng, n, tag=b).reshape(-1)
         lists.append(l)
     return lists, np.full(1024, -555.0, dtype=np.float32)
+
+
+# TPARTADD / TPARTMAX / TPARTMIN: (op, dst valid, a valid, b valid)
+PART_CASES = [(0, (64, 128), (64, 128), (64, 128)), (0, (64, 128), (40, 128), (64, 70)), (1, (50, 100), (64, 60), (30, 128)),
+              (2, (64, 128), (10, 20), (64, 128)), (1, (64, 128), (0, 0), (33, 77)), (2, (20, 30), (64, 128), (5, 128)),
+              (0, (64, 128), (17, 33), (40, 9))]
+
+
+def part_inputs(seed):
+    rng = np.random.default_rng(800 + seed)
+    a = rng.standard_normal((64, 128)).astype(np.float32)
+    b = rng.standard_normal((64, 128)).astype(np.float32)
+    return a, b, np.full((64, 128), -999.0, dtype=np.float32)

@@ -71,10 +71,25 @@ def test_tmrgsort_lists(oracle, counts, out_structs, exhausted, seed):
     assert np.array_equal(got, GOLD["lists_%d" % seed]) and np.array_equal(ex, GOLD["lists_%d_executed" % seed])
 
 
+@pytest.mark.parametrize("n", range(len(sc.PART_CASES)))
+def test_tpart(oracle, n):
+    lib = capi.load()
+    op, dv, av, bv = sc.PART_CASES[n]
+    a, b, out0 = sc.part_inputs(n)
+    ta, tb, to = _dev(a), _dev(b), _dev(out0)
+    capi.check(lib.pto_st_tpart_f32_64x128(_st(), to.data_ptr(), ta.data_ptr(), tb.data_ptr(), op, *dv, *av, *bv), "tpart")
+    torch.cuda.synchronize()
+    got = to.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oracle.tpart(out0, a, b, op, dv, av, bv).view(np.uint32))
+    assert np.array_equal(got[::3].view(np.uint32), GOLD["part_%d" % n].view(np.uint32))
+
+
 def test_sort_programs_reject_bad_arguments():
     lib = capi.load()
     p = torch.zeros(2048, device="cuda:0").data_ptr()
     assert lib.pto_st_tsort32_8x128(0, p, p, p, 9, 32, 0) == capi.ERR_BAD_ARG
+    assert lib.pto_st_tpart_f32_64x128(0, p, p, p, 3, 64, 128, 64, 128, 64, 128) == capi.ERR_BAD_ARG
+    assert lib.pto_st_tpart_f32_64x128(0, p, p, p, 0, 65, 128, 64, 128, 64, 128) == capi.ERR_BAD_ARG
     assert lib.pto_st_tmrgsort_blocks_f32_1x1024(0, p, p, 2048, 64) == capi.ERR_BAD_ARG
     assert lib.pto_st_tmrgsort_lists_f32(0, p, p, p, p, 0, 0, 64, 64, 64, 0, 256, 3, 0) == capi.ERR_BAD_ARG      # third list missing
     assert lib.pto_st_tmrgsort_lists_f32(0, p, p, p, p, p, p, 63, 64, 64, 64, 256, 4, 0) == capi.ERR_BAD_ARG      # odd column count

@@ -83,3 +83,27 @@ def test_tmrgsort_lists_vs_reference_and_stable_sort(oracle, counts, out_structs
         assert taken == min(out_structs, len(cat))
     elif taken < min(out_structs, len(cat)):
         assert any(int(ex[b]) == n for b, n in enumerate(counts))        # it stopped because a list ran empty
+
+
+@pytest.mark.parametrize("n", range(len(sc.PART_CASES)))
+def test_tpart_vs_reference(oracle, n):
+    """TPARTADD / TPARTMAX / TPARTMIN against the reference's CPU simulation (committed outputs, every third row; all
+    rows where the compiled reference is built) and against the definition applied region by region."""
+    op, dv, av, bv = sc.PART_CASES[n]
+    a, b, out0 = sc.part_inputs(n)
+    got = oracle.tpart(out0, a, b, op, dv, av, bv)
+    assert np.array_equal(got[::3].view(np.uint32), GOLD["part_%d" % n].view(np.uint32))
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        r.ref_tpart_f32_64x128(_p(o), _p(a), _p(b), op, *dv, *av, *bv)
+        assert np.array_equal(o.view(np.uint32), got.view(np.uint32))
+    f = [np.add, np.maximum, np.minimum][op]
+    rr, cc = min(dv[0], av[0], bv[0]), min(dv[1], av[1], bv[1])
+    assert np.array_equal(got[:rr, :cc], f(a[:rr, :cc], b[:rr, :cc]))                    # both valid
+    assert np.array_equal(got[dv[0]:], out0[dv[0]:]) and np.array_equal(got[:, dv[1]:], out0[:, dv[1]:])   # outside dst: untouched
+    none = np.zeros((64, 128), dtype=bool)
+    none[:dv[0], :dv[1]] = True
+    none[:av[0], :av[1]] = False
+    none[:bv[0], :bv[1]] = False
+    assert np.all(got[none] == 0)                                                          # neither source valid
