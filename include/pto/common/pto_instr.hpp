@@ -113,6 +113,8 @@ PTO_FRONT(TSHL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a 
 PTO_FRONT(TSHR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TREM, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TNOT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TSCATTER, typename D PTO_C typename I, D &dst PTO_C D &src PTO_C I &indexes, (dst, src, indexes))
+PTO_FRONT(MSCATTER, typename G PTO_C typename S PTO_C typename I, G &dst PTO_C S &src PTO_C I &indexes, (dst, src, indexes))
 PTO_FRONT(TPARTADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TPARTMAX, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TPARTMIN, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
@@ -178,6 +180,15 @@ PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
 {
     TSYNC(ev...);
     TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    return {};
+}
+
+// TCI (pto_instr.hpp:808-814 of the reference)
+template <typename TileT, typename T, int descending, typename... Ev>
+PTO_INST RecordEvent TCI(TileT &dst, T start, Ev &... ev)
+{
+    TSYNC(ev...);
+    TCI_IMPL<TileT, T, descending>(dst, start);
     return {};
 }
 

@@ -670,4 +670,77 @@ PTO_DEV void TPARTMAX_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<1>
 template <typename DstT, typename S0T, typename S1T>
 PTO_DEV void TPARTMIN_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<2>(dst, src0, src1); }
 
+// ------------------------------------------------------------ TCI, TSCATTER, MSCATTER
+// TCI (cpu/TCI.hpp:16-35): dst[0, j] = start + j (descending: start - j) over the valid columns of a one-row tile.
+template <typename TileT, typename T, int descending>
+PTO_DEV void TCI_IMPL(TileT &dst, T start)
+{
+    static_assert(TileT::Loc == TileType::Vec && TileT::Rows == 1 && std::is_same_v<typename TileT::DType, T>,
+                  "[PTO][SA] TCI: one-row Vec tile of the start value's type");
+    const int vc = dst.GetValidCol();
+    detail::for_each_owned<TileT>([&](int s, int i, int e) {
+        if (e < vc)
+            dst.st.v[s][i] = descending == 1 ? (T)(start - (T)e) : (T)(start + (T)e);
+    });
+}
+
+// TSCATTER (cpu/TScatter.hpp:21-44): dst[indexes[i, j], j] = src[i, j] over the source's valid region.  The reference
+// walks the rows in order, so where several rows send an element to the same place the last one wins: the winner is
+// found with an atomic maximum over the source row numbers in LDS.  Rows outside the tile are dropped (the reference
+// writes out of bounds there).  4-byte elements.
+template <typename TileT, typename IdxT>
+PTO_DEV void TSCATTER_IMPL(TileT &dst, TileT &src, IdxT &indexes)
+{
+    using T = typename TileT::DType;
+    static_assert(TileT::Loc == TileType::Vec && IdxT::Loc == TileType::Vec && TileT::isRowMajor && IdxT::isRowMajor && sizeof(T) == 4 &&
+                      std::is_integral_v<typename IdxT::DType> && IdxT::Rows == TileT::Rows && IdxT::Cols == TileT::Cols,
+                  "[PTO][SA] TSCATTER: row-major Vec tiles of 4-byte elements, integer index tile of the same shape");
+    constexpr int N = TileT::Numel;
+    int *owner = reinterpret_cast<int *>(detail::stage_buffer<detail::stage_bytes(8 * N)>());
+    uint32_t *value = reinterpret_cast<uint32_t *>(owner + N);
+    for (int e = hw::tid(); e < N; e += kBlockThreads)
+        owner[e] = -1;
+    hw::lds_barrier();
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    detail::for_each_owned<TileT>([&](int s, int i, int e) {
+        const int r = e / TileT::Cols, c = e % TileT::Cols;
+        const uint32_t row = (uint32_t)indexes.st.v[s][i];
+        if (e < N && r < vr && c < vc && row < (uint32_t)TileT::Rows)
+            atomicMax(&owner[row * TileT::Cols + c], r);
+    });
+    hw::lds_barrier();
+    detail::for_each_owned<TileT>([&](int s, int i, int e) {
+        const int r = e / TileT::Cols, c = e % TileT::Cols;
+        const uint32_t row = (uint32_t)indexes.st.v[s][i];
+        if (e < N && r < vr && c < vc && row < (uint32_t)TileT::Rows && owner[row * TileT::Cols + c] == r)
+            value[row * TileT::Cols + c] = __builtin_bit_cast(uint32_t, src.st.v[s][i]);
+    });
+    hw::lds_barrier();
+    detail::for_each_owned<TileT>([&](int s, int i, int e) {
+        if (e < N && owner[e] >= 0)
+            dst.st.v[s][i] = __builtin_bit_cast(T, value[e]);
+    });
+    hw::lds_barrier();
+}
+
+// MSCATTER (cpu/MGatherScatter.hpp:46-69): memory[indexes[i, j]] = src[i, j] over the source's valid region, the dual of
+// MGATHER.  Elements sent to the same address: the reference keeps the last in row-major order, here one of them
+// arrives last - callers that need the reference's result pass distinct indices.
+template <typename G, typename SrcT, typename IdxT>
+PTO_DEV void MSCATTER_IMPL(G &dst, SrcT &src, IdxT &indexes)
+{
+    static_assert(sizeof(typename SrcT::DType) == sizeof(typename G::DType), "[PTO][SA] MSCATTER: element sizes differ");
+    static_assert(SrcT::Numel == IdxT::Numel && SrcT::isRowMajor == IdxT::isRowMajor && std::is_integral_v<typename IdxT::DType>,
+                  "[PTO][SA] MSCATTER: source and integer index tiles of the same shape");
+    using T = typename SrcT::DType;
+    T *gm = reinterpret_cast<T *>(dst.data());
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    detail::for_each_owned<SrcT>([&](int s, int i, int e) {
+        int r, c;
+        detail::elem_rc<SrcT>(e, r, c);
+        if (e < SrcT::Numel && r < vr && c < vc)
+            gm[(size_t)indexes.st.v[s][i]] = src.st.v[s][i];
+    });
+}
+
 } // namespace pto

@@ -216,6 +216,15 @@ int pto_st_fillpad_f32_64x128(void *stream, float *out, const float *a, int vali
  * first and keeps its elements outside the destination's valid region. */
 int pto_st_tpart_f32_64x128(void *stream, float *out, const float *a, const float *b, int op, int dst_valid_rows, int dst_valid_cols,
                             int a_valid_rows, int a_valid_cols, int b_valid_rows, int b_valid_cols);
+/* TSCATTER (to_memory 0; cpu/TScatter.hpp:21-44): out [64,128] is read, out[idx[i,j], j] = src[i,j] for the source's valid
+ * region [valid_rows, valid_cols] (several rows to one place: the last row wins; rows outside 0..63 are dropped), the rest
+ * of out keeps its values.  MSCATTER (to_memory != 0; cpu/MGatherScatter.hpp:46-69): out[idx[i,j]] = src[i,j] with out as
+ * plain memory of 64 x 128 elements; THE CALLER guarantees 0 <= idx < 8192 there (distinct indices for a defined result). */
+int pto_st_scatter_f32_64x128(void *stream, float *out, const float *src, const int32_t *idx, int valid_rows, int valid_cols,
+                              int to_memory);
+/* TCI (pto_instr.hpp:808-814, cpu/TCI.hpp): out [1024] int32 is read, out[j] = start + j (descending: start - j) for
+ * j < valid_cols, the rest keeps its values. */
+int pto_st_tci_s32_1x1024(void *stream, int32_t *out, int32_t start, int descending, int valid_cols);
 /* TSORT32 (pto_instr.hpp:786-798, cpu/TSort32.hpp) on an [8,128] tile of fp32 (dtype 0) or int32 (dtype 1) scores with
  * uint32 indices and the valid region [valid_rows, valid_cols]: out [8,256] is read, every group of 32 valid columns
  * of a row is written back as (score, index bit pattern) structures in descending order of score, equal scores in

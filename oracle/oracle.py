@@ -196,6 +196,34 @@ def topk_f32(src, in_idx, valid_cols, topk):
     return out_s, out_i
 
 
+def tscatter(dst, src, idx, valid_row, valid_col):
+    """TSCATTER (cpu/TScatter.hpp:21-44): dst[idx[i, j], j] = src[i, j] for i < valid_row, j < valid_col in row order
+    (a later row overwrites an earlier one); rows outside dst are dropped (the reference would write out of bounds)."""
+    dst = np.array(dst, copy=True)
+    for i in range(valid_row):
+        rows = idx[i, :valid_col].astype(np.int64)
+        ok = (rows >= 0) & (rows < dst.shape[0])
+        cols = np.arange(valid_col)[ok]
+        dst[rows[ok], cols] = src[i, cols]
+    return dst
+
+
+def mscatter(mem, src, idx, valid_row, valid_col):
+    """MSCATTER (cpu/MGatherScatter.hpp:46-69): mem[idx[i, j]] = src[i, j] in row-major order."""
+    mem = np.array(mem, copy=True).reshape(-1)
+    for i in range(valid_row):
+        mem[idx[i, :valid_col]] = src[i, :valid_col]      # numpy assigns in order: the last of equal indices stays
+    return mem
+
+
+def tci(dst, start, descending, valid_col):
+    """TCI (cpu/TCI.hpp:16-35): dst[j] = start -/+ j for j < valid_col, in the tile's integer type (wrap-around)."""
+    dst = np.array(dst, copy=True).reshape(-1)
+    j = np.arange(valid_col, dtype=np.int64)
+    dst[:valid_col] = ((np.int64(start) - j) if descending else (np.int64(start) + j)).astype(dst.dtype)
+    return dst
+
+
 def tpart(dst, a, b, op, dvalid, avalid, bvalid):
     """TPARTADD (op 0) / TPARTMAX (1) / TPARTMIN (2), cpu/TPartOp.hpp:19-45: over dst's valid region [dvr, dvc]: op(a, b)
     where both sources are inside their valid regions, the element of the one that is where only one is, 0 where none

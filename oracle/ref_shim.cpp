@@ -559,6 +559,40 @@ void ref_tpart_f32_64x128(float *out, const float *a, const float *b, int op, in
         TPARTMIN(*td, *ta, *tb);
     std::memcpy(out, td->data(), sizeof(float) * 64 * 128);
 }
+void ref_tscatter_f32_64x128(float *out, const float *src, const int32_t *idx, int vr, int vc)
+{
+    using Dyn = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, -1, -1>;
+    using DynI = Tile<TileType::Vec, int32_t, 64, 128, BLayout::RowMajor, -1, -1>;
+    auto ts = std::make_unique<Dyn>(vr, vc), td = std::make_unique<Dyn>(vr, vc);
+    auto ti = std::make_unique<DynI>(vr, vc);
+    std::memcpy(ts->data(), src, sizeof(float) * 64 * 128);
+    std::memcpy(ti->data(), idx, sizeof(int32_t) * 64 * 128);
+    std::memcpy(td->data(), out, sizeof(float) * 64 * 128);
+    TSCATTER(*td, *ts, *ti);
+    std::memcpy(out, td->data(), sizeof(float) * 64 * 128);
+}
+void ref_mscatter_f32_64x128(float *out, const float *src, const int32_t *idx, int vr, int vc)
+{
+    using Dyn = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, -1, -1>;
+    using DynI = Tile<TileType::Vec, int32_t, 64, 128, BLayout::RowMajor, -1, -1>;
+    auto ts = std::make_unique<Dyn>(vr, vc);
+    auto ti = std::make_unique<DynI>(vr, vc);
+    std::memcpy(ts->data(), src, sizeof(float) * 64 * 128);
+    std::memcpy(ti->data(), idx, sizeof(int32_t) * 64 * 128);
+    GmND<float, 64, 128> go(out);
+    MSCATTER(go, *ts, *ti);
+}
+void ref_tci_s32_1x1024(int32_t *out, int32_t start, int descending, int vc)
+{
+    using Dyn = Tile<TileType::Vec, int32_t, 1, 1024, BLayout::RowMajor, 1, -1>;
+    auto td = std::make_unique<Dyn>(vc);
+    std::memcpy(td->data(), out, sizeof(int32_t) * 1024);
+    if (descending)
+        TCI<Dyn, int32_t, 1>(*td, start);
+    else
+        TCI<Dyn, int32_t, 0>(*td, start);
+    std::memcpy(out, td->data(), sizeof(int32_t) * 1024);
+}
 void ref_tmrgsort_blocks_f32_1x1024(float *out, const float *src, int valid_cols, int block_len)
 {
     using S = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;

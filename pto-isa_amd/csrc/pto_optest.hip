@@ -1157,6 +1157,74 @@ extern "C" int pto_st_tpart_f32_64x128(void *stream, float *out, const float *a,
     return pto_amd::check_launch();
 }
 
+// ---- TSCATTER on [64, 128] fp32 tiles (valid region of the source at run time), MSCATTER of the same tile into memory,
+// TCI on a [1, 1024] int32 tile ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void ScatterKernel(__gm__ float *out, __gm__ const float *srcIn, __gm__ const int32_t *idxIn,
+                                                                      int vr, int vc, int toMemory)
+{
+    using Full = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor>;
+    using FullI = Tile<TileType::Vec, int32_t, 64, 128, BLayout::RowMajor>;
+    using Dyn = Tile<TileType::Vec, float, 64, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    using DynI = Tile<TileType::Vec, int32_t, 64, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    Full fs, fo;
+    FullI fi;
+    GmND<float, 64, 128> gs(const_cast<float *>(srcIn)), go(out);
+    GmND<int32_t, 64, 128> gi(const_cast<int32_t *>(idxIn));
+    TLOAD(fs, gs);
+    TLOAD(fi, gi);
+    Dyn s(vr, vc), d(vr, vc);
+    DynI x(vr, vc);
+    s.st = fs.st;
+    x.st = fi.st;
+    if (toMemory) {
+        MSCATTER(go, s, x);
+        return;
+    }
+    TLOAD(fo, go);
+    d.st = fo.st;
+    TSCATTER(d, s, x);
+    fo.st = d.st;
+    TSTORE(go, fo);
+}
+
+template <int DESC>
+__global__ __launch_bounds__(kBlockThreads) AICORE void CiKernel(__gm__ int32_t *out, int32_t start, int vc)
+{
+    using Full = Tile<TileType::Vec, int32_t, 1, 1024, BLayout::RowMajor>;
+    using Dyn = Tile<TileType::Vec, int32_t, 1, 1024, BLayout::RowMajor, 1, DYNAMIC>;
+    Full f;
+    GmND<int32_t, 1, 1024> go(out);
+    TLOAD(f, go);
+    Dyn d(vc);
+    d.st = f.st;
+    TCI<Dyn, int32_t, DESC>(d, start);
+    f.st = d.st;
+    TSTORE(go, f);
+}
+
+extern "C" int pto_st_scatter_f32_64x128(void *stream, float *out, const float *src, const int32_t *idx, int valid_rows, int valid_cols,
+                                         int to_memory)
+{
+    PTO_ST_NONNULL(out, src, idx);
+    if (valid_rows < 0 || valid_rows > 64 || valid_cols < 0 || valid_cols > 128)
+        return PTO_ERR_BAD_ARG;
+    ScatterKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, idx, valid_rows, valid_cols, to_memory != 0);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tci_s32_1x1024(void *stream, int32_t *out, int32_t start, int descending, int valid_cols)
+{
+    PTO_ST_NONNULL(out);
+    if (valid_cols < 0 || valid_cols > 1024)
+        return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (descending)
+        CiKernel<1><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, start, valid_cols);
+    else
+        CiKernel<0><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, start, valid_cols);
+    return pto_amd::check_launch();
+}
+
 extern "C" int pto_st_tsort32_8x128(void *stream, void *out, const void *src, const uint32_t *idx, int valid_rows, int valid_cols, int dtype)
 {
     PTO_ST_NONNULL(out, src, idx);

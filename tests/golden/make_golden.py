@@ -113,6 +113,17 @@ def sort_cases(ref):
         a, b, o = sc.part_inputs(n)
         ref.ref_tpart_f32_64x128(p(o), p(a), p(b), op, *dv, *av, *bv)
         out["part_%d" % n] = o[::3].copy()      # every third row keeps the fixture small
+    for n, (vr, vc, kind) in enumerate(sc.SCATTER_CASES):
+        src, idx, o = sc.scatter_inputs(vr, vc, kind, n)
+        ref.ref_tscatter_f32_64x128(p(o), p(src), p(idx), vr, vc)
+        out["tscatter_%d" % n] = o[::3].copy()
+        src, idx, mem = sc.mscatter_inputs(vr, vc, n)
+        ref.ref_mscatter_f32_64x128(p(mem), p(src), p(idx), vr, vc)
+        out["mscatter_%d" % n] = mem[::3].copy()
+    for n, (start, desc, vc) in enumerate(sc.CI_CASES):
+        o = np.full(1024, -5, dtype=np.int32)
+        ref.ref_tci_s32_1x1024(p(o), start, desc, vc)
+        out["tci_%d" % n] = o
     return out
 
 

@@ -73,3 +73,30 @@ def part_inputs(seed):
     a = rng.standard_normal((64, 128)).astype(np.float32)
     b = rng.standard_normal((64, 128)).astype(np.float32)
     return a, b, np.full((64, 128), -999.0, dtype=np.float32)
+
+
+# TSCATTER / MSCATTER / TCI
+SCATTER_CASES = [(64, 128, "perm"), (40, 100, "perm"), (64, 128, "collide"), (17, 5, "collide")]
+
+
+def scatter_inputs(vr, vc, kind, seed):
+    """src [64,128] fp32, idx [64,128] int32 (row numbers: a permutation of the rows per column, or random rows so that
+    several source rows send an element to the same place), out0 [64,128]."""
+    rng = np.random.default_rng(900 + seed)
+    src = rng.standard_normal((64, 128)).astype(np.float32)
+    if kind == "perm":
+        idx = np.stack([rng.permutation(64) for _ in range(128)], axis=1).astype(np.int32)
+    else:
+        idx = rng.integers(0, 64, size=(64, 128)).astype(np.int32)
+    return src, idx, np.full((64, 128), -321.0, dtype=np.float32)
+
+
+def mscatter_inputs(vr, vc, seed):
+    """distinct memory positions in [0, 8192) for every element"""
+    rng = np.random.default_rng(950 + seed)
+    src = rng.standard_normal((64, 128)).astype(np.float32)
+    idx = rng.permutation(8192).astype(np.int32).reshape(64, 128)
+    return src, idx, np.full(8192, -321.0, dtype=np.float32)
+
+
+CI_CASES = [(0, 0, 1024), (1000, 1, 777), (2**31 - 5, 0, 20), (-7, 1, 1)]

@@ -84,6 +84,38 @@ def test_tpart(oracle, n):
     assert np.array_equal(got[::3].view(np.uint32), GOLD["part_%d" % n].view(np.uint32))
 
 
+@pytest.mark.parametrize("n", range(len(sc.SCATTER_CASES)))
+def test_tscatter_and_mscatter(oracle, n):
+    lib = capi.load()
+    vr, vc, kind = sc.SCATTER_CASES[n]
+    src, idx, out0 = sc.scatter_inputs(vr, vc, kind, n)
+    ts, ti, to = _dev(src), _dev(idx), _dev(out0)
+    capi.check(lib.pto_st_scatter_f32_64x128(_st(), to.data_ptr(), ts.data_ptr(), ti.data_ptr(), vr, vc, 0), "tscatter")
+    torch.cuda.synchronize()
+    got = to.cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), oracle.tscatter(out0, src, idx, vr, vc).view(np.uint32))      # incl. "last row wins"
+    assert np.array_equal(got[::3].view(np.uint32), GOLD["tscatter_%d" % n].view(np.uint32))
+    msrc, midx, mem0 = sc.mscatter_inputs(vr, vc, n)
+    ts, ti, tm = _dev(msrc), _dev(midx), _dev(mem0)
+    capi.check(lib.pto_st_scatter_f32_64x128(_st(), tm.data_ptr(), ts.data_ptr(), ti.data_ptr(), vr, vc, 1), "mscatter")
+    torch.cuda.synchronize()
+    mgot = tm.cpu().numpy()
+    assert np.array_equal(mgot.view(np.uint32), oracle.mscatter(mem0, msrc, midx, vr, vc).view(np.uint32))
+    assert np.array_equal(mgot[::3].view(np.uint32), GOLD["mscatter_%d" % n].view(np.uint32))
+
+
+@pytest.mark.parametrize("n", range(len(sc.CI_CASES)))
+def test_tci(oracle, n):
+    lib = capi.load()
+    start, desc, vc = sc.CI_CASES[n]
+    out0 = np.full(1024, -5, dtype=np.int32)
+    to = _dev(out0)
+    capi.check(lib.pto_st_tci_s32_1x1024(_st(), to.data_ptr(), start, desc, vc), "tci")
+    torch.cuda.synchronize()
+    got = to.cpu().numpy()
+    assert np.array_equal(got, oracle.tci(out0, start, desc, vc)) and np.array_equal(got, GOLD["tci_%d" % n])
+
+
 def test_sort_programs_reject_bad_arguments():
     lib = capi.load()
     p = torch.zeros(2048, device="cuda:0").data_ptr()

@@ -107,3 +107,39 @@ def test_tpart_vs_reference(oracle, n):
     none[:av[0], :av[1]] = False
     none[:bv[0], :bv[1]] = False
     assert np.all(got[none] == 0)                                                          # neither source valid
+
+
+@pytest.mark.parametrize("n", range(len(sc.SCATTER_CASES)))
+def test_scatter_vs_reference(oracle, n):
+    """TSCATTER / MSCATTER against the reference's CPU simulation (committed outputs, every third element row / word;
+    everything where the compiled reference is built), and as the inverse of a gather where the indices are a permutation."""
+    vr, vc, kind = sc.SCATTER_CASES[n]
+    src, idx, out0 = sc.scatter_inputs(vr, vc, kind, n)
+    got = oracle.tscatter(out0, src, idx, vr, vc)
+    assert np.array_equal(got[::3].view(np.uint32), GOLD["tscatter_%d" % n].view(np.uint32))
+    msrc, midx, mem0 = sc.mscatter_inputs(vr, vc, n)
+    mgot = oracle.mscatter(mem0, msrc, midx, vr, vc)
+    assert np.array_equal(mgot[::3].view(np.uint32), GOLD["mscatter_%d" % n].view(np.uint32))
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        r.ref_tscatter_f32_64x128(_p(o), _p(src), _p(idx), vr, vc)
+        assert np.array_equal(o.view(np.uint32), got.view(np.uint32))
+        m = mem0.copy()
+        r.ref_mscatter_f32_64x128(_p(m), _p(msrc), _p(midx), vr, vc)
+        assert np.array_equal(m.view(np.uint32), mgot.view(np.uint32))
+    if kind == "perm" and vr == 64:          # a gather with the same indices undoes the scatter
+        assert np.array_equal(np.take_along_axis(got[:, :vc], idx[:, :vc].astype(np.int64), axis=0), src[:, :vc])
+    assert np.array_equal(mgot[midx[:vr, :vc]], msrc[:vr, :vc])
+    touched = np.zeros(8192, dtype=bool)
+    touched[midx[:vr, :vc].ravel()] = True
+    assert np.all(mgot[~touched] == mem0[~touched])
+
+
+@pytest.mark.parametrize("n", range(len(sc.CI_CASES)))
+def test_tci_vs_reference(oracle, n):
+    start, desc, vc = sc.CI_CASES[n]
+    got = oracle.tci(np.full(1024, -5, dtype=np.int32), start, desc, vc)
+    assert np.array_equal(got, GOLD["tci_%d" % n])
+    want = (np.int64(start) + (-1 if desc else 1) * np.arange(vc, dtype=np.int64)).astype(np.int32)    # closed form, wraps
+    assert np.array_equal(got[:vc], want) and np.all(got[vc:] == -5)
