@@ -97,6 +97,7 @@ PTO_FRONT(TCOLEXPANDDIV, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C
 PTO_FRONT(TCOLEXPANDADD, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
 PTO_FRONT(TCOLEXPANDMAX, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
 PTO_FRONT(TCOLEXPANDMIN, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TCOLEXPANDEXPDIF, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
 PTO_FRONT(TABS, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TNEG, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TRELU, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))

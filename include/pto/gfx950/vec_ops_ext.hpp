@@ -267,7 +267,7 @@ PTO_DEV void col_reduce(DstT &dst, SrcT &src)
     hw::lds_barrier();
 }
 
-enum class ColOp { Copy, Sub, Mul, Div, Add, Max, Min };
+enum class ColOp { Copy, Sub, Mul, Div, Add, Max, Min, ExpDif };
 // dst[i,j] = src0[i,j] <op> src1[0,j]  (TColExpand.hpp:22-33, TColExpandOp.hpp)
 template <ColOp op, typename DstT, typename ColT>
 PTO_DEV void col_expand(DstT &dst, DstT &src0, ColT &src1)
@@ -298,6 +298,8 @@ PTO_DEV void col_expand(DstT &dst, DstT &src0, ColT &src1)
                 o = a + b;
             else if constexpr (op == ColOp::Max)
                 o = a < b ? b : a;
+            else if constexpr (op == ColOp::ExpDif)
+                o = (T)::exp((double)(T)(a - b)); // ElementOp.h:265-270, as TROWEXPANDEXPDIF
             else
                 o = b < a ? b : a;
             dst.st.v[s][i] = o;
@@ -330,6 +332,7 @@ PTO_DEFINE_COLEXPAND(TCOLEXPANDDIV, Div)
 PTO_DEFINE_COLEXPAND(TCOLEXPANDADD, Add)
 PTO_DEFINE_COLEXPAND(TCOLEXPANDMAX, Max)
 PTO_DEFINE_COLEXPAND(TCOLEXPANDMIN, Min)
+PTO_DEFINE_COLEXPAND(TCOLEXPANDEXPDIF, ExpDif) // TColExpandOp.hpp:75-79
 #undef PTO_DEFINE_COLEXPAND
 
 // ------------------------------------------------ more row reductions / broadcasts

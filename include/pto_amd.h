@@ -183,7 +183,7 @@ enum {
     PTO_VOP_ROWEXPAND = 60, PTO_VOP_ROWEXPANDSUB, PTO_VOP_ROWEXPANDMUL, PTO_VOP_ROWEXPANDDIV, PTO_VOP_ROWEXPANDADD,
     PTO_VOP_ROWEXPANDMAX, PTO_VOP_ROWEXPANDMIN, PTO_VOP_ROWEXPANDEXPDIF,
     PTO_VOP_COLEXPAND = 80, PTO_VOP_COLEXPANDSUB, PTO_VOP_COLEXPANDMUL, PTO_VOP_COLEXPANDDIV, PTO_VOP_COLEXPANDADD,
-    PTO_VOP_COLEXPANDMAX, PTO_VOP_COLEXPANDMIN
+    PTO_VOP_COLEXPANDMAX, PTO_VOP_COLEXPANDMIN, PTO_VOP_COLEXPANDEXPDIF
 };
 int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a, const float *b, const float *vec, float scalar, int op);
 /* The arithmetic subset of the same (ABS NEG RELU, ADD SUB MUL MAX MIN, ADDS SUBS MULS MAXS MINS, the row / column

@@ -456,7 +456,7 @@ VOP = dict(ABS=0, NEG=1, RELU=2, SQRT=3, RSQRT=4, LOG=5, RECIP=6, EXP=7,
            CMP_GE=32, SELS=33, ADDS=40, SUBS=41, MULS=42, DIVS=43, MAXS=44, MINS=45, LRELU=46,
            ROWEXPAND=60, ROWEXPANDSUB=61, ROWEXPANDMUL=62, ROWEXPANDDIV=63, ROWEXPANDADD=64, ROWEXPANDMAX=65, ROWEXPANDMIN=66,
            ROWEXPANDEXPDIF=67, COLEXPAND=80, COLEXPANDSUB=81, COLEXPANDMUL=82, COLEXPANDDIV=83, COLEXPANDADD=84,
-           COLEXPANDMAX=85, COLEXPANDMIN=86)
+           COLEXPANDMAX=85, COLEXPANDMIN=86, COLEXPANDEXPDIF=87)
 
 
 def vec_op(op, a, b=None, vec=None, scalar=0.0):

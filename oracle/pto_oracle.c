@@ -979,6 +979,7 @@ void po_vec_op(float *dst, const float *a, const float *b, const float *vec, flo
             case 84: o = v + cv; break;
             case 85: o = v < cv ? cv : v; break;
             case 86: o = cv < v ? cv : v; break;
+            case 87: o = (float)exp((double)(v - cv)); break;           /* TColExpandOp.hpp:75-79 */
             default: o = 0.0f; break;
             }
             dst[x] = o;

@@ -371,6 +371,7 @@ void vec_op_64x128(float *out, const float *a, const float *b, const float *vec,
     case 84: TCOLEXPANDADD(*to, *ta, *cv); break;
     case 85: TCOLEXPANDMAX(*to, *ta, *cv); break;
     case 86: TCOLEXPANDMIN(*to, *ta, *cv); break;
+    case 87: TCOLEXPANDEXPDIF(*to, *ta, *cv); break;
     default: return;
     }
     TSTORE(go, *to);

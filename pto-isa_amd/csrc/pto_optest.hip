@@ -384,7 +384,7 @@ enum VecOp : int {
     kAdd = 20, kSub, kMul, kDiv, kMax, kMin, kPrelu, kCmpEq, kCmpNe, kCmpLt, kCmpLe, kCmpGt, kCmpGe, kSels,
     kAdds = 40, kSubs, kMuls, kDivs, kMaxs, kMins, kLrelu,
     kRowExpand = 60, kRowSub, kRowMul, kRowDiv, kRowAdd, kRowMax, kRowMin, kRowExpDif,
-    kColExpand = 80, kColSub, kColMul, kColDiv, kColAdd, kColMax, kColMin,
+    kColExpand = 80, kColSub, kColMul, kColDiv, kColAdd, kColMax, kColMin, kColExpDif,
 };
 __global__ __launch_bounds__(kBlockThreads) AICORE void VecOpKernel(__gm__ float *out, __gm__ const float *aIn, __gm__ const float *bIn,
                                                                     __gm__ const float *vecIn, float k, int op)
@@ -452,6 +452,7 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void VecOpKernel(__gm__ float
     case kColAdd: TCOLEXPANDADD(o, a, cv); break;
     case kColMax: TCOLEXPANDMAX(o, a, cv); break;
     case kColMin: TCOLEXPANDMIN(o, a, cv); break;
+    case kColExpDif: TCOLEXPANDEXPDIF(o, a, cv); break;
     default: TMULS(o, a, 0.0f); break;
     }
     TSTORE(go, o);
@@ -937,7 +938,7 @@ extern "C" int pto_st_vec_op_f32_64x128(void *stream, float *out, const float *a
 {
     PTO_ST_NONNULL(out, a);
     const bool known = (op >= kAbs && op <= kExp) || (op >= kAdd && op <= kSels) || (op >= kAdds && op <= kLrelu) ||
-                       (op >= kRowExpand && op <= kRowExpDif) || (op >= kColExpand && op <= kColMin);
+                       (op >= kRowExpand && op <= kRowExpDif) || (op >= kColExpand && op <= kColExpDif);
     if (!known)
         return PTO_ERR_BAD_ARG;
     if (op >= kAdd && op <= kSels)

@@ -5,7 +5,7 @@ UNARY = ["ABS", "NEG", "RELU", "SQRT", "RSQRT", "LOG", "RECIP", "EXP"]
 BINARY = ["ADD", "SUB", "MUL", "DIV", "MAX", "MIN", "PRELU", "CMP_EQ", "CMP_NE", "CMP_LT", "CMP_LE", "CMP_GT", "CMP_GE", "SELS"]
 SCALAR = ["ADDS", "SUBS", "MULS", "DIVS", "MAXS", "MINS", "LRELU"]
 ROWOPS = ["ROWEXPAND", "ROWEXPANDSUB", "ROWEXPANDMUL", "ROWEXPANDDIV", "ROWEXPANDADD", "ROWEXPANDMAX", "ROWEXPANDMIN", "ROWEXPANDEXPDIF"]
-COLOPS = ["COLEXPAND", "COLEXPANDSUB", "COLEXPANDMUL", "COLEXPANDDIV", "COLEXPANDADD", "COLEXPANDMAX", "COLEXPANDMIN"]
+COLOPS = ["COLEXPAND", "COLEXPANDSUB", "COLEXPANDMUL", "COLEXPANDDIV", "COLEXPANDADD", "COLEXPANDMAX", "COLEXPANDMIN", "COLEXPANDEXPDIF"]
 ALL_OPS = UNARY + BINARY + SCALAR + ROWOPS + COLOPS
 POSITIVE = {"SQRT", "RSQRT", "LOG"}          # defined for positive inputs only
 NONZERO_B = {"DIV", "DIVS", "ROWEXPANDDIV", "COLEXPANDDIV", "RECIP"}
@@ -20,7 +20,7 @@ def vec_inputs(op, seed=0):
         a = (np.abs(a) + np.float32(0.01)).astype(np.float32)
     if op == "RECIP":
         a = np.where(np.abs(a) < 0.05, np.float32(0.5), a).astype(np.float32)
-    if op == "EXP" or op == "ROWEXPANDEXPDIF":
+    if op in ("EXP", "ROWEXPANDEXPDIF", "COLEXPANDEXPDIF"):
         a = (a * np.float32(2.0)).astype(np.float32)
     if op.startswith("CMP"):        # plenty of equal pairs
         eq = rng.random((64, 128)) < 0.3
@@ -59,7 +59,7 @@ def numpy_vec_op(op, a, b, vec, k):
             "ROWEXPANDMIN": lambda: np.minimum(a, r), "ROWEXPANDEXPDIF": lambda: np.exp((a - r).astype(f64)),
             "COLEXPAND": lambda: np.broadcast_to(c, a.shape), "COLEXPANDSUB": lambda: a - c, "COLEXPANDMUL": lambda: a * c,
             "COLEXPANDDIV": lambda: a / c, "COLEXPANDADD": lambda: a + c, "COLEXPANDMAX": lambda: np.maximum(a, c),
-            "COLEXPANDMIN": lambda: np.minimum(a, c),
+            "COLEXPANDMIN": lambda: np.minimum(a, c), "COLEXPANDEXPDIF": lambda: np.exp((a - c).astype(f64)),
         }
         return np.asarray(table[op]()).astype(f32)
 
