@@ -114,6 +114,7 @@ PTO_FRONT(TSHL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a 
 PTO_FRONT(TSHR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TREM, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TNOT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TGATHERB, typename D PTO_C typename S PTO_C typename O, D &dst PTO_C S &src PTO_C O &offset, (dst, src, offset))
 PTO_FRONT(TSCATTER, typename D PTO_C typename I, D &dst PTO_C D &src PTO_C I &indexes, (dst, src, indexes))
 PTO_FRONT(MSCATTER, typename G PTO_C typename S PTO_C typename I, G &dst PTO_C S &src PTO_C I &indexes, (dst, src, indexes))
 PTO_FRONT(TPARTADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))

@@ -396,6 +396,16 @@ PTO_DEV char *stage_buffer()
     __shared__ __attribute__((aligned(16))) char buf[Bytes];
     return buf;
 }
+// a Vec tile's elements as 32-bit words in row-major order
+template <typename TileT>
+PTO_DEV void stage_tile_rows_raw(TileT &t, uint32_t *lds)
+{
+    static_assert(sizeof(typename TileT::DType) == 4 && TileT::isRowMajor, "4-byte elements, row-major");
+    for_each_owned<TileT>([&](int s, int i, int e) {
+        if (e < TileT::Numel)
+            lds[e] = __builtin_bit_cast(uint32_t, t.st.v[s][i]);
+    });
+}
 } // namespace detail
 
 // ------------------------------------------------------- TMOV Acc -> Vec
@@ -744,6 +754,46 @@ PTO_DEV void MSCATTER_IMPL(G &dst, SrcT &src, IdxT &indexes)
         if (e < SrcT::Numel && r < vr && c < vc)
             gm[(size_t)indexes.st.v[s][i]] = src.st.v[s][i];
     });
+}
+
+// ---------------------------------------------------------------------- TGATHERB
+// Block gather (cpu/TGatherB.hpp:21-60): for every row r and every 32-byte block c of the destination's valid region,
+// dst block (r, c) = the 32 bytes of the source tile's storage that start at byte offset[r, c]; blocks whose source range
+// does not lie inside the source tile are left as they are.  4-byte elements: a block is one 8-element chunk of a lane.
+template <typename DstT, typename SrcT, typename OffT>
+PTO_DEV void TGATHERB_IMPL(DstT &dst, SrcT &src, OffT &offset)
+{
+    using T = typename DstT::DType;
+    static_assert(DstT::Loc == TileType::Vec && SrcT::Loc == TileType::Vec && OffT::Loc == TileType::Vec && DstT::isRowMajor && SrcT::isRowMajor &&
+                      OffT::isRowMajor,
+                  "[PTO][SA] TGATHERB: row-major Vec tiles");
+    static_assert(sizeof(T) == 4 && sizeof(typename SrcT::DType) == 4 && sizeof(typename OffT::DType) == 4 && DstT::Cols % detail::kVecChunk == 0 &&
+                      OffT::Rows == DstT::Rows,
+                  "[PTO][SA] TGATHERB: 4-byte elements, 32-bit offsets, one offset row per destination row");
+    constexpr int kSrcBytes = SrcT::Numel * 4, kOffs = OffT::Numel;
+    char *bytes = detail::stage_buffer<detail::stage_bytes(kSrcBytes + 4 * kOffs)>();
+    uint32_t *offs = reinterpret_cast<uint32_t *>(bytes + kSrcBytes);
+    detail::stage_tile_rows_raw(src, reinterpret_cast<uint32_t *>(bytes));
+    detail::stage_tile_rows_raw(offset, offs);
+    hw::lds_barrier();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    using S = typename DstT::Storage;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid(), e0 = q * detail::kVecChunk;
+        const int r = e0 / DstT::Cols, c = (e0 % DstT::Cols) / detail::kVecChunk;
+        if (e0 < DstT::Numel && r < vr && (c + 1) * detail::kVecChunk <= vc && c < OffT::Cols) {
+            const uint32_t off = offs[r * OffT::Cols + c];
+            if (off <= (uint32_t)kSrcBytes - 32u) {
+                T v[detail::kVecChunk];
+                __builtin_memcpy(v, bytes + off, 32); // any byte alignment
+#pragma unroll
+                for (int i = 0; i < detail::kVecChunk; ++i)
+                    dst.st.v[s][i] = v[i];
+            }
+        }
+    }
+    hw::lds_barrier();
 }
 
 } // namespace pto

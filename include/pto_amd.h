@@ -222,6 +222,11 @@ int pto_st_tpart_f32_64x128(void *stream, float *out, const float *a, const floa
  * plain memory of 64 x 128 elements; THE CALLER guarantees 0 <= idx < 8192 there (distinct indices for a defined result). */
 int pto_st_scatter_f32_64x128(void *stream, float *out, const float *src, const int32_t *idx, int valid_rows, int valid_cols,
                               int to_memory);
+/* TGATHERB (pto_instr.hpp:1152-1158, cpu/TGatherB.hpp:21-60): out [16,128] fp32 is read; every 32-byte block (r, c) of its
+ * valid region [valid_rows, valid_cols] (valid_cols % 8 == 0) becomes the 32 bytes of the [32,64] fp32 source tile's
+ * row-major storage that start at byte offsets[r, c] ([16,16] uint32, any alignment); a block whose source range leaves
+ * the 8192 bytes of the tile keeps its values. */
+int pto_st_tgatherb_f32_16x128(void *stream, float *out, const float *src, const uint32_t *offsets, int valid_rows, int valid_cols);
 /* TCI (pto_instr.hpp:808-814, cpu/TCI.hpp): out [1024] int32 is read, out[j] = start + j (descending: start - j) for
  * j < valid_cols, the rest keeps its values. */
 int pto_st_tci_s32_1x1024(void *stream, int32_t *out, int32_t start, int descending, int valid_cols);

@@ -196,6 +196,21 @@ def topk_f32(src, in_idx, valid_cols, topk):
     return out_s, out_i
 
 
+def tgatherb(dst, src, offsets, valid_row, valid_col):
+    """TGATHERB (cpu/TGatherB.hpp:21-60): block (r, c) of 32 bytes of dst's valid region = the 32 bytes of src's
+    row-major storage from byte offsets[r, c]; source ranges that leave the tile are skipped."""
+    dst = np.array(dst, copy=True)
+    raw = np.ascontiguousarray(src).view(np.uint8).reshape(-1)
+    per = 32 // dst.itemsize
+    out = dst.view(np.uint8).reshape(dst.shape[0], -1)
+    for r in range(valid_row):
+        for c in range(valid_col // per):
+            off = int(offsets[r, c])
+            if off + 32 <= raw.size:
+                out[r, 32 * c:32 * c + 32] = raw[off:off + 32]
+    return dst
+
+
 def tscatter(dst, src, idx, valid_row, valid_col):
     """TSCATTER (cpu/TScatter.hpp:21-44): dst[idx[i, j], j] = src[i, j] for i < valid_row, j < valid_col in row order
     (a later row overwrites an earlier one); rows outside dst are dropped (the reference would write out of bounds)."""

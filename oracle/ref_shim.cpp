@@ -583,6 +583,18 @@ void ref_mscatter_f32_64x128(float *out, const float *src, const int32_t *idx, i
     GmND<float, 64, 128> go(out);
     MSCATTER(go, *ts, *ti);
 }
+void ref_tgatherb_f32_16x128(float *out, const float *src, const uint32_t *offsets, int vr, int vc)
+{
+    using D = Tile<TileType::Vec, float, 16, 128, BLayout::RowMajor, -1, -1>;
+    auto td = std::make_unique<D>(vr, vc);
+    auto ts = std::make_unique<Tile<TileType::Vec, float, 32, 64, BLayout::RowMajor>>();
+    auto to = std::make_unique<Tile<TileType::Vec, uint32_t, 16, 16, BLayout::RowMajor>>();
+    std::memcpy(td->data(), out, sizeof(float) * 16 * 128);
+    std::memcpy(ts->data(), src, sizeof(float) * 32 * 64);
+    std::memcpy(to->data(), offsets, sizeof(uint32_t) * 16 * 16);
+    TGATHERB(*td, *ts, *to);
+    std::memcpy(out, td->data(), sizeof(float) * 16 * 128);
+}
 void ref_tci_s32_1x1024(int32_t *out, int32_t start, int descending, int vc)
 {
     using Dyn = Tile<TileType::Vec, int32_t, 1, 1024, BLayout::RowMajor, 1, -1>;

@@ -1188,6 +1188,28 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void ScatterKernel(__gm__ flo
     TSTORE(go, fo);
 }
 
+// ---- TGATHERB: dst [16, 128] fp32 (run-time valid region) from a [32, 64] source tile with [16, 16] byte offsets ----
+__global__ __launch_bounds__(kBlockThreads) AICORE void GatherBKernel(__gm__ float *out, __gm__ const float *srcIn, __gm__ const uint32_t *offIn,
+                                                                      int vr, int vc)
+{
+    using Full = Tile<TileType::Vec, float, 16, 128, BLayout::RowMajor>;
+    using Dyn = Tile<TileType::Vec, float, 16, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
+    Full f;
+    Tile<TileType::Vec, float, 32, 64, BLayout::RowMajor> s;
+    Tile<TileType::Vec, uint32_t, 16, 16, BLayout::RowMajor> o;
+    GmND<float, 16, 128> go(out);
+    GmND<float, 32, 64> gs(const_cast<float *>(srcIn));
+    GmND<uint32_t, 16, 16> gof(const_cast<uint32_t *>(offIn));
+    TLOAD(f, go);
+    TLOAD(s, gs);
+    TLOAD(o, gof);
+    Dyn d(vr, vc);
+    d.st = f.st;
+    TGATHERB(d, s, o);
+    f.st = d.st;
+    TSTORE(go, f);
+}
+
 template <int DESC>
 __global__ __launch_bounds__(kBlockThreads) AICORE void CiKernel(__gm__ int32_t *out, int32_t start, int vc)
 {
@@ -1210,6 +1232,15 @@ extern "C" int pto_st_scatter_f32_64x128(void *stream, float *out, const float *
     if (valid_rows < 0 || valid_rows > 64 || valid_cols < 0 || valid_cols > 128)
         return PTO_ERR_BAD_ARG;
     ScatterKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, idx, valid_rows, valid_cols, to_memory != 0);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_tgatherb_f32_16x128(void *stream, float *out, const float *src, const uint32_t *offsets, int valid_rows, int valid_cols)
+{
+    PTO_ST_NONNULL(out, src, offsets);
+    if (valid_rows < 0 || valid_rows > 16 || valid_cols < 0 || valid_cols > 128 || valid_cols % 8)
+        return PTO_ERR_BAD_ARG;
+    GatherBKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, offsets, valid_rows, valid_cols);
     return pto_amd::check_launch();
 }
 

@@ -44,6 +44,7 @@ SYMBOLS = {
     "pto_st_matmul_vec_operands_f16_64x64x128": (C.c_int, [C.c_void_p] * 5),
     "pto_st_tpart_f32_64x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int] * 7),
     "pto_st_scatter_f32_64x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int] * 3),
+    "pto_st_tgatherb_f32_16x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int] * 2),
     "pto_st_tci_s32_1x1024": (C.c_int, [C.c_void_p] * 2 + [C.c_int] * 3),
     "pto_st_tsort32_8x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int] * 3),
     "pto_st_tmrgsort_blocks_f32_1x1024": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 2),

@@ -120,6 +120,10 @@ def sort_cases(ref):
         src, idx, mem = sc.mscatter_inputs(vr, vc, n)
         ref.ref_mscatter_f32_64x128(p(mem), p(src), p(idx), vr, vc)
         out["mscatter_%d" % n] = mem[::3].copy()
+    for n, (vr, vc, kind) in enumerate(sc.GATHERB_CASES):
+        src, off, o = sc.gatherb_inputs(kind, n)
+        ref.ref_tgatherb_f32_16x128(p(o), p(src), p(off), vr, vc)
+        out["gatherb_%d" % n] = o
     for n, (start, desc, vc) in enumerate(sc.CI_CASES):
         o = np.full(1024, -5, dtype=np.int32)
         ref.ref_tci_s32_1x1024(p(o), start, desc, vc)

@@ -100,3 +100,21 @@ def mscatter_inputs(vr, vc, seed):
 
 
 CI_CASES = [(0, 0, 1024), (1000, 1, 777), (2**31 - 5, 0, 20), (-7, 1, 1)]
+
+
+GATHERB_CASES = [(16, 128, "aligned"), (16, 128, "any"), (9, 72, "any"), (16, 128, "edge")]
+
+
+def gatherb_inputs(kind, seed):
+    """src [32,64] fp32 (8192 bytes), offsets [16,16] uint32: block starts (multiples of 32), any byte offsets, or
+    offsets around the end of the tile (some source ranges leave it)."""
+    rng = np.random.default_rng(990 + seed)
+    src = rng.standard_normal((32, 64)).astype(np.float32)
+    if kind == "aligned":
+        off = (rng.integers(0, 256, size=(16, 16)) * 32).astype(np.uint32)
+    elif kind == "any":
+        off = rng.integers(0, 8192 - 32 + 1, size=(16, 16)).astype(np.uint32)
+    else:
+        off = rng.integers(8192 - 64, 8192 + 40, size=(16, 16)).astype(np.uint32)
+        off[0, :2] = [8192 - 32, 8192 - 31]      # (offsets near 2^32 make the reference's own range check wrap around)
+    return src, off, np.full((16, 128), -42.0, dtype=np.float32)

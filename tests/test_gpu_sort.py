@@ -104,6 +104,19 @@ def test_tscatter_and_mscatter(oracle, n):
     assert np.array_equal(mgot[::3].view(np.uint32), GOLD["mscatter_%d" % n].view(np.uint32))
 
 
+@pytest.mark.parametrize("n", range(len(sc.GATHERB_CASES)))
+def test_tgatherb(oracle, n):
+    lib = capi.load()
+    vr, vc, kind = sc.GATHERB_CASES[n]
+    src, off, out0 = sc.gatherb_inputs(kind, n)
+    ts, tf, to = _dev(src), _dev(off), _dev(out0)
+    capi.check(lib.pto_st_tgatherb_f32_16x128(_st(), to.data_ptr(), ts.data_ptr(), tf.data_ptr(), vr, vc), "tgatherb")
+    torch.cuda.synchronize()
+    got = to.cpu().numpy().view(np.uint32)
+    assert np.array_equal(got, oracle.tgatherb(out0, src, off, vr, vc).view(np.uint32))
+    assert np.array_equal(got, GOLD["gatherb_%d" % n].view(np.uint32))
+
+
 @pytest.mark.parametrize("n", range(len(sc.CI_CASES)))
 def test_tci(oracle, n):
     lib = capi.load()

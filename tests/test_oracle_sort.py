@@ -143,3 +143,20 @@ def test_tci_vs_reference(oracle, n):
     assert np.array_equal(got, GOLD["tci_%d" % n])
     want = (np.int64(start) + (-1 if desc else 1) * np.arange(vc, dtype=np.int64)).astype(np.int32)    # closed form, wraps
     assert np.array_equal(got[:vc], want) and np.all(got[vc:] == -5)
+
+
+@pytest.mark.parametrize("n", range(len(sc.GATHERB_CASES)))
+def test_tgatherb_vs_reference(oracle, n):
+    vr, vc, kind = sc.GATHERB_CASES[n]
+    src, off, out0 = sc.gatherb_inputs(kind, n)
+    got = oracle.tgatherb(out0, src, off, vr, vc)
+    assert np.array_equal(got.view(np.uint32), GOLD["gatherb_%d" % n].view(np.uint32))
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        r.ref_tgatherb_f32_16x128(_p(o), _p(src), _p(off), vr, vc)
+        assert np.array_equal(o.view(np.uint32), got.view(np.uint32))
+    if kind == "aligned":        # aligned block starts: a plain gather of 8-element blocks
+        blocks = src.reshape(-1, 8)
+        assert np.array_equal(got[:vr, :vc].reshape(vr, vc // 8, 8), blocks[(off[:vr, :vc // 8] // 32).astype(np.int64)])
+    assert np.array_equal(got[vr:], out0[vr:]) and np.array_equal(got[:, vc:], out0[:, vc:])
