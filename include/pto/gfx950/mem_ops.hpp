@@ -207,6 +207,8 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
 }
 
 // GM -> Vec register tile.  Chunk q of 8 consecutive elements (in the tile's BLayout order).
+// PTO_VEC_STREAM_NT (per translation unit): bit 0 = non-temporal 16-byte loads, bit 1 = non-temporal 16-byte stores of Vec
+// tiles, for kernels that stream data they do not touch again.
 template <typename TileT, typename G>
 PTO_DEV void tload_vec(TileT &dst, G &src)
 {
@@ -241,7 +243,11 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
             // 8 contiguous elements: one or two 16-byte loads
             // element-aligned only: rows of a strided view need not start on a 16-byte boundary
             typedef T VT __attribute__((ext_vector_type(kVecChunk), aligned(sizeof(T))));
+#if defined(PTO_VEC_STREAM_NT) && (PTO_VEC_STREAM_NT & 1)
+            VT v = __builtin_nontemporal_load(reinterpret_cast<const VT *>(gm + base + minor0));
+#else
             VT v = *reinterpret_cast<const VT *>(gm + base + minor0);
+#endif
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
                 dst.st.v[s][i] = v[i];
@@ -621,7 +627,11 @@ PTO_DEV void tstore_vec(G &dst, TileT &src)
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
                 v[i] = src.st.v[s][i];
+#if defined(PTO_VEC_STREAM_NT) && (PTO_VEC_STREAM_NT & 2)
+            __builtin_nontemporal_store(v, reinterpret_cast<VT *>(gm + base + minor0));
+#else
             *reinterpret_cast<VT *>(gm + base + minor0) = v;
+#endif
         } else {
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i) {
