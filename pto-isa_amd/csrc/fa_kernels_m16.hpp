@@ -22,7 +22,6 @@ constexpr float kMaskValue16 = -3.40282e+38f; // pto_macro_fa_softmax.hpp:67
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 // A lane holds one query column of a 16 x 16 block and four of its 16 key rows; the other twelve are in the lanes
 // 16, 32 and 48 positions away.  Both swaps leave in (a, b) the values of the two partners in both places.

@@ -278,13 +278,6 @@ AICORE inline __attribute__((always_inline)) void MixTileRows(__gm__ float *out,
                                                               int n, int k, int row0, int col0, int kLoop)
 {
     constexpr int BK = 32, HM = BM / 2;
-#ifdef PTO_GEMM_ACC_IN_AGPRS
-    // An accumulation-register operand anywhere in the kernel makes the compiler select the MFMA forms whose
-    // accumulators live in the accumulation registers (otherwise, with 512 registers per lane available to a
-    // one-wave-per-SIMD kernel, it keeps accumulators in ordinary registers and uses the accumulation registers as
-    // spill space for the operand fragments).
-    asm volatile("" ::"a"(0));
-#endif
     using TileMatA = Tile<TileType::Mat, half, BM, BK, BLayout::ColMajor, BM, BK, SLayout::RowMajor>;
     using TileMatB = Tile<TileType::Mat, half, BK, BN, BLayout::RowMajor, BK, BN, SLayout::ColMajor>;
     using LeftHalf = TileLeft<half, HM, BK, HM, BK>;
