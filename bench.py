@@ -29,8 +29,8 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 # counter reads for a plain 1 GiB device copy in the same run (--calib-copy): FETCH_SIZE reads
 # 524,300 KiB for 1,048,576 KiB actually read (factor 2.0), WRITE_SIZE reads 1,048,576 KiB for
 # 1,048,576 KiB written (factor 1.0).
-GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 369195.0, 2.0
-GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 151607.0, 1.0
+GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 295155.0, 2.0
+GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 148503.0, 1.0
 
 
 SETTLE_S = 0.0   # set from --settle-ms: the workloads under "extra" keep warming up until this much time has passed
@@ -323,7 +323,7 @@ def main():
         "dtype": "fp16 x fp16 -> fp32 accumulate",
         "data": "synthetic: A [m,k], B [n,k] i.i.d. uniform[-1,1] fp16 from seed 19 / 1019",
         "config": {"workload": "fp16->fp32 GEMM m=n=k=%d, A row-major, B column-major, full K reduction per output tile "
-                               "(256x256 C tile per workgroup, K-step 32)" % args.size},
+                               "(384x192 C tile per workgroup at 6144, K-step 32)" % args.size},
         "extra": extra,
     }
     extra["warmup_policy"] = ("headline: exactly %d untimed launches; workloads under extra: %d launches, then untimed launches "
@@ -336,7 +336,7 @@ def main():
     if gemm:
         line["roofline"] = {"bound": "mfma", "achieved": gemm["tflops"], "peak": PEAK_FP16_TFLOPS, "unit": "TFLOP/s",
                             "frac": gemm["tflops"] / PEAK_FP16_TFLOPS, "traffic": traffic,
-                            "kernel": "GemmF16F32Fine<256,256,4> (4 wavefronts per workgroup)", "flops_per_launch": gemm["flops"],
+                            "kernel": "GemmF16F32Mix<384,192,4,4,rows> (8 wavefronts per workgroup; 512 tiles = two whole rounds)", "flops_per_launch": gemm["flops"],
                             "traffic_unit": "bytes per launch (read + write at the L2 <-> fabric boundary)",
                             "algorithmic_bytes": 2.0 * 2 * args.size ** 2 + 4.0 * args.size ** 2}
     if not args.no_cpu and only in ("", "gemm"):

@@ -33,7 +33,9 @@ inline int allow_lds(K kernel, int bytes)
 // defined in pto_gemm_m16w4.hip (workgroups of four wavefronts, one per SIMD); PTO_ERR_UNSUPPORTED = no tile shape of
 // that kernel fits the problem
 int gemm_f16f32_tile256_w4(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
-// defined in pto_gemm_m16.hip (workgroups of eight wavefronts)
+// defined in pto_gemm_m16.hip (workgroups of eight wavefronts); the 384 x 192 form returns PTO_ERR_UNSUPPORTED unless its
+// tiles fill whole rounds where 256 x 256 tiles do not
+int gemm_f16f32_tile384x192_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
 int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
 // defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries, two groups of four waves in
 // opposite MFMA / softmax phases)

@@ -63,6 +63,9 @@ extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const 
     if (big) {
         // four wavefronts with the K-step written fragment by fragment where that kernel has a tile shape for the
         // problem and is the faster one (uneven rounds, or 192 x 192 tiles for a single round), else eight wavefronts
+        const int rc384 = pto_amd::gemm_f16f32_tile384x192_w8(st, c, ha, hb, m, n, k); // whole rounds of 384 x 192 tiles (6144^2)
+        if (rc384 != PTO_ERR_UNSUPPORTED)
+            return rc384;
         const int rc = pto_amd::gemm_f16f32_tile256_w4(st, c, ha, hb, m, n, k);
         if (rc != PTO_ERR_UNSUPPORTED)
             return rc;

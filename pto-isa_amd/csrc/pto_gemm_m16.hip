@@ -19,6 +19,20 @@ int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _F
         return launch_gemm_mix<256, 192, 4, 4, true>(st, c, a, b, m, n, k, 0);
     return launch_gemm_mix<256, 256, 4, 4, true>(st, c, a, b, m, n, k, 1);
 }
+// 384 x 192 C tiles (the operand traffic per flop of the 256 x 256 tile, 144 accumulator registers per wave, 144 KiB of
+// LDS) for problems that they cut into whole rounds over the compute units while 256 x 256 tiles leave a partial round:
+// 6144 x 6144 = 512 tiles = two rounds on 256 compute units (interleaved runs: 1274 against 1261 TFLOP/s for the four-wave
+// kernel with its quarter-tile round; slower wherever the rounds are not whole).  PTO_ERR_UNSUPPORTED: not such a problem.
+int gemm_f16f32_tile384x192_w8(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k)
+{
+    const int cus = compute_units();
+    if (m % 384 || n % 192 || m % 256 || n % 256)
+        return PTO_ERR_UNSUPPORTED;
+    const long long t384 = (long long)(m / 384) * (n / 192), t256 = (long long)(m / 256) * (n / 256);
+    if (t384 % cus != 0 || t256 % cus == 0)
+        return PTO_ERR_UNSUPPORTED;
+    return launch_gemm_mix<384, 192, 4, 4, true>(st, c, a, b, m, n, k, 0);
+}
 } // namespace pto_amd
 
 extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
@@ -34,6 +48,8 @@ extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_
     case 3: return launch_gemm_mix<256, 256, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
     case 10: return launch_gemm_mix<256, 192, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
     case 11: return launch_gemm_mix<256, 192, 4, 8, true>(st, c, ha, hb, m, n, k, 0);
+    case 12: return launch_gemm_mix<384, 192, 4, 4, true>(st, c, ha, hb, m, n, k, 0);
+    case 14: return launch_gemm_mix<384, 192, 4, 8, true>(st, c, ha, hb, m, n, k, 0);
     default: return PTO_ERR_BAD_ARG;
     }
 }
