@@ -33,7 +33,7 @@ PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T &obj)
 {
     if constexpr (T::Loc == TileType::Mat) {
         static_assert(Addr % 16 == 0, "[PTO][SA] TASSIGN: Mat tiles are 16-byte aligned in LDS");
-        static_assert(Addr + detail::MatGeom<T>::Bytes <= 160 * 1024, "[PTO][SA] TASSIGN: tile exceeds the 160 KiB LDS of a CU");
+        static_assert(Addr + detail::mat_tile_bytes<T>() <= detail::kLdsBytes, "[PTO][SA] TASSIGN: tile exceeds the 160 KiB LDS of a CU");
     }
     TASSIGN_IMPL(obj, Addr);
 }

@@ -13,7 +13,15 @@
 //   Vec              register tile spread over the workgroup in chunks of 8 consecutive elements of
 //                    the tile's linear (BLayout) order: chunk q -> thread q % kBlockThreads, slot q / kBlockThreads.
 //
-// Register tiles are values: pass them by reference.
+// Copies.  A PTO tile object is a handle, and kernel sources written for Ascend pass tiles by value
+// (gemm_performance_kernel.cpp:28 `MatmulAcc(OutTile cTile, ...)`).  A Mat tile copies its LDS offset.  A register
+// tile has no address; copying one is a compile error unless the translation unit defines PTO_TILE_COPY_WRITEBACK
+// before the include.  Then a COPY takes the registers' values and remembers the tile it was copied from, and hands its
+// values back when it goes out of scope: `f(TileAcc c)` updates the caller's accumulator as it does on a machine where
+// the tile is an address.  Limits of that mode: the original must outlive its copies, and while a copy is alive the
+// original and the copy are not views of each other.  After inlining the transfers are register renames.  (The mode is
+// opt-in because a class with a destructor keeps arrays of tiles in memory until late in the optimiser, which costs
+// the tuned kernels a few registers.)
 #pragma once
 #include "pto/common/types.hpp"
 #include "pto/gfx950/platform.hpp"
@@ -31,6 +39,12 @@ typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 namespace detail {
+
+#if defined(PTO_TILE_COPY_WRITEBACK)
+constexpr bool kTileCopyWriteback = true;
+#else
+constexpr bool kTileCopyWriteback = false;
+#endif
 
 static_assert(PTO_MFMA_M == 32 || PTO_MFMA_M == 16, "v_mfma_f32_32x32x16 or v_mfma_f32_16x16x32");
 constexpr int kMfmaM = PTO_MFMA_M;                     // the MFMA's output block is kMfmaM x kMfmaM
@@ -266,8 +280,28 @@ struct Tile {
     Storage st;
     int RowMaskInternal = RowValid_;
     int ColMaskInternal = ColValid_;
+    Tile *origin_ = nullptr; // register tiles: set in a copy, the tile it was copied from (values go back on destruction)
+    static constexpr bool isHandle = Loc_ == TileType::Mat; // the object itself is an address
 
     PTO_HD Tile() {}
+    PTO_HD Tile(const Tile &o) : RowMaskInternal(o.RowMaskInternal), ColMaskInternal(o.ColMaskInternal) { Bind(o); }
+    PTO_HD Tile &operator=(const Tile &o)
+    {
+        RowMaskInternal = o.RowMaskInternal;
+        ColMaskInternal = o.ColMaskInternal;
+        Bind(o);
+        return *this;
+    }
+#if defined(PTO_TILE_COPY_WRITEBACK)
+    PTO_HD ~Tile()
+    {
+        if constexpr (!isHandle)
+            if (origin_)
+                origin_->st = st;
+    }
+#endif
+    PTO_HD Storage &S() { return st; }
+    PTO_HD const Storage &S() const { return st; }
     template <int RM = ValidRow, int CM = ValidCol, std::enable_if_t<RM == DYNAMIC && CM == DYNAMIC, int> = 0>
     PTO_HD Tile(size_t vr, size_t vc) : RowMaskInternal((int)vr), ColMaskInternal((int)vc)
     {}
@@ -289,7 +323,57 @@ struct Tile {
         if constexpr (Loc_ == TileType::Mat)
             return reinterpret_cast<DType *>(hw::lds_base() + st.lds);
         else
-            return &st;
+            return &S();
+    }
+
+    // Element `offset` of the tile's linear storage order (pto_tile.hpp:1254-1266 of the reference; Vec tiles only).
+    // Every lane of the workgroup makes the call with the same arguments.  SetValue: the lane that holds the element
+    // writes it.  GetValue: that lane publishes it through LDS and every lane returns it (two workgroup barriers).
+    PTO_DEV void SetValue(const uint32_t offset, const DType val)
+    {
+        static_assert(Loc_ == TileType::Vec, "[PTO][SA] SetValue / GetValue: Vec tiles");
+        const uint32_t q = offset / detail::kVecChunk, e = offset % detail::kVecChunk;
+        if ((uint32_t)hw::tid() == q % kBlockThreads) {
+            Storage &s = S();
+#pragma unroll
+            for (int slot = 0; slot < Storage::Slots; ++slot)
+#pragma unroll
+                for (int i = 0; i < detail::kVecChunk; ++i)
+                    if ((uint32_t)slot == q / kBlockThreads && (uint32_t)i == e)
+                        s.v[slot][i] = val;
+        }
+    }
+    PTO_DEV DType GetValue(const uint32_t offset)
+    {
+        static_assert(Loc_ == TileType::Vec, "[PTO][SA] SetValue / GetValue: Vec tiles");
+        __shared__ DType pto_getvalue_slot;
+        const uint32_t q = offset / detail::kVecChunk, e = offset % detail::kVecChunk;
+        if ((uint32_t)hw::tid() == q % kBlockThreads) {
+            const Storage &s = S();
+            DType v = s.v[0][0];
+#pragma unroll
+            for (int slot = 0; slot < Storage::Slots; ++slot)
+#pragma unroll
+                for (int i = 0; i < detail::kVecChunk; ++i)
+                    if ((uint32_t)slot == q / kBlockThreads && (uint32_t)i == e)
+                        v = s.v[slot][i];
+            pto_getvalue_slot = v;
+        }
+        __syncthreads();
+        const DType out = pto_getvalue_slot;
+        __syncthreads();
+        return out;
+    }
+
+private:
+    PTO_HD void Bind(const Tile &o)
+    {
+        static_assert(isHandle || detail::kTileCopyWriteback,
+                      "[PTO][SA] a register tile (Left / Right / Acc / Vec) was copied: pass it by reference, or define "
+                      "PTO_TILE_COPY_WRITEBACK before including pto-inst.hpp to give copies write-back semantics");
+        st = o.st;
+        if constexpr (!isHandle)
+            origin_ = const_cast<Tile *>(&o);
     }
 };
 

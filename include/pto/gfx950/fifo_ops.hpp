@@ -83,13 +83,13 @@ PTO_DEV void lds_image_store(uint32_t off, TileT &tile)
 #pragma unroll
                 for (int v = 0; v < kAccElems; ++v) {
                     const int r = rbase + mb * kMfmaM + acc_elem_row(v), c = cbase + nb * kMfmaM;
-                    img[r * TileT::Cols + c] = store_cast<T>(tile.st.f[mb][nb][v]);
+                    img[r * TileT::Cols + c] = store_cast<T>(tile.S().f[mb][nb][v]);
                 }
     } else {
         static_assert(TileT::Loc == TileType::Vec && TileT::isRowMajor, "[PTO][SA] TPUSH to an LDS FIFO: Acc or row-major Vec tile");
         for_each_owned<TileT>([&](int s, int i, int e) {
             if (e < TileT::Numel)
-                img[e] = (T)tile.st.v[s][i];
+                img[e] = (T)tile.S().v[s][i];
         });
     }
 }
@@ -100,7 +100,7 @@ PTO_DEV void lds_image_load(TileT &tile, uint32_t off)
     const T *img = reinterpret_cast<const T *>(hw::lds_base() + off);
     for_each_owned<TileT>([&](int s, int i, int e) {
         if (e < TileT::Numel)
-            tile.st.v[s][i] = (typename TileT::DType)img[e];
+            tile.S().v[s][i] = (typename TileT::DType)img[e];
     });
 }
 } // namespace detail

@@ -104,12 +104,12 @@ PTO_DEV void mad(AccT &out, const AccT &in, const LeftT &a, const RightT &b)
                 for (int i = 0; i < kAccElems; ++i)
                     c[i] = 0;
             } else {
-                c = in.st.f[mb][nb];
+                c = in.S().f[mb][nb];
             }
 #pragma unroll
             for (int ks = 0; ks < SL::KS; ++ks)
-                c = mfma32(a.st.f[mb][ks], b.st.f[nb][ks], c);
-            out.st.f[mb][nb] = c;
+                c = mfma32(a.S().f[mb][ks], b.S().f[nb][ks], c);
+            out.S().f[mb][nb] = c;
         }
 }
 
@@ -168,19 +168,19 @@ PTO_DEV void mad_mx(AccT &out, const AccT &in, const LeftT &a, const LeftScaleT 
                 for (int i = 0; i < kAccElems; ++i)
                     c[i] = 0.0f;
             } else {
-                c = in.st.f[mb][nb];
+                c = in.S().f[mb][nb];
             }
 #pragma unroll
             for (int ks = 0; ks < SL::KS; ++ks) {
                 // k step ks: scale byte 0 (even step) or 2 (odd step) of register ks / 2
                 if (ks % 2 == 0)
-                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(mx_operand(a.st.f[mb][ks]), mx_operand(b.st.f[nb][ks]), c, fa, fb,
-                                                                        0, (int)sa.st.s[mb][ks / 2], 0, (int)sb.st.s[nb][ks / 2]);
+                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(mx_operand(a.S().f[mb][ks]), mx_operand(b.S().f[nb][ks]), c, fa, fb,
+                                                                        0, (int)sa.S().s[mb][ks / 2], 0, (int)sb.S().s[nb][ks / 2]);
                 else
-                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(mx_operand(a.st.f[mb][ks]), mx_operand(b.st.f[nb][ks]), c, fa, fb,
-                                                                        2, (int)sa.st.s[mb][ks / 2], 2, (int)sb.st.s[nb][ks / 2]);
+                    c = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(mx_operand(a.S().f[mb][ks]), mx_operand(b.S().f[nb][ks]), c, fa, fb,
+                                                                        2, (int)sa.S().s[mb][ks / 2], 2, (int)sb.S().s[nb][ks / 2]);
             }
-            out.st.f[mb][nb] = c;
+            out.S().f[mb][nb] = c;
         }
 }
 } // namespace detail
@@ -216,7 +216,7 @@ PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasRow bias)
         for (int mb = 0; mb < SA::MB; ++mb)
 #pragma unroll
             for (int i = 0; i < detail::kAccElems; ++i)
-                c.st.f[mb][nb][i] += bv;
+                c.S().f[mb][nb][i] += bv;
     }
 }
 

@@ -103,16 +103,45 @@ PTO_DEV T pad_value(PadValue p)
 } // namespace detail
 
 // ------------------------------------------------------------------ TASSIGN
-// Mat tiles: `addr` is a byte offset into the workgroup's dynamic LDS (the L1 address space).
+// Mat tiles: `addr` is a byte offset into the workgroup's dynamic LDS (the L1 address space), or a pointer obtained from
+// a Mat tile's data() (pto_macro_matmul.hpp:176-177 rebinds a tile to `data() + bytes`): a generic pointer into LDS has
+// the shared aperture in its upper half, its lower half is the LDS address.
 // Register tiles have no address: the call is accepted and ignored, as in the CPU simulation
 // (cpu/TAssign.hpp:20-21).  GlobalTensor: rebinding the base pointer.
+namespace detail {
+constexpr uint32_t kLdsBytes = 160 * 1024; // LDS of one gfx950 compute unit
+// bytes of a Mat tile's LDS image (a Mat tile of block scales is stored one byte per scale)
+template <typename TileT>
+constexpr uint32_t mat_tile_bytes()
+{
+    if constexpr (std::is_same_v<typename TileT::DType, float8_e8m0_t>)
+        return TileT::Rows * TileT::Cols;
+    else
+        return MatGeom<TileT>::Bytes;
+}
+// A call that survives optimisation stops the build: a TASSIGN whose address the compiler knows lies beyond the LDS
+// (the reference checks its compile-time form the same way, tassign_check.hpp:18-30).
+#if defined(__HIP_DEVICE_COMPILE__)
+__device__ void tassign_beyond_lds() __attribute__((error("[PTO][SA] TASSIGN: the Mat tile ends beyond the 160 KiB LDS of a compute unit")));
+#endif
+} // namespace detail
 template <typename T, typename AddrType>
 PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
 {
     if constexpr (is_global_data_v<T>) {
         obj.SetAddr(reinterpret_cast<typename T::DType *>(addr));
     } else if constexpr (T::Loc == TileType::Mat) {
-        obj.st.lds = static_cast<uint32_t>((uintptr_t)addr);
+        const uint64_t a = (uint64_t)(uintptr_t)addr;
+        const uint32_t off = (a >> 32) ? (uint32_t)a - (uint32_t)(uintptr_t)hw::lds_base() : (uint32_t)a;
+#if defined(__HIP_DEVICE_COMPILE__)
+        if (__builtin_constant_p(off) && off + detail::mat_tile_bytes<T>() > detail::kLdsBytes)
+            detail::tassign_beyond_lds();
+#endif
+#if defined(_DEBUG) || defined(PTO_DEBUG)
+        if (off + detail::mat_tile_bytes<T>() > detail::kLdsBytes)
+            __builtin_trap(); // the run-time form of the reference's PTO_ASSERT (debug builds only)
+#endif
+        obj.st.lds = off;
     } else {
         (void)obj;
         (void)addr;
@@ -230,7 +259,7 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
         if (S::Chunks % kBlockThreads != 0 && q >= S::Chunks) {
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
-                dst.st.v[s][i] = pad;
+                dst.S().v[s][i] = pad;
             continue;
         }
         const int major = e0 / Minor, minor0 = e0 % Minor;
@@ -250,7 +279,7 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
 #endif
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
-                dst.st.v[s][i] = v[i];
+                dst.S().v[s][i] = v[i];
         } else {
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i) {
@@ -262,7 +291,7 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
                                                     (int64_t)mj * src.GetStride(4);
                     v = gm[b + (int64_t)mn * stMinor];
                 }
-                dst.st.v[s][i] = v;
+                dst.S().v[s][i] = v;
             }
         }
     }
@@ -341,19 +370,19 @@ PTO_DEV void tload_scale(TileT &dst, G &src)
     for (int b = 0; b < blocks; ++b) {
         const char *p = gm + (int64_t)(major0 + b * kMxM) * ld;
         if constexpr (S::KB == 2) {
-            dst.st.s[b][0] = (uint32_t)*reinterpret_cast<const uint16_t *>(p) >> shift;
+            dst.S().s[b][0] = (uint32_t)*reinterpret_cast<const uint16_t *>(p) >> shift;
         } else if constexpr (S::Regs % 4 == 0) {
 #pragma unroll
             for (int r = 0; r < S::Regs; r += 4) {
                 const u32x4 v = *reinterpret_cast<const u32x4 *>(p + 4 * r);
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    dst.st.s[b][r + i] = v[i] >> shift;
+                    dst.S().s[b][r + i] = v[i] >> shift;
             }
         } else {
 #pragma unroll
             for (int r = 0; r < S::Regs; ++r)
-                dst.st.s[b][r] = *reinterpret_cast<const uint32_t *>(p + 4 * r) >> shift;
+                dst.S().s[b][r] = *reinterpret_cast<const uint32_t *>(p + 4 * r) >> shift;
         }
     }
 }
@@ -411,11 +440,11 @@ PTO_DEV void textract_mx(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol)
 #pragma unroll
         for (int ks = 0; ks < S::KS; ++ks) {
             if constexpr (is_mx4_v<T>) {
-                dst.st.f[b][ks] = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 2));
+                dst.S().f[b][ks] = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 2));
             } else {
                 const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4));
                 const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds + mat_chunk_off<Geo::RowBytes>(major0 + b * kMxM, chunk0 + ks * 4 + 2));
-                dst.st.f[b][ks] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                dst.S().f[b][ks] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
             }
         }
 }
@@ -439,11 +468,11 @@ PTO_DEV void textract_scale_mat(DstT &dst, SrcT &src, uint32_t idxMajor, uint32_
     for (int b = 0; b < blocks; ++b) {
         const char *p = lds + Geo::off(major0 + b * kMxM, kb);
         if constexpr (D::KB == 2) {
-            dst.st.s[b][0] = *reinterpret_cast<const uint8_t *>(p + lane / kMxM);
+            dst.S().s[b][0] = *reinterpret_cast<const uint8_t *>(p + lane / kMxM);
         } else {
 #pragma unroll
             for (int r = 0; r < D::Regs; ++r)
-                dst.st.s[b][r] = *reinterpret_cast<const uint32_t *>(p + r * (Geo::Major * 4)) >> shift;
+                dst.S().s[b][r] = *reinterpret_cast<const uint32_t *>(p + r * (Geo::Major * 4)) >> shift;
         }
     }
 }
@@ -461,11 +490,11 @@ PTO_DEV void textract_scale(DstT &dst, const SrcT &src, uint32_t kb)
 #pragma unroll
     for (int b = 0; b < blocks; ++b) {
         if constexpr (D::KB == 2) {
-            dst.st.s[b][0] = src.st.s[b][kb / 4] >> ((kb % 4) * 8);
+            dst.S().s[b][0] = src.S().s[b][kb / 4] >> ((kb % 4) * 8);
         } else {
 #pragma unroll
             for (int r = 0; r < D::Regs; ++r)
-                dst.st.s[b][r] = src.st.s[b][kb / 4 + r];
+                dst.S().s[b][r] = src.S().s[b][kb / 4 + r];
         }
     }
 }
@@ -493,7 +522,7 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
         for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
             for (int ks = 0; ks < S::KS; ++ks)
-                dst.st.f[mb][ks] = *reinterpret_cast<const Frag *>(
+                dst.S().f[mb][ks] = *reinterpret_cast<const Frag *>(
                     lds + detail::mat_chunk_off<Geo::RowBytes>(row0 + mb * detail::kMfmaM, chunk0 + ks * kStepChunks));
     } else if constexpr (DstT::Loc == TileType::Right) {
         static_assert(!Geo::colsK, "[PTO][SA] TEXTRACT to Right: source must be contiguous along rows (Zn / column-major)");
@@ -504,7 +533,7 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
         for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
             for (int ks = 0; ks < S::KS; ++ks)
-                dst.st.f[nb][ks] = *reinterpret_cast<const Frag *>(
+                dst.S().f[nb][ks] = *reinterpret_cast<const Frag *>(
                     lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * kStepChunks));
     } else {
         static_assert(DstT::Loc == TileType::Left, "[PTO][SA] TEXTRACT: destination must be a Left or Right tile");
@@ -586,7 +615,7 @@ PTO_DEV void tstore_acc(G &dst, TileT &src)
                 const int r = rbase + mb * kMfmaM + acc_elem_row(v);
                 if (full || (r < vr && c < vc)) {
                     GT *p = gm + (int64_t)r * st_r + (int64_t)c * st_c;
-                    auto x = src.st.f[mb][nb][v];
+                    auto x = src.S().f[mb][nb][v];
                     if constexpr (relu == ReluPreMode::NormalRelu)
                         x = x < 0 ? 0 : x; // before the conversion, as the fix pipe does (a2a3/TStore.hpp:328)
                     if constexpr (atomic == AtomicType::AtomicAdd)
@@ -626,7 +655,7 @@ PTO_DEV void tstore_vec(G &dst, TileT &src)
             VT v;
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
-                v[i] = src.st.v[s][i];
+                v[i] = src.S().v[s][i];
 #if defined(PTO_VEC_STREAM_NT) && (PTO_VEC_STREAM_NT & 2)
             __builtin_nontemporal_store(v, reinterpret_cast<VT *>(gm + base + minor0));
 #else
@@ -640,7 +669,7 @@ PTO_DEV void tstore_vec(G &dst, TileT &src)
                 if (e < TileT::Numel && mj < vMajor && mn < vMinor) {
                     int64_t b = TileT::isRowMajor ? (stacked ? gm_row_offset(dst, mj) : (int64_t)mj * dst.GetStride(3)) :
                                                     (int64_t)mj * dst.GetStride(4);
-                    gm[b + (int64_t)mn * stMinor] = src.st.v[s][i];
+                    gm[b + (int64_t)mn * stMinor] = src.S().v[s][i];
                 }
             }
         }

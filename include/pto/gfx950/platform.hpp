@@ -103,13 +103,23 @@ constexpr int EVENT_ID_MAX = 8;
 PTO_DEV void set_flag(pipe_t, pipe_t, event_t) {}
 
 // wait_flag(src, dst): later `dst` work may start once earlier `src` work is complete.
+// The forms that order memory across wavefronts (src MTE2; dst MTE2 after MTE1 / V / MTE3 / FIX) contain a workgroup
+// barrier: every wave of the workgroup must reach them, so they may not sit under wave-divergent control flow.
 PTO_DEV void wait_flag(pipe_t src, pipe_t dst, event_t)
 {
     if (src == PIPE_MTE2) {
         // global->LDS copies of every wave must have landed before anyone reads the tile
         pto::hw::wait_vm0();
         pto::hw::lds_barrier();
-    } else if (dst == PIPE_MTE2 && (src == PIPE_MTE1 || src == PIPE_V || src == PIPE_MTE3)) {
+    } else if (dst == PIPE_MTE2 && (src == PIPE_MTE3 || src == PIPE_FIX)) {
+        // a tile that TSTORE wrote to global memory (from a Vec tile: MTE3, from an Acc tile: FIX) is loaded back, possibly
+        // by another wave of the workgroup (the reference's global-memory FIFO / workspace pattern): the stores of every
+        // wave must have completed and be visible to the workgroup before any wave's load
+        pto::hw::wait_vm0();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        pto::hw::lds_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    } else if (dst == PIPE_MTE2 && (src == PIPE_MTE1 || src == PIPE_V)) {
         // every wave must be done reading an LDS tile before a load overwrites it
         pto::hw::lds_barrier();
     } else if (src == PIPE_MTE3 && dst != PIPE_S) {

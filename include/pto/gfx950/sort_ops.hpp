@@ -43,7 +43,7 @@ PTO_DEV void stage_tile_rows(TileT &t, uint32_t *lds, int ld)
         if (e < TileT::Numel) {
             int r, c;
             elem_rc<TileT>(e, r, c);
-            lds[r * ld + c] = bits_of(t.st.v[s][i]);
+            lds[r * ld + c] = bits_of(t.S().v[s][i]);
         }
     });
 }
@@ -107,7 +107,7 @@ PTO_DEV void TSORT32_IMPL(DstT &dst, SrcT &src, IdxT &idx)
     detail::for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && r < vr && c < 2 * vc)
-            dst.st.v[s][i] = __builtin_bit_cast(T, image[r * 2 * C + c]);
+            dst.S().v[s][i] = __builtin_bit_cast(T, image[r * 2 * C + c]);
     });
     hw::lds_barrier();
 }
@@ -157,7 +157,7 @@ PTO_DEV void TMRGSORT_IMPL(DstT &dst, SrcT &src, uint32_t blockLen)
     hw::lds_barrier();
     detail::for_each_owned<DstT>([&](int s, int i, int e) {
         if (e < merged)
-            dst.st.v[s][i] = __builtin_bit_cast(T, image[e]);
+            dst.S().v[s][i] = __builtin_bit_cast(T, image[e]);
     });
     hw::lds_barrier();
 }
@@ -235,7 +235,7 @@ PTO_DEV void merge_lists(DstT &dst, MrgSortExecutedNumList &executed, S0 &src0, 
     hw::lds_barrier();
     for_each_owned<DstT>([&](int s, int i, int e) {
         if (e < 2 * stop)
-            dst.st.v[s][i] = __builtin_bit_cast(T, image[e]);
+            dst.S().v[s][i] = __builtin_bit_cast(T, image[e]);
     });
     executed.mrgSortList0 = (uint16_t)shared[1];
     executed.mrgSortList1 = (uint16_t)shared[2];

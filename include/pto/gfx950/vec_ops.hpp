@@ -166,9 +166,9 @@ PTO_DEV void stage_row_values(RowT &t, typename RowT::DType *lds)
             // the per-row scalar is element (r,0) of a column tile or (0,r) of a row tile (TRowExpandOp.hpp:20-33)
             if (RowT::Cols == 1 || (RowT::Rows != 1 && c == 0)) {
                 if (c == 0 && r < R)
-                    lds[r] = t.st.v[s][i];
+                    lds[r] = t.S().v[s][i];
             } else if (RowT::Rows == 1 && c < R) {
-                lds[c] = t.st.v[s][i];
+                lds[c] = t.S().v[s][i];
             }
         }
     });
@@ -186,7 +186,7 @@ PTO_DEV void TCVT_IMPL(DstT &dst, SrcT &src, RoundMode mode)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = detail::convert<typename DstT::DType>(src.st.v[s][i], mode);
+            dst.S().v[s][i] = detail::convert<typename DstT::DType>(src.S().v[s][i], mode);
 }
 template <typename DstT, typename SrcT>
 PTO_DEV void TCVT_IMPL(DstT &dst, SrcT &src, RoundMode mode, SaturationMode)
@@ -205,8 +205,8 @@ PTO_DEV void TCVT_IMPL(DstT &dst, SrcT &src, RoundMode mode, SaturationMode)
         using S = typename DstT::Storage;                                                               \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src0.st.v[s][i], b = src1.st.v[s][i];                                           \
-            dst.st.v[s][i] = (EXPR);                                                                    \
+            const T a = src0.S().v[s][i], b = src1.S().v[s][i];                                           \
+            dst.S().v[s][i] = (EXPR);                                                                    \
         }                                                                                               \
     }
 PTO_DEFINE_BINARY(TADD, a + b)
@@ -226,8 +226,8 @@ PTO_DEFINE_BINARY(TMIN, (b < a ? b : a))
         using S = typename DstT::Storage;                                                               \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src.st.v[s][i];                                                                 \
-            dst.st.v[s][i] = (EXPR);                                                                    \
+            const T a = src.S().v[s][i];                                                                 \
+            dst.S().v[s][i] = (EXPR);                                                                    \
         }                                                                                               \
     }
 PTO_DEFINE_SCALAR(TMULS, a *k)
@@ -246,7 +246,7 @@ PTO_DEV void TEXP_IMPL(TileT &dst, TileT &src)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = (typename TileT::DType)::exp((double)src.st.v[s][i]); // evaluated in double: TExp.hpp:36
+            dst.S().v[s][i] = (typename TileT::DType)::exp((double)src.S().v[s][i]); // evaluated in double: TExp.hpp:36
 }
 
 template <typename TileT>
@@ -257,7 +257,7 @@ PTO_DEV void TEXPANDS_IMPL(TileT &dst, typename TileT::DType k)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = k;
+            dst.S().v[s][i] = k;
 }
 
 // same storage, new logical shape: both tiles have the same element count and so the same
@@ -273,7 +273,7 @@ PTO_DEV void TRESHAPE_IMPL(DstT &dst, SrcT &src)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = __builtin_bit_cast(typename DstT::DType, src.st.v[s][i]);
+            dst.S().v[s][i] = __builtin_bit_cast(typename DstT::DType, src.S().v[s][i]);
 }
 
 // upper (1) / lower (0) triangular 0/1 mask: TTRI.hpp:31-63
@@ -287,7 +287,7 @@ PTO_DEV void TTRI_IMPL(TileT &dst, int diagonal)
         const int r = e / TileT::Cols, c = e % TileT::Cols;
         if (r < vr && c < vc) {
             const bool one = isUpperOrLower ? (c >= diagonal + r) : (c < diagonal + r + 1);
-            dst.st.v[s][i] = one ? (T)1 : (T)0;
+            dst.S().v[s][i] = one ? (T)1 : (T)0;
         }
     });
 }
@@ -316,7 +316,7 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
                 if (c0 + i < vc) {
-                    const A v = (A)src.st.v[s][i];
+                    const A v = (A)src.S().v[s][i];
                     acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : acc + v;
                 }
             part[q] = acc;
@@ -333,7 +333,7 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
                     const A v = part[r * CPR + j];
                     acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : acc + v;
                 }
-                dst.st.v[s][i] = (typename DstT::DType)acc;
+                dst.S().v[s][i] = (typename DstT::DType)acc;
             }
         }
     });
@@ -354,7 +354,7 @@ PTO_DEV void row_expand(DstT &dst, DstT &src0, RowT &src1)
     for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && r < vr && c < vc) {
-            const T a = src0.st.v[s][i], b = (T)rowv[r];
+            const T a = src0.S().v[s][i], b = (T)rowv[r];
             T o;
             if constexpr (op == RowOp::Sub)
                 o = a - b;
@@ -368,7 +368,7 @@ PTO_DEV void row_expand(DstT &dst, DstT &src0, RowT &src1)
                 o = a < b ? b : a;
             else
                 o = b < a ? b : a;
-            dst.st.v[s][i] = o;
+            dst.S().v[s][i] = o;
         }
     });
     hw::lds_barrier();
@@ -417,7 +417,7 @@ PTO_DEV void TGATHER_IMPL(DstT &dst, Src0T &src0, IdxT &idx)
         if (e < Src0T::Numel) {
             int r, c;
             detail::elem_rc<Src0T>(e, r, c);
-            stage[r * Src0T::Cols + c] = src0.st.v[s][i];
+            stage[r * Src0T::Cols + c] = src0.S().v[s][i];
         }
     });
     hw::lds_barrier();
@@ -426,9 +426,9 @@ PTO_DEV void TGATHER_IMPL(DstT &dst, Src0T &src0, IdxT &idx)
         int r, c;
         detail::elem_rc<DstT>(e, r, c);
         if (e < DstT::Numel && r < vr && c < vc) {
-            const int32_t raw = (int32_t)idx.st.v[s][i];
+            const int32_t raw = (int32_t)idx.S().v[s][i];
             const bool ok = raw >= 0 && raw < Src0T::Numel;
-            dst.st.v[s][i] = ok ? stage[raw] : (T)0;
+            dst.S().v[s][i] = ok ? stage[raw] : (T)0;
         }
     });
     hw::lds_barrier();
@@ -453,14 +453,14 @@ PTO_DEV void TGATHER_IMPL(DstT &dst, SrcT &src)
         if (e < SrcT::Numel && r < vr && c < vc && (c % div) == phase) {
             const int pos = r * perRow + c / div;
             if (pos < DstT::Numel)
-                stage[pos] = src.st.v[s][i];
+                stage[pos] = src.S().v[s][i];
         }
     });
     hw::lds_barrier();
     const int total = vr * perRow;
     detail::for_each_owned<DstT>([&](int s, int i, int e) {
         if (e < DstT::Numel && e < total)
-            dst.st.v[s][i] = __builtin_bit_cast(typename DstT::DType, stage[e]);
+            dst.S().v[s][i] = __builtin_bit_cast(typename DstT::DType, stage[e]);
     });
     hw::lds_barrier();
 }
@@ -480,7 +480,7 @@ PTO_DEV void MGATHER_IMPL(DstT &dst, G &src, IdxT &idx)
         int r, c;
         detail::elem_rc<DstT>(e, r, c);
         if (e < DstT::Numel && r < vr && c < vc)
-            dst.st.v[s][i] = gm[(size_t)idx.st.v[s][i]];
+            dst.S().v[s][i] = gm[(size_t)idx.S().v[s][i]];
     });
 }
 
@@ -514,7 +514,7 @@ PTO_DEV void MGATHER_ROWS_IMPL(DstT &dst, G &table, IdxT &rowIdx, int tableRows)
         }
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = v[i];
+            dst.S().v[s][i] = v[i];
     }
     hw::lds_barrier();
 }

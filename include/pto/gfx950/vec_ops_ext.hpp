@@ -19,8 +19,8 @@ namespace pto {
         using S = typename DstT::Storage;                                                               \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src.st.v[s][i];                                                                 \
-            dst.st.v[s][i] = (EXPR);                                                                    \
+            const T a = src.S().v[s][i];                                                                 \
+            dst.S().v[s][i] = (EXPR);                                                                    \
         }                                                                                               \
     }
 PTO_DEFINE_UNARY(TABS, (a < (T)0 ? -a : a))                                // TAbs.hpp:24
@@ -43,8 +43,8 @@ PTO_DEV void TPRELU_IMPL(DstT &dst, S0T &src0, S1T &src1)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i) {
-            const T a = src0.st.v[s][i], b = src1.st.v[s][i];
-            dst.st.v[s][i] = a > (T)0 ? a : (T)(a * b);
+            const T a = src0.S().v[s][i], b = src1.S().v[s][i];
+            dst.S().v[s][i] = a > (T)0 ? a : (T)(a * b);
         }
 }
 // dst = src > 0 ? src : src * k  (ElementOp.h:503-508)
@@ -58,8 +58,8 @@ PTO_DEV void TLRELU_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i) {
-            const T a = src.st.v[s][i];
-            dst.st.v[s][i] = a > (T)0 ? a : (T)(a * k);
+            const T a = src.S().v[s][i];
+            dst.S().v[s][i] = a > (T)0 ? a : (T)(a * k);
         }
 }
 
@@ -106,7 +106,7 @@ PTO_DEV void TCMP_IMPL(TileT &dst, TileT &src0, TileT &src1, CmpMode mode)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = detail::cmp_exact<T>(src0.st.v[s][i], src1.st.v[s][i], mode) ? (T)1 : (T)0;
+            dst.S().v[s][i] = detail::cmp_exact<T>(src0.S().v[s][i], src1.S().v[s][i], mode) ? (T)1 : (T)0;
 }
 
 // Packed form: bit (c % 8) of byte c / 8 of row r of dst = (src0[r,c] <mode> scalar); dst is a
@@ -130,7 +130,7 @@ PTO_DEV void TCMPS_IMPL(DstT &dst, SrcT &src0, T scalar, CmpMode mode)
             uint32_t byte = 0;
 #pragma unroll
             for (int i = 0; i < 8; ++i)
-                if (r < vr && c0 + i < vc && detail::cmp_scalar<typename SrcT::DType>(src0.st.v[s][i], (typename SrcT::DType)scalar, mode))
+                if (r < vr && c0 + i < vc && detail::cmp_scalar<typename SrcT::DType>(src0.S().v[s][i], (typename SrcT::DType)scalar, mode))
                     byte |= 1u << i;
             packed[q] = (uint8_t)byte;
         }
@@ -139,7 +139,7 @@ PTO_DEV void TCMPS_IMPL(DstT &dst, SrcT &src0, T scalar, CmpMode mode)
     detail::for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && c < SrcT::Cols / 8)
-            dst.st.v[s][i] = packed[r * (SrcT::Cols / 8) + c];
+            dst.S().v[s][i] = packed[r * (SrcT::Cols / 8) + c];
     });
     hw::lds_barrier();
 }
@@ -154,7 +154,7 @@ PTO_DEV void TSEL_IMPL(TileT &dst, MaskT &selMask, TileT &src0, TileT &src1)
     __shared__ uint8_t bits[MaskT::Numel];
     detail::for_each_owned<MaskT>([&](int s, int i, int e) {
         if (e < MaskT::Numel)
-            bits[e] = (uint8_t)selMask.st.v[s][i];
+            bits[e] = (uint8_t)selMask.S().v[s][i];
     });
     hw::lds_barrier();
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol(), vmc = selMask.GetValidCol();
@@ -163,7 +163,7 @@ PTO_DEV void TSEL_IMPL(TileT &dst, MaskT &selMask, TileT &src0, TileT &src1)
         if (e < TileT::Numel && r < vr && c < vc) {
             const int k = r * vc + c, b = k >> 3;
             const uint32_t byte = bits[(b / vmc) * MaskT::Cols + (b % vmc)];
-            dst.st.v[s][i] = ((byte >> (k & 7)) & 1u) ? src0.st.v[s][i] : src1.st.v[s][i];
+            dst.S().v[s][i] = ((byte >> (k & 7)) & 1u) ? src0.S().v[s][i] : src1.S().v[s][i];
         }
     });
     hw::lds_barrier();
@@ -178,7 +178,7 @@ PTO_DEV void TSELS_IMPL(TileT &dst, TileT &src0, TileT &src1, uint8_t selectMode
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = selectMode == 1 ? src0.st.v[s][i] : src1.st.v[s][i];
+            dst.S().v[s][i] = selectMode == 1 ? src0.S().v[s][i] : src1.S().v[s][i];
 }
 
 // ------------------------------------------------------------------ TFILLPAD
@@ -197,7 +197,7 @@ PTO_DEV void TFILLPAD_IMPL(DstT &dst, SrcT &src)
         int r, c;
         detail::elem_rc<DstT>(e, r, c);
         if (e < DstT::Numel)
-            dst.st.v[s][i] = (r < vr && c < vc) ? __builtin_bit_cast(T, src.st.v[s][i]) : pad;
+            dst.S().v[s][i] = (r < vr && c < vc) ? __builtin_bit_cast(T, src.S().v[s][i]) : pad;
     });
 }
 
@@ -230,7 +230,7 @@ PTO_DEV void col_reduce(DstT &dst, SrcT &src)
         if (r < vr && r < SrcT::Rows) {
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i) {
-                const A v = (A)src.st.v[s][i];
+                const A v = (A)src.S().v[s][i];
                 if (!any)
                     acc[i] = v;
                 else if (red == Red::Max)
@@ -261,7 +261,7 @@ PTO_DEV void col_reduce(DstT &dst, SrcT &src)
                     const A v = part[k][e];
                     a = red == Red::Max ? (a < v ? v : a) : red == Red::Min ? (v < a ? v : a) : a + v;
                 }
-            dst.st.v[s][i] = (typename DstT::DType)a;
+            dst.S().v[s][i] = (typename DstT::DType)a;
         }
     });
     hw::lds_barrier();
@@ -277,14 +277,14 @@ PTO_DEV void col_expand(DstT &dst, DstT &src0, ColT &src1)
     __shared__ typename ColT::DType colv[DstT::Cols];
     for_each_owned<ColT>([&](int s, int i, int e) {
         if (e < ColT::Numel)
-            colv[e] = src1.st.v[s][i];
+            colv[e] = src1.S().v[s][i];
     });
     hw::lds_barrier();
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && r < vr && c < vc) {
-            const T a = src0.st.v[s][i], b = (T)colv[c];
+            const T a = src0.S().v[s][i], b = (T)colv[c];
             T o;
             if constexpr (op == ColOp::Copy)
                 o = b;
@@ -302,7 +302,7 @@ PTO_DEV void col_expand(DstT &dst, DstT &src0, ColT &src1)
                 o = (T)::exp((double)(T)(a - b)); // ElementOp.h:265-270, as TROWEXPANDEXPDIF
             else
                 o = b < a ? b : a;
-            dst.st.v[s][i] = o;
+            dst.S().v[s][i] = o;
         }
     });
     hw::lds_barrier();
@@ -356,7 +356,7 @@ PTO_DEV void TROWEXPAND_IMPL(DstT &dst, RowT &src)
     detail::for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && r < vr && c < vc)
-            dst.st.v[s][i] = (typename DstT::DType)rowv[r];
+            dst.S().v[s][i] = (typename DstT::DType)rowv[r];
     });
     hw::lds_barrier();
 }
@@ -372,8 +372,8 @@ PTO_DEV void TROWEXPANDEXPDIF_IMPL(DstT &dst, DstT &src0, RowT &src1)
     detail::for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && r < vr && c < vc) {
-            const T d = src0.st.v[s][i] - (T)rowv[r];
-            dst.st.v[s][i] = (T)::exp((double)d);
+            const T d = src0.S().v[s][i] - (T)rowv[r];
+            dst.S().v[s][i] = (T)::exp((double)d);
         }
     });
     hw::lds_barrier();
@@ -403,7 +403,7 @@ PTO_DEV void stage_tile_rows_raw(TileT &t, uint32_t *lds)
     static_assert(sizeof(typename TileT::DType) == 4 && TileT::isRowMajor, "4-byte elements, row-major");
     for_each_owned<TileT>([&](int s, int i, int e) {
         if (e < TileT::Numel)
-            lds[e] = __builtin_bit_cast(uint32_t, t.st.v[s][i]);
+            lds[e] = __builtin_bit_cast(uint32_t, t.S().v[s][i]);
     });
 }
 } // namespace detail
@@ -430,7 +430,7 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
 #pragma unroll
             for (int v = 0; v < detail::kAccElems; ++v) {
                 const int r = rbase + mb * detail::kMfmaM + detail::acc_elem_row(v), c = cbase + nb * detail::kMfmaM;
-                stage[r * AccT::Cols + c] = (T)src.st.f[mb][nb][v];
+                stage[r * AccT::Cols + c] = (T)src.S().f[mb][nb][v];
             }
     hw::lds_barrier();
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
@@ -440,7 +440,7 @@ PTO_DEV void TMOV_ACC2VEC_IMPL(DstT &dst, AccT &src)
             T v = stage[e];
             if (relu == ReluPreMode::NormalRelu && v < (T)0)
                 v = (T)0;
-            dst.st.v[s][i] = v;
+            dst.S().v[s][i] = v;
         }
     });
     hw::lds_barrier();
@@ -469,14 +469,14 @@ PTO_DEV void stage_write(SrcT &src, T *stage, IndexF &&index)
             for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
                 for (int v = 0; v < kAccElems; ++v)
-                    stage[index(rbase + mb * kMfmaM + acc_elem_row(v), cbase + nb * kMfmaM)] = (T)src.st.f[mb][nb][v];
+                    stage[index(rbase + mb * kMfmaM + acc_elem_row(v), cbase + nb * kMfmaM)] = (T)src.S().f[mb][nb][v];
     } else {
         static_assert(SrcT::Loc == TileType::Vec, "[PTO][SA] TMOV / TTRANS: Vec or Acc source");
         for_each_owned<SrcT>([&](int s, int i, int e) {
             if (e < SrcT::Numel) {
                 int r, c;
                 elem_rc<SrcT>(e, r, c);
-                stage[index(r, c)] = (T)src.st.v[s][i];
+                stage[index(r, c)] = (T)src.S().v[s][i];
             }
         });
     }
@@ -506,7 +506,7 @@ PTO_DEV void TMOV_TO_OPERAND_IMPL(DstT &dst, SrcT &src)
         for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
             for (int ks = 0; ks < S::KS; ++ks)
-                dst.st.f[mb][ks] =
+                dst.S().f[mb][ks] =
                     *reinterpret_cast<const Frag *>(stage + (row0 + mb * detail::kMfmaM) * K + (kgroup + ks * kStepChunks) * kChunkElems);
     } else {
         const int col0 = hw::wave_n() * (S::NB * detail::kMfmaM) + major;
@@ -514,7 +514,7 @@ PTO_DEV void TMOV_TO_OPERAND_IMPL(DstT &dst, SrcT &src)
         for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
             for (int ks = 0; ks < S::KS; ++ks)
-                dst.st.f[nb][ks] =
+                dst.S().f[nb][ks] =
                     *reinterpret_cast<const Frag *>(stage + (col0 + nb * detail::kMfmaM) * K + (kgroup + ks * kStepChunks) * kChunkElems);
     }
     hw::lds_barrier();
@@ -535,7 +535,7 @@ PTO_DEV void TTRANS_IMPL(DstT &dst, SrcT &src)
         if (e < DstT::Numel) {
             int r, c;
             detail::elem_rc<DstT>(e, r, c);
-            dst.st.v[s][i] = stage[r * DstT::Cols + c];
+            dst.S().v[s][i] = stage[r * DstT::Cols + c];
         }
     });
     hw::lds_barrier();
@@ -567,8 +567,8 @@ PTO_DEV T elem_rem(T a, T b)
         using S = typename DstT::Storage;                                                               \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src0.st.v[s][i], b = src1.st.v[s][i];                                           \
-            dst.st.v[s][i] = (T)(EXPR);                                                                 \
+            const T a = src0.S().v[s][i], b = src1.S().v[s][i];                                           \
+            dst.S().v[s][i] = (T)(EXPR);                                                                 \
         }                                                                                               \
     }
 PTO_DEFINE_BINARY_EXT(TAND, true, a & b)
@@ -589,8 +589,8 @@ PTO_DEFINE_BINARY_EXT(TREM, false, detail::elem_rem<T>(a, b))
         using S = typename DstT::Storage;                                                               \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src.st.v[s][i];                                                                 \
-            dst.st.v[s][i] = (T)(EXPR);                                                                 \
+            const T a = src.S().v[s][i];                                                                 \
+            dst.S().v[s][i] = (T)(EXPR);                                                                 \
         }                                                                                               \
     }
 PTO_DEFINE_SCALAR_EXT(TANDS, true, a & k)
@@ -610,7 +610,7 @@ PTO_DEV void TNOT_IMPL(DstT &dst, SrcT &src)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i)
-            dst.st.v[s][i] = (typename DstT::DType)~src.st.v[s][i];
+            dst.S().v[s][i] = (typename DstT::DType)~src.S().v[s][i];
 }
 
 // dst = src0 +/- src1 + src2; the scalar forms take the scalar as the second operand
@@ -622,8 +622,8 @@ PTO_DEV void vec_addc(TileT &dst, TileT &src0, TileT &src1, TileT &src2)
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i) {
-            const auto a = src0.st.v[s][i], b = src1.st.v[s][i], c = src2.st.v[s][i];
-            dst.st.v[s][i] = kSub ? a - b + c : a + b + c;
+            const auto a = src0.S().v[s][i], b = src1.S().v[s][i], c = src2.S().v[s][i];
+            dst.S().v[s][i] = kSub ? a - b + c : a + b + c;
         }
 }
 template <typename TileT>
@@ -638,8 +638,8 @@ PTO_DEV void vec_addsc(TileT &dst, TileT &src0, typename TileT::DType k, TileT &
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i) {
-            const auto a = src0.st.v[s][i], c = src1.st.v[s][i];
-            dst.st.v[s][i] = kSub ? a - k + c : a + k + c;
+            const auto a = src0.S().v[s][i], c = src1.S().v[s][i];
+            dst.S().v[s][i] = kSub ? a - k + c : a + k + c;
         }
 }
 template <typename TileT>
@@ -668,9 +668,9 @@ PTO_DEV void part_op(DstT &dst, S0T &src0, S1T &src1)
             elem_rc<DstT>(e, r, c);
             if (r < dvr && c < dvc) {
                 const bool in0 = r < avr && c < avc, in1 = r < bvr && c < bvc;
-                const T a = src0.st.v[s][i], b = src1.st.v[s][i];
+                const T a = src0.S().v[s][i], b = src1.S().v[s][i];
                 const T both = KIND == 0 ? (T)(a + b) : KIND == 1 ? (a < b ? b : a) : (b < a ? b : a);
-                dst.st.v[s][i] = in0 && in1 ? both : in0 ? a : in1 ? b : (T)0;
+                dst.S().v[s][i] = in0 && in1 ? both : in0 ? a : in1 ? b : (T)0;
             }
         }
     });
@@ -693,7 +693,7 @@ PTO_DEV void TCI_IMPL(TileT &dst, T start)
     const int vc = dst.GetValidCol();
     detail::for_each_owned<TileT>([&](int s, int i, int e) {
         if (e < vc)
-            dst.st.v[s][i] = descending == 1 ? (T)(start - (T)e) : (T)(start + (T)e);
+            dst.S().v[s][i] = descending == 1 ? (T)(start - (T)e) : (T)(start + (T)e);
     });
 }
 
@@ -717,21 +717,21 @@ PTO_DEV void TSCATTER_IMPL(TileT &dst, TileT &src, IdxT &indexes)
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
     detail::for_each_owned<TileT>([&](int s, int i, int e) {
         const int r = e / TileT::Cols, c = e % TileT::Cols;
-        const uint32_t row = (uint32_t)indexes.st.v[s][i];
+        const uint32_t row = (uint32_t)indexes.S().v[s][i];
         if (e < N && r < vr && c < vc && row < (uint32_t)TileT::Rows)
             atomicMax(&owner[row * TileT::Cols + c], r);
     });
     hw::lds_barrier();
     detail::for_each_owned<TileT>([&](int s, int i, int e) {
         const int r = e / TileT::Cols, c = e % TileT::Cols;
-        const uint32_t row = (uint32_t)indexes.st.v[s][i];
+        const uint32_t row = (uint32_t)indexes.S().v[s][i];
         if (e < N && r < vr && c < vc && row < (uint32_t)TileT::Rows && owner[row * TileT::Cols + c] == r)
-            value[row * TileT::Cols + c] = __builtin_bit_cast(uint32_t, src.st.v[s][i]);
+            value[row * TileT::Cols + c] = __builtin_bit_cast(uint32_t, src.S().v[s][i]);
     });
     hw::lds_barrier();
     detail::for_each_owned<TileT>([&](int s, int i, int e) {
         if (e < N && owner[e] >= 0)
-            dst.st.v[s][i] = __builtin_bit_cast(T, value[e]);
+            dst.S().v[s][i] = __builtin_bit_cast(T, value[e]);
     });
     hw::lds_barrier();
 }
@@ -752,7 +752,7 @@ PTO_DEV void MSCATTER_IMPL(G &dst, SrcT &src, IdxT &indexes)
         int r, c;
         detail::elem_rc<SrcT>(e, r, c);
         if (e < SrcT::Numel && r < vr && c < vc)
-            gm[(size_t)indexes.st.v[s][i]] = src.st.v[s][i];
+            gm[(size_t)indexes.S().v[s][i]] = src.S().v[s][i];
     });
 }
 
@@ -789,7 +789,7 @@ PTO_DEV void TGATHERB_IMPL(DstT &dst, SrcT &src, OffT &offset)
                 __builtin_memcpy(v, bytes + off, 32); // any byte alignment
 #pragma unroll
                 for (int i = 0; i < detail::kVecChunk; ++i)
-                    dst.st.v[s][i] = v[i];
+                    dst.S().v[s][i] = v[i];
             }
         }
     }

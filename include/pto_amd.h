@@ -96,8 +96,11 @@ int pto_attention_auto_f32(void *stream, float *out, const float *q, const float
 /* Flash-attention forward.  q [batch, heads, seq_q, head_dim], k and v [batch, heads, seq_kv, head_dim],
  * fp16, contiguous.  o: fp16 (o_fp32 == 0) or fp32 (o_fp32 != 0) [batch, heads, seq_q, head_dim];
  * lse: NULL or fp32 [batch, heads, seq_q] = max*scale + ln(sum).  scale = 1/sqrt(head_dim) is applied
- * to (x - max) as in the reference's softmax stage (pto_macro_fa_softmax.hpp:82-97).  causal != 0:
- * key j is visible to query i iff j <= i + (seq_kv - seq_q); seq_kv >= seq_q is required then.
+ * to (x - max) as in the reference's softmax stage (pto_macro_fa_softmax.hpp:82-97).  causal == 1:
+ * key j is visible to query i iff j <= i + (seq_kv - seq_q) (the diagonal ends in the last key); seq_kv >= seq_q is
+ * required then.  causal == 2: iff j <= i (the diagonal starts in the first key: the rule of the reference's kernel,
+ * fa_performance_kernel.cpp:298-299, :757, and of its generator, scripts/gen_data.py:53), any seq_kv.  The two agree
+ * when seq_kv == seq_q.
  * head_dim in {64, 128}; seq_q % 128 == 0, seq_kv % 64 == 0.  No workspace: scores and probabilities
  * never leave the compute unit (the reference's caller-provided GM FIFOs have no counterpart). */
 int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,

@@ -65,6 +65,54 @@ def build_host(verbose=True):
             print("built", out)
 
 
+REFERENCE = os.environ.get("PTO_REFERENCE", "/root/reference")
+PORTED_DIR = os.path.join(ROOT, "oracle", "_ref")
+# (library, reference source, constants rewritten for 160 KiB of LDS, dynamic LDS bytes of the launch)
+PORTED = [
+    ("libpto_ported_gemm.so", "kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp",
+     [("stepKa", "1"), ("stepKb", "1")], 160 * 1024),
+]
+
+
+def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includes=()):
+    """Runs a kernel source of the reference through port_ascend_source.py into a temporary directory and compiles the
+    result against include/pto with hipcc; `out` ends in .o (compile only) or .so.  The ported text never enters the
+    repository tree."""
+    import importlib.util
+    import tempfile
+    spec = importlib.util.spec_from_file_location("port_ascend_source", os.path.join(HERE, "port_ascend_source.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    src = os.path.join(REFERENCE, rel_src)
+    with open(src) as f:
+        text, _ = mod.port(f.read(), sets, lds_bytes)
+    with tempfile.TemporaryDirectory() as tmp:
+        hip = os.path.join(tmp, os.path.basename(rel_src).replace(".cpp", ".hip"))
+        with open(hip, "w") as f:
+            f.write(text)
+        mode = ["-c"] if out.endswith(".o") else ["-shared"]
+        cmd = [HIPCC] + FLAGS + ["-I" + os.path.dirname(src)] + ["-I" + i for i in extra_includes] + list(extra_flags) + mode + [hip, "-o", out]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
+    return r.returncode, err
+
+
+def build_ported(verbose=True):
+    """The reference's own kernel sources compiled against this library's headers (only where the reference tree is
+    mounted; the libraries go to oracle/_ref/, which is kept out of the history)."""
+    if not os.path.isdir(REFERENCE):
+        return
+    os.makedirs(PORTED_DIR, exist_ok=True)
+    for lib, rel_src, sets, lds in PORTED:
+        out = os.path.join(PORTED_DIR, lib)
+        rc, err = port_and_compile(rel_src, sets, lds, out)
+        if rc != 0:
+            raise RuntimeError("ported build failed for %s:\n%s" % (rel_src, err))
+        if verbose:
+            print("built", out)
+
+
 if __name__ == "__main__":
     build()
+    build_ported()
     sys.exit(0)

@@ -1,7 +1,8 @@
 // `call_kernel` of the flash-attention demo (demos/torch_jit/flash_atten/fa_kernel.cpp:1017-1092): one head,
 // q [s0, 128], k and v [s1, 128] fp16, o_out [s0, 128] fp32.  Same signature.  The workspace arguments are the
 // reference's global-memory FIFOs and intermediates; this back end keeps scores and probabilities on chip and
-// does not touch them.  Unsupported parameters return without launching, as the reference does
+// does not touch them.  The causal mask follows the reference's rule (key j is visible to query i iff j <= i, whatever
+// s1 is: fa_kernel.cpp's runTFA skips tiles with s1_index > s0_index).  Unsupported parameters return without launching, as the reference does
 // (fa_kernel.cpp:1050-1058); pto_last_status_fa() tells why.
 #include <cstdint>
 
@@ -27,5 +28,5 @@ extern "C" void call_kernel(void *stream, int headSize, int s0, int s1, bool is_
         return;
     }
     g_last = pto_fa_fwd_f16(stream, o_out, nullptr, reinterpret_cast<const uint16_t *>(q), reinterpret_cast<const uint16_t *>(k),
-                            reinterpret_cast<const uint16_t *>(v), 1, 1, s0, s1, headSize, is_causal ? 1 : 0, 1);
+                            reinterpret_cast<const uint16_t *>(v), 1, 1, s0, s1, headSize, is_causal ? 2 : 0, 1);
 }

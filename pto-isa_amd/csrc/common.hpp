@@ -40,8 +40,8 @@ int gemm_f16f32_tile256_w8(hipStream_t st, float *c, const _Float16 *a, const _F
 // defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries, two groups of four waves in
 // opposite MFMA / softmax phases)
 int fa_fwd_d128_w8(hipStream_t st, void *o, float *lse, const _Float16 *q, const _Float16 *k, const _Float16 *v, int batch, int heads,
-                   int seqQ, int seqKv, bool causal, bool oFp32);
+                   int seqQ, int seqKv, bool causal, bool oFp32, int causalOff);
 // defined in pto_fa_w8m16.hip: the same schedule on v_mfma_f32_16x16x32_f16
 int fa_fwd_d128_w8m16(hipStream_t st, void *o, float *lse, const _Float16 *q, const _Float16 *k, const _Float16 *v, int batch, int heads,
-                      int seqQ, int seqKv, bool causal, bool oFp32);
+                      int seqQ, int seqKv, bool causal, bool oFp32, int causalOff);
 } // namespace pto_amd

@@ -142,7 +142,7 @@ template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int kBKV = kBKVDefau
 __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
                                                                       __gm__ const half *qAll, __gm__ const half *kAll,
                                                                       __gm__ const half *vAll, int heads, int seqQ,
-                                                                      int seqKv, int numBH)
+                                                                      int seqKv, int numBH, int causalOff)
 {
     constexpr int NQ = 1;          // 32-query blocks per wave
     constexpr int kBQ = kBQ1 * NQ; // queries per workgroup
@@ -189,7 +189,6 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
     __gm__ half *kBase = const_cast<half *>(kAll) + (int64_t)bh * seqKv * D;
     __gm__ half *vBase = const_cast<half *>(vAll) + (int64_t)bh * seqKv * D;
 
-    const int causalOff = seqKv - seqQ;
     int numTiles = seqKv / kBKV;
     if (CAUSAL) { // tiles wholly above the diagonal are skipped (fa_performance_kernel.cpp:757-758)
         const int lastKey = q0 + kBQ - 1 + causalOff;
@@ -565,7 +564,7 @@ PTO_DEVICE_CODE_END
 namespace {
 template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS = 1, int kBKV = kBKVDefault, bool PP = false>
 int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads,
-              int seqQ, int seqKv)
+              int seqQ, int seqKv, int causalOff)
 {
     if (seqQ % kBQ1 || seqKv % kBKV)
         return PTO_ERR_UNSUPPORTED;
@@ -579,7 +578,7 @@ int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k,
     const long long blocks = (long long)numBH * (seqQ / kBQ1);
     if (blocks > 0x7fffffffLL)
         return PTO_ERR_UNSUPPORTED;
-    kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH);
+    kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH, causalOff);
     return pto_amd::check_launch();
 }
 } // namespace

@@ -106,7 +106,7 @@ AICORE inline s16x4 DsReadTr16b(uint32_t addr)
 template <int D, bool CAUSAL, bool OUT_F32>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE void FlashAttnFwdM16(__gm__ void *outO, __gm__ float *outLse, __gm__ const half *qAll,
                                                                            __gm__ const half *kAll, __gm__ const half *vAll, int heads,
-                                                                           int seqQ, int seqKv, int numBH)
+                                                                           int seqQ, int seqKv, int numBH, int causalOff)
 {
     constexpr int kBQ = kBQ16, kBKV = kBKV16;
     constexpr int NQ = 2;          // 16-query column blocks per wave
@@ -148,7 +148,6 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE void FlashAttnFwdM16(__gm_
     __gm__ half *qBase = const_cast<half *>(qAll) + ((int64_t)bh * seqQ + q0) * D;
     __gm__ half *kBase = const_cast<half *>(kAll) + (int64_t)bh * seqKv * D;
     __gm__ half *vBase = const_cast<half *>(vAll) + (int64_t)bh * seqKv * D;
-    const int causalOff = seqKv - seqQ;
     int numTiles = seqKv / kBKV;
     if (CAUSAL) {
         const int lim = (q0 + kBQ - 1 + causalOff) / kBKV + 1;
@@ -450,7 +449,7 @@ PTO_DEVICE_CODE_END
 
 namespace {
 template <int D, bool CAUSAL, bool OUT_F32>
-int launch_fa_m16(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads, int seqQ, int seqKv)
+int launch_fa_m16(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads, int seqQ, int seqKv, int causalOff)
 {
     if (seqQ % kBQ16 || seqKv % kBKV16)
         return PTO_ERR_UNSUPPORTED;
@@ -463,7 +462,7 @@ int launch_fa_m16(hipStream_t st, void *o, float *lse, const half *q, const half
     const long long blocks = (long long)numBH * (seqQ / kBQ16);
     if (blocks > 0x7fffffffLL)
         return PTO_ERR_UNSUPPORTED;
-    kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH);
+    kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH, causalOff);
     return pto_amd::check_launch();
 }
 } // namespace

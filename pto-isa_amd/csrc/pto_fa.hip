@@ -30,12 +30,17 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
                                       const uint16_t *v, int batch, int heads, int seq_q, int seq_kv, int head_dim,
                                       int causal, int variant)
 {
+    if (!o || !q || !k || !v || batch <= 0 || heads <= 0 || seq_q <= 0 || seq_kv <= 0)
+        return PTO_ERR_BAD_ARG;
+    if (causal && seq_kv < seq_q)
+        return PTO_ERR_UNSUPPORTED;
+    const int causalOff = seq_kv - seq_q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *hq = reinterpret_cast<const half *>(q), *hk = reinterpret_cast<const half *>(k),
                *hv = reinterpret_cast<const half *>(v);
 #define PTO_FA_VARIANT(VV, DD, CC, MB)                           \
     if (variant == VV && head_dim == DD && (causal != 0) == CC) \
-        return launch_fa<DD, CC, false, MB>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+        return launch_fa<DD, CC, false, MB>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     PTO_FA_VARIANT(1, 128, false, 1)
     PTO_FA_VARIANT(2, 128, false, 2)
     PTO_FA_VARIANT(2, 128, true, 2)
@@ -44,15 +49,15 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
     PTO_FA_VARIANT(5, 64, true, 3)
 #undef PTO_FA_VARIANT
     if (variant == 10 && head_dim == 128)
-        return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false);
+        return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false, causalOff);
     if (variant == 20 && head_dim == 128)
-        return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false);
+        return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false, causalOff);
     if (variant == 21 && head_dim == 128) // fp32 output and LSE
-        return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, true);
+        return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, true, causalOff);
     if (variant == 6 && head_dim == 128 && !causal)
-        return launch_fa<128, false, false, 2, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+        return launch_fa<128, false, false, 2, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     if (variant == 6 && head_dim == 64 && causal)
-        return launch_fa<64, true, false, 3, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+        return launch_fa<64, true, false, 3, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     return PTO_ERR_BAD_ARG;
 }
 
@@ -63,8 +68,14 @@ extern "C" int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t 
         return PTO_ERR_BAD_ARG;
     if ((head_dim != 64 && head_dim != 128) || seq_q % kBQ1 || seq_kv % kBKVDefault)
         return PTO_ERR_UNSUPPORTED;
-    if (causal && seq_kv < seq_q)
+    // causal == 1: the diagonal ends in the last key (query i sees keys j <= i + seq_kv - seq_q; needs seq_kv >= seq_q);
+    // causal == 2: the diagonal starts in the first key (j <= i, the rule of the reference's kernel and generator:
+    // fa_performance_kernel.cpp:298-299 and :757, scripts/gen_data.py:53), any seq_kv.  The same when seq_kv == seq_q.
+    if (causal != 0 && causal != 1 && causal != 2)
+        return PTO_ERR_BAD_ARG;
+    if (causal == 1 && seq_kv < seq_q)
         return PTO_ERR_UNSUPPORTED;
+    const int causalOff = causal == 2 ? 0 : seq_kv - seq_q;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *hq = reinterpret_cast<const half *>(q), *hk = reinterpret_cast<const half *>(k),
                *hv = reinterpret_cast<const half *>(v);
@@ -82,14 +93,14 @@ extern "C" int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t 
             // the same schedule on 16 x 16 x 32 MFMAs: +1.5 .. 3.6 % without a mask and for long causal sequences
             // (interleaved runs; B2 H16 S2048 causal is 6 % slower on it and stays on the 32 x 32 x 16 kernel)
             if (!causal || seq_kv >= 4096)
-                return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, o_fp32 != 0);
-            return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, o_fp32 != 0);
+                return pto_amd::fa_fwd_d128_w8m16(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, o_fp32 != 0, causalOff);
+            return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, o_fp32 != 0, causalOff);
         }
     }
     // otherwise workgroups of four wavefronts (128 queries): two per compute unit at head_dim 128, three at 64
 #define PTO_FA_CASE(DD, CC, FF)                                                                      \
     if (head_dim == DD && (causal != 0) == CC && (o_fp32 != 0) == FF)                                \
-        return launch_fa<DD, CC, FF, (DD == 128 ? 2 : 3)>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv);
+        return launch_fa<DD, CC, FF, (DD == 128 ? 2 : 3)>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     PTO_FA_CASE(128, false, false)
     PTO_FA_CASE(128, false, true)
     PTO_FA_CASE(128, true, false)

@@ -10,12 +10,12 @@
 
 namespace pto_amd {
 int fa_fwd_d128_w8(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads, int seqQ,
-                   int seqKv, bool causal, bool oFp32)
+                   int seqKv, bool causal, bool oFp32, int causalOff)
 {
     if (causal)
-        return oFp32 ? launch_fa<128, true, true, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv)
-                     : launch_fa<128, true, false, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv);
-    return oFp32 ? launch_fa<128, false, true, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv)
-                 : launch_fa<128, false, false, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv);
+        return oFp32 ? launch_fa<128, true, true, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff)
+                     : launch_fa<128, true, false, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff);
+    return oFp32 ? launch_fa<128, false, true, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff)
+                 : launch_fa<128, false, false, 1, kBKVDefault, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff);
 }
 } // namespace pto_amd

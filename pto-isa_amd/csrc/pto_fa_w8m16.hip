@@ -9,12 +9,12 @@
 
 namespace pto_amd {
 int fa_fwd_d128_w8m16(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads, int seqQ,
-                      int seqKv, bool causal, bool oFp32)
+                      int seqKv, bool causal, bool oFp32, int causalOff)
 {
     if (causal)
-        return oFp32 ? launch_fa_m16<128, true, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv)
-                     : launch_fa_m16<128, true, false>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv);
-    return oFp32 ? launch_fa_m16<128, false, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv)
-                 : launch_fa_m16<128, false, false>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv);
+        return oFp32 ? launch_fa_m16<128, true, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff)
+                     : launch_fa_m16<128, true, false>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff);
+    return oFp32 ? launch_fa_m16<128, false, true>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff)
+                 : launch_fa_m16<128, false, false>(st, o, lse, q, k, v, batch, heads, seqQ, seqKv, causalOff);
 }
 } // namespace pto_amd

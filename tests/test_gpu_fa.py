@@ -43,6 +43,32 @@ def dense_fp64(q, k, v, causal=False):
     return (p / l) @ v, (m + np.log(l)).reshape(-1)
 
 
+def rows_fp64(q, k, v, rows, causal=False):
+    """The rows `rows` of one head's attention output and log-sum-exp in float64 (seq_q == seq_kv when causal)."""
+    q, k, v = q[rows].astype(np.float64), k.astype(np.float64), v.astype(np.float64)
+    s = q @ k.T / np.sqrt(q.shape[1])
+    if causal:
+        s = np.where(np.arange(k.shape[0])[None, :] > np.asarray(rows)[:, None], -np.inf, s)
+    m = s.max(axis=1, keepdims=True)
+    p = np.exp(s - m)
+    l = p.sum(axis=1, keepdims=True)
+    return (p / l) @ v, (m + np.log(l)).reshape(-1)
+
+
+def check_sampled_rows_of_every_head(q, k, v, o, lse, causal, seed):
+    """8 query rows of EVERY (batch, head) against float64, output and log-sum-exp: a wrong batch / head stride or a
+    query tile written to the wrong place cannot hide in the heads that are checked in full."""
+    B, H, S, _ = q.shape
+    rng = np.random.default_rng(seed)
+    for b in range(B):
+        for h in range(H):
+            rows = np.sort(np.r_[0, S - 1, rng.integers(0, S, size=6)])
+            want, want_lse = rows_fp64(q[b, h], k[b, h], v[b, h], rows, causal)
+            scale = max(np.max(np.abs(want)), 0.05)
+            assert np.max(np.abs(o[b, h][rows] - want)) <= TOL * scale, (b, h)
+            assert np.max(np.abs(lse[b, h][rows] - want_lse)) <= 1e-3, (b, h)
+
+
 def rel(got, want):
     return float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
 
@@ -103,6 +129,7 @@ def test_fa_config3_noncausal_b1_h16_s4096_d128():
         want, want_lse = dense_fp64(q[0, h], k[0, h], v[0, h])
         assert rel(o[0, h], want) <= TOL
         assert np.max(np.abs(lse[0, h] - want_lse)) <= 1e-3
+    check_sampled_rows_of_every_head(q, k, v, o, lse, False, seed=3)
     # all heads: rows of the output are convex combinations of V rows -> bounded by V's range per column
     assert np.all(o.max(axis=2) <= v.astype(np.float32).max(axis=2) + 1e-3)
     assert np.all(o.min(axis=2) >= v.astype(np.float32).min(axis=2) - 1e-3)
@@ -174,6 +201,7 @@ def test_fa_config4_causal_b4_h32_s2048_d64():
         want, want_lse = dense_fp64(q[b, h], k[b, h], v[b, h], causal=True)
         assert rel(o[b, h], want) <= TOL
         assert np.max(np.abs(lse[b, h] - want_lse)) <= 1e-3
+    check_sampled_rows_of_every_head(q, k, v, o, lse, True, seed=4)
     # first query of every head sees exactly key 0: output = v[0], lse = q0.k0/sqrt(D)
     assert np.array_equal(o[:, :, 0, :], v[:, :, 0, :].astype(np.float32))
     s00 = np.einsum("bhd,bhd->bh", q[:, :, 0].astype(np.float64), k[:, :, 0].astype(np.float64)) / np.sqrt(D)
@@ -188,3 +216,31 @@ def test_fa_rejects_bad_shapes():
     assert lib.pto_fa_fwd_f16(0, p, 0, p, p, p, 1, 1, 128, 128, 96, 0, 0) == capi.ERR_UNSUPPORTED
     assert lib.pto_fa_fwd_f16(0, p, 0, p, p, p, 1, 1, 256, 128, 64, 1, 0) == capi.ERR_UNSUPPORTED
     assert lib.pto_fa_fwd_f16(0, 0, 0, p, p, p, 1, 1, 128, 128, 64, 0, 0) == capi.ERR_BAD_ARG
+
+
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("Sq,Skv", [(256, 512), (512, 256), (256, 256)])
+def test_fa_causal_diagonal_from_the_first_key(oracle, D, Sq, Skv):
+    """causal == 2: key j visible to query i iff j <= i (the reference kernel's rule), seq_kv larger or smaller than
+    seq_q; against the oracle's streaming recurrence with q_offset = 0 and dense float64."""
+    from gpu_util import to_dev, stream
+    lib = capi.load()
+    B, H = 2, 2
+    q, k, v = datagen.fa_inputs(B, H, Sq, Skv, D, scale=1.0)
+    tq, tk, tv = to_dev(q), to_dev(k), to_dev(v)
+    to = torch.full((B, H, Sq, D), float("nan"), dtype=torch.float32, device="cuda:0")
+    tl = torch.full((B, H, Sq), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(lib.pto_fa_fwd_f16(stream(), to.data_ptr(), tl.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(),
+                                  B, H, Sq, Skv, D, 2, 1), "pto_fa_fwd_f16")
+    torch.cuda.synchronize()
+    o, lse = to.cpu().numpy(), tl.cpu().numpy()
+    for b, h in ((0, 0), (1, 1)):
+        s = q[b, h].astype(np.float64) @ k[b, h].astype(np.float64).T / np.sqrt(D)
+        s = np.where(np.triu(np.ones((Sq, Skv), dtype=bool), 1), -np.inf, s)
+        m = s.max(axis=1, keepdims=True)
+        p = np.exp(s - m)
+        want = (p / p.sum(axis=1, keepdims=True)) @ v[b, h].astype(np.float64)
+        assert rel(o[b, h], want) <= TOL
+        assert np.max(np.abs(lse[b, h] - (m + np.log(p.sum(axis=1, keepdims=True))).reshape(-1))) <= 1e-3
+        oo, mm, ll = oracle.fa_stream_f16(q[b, h], k[b, h], v[b, h], tile_s1=64, causal=True, q_offset=0, round_away=False)
+        assert rel(o[b, h], oo) <= 5e-4

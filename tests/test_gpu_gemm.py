@@ -66,6 +66,47 @@ def test_gemm_four_wave_tile_shapes_exact():
             assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
 
 
+def test_gemm_eight_wave_tile_shapes_exact():
+    """Every tile shape of the eight-wave kernel on 16 x 16 x 32 MFMAs (tuning hook: 256 x 256 with and without quarter
+    tiles, 256 x 192, 384 x 192 = the kernel that the 6144 x 6144 problem selects) on integer inputs: the whole matrix,
+    exactly."""
+    import ctypes as C
+    import torch
+    from gpu_util import to_dev
+    lib = capi.load()
+    fn = lib.pto_gemm_f16f32_m16_variant
+    fn.restype, fn.argtypes = C.c_int, [C.c_void_p] * 4 + [C.c_int] * 4
+    for m, n, k in ((768, 768, 512), (1536, 2304, 256)):
+        a, b = datagen.gemm_inputs_integer(m, n, k)
+        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
+        ta, tb = to_dev(a), to_dev(b)
+        for variant in (0, 3, 10, 12):
+            tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "eight-wave GEMM variant %d" % variant)
+            torch.cuda.synchronize()
+            assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
+
+
+def test_gemm_6144_every_element_exact():
+    """The headline problem through the public entry point (it selects the 384 x 192-tile kernel) on integer operands in
+    [1, 5): all 6144 x 6144 sums (at most 16 * 6144 < 2^24) are exact in fp32, so every element must equal the product
+    taken in float64 by the BLAS behind torch (an independent code path)."""
+    import torch
+    from gpu_util import to_dev, stream
+    lib = capi.load()
+    m = n = k = 6144
+    a, b = datagen.gemm_inputs_integer(m, n, k)
+    ta, tb = to_dev(a), to_dev(b)
+    tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(lib.pto_gemm_f16f32(stream(), tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k), "pto_gemm_f16f32")
+    torch.cuda.synchronize()
+    want = ta.view(torch.float16).double() @ tb.view(torch.float16).double().T
+    assert torch.equal(tc.double(), want)
+    # and the float64 product itself against int64 numpy on a band of rows
+    rows = np.r_[0:8, 3000:3008, 6136:6144]
+    assert np.array_equal(want[rows].cpu().numpy(), (a[rows].astype(np.int64) @ b.astype(np.int64).T).astype(np.float64))
+
+
 def test_gemm_integer_inputs_exact(oracle):
     """Integer operands in [1,5): every partial sum is exact in fp32 whatever the summation order, so a
     wrong fragment layout, a dropped K step or a transposed operand cannot hide inside a tolerance."""

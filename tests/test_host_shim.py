@@ -139,3 +139,34 @@ def test_call_kernel_flash_attention(causal):
     lib.call_kernel(torch.cuda.current_stream().cuda_stream, 64, s0, s1, causal, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(),
                     0, 0, 0, 0, 0, 0, 0)
     assert lib.pto_last_status_fa() != 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("s0,s1", [(256, 512), (512, 256), (128, 1024)])
+def test_call_kernel_flash_attention_causal_rule_of_the_reference(oracle, s0, s1):
+    """s1 != s0 with is_causal: key j is visible to query i iff j <= i, with no offset (np.triu(..., 1) in the
+    reference's gen_data.py:53; runTFA skips tiles with s1_index > s0_index, fa_performance_kernel.cpp:298-299 and :757).
+    Checked against the oracle's streaming recurrence with q_offset = 0 and against a dense float64 softmax."""
+    import torch
+    lib = _lib("libpto_call_fa.so")
+    lib.call_kernel.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_bool] + [C.c_void_p] * 11
+    lib.call_kernel.restype = None
+    d = 128
+    rng = np.random.default_rng(7)
+    q = (rng.standard_normal((s0, d)) * 1.5).astype(np.float16)
+    k = (rng.standard_normal((s1, d)) * 1.2).astype(np.float16)
+    v = rng.standard_normal((s1, d)).astype(np.float16)
+    tq, tk, tv = (torch.from_numpy(t.view(np.int16)).cuda() for t in (q, k, v))
+    o = torch.full((s0, d), float("nan"), dtype=torch.float32, device="cuda")
+    lib.call_kernel(torch.cuda.current_stream().cuda_stream, d, s0, s1, True, tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(),
+                    0, 0, 0, 0, 0, 0, 0)
+    torch.cuda.synchronize()
+    assert lib.pto_last_status_fa() == 0
+    got = o.cpu().numpy()
+    s = q.astype(np.float64) @ k.astype(np.float64).T / np.sqrt(d)
+    s = np.where(np.triu(np.ones((s0, s1), dtype=bool), 1), -np.inf, s)
+    p = np.exp(s - s.max(axis=1, keepdims=True))
+    want = (p / p.sum(axis=1, keepdims=True)) @ v.astype(np.float64)
+    assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 2e-3
+    oo, _, _ = oracle.fa_stream_f16(q, k, v, tile_s1=64, causal=True, q_offset=0, round_away=False)
+    assert np.max(np.abs(got - oo)) / np.max(np.abs(oo)) < 5e-4

@@ -1,0 +1,100 @@
+"""The C++ boundary as a drop-in: kernel sources of the reference compile against include/pto with hipcc for gfx950
+after the mechanical edits of pto-isa_amd/port_ascend_source.py (device-code brackets, the launch statement, tile-size
+constants that fit 160 KiB of LDS), and the mistakes a port can make are compile errors, not wrong results.
+
+The reference sources are read where they lie; the tests are skipped where the reference tree is not mounted.  Nothing
+here needs a GPU: hipcc cross-compiles."""
+import importlib.util
+import os
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "pto-isa_amd")
+
+
+def _build_mod():
+    spec = importlib.util.spec_from_file_location("pto_amd_build", os.path.join(PKG, "build.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+B = _build_mod()
+needs_reference = pytest.mark.skipif(not os.path.isdir(B.REFERENCE), reason="reference tree not mounted")
+GEMM_SRC = "kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp"
+
+
+def _hipcc_snippet(tmp_path, body, defines=()):
+    src = tmp_path / "snippet.hip"
+    src.write_text(body)
+    cmd = [B.HIPCC] + B.FLAGS + ["-D" + d for d in defines] + ["-c", str(src), "-o", str(tmp_path / "snippet.o")]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    return r.returncode, r.stderr
+
+
+@needs_reference
+def test_reference_gemm_kernel_compiles(tmp_path):
+    """gemm_performance_kernel.cpp with stepKa = stepKb = 1 (two 16 KiB A panels and two 32 KiB B panels in LDS)."""
+    rc, err = B.port_and_compile(GEMM_SRC, [("stepKa", "1"), ("stepKb", "1")], 160 * 1024, str(tmp_path / "gemm.o"))
+    assert rc == 0, err
+
+
+@needs_reference
+def test_reference_gemm_kernel_with_its_own_l1_sizes_is_a_compile_error(tmp_path):
+    """Unchanged, the kernel TASSIGNs 384 KiB of L1: the build stops with a [PTO][SA] message instead of overrunning LDS."""
+    rc, err = B.port_and_compile(GEMM_SRC, [], 160 * 1024, str(tmp_path / "gemm.o"))
+    assert rc != 0 and "[PTO][SA] TASSIGN" in err and "160 KiB" in err, err
+
+
+SNIPPET = r"""
+#include <hip/hip_runtime.h>
+#include <pto/pto-inst.hpp>
+#include <pto/common/constants.hpp>
+#include <pto/common/utils.hpp>
+#include <pto/common/pto_tile.hpp>
+#include <pto/common/memory.hpp>
+#include <pto/common/type.hpp>
+using namespace pto;
+PTO_DEVICE_CODE_BEGIN
+template <typename AccT, typename LeftT, typename RightT>
+AICORE inline void ByValue(AccT c, LeftT a, RightT b) { TMATMUL(c, a, b); }
+__global__ void k(float *out, half *src)
+{
+    using MatA = Tile<TileType::Mat, half, 128, 64, BLayout::ColMajor, 128, 64, SLayout::RowMajor>;
+    using MatB = Tile<TileType::Mat, half, 64, 256, BLayout::RowMajor, 64, 256, SLayout::ColMajor>;
+    MatA am; MatB bm;
+    TASSIGN(am, 0x0);
+    TASSIGN(bm, 0x0 + 128 * 64 * 2);
+    MatA am2 = am;               // Mat tiles are handles: copies are fine
+    TileLeft<half, 128, 64> a; TileRight<half, 64, 256> b; TileAcc<float, 128, 256> c;
+    GlobalTensor<half, pto::Shape<1, 1, 1, 128, 64>, pto::Stride<1, 1, 1, 64, 1>> ga(src);
+    GlobalTensor<half, pto::Shape<1, 1, 1, 64, 256>, pto::Stride<1, 1, 1, 1, 64>, Layout::DN> gb(src + 128 * 64);
+    TLOAD(am2, ga); TLOAD(bm, gb);
+    set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0); wait_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
+    TEXTRACT(a, am, 0, 0); TEXTRACT(b, bm, 0, 0);
+    ByValue(c, a, b);
+    GlobalTensor<float, pto::Shape<1, 1, 1, 128, 256>, pto::Stride<1, 1, 1, 256, 1>> gc(out);
+    TSTORE(gc, c);
+    static_assert(CeilDivision(7, 2) == 4 && CeilAlignment(7, 4) == 8, "utils.hpp");
+}
+PTO_DEVICE_CODE_END
+"""
+
+
+def test_register_tile_by_value_is_a_compile_error(tmp_path):
+    rc, err = _hipcc_snippet(tmp_path, SNIPPET)
+    assert rc != 0 and "[PTO][SA] a register tile" in err, err
+
+
+def test_register_tile_by_value_compiles_in_write_back_mode(tmp_path):
+    """With PTO_TILE_COPY_WRITEBACK the spelling of gemm_performance_kernel.cpp:28 is accepted (the copy hands its
+    values back to the tile it was copied from)."""
+    rc, err = _hipcc_snippet(tmp_path, SNIPPET, defines=["PTO_TILE_COPY_WRITEBACK=1"])
+    assert rc == 0, err
+
+
+def test_forwarding_headers_exist():
+    for name in ("pto_tile.hpp", "memory.hpp", "type.hpp", "utils.hpp", "pto_instr.hpp", "constants.hpp", "event.hpp"):
+        assert os.path.exists(os.path.join(ROOT, "include", "pto", "common", name)), name
