@@ -13,17 +13,24 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libpto_amd.so")
-SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_mx.hip", "pto_elementwise.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_fa_w8m16.hip", "pto_optest.hip"]
+# libpto_st.so: the same sources with the tuning hooks compiled in (PTO_ST_HOOKS) plus the single-tile test programs; what
+# the parity tests load to drive single instructions and kernel variants.  Not part of the product.
+OUT_ST = os.path.join(HERE, "libpto_st.so")
+SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_mx.hip", "pto_elementwise.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_fa_w8m16.hip"]
+ST_ONLY_SOURCES = ["pto_optest.hip"]
+# sources of libpto_st.so that differ from the product's objects (they hold a hook); the others are linked as they are
+HOOK_SOURCES = ["pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_mx.hip", "pto_fa.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC,
          # packed-fp32 VALU forms are kept off for every device function
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unknown-warning-option"]
 
 
-def _compile(src):
-    obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+def _compile(job):
+    src, st = job
+    obj = os.path.join(HERE, "build", ("st_" if st else "") + src.replace(".hip", ".o"))
     os.makedirs(os.path.dirname(obj), exist_ok=True)
-    cmd = [HIPCC] + FLAGS + ["-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC] + FLAGS + (["-DPTO_ST_HOOKS=1"] if st else []) + ["-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and "is not a recognized feature" not in l)
     if r.returncode != 0:
@@ -32,14 +39,17 @@ def _compile(src):
 
 
 def build(verbose=True):
-    srcs = [s for s in SOURCES if os.path.exists(os.path.join(CSRC, s))]
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as ex:
-        objs = list(ex.map(_compile, srcs))
-    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", OUT] + objs, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed:\n" + r.stderr)
-    if verbose:
-        print("built", OUT)
+    jobs = [(s, False) for s in SOURCES] + [(s, True) for s in HOOK_SOURCES + ST_ONLY_SOURCES]
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        objs = dict(zip(jobs, ex.map(_compile, jobs)))
+    product = [objs[(s, False)] for s in SOURCES]
+    st = [objs[(s, s in HOOK_SOURCES)] for s in SOURCES] + [objs[(s, True)] for s in ST_ONLY_SOURCES]
+    for out, group in ((OUT, product), (OUT_ST, st)):
+        r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + group, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("link failed:\n" + r.stderr)
+        if verbose:
+            print("built", out)
     build_host(verbose)
     return OUT
 

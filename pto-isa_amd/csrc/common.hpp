@@ -3,6 +3,9 @@
 #include <hip/hip_runtime.h>
 
 #include "pto_amd.h"
+#if defined(PTO_ST_HOOKS)
+#include "pto_amd_st.h" // test-only entry points (libpto_st.so)
+#endif
 
 namespace pto_amd {
 extern thread_local int g_last_hip_error;

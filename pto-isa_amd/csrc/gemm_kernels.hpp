@@ -51,7 +51,7 @@ AICORE inline void TileOfBlock(int block, int tilesM, int tilesN, int &tm, int &
     TileOfId<GROUP_M>(RegroupXcd(block, tilesM * tilesN), tilesM, tilesN, tm, tn);
 }
 
-template <int BM, int BN, int BK, int STAGES, int MIN_BLOCKS, int GROUP_M, int MODE = 0>
+template <int BM, int BN, int BK, int STAGES, int MIN_BLOCKS, int GROUP_M>
 __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
     void GemmF16F32(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k)
 {
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
                 else
                     wait_flag(PIPE_MTE2, PIPE_MTE1, static_cast<event_t>(s));
                 const int nxt = it + STAGES - 1;
-                if (MODE != 2 && nxt < kLoop) {
+                if (nxt < kLoop) {
                     const int ns = (s + STAGES - 1) % STAGES;
                     GlobalA gmA(aPanel + (int64_t)nxt * BK, ShapeA(), strideA);
                     GlobalB gmB(bPanel + (int64_t)nxt * BK, ShapeB(), strideB);
@@ -126,17 +126,15 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE
                     TLOAD(bMat[ns], gmB);
                     set_flag(PIPE_MTE2, PIPE_MTE1, static_cast<event_t>(ns));
                 }
-                if (MODE != 1 || it == 0) {
-                    TEXTRACT(aTile, aMat[s], 0, 0);
-                    TEXTRACT(bTile, bMat[s], 0, 0);
-                    set_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
-                    wait_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
-                    if (it == 0)
-                        TMATMUL(cTile, aTile, bTile);
-                    else
-                        TMATMUL_ACC(cTile, cTile, aTile, bTile);
-                    set_flag(PIPE_M, PIPE_MTE1, EVENT_ID0);
-                }
+                TEXTRACT(aTile, aMat[s], 0, 0);
+                TEXTRACT(bTile, bMat[s], 0, 0);
+                set_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+                wait_flag(PIPE_MTE1, PIPE_M, EVENT_ID0);
+                if (it == 0)
+                    TMATMUL(cTile, aTile, bTile);
+                else
+                    TMATMUL_ACC(cTile, cTile, aTile, bTile);
+                set_flag(PIPE_M, PIPE_MTE1, EVENT_ID0);
             }
         }
     }
@@ -470,13 +468,13 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE void GemmZeroTailTiles(__g
 PTO_DEVICE_CODE_END
 
 namespace {
-template <int BM, int BN, int BK, int STAGES, int MIN_BLOCKS, int GROUP_M, int MODE = 0>
+template <int BM, int BN, int BK, int STAGES, int MIN_BLOCKS, int GROUP_M>
 int launch_gemm(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k)
 {
     if (m % BM || n % BN || k % BK)
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = STAGES * (BM * BK + BK * BN) * (int)sizeof(half);
-    auto kernel = GemmF16F32<BM, BN, BK, STAGES, MIN_BLOCKS, GROUP_M, MODE>;
+    auto kernel = GemmF16F32<BM, BN, BK, STAGES, MIN_BLOCKS, GROUP_M>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;

@@ -25,6 +25,7 @@
 
 #include "fa_kernels.hpp"
 
+#if defined(PTO_ST_HOOKS)
 // Tuning hook (not part of the public header).
 extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k,
                                       const uint16_t *v, int batch, int heads, int seq_q, int seq_kv, int head_dim,
@@ -60,6 +61,7 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
         return launch_fa<64, true, false, 3, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     return PTO_ERR_BAD_ARG;
 }
+#endif // PTO_ST_HOOKS
 
 extern "C" int pto_fa_fwd_f16(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,
                               int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int o_fp32)

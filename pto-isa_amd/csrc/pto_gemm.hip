@@ -11,6 +11,7 @@
 // instead of a 24-core loop nest, and an XCD-aware block -> tile map.
 #include "gemm_kernels.hpp"
 
+#if defined(PTO_ST_HOOKS)
 // Tuning hook (not part of the public header): the same GEMM with another tiling / pipeline depth.
 extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
                                        int variant)
@@ -39,14 +40,10 @@ extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a
     case 35: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 3);
     case 36: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 3);
     case 34: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 0);
-    case 105: return launch_gemm<256, 256, 64, 2, 1, 8, 1>(st, c, ha, hb, m, n, k); // loads only, 128-byte rows
-    case 103: return launch_gemm<256, 256, 32, 4, 1, 8, 1>(st, c, ha, hb, m, n, k); // loads only
-    case 104: return launch_gemm<256, 256, 32, 4, 1, 8, 2>(st, c, ha, hb, m, n, k); // compute only
-    case 101: return launch_gemm<128, 256, 32, 3, 2, 8, 1>(st, c, ha, hb, m, n, k); // loads only
-    case 102: return launch_gemm<128, 256, 32, 3, 2, 8, 2>(st, c, ha, hb, m, n, k); // compute only
     default: return PTO_ERR_BAD_ARG;
     }
 }
+#endif // PTO_ST_HOOKS
 
 extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k)
 {

@@ -35,6 +35,7 @@ int gemm_f16f32_tile384x192_w8(hipStream_t st, float *c, const _Float16 *a, cons
 }
 } // namespace pto_amd
 
+#if defined(PTO_ST_HOOKS)
 extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
                                            int variant)
 {
@@ -53,3 +54,4 @@ extern "C" int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_
     default: return PTO_ERR_BAD_ARG;
     }
 }
+#endif // PTO_ST_HOOKS

@@ -202,6 +202,7 @@ int gemm_f16f32_tile256_w4(hipStream_t st, float *c, const _Float16 *a, const _F
 }
 } // namespace pto_amd
 
+#if defined(PTO_ST_HOOKS)
 extern "C" int pto_gemm_f16f32_m16w4_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
                                              int variant)
 {
@@ -218,3 +219,4 @@ extern "C" int pto_gemm_f16f32_m16w4_variant(void *stream, float *c, const uint1
     default: return PTO_ERR_BAD_ARG;
     }
 }
+#endif // PTO_ST_HOOKS

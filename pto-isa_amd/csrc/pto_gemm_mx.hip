@@ -356,6 +356,7 @@ extern "C" int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uin
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, 4, c_fp32, 1);
 }
 
+#if defined(PTO_ST_HOOKS)
 // Tuning hook (not part of the public header): variant bit 0 = quarter tiles in the last round, bit 1 = the shallower copy
 // pipeline; format 0 / 1 = fp8 e4m3 / e5m2, 4 = fp4 e2m1.
 extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
@@ -365,3 +366,4 @@ extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, c
         return PTO_ERR_BAD_ARG;
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, variant);
 }
+#endif // PTO_ST_HOOKS

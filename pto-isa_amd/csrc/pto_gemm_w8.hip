@@ -8,6 +8,7 @@ namespace pto_amd {
 int gemm_compute_units() { return compute_units(); }
 } // namespace pto_amd
 
+#if defined(PTO_ST_HOOKS)
 extern "C" int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k,
                                           int variant)
 {
@@ -28,3 +29,4 @@ extern "C" int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t
     default: return PTO_ERR_BAD_ARG;
     }
 }
+#endif // PTO_ST_HOOKS

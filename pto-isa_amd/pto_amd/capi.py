@@ -28,6 +28,18 @@ SYMBOLS = {
     "pto_tcvt_f32_bf16": (C.c_int, [C.c_void_p] * 3 + [C.c_size_t, C.c_int]),
     "pto_gather_rows": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t] * 3 + [C.c_int]),
     "pto_tgather_index_f16_16x1024_16x128": (C.c_int, [C.c_void_p] * 4),
+}
+
+# Test-only library (include/pto_amd_st.h): single-tile programs and tuning hooks, on top of every product symbol.
+ST_LIB_PATH = os.path.join(_HERE, "libpto_st.so")
+_V = [C.c_void_p] * 4 + [C.c_int] * 4
+ST_SYMBOLS = {
+    "pto_gemm_f16f32_variant": (C.c_int, _V),
+    "pto_gemm_f16f32_w8_variant": (C.c_int, _V),
+    "pto_gemm_f16f32_m16_variant": (C.c_int, _V),
+    "pto_gemm_f16f32_m16w4_variant": (C.c_int, _V),
+    "pto_gemm_mxfp8_variant": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 6),
+    "pto_fa_fwd_f16_variant": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 7),
     "pto_st_softmax_step_f32_64x256": (C.c_int, [C.c_void_p] * 8 + [C.c_float, C.c_int, C.c_int]),
     "pto_st_gu_step_f32_64x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int]),
     "pto_st_tri_mask_f32_64x128": (C.c_int, [C.c_void_p] * 3 + [C.c_int, C.c_float, C.c_int]),
@@ -60,6 +72,7 @@ SYMBOLS = {
 }
 
 _lib = None
+_st_lib = None
 
 
 def load():
@@ -75,6 +88,22 @@ def load():
             fn.argtypes = args
         _lib = lib
     return _lib
+
+
+def load_st():
+    """Load the test-only library and declare every symbol of include/pto_amd_st.h (and of pto_amd.h: it holds the
+    product's entry points too, so a test can drive both through one handle)."""
+    global _st_lib
+    if _st_lib is None:
+        if not os.path.exists(ST_LIB_PATH):
+            raise RuntimeError("libpto_st.so is not built: run `python pto-isa_amd/build.py`")
+        lib = C.CDLL(ST_LIB_PATH)
+        for name, (res, args) in list(SYMBOLS.items()) + list(ST_SYMBOLS.items()):
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _st_lib = lib
+    return _st_lib
 
 
 class PtoError(RuntimeError):

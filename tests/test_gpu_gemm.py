@@ -49,9 +49,7 @@ def test_gemm_four_wave_tile_shapes_exact():
     import ctypes as C
     import torch
     from gpu_util import to_dev
-    lib = capi.load()
-    fn = lib.pto_gemm_f16f32_m16w4_variant
-    fn.restype, fn.argtypes = C.c_int, [C.c_void_p] * 4 + [C.c_int] * 4
+    fn = capi.load_st().pto_gemm_f16f32_m16w4_variant
     for m, n, k in ((768, 1536, 512), (4352, 4096, 256)):
         a, b = datagen.gemm_inputs_integer(m, n, k)
         want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
@@ -73,9 +71,7 @@ def test_gemm_eight_wave_tile_shapes_exact():
     import ctypes as C
     import torch
     from gpu_util import to_dev
-    lib = capi.load()
-    fn = lib.pto_gemm_f16f32_m16_variant
-    fn.restype, fn.argtypes = C.c_int, [C.c_void_p] * 4 + [C.c_int] * 4
+    fn = capi.load_st().pto_gemm_f16f32_m16_variant
     for m, n, k in ((768, 768, 512), (1536, 2304, 256)):
         a, b = datagen.gemm_inputs_integer(m, n, k)
         want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)

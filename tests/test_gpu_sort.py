@@ -26,7 +26,7 @@ def _st():
 
 @pytest.mark.parametrize("dtype,vr,vc,seed", sc.SORT32_CASES)
 def test_tsort32(oracle, dtype, vr, vc, seed):
-    lib = capi.load()
+    lib = capi.load_st()
     src, idx, out0 = sc.sort32_inputs(dtype, vr, vc, seed)
     ts, ti, to = _dev(src), _dev(idx), _dev(out0)
     capi.check(lib.pto_st_tsort32_8x128(_st(), to.data_ptr(), ts.data_ptr(), ti.data_ptr(), vr, vc, 0 if dtype == "f32" else 1), "tsort32")
@@ -42,7 +42,7 @@ def test_tsort32(oracle, dtype, vr, vc, seed):
 
 @pytest.mark.parametrize("valid_cols,block_len,seed", sc.BLOCK_CASES)
 def test_tmrgsort_blocks(oracle, valid_cols, block_len, seed):
-    lib = capi.load()
+    lib = capi.load_st()
     src, out0 = sc.block_inputs(valid_cols, block_len, seed)
     ts, to = _dev(src), _dev(out0)
     capi.check(lib.pto_st_tmrgsort_blocks_f32_1x1024(_st(), to.data_ptr(), ts.data_ptr(), valid_cols, block_len), "tmrgsort blocks")
@@ -54,7 +54,7 @@ def test_tmrgsort_blocks(oracle, valid_cols, block_len, seed):
 
 @pytest.mark.parametrize("counts,out_structs,exhausted,seed", sc.LIST_CASES)
 def test_tmrgsort_lists(oracle, counts, out_structs, exhausted, seed):
-    lib = capi.load()
+    lib = capi.load_st()
     lists, out0 = sc.list_inputs(counts, seed)
     tl = [_dev(l) for l in lists]
     to = _dev(out0)
@@ -73,7 +73,7 @@ def test_tmrgsort_lists(oracle, counts, out_structs, exhausted, seed):
 
 @pytest.mark.parametrize("n", range(len(sc.PART_CASES)))
 def test_tpart(oracle, n):
-    lib = capi.load()
+    lib = capi.load_st()
     op, dv, av, bv = sc.PART_CASES[n]
     a, b, out0 = sc.part_inputs(n)
     ta, tb, to = _dev(a), _dev(b), _dev(out0)
@@ -86,7 +86,7 @@ def test_tpart(oracle, n):
 
 @pytest.mark.parametrize("n", range(len(sc.SCATTER_CASES)))
 def test_tscatter_and_mscatter(oracle, n):
-    lib = capi.load()
+    lib = capi.load_st()
     vr, vc, kind = sc.SCATTER_CASES[n]
     src, idx, out0 = sc.scatter_inputs(vr, vc, kind, n)
     ts, ti, to = _dev(src), _dev(idx), _dev(out0)
@@ -106,7 +106,7 @@ def test_tscatter_and_mscatter(oracle, n):
 
 @pytest.mark.parametrize("n", range(len(sc.GATHERB_CASES)))
 def test_tgatherb(oracle, n):
-    lib = capi.load()
+    lib = capi.load_st()
     vr, vc, kind = sc.GATHERB_CASES[n]
     src, off, out0 = sc.gatherb_inputs(kind, n)
     ts, tf, to = _dev(src), _dev(off), _dev(out0)
@@ -119,7 +119,7 @@ def test_tgatherb(oracle, n):
 
 @pytest.mark.parametrize("n", range(len(sc.CI_CASES)))
 def test_tci(oracle, n):
-    lib = capi.load()
+    lib = capi.load_st()
     start, desc, vc = sc.CI_CASES[n]
     out0 = np.full(1024, -5, dtype=np.int32)
     to = _dev(out0)
@@ -130,7 +130,7 @@ def test_tci(oracle, n):
 
 
 def test_sort_programs_reject_bad_arguments():
-    lib = capi.load()
+    lib = capi.load_st()
     p = torch.zeros(2048, device="cuda:0").data_ptr()
     assert lib.pto_st_tsort32_8x128(0, p, p, p, 9, 32, 0) == capi.ERR_BAD_ARG
     assert lib.pto_st_tpart_f32_64x128(0, p, p, p, 3, 64, 128, 64, 128, 64, 128) == capi.ERR_BAD_ARG

@@ -46,7 +46,7 @@ def softmax_step_oracle(oracle, x, m_in, s_in, scale, first, ties_away):
 @pytest.mark.parametrize("first", [1, 0])
 @pytest.mark.parametrize("mode", [capi.CAST_RINT, capi.CAST_ROUND])
 def test_softmax_step(oracle, first, mode):
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(3 + first)
     x = (rng.standard_normal((64, 256)) * 4).astype(np.float32)
     m_in = (rng.standard_normal(64) * 2 + 6).astype(np.float32)      # some rows keep the old max, some raise it
@@ -70,7 +70,7 @@ def test_softmax_step(oracle, first, mode):
 
 @pytest.mark.parametrize("last", [0, 1])
 def test_gu_step(last):
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(5)
     o = rng.standard_normal((64, 128)).astype(np.float32)
     pv = rng.standard_normal((64, 128)).astype(np.float32)
@@ -93,7 +93,7 @@ def test_gu_step(last):
 
 @pytest.mark.parametrize("upper,diag", [(1, 1), (1, 37), (1, -5), (0, 0), (0, 20)])
 def test_tri_mask(oracle, upper, diag):
-    lib = capi.load()
+    lib = capi.load_st()
     x = np.random.default_rng(7).standard_normal((64, 128)).astype(np.float32)
     out = torch.zeros((64, 128), device=DEV)
     tx = dev(x)
@@ -109,7 +109,7 @@ def test_tri_mask(oracle, upper, diag):
                                             (4, slice(1, None, 4), 4), (5, slice(2, None, 4), 4), (6, slice(3, None, 4), 4),
                                             (7, slice(None), 1)])
 def test_tgather_mask(oracle, pattern, sl, div):
-    lib = capi.load()
+    lib = capi.load_st()
     src = np.random.default_rng(pattern).integers(0, 2**16, size=(16, 64), dtype=np.uint16)
     out = torch.zeros((16, 64 // div), dtype=torch.int16, device=DEV)
     tsrc = dev(src)
@@ -122,7 +122,7 @@ def test_tgather_mask(oracle, pattern, sl, div):
 
 
 def test_mgather_elements(oracle):
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(11)
     gm = rng.integers(0, 2**16, size=65536, dtype=np.uint16)
     idx = rng.integers(0, 65536, size=(8, 128), dtype=np.int32)
@@ -134,7 +134,7 @@ def test_mgather_elements(oracle):
 
 
 def test_tload_pad_and_valid_region(oracle):
-    lib = capi.load()
+    lib = capi.load_st()
     x = np.arange(200, dtype=np.float32)
     img = torch.zeros((16, 32), device=DEV)
     tx = dev(x)
@@ -146,7 +146,7 @@ def test_tload_pad_and_valid_region(oracle):
 
 
 def test_tload_tstore_5d(oracle):
-    lib = capi.load()
+    lib = capi.load_st()
     gm = np.arange(2000, dtype=np.float32)
     dense = torch.zeros((24, 8), device=DEV)
     strided = torch.full((2000,), -1.0, device=DEV)
@@ -165,7 +165,7 @@ def test_tload_tstore_5d(oracle):
 def test_textract_windows(oracle, col0, row0):
     """dst[i,j] = src[r0+i, c0+j] for windows that are not the suffix (the reference CPU simulation only
     takes the suffix; the ISA definition is the oracle's mode 1)."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(13)
     a = rng.integers(-8, 8, size=(128, 256)).astype(np.float16)
     b = rng.integers(-8, 8, size=(256, 256)).astype(np.float16)      # logical [k, n]
@@ -194,7 +194,7 @@ def test_textract_windows(oracle, col0, row0):
 @pytest.mark.parametrize("bf16", [0, 1])
 @pytest.mark.parametrize("with_bias", [0, 1])
 def test_matmul_bias_and_bf16(oracle, bf16, with_bias):
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(17)
     a = rng.integers(1, 5, size=(128, 64)).astype(np.float32)
     b = rng.integers(1, 5, size=(64, 256)).astype(np.float32)
@@ -227,7 +227,7 @@ def test_matmul_bias_and_bf16(oracle, bf16, with_bias):
 def test_tpush_tpop_pipeline(lds_fifo):
     """Accumulator -> FIFO -> Vec tile and Vec -> FIFO -> Mat tile hand-offs; integer-valued data, so every
     product, sum and the fp16 cast are exact and the result must equal numpy's."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(31 + lds_fifo)
     a = rng.integers(-2, 3, size=(64, 64)).astype(np.float32)
     b = rng.integers(-2, 3, size=(2, 64, 128)).astype(np.float32)
@@ -263,7 +263,7 @@ def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b, via_lds):
     scale tiles loaded from memory (MX_A_ND / MX_B_DN) and windowed, or staged in Mat tiles of block scales and
     TEXTRACTed: exact on integer operands, <= 2e-3 on random ones."""
     from pto_amd import datagen
-    lib = capi.load()
+    lib = capi.load_st()
     for dist, lo, hi in (("integer", 125, 130), ("uniform", 120, 135), ("bytes", 110, 140)):
         a, _, sa, _ = datagen.mx_inputs(128, 128, 256, fmt_a, dist=dist, scale_lo=lo, scale_hi=hi)
         _, b, _, sb = datagen.mx_inputs(128, 128, 256, fmt_b, dist=dist, scale_lo=lo, scale_hi=hi)
@@ -282,7 +282,7 @@ def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b, via_lds):
 
 def test_tmatmul_int8_to_int32(oracle):
     """int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), TMATMUL then TMATMUL_ACC over two k halves: exact."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(23)
     a = rng.integers(-128, 128, size=(128, 128), dtype=np.int8)
     b = rng.integers(-128, 128, size=(128, 256), dtype=np.int8)
@@ -311,7 +311,7 @@ def test_tmatmul_int8_to_int32(oracle):
 
 def test_tmatmul_fp32(oracle):
     """fp32 x fp32 -> fp32 (v_mfma_f32_32x32x2_f32): exact on integers, fp32 rounding only otherwise."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(29)
     for integer in (True, False):
         if integer:

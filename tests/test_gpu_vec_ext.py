@@ -32,7 +32,7 @@ def ulp_diff(a, b):
 
 @pytest.mark.parametrize("op", ALL_OPS)
 def test_vec_op(oracle, op):
-    lib = capi.load()
+    lib = capi.load_st()
     a, b, vec, k = vec_inputs(op)
     ta, tb = dev(a), dev(b)
     tv = dev(vec) if vec is not None else None
@@ -49,7 +49,7 @@ def test_vec_op(oracle, op):
 
 
 def test_vec_op_bad_code():
-    lib = capi.load()
+    lib = capi.load_st()
     out = torch.zeros((64, 128), device=DEV)
     assert lib.pto_st_vec_op_f32_64x128(st(), out.data_ptr(), out.data_ptr(), out.data_ptr(), 0, 0.0, 999) == capi.ERR_BAD_ARG
 
@@ -57,7 +57,7 @@ def test_vec_op_bad_code():
 @pytest.mark.parametrize("op", range(6))
 @pytest.mark.parametrize("shape", REDUCE_SHAPES)
 def test_reduce(oracle, op, shape):
-    lib = capi.load()
+    lib = capi.load_st()
     vr, vc = shape
     full = reduce_inputs()
     ta = dev(full)
@@ -77,7 +77,7 @@ def test_reduce(oracle, op, shape):
 
 @pytest.mark.parametrize("mode", range(6))
 def test_cmps_sel(oracle, mode):
-    lib = capi.load()
+    lib = capi.load_st()
     a, b, _, _ = vec_inputs("CMP_EQ", seed=mode)
     scalar = np.float32(a[3, 5])
     a[::7, ::3] = scalar
@@ -97,7 +97,7 @@ def test_cmps_sel(oracle, mode):
 @pytest.mark.parametrize("pad_kind", [1, 2, 3])
 @pytest.mark.parametrize("shape", [(64, 128), (10, 20), (64, 5), (1, 1)])
 def test_fillpad(oracle, pad_kind, shape):
-    lib = capi.load()
+    lib = capi.load_st()
     vr, vc = shape
     a = reduce_inputs(3)
     ta = dev(a)
@@ -109,7 +109,7 @@ def test_fillpad(oracle, pad_kind, shape):
 
 @pytest.mark.parametrize("relu", [0, 1])
 def test_matmul_tmov_acc_to_vec(oracle, relu):
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(21)
     a = rng.integers(-4, 5, size=(64, 64)).astype(np.float32)     # integer values: the fp32 products and sums are exact
     b = rng.integers(-4, 5, size=(64, 128)).astype(np.float32)
@@ -141,7 +141,7 @@ TYPED_OPS = {
 def test_vec_op_fp16_and_int32(oracle, op, dtype):
     """The arithmetic Vec instructions on fp16 tiles (one IEEE rounding per operation, as numpy's float16) and on int32
     tiles (wrap-around arithmetic): bit-exact."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(101 + len(op))
     if dtype == "f16":
         a = (rng.standard_normal((64, 128)) * 8).astype(np.float16)
@@ -188,7 +188,7 @@ def c_rem(a, b):
 def test_vec_bitwise_shift_rem_carry(op, dtype):
     """TAND .. TSUBSC against numpy's integer / float rules (wrap-around int32; shifts by 0..31, arithmetic right
     shift; remainder with the dividend's sign; a + b + c evaluated left to right in the element type): bit-exact."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(300 + BIT_OPS.index(op))
     if dtype == "s32":
         a = rng.integers(-2**31, 2**31, size=(64, 128), dtype=np.int64).astype(np.int32)
@@ -227,7 +227,7 @@ def test_vec_bitwise_shift_rem_carry(op, dtype):
 
 
 def test_vec_bitop_rejects_bad_arguments():
-    lib = capi.load()
+    lib = capi.load_st()
     t = torch.zeros((64, 128), dtype=torch.int32, device=DEV)
     p = t.data_ptr()
     assert lib.pto_st_vec_bitop_64x128(st(), p, p, p, p, 0.0, 0, 17, 1) == capi.ERR_BAD_ARG
@@ -238,7 +238,7 @@ def test_vec_bitop_rejects_bad_arguments():
 def test_ttrans_and_tmov_to_operands():
     """TTRANS is a permutation (bit-exact); TMOV Vec -> Left / Right and Acc -> Left feed matmuls whose small-integer
     inputs make every product and sum exact in fp16 / fp32."""
-    lib = capi.load()
+    lib = capi.load_st()
     rng = np.random.default_rng(55)
     x = rng.standard_normal((64, 128)).astype(np.float32)
     x[0, :3] = [np.nan, np.inf, -0.0]
