@@ -2,6 +2,8 @@
 // events to wait on (reference: include/pto/common/event.hpp:19-140, npu/a2a3/TSync.hpp:137-226).
 // On gfx950 an Event between two pipes reduces to the wait_flag rule of that pipe pair.
 #pragma once
+#include <type_traits>
+#include <utility>
 #include "pto/gfx950/platform.hpp"
 
 namespace pto {
@@ -50,6 +52,13 @@ struct Event {
     }
     PTO_DEV Event &operator=(RecordEvent) { return Record(); }
 };
+
+// true for the types an instruction may take after its operands: anything with a Wait() member (event.hpp:136-140 of the
+// reference waits on each of them)
+template <typename T, typename = void>
+struct is_wait_event : std::false_type {};
+template <typename T>
+struct is_wait_event<T, std::void_t<decltype(std::declval<T &>().Wait())>> : std::true_type {};
 
 template <typename... WaitEvents>
 PTO_DEV void WaitAllEvents(WaitEvents &... events)

@@ -280,7 +280,9 @@ PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
     TSTORE_IMPL<TileT, G, atomic, relu>(dst, src);
     return {};
 }
-template <typename D, typename S, typename... Ev>
+// the form without indices; index arguments that are lvalues (`TEXTRACT(dst, src, row, col)` with int variables) must
+// not be taken for events
+template <typename D, typename S, typename... Ev, std::enable_if_t<(is_wait_event<Ev>::value && ...), int> = 0>
 PTO_INST RecordEvent TEXTRACT(D &dst, S &src, Ev &... ev)
 {
     TSYNC(ev...);

@@ -24,6 +24,9 @@ int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_t *a, const
 /* four wavefronts on 16 x 16 x 32 MFMAs: 0 / 1 = 256 x 256 with / without quarter tiles, 2 = 192 x 256, 3 = 256 x 192,
  * 4 = 192 x 192 (csrc/pto_gemm_m16w4.hip) */
 int pto_gemm_f16f32_m16w4_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
+/* eight wavefronts on a 4 x 2 wave grid, K-steps of 64 (whole 128-byte lines), two LDS stages: 0 = 384 x 192 tiles,
+ * 1 = 256 x 256, 2 = 256 x 192 (csrc/pto_gemm_k64.hip) */
+int pto_gemm_f16f32_k64_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
 /* MX GEMM: variant bit 0 = quarter tiles in the last round, bit 1 = the shallower copy pipeline (csrc/pto_gemm_mx.hip) */
 int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                            const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant);

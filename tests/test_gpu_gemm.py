@@ -83,8 +83,26 @@ def test_gemm_eight_wave_tile_shapes_exact():
             assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
 
 
+def test_gemm_k64_tile_shapes_exact():
+    """Every tile shape of the kernel with K-steps of 64 (384 x 192 = the kernel that the 6144 x 6144 problem selects,
+    256 x 256, 256 x 192) on integer inputs, two and six K-steps: the whole matrix, exactly; and an unsupported K."""
+    import torch
+    from gpu_util import to_dev
+    fn = capi.load_st().pto_gemm_f16f32_k64_variant
+    for m, n, k in ((768, 768, 128), (1536, 2304, 384)):
+        a, b = datagen.gemm_inputs_integer(m, n, k)
+        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
+        ta, tb = to_dev(a), to_dev(b)
+        for variant in (0, 1, 2):
+            tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "K-64 GEMM variant %d" % variant)
+            torch.cuda.synchronize()
+            assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
+        assert fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k + 64, 0) == capi.ERR_UNSUPPORTED
+
+
 def test_gemm_6144_every_element_exact():
-    """The headline problem through the public entry point (it selects the 384 x 192-tile kernel) on integer operands in
+    """The headline problem through the public entry point (it selects the 384 x 192-tile kernel with K-steps of 64) on integer operands in
     [1, 5): all 6144 x 6144 sums (at most 16 * 6144 < 2^24) are exact in fp32, so every element must equal the product
     taken in float64 by the BLAS behind torch (an independent code path)."""
     import torch
