@@ -38,12 +38,41 @@ PTO_INST std::enable_if_t<is_tile_data_v<T>> TASSIGN(T &obj)
     TASSIGN_IMPL(obj, Addr);
 }
 
+namespace detail {
+// Vec tiles in memory (PTO_VEC_TILES_IN_MEMORY): an instruction loads the valid region of every Vec tile among its
+// operands from the unified buffer into the tile's registers (UbFetch), runs on the registers, and writes the valid
+// region of its destination, the first operand, back (UbCommit), after which the stores are drained and the workgroup
+// meets at a barrier: the next instruction, in any wave, sees the result.  Other translation units: nothing.
+template <typename T>
+PTO_DEV void UbFetchOne(T &t)
+{
+    if constexpr (is_tile_data_v<T>) {
+        static_assert(!(T::inMemory && T::isBoxedLayout), "[PTO][SA] Vec tiles in memory: plain row-major or column-major tiles");
+        UbFetchTile(t);
+    }
+}
+template <typename... Ts>
+PTO_DEV void UbFetch(Ts &... ts)
+{
+    (UbFetchOne(ts), ...);
+}
+PTO_DEV void UbFetch() {}
+template <typename T, typename... Rest>
+PTO_DEV void UbCommit(T &dst, Rest &...)
+{
+    if constexpr (is_tile_data_v<T>)
+        UbCommitTile(dst);
+}
+} // namespace detail
+
 #define PTO_FRONT(NAME, TPARAMS, PARAMS, ARGS)          \
     template <TPARAMS, typename... Ev>                  \
     PTO_INST RecordEvent NAME(PARAMS, Ev &... ev)       \
     {                                                   \
         TSYNC(ev...);                                   \
+        detail::UbFetch ARGS;                           \
         NAME##_IMPL ARGS;                               \
+        detail::UbCommit ARGS;                          \
         return {};                                      \
     }
 #define PTO_C ,
@@ -75,7 +104,6 @@ PTO_FRONT(TMAXS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename
 PTO_FRONT(TMINS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TEXP, typename T, T &dst PTO_C T &src, (dst, src))
 PTO_FRONT(TEXPANDS, typename T, T &dst PTO_C typename T::DType k, (dst, k))
-PTO_FRONT(TRESHAPE, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TROWMAX, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
 PTO_FRONT(TROWSUM, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
 PTO_FRONT(TROWEXPANDSUB, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
@@ -154,6 +182,48 @@ PTO_FRONT(TPUSH, typename P PTO_C typename T PTO_C typename F, P &prod PTO_C T &
 PTO_FRONT(TPOP, typename P PTO_C typename T PTO_C typename F, P &cons PTO_C T &tile PTO_C F &fifo, (cons, tile, fifo))
 #undef PTO_FRONT
 #undef PTO_C
+// the forms that name the pipe (pto_instr.hpp:1442-1471 of the reference)
+template <typename TileData, typename Pipe, typename... Ev, std::enable_if_t<is_tile_data_v<TileData>, int> = 0>
+PTO_INST RecordEvent TPUSH(TileData &tile, Pipe &pipe, Ev &... ev)
+{
+    TSYNC(ev...);
+    TPUSH_IMPL(tile, pipe);
+    return {};
+}
+template <typename TileData, typename Pipe, typename... Ev, std::enable_if_t<is_tile_data_v<TileData>, int> = 0>
+PTO_INST RecordEvent TPOP(TileData &tile, Pipe &pipe, Ev &... ev)
+{
+    TSYNC(ev...);
+    TPOP_IMPL(tile, pipe);
+    return {};
+}
+template <typename Pipe, typename... Ev>
+PTO_INST RecordEvent TFREE(Pipe &pipe, Ev &... ev)
+{
+    TSYNC(ev...);
+    TFREE_IMPL(pipe);
+    return {};
+}
+
+// TRESHAPE (pto_instr.hpp:998 of the reference): the same storage under another shape.  Register tiles: a copy of the
+// registers (both shapes have the same distribution).  Vec tiles in memory: dst becomes a VIEW of src's storage, as on a
+// machine where the tile is an address (the reference's softmax stage writes a [R,1] tile through its [1,R] view).
+template <typename D, typename S, typename... Ev>
+PTO_INST RecordEvent TRESHAPE(D &dst, S &src, Ev &... ev)
+{
+    TSYNC(ev...);
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+    if constexpr (D::inMemory && S::inMemory) {
+        static_assert(D::Numel * sizeof(typename D::DType) == S::Numel * sizeof(typename S::DType), "[PTO][SA] TRESHAPE: same storage size");
+        if (src.mem_ != nullptr) {
+            dst.mem_ = reinterpret_cast<typename D::DType *>(src.mem_);
+            return {};
+        }
+    }
+#endif
+    TRESHAPE_IMPL(dst, src);
+    return {};
+}
 
 // TMOV (pto_instr.hpp:881-940): Mat -> Left / Right, register tile copies, and accumulator -> Vec with an
 // optional clamp at zero; the split mode over Vec cores is an Ascend hint
@@ -161,12 +231,14 @@ template <typename D, typename S, ReluPreMode relu = ReluPreMode::NoRelu, typena
 PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src);
     if constexpr (S::Loc == TileType::Acc && D::Loc == TileType::Vec)
         TMOV_ACC2VEC_IMPL<relu>(dst, src);
     else if constexpr ((S::Loc == TileType::Acc || S::Loc == TileType::Vec) && (D::Loc == TileType::Left || D::Loc == TileType::Right))
         TMOV_TO_OPERAND_IMPL(dst, src); // the chained matmuls of the Auto-mode programs
     else
         TMOV_IMPL(dst, src);
+    detail::UbCommit(dst);
     return {};
 }
 // TTRANS (pto_instr.hpp:1032 of the reference): the scratch tile is accepted and ignored
@@ -241,6 +313,7 @@ template <typename TileT, typename G, typename... Ev>
 PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(src);
     TSTORE_IMPL<TileT, G, AtomicType::AtomicNone>(dst, src);
     return {};
 }
@@ -248,6 +321,7 @@ template <STPhase Phase, typename TileT, typename G, typename... Ev>
 PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
 { // the unit-flag phase is an Ascend fix-pipe hint; a store is a store here
     TSYNC(ev...);
+    detail::UbFetch(src);
     TSTORE_IMPL<TileT, G, AtomicType::AtomicNone>(dst, src);
     return {};
 }
@@ -255,6 +329,7 @@ template <typename TileT, typename G, AtomicType atomic, typename... Ev>
 PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(src);
     TSTORE_IMPL<TileT, G, atomic>(dst, src);
     return {};
 }
@@ -263,6 +338,7 @@ template <typename TileT, typename G, AtomicType atomic, STPhase Phase, typename
 PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(src);
     TSTORE_IMPL<TileT, G, atomic>(dst, src);
     return {};
 }
@@ -270,6 +346,7 @@ template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu, typen
 PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(src);
     TSTORE_IMPL<TileT, G, atomic, relu>(dst, src);
     return {};
 }
@@ -277,6 +354,7 @@ template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu, STPha
 PTO_INST RecordEvent TSTORE(G &dst, TileT &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(src);
     TSTORE_IMPL<TileT, G, atomic, relu>(dst, src);
     return {};
 }
@@ -330,21 +408,27 @@ template <typename D, typename S, typename... Ev>
 PTO_INST RecordEvent TCVT(D &dst, S &src, RoundMode mode, SaturationMode sat, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src);
     TCVT_IMPL(dst, src, mode, sat);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename S, MaskPattern pattern, typename... Ev>
 PTO_INST RecordEvent TGATHER(D &dst, S &src, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src);
     TGATHER_IMPL<D, S, pattern>(dst, src);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename TileT, int isUpperOrLower, typename... Ev>
 PTO_INST RecordEvent TTRI(TileT &dst, int diagonal, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst);
     TTRI_IMPL<TileT, isUpperOrLower>(dst, diagonal);
+    detail::UbCommit(dst);
     return {};
 }
 

@@ -22,6 +22,16 @@
 // original and the copy are not views of each other.  After inlining the transfers are register renames.  (The mode is
 // opt-in because a class with a destructor keeps arrays of tiles in memory until late in the optimiser, which costs
 // the tuned kernels a few registers.)
+//
+// Vec tiles in memory.  Kernel sources written for Ascend also treat a Vec tile as an address in the unified buffer: they
+// TASSIGN a tile to `other.data() + offset` to get a view of a few rows or columns of another tile, re-view a [R,1] tile
+// as [1,R] with TRESHAPE and expect a write through one view to show in the other, and pass tiles by value
+// (pto_macro_fa_softmax.hpp:141-215, fa_performance_kernel.cpp:504-515).  A translation unit that defines
+// PTO_VEC_TILES_IN_MEMORY before the include gets exactly that: a Vec tile is a handle to `Rows * Cols` elements in the
+// reference's storage order inside a per-workgroup unified buffer in global memory (pto/gfx950/ub_mode.hpp); every
+// instruction loads its Vec operands from there into the register distribution described above, runs, and writes its
+// destination back, followed by a workgroup barrier.  It is the compatibility mode for unmodified sources, several
+// times slower than register-resident Vec tiles, which stay the default.
 #pragma once
 #include "pto/common/types.hpp"
 #include "pto/gfx950/platform.hpp"
@@ -44,6 +54,11 @@ namespace detail {
 constexpr bool kTileCopyWriteback = true;
 #else
 constexpr bool kTileCopyWriteback = false;
+#endif
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+constexpr bool kVecTilesInMemory = true;
+#else
+constexpr bool kVecTilesInMemory = false;
 #endif
 
 static_assert(PTO_MFMA_M == 32 || PTO_MFMA_M == 16, "v_mfma_f32_32x32x16 or v_mfma_f32_16x16x32");
@@ -281,7 +296,12 @@ struct Tile {
     int RowMaskInternal = RowValid_;
     int ColMaskInternal = ColValid_;
     Tile *origin_ = nullptr; // register tiles: set in a copy, the tile it was copied from (values go back on destruction)
-    static constexpr bool isHandle = Loc_ == TileType::Mat; // the object itself is an address
+    // the object itself is an address: Mat tiles, and Vec tiles of a translation unit that keeps them in memory
+    static constexpr bool inMemory = Loc_ == TileType::Vec && detail::kVecTilesInMemory;
+    static constexpr bool isHandle = Loc_ == TileType::Mat || inMemory;
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+    DType *mem_ = nullptr; // Vec tiles: element 0 of the tile in the unified buffer (nullptr: not assigned, registers only)
+#endif
 
     PTO_HD Tile() {}
     PTO_HD Tile(const Tile &o) : RowMaskInternal(o.RowMaskInternal), ColMaskInternal(o.ColMaskInternal) { Bind(o); }
@@ -320,10 +340,16 @@ struct Tile {
     // Mat tiles: pointer to the LDS image (swizzled, see mem_ops.hpp).  Register tiles: their fragments.
     PTO_DEV auto data()
     {
-        if constexpr (Loc_ == TileType::Mat)
+        if constexpr (Loc_ == TileType::Mat) {
             return reinterpret_cast<DType *>(hw::lds_base() + st.lds);
-        else
-            return &S();
+        } else {
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+            if constexpr (inMemory)
+                return mem_;
+            else
+#endif
+                return &S();
+        }
     }
 
     // Element `offset` of the tile's linear storage order (pto_tile.hpp:1254-1266 of the reference; Vec tiles only).
@@ -332,6 +358,17 @@ struct Tile {
     PTO_DEV void SetValue(const uint32_t offset, const DType val)
     {
         static_assert(Loc_ == TileType::Vec, "[PTO][SA] SetValue / GetValue: Vec tiles");
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+        if (mem_ != nullptr) { // the tile is an address: one lane writes, the workgroup waits for the store
+            if (hw::tid() == 0)
+                mem_[offset] = val;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            return;
+        }
+#endif
         const uint32_t q = offset / detail::kVecChunk, e = offset % detail::kVecChunk;
         if ((uint32_t)hw::tid() == q % kBlockThreads) {
             Storage &s = S();
@@ -346,6 +383,10 @@ struct Tile {
     PTO_DEV DType GetValue(const uint32_t offset)
     {
         static_assert(Loc_ == TileType::Vec, "[PTO][SA] SetValue / GetValue: Vec tiles");
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+        if (mem_ != nullptr)
+            return mem_[offset];
+#endif
         __shared__ DType pto_getvalue_slot;
         const uint32_t q = offset / detail::kVecChunk, e = offset % detail::kVecChunk;
         if ((uint32_t)hw::tid() == q % kBlockThreads) {
@@ -372,6 +413,9 @@ private:
                       "[PTO][SA] a register tile (Left / Right / Acc / Vec) was copied: pass it by reference, or define "
                       "PTO_TILE_COPY_WRITEBACK before including pto-inst.hpp to give copies write-back semantics");
         st = o.st;
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+        mem_ = o.mem_;
+#endif
         if constexpr (!isHandle)
             origin_ = const_cast<Tile *>(&o);
     }

@@ -10,7 +10,6 @@
 namespace pto {
 
 using half = _Float16;
-using aclFloat16 = _Float16;
 using bfloat16_t = __bf16;
 // 8-bit storage types of the MX formats (element types of `TMATMUL_MX` operands and their block scales)
 struct float8_e4m3_t { uint8_t bits; };

@@ -108,6 +108,11 @@ PTO_DEV T pad_value(PadValue p)
 // the shared aperture in its upper half, its lower half is the LDS address.
 // Register tiles have no address: the call is accepted and ignored, as in the CPU simulation
 // (cpu/TAssign.hpp:20-21).  GlobalTensor: rebinding the base pointer.
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+} // namespace pto
+#include "pto/gfx950/ub_mode.hpp"
+namespace pto {
+#endif
 namespace detail {
 constexpr uint32_t kLdsBytes = 160 * 1024; // LDS of one gfx950 compute unit
 // bytes of a Mat tile's LDS image (a Mat tile of block scales is stored one byte per scale)
@@ -143,6 +148,15 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
 #endif
         obj.st.lds = off;
     } else {
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+        if constexpr (T::inMemory) {
+            // a byte offset into the workgroup's unified buffer, or a pointer obtained from another Vec tile's data()
+            const uint64_t a = (uint64_t)(uintptr_t)addr;
+            obj.mem_ = a < (uint64_t)PTO_UB_BYTES ? reinterpret_cast<typename T::DType *>(detail::ub_base() + a) :
+                                                   reinterpret_cast<typename T::DType *>((uintptr_t)a);
+            return;
+        }
+#endif
         (void)obj;
         (void)addr;
     }
@@ -514,27 +528,59 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
     constexpr uint32_t kStepChunks = kWaveSize / detail::kMfmaM; // 16-byte chunks per fragment (one per lane group)
     constexpr uint32_t kChunkElems = 16 / sizeof(ElemT);
     if constexpr (DstT::Loc == TileType::Left) {
-        static_assert(Geo::colsK, "[PTO][SA] TEXTRACT to Left: source must be contiguous along columns (Nz / row-major)");
         using S = typename DstT::Storage;
         const uint32_t row0 = idxRow + (uint32_t)hw::wave_m() * (S::MB * detail::kMfmaM) + l32;
-        const uint32_t chunk0 = idxCol / kChunkElems + khalf;
+        if constexpr (Geo::colsK) {
+            const uint32_t chunk0 = idxCol / kChunkElems + khalf;
 #pragma unroll
-        for (int mb = 0; mb < S::MB; ++mb)
+            for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
-            for (int ks = 0; ks < S::KS; ++ks)
-                dst.S().f[mb][ks] = *reinterpret_cast<const Frag *>(
-                    lds + detail::mat_chunk_off<Geo::RowBytes>(row0 + mb * detail::kMfmaM, chunk0 + ks * kStepChunks));
+                for (int ks = 0; ks < S::KS; ++ks)
+                    dst.S().f[mb][ks] = *reinterpret_cast<const Frag *>(
+                        lds + detail::mat_chunk_off<Geo::RowBytes>(row0 + mb * detail::kMfmaM, chunk0 + ks * kStepChunks));
+        } else {
+            // the source is contiguous along its rows (an A operand stored transposed): element-wise gather, the slow path
+            // that keeps every layout pair of the reference's TEXTRACT legal (a2a3/TExtract.hpp:537-548)
+            static_assert(sizeof(ElemT) == 2, "[PTO][SA] TEXTRACT across the contiguous dimension: 16-bit elements");
+#pragma unroll
+            for (int mb = 0; mb < S::MB; ++mb)
+#pragma unroll
+                for (int ks = 0; ks < S::KS; ++ks) {
+                    Frag f;
+#pragma unroll
+                    for (uint32_t j = 0; j < kChunkElems; ++j)
+                        f[j] = *reinterpret_cast<const ElemT *>(
+                            lds + Geo::elem_off(row0 + mb * detail::kMfmaM, idxCol + (khalf + ks * kStepChunks) * kChunkElems + j));
+                    dst.S().f[mb][ks] = f;
+                }
+        }
     } else if constexpr (DstT::Loc == TileType::Right) {
-        static_assert(!Geo::colsK, "[PTO][SA] TEXTRACT to Right: source must be contiguous along rows (Zn / column-major)");
         using S = typename DstT::Storage;
         const uint32_t col0 = idxCol + (uint32_t)hw::wave_n() * (S::NB * detail::kMfmaM) + l32;
-        const uint32_t chunk0 = idxRow / kChunkElems + khalf;
+        if constexpr (!Geo::colsK) {
+            const uint32_t chunk0 = idxRow / kChunkElems + khalf;
 #pragma unroll
-        for (int nb = 0; nb < S::NB; ++nb)
+            for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
-            for (int ks = 0; ks < S::KS; ++ks)
-                dst.S().f[nb][ks] = *reinterpret_cast<const Frag *>(
-                    lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * kStepChunks));
+                for (int ks = 0; ks < S::KS; ++ks)
+                    dst.S().f[nb][ks] = *reinterpret_cast<const Frag *>(
+                        lds + detail::mat_chunk_off<Geo::RowBytes>(col0 + nb * detail::kMfmaM, chunk0 + ks * kStepChunks));
+        } else {
+            // the source is contiguous along its columns (a B operand [k, n] stored row-major, the V tile of the
+            // reference's attention kernel: fa_performance_kernel.cpp:676-677): element-wise gather, the slow path
+            static_assert(sizeof(ElemT) == 2, "[PTO][SA] TEXTRACT across the contiguous dimension: 16-bit elements");
+#pragma unroll
+            for (int nb = 0; nb < S::NB; ++nb)
+#pragma unroll
+                for (int ks = 0; ks < S::KS; ++ks) {
+                    Frag f;
+#pragma unroll
+                    for (uint32_t j = 0; j < kChunkElems; ++j)
+                        f[j] = *reinterpret_cast<const ElemT *>(
+                            lds + Geo::elem_off(idxRow + (khalf + ks * kStepChunks) * kChunkElems + j, col0 + nb * detail::kMfmaM));
+                    dst.S().f[nb][ks] = f;
+                }
+        }
     } else {
         static_assert(DstT::Loc == TileType::Left, "[PTO][SA] TEXTRACT: destination must be a Left or Right tile");
     }

@@ -19,6 +19,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <type_traits>
 
 #define PTO_HD __host__ __device__ __forceinline__
 #define PTO_DEV __device__ __forceinline__
@@ -128,6 +129,18 @@ PTO_DEV void wait_flag(pipe_t src, pipe_t dst, event_t)
     // MTE1->M, M->MTE1, M->FIX, FIX->M, V<->M ...: register dependences, nothing to do
 }
 
+// kernel sources also pass the event id as a plain integer (pto_macro_matmul.hpp:173: a uint64_t ping-pong index)
+template <typename I, std::enable_if_t<std::is_integral<I>::value, int> = 0>
+PTO_DEV void set_flag(pipe_t s, pipe_t d, I id)
+{
+    set_flag(s, d, static_cast<event_t>(id));
+}
+template <typename I, std::enable_if_t<std::is_integral<I>::value, int> = 0>
+PTO_DEV void wait_flag(pipe_t s, pipe_t d, I id)
+{
+    wait_flag(s, d, static_cast<event_t>(id));
+}
+
 // Pipelined form of wait_flag(PIPE_MTE2, PIPE_MTE1, id) for software pipelines that keep several
 // TLOADs in flight: returns once all but the `Pending` most recently issued asynchronous copy
 // instructions of every wave have landed in LDS (vmcnt retires in order).  Pending is a count of
@@ -155,3 +168,56 @@ PTO_DEV int64_t get_subblockid() { return 0; }
 PTO_DEV int64_t get_subblockdim() { return 1; }
 PTO_DEV int64_t get_coreid() { return static_cast<int64_t>(blockIdx.x); }
 PTO_DEV int64_t get_sys_cnt() { return static_cast<int64_t>(wall_clock64()); }
+
+// ---- cross-core flags of the Cube / Vec kernels (fa_performance_kernel.cpp:617, TPush.hpp:140-160 of the reference) ----
+// On Ascend a Cube core and its Vec cores are separate instruction streams that signal each other through FFTS flags.
+// Here one workgroup runs both roles in program order, so the producer's code has always run before the consumer's: what
+// is left of a signal is "my global-memory stores are complete and visible to the workgroup", of a wait "the workgroup
+// has got this far".  Both are reached by every wave (kernel control flow around them is uniform).
+PTO_DEV void set_ffts_base_addr(uint64_t) {}
+PTO_DEV void ffts_cross_core_sync(pipe_t, uint64_t)
+{
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+}
+PTO_DEV void wait_flag_dev(int64_t)
+{
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+}
+
+// ---- function-local `static` variables of a core (pto_macro_matmul.hpp:58-65, fa_performance_kernel.cpp:263-275) ----
+// On Ascend such a variable is private to the core and keeps its value between calls for the length of the kernel.  A GPU
+// function cannot hold a `static` in a register; port_ascend_source.py rewrites `static T name = init;` inside device
+// functions into PTO_CORE_STATIC(T, name, init): `name` becomes a reference to one of 32 eight-byte slots in LDS, private
+// to the wave (every wave runs the same scalar program, so each keeps its own copy and no barrier is needed), initialised
+// on first use after PTO_KERNEL_PROLOGUE(), which the script puts at the top of every kernel.  Instantiations of one
+// template share the slot of the declaration.
+namespace pto {
+namespace detail {
+struct CoreStaticArea {
+    uint64_t slot[kBlockWaves][32];
+    uint32_t inited[kBlockWaves];
+};
+PTO_DEV CoreStaticArea &core_static_area()
+{
+    __shared__ CoreStaticArea area;
+    return area;
+}
+template <typename T, int ID>
+PTO_DEV T &core_static(T init)
+{
+    static_assert(sizeof(T) <= 8 && ID >= 0 && ID < 32, "[PTO][SA] PTO_CORE_STATIC: up to 32 variables of up to 8 bytes");
+    CoreStaticArea &a = core_static_area();
+    const int w = hw::wave();
+    T *p = reinterpret_cast<T *>(&a.slot[w][ID]);
+    if (!((a.inited[w] >> ID) & 1u)) {
+        *p = init;
+        a.inited[w] |= 1u << ID;
+    }
+    return *p;
+}
+} // namespace detail
+} // namespace pto
+#define PTO_KERNEL_PROLOGUE() (pto::detail::core_static_area().inited[pto::hw::wave()] = 0u)
+#define PTO_CORE_STATIC(T, NAME, INIT) T &NAME = pto::detail::core_static<T, __COUNTER__ % 32>(INIT)

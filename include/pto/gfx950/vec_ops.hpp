@@ -265,8 +265,11 @@ PTO_DEV void TEXPANDS_IMPL(TileT &dst, typename TileT::DType k)
 template <typename DstT, typename SrcT>
 PTO_DEV void TRESHAPE_IMPL(DstT &dst, SrcT &src)
 {
+    // a [R, 1] column-major tile and a [1, R] row-major tile store the same sequence: vectors may change their major order
+    constexpr bool vectors = (DstT::Rows == 1 || DstT::Cols == 1) && (SrcT::Rows == 1 || SrcT::Cols == 1) &&
+                             (DstT::isRowMajor ? DstT::Rows == 1 : DstT::Cols == 1) && (SrcT::isRowMajor ? SrcT::Rows == 1 : SrcT::Cols == 1);
     static_assert(detail::same_dist<DstT, SrcT> && sizeof(typename DstT::DType) == sizeof(typename SrcT::DType) &&
-                      DstT::isRowMajor == SrcT::isRowMajor,
+                      (DstT::isRowMajor == SrcT::isRowMajor || vectors),
                   "[PTO][SA] TRESHAPE: same element count, element size and major order");
     using S = typename SrcT::Storage;
 #pragma unroll

@@ -77,14 +77,21 @@ def build_host(verbose=True):
 
 REFERENCE = os.environ.get("PTO_REFERENCE", "/root/reference")
 PORTED_DIR = os.path.join(ROOT, "oracle", "_ref")
-# (library, reference source, constants rewritten for 160 KiB of LDS, dynamic LDS bytes of the launch)
+# (library, reference source, constants rewritten for 160 KiB of LDS, dynamic LDS bytes of the launch, further options)
 PORTED = [
     ("libpto_ported_gemm.so", "kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp",
-     [("stepKa", "1"), ("stepKb", "1")], 160 * 1024),
+     [("stepKa", "1"), ("stepKb", "1")], 160 * 1024, {}),
+    # the flash-attention kernel: Cube and Vec roles in one workgroup (both __DAV_* families defined), one Vec core per
+    # Cube core, single-buffered Q / K / P / V panels (128 KiB of LDS), Vec tiles in the unified buffer in memory
+    ("libpto_ported_fa.so", "kernels/manual/common/flash_atten/fa_performance_kernel.cpp",
+     [("VEC_CORES", "1"), ("MAX_VEC_UB_BYTES", "512U * 1024U"), ("kMatTNBuffers", "1"), ("pMatTNBuffers", "1"), ("vMatTNBuffers", "1")],
+     128 * 1024,
+     dict(defines=("__DAV_CUBE__", "__DAV_VEC__", "__DAV_C220_CUBE__", "__DAV_C220_VEC__"), vec_in_memory=True,
+          extra_includes=(os.path.join(HERE, "host", "port_cases"),), extra_flags=("-Wno-unknown-attributes",))),
 ]
 
 
-def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includes=()):
+def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includes=(), defines=(), vec_in_memory=False):
     """Runs a kernel source of the reference through port_ascend_source.py into a temporary directory and compiles the
     result against include/pto with hipcc; `out` ends in .o (compile only) or .so.  The ported text never enters the
     repository tree."""
@@ -95,7 +102,7 @@ def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includ
     spec.loader.exec_module(mod)
     src = os.path.join(REFERENCE, rel_src)
     with open(src) as f:
-        text, _ = mod.port(f.read(), sets, lds_bytes)
+        text, _ = mod.port(f.read(), sets, lds_bytes, defines, os.path.dirname(src), vec_in_memory)
     with tempfile.TemporaryDirectory() as tmp:
         hip = os.path.join(tmp, os.path.basename(rel_src).replace(".cpp", ".hip"))
         with open(hip, "w") as f:
@@ -113,9 +120,9 @@ def build_ported(verbose=True):
     if not os.path.isdir(REFERENCE):
         return
     os.makedirs(PORTED_DIR, exist_ok=True)
-    for lib, rel_src, sets, lds in PORTED:
+    for lib, rel_src, sets, lds, opts in PORTED:
         out = os.path.join(PORTED_DIR, lib)
-        rc, err = port_and_compile(rel_src, sets, lds, out)
+        rc, err = port_and_compile(rel_src, sets, lds, out, **opts)
         if rc != 0:
             raise RuntimeError("ported build failed for %s:\n%s" % (rel_src, err))
         if verbose:

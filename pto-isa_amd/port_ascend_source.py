@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Mechanical edits that turn a PTO kernel source written for the Ascend toolchain into a gfx950 translation unit.
 
-    python pto-isa_amd/port_ascend_source.py IN.cpp OUT.hip [--set NAME=VALUE ...] [--lds BYTES]
+    python pto-isa_amd/port_ascend_source.py IN.cpp OUT.hip [--set NAME=VALUE ...] [--define NAME[=VALUE] ...]
+                                             [--lds BYTES] [--vec-in-memory] [--no-inline]
 
 What a kernel source of the reference needs before `hipcc --offload-arch=gfx950 -I include` accepts it, and what this
 script therefore does (nothing else is touched; the tile code itself compiles as it is):
@@ -17,16 +18,53 @@ script therefore does (nothing else is touched; the tile code itself compiles as
    (see include/pto/common/tile.hpp).
 4. `--set NAME=VALUE` rewrites `constexpr <type> NAME = <old>;`: tile-size constants chosen for 512 KiB of L1 have
    to fit the 160 KiB of LDS (the TASSIGN of a tile that does not fit is a compile error, not a silent overrun).
+5. Headers that sit next to the source (`#include "name"`) are inlined so that the edits reach them; an inlined `.hpp`
+   is device code as a whole.
+6. `static T name = init;` inside a function becomes `PTO_CORE_STATIC(T, name, init);` (a per-wave slot in LDS: a GPU
+   function cannot keep a core-private `static`), and every `__global__` function starts with `PTO_KERNEL_PROLOGUE();`.
+7. `--define NAME[=VALUE]` puts `#define`s in front of everything (the `__DAV_*` macros by which a source asks which
+   kind of core it is compiled for: a workgroup plays both, so both may be defined).
+9. `__global__` becomes `__global__ __launch_bounds__(pto::kBlockThreads)`.
+8. `--vec-in-memory` defines PTO_VEC_TILES_IN_MEMORY (Vec tiles are addresses in a per-workgroup unified buffer, see
+   include/pto/common/tile.hpp) and makes every launch prepare that buffer (`pto::host::LaunchBlocks`).
 """
 import argparse
+import os
 import re
 import sys
 
 LAUNCH = re.compile(r"<<<\s*([^,<>]+?)\s*,\s*nullptr\s*,\s*([^<>]+?)\s*>>>")
+LOCAL_INCLUDE = re.compile(r'^[ \t]*#include[ \t]+"([^"]+)"[ \t]*$', re.M)
+STATIC_LOCAL = re.compile(r"^([ \t]+)static[ \t]+([A-Za-z_][\w:]*(?:[ \t]+[A-Za-z_][\w:]*)*)[ \t]+([A-Za-z_]\w*)[ \t]*=[ \t]*([^;]+);", re.M)
+KERNEL_HEAD = re.compile(r"__global__[^;{}]*?\)\s*\{")
+BEGIN_MARK, END_MARK = "//@@PTO_INLINED_BEGIN ", "//@@PTO_INLINED_END "
 
 
-def port(text, sets=(), lds_bytes=160 * 1024):
+def inline_local_includes(text, directory, seen=None):
+    """Replaces `#include "name"` by the text of `directory/name` where that file exists (headers that sit next to the kernel
+    source: the edits below have to reach them too).  Each file once; the rest of its includes are left alone."""
+    seen = set() if seen is None else seen
+
+    def repl(m):
+        name = m.group(1)
+        path = os.path.join(directory, name)
+        if not os.path.isfile(path):
+            return m.group(0)
+        if path in seen:
+            return "// (already included above: %s)" % name
+        seen.add(path)
+        with open(path) as f:
+            body = inline_local_includes(f.read(), os.path.dirname(path), seen)
+        return BEGIN_MARK + name + "\n" + body + "\n" + END_MARK + name
+    return LOCAL_INCLUDE.sub(repl, text)
+
+
+def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in_memory=False):
     notes = []
+    if directory is not None:
+        before = text
+        text = inline_local_includes(text, directory)
+        notes.append("%d local include%s inlined" % (text.count(BEGIN_MARK), "" if text.count(BEGIN_MARK) == 1 else "s"))
     for name, value in sets:
         pat = re.compile(r"(constexpr\s+[\w:]+\s+%s\s*=\s*)([^;]+)(;)" % re.escape(name))
         text, n = pat.subn(lambda m: m.group(1) + value + m.group(3), text)
@@ -35,17 +73,53 @@ def port(text, sets=(), lds_bytes=160 * 1024):
         notes.append("set %s = %s (%d place%s)" % (name, value, n, "" if n == 1 else "s"))
 
     # 2. launch statements
-    text, n = LAUNCH.subn(lambda m: "<<<%s, pto::kBlockThreads, %d, (hipStream_t)(%s)>>>" % (m.group(1), lds_bytes, m.group(2)), text)
+    blocks = "pto::host::LaunchBlocks(%s, (hipStream_t)(%s))" if vec_in_memory else "%s"
+
+    def launch(m):
+        b = blocks % (m.group(1), m.group(2)) if vec_in_memory else m.group(1)
+        return "<<<%s, pto::kBlockThreads, %d, (hipStream_t)(%s)>>>" % (b, lds_bytes, m.group(2))
+    text, n = LAUNCH.subn(launch, text)
     notes.append("%d launch statement%s rewritten" % (n, "" if n == 1 else "s"))
 
-    # 1. brackets: open after the prologue (comments, includes, using-directives, macro definitions and file-scope
-    # constants come first in these sources; the first AICORE / template line starts the device code)
+    # 9. kernels are launched with pto::kBlockThreads threads: tell the compiler (it assumes 1024 otherwise and has half the
+    # registers per thread to work with)
+    text, n = re.subn(r"__global__(?!\s*__launch_bounds__)", "__global__ __launch_bounds__(pto::kBlockThreads)", text)
+
+    # 5. function-local statics of device functions, and the prologue that resets them
+    text, n = STATIC_LOCAL.subn(lambda m: "%sPTO_CORE_STATIC(%s, %s, %s);" % (m.group(1), m.group(2), m.group(3), m.group(4).strip()), text)
+    if n:
+        notes.append("%d function-local static%s rewritten" % (n, "" if n == 1 else "s"))
+        text, k = KERNEL_HEAD.subn(lambda m: m.group(0) + "\n    PTO_KERNEL_PROLOGUE();", text)
+        notes.append("%d kernel prologue%s inserted" % (k, "" if k == 1 else "s"))
+
+    # 1. brackets.  Inlined .hpp files are device code as a whole; in the main file the device code opens after the
+    # prologue (comments, includes, using-directives, macro definitions and file-scope constants come first in these
+    # sources; the first AICORE / template / enum line starts the device code) and closes before the first host function.
     lines = text.split("\n")
-    first_dev = next((i for i, l in enumerate(lines) if re.match(r"\s*(template\s*<|AICORE\b|__global__\b|constexpr\s+AICORE|enum\b)", l)), None)
+    out, depth, main_idx = [], 0, []
+    for l in lines:
+        if l.startswith(BEGIN_MARK):
+            depth += 1
+            out.append("// ---- " + l[len(BEGIN_MARK):] + " (inlined)")
+            if depth == 1 and l.rstrip().endswith(".hpp"):
+                out.append("PTO_DEVICE_CODE_BEGIN")
+            continue
+        if l.startswith(END_MARK):
+            if depth == 1 and l.rstrip().endswith(".hpp"):
+                out.append("PTO_DEVICE_CODE_END")
+            depth -= 1
+            out.append("// ---- end of " + l[len(END_MARK):])
+            continue
+        if depth == 0:
+            main_idx.append(len(out))
+        out.append(l)
+    lines = out
+    is_main = set(main_idx)
+    first_dev = next((i for i in main_idx if re.match(r"\s*(template\s*<|AICORE\b|__global__\b|constexpr\s+AICORE|enum\b)", lines[i])), None)
     if first_dev is None:
         raise SystemExit("port_ascend_source: no device function found")
     # the first host function: the first file-scope function whose body launches a kernel
-    launch_line = next((i for i, l in enumerate(lines) if "<<<" in l), None)
+    launch_line = next((i for i in main_idx if "<<<" in lines[i]), None)
     host_start = None
     if launch_line is not None:
         # walk back to the first line of the top-level declaration that encloses it: a line that starts at column 0
@@ -58,15 +132,21 @@ def port(text, sets=(), lds_bytes=160 * 1024):
                 break
             i -= 1
         host_start = i
-    out = lines[:first_dev] + ["PTO_DEVICE_CODE_BEGIN"]
+    res = lines[:first_dev] + ["PTO_DEVICE_CODE_BEGIN"]
     if host_start is not None and host_start > first_dev:
-        out += lines[first_dev:host_start] + ["PTO_DEVICE_CODE_END"] + lines[host_start:]
+        res += lines[first_dev:host_start] + ["PTO_DEVICE_CODE_END"] + lines[host_start:]
         notes.append("device code: lines %d-%d" % (first_dev + 1, host_start))
     else:
-        out += lines[first_dev:] + ["PTO_DEVICE_CODE_END"]
+        res += lines[first_dev:] + ["PTO_DEVICE_CODE_END"]
         notes.append("device code: line %d to the end" % (first_dev + 1))
-    head = "#define PTO_TILE_COPY_WRITEBACK 1\n#include <hip/hip_runtime.h>\n"
-    return head + "\n".join(out), notes
+    head = "#define PTO_TILE_COPY_WRITEBACK 1\n"
+    if vec_in_memory:
+        head += "#define PTO_VEC_TILES_IN_MEMORY 1\n"
+    for d in defines:
+        name, _, value = d.partition("=")
+        head += "#define %s %s\n" % (name, value or "1")
+    head += "#include <hip/hip_runtime.h>\n"
+    return head + "\n".join(res), notes
 
 
 def main():
@@ -74,12 +154,16 @@ def main():
     ap.add_argument("src")
     ap.add_argument("dst")
     ap.add_argument("--set", action="append", default=[], metavar="NAME=VALUE")
+    ap.add_argument("--define", action="append", default=[], metavar="NAME[=VALUE]")
     ap.add_argument("--lds", type=int, default=160 * 1024)
+    ap.add_argument("--vec-in-memory", action="store_true")
+    ap.add_argument("--no-inline", action="store_true", help="leave `#include \"...\"` of files next to the source alone")
     args = ap.parse_args()
     sets = [tuple(s.split("=", 1)) for s in args.set]
     with open(args.src) as f:
         text = f.read()
-    out, notes = port(text, sets, args.lds)
+    out, notes = port(text, sets, args.lds, args.define, None if args.no_inline else os.path.dirname(os.path.abspath(args.src)),
+                      args.vec_in_memory)
     with open(args.dst, "w") as f:
         f.write(out)
     for n in notes:

@@ -46,3 +46,47 @@ def test_reference_gemm_performance_kernel_6144(oracle):
     rows = np.array([0, 1, 127, 128, 1535, 1536, 4097, 6143])
     want = oracle.gemm_f16f32(a[rows], b, base_k=64)
     assert np.abs(got[rows] - want).max() <= 2e-3 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("S0,S1,causal,tile_s1,preload", [(128, 1024, False, 256, 4), (256, 2048, False, 128, 4),
+                                                          (256, 1024, True, 128, 4), (512, 2048, True, 128, 2)])
+def test_reference_flash_attention_kernel(oracle, S0, S1, causal, tile_s1, preload):
+    """fa_performance_kernel.cpp: runTFA with its Cube / Vec stage functions, stage macros, TPipe FIFOs in global memory and
+    Vec tiles as views of a unified buffer, launched through its own LaunchTFA<S0, 128, S1, 128, 128, TILE_S1, QK_PRELOAD, 8,
+    false, CAUSAL, 4> with the workspace its host program allocates (main.cpp:126-207).  O [S0, 128] fp32 against a dense
+    float64 softmax (2e-3 of the largest |O|) and against the oracle's restatement of the streaming recurrence with the same
+    key tile and the NPU's round-half-away cast of P (5e-4: rounding only).  Data as the reference's generator draws them
+    (scripts/gen_data.py:26-35: seed 7, N(0,1) * 1.5 / 1.2 / 1)."""
+    import torch
+    lib = _ported("libpto_ported_fa.so")
+    name = ("_Z9LaunchTFAILi%dELi128ELi%dELi128ELi128ELi%dELi%dELi8ELb0ELb%dELi4EEvPtS0_S0_S0_S0_PfS1_S1_S1_S1_S1_S1_P12ihipStream_tPh"
+            % (S0, S1, tile_s1, preload, int(causal)))
+    fn = getattr(lib, name)
+    fn.restype, fn.argtypes = None, [C.c_void_p] * 14
+    head, cube_s0, fifo = 128, 128, 8
+    rng = np.random.default_rng(7)
+    q = (rng.standard_normal((S0, head)) * 1.5).astype(np.float16)
+    k = (rng.standard_normal((S1, head)) * 1.2).astype(np.float16)
+    v = rng.standard_normal((S1, head)).astype(np.float16)
+    dev = "cuda:0"
+    tq, tk, tv = (torch.from_numpy(t.view(np.int16)).to(dev) for t in (q, k, v))
+    blocks = S0 // cube_s0
+    z = lambda n, dt: torch.zeros(n, dtype=dt, device=dev)
+    ffts, p_fifo, expmax_fifo = z(64, torch.int16), z(blocks * fifo * cube_s0 * tile_s1, torch.int16), z(blocks * fifo * cube_s0, torch.float32)
+    gsum, expmax, oparts = z(S0, torch.float32), z(S0, torch.float32), z(S0 * head, torch.float32)
+    qk_fifo, pv_fifo = z(blocks * fifo * cube_s0 * tile_s1, torch.float32), z(blocks * fifo * cube_s0 * head, torch.float32)
+    o = torch.full((S0, head), float("nan"), dtype=torch.float32, device=dev)
+    print("ported flash attention launch", S0, S1, causal, flush=True)
+    fn(ffts.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), p_fifo.data_ptr(), expmax_fifo.data_ptr(), gsum.data_ptr(),
+       expmax.data_ptr(), o.data_ptr(), oparts.data_ptr(), qk_fifo.data_ptr(), pv_fifo.data_ptr(), None, None)
+    torch.cuda.synchronize()
+    got = o.cpu().numpy()
+    s = q.astype(np.float64) @ k.astype(np.float64).T / np.sqrt(head)
+    if causal:
+        s = np.where(np.triu(np.ones((S0, S1), dtype=bool), 1), -np.inf, s)
+    p = np.exp(s - s.max(axis=1, keepdims=True))
+    want = (p / p.sum(axis=1, keepdims=True)) @ v.astype(np.float64)
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= 2e-3 * np.abs(want).max()
+    oo, _, _ = oracle.fa_stream_f16(q, k, v, tile_s1=tile_s1, causal=causal, q_offset=0, round_away=True)
+    assert np.abs(got - oo).max() <= 5e-4 * np.abs(oo).max()

@@ -48,6 +48,47 @@ def test_reference_gemm_kernel_with_its_own_l1_sizes_is_a_compile_error(tmp_path
     assert rc != 0 and "[PTO][SA] TASSIGN" in err and "160 KiB" in err, err
 
 
+@needs_reference
+def test_reference_flash_attention_kernel_compiles(tmp_path):
+    """fa_performance_kernel.cpp with its stage macros (pto_macro_matmul / _fa_softmax / _fa_gu.hpp, inlined by the port
+    script), runTFA and LaunchTFA for the committed case list: the options of build_ported()."""
+    lib, rel_src, sets, lds, opts = [p for p in B.PORTED if p[0] == "libpto_ported_fa.so"][0]
+    rc, err = B.port_and_compile(rel_src, sets, lds, str(tmp_path / "fa.o"), **opts)
+    assert rc == 0, err
+
+
+def test_port_script_rewrites():
+    """The mechanical edits on a synthetic source: launch statement, function-local static, kernel prologue, brackets."""
+    spec = importlib.util.spec_from_file_location("port_ascend_source", os.path.join(PKG, "port_ascend_source.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    src = """#include <pto/pto-inst.hpp>
+using namespace pto;
+constexpr int kSize = 512;
+AICORE inline int counter()
+{
+    static int calls = 0;
+    return ++calls;
+}
+__global__ AICORE void kern(__gm__ float *out)
+{
+    out[0] = counter();
+}
+void Launch(float *out, void *stream)
+{
+    kern<<<4, nullptr, stream>>>(out);
+}
+"""
+    text, notes = mod.port(src, [("kSize", "128")], 4096, ("__DAV_VEC__",), None, True)
+    assert "constexpr int kSize = 128;" in text
+    assert "PTO_CORE_STATIC(int, calls, 0);" in text and "PTO_KERNEL_PROLOGUE();" in text
+    assert "<<<pto::host::LaunchBlocks(4, (hipStream_t)(stream)), pto::kBlockThreads, 4096, (hipStream_t)(stream)>>>" in text
+    assert "__global__ __launch_bounds__(pto::kBlockThreads) AICORE void kern" in text
+    assert text.startswith("#define PTO_TILE_COPY_WRITEBACK 1\n#define PTO_VEC_TILES_IN_MEMORY 1\n#define __DAV_VEC__ 1\n")
+    begin, end, launch = text.index("PTO_DEVICE_CODE_BEGIN"), text.index("PTO_DEVICE_CODE_END"), text.index("void Launch")
+    assert begin < text.index("AICORE inline int counter") and text.index("void kern") < end < launch
+
+
 SNIPPET = r"""
 #include <hip/hip_runtime.h>
 #include <pto/pto-inst.hpp>
