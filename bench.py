@@ -25,15 +25,15 @@ PEAK_FP4_TFLOPS = 10066.3   # dense fp4 matrix peak (published)
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E peak (published)
 # row gather, 65536 x 1024 fp16 from a 32 MiB table: bytes per launch at the L2 <-> fabric boundary (FETCH_SIZE + WRITE_SIZE
 # runs summarised in profiles/cvt_f32_16384x8192_and_gather_rows_65536x1024.md)
-GATHER_HBM_SIDE_BYTES = 85.1e6 + 134.3e6
+GATHER_HBM_SIDE_BYTES = 85.0e6 + 134.3e6
 
 # HBM-side traffic of one 6144^3 GEMM launch, from two rocprofv3 --pmc runs of this script
 # (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch of the GEMM kernel), each scaled by what the same
 # counter reads for a plain 1 GiB device copy in the same run (--calib-copy): FETCH_SIZE reads
 # 524,300 KiB for 1,048,576 KiB actually read (factor 2.0), WRITE_SIZE reads 1,048,576 KiB for
 # 1,048,576 KiB written (factor 1.0).
-GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 295155.0, 2.0
-GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 148503.0, 1.0
+GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 295758.0, 2.0
+GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 149166.0, 1.0
 
 
 SETTLE_S = 0.0   # set from --settle-ms: the workloads under "extra" keep warming up until this much time has passed
@@ -326,7 +326,7 @@ def main():
                                                "frac_hbm_peak_hbm_side": hbm_side / (r["ms"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
                                                "note": "cache-resident figure, not an HBM roofline number: gbs_algorithmic counts rows read + "
                                                        "rows written + indices (268.7 MB), but the 32 MiB table is served from cache; the "
-                                                       "FETCH_SIZE / WRITE_SIZE counters (profiles/) read 85.1 MB + 134.3 MB per launch at the "
+                                                       "FETCH_SIZE / WRITE_SIZE counters (profiles/) read 85.0 MB + 134.3 MB per launch at the "
                                                        "L2 <-> fabric boundary, which gbs_hbm_side is computed from"}
 
     if only in ("", "gemm") and args.size == 6144:
