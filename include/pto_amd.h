@@ -58,7 +58,8 @@ int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b
 
 /* MXFP8 GEMM: C[m,n] row-major = (A .* 2^(scale_a - 127)) x (B .* 2^(scale_b - 127)) with fp32 accumulation.
  * a [m,k] and b stored [n,k] (a column-major k x n operand) hold 8-bit floats: format 0 = e4m3 (OCP, no infinities),
- * 1 = e5m2, the same for both operands.  scale_a [m,k/32] and scale_b stored [n,k/32] hold one e8m0 exponent per row
+ * 1 = e5m2 for both operands; 2 = a in e4m3 and b in e5m2, 3 = a in e5m2 and b in e4m3 (the matrix instruction takes a
+ * format per operand).  scale_a [m,k/32] and scale_b stored [n,k/32] hold one e8m0 exponent per row
  * (column) and 32 consecutive k (the reference's x1_gm / x2_gm / x1_scale_gm / x2_scale_gm files).  c: bf16
  * (c_fp32 == 0, round-to-nearest-even of the fp32 sum) or fp32.  m >= 256, n >= 256 (any value: the last tile row /
  * column is moved back to end at m / n and recomputes what it overlaps), k % 512 == 0. */

@@ -322,6 +322,13 @@ int gemm_mx_dispatch_fmt(hipStream_t st, void *c, const uint8_t *a, const uint8_
     if (format == 1)
         return c_fp32 ? launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
                         launch_gemm_mx<float8_e5m2_t, float8_e5m2_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
+    // mixed fp8 operands (the MFMA takes a format per operand): 2 = A e4m3 x B e5m2, 3 = A e5m2 x B e4m3
+    if (format == 2)
+        return c_fp32 ? launch_gemm_mx<float8_e4m3_t, float8_e5m2_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float8_e4m3_t, float8_e5m2_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
+    if (format == 3)
+        return c_fp32 ? launch_gemm_mx<float8_e5m2_t, float8_e4m3_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
+                        launch_gemm_mx<float8_e5m2_t, float8_e4m3_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
     if (format == 4)
         return c_fp32 ? launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, float, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode) :
                         launch_gemm_mx<float4_e2m1x2_t, float4_e2m1x2_t, bfloat16_t, DEEP>(st, c, a, b, sa, sb, m, n, k, tailMode);
@@ -343,7 +350,7 @@ extern "C" int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uin
 {
     if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0)
         return PTO_ERR_BAD_ARG;
-    if (format != 0 && format != 1)
+    if (format < 0 || format > 3)
         return PTO_ERR_UNSUPPORTED;
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 1);
 }

@@ -812,6 +812,21 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void VecOpTyped(__gm__ T *out
         GmND<T, 1, 128> gc(const_cast<T *>(vecIn));
         TLOAD(cv, gc);
     }
+    bool floatOp = false;
+    if constexpr (!std::is_integral_v<T>) { // the transcendental and division instructions: floating-point tiles
+        floatOp = true;
+        switch (op) {
+        case kSqrt: TSQRT(o, a); break;
+        case kRsqrt: TRSQRT(o, a); break;
+        case kLog: TLOG(o, a); break;
+        case kRecip: TRECIP(o, a); break;
+        case kExp: TEXP(o, a); break;
+        case kDiv: TDIV(o, a, b); break;
+        case kDivs: TDIVS(o, a, k); break;
+        default: floatOp = false; break;
+        }
+    }
+    if (!floatOp)
     switch (op) {
     case kAbs: TABS(o, a); break;
     case kNeg: TNEG(o, a); break;
@@ -850,7 +865,8 @@ extern "C" int pto_st_vec_op_typed_64x128(void *stream, void *out, const void *a
     const bool known = (op >= kAbs && op <= kRelu) || (op >= kAdd && op <= kMin && op != kDiv) ||
                        (op >= kAdds && op <= kMins && op != kDivs) || (op >= kRowExpand && op <= kRowMin && op != kRowDiv) ||
                        (op >= kColExpand && op <= kColMin && op != kColDiv);
-    if (!known || dtype < 0 || dtype > 1)
+    const bool floatOnly = (op >= kSqrt && op <= kExp) || op == kDiv || op == kDivs;
+    if (!(known || (floatOnly && dtype == 0)) || dtype < 0 || dtype > 1)
         return PTO_ERR_BAD_ARG;
     if (op >= kAdd && op <= kMin)
         PTO_ST_NONNULL(b);

@@ -37,6 +37,26 @@ def test_mx_gemm_small_vs_oracle(oracle, m, n, k, fmt):
     assert np.array_equal(got16, bf16_rne(got))
 
 
+@pytest.mark.parametrize("fmt_a,fmt_b,code", [(0, 1, 2), (1, 0, 3)])
+def test_mx_gemm_mixed_fp8_formats(oracle, fmt_a, fmt_b, code):
+    """A in e4m3 and B in e5m2 (format 2) and the other way round (3): every finite byte pattern of either format meets the
+    other (the byte 0x7c is 320 in e4m3 and +inf in e5m2, so a swapped format pair cannot pass), then integers, exactly."""
+    from gpu_util import gemm_mx
+    m, n, k = 512, 768, 1024
+    a, _, sa, sb = datagen.mx_inputs(m, n, k, fmt_a, dist="bytes")
+    _, b, _, _ = datagen.mx_inputs(m, n, k, fmt_b, dist="bytes")
+    got = gemm_mx(a, b, sa, sb, code)
+    want = oracle.mx_gemm(a, b, sa, sb, fmt_a, fmt_b)
+    assert np.all(np.isfinite(got)) and rel_err(got, want) <= TOL
+    wrong = oracle.mx_gemm(a, b, sa, sb, fmt_b, fmt_a)
+    assert rel_err(got, wrong) > 10 * TOL or not np.all(np.isfinite(wrong))
+    ai, _, sa, sb = datagen.mx_inputs(m, n, k, fmt_a, dist="integer")
+    _, bi, _, _ = datagen.mx_inputs(m, n, k, fmt_b, dist="integer")
+    assert np.array_equal(gemm_mx(ai, bi, sa, sb, code), oracle.mx_gemm(ai, bi, sa, sb, fmt_a, fmt_b))
+    got16 = gemm_mx(a, b, sa, sb, code, c_fp32=False)
+    assert np.array_equal(got16, bf16_rne(got))
+
+
 @pytest.mark.parametrize("fmt", [0, 1, 4])
 def test_mx_gemm_integer_operands_exact(oracle, fmt):
     """Integers in [-10, 10) (those fp8 can hold) and scales 2^0 .. 2^2: every partial sum is an integer below 2^24,
@@ -168,6 +188,6 @@ def test_mx_gemm_rejects_bad_arguments():
     assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 256, 512, 4, 1) == capi.ERR_UNSUPPORTED   # fp4 has its own entry point
     assert lib.pto_gemm_mxfp4(0, p, p, p, p, p, 256, 256, 768, 1) == capi.ERR_UNSUPPORTED      # k % 512
     assert lib.pto_gemm_mxfp4(0, p, 0, p, p, p, 256, 256, 512, 1) == capi.ERR_BAD_ARG
-    assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 256, 512, 2, 1) == capi.ERR_UNSUPPORTED   # unknown format
+    assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 256, 512, 5, 1) == capi.ERR_UNSUPPORTED   # unknown format
     assert lib.pto_gemm_mxfp8(0, p, p, p, 0, p, 256, 256, 512, 0, 1) == capi.ERR_BAD_ARG
     assert lib.pto_gemm_mxfp8(0, p, p, p, p, p, 256, 0, 512, 0, 1) == capi.ERR_BAD_ARG

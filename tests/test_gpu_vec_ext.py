@@ -136,6 +136,46 @@ TYPED_OPS = {
 }
 
 
+FP16_MATH_OPS = {
+    # the CPU simulation evaluates these in double and casts to the element type (ElementOp.h:265-340, TSqrt.hpp:23,
+    # TRSqrt.hpp:29-31, TExp.hpp:36); division and reciprocal are one operation in the element type (numpy's float16
+    # divides in float32 and rounds once more, which is what a host compiler does with _Float16 as well)
+    "SQRT": lambda a, b, k: np.sqrt(np.abs(a).astype(np.float64)).astype(np.float16),
+    "RSQRT": lambda a, b, k: (1.0 / np.sqrt(np.abs(a).astype(np.float64))).astype(np.float16),
+    "LOG": lambda a, b, k: np.log(np.abs(a).astype(np.float64)).astype(np.float16),
+    "EXP": lambda a, b, k: np.exp(a.astype(np.float64)).astype(np.float16),
+    "RECIP": lambda a, b, k: (np.float16(1) / a).astype(np.float16),
+    "DIV": lambda a, b, k: (a / b).astype(np.float16),
+    "DIVS": lambda a, b, k: (a / k).astype(np.float16),
+}
+
+
+@pytest.mark.parametrize("op", sorted(FP16_MATH_OPS))
+def test_vec_math_ops_fp16(oracle, op):
+    """TSQRT, TRSQRT, TLOG, TEXP, TRECIP, TDIV, TDIVS on fp16 tiles, bit-exact against the rule of the CPU simulation
+    (double evaluation + one cast for the transcendental ones), subnormal results and overflow to infinity included."""
+    lib = capi.load_st()
+    rng = np.random.default_rng(500 + len(op))
+    a = (rng.standard_normal((64, 128)) * (3 if op == "EXP" else 40)).astype(np.float16)
+    a[0, :8] = np.array([0.0, 6.1e-5, 5.96e-8, 65504.0, 1.0, 0.5, 11.1, 3.0e-5], dtype=np.float16)
+    if op == "EXP":
+        a[1, :4] = np.array([11.0, 11.1, -17.0, -16.0], dtype=np.float16)   # overflow to inf, subnormal results
+    b = (rng.standard_normal((64, 128)) * 8).astype(np.float16)
+    b[b == 0] = np.float16(1)
+    k = np.float16(1.75)
+    src = np.abs(a) if op in ("SQRT", "RSQRT", "LOG") else a
+    with np.errstate(over="ignore", invalid="ignore", divide="ignore"):
+        want = FP16_MATH_OPS[op](src, b, k)
+    ta, tb = dev(src), dev(b)
+    out = torch.zeros((64, 128), dtype=torch.int16, device=DEV)
+    capi.check(lib.pto_st_vec_op_typed_64x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), 0, float(k), oracle.VOP[op], 0), op)
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().view(np.float16)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint16), want[~nan].view(np.uint16)), op
+
+
 @pytest.mark.parametrize("dtype", ["f16", "s32"])
 @pytest.mark.parametrize("op", sorted(TYPED_OPS))
 def test_vec_op_fp16_and_int32(oracle, op, dtype):
