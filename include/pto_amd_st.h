@@ -146,20 +146,27 @@ int pto_st_tgatherb_f32_16x128(void *stream, float *out, const float *src, const
 /* TCI (pto_instr.hpp:808-814, cpu/TCI.hpp): out [1024] int32 is read, out[j] = start + j (descending: start - j) for
  * j < valid_cols, the rest keeps its values. */
 int pto_st_tci_s32_1x1024(void *stream, int32_t *out, int32_t start, int descending, int valid_cols);
-/* TSORT32 (pto_instr.hpp:786-798, cpu/TSort32.hpp) on an [8,128] tile of fp32 (dtype 0) or int32 (dtype 1) scores with
- * uint32 indices and the valid region [valid_rows, valid_cols]: out [8,256] is read, every group of 32 valid columns
- * of a row is written back as (score, index bit pattern) structures in descending order of score, equal scores in
+/* TSORT32 (pto_instr.hpp:786-798, cpu/TSort32.hpp) on an [8,128] tile of fp32 (dtype 0), int32 (1), fp16 (2) or int16 (3)
+ * scores with uint32 indices and the valid region [valid_rows, valid_cols]: out [8,256] (4-byte scores) or [8,512] (2-byte
+ * scores) is read, every group of 32 valid columns of a row is written back as 8-byte structures -- (score, index bit
+ * pattern), or (score, 0, index & 0xffff, index >> 16) for 2-byte scores -- in descending order of score, equal scores in
  * ascending order of index, and the rest of out is left as it was. */
 int pto_st_tsort32_8x128(void *stream, void *out, const void *src, const uint32_t *idx, int valid_rows, int valid_cols, int dtype);
 /* TMRGSORT with one source (pto_instr.hpp:616-622, cpu/TMrgSort.hpp:181-230) on [1,1024] fp32 tiles: every complete
  * group of four sorted blocks of block_len elements (block_len / 2 structures) inside the first valid_cols columns is
  * merged; out is read first and keeps its other elements. */
 int pto_st_tmrgsort_blocks_f32_1x1024(void *stream, float *out, const float *src, int valid_cols, int block_len);
+/* the same on [1,2048] tiles of 2-byte elements, four to a structure with the score first (block_len / 4 structures a block):
+ * dtype 0 = fp16, 1 = uint16, 2 = int16 scores (the reference's own cases use uint16: tests/cpu/st/testcase/tmrgsort/main.cpp:276-324) */
+int pto_st_tmrgsort_blocks_16_1x2048(void *stream, void *out, const void *src, int valid_cols, int block_len, int dtype);
 /* TMRGSORT with 2..4 lists (pto_instr.hpp:582-614, cpu/TMrgSort.hpp:118-178): src_i [256] fp32 hold cols_i / 2 sorted
  * (score, index) structures; the merge fills the first out_cols columns of out [1024] (read first), stops early when
  * exhausted != 0 and a list runs empty, and reports in executed[4] how many structures of each list it took. */
 int pto_st_tmrgsort_lists_f32(void *stream, float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2,
                               const float *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted);
+/* the same with lists of 2-byte elements: src_i [512] hold cols_i / 4 structures, out [2048]; dtype 0 = fp16, 1 = uint16 */
+int pto_st_tmrgsort_lists_16(void *stream, void *out, uint32_t *executed, const void *src0, const void *src1, const void *src2,
+                             const void *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted, int dtype);
 /* TMOV Vec -> Left / Right, Acc -> Left and TTRANS (the operand moves of the Auto-mode programs, cpu/TMov.hpp,
  * cpu/TTrans.hpp): a [64,64], b [64,128] fp16 row-major are loaded as Vec tiles and moved into operand tiles;
  * mid [64,128] = a b (fp32); out [64,64] = half(mid) b^T, with b^T made by TTRANS and half(mid) by the Acc -> Left move. */

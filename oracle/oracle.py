@@ -256,20 +256,30 @@ def tpart(dst, a, b, op, dvalid, avalid, bvalid):
 def tsort32(dst, src, idx, valid_row, valid_col, index_as_value=False):
     """TSORT32 (cpu/TSort32.hpp:44-88): in every row, every group of 32 valid columns is put in descending order of
     score, equal scores in ascending order of index (a stable sort, so equal pairs keep their order), and written as
-    (score, index) structures at columns 2 j, 2 j + 1 of dst [rows, >= 2 cols] (the rest of dst is left as it is).
-    The index is stored as its bit pattern (the NPU form) or, index_as_value, converted to the element type by value
-    (what the CPU simulation's assignment does).  Pure Python: single tiles only."""
+    8-byte structures: (score, index) for 4-byte elements at columns 2 j, 2 j + 1 of dst, (score, 0, index & 0xffff,
+    index >> 16) for 2-byte elements at columns 4 j .. 4 j + 3 (the rest of dst is left as it is).
+    The index is stored as its bit pattern (the NPU form: tests/npu/a2a3/src/st/testcase/tsort32/gen_data.py:20-27)
+    or, index_as_value, exactly as the CPU simulation does it: the index (its two halves for 2-byte elements) converted
+    to the element type by value, and every group of a 2-byte tile starting at column 2 j (cpu/TSort32.hpp:49), so
+    that groups after the first overwrite the second half of the one before.  Pure Python: single tiles only."""
     dst = np.array(dst, copy=True)
+    per = 8 // dst.dtype.itemsize
     for r in range(valid_row):
         for j in range(0, valid_col, 32):
             n = min(32, valid_col - j)
             order = sorted(range(n), key=lambda t: (-_sort_key(src[r, j + t]), int(idx[r, j + t]), t))
+            base = 2 * j if index_as_value else per * j
             for m, t in enumerate(order):
-                dst[r, 2 * (j + m)] = src[r, j + t]
-                if index_as_value:
-                    dst[r, 2 * (j + m) + 1] = dst.dtype.type(idx[r, j + t])
+                c = base + per * m
+                ix = np.array([idx[r, j + t]], dtype=np.uint32)
+                dst[r, c] = src[r, j + t]
+                if per == 2:
+                    dst[r, c + 1:c + 2] = ix.astype(dst.dtype) if index_as_value else ix.view(dst.dtype)
                 else:
-                    dst[r, 2 * (j + m) + 1:2 * (j + m) + 2] = np.array([idx[r, j + t]], dtype=np.uint32).view(dst.dtype)
+                    dst[r, c + 1] = 0
+                    with np.errstate(over="ignore"):
+                        dst[r, c + 2:c + 4] = (np.array([ix[0], ix[0] >> 16]).astype(dst.dtype) if index_as_value
+                                               else ix.view(np.uint16).view(dst.dtype))
     return dst
 
 
@@ -280,7 +290,7 @@ def _sort_key(x):
 def _merge(lists, out_max, exhausted):
     """The sequential merge of cpu/TMrgSort.hpp:118-178: take the head with the largest score, the lowest list
     number on ties; stop at out_max structures, when everything is taken, or (exhausted) right after the structure
-    that empties a list.  lists: arrays [n_i, 2].  Returns (merged [m, 2], taken counts)."""
+    that empties a list.  lists: arrays [n_i, elements per structure], the score in column 0.  Returns (merged, taken counts)."""
     pos = [0] * len(lists)
     out = []
     while len(out) < out_max:
@@ -295,30 +305,33 @@ def _merge(lists, out_max, exhausted):
         if exhausted and any(pos[b] == len(l) for b, l in enumerate(lists)):
             break
     dt = lists[0].dtype
-    return (np.array(out, dtype=dt).reshape(-1, 2), pos)
+    return (np.array(out, dtype=dt).reshape(-1, lists[0].shape[1]), pos)
 
 
 def tmrgsort_blocks(dst, src, valid_cols, block_len):
     """TMRGSORT with one source (cpu/TMrgSort.hpp:181-230): every complete group of four blocks of block_len
-    elements inside the first valid_cols columns is merged; the rest of dst is left as it is."""
+    elements (8-byte structures: 2 elements of 4 bytes, 4 of 2 bytes, :41-46) inside the first valid_cols columns is
+    merged; the rest of dst is left as it is."""
     dst = np.array(dst, copy=True).reshape(-1)
     src = np.asarray(src).reshape(-1)
-    if block_len == 0 or block_len % 2:
+    per = 8 // dst.dtype.itemsize
+    if block_len == 0 or block_len % per:
         return dst
     group = 4 * block_len
     for c in range(0, valid_cols - group + 1, group):
-        lists = [src[c + b * block_len:c + (b + 1) * block_len].reshape(-1, 2) for b in range(4)]
-        merged, _ = _merge(lists, 2 * block_len, False)
+        lists = [src[c + b * block_len:c + (b + 1) * block_len].reshape(-1, per) for b in range(4)]
+        merged, _ = _merge(lists, 4 * block_len // per, False)
         dst[c:c + group] = merged.reshape(-1)
     return dst
 
 
 def tmrgsort_lists(dst, lists, cols, out_cols, exhausted):
-    """TMRGSORT with two to four lists (cpu/TMrgSort.hpp:232-297): lists[i][:cols[i]] are (score, index) structures
+    """TMRGSORT with two to four lists (cpu/TMrgSort.hpp:232-297): lists[i][:cols[i]] are 8-byte structures (score first)
     in descending order of score; returns (dst with the merged structures in front, executed counts [4])."""
     dst = np.array(dst, copy=True).reshape(-1)
-    ls = [np.asarray(l).reshape(-1)[:c // 2 * 2].reshape(-1, 2) for l, c in zip(lists, cols)]
-    merged, pos = _merge(ls, out_cols // 2, exhausted)
+    per = 8 // dst.dtype.itemsize
+    ls = [np.asarray(l).reshape(-1)[:c // per * per].reshape(-1, per) for l, c in zip(lists, cols)]
+    merged, pos = _merge(ls, out_cols // per, exhausted)
     dst[:merged.size] = merged.reshape(-1)
     return dst, np.array(pos + [0] * (4 - len(pos)), dtype=np.uint32)
 

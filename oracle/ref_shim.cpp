@@ -529,21 +529,31 @@ void sort32_8x128(T *out, const T *src, const uint32_t *idx, int vr, int vc)
 {
     using S = Tile<TileType::Vec, T, 8, 128, BLayout::RowMajor, -1, -1>;
     using I = Tile<TileType::Vec, uint32_t, 8, 128, BLayout::RowMajor, -1, -1>;
-    using D = Tile<TileType::Vec, T, 8, 256, BLayout::RowMajor>;
+    constexpr int DC = 128 * 8 / (int)sizeof(T); // 8 bytes of destination per source element
+    using D = Tile<TileType::Vec, T, 8, DC, BLayout::RowMajor>;
     auto s = std::make_unique<S>(vr, vc);
     auto x = std::make_unique<I>(vr, vc);
     auto d = std::make_unique<D>();
     std::memcpy(s->data(), src, sizeof(T) * 8 * 128);
     std::memcpy(x->data(), idx, sizeof(uint32_t) * 8 * 128);
-    std::memcpy(d->data(), out, sizeof(T) * 8 * 256);
+    std::memcpy(d->data(), out, sizeof(T) * 8 * DC);
     TSORT32(*d, *s, *x);
-    std::memcpy(out, d->data(), sizeof(T) * 8 * 256);
+    std::memcpy(out, d->data(), sizeof(T) * 8 * DC);
 }
 } // extern "C++"
 void ref_tsort32_f32_8x128(float *out, const float *src, const uint32_t *idx, int vr, int vc) { sort32_8x128<float>(out, src, idx, vr, vc); }
 void ref_tsort32_s32_8x128(int32_t *out, const int32_t *src, const uint32_t *idx, int vr, int vc)
 {
     sort32_8x128<int32_t>(out, src, idx, vr, vc);
+}
+// 2-byte scores: out [8,512]
+void ref_tsort32_f16_8x128(uint16_t *out, const uint16_t *src, const uint32_t *idx, int vr, int vc)
+{
+    sort32_8x128<half>(reinterpret_cast<half *>(out), reinterpret_cast<const half *>(src), idx, vr, vc);
+}
+void ref_tsort32_s16_8x128(int16_t *out, const int16_t *src, const uint32_t *idx, int vr, int vc)
+{
+    sort32_8x128<int16_t>(out, src, idx, vr, vc);
 }
 void ref_tpart_f32_64x128(float *out, const float *a, const float *b, int op, int dvr, int dvc, int avr, int avc, int bvr, int bvc)
 {
@@ -606,33 +616,38 @@ void ref_tci_s32_1x1024(int32_t *out, int32_t start, int descending, int vc)
         TCI<Dyn, int32_t, 0>(*td, start);
     std::memcpy(out, td->data(), sizeof(int32_t) * 1024);
 }
-void ref_tmrgsort_blocks_f32_1x1024(float *out, const float *src, int valid_cols, int block_len)
+extern "C++" {
+// one source of 4 KiB: [1,1024] 4-byte or [1,2048] 2-byte elements
+template <typename T>
+void mrgsort_blocks(T *out, const T *src, int valid_cols, int block_len)
 {
-    using S = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
-    using D = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, -1>;
+    constexpr int N = 4096 / (int)sizeof(T);
+    using S = Tile<TileType::Vec, T, 1, N, BLayout::RowMajor>;
+    using D = Tile<TileType::Vec, T, 1, N, BLayout::RowMajor, 1, -1>;
     auto s = std::make_unique<S>();
     auto d = std::make_unique<D>(valid_cols);
-    std::memcpy(s->data(), src, sizeof(float) * 1024);
-    std::memcpy(d->data(), out, sizeof(float) * 1024);
+    std::memcpy(s->data(), src, sizeof(T) * N);
+    std::memcpy(d->data(), out, sizeof(T) * N);
     TMRGSORT(*d, *s, static_cast<uint32_t>(block_len));
-    std::memcpy(out, d->data(), sizeof(float) * 1024);
+    std::memcpy(out, d->data(), sizeof(T) * N);
 }
-extern "C++" {
-template <bool EXH>
-void mrgsort_lists(float *out, uint32_t *executed, const float *const *src, const int *cols, int out_cols, int lists)
+// lists of 1 KiB (up to 128 structures) into a destination of 4 KiB
+template <typename T, bool EXH>
+void mrgsort_lists(T *out, uint32_t *executed, const T *const *src, const int *cols, int out_cols, int lists)
 {
-    using L = Tile<TileType::Vec, float, 1, 256, BLayout::RowMajor, 1, -1>;
-    using D = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, -1>;
-    using Tmp = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
+    constexpr int LC = 1024 / (int)sizeof(T), DC = 4 * LC;
+    using L = Tile<TileType::Vec, T, 1, LC, BLayout::RowMajor, 1, -1>;
+    using D = Tile<TileType::Vec, T, 1, DC, BLayout::RowMajor, 1, -1>;
+    using Tmp = Tile<TileType::Vec, T, 1, DC, BLayout::RowMajor>;
     std::unique_ptr<L> l[4];
     for (int i = 0; i < 4; ++i) {
         l[i] = std::make_unique<L>(i < lists ? cols[i] : 0);
         if (i < lists)
-            std::memcpy(l[i]->data(), src[i], sizeof(float) * 256);
+            std::memcpy(l[i]->data(), src[i], sizeof(T) * LC);
     }
     auto d = std::make_unique<D>(out_cols);
     auto tmp = std::make_unique<Tmp>();
-    std::memcpy(d->data(), out, sizeof(float) * 1024);
+    std::memcpy(d->data(), out, sizeof(T) * DC);
     MrgSortExecutedNumList ex = {};
     if (lists == 4)
         TMRGSORT<D, Tmp, L, L, L, L, EXH>(*d, ex, *tmp, *l[0], *l[1], *l[2], *l[3]);
@@ -640,22 +655,51 @@ void mrgsort_lists(float *out, uint32_t *executed, const float *const *src, cons
         TMRGSORT<D, Tmp, L, L, L, EXH>(*d, ex, *tmp, *l[0], *l[1], *l[2]);
     else
         TMRGSORT<D, Tmp, L, L, EXH>(*d, ex, *tmp, *l[0], *l[1]);
-    std::memcpy(out, d->data(), sizeof(float) * 1024);
+    std::memcpy(out, d->data(), sizeof(T) * DC);
     executed[0] = ex.mrgSortList0;
     executed[1] = ex.mrgSortList1;
     executed[2] = ex.mrgSortList2;
     executed[3] = ex.mrgSortList3;
 }
+template <typename T>
+void mrgsort_lists_any(void *out, uint32_t *executed, const void *src0, const void *src1, const void *src2, const void *src3, int cols0,
+                       int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
+{
+    const T *src[4] = {static_cast<const T *>(src0), static_cast<const T *>(src1), static_cast<const T *>(src2), static_cast<const T *>(src3)};
+    const int cols[4] = {cols0, cols1, cols2, cols3};
+    if (exhausted)
+        mrgsort_lists<T, true>(static_cast<T *>(out), executed, src, cols, out_cols, lists);
+    else
+        mrgsort_lists<T, false>(static_cast<T *>(out), executed, src, cols, out_cols, lists);
+}
 } // extern "C++"
+void ref_tmrgsort_blocks_f32_1x1024(float *out, const float *src, int valid_cols, int block_len)
+{
+    mrgsort_blocks<float>(out, src, valid_cols, block_len);
+}
+// dtype 0 = half, 1 = uint16_t, 2 = int16_t
+void ref_tmrgsort_blocks_16_1x2048(void *out, const void *src, int valid_cols, int block_len, int dtype)
+{
+    if (dtype == 0)
+        mrgsort_blocks<half>(static_cast<half *>(out), static_cast<const half *>(src), valid_cols, block_len);
+    else if (dtype == 1)
+        mrgsort_blocks<uint16_t>(static_cast<uint16_t *>(out), static_cast<const uint16_t *>(src), valid_cols, block_len);
+    else
+        mrgsort_blocks<int16_t>(static_cast<int16_t *>(out), static_cast<const int16_t *>(src), valid_cols, block_len);
+}
 void ref_tmrgsort_lists_f32(float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2, const float *src3,
                             int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
 {
-    const float *src[4] = {src0, src1, src2, src3};
-    const int cols[4] = {cols0, cols1, cols2, cols3};
-    if (exhausted)
-        mrgsort_lists<true>(out, executed, src, cols, out_cols, lists);
+    mrgsort_lists_any<float>(out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols, lists, exhausted);
+}
+// dtype 0 = half, 1 = uint16_t
+void ref_tmrgsort_lists_16(void *out, uint32_t *executed, const void *src0, const void *src1, const void *src2, const void *src3, int cols0,
+                           int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted, int dtype)
+{
+    if (dtype == 0)
+        mrgsort_lists_any<half>(out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols, lists, exhausted);
     else
-        mrgsort_lists<false>(out, executed, src, cols, out_cols, lists);
+        mrgsort_lists_any<uint16_t>(out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols, lists, exhausted);
 }
 void ref_fa_auto_128x64(float *out, const float *q, const float *k, const float *v) { fa_auto<128, 64>(out, q, k, v); }
 

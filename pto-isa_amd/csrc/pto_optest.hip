@@ -1046,7 +1046,7 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void TransKernel(__gm__ float
     TSTORE(go, y);
 }
 
-// ---- TSORT32 on an [8, 128] tile with valid region [vr, vc]; out [8, 256] is loaded first so that the elements the
+// ---- TSORT32 on an [8, 128] tile with valid region [vr, vc]; out [8, 256] (4-byte scores) or [8, 512] (2-byte) is loaded first so that the elements the
 // instruction leaves alone keep what the caller put there ----
 template <typename T>
 __global__ __launch_bounds__(kBlockThreads) AICORE void Sort32Kernel(__gm__ T *out, __gm__ const T *srcIn, __gm__ const uint32_t *idxIn,
@@ -1056,13 +1056,14 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void Sort32Kernel(__gm__ T *o
     using FullI = Tile<TileType::Vec, uint32_t, 8, 128, BLayout::RowMajor>;
     using Src = Tile<TileType::Vec, T, 8, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
     using Idx = Tile<TileType::Vec, uint32_t, 8, 128, BLayout::RowMajor, DYNAMIC, DYNAMIC>;
-    using Dst = Tile<TileType::Vec, T, 8, 256, BLayout::RowMajor>;
+    constexpr int kDstCols = 128 * 8 / (int)sizeof(T);
+    using Dst = Tile<TileType::Vec, T, 8, kDstCols, BLayout::RowMajor>;
     Full sf;
     FullI xf;
     Dst d;
     GmND<T, 8, 128> gs(const_cast<T *>(srcIn));
     GmND<uint32_t, 8, 128> gi(const_cast<uint32_t *>(idxIn));
-    GmND<T, 8, 256> go(out);
+    GmND<T, 8, kDstCols> go(out);
     TLOAD(sf, gs);
     TLOAD(xf, gi);
     TLOAD(d, go);
@@ -1074,14 +1075,15 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void Sort32Kernel(__gm__ T *o
     TSTORE(go, d);
 }
 
-// ---- TMRGSORT, one source: [1, 1024] tile, the destination's valid columns and the block length at run time ----
-__global__ __launch_bounds__(kBlockThreads) AICORE void MergeBlocksKernel(__gm__ float *out, __gm__ const float *srcIn, int validCols,
-                                                                          int blockLen)
+// ---- TMRGSORT, one source: [1, COLS] tile (8 KiB), the destination's valid columns and the block length at run time ----
+template <typename T>
+__global__ __launch_bounds__(kBlockThreads) AICORE void MergeBlocksKernel(__gm__ T *out, __gm__ const T *srcIn, int validCols, int blockLen)
 {
-    using Full = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
-    using Dst = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, DYNAMIC>;
+    constexpr int COLS = 4096 / (int)sizeof(T);
+    using Full = Tile<TileType::Vec, T, 1, COLS, BLayout::RowMajor>;
+    using Dst = Tile<TileType::Vec, T, 1, COLS, BLayout::RowMajor, 1, DYNAMIC>;
     Full s, d0;
-    GmND<float, 1, 1024> gs(const_cast<float *>(srcIn)), go(out);
+    GmND<T, 1, COLS> gs(const_cast<T *>(srcIn)), go(out);
     TLOAD(s, gs);
     TLOAD(d0, go);
     Dst d(validCols);
@@ -1092,25 +1094,25 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MergeBlocksKernel(__gm__
 }
 
 // ---- TMRGSORT, two to four lists of up to 128 structures each into a destination of up to 512 ----
-template <int LISTS, bool EXHAUSTED>
-__global__ __launch_bounds__(kBlockThreads) AICORE void MergeListsKernel(__gm__ float *out, __gm__ uint32_t *executedOut,
-                                                                         __gm__ const float *in0, __gm__ const float *in1,
-                                                                         __gm__ const float *in2, __gm__ const float *in3, int c0, int c1,
-                                                                         int c2, int c3, int outCols)
+template <typename T, int LISTS, bool EXHAUSTED>
+__global__ __launch_bounds__(kBlockThreads) AICORE void MergeListsKernel(__gm__ T *out, __gm__ uint32_t *executedOut, __gm__ const T *in0,
+                                                                         __gm__ const T *in1, __gm__ const T *in2, __gm__ const T *in3, int c0,
+                                                                         int c1, int c2, int c3, int outCols)
 {
-    using Full = Tile<TileType::Vec, float, 1, 256, BLayout::RowMajor>;
-    using List = Tile<TileType::Vec, float, 1, 256, BLayout::RowMajor, 1, DYNAMIC>;
-    using FullD = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor>;
-    using Dst = Tile<TileType::Vec, float, 1, 1024, BLayout::RowMajor, 1, DYNAMIC>;
+    constexpr int LC = 1024 / (int)sizeof(T), DC = 4 * LC;
+    using Full = Tile<TileType::Vec, T, 1, LC, BLayout::RowMajor>;
+    using List = Tile<TileType::Vec, T, 1, LC, BLayout::RowMajor, 1, DYNAMIC>;
+    using FullD = Tile<TileType::Vec, T, 1, DC, BLayout::RowMajor>;
+    using Dst = Tile<TileType::Vec, T, 1, DC, BLayout::RowMajor, 1, DYNAMIC>;
     Full f;
     FullD d0, tmp;
     List l0(c0), l1(c1), l2(c2), l3(c3);
-    GmND<float, 1, 1024> go(out);
-    const float *ins[4] = {in0, in1, in2, in3};
+    GmND<T, 1, DC> go(out);
+    const T *ins[4] = {in0, in1, in2, in3};
     List *lists[4] = {&l0, &l1, &l2, &l3};
 #pragma unroll
     for (int i = 0; i < LISTS; ++i) {
-        GmND<float, 1, 256> g(const_cast<float *>(ins[i]));
+        GmND<T, 1, LC> g(const_cast<T *>(ins[i]));
         TLOAD(f, g);
         lists[i]->st = f.st;
     }
@@ -1276,15 +1278,20 @@ extern "C" int pto_st_tci_s32_1x1024(void *stream, int32_t *out, int32_t start, 
 extern "C" int pto_st_tsort32_8x128(void *stream, void *out, const void *src, const uint32_t *idx, int valid_rows, int valid_cols, int dtype)
 {
     PTO_ST_NONNULL(out, src, idx);
-    if (valid_rows < 0 || valid_rows > 8 || valid_cols < 0 || valid_cols > 128 || dtype < 0 || dtype > 1)
+    if (valid_rows < 0 || valid_rows > 8 || valid_cols < 0 || valid_cols > 128 || dtype < 0 || dtype > 3)
         return PTO_ERR_BAD_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
+#define PTO_ST_SORT32(T) \
+    Sort32Kernel<T><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<T *>(out), static_cast<const T *>(src), idx, valid_rows, valid_cols)
     if (dtype == 0)
-        Sort32Kernel<float><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<float *>(out), static_cast<const float *>(src), idx, valid_rows,
-                                                                    valid_cols);
+        PTO_ST_SORT32(float);
+    else if (dtype == 1)
+        PTO_ST_SORT32(int32_t);
+    else if (dtype == 2)
+        PTO_ST_SORT32(half);
     else
-        Sort32Kernel<int32_t><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<int32_t *>(out), static_cast<const int32_t *>(src), idx,
-                                                                      valid_rows, valid_cols);
+        PTO_ST_SORT32(int16_t);
+#undef PTO_ST_SORT32
     return pto_amd::check_launch();
 }
 
@@ -1293,23 +1300,44 @@ extern "C" int pto_st_tmrgsort_blocks_f32_1x1024(void *stream, float *out, const
     PTO_ST_NONNULL(out, src);
     if (valid_cols < 0 || valid_cols > 1024 || block_len < 0 || block_len > 256)
         return PTO_ERR_BAD_ARG;
-    MergeBlocksKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, valid_cols, block_len);
+    MergeBlocksKernel<float><<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, valid_cols, block_len);
     return pto_amd::check_launch();
 }
 
-extern "C" int pto_st_tmrgsort_lists_f32(void *stream, float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2,
-                                         const float *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
+extern "C" int pto_st_tmrgsort_blocks_16_1x2048(void *stream, void *out, const void *src, int valid_cols, int block_len, int dtype)
 {
+    PTO_ST_NONNULL(out, src);
+    if (valid_cols < 0 || valid_cols > 2048 || block_len < 0 || block_len > 512 || dtype < 0 || dtype > 2)
+        return PTO_ERR_BAD_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PTO_ST_BLOCKS(T) \
+    MergeBlocksKernel<T><<<dim3(1), dim3(kBlockThreads), 0, st>>>(static_cast<T *>(out), static_cast<const T *>(src), valid_cols, block_len)
+    if (dtype == 0)
+        PTO_ST_BLOCKS(half);
+    else if (dtype == 1)
+        PTO_ST_BLOCKS(uint16_t);
+    else
+        PTO_ST_BLOCKS(int16_t);
+#undef PTO_ST_BLOCKS
+    return pto_amd::check_launch();
+}
+
+namespace {
+template <typename T>
+int merge_lists_launch(void *stream, T *out, uint32_t *executed, const T *src0, const T *src1, const T *src2, const T *src3, int cols0,
+                       int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
+{
+    constexpr int E = 8 / (int)sizeof(T), LC = 1024 / (int)sizeof(T);
     PTO_ST_NONNULL(out, executed, src0, src1);
-    if (lists < 2 || lists > 4 || (lists > 2 && !src2) || (lists > 3 && !src3) || out_cols < 0 || out_cols > 1024)
+    if (lists < 2 || lists > 4 || (lists > 2 && !src2) || (lists > 3 && !src3) || out_cols < 0 || out_cols > 4 * LC)
         return PTO_ERR_BAD_ARG;
     const int cols[4] = {cols0, cols1, cols2, cols3};
     for (int i = 0; i < lists; ++i)
-        if (cols[i] < 0 || cols[i] > 256 || cols[i] % 2)
+        if (cols[i] < 0 || cols[i] > LC || cols[i] % E)
             return PTO_ERR_BAD_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
-#define PTO_ST_MERGE(L, E) \
-    MergeListsKernel<L, E><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols)
+#define PTO_ST_MERGE(L, X) \
+    MergeListsKernel<T, L, X><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols)
     if (lists == 4 && exhausted)
         PTO_ST_MERGE(4, true);
     else if (lists == 4)
@@ -1324,6 +1352,28 @@ extern "C" int pto_st_tmrgsort_lists_f32(void *stream, float *out, uint32_t *exe
         PTO_ST_MERGE(2, false);
 #undef PTO_ST_MERGE
     return pto_amd::check_launch();
+}
+} // namespace
+
+extern "C" int pto_st_tmrgsort_lists_f32(void *stream, float *out, uint32_t *executed, const float *src0, const float *src1, const float *src2,
+                                         const float *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted)
+{
+    return merge_lists_launch<float>(stream, out, executed, src0, src1, src2, src3, cols0, cols1, cols2, cols3, out_cols, lists, exhausted);
+}
+
+extern "C" int pto_st_tmrgsort_lists_16(void *stream, void *out, uint32_t *executed, const void *src0, const void *src1, const void *src2,
+                                        const void *src3, int cols0, int cols1, int cols2, int cols3, int out_cols, int lists, int exhausted,
+                                        int dtype)
+{
+    if (dtype < 0 || dtype > 1)
+        return PTO_ERR_BAD_ARG;
+    if (dtype == 0)
+        return merge_lists_launch<half>(stream, static_cast<half *>(out), executed, static_cast<const half *>(src0),
+                                        static_cast<const half *>(src1), static_cast<const half *>(src2), static_cast<const half *>(src3), cols0,
+                                        cols1, cols2, cols3, out_cols, lists, exhausted);
+    return merge_lists_launch<uint16_t>(stream, static_cast<uint16_t *>(out), executed, static_cast<const uint16_t *>(src0),
+                                        static_cast<const uint16_t *>(src1), static_cast<const uint16_t *>(src2),
+                                        static_cast<const uint16_t *>(src3), cols0, cols1, cols2, cols3, out_cols, lists, exhausted);
 }
 
 extern "C" int pto_st_matmul_vec_operands_f16_64x64x128(void *stream, float *out, float *mid, const uint16_t *a, const uint16_t *b)

@@ -109,6 +109,22 @@ def sort_cases(ref):
         ref.ref_tmrgsort_lists_f32(p(o), p(ex), *ptrs, *cols, 2 * out_structs, len(counts), exhausted)
         out["lists_%d" % seed] = o.view(np.uint32)
         out["lists_%d_executed" % seed] = ex
+    for dtype, vr, vc, seed in sc.SORT32_CASES_16:
+        src, idx, o = sc.sort32_inputs_16(dtype, vr, vc, seed)
+        (ref.ref_tsort32_f16_8x128 if dtype == "f16" else ref.ref_tsort32_s16_8x128)(p(o), p(src), p(idx), vr, vc)
+        out["sort32_%d" % seed] = o.view(np.uint16)
+    for dtype, valid_cols, block_len, seed in sc.BLOCK_CASES_16:
+        src, o = sc.block_inputs_16(dtype, valid_cols, block_len, seed)
+        ref.ref_tmrgsort_blocks_16_1x2048(p(o), p(src), valid_cols, block_len, sc.DT16[dtype])
+        out["blocks_%d" % seed] = o.view(np.uint16)
+    for dtype, counts, out_structs, exhausted, seed in sc.LIST_CASES_16:
+        lists, o = sc.list_inputs_16(dtype, counts, seed)
+        ex = np.zeros(4, dtype=np.uint32)
+        ptrs = [p(l) for l in lists] + [None] * (4 - len(lists))
+        cols = [4 * n for n in counts] + [0] * (4 - len(counts))
+        ref.ref_tmrgsort_lists_16(p(o), p(ex), *ptrs, *cols, 4 * out_structs, len(counts), exhausted, sc.DT16[dtype])
+        out["lists_%d" % seed] = o.view(np.uint16)
+        out["lists_%d_executed" % seed] = ex
     for n, (op, dv, av, bv) in enumerate(sc.PART_CASES):
         a, b, o = sc.part_inputs(n)
         ref.ref_tpart_f32_64x128(p(o), p(a), p(b), op, *dv, *av, *bv)

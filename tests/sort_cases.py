@@ -62,6 +62,77 @@ def list_inputs(counts, seed):
     return lists, np.full(1024, -555.0, dtype=np.float32)
 
 
+# ---- 2-byte elements: four to a structure (score, 0 / payload, index low, index high) ----
+NP16 = {"f16": np.float16, "s16": np.int16, "u16": np.uint16}
+DT16 = {"f16": 0, "u16": 1, "s16": 2}          # dtype argument of the 16-bit TMRGSORT programs
+SORT32_CASES_16 = [("f16", 8, 32, 20), ("f16", 5, 17, 21), ("s16", 8, 32, 22), ("s16", 3, 16, 23), ("f16", 8, 128, 24),
+                   ("s16", 7, 100, 25)]
+
+
+def sort32_inputs_16(dtype, vr, vc, seed):
+    """src [8,128] fp16 / int16, idx [8,128] uint32, out0 [8,512]; ties, repeated indices, signed zeros, indices above 2^16."""
+    rng = np.random.default_rng(500 + seed)
+    if dtype == "f16":
+        src = (rng.integers(-12, 13, size=(8, 128)) * 0.25).astype(np.float16)
+        src[0, 3], src[0, 9] = -0.0, 0.0
+        src[1, :3] = [65504.0, -65504.0, 6.0e-8]
+        out0 = np.full((8, 512), -777.0, dtype=np.float16)
+    else:
+        src = rng.integers(-6, 7, size=(8, 128)).astype(np.int16)
+        src[1, :4] = [32767, -32768, 0, -1]
+        out0 = np.full((8, 512), -777, dtype=np.int16)
+    idx = rng.integers(0, 40, size=(8, 128)).astype(np.uint32)
+    idx[2, :] = np.arange(128, dtype=np.uint32) + 3000000000
+    idx[3, :] = np.arange(128, dtype=np.uint32) * 1031 + 70000
+    return src, idx, out0
+
+
+def sorted_list_16(rng, n, dtype, tag=0):
+    """n structures [score, payload, position, list tag] of 2-byte elements in descending order of score, with ties."""
+    np_t = NP16[dtype]
+    if dtype == "f16":
+        scores = np.sort((rng.integers(-8, 9, size=n) * 0.5).astype(np.float16))[::-1]
+    elif dtype == "u16":
+        scores = np.sort(rng.integers(0, 12, size=n).astype(np.uint16) * np.uint16(6000))[::-1]      # values above 32767: unsigned order
+    else:
+        scores = np.sort(rng.integers(-8, 9, size=n).astype(np.int16) * np.int16(4000))[::-1]
+    out = np.empty((n, 4), dtype=np.uint16)
+    out[:, 0] = scores.view(np.uint16)
+    out[:, 1] = 0xA000 + tag
+    out[:, 2] = np.arange(n, dtype=np.uint16)
+    out[:, 3] = 100 * tag + 7
+    return out.view(np_t)
+
+
+BLOCK_CASES_16 = [("u16", 2048, 256, 30), ("u16", 1024, 64, 31), ("f16", 2048, 512, 32), ("f16", 1400, 128, 33), ("s16", 2048, 16, 34),
+                  ("u16", 100, 64, 35), ("f16", 2048, 6, 36)]
+
+
+def block_inputs_16(dtype, valid_cols, block_len, seed):
+    rng = np.random.default_rng(600 + seed)
+    src = np.zeros(2048, dtype=NP16[dtype])
+    if block_len % 4 == 0:
+        for b in range(2048 // block_len):
+            src[b * block_len:(b + 1) * block_len] = sorted_list_16(rng, block_len // 4, dtype, tag=b).reshape(-1)
+    return src, np.full(2048, 555, dtype=np.uint16).view(NP16[dtype])
+
+
+# (dtype, structures per list, out structures, exhausted, seed)
+LIST_CASES_16 = [("u16", (128, 128, 128, 128), 512, 0, 40), ("u16", (64, 64, 64), 192, 1, 41), ("f16", (100, 7, 64, 33), 204, 1, 42),
+                 ("f16", (64, 128), 100, 0, 43), ("f16", (5, 0, 9, 3), 17, 1, 44), ("u16", (128, 90, 50), 268, 0, 45),
+                 ("f16", (128, 128, 128, 128), 512, 1, 46)]
+
+
+def list_inputs_16(dtype, counts, seed):
+    rng = np.random.default_rng(700 + seed)
+    lists = []
+    for b, n in enumerate(counts):
+        l = np.full(512, 123, dtype=np.uint16).view(NP16[dtype])
+        l[:4 * n] = sorted_list_16(rng, n, dtype, tag=b).reshape(-1)
+        lists.append(l)
+    return lists, np.full(2048, 555, dtype=np.uint16).view(NP16[dtype])
+
+
 # TPARTADD / TPARTMAX / TPARTMIN: (op, dst valid, a valid, b valid)
 PART_CASES = [(0, (64, 128), (64, 128), (64, 128)), (0, (64, 128), (40, 128), (64, 70)), (1, (50, 100), (64, 60), (30, 128)),
               (2, (64, 128), (10, 20), (64, 128)), (1, (64, 128), (0, 0), (33, 77)), (2, (20, 30), (64, 128), (5, 128)),

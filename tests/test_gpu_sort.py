@@ -71,6 +71,51 @@ def test_tmrgsort_lists(oracle, counts, out_structs, exhausted, seed):
     assert np.array_equal(got, GOLD["lists_%d" % seed]) and np.array_equal(ex, GOLD["lists_%d_executed" % seed])
 
 
+@pytest.mark.parametrize("dtype,vr,vc,seed", sc.SORT32_CASES_16)
+def test_tsort32_16bit(oracle, dtype, vr, vc, seed):
+    """fp16 / int16 scores: structures of four elements (score, 0, index & 0xffff, index >> 16), the index as its bits."""
+    lib = capi.load_st()
+    src, idx, out0 = sc.sort32_inputs_16(dtype, vr, vc, seed)
+    ts, ti, to = _dev(src.view(np.int16)), _dev(idx), _dev(out0.view(np.int16))
+    capi.check(lib.pto_st_tsort32_8x128(_st(), to.data_ptr(), ts.data_ptr(), ti.data_ptr(), vr, vc, 2 if dtype == "f16" else 3), "tsort32")
+    torch.cuda.synchronize()
+    got = to.cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, oracle.tsort32(out0, src, idx, vr, vc).view(np.uint16))
+    if dtype == "s16" and vc <= 32:          # there the CPU simulation's by-value form is the same thing
+        assert np.array_equal(got, GOLD["sort32_%d" % seed])
+
+
+@pytest.mark.parametrize("dtype,valid_cols,block_len,seed", sc.BLOCK_CASES_16)
+def test_tmrgsort_blocks_16bit(oracle, dtype, valid_cols, block_len, seed):
+    lib = capi.load_st()
+    src, out0 = sc.block_inputs_16(dtype, valid_cols, block_len, seed)
+    ts, to = _dev(src.view(np.int16)), _dev(out0.view(np.int16))
+    capi.check(lib.pto_st_tmrgsort_blocks_16_1x2048(_st(), to.data_ptr(), ts.data_ptr(), valid_cols, block_len, sc.DT16[dtype]), "tmrgsort blocks")
+    torch.cuda.synchronize()
+    got = to.cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, oracle.tmrgsort_blocks(out0, src, valid_cols, block_len).view(np.uint16))
+    assert np.array_equal(got, GOLD["blocks_%d" % seed])
+
+
+@pytest.mark.parametrize("dtype,counts,out_structs,exhausted,seed", sc.LIST_CASES_16)
+def test_tmrgsort_lists_16bit(oracle, dtype, counts, out_structs, exhausted, seed):
+    lib = capi.load_st()
+    lists, out0 = sc.list_inputs_16(dtype, counts, seed)
+    tl = [_dev(l.view(np.int16)) for l in lists]
+    to = _dev(out0.view(np.int16))
+    tex = torch.full((4,), -1, dtype=torch.int32, device="cuda:0")
+    ptrs = [t.data_ptr() for t in tl] + [0] * (4 - len(tl))
+    cols = [4 * n for n in counts] + [0] * (4 - len(counts))
+    capi.check(lib.pto_st_tmrgsort_lists_16(_st(), to.data_ptr(), tex.data_ptr(), *ptrs, *cols, 4 * out_structs, len(counts), exhausted,
+                                            sc.DT16[dtype]), "tmrgsort lists")
+    torch.cuda.synchronize()
+    got, ex = to.cpu().numpy().view(np.uint16), tex.cpu().numpy().view(np.uint32)
+    want, want_ex = oracle.tmrgsort_lists(out0, lists, cols[:len(counts)], 4 * out_structs, exhausted)
+    assert np.array_equal(ex, want_ex)
+    assert np.array_equal(got, want.view(np.uint16))
+    assert np.array_equal(got, GOLD["lists_%d" % seed]) and np.array_equal(ex, GOLD["lists_%d_executed" % seed])
+
+
 @pytest.mark.parametrize("n", range(len(sc.PART_CASES)))
 def test_tpart(oracle, n):
     lib = capi.load_st()

@@ -59,6 +59,75 @@ def test_tmrgsort_blocks_vs_reference_and_stable_sort(oracle, valid_cols, block_
     assert np.array_equal(got[done:], out0[done:])
 
 
+@pytest.mark.parametrize("dtype,vr,vc,seed", sc.SORT32_CASES_16)
+def test_tsort32_16bit_vs_reference_and_lexsort(oracle, dtype, vr, vc, seed):
+    """2-byte scores: the by-value form (with the CPU simulation's group offset 2 j) against the compiled reference's
+    committed outputs; the bit-pattern form, four elements a structure at 4 j, against numpy's lexsort."""
+    src, idx, out0 = sc.sort32_inputs_16(dtype, vr, vc, seed)
+    got = oracle.tsort32(out0, src, idx, vr, vc, index_as_value=True)
+    assert np.array_equal(got.view(np.uint16), GOLD["sort32_%d" % seed])
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        (r.ref_tsort32_f16_8x128 if dtype == "f16" else r.ref_tsort32_s16_8x128)(_p(o), _p(src), _p(idx), vr, vc)
+        assert np.array_equal(o.view(np.uint16), got.view(np.uint16))
+    bits = oracle.tsort32(out0, src, idx, vr, vc)
+    if dtype == "s16" and vc <= 32:          # integer conversions keep the bits and one group has nothing to overlap: the two forms agree
+        assert np.array_equal(bits, got)
+    for row in range(vr):
+        for j in range(0, vc, 32):
+            n = min(32, vc - j)
+            order = np.lexsort((np.arange(n), idx[row, j:j + n], -src[row, j:j + n].astype(np.float64)))
+            st = bits[row, 4 * j:4 * (j + n)].reshape(n, 4)
+            assert np.array_equal(st[:, 0], src[row, j + order])
+            assert not st[:, 1].view(np.uint16).any()
+            assert np.array_equal(st[:, 2:].copy().view(np.uint16).astype(np.uint32) @ np.array([1, 65536], dtype=np.uint32),
+                                  idx[row, j + order])
+    assert np.array_equal(bits[vr:], out0[vr:]) and np.array_equal(bits[:, 4 * vc:], out0[:, 4 * vc:])
+
+
+@pytest.mark.parametrize("dtype,valid_cols,block_len,seed", sc.BLOCK_CASES_16)
+def test_tmrgsort_blocks_16bit_vs_reference_and_stable_sort(oracle, dtype, valid_cols, block_len, seed):
+    src, out0 = sc.block_inputs_16(dtype, valid_cols, block_len, seed)
+    got = oracle.tmrgsort_blocks(out0, src, valid_cols, block_len)
+    assert np.array_equal(got.view(np.uint16), GOLD["blocks_%d" % seed])
+    r = oracle.ref()
+    if r is not None:
+        o = out0.copy()
+        r.ref_tmrgsort_blocks_16_1x2048(_p(o), _p(src), valid_cols, block_len, sc.DT16[dtype])
+        assert np.array_equal(o.view(np.uint16), got.view(np.uint16))
+    done = 0
+    if block_len % 4 == 0:                   # a block length that is not whole structures merges nothing
+        group = 4 * block_len
+        done = valid_cols // group * group
+        for c in range(0, done, group):
+            st = src[c:c + group].reshape(-1, 4)
+            order = np.argsort(-st[:, 0].astype(np.float64), kind="stable")      # uint16 scores order as unsigned numbers
+            assert np.array_equal(got[c:c + group].view(np.uint16), st[order].reshape(-1).view(np.uint16))
+    assert np.array_equal(got[done:], out0[done:])
+
+
+@pytest.mark.parametrize("dtype,counts,out_structs,exhausted,seed", sc.LIST_CASES_16)
+def test_tmrgsort_lists_16bit_vs_reference_and_stable_sort(oracle, dtype, counts, out_structs, exhausted, seed):
+    lists, out0 = sc.list_inputs_16(dtype, counts, seed)
+    got, ex = oracle.tmrgsort_lists(out0, lists, [4 * n for n in counts], 4 * out_structs, exhausted)
+    assert np.array_equal(got.view(np.uint16), GOLD["lists_%d" % seed])
+    assert np.array_equal(ex, GOLD["lists_%d_executed" % seed])
+    r = oracle.ref()
+    if r is not None:
+        o, e = out0.copy(), np.zeros(4, dtype=np.uint32)
+        ptrs = [_p(l) for l in lists] + [None] * (4 - len(lists))
+        cols = [4 * n for n in counts] + [0] * (4 - len(counts))
+        r.ref_tmrgsort_lists_16(_p(o), _p(e), *ptrs, *cols, 4 * out_structs, len(counts), exhausted, sc.DT16[dtype])
+        assert np.array_equal(o.view(np.uint16), got.view(np.uint16)) and np.array_equal(e, ex)
+    cat = np.concatenate([l[:4 * n].reshape(-1, 4) for l, n in zip(lists, counts)])
+    full = cat[np.argsort(-cat[:, 0].astype(np.float64), kind="stable")] if len(cat) else cat
+    taken = int(ex.sum())
+    assert taken <= min(out_structs, len(cat))
+    assert np.array_equal(got[:4 * taken].view(np.uint16), full[:taken].reshape(-1).view(np.uint16))
+    assert np.array_equal(got[4 * taken:], out0[4 * taken:])
+
+
 @pytest.mark.parametrize("counts,out_structs,exhausted,seed", sc.LIST_CASES)
 def test_tmrgsort_lists_vs_reference_and_stable_sort(oracle, counts, out_structs, exhausted, seed):
     lists, out0 = sc.list_inputs(counts, seed)
