@@ -271,45 +271,72 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
                     }
             }
         }
-        anyRaise = t == 0;
+        // The running max only has to bound the scores well enough to keep exp() in range: it is raised (and O, S
+        // rescaled by alpha) when a tile exceeds it by more than kSlack in the exponent, i.e. P stays below 2^kSlack.
+        // O / S and max*s + ln(S) do not depend on the choice.
+        // Every tile but the first is tried with the running max as it stands.  A lane's partial row sum bounds each
+        // of its P from above, so a sum of at most 2^kSlack proves that no score of the tile exceeds the running max
+        // by more than the slack: the max stays, nothing is rescaled, and the row max of the tile is never computed.
+        // Otherwise (a larger sum, an infinity or a NaN in any lane of the wave) the wave finds the row max, raises
+        // the running max where it has to, and runs the exponentials a second time.
+        constexpr float kSlack = 8.0f;
+        anyRaise = false;
+        float locSum[NQ];
 #pragma unroll
-        for (int nb = 0; nb < NQ; ++nb) {
-            float locMax = sAcc[0].st.f[0][nb][0];
+        for (int nb = 0; nb < NQ; ++nb)
+            alpha[nb] = 1.0f;
+        bool needMax = t == 0; // wave-uniform
+#pragma nounroll
+        for (;;) {             // at most two rounds
+            if (needMax) {
+                anyRaise = t == 0;
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
+                for (int nb = 0; nb < NQ; ++nb) {
+                    float locMax = sAcc[0].st.f[0][nb][0];
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    locMax = fmaxf(locMax, sAcc[kb].st.f[0][nb][v]);
-            locMax = MaxOverHalves(locMax);
-            // The running max only has to bound the scores well enough to keep exp() in range: it is
-            // raised (and O, S rescaled by alpha) when a tile exceeds it by more than kSlack in the
-            // exponent, i.e. P stays below 2^kSlack.  O / S and max*s + ln(S) do not depend on the choice.
-            constexpr float kSlack = 8.0f;
-            const bool raise = t == 0 || (locMax - runMax[nb]) * sLog2e > kSlack;
-            const float newMax = raise ? locMax : runMax[nb];
-            if (t > 0)
-                anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
-            alpha[nb] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nb] - newMax) * sLog2e);
-            runMax[nb] = newMax;
-            const float negMax = -newMax * sLog2e;
-            float part[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // four partial sums: no long chain of dependent additions
+                    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int half_ = 0; half_ < 2; ++half_) {
-                    f16x8 pk;
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const float p =
-                            __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][nb][half_ * 8 + j], sLog2e, negMax));
-                        part[j & 3] += p; // row sum over the fp32 P, as the reference does
-                        pk[j] = (half)p;
-                    }
-                    pRight.st.f[nb][kb * 2 + half_] = pk;
+                        for (int v = 0; v < 16; ++v)
+                            locMax = fmaxf(locMax, sAcc[kb].st.f[0][nb][v]);
+                    locMax = MaxOverHalves(locMax);
+                    const bool raise = t == 0 || (locMax - runMax[nb]) * sLog2e > kSlack;
+                    const float newMax = raise ? locMax : runMax[nb];
+                    if (t > 0)
+                        anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
+                    alpha[nb] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nb] - newMax) * sLog2e);
+                    runMax[nb] = newMax;
                 }
-            const float locSum = (part[0] + part[1]) + (part[2] + part[3]);
-            runSum[nb] = t == 0 ? locSum : runSum[nb] * alpha[nb] + locSum;
+            }
+            bool within = true;
+#pragma unroll
+            for (int nb = 0; nb < NQ; ++nb) {
+                const float negMax = -runMax[nb] * sLog2e;
+                float part[4] = {0.0f, 0.0f, 0.0f, 0.0f}; // four partial sums: no long chain of dependent additions
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                    for (int half_ = 0; half_ < 2; ++half_) {
+                        f16x8 pk;
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const float p =
+                                __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[kb].st.f[0][nb][half_ * 8 + j], sLog2e, negMax));
+                            part[j & 3] += p; // row sum over the fp32 P, as the reference does
+                            pk[j] = (half)p;
+                        }
+                        pRight.st.f[nb][kb * 2 + half_] = pk;
+                    }
+                locSum[nb] = (part[0] + part[1]) + (part[2] + part[3]);
+                within = within && locSum[nb] <= 256.0f; // 2^kSlack; false for a NaN
+            }
+            static_assert(kSlack == 8.0f, "the bound above is 2^kSlack");
+            if (needMax || __builtin_amdgcn_ballot_w64(!within) == 0)
+                break;
+            needMax = true;
         }
+#pragma unroll
+        for (int nb = 0; nb < NQ; ++nb)
+            runSum[nb] = t == 0 ? locSum[nb] : runSum[nb] * alpha[nb] + locSum[nb];
     };
     using VT = VTReader<D, kBKV>;
     VT vt;

@@ -227,39 +227,65 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE void FlashAttnFwdM16(__gm_
                     }
             }
         }
-        anyRaise = t == 0;
+        // The running max is raised lazily and every tile but the first is tried with the running max as it stands, as in
+        // fa_kernels.hpp: a lane's partial row sum of at most 2^kSlack proves that none of its P exceeds 2^kSlack, and
+        // the row max of the tile is then never computed; otherwise the wave finds the row max and runs the
+        // exponentials a second time.
+        constexpr float kSlack = 8.0f;
+        anyRaise = false;
+        float locSum[NQ];
 #pragma unroll
-        for (int nq = 0; nq < NQ; ++nq) {
-            float locMax = sAcc[0][nq][0];
+        for (int nq = 0; nq < NQ; ++nq)
+            alpha[nq] = 1.0f;
+        bool needMax = t == 0; // wave-uniform
+#pragma nounroll
+        for (;;) {             // at most two rounds
+            if (needMax) {
+                anyRaise = t == 0;
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
+                for (int nq = 0; nq < NQ; ++nq) {
+                    float locMax = sAcc[0][nq][0];
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    locMax = fmaxf(locMax, sAcc[kb][nq][v]);
-            locMax = MaxOverRowGroups(locMax);
-            constexpr float kSlack = 8.0f; // the running max is raised lazily, as in fa_kernels.hpp
-            const bool raise = t == 0 || (locMax - runMax[nq]) * sLog2e > kSlack;
-            const float newMax = raise ? locMax : runMax[nq];
-            if (t > 0)
-                anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
-            alpha[nq] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nq] - newMax) * sLog2e);
-            runMax[nq] = newMax;
-            const float negMax = -newMax * sLog2e;
-            float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+                    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-            for (int kt = 0; kt < KT; ++kt) {
-                f16x8 pk;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[2 * kt + j / 4][nq][j % 4], sLog2e, negMax));
-                    part[j & 3] += p; // row sum over the fp32 P, as the reference does
-                    pk[j] = (half)p;
+                        for (int v = 0; v < 4; ++v)
+                            locMax = fmaxf(locMax, sAcc[kb][nq][v]);
+                    locMax = MaxOverRowGroups(locMax);
+                    const bool raise = t == 0 || (locMax - runMax[nq]) * sLog2e > kSlack;
+                    const float newMax = raise ? locMax : runMax[nq];
+                    if (t > 0)
+                        anyRaise = anyRaise || __builtin_amdgcn_ballot_w64(raise) != 0;
+                    alpha[nq] = (t == 0 || !raise) ? 1.0f : __builtin_amdgcn_exp2f((runMax[nq] - newMax) * sLog2e);
+                    runMax[nq] = newMax;
                 }
-                pRight[kt][nq] = pk;
             }
-            const float locSum = (part[0] + part[1]) + (part[2] + part[3]);
-            runSum[nq] = t == 0 ? locSum : runSum[nq] * alpha[nq] + locSum;
+            bool within = true;
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq) {
+                const float negMax = -runMax[nq] * sLog2e;
+                float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                for (int kt = 0; kt < KT; ++kt) {
+                    f16x8 pk;
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sAcc[2 * kt + j / 4][nq][j % 4], sLog2e, negMax));
+                        part[j & 3] += p; // row sum over the fp32 P, as the reference does
+                        pk[j] = (half)p;
+                    }
+                    pRight[kt][nq] = pk;
+                }
+                locSum[nq] = (part[0] + part[1]) + (part[2] + part[3]);
+                within = within && locSum[nq] <= 256.0f; // 2^kSlack; false for a NaN
+            }
+            static_assert(kSlack == 8.0f, "the bound above is 2^kSlack");
+            if (needMax || __builtin_amdgcn_ballot_w64(!within) == 0)
+                break;
+            needMax = true;
         }
+#pragma unroll
+        for (int nq = 0; nq < NQ; ++nq)
+            runSum[nq] = t == 0 ? locSum[nq] : runSum[nq] * alpha[nq] + locSum[nq];
     };
     // ---- O^T += V^T P^T.  One step = four head-dim blocks of one 32-key step: 8 transposing reads, 8 MFMAs ----
     struct VStep {

@@ -48,6 +48,7 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
     PTO_FA_VARIANT(1, 64, true, 1)
     PTO_FA_VARIANT(2, 64, true, 2)
     PTO_FA_VARIANT(5, 64, true, 3)
+    PTO_FA_VARIANT(7, 64, true, 4)
 #undef PTO_FA_VARIANT
     if (variant == 10 && head_dim == 128)
         return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false, causalOff);

@@ -192,6 +192,36 @@ def test_fa_d128_eight_wave_kernel_on_16x16x32_vs_streaming_oracle(oracle):
         assert np.max(np.abs(lse[b, h] - (m / np.sqrt(D) + np.log(l)))) <= 1e-4
 
 
+@pytest.mark.parametrize("B,H,Sq,Skv,D,causal", [(1, 2, 128, 512, 64, False), (1, 2, 256, 512, 64, True), (1, 2, 128, 512, 128, False),
+                                                 (16, 16, 256, 512, 128, False), (16, 16, 256, 512, 128, True),
+                                                 (1, 16, 4096, 4096, 128, False)])
+def test_fa_running_max_raised_in_later_tiles(B, H, Sq, Skv, D, causal):
+    """Scores that grow along the keys: a tile tried with the running max of the tiles before it overshoots the slack, so
+    the kernels must fall back to the row max, raise the running max and rescale O and S (every kernel variant: four
+    waves at head_dim 64 and 128, eight waves on 32 x 32 x 16 and on 16 x 16 x 32 MFMAs).  Half of the query rows get flat
+    scores, so waves whose lanes disagree about the fallback are covered as well."""
+    rng = np.random.default_rng(77)
+    q, k, v = datagen.fa_inputs(B, H, Sq, Skv, D, scale=1.0)
+    ramp = (1.0 + 7.0 * np.arange(Skv) / Skv).astype(np.float32)[None, None, :, None]
+    k = (np.sign(k.astype(np.float32)) * 0.6 * ramp).astype(np.float16)           # |q.k| grows eightfold towards the last keys
+    q = np.abs(q.astype(np.float32)).astype(np.float16)
+    q[:, :, 1::2, :] = (q[:, :, 1::2, :].astype(np.float32) * 0.02).astype(np.float16)   # odd rows: nearly flat scores
+    k[:, :, :, D // 2:] = np.abs(k[:, :, :, D // 2:])                              # scores with a positive drift
+    o, lse = fa_gpu(q, k, v, causal=causal, o_fp32=True)
+    assert np.all(np.isfinite(o)) and np.all(np.isfinite(lse))
+    for b, h in ((0, 0), (B - 1, H - 1)):
+        rows = np.sort(np.r_[0, 1, Sq - 2, Sq - 1, rng.integers(0, Sq, size=28)]) if Sq > 512 else np.arange(Sq)
+        if causal:
+            want, want_lse = dense_fp64(q[b, h], k[b, h], v[b, h], causal=True)
+            want, want_lse = want[rows], want_lse[rows]
+        else:
+            want, want_lse = rows_fp64(q[b, h], k[b, h], v[b, h], rows)
+        scores = (q[b, h][rows].astype(np.float64) @ k[b, h].astype(np.float64).T) / np.sqrt(D)
+        assert np.max(scores[:, -64:].max(axis=1) - scores[:, :64].max(axis=1)) > 12.0     # the case does what it says
+        assert rel(o[b, h][rows], want) <= TOL
+        assert np.max(np.abs(lse[b, h][rows] - want_lse)) <= 1e-3
+
+
 def test_fa_config4_causal_b4_h32_s2048_d64():
     """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row."""
     B, H, S, D = 4, 32, 2048, 64
