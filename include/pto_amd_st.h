@@ -30,7 +30,9 @@ int pto_gemm_f16f32_k64_variant(void *stream, float *c, const uint16_t *a, const
 /* MX GEMM: variant bit 0 = quarter tiles in the last round, bit 1 = the shallower copy pipeline (csrc/pto_gemm_mx.hip) */
 int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                            const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant);
-/* flash attention: workgroup size, occupancy and MFMA shape by number (csrc/pto_fa.hip); causal as in pto_fa_fwd_f16 */
+/* flash attention: workgroup size, occupancy, queries per wave and MFMA shape by number (csrc/pto_fa.hip: 1 / 2 / 5 = four
+ * waves at 1 / 2 / 3 workgroups per compute unit, 6 = key tiles of 32, 8 = 64 queries per wave, 10 / 20 / 21 = eight waves on
+ * 32 x 32 x 16 / 16 x 16 x 32 MFMAs / the latter with fp32 output); causal != 0: the diagonal ends in the last key */
 int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const uint16_t *q, const uint16_t *k, const uint16_t *v,
                            int batch, int heads, int seq_q, int seq_kv, int head_dim, int causal, int variant);
 

@@ -138,13 +138,13 @@ struct VTReader {
     }
 };
 
-template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int kBKV = kBKVDefault, bool PP = false>
+template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS, int kBKV = kBKVDefault, bool PP = false, int NQ_ = 1>
 __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd(__gm__ void *outO, __gm__ float *outLse,
                                                                       __gm__ const half *qAll, __gm__ const half *kAll,
                                                                       __gm__ const half *vAll, int heads, int seqQ,
                                                                       int seqKv, int numBH, int causalOff)
 {
-    constexpr int NQ = 1;          // 32-query blocks per wave
+    constexpr int NQ = NQ_;        // 32-query blocks per wave
     constexpr int kBQ = kBQ1 * NQ; // queries per workgroup
     constexpr int KB = kBKV / 32;  // 32-key blocks per tile
     constexpr int DB = D / 32;    // 32-wide blocks of the head dimension
@@ -417,7 +417,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
         const int tc = t < numTiles ? t : numTiles - 1; // past the end: re-fetch the last tile (nobody reads it)
         return GlobalKV(base + (int64_t)tc * kBKV * D);
     };
-    constexpr int kScoreMfma = KB * NQ * (D / 16);
+    constexpr int kScoreFrags = KB * (D / 16); // K fragments of one tile = calls of the score stage's hook
 
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -533,7 +533,7 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
                 GlobalKV gmK = keyTile(kBase, t + 1);
                 TLOAD(kMat[st ^ 1], gmK);
             }
-            if constexpr (I == kScoreMfma / 2 + 1) {
+            if constexpr (I == kScoreFrags / 2 + 1) {
                 GlobalKV gmV = keyTile(vBase, t + 1);
                 TLOAD(vMat[st ^ 1], gmV);
                 set_flag(PIPE_MTE2, PIPE_MTE1, EVENT_ID0);
@@ -589,20 +589,21 @@ __global__ __launch_bounds__(kBlockThreads, MIN_BLOCKS) AICORE void FlashAttnFwd
 PTO_DEVICE_CODE_END
 
 namespace {
-template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS = 1, int kBKV = kBKVDefault, bool PP = false>
+template <int D, bool CAUSAL, bool OUT_F32, int MIN_BLOCKS = 1, int kBKV = kBKVDefault, bool PP = false, int NQ = 1>
 int launch_fa(hipStream_t st, void *o, float *lse, const half *q, const half *k, const half *v, int batch, int heads,
               int seqQ, int seqKv, int causalOff)
 {
-    if (seqQ % kBQ1 || seqKv % kBKV)
+    constexpr int kBQ = kBQ1 * NQ;
+    if (seqQ % kBQ || seqKv % kBKV)
         return PTO_ERR_UNSUPPORTED;
-    static_assert(D * kBQ1 <= 4 * kBKV * D, "Q^T must fit the K/V stages it is staged in");
+    static_assert(D * kBQ <= 4 * kBKV * D, "Q^T must fit the K/V stages it is staged in");
     constexpr int lds = 2 * 2 * kBKV * D * (int)sizeof(half);
-    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32, MIN_BLOCKS, kBKV, PP>;
+    auto kernel = FlashAttnFwd<D, CAUSAL, OUT_F32, MIN_BLOCKS, kBKV, PP, NQ>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
     const int numBH = batch * heads;
-    const long long blocks = (long long)numBH * (seqQ / kBQ1);
+    const long long blocks = (long long)numBH * (seqQ / kBQ);
     if (blocks > 0x7fffffffLL)
         return PTO_ERR_UNSUPPORTED;
     kernel<<<dim3((unsigned)blocks), dim3(kBlockThreads), lds, st>>>(o, lse, q, k, v, heads, seqQ, seqKv, numBH, causalOff);

@@ -48,7 +48,6 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
     PTO_FA_VARIANT(1, 64, true, 1)
     PTO_FA_VARIANT(2, 64, true, 2)
     PTO_FA_VARIANT(5, 64, true, 3)
-    PTO_FA_VARIANT(7, 64, true, 4)
 #undef PTO_FA_VARIANT
     if (variant == 10 && head_dim == 128)
         return pto_amd::fa_fwd_d128_w8(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causal != 0, false, causalOff);
@@ -60,6 +59,10 @@ extern "C" int pto_fa_fwd_f16_variant(void *stream, void *o, float *lse, const u
         return launch_fa<128, false, false, 2, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     if (variant == 6 && head_dim == 64 && causal)
         return launch_fa<64, true, false, 3, 32>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
+    if (variant == 8 && head_dim == 64 && causal) // 64 queries per wave
+        return launch_fa<64, true, false, 2, 64, false, 2>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
+    if (variant == 8 && head_dim == 64 && !causal)
+        return launch_fa<64, false, false, 2, 64, false, 2>(st, o, lse, hq, hk, hv, batch, heads, seq_q, seq_kv, causalOff);
     return PTO_ERR_BAD_ARG;
 }
 #endif // PTO_ST_HOOKS

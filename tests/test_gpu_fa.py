@@ -222,6 +222,27 @@ def test_fa_running_max_raised_in_later_tiles(B, H, Sq, Skv, D, causal):
         assert np.max(np.abs(lse[b, h][rows] - want_lse)) <= 1e-3
 
 
+@pytest.mark.parametrize("D,causal,variant", [(64, True, 5), (64, True, 8), (64, False, 8), (128, False, 2), (128, True, 10), (128, False, 20)])
+def test_fa_kernel_variants_of_the_test_library(D, causal, variant):
+    """The kernels the dispatch chooses between, each called by number through the test library: four waves (variant 2 / 5),
+    64 queries per wave (8), eight waves on 32 x 32 x 16 (10) and on 16 x 16 x 32 MFMAs (20)."""
+    from gpu_util import to_dev, stream
+    lib = capi.load_st()
+    B, H, S = 1, 2, 512
+    q, k, v = datagen.fa_inputs(B, H, S, S, D, scale=1.0)
+    tq, tk, tv = to_dev(q), to_dev(k), to_dev(v)
+    to = torch.full((B, H, S, D), float("nan"), dtype=torch.float16, device="cuda:0")
+    tl = torch.full((B, H, S), float("nan"), dtype=torch.float32, device="cuda:0")
+    capi.check(lib.pto_fa_fwd_f16_variant(stream(), to.data_ptr(), tl.data_ptr(), tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), B, H, S, S, D,
+                                          int(causal), variant), "pto_fa_fwd_f16_variant")
+    torch.cuda.synchronize()
+    o, lse = to.cpu().numpy().astype(np.float32), tl.cpu().numpy()
+    for h in range(H):
+        want, want_lse = dense_fp64(q[0, h], k[0, h], v[0, h], causal=causal)
+        assert rel(o[0, h], want) <= TOL
+        assert np.max(np.abs(lse[0, h] - want_lse)) <= 1e-3
+
+
 def test_fa_config4_causal_b4_h32_s2048_d64():
     """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row."""
     B, H, S, D = 4, 32, 2048, 64
