@@ -83,14 +83,16 @@ __device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
                     for (int e = 0; e < E; ++e)
                         other[e] = LaneXor64<j / E>(k[e], lane);
                 } else {
+                    // partners are E (j / E) ranks apart: the same register of thread tid ^ (j / E).  Register e of all
+                    // threads is one contiguous run of LDS, so a wave's 64 lanes touch 64 consecutive 8-byte words
                     __syncthreads(); // everyone is done reading the previous exchange
 #pragma unroll
                     for (int e = 0; e < E; ++e)
-                        lds[tid * E + e] = k[e];
+                        lds[e * kTopkThreads + tid] = k[e];
                     __syncthreads();
 #pragma unroll
                     for (int e = 0; e < E; ++e)
-                        other[e] = lds[(tid * E + e) ^ j];
+                        other[e] = lds[e * kTopkThreads + (tid ^ (j / E))];
                 }
                 // the lower rank of a pair keeps the larger key where the run is descending
                 const bool lower = ((tid * E) & j) == 0, descending = ((tid * E) & kk) == 0;
