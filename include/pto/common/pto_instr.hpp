@@ -266,45 +266,60 @@ PTO_INST RecordEvent TCI(TileT &dst, T start, Ev &... ev)
     return {};
 }
 
-// TSORT32 (pto_instr.hpp:786-798 of the reference; it takes no events) and TMRGSORT (pto_instr.hpp:582-622)
+// TSORT32 (pto_instr.hpp:786-798 of the reference; it takes no events) and TMRGSORT (pto_instr.hpp:582-622).  Both leave
+// parts of the destination as they were, so the destination is fetched as well where Vec tiles live in memory; the
+// sources may alias it (the reference's top-k kernel merges in place, topk_kernel.cpp:77-82): every operand is in
+// registers before the instruction runs.
 template <typename D, typename S, typename I>
 PTO_INST RecordEvent TSORT32(D &dst, S &src, I &idx)
 {
+    detail::UbFetch(dst, src, idx);
     TSORT32_IMPL(dst, src, idx);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename S, typename I, typename Tmp>
 PTO_INST RecordEvent TSORT32(D &dst, S &src, I &idx, Tmp &tmp)
 {
+    detail::UbFetch(dst, src, idx);
     TSORT32_IMPL(dst, src, idx, tmp);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename Tmp, typename S0, typename S1, typename S2, typename S3, bool exhausted, typename... Ev>
 PTO_INST RecordEvent TMRGSORT(D &dst, MrgSortExecutedNumList &executed, Tmp &tmp, S0 &src0, S1 &src1, S2 &src2, S3 &src3, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src0, src1, src2, src3);
     TMRGSORT_IMPL<D, Tmp, S0, S1, S2, S3, exhausted>(dst, executed, tmp, src0, src1, src2, src3);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename Tmp, typename S0, typename S1, typename S2, bool exhausted, typename... Ev>
 PTO_INST RecordEvent TMRGSORT(D &dst, MrgSortExecutedNumList &executed, Tmp &tmp, S0 &src0, S1 &src1, S2 &src2, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src0, src1, src2);
     TMRGSORT_IMPL<D, Tmp, S0, S1, S2, exhausted>(dst, executed, tmp, src0, src1, src2);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename Tmp, typename S0, typename S1, bool exhausted, typename... Ev>
 PTO_INST RecordEvent TMRGSORT(D &dst, MrgSortExecutedNumList &executed, Tmp &tmp, S0 &src0, S1 &src1, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src0, src1);
     TMRGSORT_IMPL<D, Tmp, S0, S1, exhausted>(dst, executed, tmp, src0, src1);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename S, typename... Ev>
 PTO_INST RecordEvent TMRGSORT(D &dst, S &src, uint32_t blockLen, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src);
     TMRGSORT_IMPL(dst, src, blockLen);
+    detail::UbCommit(dst);
     return {};
 }
 

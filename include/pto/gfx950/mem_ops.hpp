@@ -331,15 +331,17 @@ template <typename TileT>
 constexpr bool is_scale_mat_v = TileT::Loc == TileType::Mat && std::is_same_v<typename TileT::DType, float8_e8m0_t>;
 
 // GM -> Mat tile of block scales ([rows, k blocks] row-major for a left operand, [k blocks, columns] column-major for a
-// right one; k blocks contiguous in memory).  LDS image: [k block / 4][row (column)][4 k blocks], so that the scales
+// right one; k blocks contiguous in memory; plain or boxed tile types alike).  LDS image: [k block / 4][row (column)][4 k blocks], so that the scales
 // of one k step of 32 consecutive rows are 32 consecutive words (fragment reads without bank conflicts).  One 4-byte
 // asynchronous copy instruction per 64 rows and 4 k blocks.
 template <typename TileT>
 struct ScaleMatGeom {
     static constexpr bool left = TileT::isRowMajor;
     static constexpr int Major = left ? TileT::Rows : TileT::Cols, KB = left ? TileT::Cols : TileT::Rows;
-    static_assert(!TileT::isBoxedLayout && KB % 4 == 0 && Major % kWaveSize == 0,
-                  "[PTO][SA] Mat tile of block scales: unboxed, multiples of 64 rows (columns) and of 4 k blocks");
+    // The box layout of the tile type (the reference keeps its scale panels as zZ / nN boxes of 32 bytes in L1:
+    // mxmatmul_performance_kernel.cpp:314-317) names a physical arrangement that this image replaces; only the logical
+    // (row, k block) contract is kept.
+    static_assert(KB % 4 == 0 && Major % kWaveSize == 0, "[PTO][SA] Mat tile of block scales: multiples of 64 rows (columns) and of 4 k blocks");
     static constexpr int nInst = (Major / kWaveSize) * (KB / 4);
     PTO_DEV static uint32_t off(uint32_t major, uint32_t kb) { return ((kb / 4) * Major + major) * 4 + kb % 4; }
 };

@@ -165,6 +165,10 @@ PTO_DEV void pipe_barrier(pipe_t p)
 PTO_DEV int64_t get_block_idx() { return static_cast<int64_t>(blockIdx.x); }
 PTO_DEV int64_t get_block_num() { return static_cast<int64_t>(gridDim.x); }
 PTO_DEV int64_t get_subblockid() { return 0; }
+// Address of the scale buffer that belongs to an L0A / L0B address (include/pto/npu/a5/utils.hpp:82-87).  Scale tiles are
+// register tiles here and TASSIGN on them binds nothing: any value will do.
+template <typename T>
+PTO_DEV uint64_t GetScaleAddr(T *) { return 0; }
 PTO_DEV int64_t get_subblockdim() { return 1; }
 PTO_DEV int64_t get_coreid() { return static_cast<int64_t>(blockIdx.x); }
 PTO_DEV int64_t get_sys_cnt() { return static_cast<int64_t>(wall_clock64()); }

@@ -46,7 +46,7 @@ PTO_DEV T score_of(uint64_t structure)
 {
     return __builtin_bit_cast(T, (SortBits<T>)structure);
 }
-// all elements of a Vec tile -> LDS in the tile's (row, col) order with row stride ld (in elements)
+// the first ld columns of every row of a Vec tile -> LDS in (row, col) order with row stride ld (in elements)
 template <typename TileT>
 PTO_DEV void stage_tile_rows(TileT &t, SortBits<typename TileT::DType> *lds, int ld)
 {
@@ -55,7 +55,8 @@ PTO_DEV void stage_tile_rows(TileT &t, SortBits<typename TileT::DType> *lds, int
         if (e < TileT::Numel) {
             int r, c;
             elem_rc<TileT>(e, r, c);
-            lds[r * ld + c] = __builtin_bit_cast(SortBits<T>, t.S().v[s][i]);
+            if (c < ld)
+                lds[r * ld + c] = __builtin_bit_cast(SortBits<T>, t.S().v[s][i]);
         }
     });
 }
@@ -90,14 +91,18 @@ PTO_DEV void TSORT32_IMPL(DstT &dst, SrcT &src, IdxT &idx)
     static_assert(std::is_same_v<typename DstT::DType, T> && detail::kSortable<T> && !std::is_same_v<T, uint16_t>,
                   "[PTO][SA] TSORT32: float, half, int32 or int16 scores, destination of the same type");
     static_assert(std::is_same_v<typename IdxT::DType, uint32_t>, "[PTO][SA] TSORT32: uint32 indices");
-    static_assert(SrcT::Rows == IdxT::Rows && SrcT::Cols == IdxT::Cols && DstT::Rows == SrcT::Rows && DstT::Cols >= E * SrcT::Cols,
-                  "[PTO][SA] TSORT32: index tile of the source's shape, destination of 8 bytes per source element");
-    constexpr int R = SrcT::Rows, C = SrcT::Cols, N = R * C;
+    static_assert(SrcT::Rows == IdxT::Rows && DstT::Rows == SrcT::Rows, "[PTO][SA] TSORT32: source, index and destination rows");
+    // The valid columns decide what is sorted; the tiles' own widths may differ (the reference's top-k kernel views one
+    // row buffer through a tile type twice as wide as its scores, kernels/manual/a2a3/topk/topk_kernel.cpp:132-145).
+    // C: the most columns that source, index and destination (8 bytes a column) can all hold.
+    constexpr int R = SrcT::Rows;
+    constexpr int C0 = SrcT::Cols < IdxT::Cols ? SrcT::Cols : IdxT::Cols, C = C0 < DstT::Cols / E ? C0 : DstT::Cols / E, N = R * C;
+    static_assert(C >= 1, "[PTO][SA] TSORT32: destination of 8 bytes per source element");
     uint64_t *image = reinterpret_cast<uint64_t *>(detail::stage_buffer<detail::stage_bytes(16 * N)>()); // [R][C] structures
     uint32_t *index = reinterpret_cast<uint32_t *>(image + N);
     B *score = reinterpret_cast<B *>(index + N);
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
-    if (vr != idx.GetValidRow() || vc != idx.GetValidCol())
+    if (vr != idx.GetValidRow() || vc != idx.GetValidCol() || vc > C)
         return; // as the reference does (cpu/TSort32.hpp:113-115); the valid extents are uniform over the workgroup
     detail::stage_tile_rows(src, score, C);
     detail::stage_tile_rows(idx, index, C);

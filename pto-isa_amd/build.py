@@ -88,6 +88,12 @@ PORTED = [
      128 * 1024,
      dict(defines=("__DAV_CUBE__", "__DAV_VEC__", "__DAV_C220_CUBE__", "__DAV_C220_VEC__"), vec_in_memory=True,
           extra_includes=(os.path.join(HERE, "host", "port_cases"),), extra_flags=("-Wno-unknown-attributes",))),
+    # the top-k kernel: every tile a Vec tile at an address of the unified buffer, re-viewed through tiles of other shapes
+    ("libpto_ported_topk.so", "kernels/manual/a2a3/topk/topk_kernel.cpp", [], 0,
+     dict(vec_in_memory=True, extra_flags=("-Wno-unknown-attributes",))),
+    # the MXFP8 matmul kernel (e5m2 operands, e8m0 block scales, bf16 output): one K-128 step per L1 panel instead of four
+    ("libpto_ported_mxfp8.so", "kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp",
+     [("stepKa", "1"), ("stepKb", "1")], 160 * 1024, dict(extra_flags=("-Wno-unknown-attributes",))),
 ]
 
 

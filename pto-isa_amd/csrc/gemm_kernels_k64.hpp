@@ -17,7 +17,7 @@ PTO_DEVICE_CODE_BEGIN
 
 namespace {
 
-template <int BM, int BN, int TUNE = 0>
+template <int BM, int BN>
 AICORE inline __attribute__((always_inline)) void MixTileRowsK64(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1,
                                                                  int m, int n, int k, int row0, int col0, int kLoop)
 {
@@ -43,11 +43,9 @@ AICORE inline __attribute__((always_inline)) void MixTileRowsK64(__gm__ float *o
     constexpr int kMfmaPerHalfK = 2 * AccHalf::Storage::MB * AccHalf::Storage::NB; // both row halves, one 32-wide K half
     constexpr int kReadsPerHalfK = 2 * LeftHalf::Storage::MB + RightTile::Storage::NB;
     static_assert(LeftHalf::Storage::KS == 1 && RightTile::Storage::KS == 1, "one MFMA spans a 32-wide K half");
-    // issue-pattern knobs (tuning hook): eighths of a half's MFMAs that have a read / copy after them, and the order of
-    // copies and reads in the second half
-    constexpr int kF1 = TUNE % 10 == 0 ? 6 : TUNE % 10 == 1 ? 8 : TUNE % 10 == 2 ? 4 : 7;
-    constexpr int kF2 = TUNE / 10 % 10 == 0 ? 7 : TUNE / 10 % 10 == 1 ? 8 : TUNE / 10 % 10 == 2 ? 6 : 5;
-    constexpr int kOrder = TUNE / 100 % 10;
+    // issue pattern (measured): the reads of the first half are spread over the first 6/8 of its MFMAs, the copies and
+    // then the reads of the second half over its first 7/8
+    constexpr int kF1 = 6, kF2 = 7;
 
     __gm__ half *aPanel = const_cast<half *>(src0) + (int64_t)row0 * k;
     __gm__ half *bPanel = const_cast<half *>(src1) + (int64_t)col0 * k;
@@ -140,11 +138,7 @@ AICORE inline __attribute__((always_inline)) void MixTileRowsK64(__gm__ float *o
             constexpr int nMfma = (i + 1) * budget / kSlots - i * budget / kSlots;
             if constexpr (nMfma > 0)
                 __builtin_amdgcn_sched_group_barrier(0x008, nMfma, 0);
-            // order 0: the copies, then the reads; 1: the reads, then the copies; 2: alternating while both last
-            constexpr bool isCopy = kOrder == 0 ? i < kLoadsPerStep
-                                  : kOrder == 1 ? i >= kReadsPerHalfK
-                                  : (i < 2 * (kLoadsPerStep < kReadsPerHalfK ? kLoadsPerStep : kReadsPerHalfK) ? i % 2 == 0 : kLoadsPerStep > kReadsPerHalfK);
-            if constexpr (isCopy)
+            if constexpr (i < kLoadsPerStep) // the copies, then the reads (the other orders spill)
                 __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);
             else
                 __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
@@ -166,14 +160,14 @@ AICORE inline __attribute__((always_inline)) void MixTileRowsK64(__gm__ float *o
 }
 
 // One BM x BN tile of C per workgroup, whole tiles only.
-template <int BM, int BN, int GROUP_M, int TUNE = 0>
+template <int BM, int BN, int GROUP_M>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     void GemmF16F32K64(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k)
 {
     const int tilesM = m / BM, tilesN = n / BN;
     int tm, tn;
     TileOfId<GROUP_M>(RegroupXcd((int)get_block_idx(), tilesM * tilesN), tilesM, tilesN, tm, tn);
-    MixTileRowsK64<BM, BN, TUNE>(out, src0, src1, m, n, k, tm * BM, tn * BN, k / 64);
+    MixTileRowsK64<BM, BN>(out, src0, src1, m, n, k, tm * BM, tn * BN, k / 64);
 }
 
 } // namespace
@@ -181,14 +175,14 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE
 PTO_DEVICE_CODE_END
 
 namespace {
-template <int BM, int BN, int GROUP_M, int TUNE = 0>
+template <int BM, int BN, int GROUP_M>
 int launch_gemm_k64(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k)
 {
     if (m % BM || n % BN || k % 128 || k < 128)
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = 2 * (BM * 64 + 64 * BN) * (int)sizeof(half);
     static_assert(lds <= 160 * 1024, "two K-64 stages must fit the LDS");
-    auto kernel = GemmF16F32K64<BM, BN, GROUP_M, TUNE>;
+    auto kernel = GemmF16F32K64<BM, BN, GROUP_M>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;

@@ -90,3 +90,70 @@ def test_reference_flash_attention_kernel(oracle, S0, S1, causal, tile_s1, prelo
     assert np.abs(got - want).max() <= 2e-3 * np.abs(want).max()
     oo, _, _ = oracle.fa_stream_f16(q, k, v, tile_s1=tile_s1, causal=causal, q_offset=0, round_away=True)
     assert np.abs(got - oo).max() <= 5e-4 * np.abs(oo).max()
+
+
+@pytest.mark.parametrize("ties", [False, True])
+def test_reference_topk_kernel(oracle, ties):
+    """topk_kernel.cpp (launchTopk<float>: 4800 rows of 1024 scores, row stride 1280, top 1000, 48 blocks): TLOAD -> TSORT32 ->
+    TMRGSORT (one source with block lengths 64 and 256, then two lists merged in place) -> TMOV -> TGATHER P0101 / P1010 ->
+    TSTORE, every tile a view of the unified buffer.  Scores and indices bit-exact against the native row sort and the
+    oracle (the order of the reference's generator, scripts/gen_data.py:55-64: np.lexsort((idx, -row))[:topk]); data as the
+    generator draws them, and with many equal scores (where TMRGSORT's order among equals -- list number, then position --
+    and TSORT32's -- index -- agree because the indices increase with the column)."""
+    import torch
+    import gpu_util as G
+    from pto_amd import capi, datagen
+    lib = _ported("libpto_ported_topk.so")
+    fn = lib._Z10launchTopkIfEvPhS0_S0_S0_Pv        # template void launchTopk<float>(uint8_t*, uint8_t*, uint8_t*, uint8_t*, void*)
+    fn.argtypes, fn.restype = [C.c_void_p] * 5, None
+    rows, cols, ld, k = 4800, 1024, 1280, 1000
+    src, idx = datagen.topk_inputs(rows, cols, ld, distinct=37 if ties else 0)
+    ts, ti = G.to_dev(src), G.to_dev(idx)
+    out_s = torch.full((rows, k), float("nan"), dtype=torch.float32, device=G.DEV)
+    out_i = torch.full((rows, k), -1, dtype=torch.int32, device=G.DEV)
+    print("ported top-k launch", ties, flush=True)
+    fn(out_s.data_ptr(), out_i.data_ptr(), ts.data_ptr(), ti.data_ptr(), None)
+    torch.cuda.synchronize()
+    got_s, got_i = out_s.cpu().numpy(), out_i.cpu().numpy().view(np.uint32)
+    nat_s = torch.zeros((rows, k), dtype=torch.float32, device=G.DEV)
+    nat_i = torch.zeros((rows, k), dtype=torch.int32, device=G.DEV)
+    capi.check(capi.load().pto_topk_f32(G.stream(), nat_s.data_ptr(), nat_i.data_ptr(), ts.data_ptr(), ti.data_ptr(), rows, cols, ld, k), "topk")
+    torch.cuda.synchronize()
+    assert np.array_equal(got_s.view(np.uint32), nat_s.cpu().numpy().view(np.uint32))
+    assert np.array_equal(got_i, nat_i.cpu().numpy().view(np.uint32))
+    sel = np.array([0, 1, 2399, 4799])
+    want_s, want_i = oracle.topk_f32(src[sel], idx, cols, k)
+    assert np.array_equal(got_s[sel].view(np.uint32), want_s.view(np.uint32)) and np.array_equal(got_i[sel], want_i)
+
+
+def test_reference_mxfp8_matmul_kernel(oracle):
+    """mxmatmul_performance_kernel.cpp of a5/matmul_mxfp8_performance (LaunchMxMatmul: m = n = k = 6144, e5m2 operands, e8m0
+    scales per 32 k, bf16 output, 32 blocks of 1536 x 768) with stepKa = stepKb = 1: TLOAD of operand and scale panels ->
+    TEXTRACT -> TMATMUL_MX -> TSTORE.  Every element against the native MX GEMM (both round an fp32 sum of different
+    order to bf16: one bf16 step of the largest |C| at most, and nearly all equal), 8 rows against the oracle."""
+    import torch
+    import gpu_util as G
+    from pto_amd import capi, datagen
+    lib = _ported("libpto_ported_mxfp8.so")
+    fn = lib._Z14LaunchMxMatmulPhS_S_S_S_Pv         # void LaunchMxMatmul(uint8_t*, uint8_t*, uint8_t*, uint8_t*, uint8_t*, void*)
+    fn.argtypes, fn.restype = [C.c_void_p] * 6, None
+    m = n = k = 6144
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 1)
+    ta, tb, tsa, tsb = (torch.from_numpy(x).to(G.DEV) for x in (a, b, sa, sb))
+    tc = torch.full((m, n), -1, dtype=torch.int16, device=G.DEV)
+    print("ported mxfp8 launch", flush=True)
+    fn(tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), None)
+    torch.cuda.synchronize()
+    got = tc.view(torch.bfloat16).float().cpu().numpy()
+    native = torch.zeros((m, n), dtype=torch.int16, device=G.DEV)
+    capi.check(capi.load().pto_gemm_mxfp8(G.stream(), native.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                          m, n, k, 1, 0), "pto_gemm_mxfp8")
+    torch.cuda.synchronize()
+    nat = native.view(torch.bfloat16).float().cpu().numpy()
+    assert np.isfinite(got).all()
+    scale = np.abs(nat).max()
+    assert np.abs(got - nat).max() <= scale * 2.0 ** -7
+    assert np.mean(got == nat) > 0.99
+    rows = np.array([0, 127, 128, 1535, 1536, 3000, 4607, 6143])
+    want = oracle.mx_gemm(a[rows], b, sa[rows], sb, 1)
+    assert np.abs(got[rows] - want).max() <= 2.0 ** -7 * np.abs(want).max()

@@ -57,6 +57,26 @@ def test_reference_flash_attention_kernel_compiles(tmp_path):
     assert rc == 0, err
 
 
+@needs_reference
+def test_reference_topk_kernel_compiles(tmp_path):
+    """topk_kernel.cpp as it is (no constant rewritten): TSORT32 / TMRGSORT / TGATHER on Vec tiles that are views of the
+    unified buffer, launchTopk<float>."""
+    lib, rel_src, sets, lds, opts = [p for p in B.PORTED if p[0] == "libpto_ported_topk.so"][0]
+    assert sets == []
+    rc, err = B.port_and_compile(rel_src, sets, lds, str(tmp_path / "topk.o"), **opts)
+    assert rc == 0, err
+
+
+@needs_reference
+def test_reference_mxfp8_matmul_kernel_compiles(tmp_path):
+    """mxmatmul_performance_kernel.cpp of a5/matmul_mxfp8_performance with stepKa = stepKb = 1 (its own four K-steps per L1
+    panel need 384 KiB): scale panels as boxed Mat tiles, TileLeftScale / TileRightScale, GetScaleAddr, TMATMUL_MX, tiles by
+    value."""
+    lib, rel_src, sets, lds, opts = [p for p in B.PORTED if p[0] == "libpto_ported_mxfp8.so"][0]
+    rc, err = B.port_and_compile(rel_src, sets, lds, str(tmp_path / "mx.o"), **opts)
+    assert rc == 0, err
+
+
 def test_port_script_rewrites():
     """The mechanical edits on a synthetic source: launch statement, function-local static, kernel prologue, brackets."""
     spec = importlib.util.spec_from_file_location("port_ascend_source", os.path.join(PKG, "port_ascend_source.py"))
