@@ -41,17 +41,29 @@ struct Dims5 {
 template <int64_t N1 = DYNAMIC, int64_t N2 = DYNAMIC, int64_t N3 = DYNAMIC, int64_t N4 = DYNAMIC, int64_t N5 = DYNAMIC>
 struct Shape : detail::Dims5<N1, N2, N3, N4, N5> {
     using Base = detail::Dims5<N1, N2, N3, N4, N5>;
-    using Base::Base;
     static constexpr int64_t staticShape[5] = {N1, N2, N3, N4, N5};
     PTO_HD constexpr Shape() : Base() {}
+    // declared here rather than inherited: `pto::Shape(1, 1, 1, rows, cols)` without template arguments then names the
+    // all-dynamic type, as with the reference's constructors (pto_tile.hpp:26-131)
+    PTO_HD constexpr Shape(int64_t a, int64_t b, int64_t c, int64_t d, int64_t e) : Base(a, b, c, d, e) {}
+    PTO_HD constexpr Shape(int64_t a, int64_t b, int64_t c, int64_t d) : Base(a, b, c, d) {}
+    PTO_HD constexpr Shape(int64_t a, int64_t b, int64_t c) : Base(a, b, c) {}
+    PTO_HD constexpr Shape(int64_t a, int64_t b) : Base(a, b) {}
+    PTO_HD constexpr explicit Shape(int64_t a) : Base(a) {}
 };
 
 template <int64_t N1 = DYNAMIC, int64_t N2 = DYNAMIC, int64_t N3 = DYNAMIC, int64_t N4 = DYNAMIC, int64_t N5 = DYNAMIC>
 struct Stride : detail::Dims5<N1, N2, N3, N4, N5> {
     using Base = detail::Dims5<N1, N2, N3, N4, N5>;
-    using Base::Base;
     static constexpr int64_t staticStride[5] = {N1, N2, N3, N4, N5};
     PTO_HD constexpr Stride() : Base() {}
+    // declared here rather than inherited: `pto::Stride(1, 1, 1, rows, cols)` without template arguments then names the
+    // all-dynamic type, as with the reference's constructors (pto_tile.hpp:26-131)
+    PTO_HD constexpr Stride(int64_t a, int64_t b, int64_t c, int64_t d, int64_t e) : Base(a, b, c, d, e) {}
+    PTO_HD constexpr Stride(int64_t a, int64_t b, int64_t c, int64_t d) : Base(a, b, c, d) {}
+    PTO_HD constexpr Stride(int64_t a, int64_t b, int64_t c) : Base(a, b, c) {}
+    PTO_HD constexpr Stride(int64_t a, int64_t b) : Base(a, b) {}
+    PTO_HD constexpr explicit Stride(int64_t a) : Base(a) {}
 };
 
 // [1,1,1,rows,cols] extent of one 2-D tile in memory (pto_tile.hpp:452-556, ND and DN forms).

@@ -105,17 +105,19 @@ PTO_FRONT(TMINS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename
 PTO_FRONT(TEXP, typename T, T &dst PTO_C T &src, (dst, src))
 PTO_FRONT(TEXPANDS, typename T, T &dst PTO_C typename T::DType k, (dst, k))
 PTO_FRONT(TROWMAX, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
+PTO_FRONT(TROWPROD, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
 PTO_FRONT(TROWSUM, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
-PTO_FRONT(TROWEXPANDSUB, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
-PTO_FRONT(TROWEXPANDMUL, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
-PTO_FRONT(TROWEXPANDDIV, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
-PTO_FRONT(TROWEXPANDADD, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
-PTO_FRONT(TROWEXPANDMAX, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
-PTO_FRONT(TROWEXPANDMIN, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
-PTO_FRONT(TROWEXPANDEXPDIF, typename D PTO_C typename R, D &dst PTO_C D &src0 PTO_C R &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDSUB, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDMUL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDDIV, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDMAX, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDMIN, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
+PTO_FRONT(TROWEXPANDEXPDIF, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &src0 PTO_C B &src1, (dst, src0, src1))
 PTO_FRONT(TROWEXPAND, typename D PTO_C typename R, D &dst PTO_C R &src, (dst, src))
 PTO_FRONT(TROWMIN, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src PTO_C T &tmp, (dst, src, tmp))
 PTO_FRONT(TCOLMAX, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TCOLPROD, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TCOLMIN, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TCOLSUM, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TCOLEXPAND, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
@@ -133,7 +135,15 @@ PTO_FRONT(TSQRT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TRSQRT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TLOG, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TRECIP, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
-PTO_FRONT(TPRELU, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+template <typename D, typename A, typename B, typename... Ev>
+PTO_INST std::enable_if_t<(... && is_wait_event<Ev>::value), RecordEvent> TPRELU(D &dst, A &a, B &b, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, a, b);
+    TPRELU_IMPL(dst, a, b);
+    detail::UbCommit(dst);
+    return {};
+}
 // bitwise / shift / remainder / three-operand forms (pto_instr.hpp:72-86, 246-333, 1137, 1215-1300, 1418 of the reference;
 // the forms that take a scratch tile accept and ignore it)
 PTO_FRONT(TAND, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
@@ -141,6 +151,7 @@ PTO_FRONT(TOR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a P
 PTO_FRONT(TSHL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TSHR, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TREM, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TFMOD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TNOT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TGATHERB, typename D PTO_C typename S PTO_C typename O, D &dst PTO_C S &src PTO_C O &offset, (dst, src, offset))
 PTO_FRONT(TSCATTER, typename D PTO_C typename I, D &dst PTO_C D &src PTO_C I &indexes, (dst, src, indexes))
@@ -148,11 +159,13 @@ PTO_FRONT(MSCATTER, typename G PTO_C typename S PTO_C typename I, G &dst PTO_C S
 PTO_FRONT(TPARTADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TPARTMAX, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TPARTMIN, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
+PTO_FRONT(TPARTMUL, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TANDS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TORS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TSHLS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TSHRS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TREMS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
+PTO_FRONT(TFMODS, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
 PTO_FRONT(TADDC, typename T, T &dst PTO_C T &a PTO_C T &b PTO_C T &c, (dst, a, b, c))
 PTO_FRONT(TSUBC, typename T, T &dst PTO_C T &a PTO_C T &b PTO_C T &c, (dst, a, b, c))
 PTO_FRONT(TADDSC, typename T, T &dst PTO_C T &a PTO_C typename T::DType k PTO_C T &b, (dst, a, k, b))
@@ -161,14 +174,18 @@ template <typename D, typename A, typename B, typename Tmp, typename... Ev>
 PTO_INST std::enable_if_t<is_tile_data_v<Tmp>, RecordEvent> TXOR(D &dst, A &a, B &b, Tmp &, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, a, b);
     TXOR_IMPL(dst, a, b);
+    detail::UbCommit(dst);
     return {};
 }
 template <typename D, typename S, typename Tmp, typename... Ev>
 PTO_INST std::enable_if_t<is_tile_data_v<Tmp>, RecordEvent> TXORS(D &dst, S &src, typename S::DType k, Tmp &, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(dst, src);
     TXORS_IMPL(dst, src, k);
+    detail::UbCommit(dst);
     return {};
 }
 PTO_FRONT(TLRELU, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C typename D::DType k, (dst, src, k))
@@ -319,6 +336,48 @@ PTO_INST RecordEvent TMRGSORT(D &dst, S &src, uint32_t blockLen, Ev &... ev)
     TSYNC(ev...);
     detail::UbFetch(dst, src);
     TMRGSORT_IMPL(dst, src, blockLen);
+    detail::UbCommit(dst);
+    return {};
+}
+
+// TPRELU with a scratch tile (pto_instr.hpp:306-313 of the reference): accepted and ignored
+template <typename D, typename A, typename B, typename Tmp, typename... Ev>
+PTO_INST std::enable_if_t<is_tile_data_v<Tmp>, RecordEvent> TPRELU(D &dst, A &a, B &b, Tmp &, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, a, b);
+    TPRELU_IMPL(dst, a, b);
+    detail::UbCommit(dst);
+    return {};
+}
+// TCMP with a uint8 destination: packed bits, the NPU's form (the CPU simulation's writes 0 / 1 in the sources' type)
+template <typename D, typename S, typename... Ev>
+PTO_INST std::enable_if_t<!std::is_same_v<D, S> && sizeof(typename D::DType) == 1, RecordEvent> TCMP(D &dst, S &src0, S &src1, CmpMode mode,
+                                                                                                     Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src0, src1);
+    TCMP_PACKED_IMPL(dst, src0, src1, mode);
+    detail::UbCommit(dst);
+    return {};
+}
+// TDIVS(dst, scalar, src) = scalar / src (pto_instr.hpp:1176-1182 of the reference)
+template <typename D, typename S, typename... Ev>
+PTO_INST std::enable_if_t<is_tile_data_v<S>, RecordEvent> TDIVS(D &dst, typename D::DType k, S &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src);
+    TDIVS_SCALAR_FIRST_IMPL(dst, src, k);
+    detail::UbCommit(dst);
+    return {};
+}
+// TCOLSUM with a scratch tile and the choice of a pairwise order (pto_instr.hpp:966-972): both accepted and ignored
+template <typename D, typename S, typename Tmp, typename... Ev>
+PTO_INST RecordEvent TCOLSUM(D &dst, S &src, Tmp &tmp, bool isBinary, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src);
+    TCOLSUM_IMPL(dst, src, tmp, isBinary);
     detail::UbCommit(dst);
     return {};
 }

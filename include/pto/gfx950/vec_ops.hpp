@@ -155,6 +155,54 @@ PTO_DEV void for_each_owned(F &&fn)
 template <typename A, typename B>
 constexpr bool same_dist = A::Numel == B::Numel && A::Loc == TileType::Vec && B::Loc == TileType::Vec;
 
+// An elementwise instruction pairs the elements of its operands by (row, column) over the valid region.  Operands with
+// the destination's number of elements pair up lane by lane as they are.  A Vec operand of another static shape (the
+// reference's per-instruction tests give source and destination tiles different widths, e.g. 32 x 128 and 32 x 112 with
+// a 32 x 111 valid region: tests/npu/a2a3/src/st/testcase/tadds) is first brought into the destination's distribution
+// through LDS: Conformed<DstT, SrcT>(src).S() then holds src's element (r, c) where dst keeps its (r, c).
+template <int Bytes>
+PTO_DEV char *conform_buffer()
+{
+    __shared__ __attribute__((aligned(16))) char buf[Bytes];
+    return buf;
+}
+template <typename DstT, typename SrcT, bool kAsIs = same_dist<DstT, SrcT>>
+struct Conformed {
+    SrcT &t;
+    PTO_DEV explicit Conformed(SrcT &src) : t(src) {}
+    PTO_DEV auto &S() { return t.S(); }
+};
+template <typename DstT, typename SrcT>
+struct Conformed<DstT, SrcT, false> {
+    using T = typename SrcT::DType;
+    using Storage = ::pto::detail::TileStorage<TileType::Vec, T, DstT::Rows, DstT::Cols>;
+    Storage st;
+    PTO_DEV explicit Conformed(SrcT &src)
+    {
+        static_assert(DstT::Loc == TileType::Vec && SrcT::Loc == TileType::Vec, "[PTO][SA] elementwise instruction: Vec tiles");
+        constexpr int kBytes = (int)sizeof(T) * DstT::Numel;
+        T *lds = reinterpret_cast<T *>(conform_buffer<(kBytes + 1023) / 1024 * 1024>());
+        for_each_owned<SrcT>([&](int s, int i, int e) {
+            if (e < SrcT::Numel) {
+                int r, c;
+                elem_rc<SrcT>(e, r, c);
+                if (r < DstT::Rows && c < DstT::Cols)
+                    lds[r * DstT::Cols + c] = src.S().v[s][i];
+            }
+        });
+        hw::lds_barrier();
+        for_each_owned<DstT>([&](int s, int i, int e) {
+            if (e < DstT::Numel) {
+                int r, c;
+                elem_rc<DstT>(e, r, c);
+                st.v[s][i] = (r < SrcT::Rows && c < SrcT::Cols) ? lds[r * DstT::Cols + c] : T{};
+            }
+        });
+        hw::lds_barrier();
+    }
+    PTO_DEV Storage &S() { return st; }
+};
+
 // one value per row (a [R,1] / [1,R] / first-column tile) -> LDS array of R floats, visible to all lanes
 template <typename RowT, int R>
 PTO_DEV void stage_row_values(RowT &t, typename RowT::DType *lds)
@@ -199,13 +247,13 @@ PTO_DEV void TCVT_IMPL(DstT &dst, SrcT &src, RoundMode mode, SaturationMode)
     template <typename DstT, typename S0T, typename S1T>                                                \
     PTO_DEV void NAME##_IMPL(DstT &dst, S0T &src0, S1T &src1)                                           \
     {                                                                                                   \
-        static_assert(detail::same_dist<DstT, S0T> && detail::same_dist<DstT, S1T>,                     \
-                      "[PTO][SA] " #NAME ": Vec tiles with the same number of elements");              \
         using T = typename DstT::DType;                                                                 \
         using S = typename DstT::Storage;                                                               \
+        detail::Conformed<DstT, S0T> c0(src0);                                                          \
+        detail::Conformed<DstT, S1T> c1(src1);                                                          \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src0.S().v[s][i], b = src1.S().v[s][i];                                           \
+            const T a = c0.S().v[s][i], b = c1.S().v[s][i];                                               \
             dst.S().v[s][i] = (EXPR);                                                                    \
         }                                                                                               \
     }
@@ -221,12 +269,12 @@ PTO_DEFINE_BINARY(TMIN, (b < a ? b : a))
     template <typename DstT, typename SrcT>                                                             \
     PTO_DEV void NAME##_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)                              \
     {                                                                                                   \
-        static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] " #NAME ": Vec tiles of equal size"); \
         using T = typename DstT::DType;                                                                 \
         using S = typename DstT::Storage;                                                               \
+        detail::Conformed<DstT, SrcT> c0(src);                                                          \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src.S().v[s][i];                                                                 \
+            const T a = c0.S().v[s][i];                                                                  \
             dst.S().v[s][i] = (EXPR);                                                                    \
         }                                                                                               \
     }
@@ -234,6 +282,7 @@ PTO_DEFINE_SCALAR(TMULS, a *k)
 PTO_DEFINE_SCALAR(TADDS, a + k)
 PTO_DEFINE_SCALAR(TSUBS, a - k)
 PTO_DEFINE_SCALAR(TDIVS, a / k)
+PTO_DEFINE_SCALAR(TDIVS_SCALAR_FIRST, k / a)
 PTO_DEFINE_SCALAR(TMAXS, (a < k ? k : a))
 PTO_DEFINE_SCALAR(TMINS, (k < a ? k : a))
 #undef PTO_DEFINE_SCALAR
@@ -297,7 +346,7 @@ PTO_DEV void TTRI_IMPL(TileT &dst, int diagonal)
 
 // --------------------------------------------------------- row reductions
 namespace detail {
-// KIND: 0 sum, 1 maximum, 2 minimum
+// KIND: 0 sum, 1 maximum, 2 minimum, 3 product
 template <int KIND, typename DstT, typename SrcT>
 PTO_DEV void row_reduce(DstT &dst, SrcT &src)
 {
@@ -315,12 +364,12 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
         const int q = s * kBlockThreads + hw::tid();
         if (q < S::Chunks) {
             const int c0 = (q % CPR) * kVecChunk;
-            A acc = KIND == 1 ? -__builtin_huge_valf() : KIND == 2 ? __builtin_huge_valf() : 0.0f;
+            A acc = KIND == 1 ? -__builtin_huge_valf() : KIND == 2 ? __builtin_huge_valf() : KIND == 3 ? 1.0f : 0.0f;
 #pragma unroll
             for (int i = 0; i < kVecChunk; ++i)
                 if (c0 + i < vc) {
                     const A v = (A)src.S().v[s][i];
-                    acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : acc + v;
+                    acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : KIND == 3 ? acc * v : acc + v;
                 }
             part[q] = acc;
         }
@@ -334,7 +383,7 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
                 A acc = part[r * CPR];
                 for (int j = 1; j < CPR; ++j) {
                     const A v = part[r * CPR + j];
-                    acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : acc + v;
+                    acc = KIND == 1 ? (acc < v ? v : acc) : KIND == 2 ? (v < acc ? v : acc) : KIND == 3 ? acc * v : acc + v;
                 }
                 dst.S().v[s][i] = (typename DstT::DType)acc;
             }
@@ -343,21 +392,41 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
     hw::lds_barrier();
 }
 
-enum class RowOp { Sub, Mul, Div, Add, Max, Min };
+enum class RowOp { Sub, Mul, Div, Add, Max, Min, ExpDif };
 
-template <RowOp op, typename DstT, typename RowT>
-PTO_DEV void row_expand(DstT &dst, DstT &src0, RowT &src1)
+// The per-row operand of a row-broadcast instruction: a [R,1] column (or [1,R] row) tile with one value per row, or, on
+// the NPU, a row-major [R, 32 / sizeof(T)] tile whose row r is applied to every 32-byte block of row r of the other
+// operand: value (r, c % width) (npu/a2a3/TRowExpandSub.hpp:59-77 and its test generator, trowexpandadd/gen_data.py:24-34).
+template <typename RowT, typename DstT>
+inline constexpr int kRowOperandWidth =
+    (RowT::isRowMajor && RowT::Rows > 1 && RowT::Cols * (int)sizeof(typename RowT::DType) == 32 && RowT::Cols != DstT::Cols) ? RowT::Cols : 1;
+template <typename T, typename DstT>
+inline constexpr bool kIsRowOperand = !(T::Rows == DstT::Rows && T::Cols == DstT::Cols);
+
+// dst = mat (op) row, or row (op) mat when kRowFirst (the instruction computes src0 (op) src1 in argument order; either
+// of them may be the per-row operand: TRowExpandSub.hpp:63-77)
+template <RowOp op, bool kRowFirst, typename DstT, typename MatT, typename RowT>
+PTO_DEV void row_expand(DstT &dst, MatT &mat, RowT &row)
 {
-    static_assert(DstT::isRowMajor, "[PTO][SA] row broadcast: row-major Vec tile");
+    static_assert(DstT::isRowMajor && same_dist<DstT, MatT> && MatT::Cols == DstT::Cols, "[PTO][SA] row broadcast: row-major Vec tiles of one shape");
     using T = typename DstT::DType;
-    __shared__ typename RowT::DType rowv[DstT::Rows];
-    stage_row_values<RowT, DstT::Rows>(src1, rowv);
+    constexpr int K = kRowOperandWidth<RowT, DstT>;
+    __shared__ typename RowT::DType rowv[DstT::Rows * K];
+    if constexpr (K == 1) {
+        stage_row_values<RowT, DstT::Rows>(row, rowv);
+    } else {
+        for_each_owned<RowT>([&](int s, int i, int e) {
+            if (e < RowT::Numel && e < DstT::Rows * K)
+                rowv[e] = row.S().v[s][i];
+        });
+    }
     hw::lds_barrier();
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     for_each_owned<DstT>([&](int s, int i, int e) {
         const int r = e / DstT::Cols, c = e % DstT::Cols;
         if (e < DstT::Numel && r < vr && c < vc) {
-            const T a = src0.S().v[s][i], b = (T)rowv[r];
+            const T m = mat.S().v[s][i], v = (T)rowv[r * K + (K == 1 ? 0 : c % K)];
+            const T a = kRowFirst ? v : m, b = kRowFirst ? m : v;
             T o;
             if constexpr (op == RowOp::Sub)
                 o = a - b;
@@ -369,12 +438,22 @@ PTO_DEV void row_expand(DstT &dst, DstT &src0, RowT &src1)
                 o = a + b;
             else if constexpr (op == RowOp::Max)
                 o = a < b ? b : a;
-            else
+            else if constexpr (op == RowOp::Min)
                 o = b < a ? b : a;
+            else
+                o = (T)::exp((double)(T)(a - b)); // exp evaluated in double (cpu/TRowExpandOp.hpp:93-96, ElementOp.h:265-270)
             dst.S().v[s][i] = o;
         }
     });
     hw::lds_barrier();
+}
+template <RowOp op, typename DstT, typename A, typename B>
+PTO_DEV void row_expand_any(DstT &dst, A &src0, B &src1)
+{
+    if constexpr (kIsRowOperand<B, DstT>)
+        row_expand<op, false>(dst, src0, src1);
+    else
+        row_expand<op, true>(dst, src1, src0);
 }
 } // namespace detail
 
@@ -389,10 +468,10 @@ PTO_DEV void TROWSUM_IMPL(DstT &dst, SrcT &src, TmpT &)
     detail::row_reduce<0>(dst, src);
 }
 #define PTO_DEFINE_ROWEXPAND(NAME, OP)                                \
-    template <typename DstT, typename RowT>                           \
-    PTO_DEV void NAME##_IMPL(DstT &dst, DstT &src0, RowT &src1)       \
+    template <typename DstT, typename A, typename B>                  \
+    PTO_DEV void NAME##_IMPL(DstT &dst, A &src0, B &src1)             \
     {                                                                 \
-        detail::row_expand<detail::RowOp::OP>(dst, src0, src1);       \
+        detail::row_expand_any<detail::RowOp::OP>(dst, src0, src1);   \
     }
 PTO_DEFINE_ROWEXPAND(TROWEXPANDSUB, Sub)
 PTO_DEFINE_ROWEXPAND(TROWEXPANDMUL, Mul)
@@ -400,6 +479,7 @@ PTO_DEFINE_ROWEXPAND(TROWEXPANDDIV, Div)
 PTO_DEFINE_ROWEXPAND(TROWEXPANDADD, Add)
 PTO_DEFINE_ROWEXPAND(TROWEXPANDMAX, Max)
 PTO_DEFINE_ROWEXPAND(TROWEXPANDMIN, Min)
+PTO_DEFINE_ROWEXPAND(TROWEXPANDEXPDIF, ExpDif)
 #undef PTO_DEFINE_ROWEXPAND
 
 // ------------------------------------------------------------------ TGATHER

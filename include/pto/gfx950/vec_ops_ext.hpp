@@ -14,12 +14,12 @@ namespace pto {
     template <typename DstT, typename SrcT>                                                             \
     PTO_DEV void NAME##_IMPL(DstT &dst, SrcT &src)                                                      \
     {                                                                                                   \
-        static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] " #NAME ": Vec tiles of equal size"); \
         using T = typename DstT::DType;                                                                 \
         using S = typename DstT::Storage;                                                               \
+        detail::Conformed<DstT, SrcT> c0(src);                                                          \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src.S().v[s][i];                                                                 \
+            const T a = c0.S().v[s][i];                                                                  \
             dst.S().v[s][i] = (EXPR);                                                                    \
         }                                                                                               \
     }
@@ -36,14 +36,15 @@ PTO_DEFINE_UNARY(TRECIP, (T)((T)1 / a))                                    // El
 template <typename DstT, typename S0T, typename S1T>
 PTO_DEV void TPRELU_IMPL(DstT &dst, S0T &src0, S1T &src1)
 {
-    static_assert(detail::same_dist<DstT, S0T> && detail::same_dist<DstT, S1T>, "[PTO][SA] TPRELU: Vec tiles of equal size");
     using T = typename DstT::DType;
     using S = typename DstT::Storage;
+    detail::Conformed<DstT, S0T> c0(src0);
+    detail::Conformed<DstT, S1T> c1(src1);
 #pragma unroll
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i) {
-            const T a = src0.S().v[s][i], b = src1.S().v[s][i];
+            const T a = c0.S().v[s][i], b = c1.S().v[s][i];
             dst.S().v[s][i] = a > (T)0 ? a : (T)(a * b);
         }
 }
@@ -51,14 +52,14 @@ PTO_DEV void TPRELU_IMPL(DstT &dst, S0T &src0, S1T &src1)
 template <typename DstT, typename SrcT>
 PTO_DEV void TLRELU_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)
 {
-    static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] TLRELU: Vec tiles of equal size");
     using T = typename DstT::DType;
     using S = typename DstT::Storage;
+    detail::Conformed<DstT, SrcT> c0(src);
 #pragma unroll
     for (int s = 0; s < S::Slots; ++s)
 #pragma unroll
         for (int i = 0; i < detail::kVecChunk; ++i) {
-            const T a = src.S().v[s][i];
+            const T a = c0.S().v[s][i];
             dst.S().v[s][i] = a > (T)0 ? a : (T)(a * k);
         }
 }
@@ -144,6 +145,40 @@ PTO_DEV void TCMPS_IMPL(DstT &dst, SrcT &src0, T scalar, CmpMode mode)
     hw::lds_barrier();
 }
 
+// The NPU's tile-tile compare writes packed bits like TCMPS (npu/a2a3/TCmp.hpp; its test compares 8 elements a byte):
+// bit (c % 8) of byte c / 8 of row r of the uint8 destination = (src0[r,c] <mode> src1[r,c]).
+template <typename DstT, typename SrcT>
+PTO_DEV void TCMP_PACKED_IMPL(DstT &dst, SrcT &src0, SrcT &src1, CmpMode mode)
+{
+    static_assert(sizeof(typename DstT::DType) == 1 && SrcT::isRowMajor && DstT::isRowMajor && SrcT::Cols % 8 == 0 &&
+                      DstT::Rows == SrcT::Rows && DstT::Cols >= SrcT::Cols / 8,
+                  "[PTO][SA] TCMP: uint8 destination with the source's rows, source columns a multiple of 8");
+    using S = typename SrcT::Storage;
+    constexpr int kBytes = SrcT::Rows * (SrcT::Cols / 8);
+    __shared__ uint8_t packed[kBytes];
+    const int vr = src0.GetValidRow(), vc = src0.GetValidCol();
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s) {
+        const int q = s * kBlockThreads + hw::tid();
+        if (q < S::Chunks) {
+            const int r = (q * 8) / SrcT::Cols, c0 = (q * 8) % SrcT::Cols;
+            uint32_t byte = 0;
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (r < vr && c0 + i < vc && detail::cmp_exact<typename SrcT::DType>(src0.S().v[s][i], src1.S().v[s][i], mode))
+                    byte |= 1u << i;
+            packed[q] = (uint8_t)byte;
+        }
+    }
+    hw::lds_barrier();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && c < SrcT::Cols / 8)
+            dst.S().v[s][i] = packed[r * (SrcT::Cols / 8) + c];
+    });
+    hw::lds_barrier();
+}
+
 // dst[i,j] = bit ? src0[i,j] : src1[i,j]; the bits are consumed in running order over the valid
 // region, byte after byte along the mask tile's valid columns, then its next row (TSel.hpp:22-49).
 template <typename TileT, typename MaskT>
@@ -203,7 +238,7 @@ PTO_DEV void TFILLPAD_IMPL(DstT &dst, SrcT &src)
 
 // ------------------------------------------------------- column reductions
 namespace detail {
-enum class Red { Max, Min, Sum };
+enum class Red { Max, Min, Sum, Prod };
 // One value per column into a [1, Cols] tile.  A lane owns the same 8 columns in every slot (the
 // number of chunks per row divides the workgroup size); its rows are g, g + G, g + 2G, ... for its
 // group g of G = threads / chunks-per-row.  Per-lane partials over its rows, then the G partials of a
@@ -237,6 +272,8 @@ PTO_DEV void col_reduce(DstT &dst, SrcT &src)
                     acc[i] = acc[i] < v ? v : acc[i];
                 else if (red == Red::Min)
                     acc[i] = v < acc[i] ? v : acc[i];
+                else if (red == Red::Prod)
+                    acc[i] *= v;
                 else
                     acc[i] += v;
             }
@@ -259,7 +296,7 @@ PTO_DEV void col_reduce(DstT &dst, SrcT &src)
             for (int k = 1; k < G; ++k)
                 if (has[k]) {
                     const A v = part[k][e];
-                    a = red == Red::Max ? (a < v ? v : a) : red == Red::Min ? (v < a ? v : a) : a + v;
+                    a = red == Red::Max ? (a < v ? v : a) : red == Red::Min ? (v < a ? v : a) : red == Red::Prod ? a * v : a + v;
                 }
             dst.S().v[s][i] = (typename DstT::DType)a;
         }
@@ -317,6 +354,8 @@ template <typename DstT, typename SrcT>
 PTO_DEV void TCOLSUM_IMPL(DstT &dst, SrcT &src) { detail::col_reduce<detail::Red::Sum>(dst, src); } // TColSum.hpp:22-31
 template <typename DstT, typename SrcT, typename TmpT>
 PTO_DEV void TCOLSUM_IMPL(DstT &dst, SrcT &src, TmpT &, bool) { detail::col_reduce<detail::Red::Sum>(dst, src); }
+template <typename DstT, typename SrcT>
+PTO_DEV void TCOLPROD_IMPL(DstT &dst, SrcT &src) { detail::col_reduce<detail::Red::Prod>(dst, src); } // npu/a2a3/TColProd.hpp
 
 template <typename DstT, typename ColT>
 PTO_DEV void TCOLEXPAND_IMPL(DstT &dst, ColT &src) { detail::col_expand<detail::ColOp::Copy>(dst, dst, src); }
@@ -342,9 +381,14 @@ PTO_DEV void TROWMIN_IMPL(DstT &dst, SrcT &src, TmpT &)
 {
     detail::row_reduce<2>(dst, src);
 }
+// product of the valid columns of every row (npu/a2a3/TRowProd.hpp; the reference's generator: prod(axis=1))
+template <typename DstT, typename SrcT, typename TmpT>
+PTO_DEV void TROWPROD_IMPL(DstT &dst, SrcT &src, TmpT &)
+{
+    detail::row_reduce<3>(dst, src);
+}
 
-// dst[i,j] = src[i]  (TRowExpand.hpp) and dst[i,j] = exp(src0[i,j] - src1[i]) with the exponential
-// evaluated in double (TRowExpandOp.hpp:93-96, ElementOp.h:265-270)
+// dst[i,j] = src[i]  (TRowExpand.hpp)
 template <typename DstT, typename RowT>
 PTO_DEV void TROWEXPAND_IMPL(DstT &dst, RowT &src)
 {
@@ -360,25 +404,6 @@ PTO_DEV void TROWEXPAND_IMPL(DstT &dst, RowT &src)
     });
     hw::lds_barrier();
 }
-template <typename DstT, typename RowT>
-PTO_DEV void TROWEXPANDEXPDIF_IMPL(DstT &dst, DstT &src0, RowT &src1)
-{
-    static_assert(DstT::isRowMajor, "[PTO][SA] TROWEXPANDEXPDIF: row-major tiles");
-    using T = typename DstT::DType;
-    __shared__ typename RowT::DType rowv[DstT::Rows];
-    detail::stage_row_values<RowT, DstT::Rows>(src1, rowv);
-    hw::lds_barrier();
-    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
-    detail::for_each_owned<DstT>([&](int s, int i, int e) {
-        const int r = e / DstT::Cols, c = e % DstT::Cols;
-        if (e < DstT::Numel && r < vr && c < vc) {
-            const T d = src0.S().v[s][i] - (T)rowv[r];
-            dst.S().v[s][i] = (T)::exp((double)d);
-        }
-    });
-    hw::lds_barrier();
-}
-
 // LDS staging arrays of the moves that redistribute a tile over the workgroup (Acc -> Vec, Vec / Acc -> Left / Right,
 // TTRANS): one array per power-of-two size class, shared by every move of that class in a kernel.
 namespace detail {
@@ -560,14 +585,14 @@ PTO_DEV T elem_rem(T a, T b)
     template <typename DstT, typename S0T, typename S1T>                                                \
     PTO_DEV void NAME##_IMPL(DstT &dst, S0T &src0, S1T &src1)                                           \
     {                                                                                                   \
-        static_assert(detail::same_dist<DstT, S0T> && detail::same_dist<DstT, S1T>,                     \
-                      "[PTO][SA] " #NAME ": Vec tiles with the same number of elements");              \
         using T = typename DstT::DType;                                                                 \
         static_assert(!(INT_ONLY) || std::is_integral_v<T>, "[PTO][SA] " #NAME ": integer tiles");      \
         using S = typename DstT::Storage;                                                               \
+        detail::Conformed<DstT, S0T> c0(src0);                                                          \
+        detail::Conformed<DstT, S1T> c1(src1);                                                          \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src0.S().v[s][i], b = src1.S().v[s][i];                                           \
+            const T a = c0.S().v[s][i], b = c1.S().v[s][i];                                               \
             dst.S().v[s][i] = (T)(EXPR);                                                                 \
         }                                                                                               \
     }
@@ -577,19 +602,20 @@ PTO_DEFINE_BINARY_EXT(TXOR, true, a ^ b)
 PTO_DEFINE_BINARY_EXT(TSHL, true, a << b)
 PTO_DEFINE_BINARY_EXT(TSHR, true, a >> b)
 PTO_DEFINE_BINARY_EXT(TREM, false, detail::elem_rem<T>(a, b))
+PTO_DEFINE_BINARY_EXT(TFMOD, false, detail::elem_rem<T>(a, b)) // C fmod / integer %: the sign of the dividend (tfmod/gen_data.py:32)
 #undef PTO_DEFINE_BINARY_EXT
 
 #define PTO_DEFINE_SCALAR_EXT(NAME, INT_ONLY, EXPR)                                                     \
     template <typename DstT, typename SrcT>                                                             \
     PTO_DEV void NAME##_IMPL(DstT &dst, SrcT &src, typename DstT::DType k)                              \
     {                                                                                                   \
-        static_assert(detail::same_dist<DstT, SrcT>, "[PTO][SA] " #NAME ": Vec tiles of equal size"); \
         using T = typename DstT::DType;                                                                 \
         static_assert(!(INT_ONLY) || std::is_integral_v<T>, "[PTO][SA] " #NAME ": integer tiles");      \
         using S = typename DstT::Storage;                                                               \
+        detail::Conformed<DstT, SrcT> c0(src);                                                          \
         _Pragma("unroll") for (int s = 0; s < S::Slots; ++s) _Pragma("unroll") for (int i = 0; i < detail::kVecChunk; ++i) \
         {                                                                                               \
-            const T a = src.S().v[s][i];                                                                 \
+            const T a = c0.S().v[s][i];                                                                  \
             dst.S().v[s][i] = (T)(EXPR);                                                                 \
         }                                                                                               \
     }
@@ -599,6 +625,7 @@ PTO_DEFINE_SCALAR_EXT(TXORS, true, a ^ k)
 PTO_DEFINE_SCALAR_EXT(TSHLS, true, a << k)
 PTO_DEFINE_SCALAR_EXT(TSHRS, true, a >> k)
 PTO_DEFINE_SCALAR_EXT(TREMS, false, detail::elem_rem<T>(a, k))
+PTO_DEFINE_SCALAR_EXT(TFMODS, false, detail::elem_rem<T>(a, k))
 #undef PTO_DEFINE_SCALAR_EXT
 
 template <typename DstT, typename SrcT>
@@ -651,7 +678,7 @@ PTO_DEV void TSUBSC_IMPL(TileT &dst, TileT &src0, typename TileT::DType k, TileT
 // Elementwise over the destination's valid region where the sources' valid regions may be smaller (cpu/TPartOp.hpp:19-45):
 // both sources valid -> op(src0, src1); one valid -> that source's element; none -> 0.  Tiles of one shape.
 namespace detail {
-template <int KIND, typename DstT, typename S0T, typename S1T> // KIND: 0 add, 1 max, 2 min
+template <int KIND, typename DstT, typename S0T, typename S1T> // KIND: 0 add, 1 max, 2 min, 3 mul
 PTO_DEV void part_op(DstT &dst, S0T &src0, S1T &src1)
 {
     using T = typename DstT::DType;
@@ -669,7 +696,7 @@ PTO_DEV void part_op(DstT &dst, S0T &src0, S1T &src1)
             if (r < dvr && c < dvc) {
                 const bool in0 = r < avr && c < avc, in1 = r < bvr && c < bvc;
                 const T a = src0.S().v[s][i], b = src1.S().v[s][i];
-                const T both = KIND == 0 ? (T)(a + b) : KIND == 1 ? (a < b ? b : a) : (b < a ? b : a);
+                const T both = KIND == 0 ? (T)(a + b) : KIND == 1 ? (a < b ? b : a) : KIND == 2 ? (b < a ? b : a) : (T)(a * b);
                 dst.S().v[s][i] = in0 && in1 ? both : in0 ? a : in1 ? b : (T)0;
             }
         }
@@ -682,6 +709,8 @@ template <typename DstT, typename S0T, typename S1T>
 PTO_DEV void TPARTMAX_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<1>(dst, src0, src1); }
 template <typename DstT, typename S0T, typename S1T>
 PTO_DEV void TPARTMIN_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<2>(dst, src0, src1); }
+template <typename DstT, typename S0T, typename S1T>
+PTO_DEV void TPARTMUL_IMPL(DstT &dst, S0T &src0, S1T &src1) { detail::part_op<3>(dst, src0, src1); }
 
 // ------------------------------------------------------------ TCI, TSCATTER, MSCATTER
 // TCI (cpu/TCI.hpp:16-35): dst[0, j] = start + j (descending: start - j) over the valid columns of a one-row tile.

@@ -16,9 +16,9 @@ PTO_DEV uint16_t _getFFTSMsg(CVSyncMode mode, uint16_t flag_id, uint16_t base_co
 }
 
 template <int CV_COMM_SLOT_BYTES = kCvCommSlotBytes, int CV_MAX_CORES = kCvMaxCores>
-PTO_DEV int TSYNC_CVID(int block_idx, uint8_t *cv_comm_buf)
+PTO_DEV int TSYNC_CVID(int blockId, uint8_t *cv_comm_buf)
 {
     (void)cv_comm_buf;
-    return block_idx;
+    return blockId;
 }
 } // namespace pto

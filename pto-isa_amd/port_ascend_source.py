@@ -24,9 +24,11 @@ script therefore does (nothing else is touched; the tile code itself compiles as
    function cannot keep a core-private `static`), and every `__global__` function starts with `PTO_KERNEL_PROLOGUE();`.
 7. `--define NAME[=VALUE]` puts `#define`s in front of everything (the `__DAV_*` macros by which a source asks which
    kind of core it is compiled for: a workgroup plays both, so both may be defined).
-9. `__global__` becomes `__global__ __launch_bounds__(pto::kBlockThreads)`.
-8. `--vec-in-memory` defines PTO_VEC_TILES_IN_MEMORY (Vec tiles are addresses in a per-workgroup unified buffer, see
+8. `__global__` becomes `__global__ __launch_bounds__(pto::kBlockThreads)`.
+9. `--vec-in-memory` defines PTO_VEC_TILES_IN_MEMORY (Vec tiles are addresses in a per-workgroup unified buffer, see
    include/pto/common/tile.hpp) and makes every launch prepare that buffer (`pto::host::LaunchBlocks`).
+10. A source that names the Ascend compiler's built-in variables `block_idx` / `block_num` gets them as macros over
+    `get_block_idx()` / `get_block_num()`, defined after the library's headers.
 """
 import argparse
 import os
@@ -118,27 +120,59 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
     first_dev = next((i for i in main_idx if re.match(r"\s*(template\s*<|AICORE\b|__global__\b|constexpr\s+AICORE|enum\b)", lines[i])), None)
     if first_dev is None:
         raise SystemExit("port_ascend_source: no device function found")
-    # the first host function: the first file-scope function whose body launches a kernel
-    launch_line = next((i for i in main_idx if "<<<" in lines[i]), None)
-    host_start = None
-    if launch_line is not None:
-        # walk back to the first line of the top-level declaration that encloses it: a line that starts at column 0
-        # with a name and follows an empty line, a closing brace, a semicolon, a comment or a directive
-        i = launch_line
-        while i > 0:
-            prev = lines[i - 1].strip()
-            starts = re.match(r"^[A-Za-z_]", lines[i]) is not None
-            if starts and (prev == "" or prev.endswith(("}", ";", "*/")) or prev.startswith(("//", "#"))):
-                break
-            i -= 1
-        host_start = i
-    res = lines[:first_dev] + ["PTO_DEVICE_CODE_BEGIN"]
-    if host_start is not None and host_start > first_dev:
-        res += lines[first_dev:host_start] + ["PTO_DEVICE_CODE_END"] + lines[host_start:]
-        notes.append("device code: lines %d-%d" % (first_dev + 1, host_start))
-    else:
-        res += lines[first_dev:] + ["PTO_DEVICE_CODE_END"]
-        notes.append("device code: line %d to the end" % (first_dev + 1))
+    # Top-level declarations of the main file from there on: a declaration ends where braces and parentheses are balanced
+    # and the line ends in `}` or `;`.  A host declaration is one that launches a kernel (`<<<`) or explicitly instantiates
+    # a host template (`template void ...;`); device regions are the runs between host declarations (sources that
+    # alternate kernels and their launchers get one region per run).
+    def strip_code(l):
+        l = re.sub(r'"(?:[^"\\]|\\.)*"', '""', l)
+        l = re.sub(r"'(?:[^'\\]|\\.)'", "''", l)
+        return l.split("//", 1)[0]
+    chunks, start, braces, parens, in_comment = [], None, 0, 0, False     # (first line, last line, is host)
+    for i in range(first_dev, len(lines)):
+        if i not in is_main:
+            continue
+        l = lines[i]
+        if in_comment:
+            if "*/" in l:
+                in_comment = False
+            continue
+        code = strip_code(l).strip()
+        if code.startswith("/*") and "*/" not in code:
+            in_comment = True
+            continue
+        if start is None:
+            if code == "" or code.startswith(("#", "/*")):
+                continue
+            start = i
+        braces += code.count("{") - code.count("}")
+        parens += code.count("(") - code.count(")")
+        if braces == 0 and parens == 0 and code.endswith(("}", ";")):
+            body = "\n".join(lines[start:i + 1])
+            host = "<<<" in body or re.match(r"\s*template\s+(?!<)", lines[start]) is not None or \
+                re.match(r'\s*extern\s+"C"\s+(?!.*__global__)', lines[start]) is not None and "AICORE" not in lines[start]
+            marked = re.search(r"\b(AICORE|__aicore__|__global__|PTO_INTERNAL|PTO_INST)\b", body.split("{", 1)[0]) is not None
+            chunks.append((start, i, host, marked))
+            start = None
+    res, pos, open_region, regions = lines[:first_dev], first_dev, False, 0
+    seen_host = False
+    for (c0, c1, host, marked) in chunks:
+        if host and open_region:
+            res.append("PTO_DEVICE_CODE_END")
+            open_region = False
+        seen_host = seen_host or host
+        res += lines[pos:c0]
+        # after the first host declaration only a declaration that carries a device marker opens a region again
+        if not host and not open_region and (marked or not seen_host):
+            res.append("PTO_DEVICE_CODE_BEGIN")
+            open_region = True
+            regions += 1
+        res += lines[c0:c1 + 1]
+        pos = c1 + 1
+    res += lines[pos:]
+    if open_region:
+        res.append("PTO_DEVICE_CODE_END")
+    notes.append("device code: %d region%s from line %d" % (regions, "" if regions == 1 else "s", first_dev + 1))
     head = "#define PTO_TILE_COPY_WRITEBACK 1\n"
     if vec_in_memory:
         head += "#define PTO_VEC_TILES_IN_MEMORY 1\n"
@@ -146,6 +180,13 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
         name, _, value = d.partition("=")
         head += "#define %s %s\n" % (name, value or "1")
     head += "#include <hip/hip_runtime.h>\n"
+    # the Ascend compiler's built-in variables `block_idx` / `block_num`
+    # (not where the source declares a variable of that name itself)
+    builtins = [n for n in ("block_idx", "block_num")
+                if re.search(r"\b%s\b" % n, text) and not re.search(r"\b(?:int|auto|unsigned|u?int(?:32|64)_t)\s+%s\b" % n, text)]
+    if builtins:
+        head += "#include <pto/pto-inst.hpp>\n" + "".join("#define %s (get_%s())\n" % (n, n) for n in builtins)
+        notes.append(" / ".join(builtins) + " -> get_...()")
     return head + "\n".join(res), notes
 
 
