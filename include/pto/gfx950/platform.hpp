@@ -93,6 +93,23 @@ PTO_DEV void lds_barrier()
     asm volatile("" ::: "memory");
 }
 } // namespace hw
+
+namespace host {
+constexpr unsigned kCuLdsBytes = 160 * 1024;
+// Dynamic LDS size for the launch of `kernel`: `want`, less whatever would push the workgroup's total past the
+// compute unit's 160 KiB.  The kernel's `__shared__` variables (staging buffers of tile instructions, per-wave slots
+// of function-local statics) are part of that total, and a dispatch that asks for more aborts the queue.
+inline unsigned LaunchLds(const void *kernel, unsigned want)
+{
+    hipFuncAttributes attr{};
+    if (hipFuncGetAttributes(&attr, kernel) != hipSuccess)
+        return want;
+    const unsigned fixed = static_cast<unsigned>(attr.sharedSizeBytes);
+    if (fixed >= kCuLdsBytes)
+        return 0;
+    return want + fixed > kCuLdsBytes ? kCuLdsBytes - fixed : want;
+}
+} // namespace host
 } // namespace pto
 
 // ---- pipes and events (global names, as kernel sources use them unqualified) ----

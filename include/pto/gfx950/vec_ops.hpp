@@ -397,9 +397,10 @@ enum class RowOp { Sub, Mul, Div, Add, Max, Min, ExpDif };
 // The per-row operand of a row-broadcast instruction: a [R,1] column (or [1,R] row) tile with one value per row, or, on
 // the NPU, a row-major [R, 32 / sizeof(T)] tile whose row r is applied to every 32-byte block of row r of the other
 // operand: value (r, c % width) (npu/a2a3/TRowExpandSub.hpp:59-77 and its test generator, trowexpandadd/gen_data.py:24-34).
+// A destination that is itself 32 bytes wide makes that form the elementwise operation.
 template <typename RowT, typename DstT>
 inline constexpr int kRowOperandWidth =
-    (RowT::isRowMajor && RowT::Rows > 1 && RowT::Cols * (int)sizeof(typename RowT::DType) == 32 && RowT::Cols != DstT::Cols) ? RowT::Cols : 1;
+    (RowT::isRowMajor && RowT::Rows > 1 && RowT::Cols * (int)sizeof(typename RowT::DType) == 32) ? RowT::Cols : 1;
 template <typename T, typename DstT>
 inline constexpr bool kIsRowOperand = !(T::Rows == DstT::Rows && T::Cols == DstT::Cols);
 

@@ -179,8 +179,11 @@ PTO_DEV void TCMP_PACKED_IMPL(DstT &dst, SrcT &src0, SrcT &src1, CmpMode mode)
     hw::lds_barrier();
 }
 
-// dst[i,j] = bit ? src0[i,j] : src1[i,j]; the bits are consumed in running order over the valid
-// region, byte after byte along the mask tile's valid columns, then its next row (TSel.hpp:22-49).
+// dst[i,j] = bit (i,j) ? src0[i,j] : src1[i,j]; row i of the mask tile holds the bits of row i, column j in byte j / 8,
+// lowest bit first (npu/a2a3/TSel.hpp:46-57: one compare mask per row, read at the mask tile's row stride; its test
+// generator tsel/gen_data.py:31-47).  The CPU simulation (cpu/TSel.hpp:27-47) consumes the bits in running order over
+// the valid region instead; the two agree whenever the valid width is a multiple of 8 and the mask's valid width is
+// exactly that many bytes, which is every case the simulation is tested on.
 template <typename TileT, typename MaskT>
 PTO_DEV void TSEL_IMPL(TileT &dst, MaskT &selMask, TileT &src0, TileT &src1)
 {
@@ -192,13 +195,12 @@ PTO_DEV void TSEL_IMPL(TileT &dst, MaskT &selMask, TileT &src0, TileT &src1)
             bits[e] = (uint8_t)selMask.S().v[s][i];
     });
     hw::lds_barrier();
-    const int vr = dst.GetValidRow(), vc = dst.GetValidCol(), vmc = selMask.GetValidCol();
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
     detail::for_each_owned<TileT>([&](int s, int i, int e) {
         const int r = e / TileT::Cols, c = e % TileT::Cols;
-        if (e < TileT::Numel && r < vr && c < vc) {
-            const int k = r * vc + c, b = k >> 3;
-            const uint32_t byte = bits[(b / vmc) * MaskT::Cols + (b % vmc)];
-            dst.S().v[s][i] = ((byte >> (k & 7)) & 1u) ? src0.S().v[s][i] : src1.S().v[s][i];
+        if (e < TileT::Numel && r < vr && c < vc && r < MaskT::Rows && (c >> 3) < MaskT::Cols) {
+            const uint32_t byte = bits[r * MaskT::Cols + (c >> 3)];
+            dst.S().v[s][i] = ((byte >> (c & 7)) & 1u) ? src0.S().v[s][i] : src1.S().v[s][i];
         }
     });
     hw::lds_barrier();
@@ -571,6 +573,18 @@ PTO_DEV void TTRANS_IMPL(DstT &dst, SrcT &src)
 // integer tiles for the bitwise and shift ops; TREM is `%` on integers and fmod (evaluated in double) on floats, a
 // zero divisor is the caller's error as in the reference; TADDC = a + b + c, TSUBC = a - b + c.
 namespace detail {
+// bitwise instructions on floating-point tiles work on the bit patterns (the NPU's vand / vor take any 16- or 32-bit type:
+// the reference's tand test has an fp16 case)
+template <typename T>
+using BitsOf = std::conditional_t<sizeof(T) == 1, uint8_t, std::conditional_t<sizeof(T) == 2, uint16_t, uint32_t>>;
+template <typename T, typename F>
+PTO_DEV T bitwise(T a, T b, F f)
+{
+    if constexpr (std::is_integral_v<T>)
+        return (T)f(a, b);
+    else
+        return __builtin_bit_cast(T, (BitsOf<T>)f(__builtin_bit_cast(BitsOf<T>, a), __builtin_bit_cast(BitsOf<T>, b)));
+}
 template <typename T>
 PTO_DEV T elem_rem(T a, T b)
 {
@@ -596,9 +610,9 @@ PTO_DEV T elem_rem(T a, T b)
             dst.S().v[s][i] = (T)(EXPR);                                                                 \
         }                                                                                               \
     }
-PTO_DEFINE_BINARY_EXT(TAND, true, a & b)
-PTO_DEFINE_BINARY_EXT(TOR, true, a | b)
-PTO_DEFINE_BINARY_EXT(TXOR, true, a ^ b)
+PTO_DEFINE_BINARY_EXT(TAND, false, detail::bitwise(a, b, [](auto x, auto y) { return x & y; }))
+PTO_DEFINE_BINARY_EXT(TOR, false, detail::bitwise(a, b, [](auto x, auto y) { return x | y; }))
+PTO_DEFINE_BINARY_EXT(TXOR, false, detail::bitwise(a, b, [](auto x, auto y) { return x ^ y; }))
 PTO_DEFINE_BINARY_EXT(TSHL, true, a << b)
 PTO_DEFINE_BINARY_EXT(TSHR, true, a >> b)
 PTO_DEFINE_BINARY_EXT(TREM, false, detail::elem_rem<T>(a, b))
@@ -619,9 +633,9 @@ PTO_DEFINE_BINARY_EXT(TFMOD, false, detail::elem_rem<T>(a, b)) // C fmod / integ
             dst.S().v[s][i] = (T)(EXPR);                                                                 \
         }                                                                                               \
     }
-PTO_DEFINE_SCALAR_EXT(TANDS, true, a & k)
-PTO_DEFINE_SCALAR_EXT(TORS, true, a | k)
-PTO_DEFINE_SCALAR_EXT(TXORS, true, a ^ k)
+PTO_DEFINE_SCALAR_EXT(TANDS, false, detail::bitwise(a, (T)k, [](auto x, auto y) { return x & y; }))
+PTO_DEFINE_SCALAR_EXT(TORS, false, detail::bitwise(a, (T)k, [](auto x, auto y) { return x | y; }))
+PTO_DEFINE_SCALAR_EXT(TXORS, false, detail::bitwise(a, (T)k, [](auto x, auto y) { return x ^ y; }))
 PTO_DEFINE_SCALAR_EXT(TSHLS, true, a << k)
 PTO_DEFINE_SCALAR_EXT(TSHRS, true, a >> k)
 PTO_DEFINE_SCALAR_EXT(TREMS, false, detail::elem_rem<T>(a, k))

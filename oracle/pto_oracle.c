@@ -1036,19 +1036,14 @@ void po_tcmps_packed(uint8_t *dst, int dst_ld, const float *a, int ld, int rows,
 void po_tsel_packed(float *dst, const uint8_t *mask, int mask_ld, int mask_valid_cols, const float *a, const float *b, int ld,
                     int rows, int cols)
 {
-    size_t mr = 0, mc = 0;
-    unsigned bit = 0;
+    /* npu/a2a3/TSel.hpp:46-57 and tsel/gen_data.py:31-47: mask row i serves row i, column j is bit j % 8 of byte j / 8.
+       cpu/TSel.hpp:27-47 runs on through the mask's valid columns instead; the same thing when cols == 8 * mask_valid_cols,
+       which holds for every case of the simulation's own tests. */
+    (void)mask_valid_cols;
     for (int i = 0; i < rows; i++)
-        for (int j = 0; j < cols; j++) { /* TSel.hpp:27-47 */
+        for (int j = 0; j < cols; j++) {
             size_t x = (size_t)i * (size_t)ld + (size_t)j;
-            unsigned sel = (mask[mr * (size_t)mask_ld + mc] >> bit) & 1u;
-            if (++bit == 8) {
-                bit = 0;
-                if (++mc == (size_t)mask_valid_cols) {
-                    mr++;
-                    mc = 0;
-                }
-            }
+            unsigned sel = (mask[(size_t)i * (size_t)mask_ld + (size_t)(j >> 3)] >> (j & 7)) & 1u;
             dst[x] = sel ? a[x] : b[x];
         }
 }

@@ -5,6 +5,7 @@
 hipcc cross-compiles without a GPU.  The library has no dependency on PyTorch.
 """
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -135,7 +136,65 @@ def build_ported(verbose=True):
             print("built", out)
 
 
+# Per-instruction test kernels of the reference (tests/npu/a2a3/src/st/testcase/<op>/<op>_kernel.cpp) that tests/st_ref_cases.py
+# runs on the GPU: each compiled unchanged (register tiles; no constant rewritten) into oracle/_ref/st/<op>.so.
+# oracle/_ref/st/manifest.json holds, per test, the launcher symbols (mangled -> demangled, so that the tests need no
+# binutils) and, for sources whose launchers are numbered cases (`launch<OP>Case<N>` kernels that fix the template arguments
+# of one run function each), the table case number -> [run function, template arguments] read from the source.
+ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip", "trelu", "tmov_vect", "tsub", "tmul", "tdiv", "tadd",
+              "tand", "tor", "tshl", "tshr", "tprelu", "taddplus", "tfmod", "trem", "txor", "tands", "tors", "txors", "tshls", "tshrs",
+              "tadds", "tsubs", "tmuls", "tdivs", "tmaxs", "tfmods", "trems", "tlrelu",
+              "tcolsum", "tcolmax", "tcolmin", "tcolprod", "trowexpand",
+              "trowexpandadd", "trowexpandsub", "trowexpandmul", "trowexpanddiv", "trowexpandmax", "trowexpandmin", "trowexpandexpdif",
+              "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
+              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt"]
+_ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
+
+
+def st_case_table(source_text):
+    """{case number: {"run": run function, "targs": [template arguments], "params": kernel parameter list}}"""
+    table = {}
+    for m in _ST_CASE.finditer(source_text):
+        table[m.group(1)] = {"run": m.group(3), "targs": [a.strip() for a in m.group(4).split(",")],
+                             "params": " ".join(m.group(2).replace("__gm__", "").split())}
+    return table
+
+
+def build_ported_st(verbose=True, jobs=8):
+    import concurrent.futures
+    import json
+    if not os.path.isdir(REFERENCE):
+        if verbose:
+            print("reference tree not mounted: per-instruction test kernels not built")
+        return
+    out_dir = os.path.join(PORTED_DIR, "st")
+    os.makedirs(out_dir, exist_ok=True)
+
+    def one(name):
+        rel = "tests/npu/a2a3/src/st/testcase/%s/%s_kernel.cpp" % (name, name)
+        lib = os.path.join(out_dir, name + ".so")
+        rc, err = port_and_compile(rel, [], 160 * 1024, lib, extra_flags=("-Wno-unknown-attributes",))
+        if rc != 0:
+            raise RuntimeError("ported build failed for %s:\n%s" % (rel, err))
+        syms = subprocess.run(["nm", "-D", "--defined-only", lib], capture_output=True, text=True, check=True).stdout.split("\n")
+        mangled = [l.split()[2] for l in syms if len(l.split()) == 3 and l.split()[1] in "TW"]
+        demangled = subprocess.run(["c++filt"], input="\n".join(mangled), capture_output=True, text=True, check=True).stdout.split("\n")
+        with open(os.path.join(REFERENCE, rel)) as f:
+            table = st_case_table(f.read())
+        return name, {"launchers": {m: d for m, d in zip(mangled, demangled) if d.startswith("void ") and "pto::" not in d.split("(")[0]},
+                      "cases": table}
+    manifest = {}
+    with concurrent.futures.ThreadPoolExecutor(jobs) as ex:
+        for name, entry in ex.map(one, ST_KERNELS):
+            manifest[name] = entry
+            if verbose:
+                print("built", os.path.join(out_dir, name + ".so"), "(%d launchers)" % len(entry["launchers"]))
+    with open(os.path.join(out_dir, "manifest.json"), "w") as f:
+        json.dump(manifest, f, indent=1, sort_keys=True)
+
+
 if __name__ == "__main__":
     build()
     build_ported()
+    build_ported_st()
     sys.exit(0)

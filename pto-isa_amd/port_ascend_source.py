@@ -61,6 +61,36 @@ def inline_local_includes(text, directory, seen=None):
     return LOCAL_INCLUDE.sub(repl, text)
 
 
+def kernel_before(text, pos):
+    """The kernel expression (`name` or `name<template arguments>`) that ends just before the `<<<` at text[pos]."""
+    i = pos
+    while i > 0 and text[i - 1].isspace():
+        i -= 1
+    end = i
+    if i > 0 and text[i - 1] == ">":
+        depth = 0
+        while i > 0:
+            i -= 1
+            if text[i] == ">":
+                depth += 1
+            elif text[i] == "<":
+                depth -= 1
+                if depth == 0:
+                    break
+            elif text[i] in ";{}":
+                return None
+        if depth != 0:
+            return None
+        while i > 0 and text[i - 1].isspace():
+            i -= 1
+    start = i
+    while start > 0 and (text[start - 1].isalnum() or text[start - 1] in "_:"):
+        start -= 1
+    if start == i:
+        return None
+    return " ".join(text[start:end].split())
+
+
 def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in_memory=False):
     notes = []
     if directory is not None:
@@ -79,7 +109,11 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
 
     def launch(m):
         b = blocks % (m.group(1), m.group(2)) if vec_in_memory else m.group(1)
-        return "<<<%s, pto::kBlockThreads, %d, (hipStream_t)(%s)>>>" % (b, lds_bytes, m.group(2))
+        kernel = kernel_before(m.string, m.start())
+        # the kernel's own static LDS (staging buffers of the tile library, PTO_CORE_STATIC slots) comes out of the same
+        # 160 KiB: the dynamic part shrinks by it, or the dispatch would be refused by the hardware queue
+        lds = "pto::host::LaunchLds((const void *)(%s), %d)" % (kernel, lds_bytes) if kernel else "%d" % lds_bytes
+        return "<<<%s, pto::kBlockThreads, %s, (hipStream_t)(%s)>>>" % (b, lds, m.group(2))
     text, n = LAUNCH.subn(launch, text)
     notes.append("%d launch statement%s rewritten" % (n, "" if n == 1 else "s"))
 

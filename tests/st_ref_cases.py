@@ -1,0 +1,470 @@
+"""Cases for running the reference's own per-instruction NPU test kernels (tests/npu/a2a3/src/st/testcase/<op>/<op>_kernel.cpp,
+compiled unchanged through pto-isa_amd/port_ascend_source.py into oracle/_ref/st/<op>.so by pto-isa_amd/build.py) on the
+GPU.  Every explicit instantiation of a launcher that a kernel source exports is one case; its template arguments, read
+from the demangled symbol, give the element type, the tile shapes and the valid region; launchers that are numbered cases
+(`launch<OP>TestCase<N>`) take them from the case table that the build reads from the kernel source (manifest.json).  What
+the launcher expects in memory is restated per test from the kernel source (cited), the expected result from the test's
+generator (<op>/gen_data.py: plain numpy formulas)."""
+import ctypes as C
+import json
+import os
+import re
+from types import SimpleNamespace
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ST_DIR = os.path.join(ROOT, "oracle", "_ref", "st")
+
+CTYPE = {"float": (np.float32, C.c_float), "int": (np.int32, C.c_int32), "short": (np.int16, C.c_int16),
+         "unsigned short": (np.uint16, C.c_uint16), "signed char": (np.int8, C.c_int8), "unsigned char": (np.uint8, C.c_uint8),
+         "unsigned int": (np.uint32, C.c_uint32), "long": (np.int64, C.c_int64)}
+CTYPE.update({"int32_t": CTYPE["int"], "int16_t": CTYPE["short"], "uint16_t": CTYPE["unsigned short"], "uint32_t": CTYPE["unsigned int"],
+              "int8_t": CTYPE["signed char"], "uint8_t": CTYPE["unsigned char"]})
+
+
+def _ints(m, names):
+    return {n: int(m.group(n).rstrip("u")) for n in names}
+
+
+# ---- families: how the template arguments map to buffers -------------------------------------------------------------
+# Every family returns (buffers, valid) with buffers = [(rows, leading dimension), ...] in argument order, output first,
+# and valid = (rows, cols) of the region that is computed and stored.
+
+def fam_g_t(p):        # <T, gRows, gCols, tRows, tCols, ...>: memory [gRows, gCols] contiguous (e.g. tabs_kernel.cpp:20-22)
+    return (p.g0, p.g1), (p.g0, p.g1)
+
+
+def fam_t_v_ld_tile(p):  # <T, tRows, tCols, vRows, vCols>, row stride tCols (tadd_kernel.cpp:20-21)
+    return (p.v0, p.t1), (p.v0, p.v1)
+
+
+def fam_t_v_ld_valid(p):  # <T, tRows, tCols, vRows, vCols>, row stride vCols (tor_kernel.cpp:20-21)
+    return (p.v0, p.v1), (p.v0, p.v1)
+
+
+UNARY = r"<(?P<T>[a-z ]+), (?P<g0>\d+), (?P<g1>\d+), (?P<t0>\d+), (?P<t1>\d+)(?:, (?P<flag>true|false))?>\((?:[a-z ]+\*, ){2}void\*\)"
+BINARY5 = r"<(?P<T>[a-z ]+), (?P<a>\d+), (?P<b>\d+), (?P<c>\d+), (?P<d>\d+)>\((?:[a-z ]+\*, ){3}void\*\)"
+BINARY9 = (r"<(?P<T>[a-z ]+), (?P<dH>\d+), (?P<dW>\d+), (?P<aH>\d+), (?P<aW>\d+), (?P<bH>\d+), (?P<bW>\d+), (?P<vR>\d+), (?P<vC>\d+)>"
+           r"\((?:[a-z ]+\*, ){3}void\*\)")
+SCALAR7 = (r"<(?P<T>[a-z ]+), (?P<dH>\d+), (?P<dW>\d+), (?P<sH>\d+), (?P<sW>\d+), (?P<vR>\d+), (?P<vC>\d+)>"
+           r"\((?:[a-z ]+\*, ){2}[a-z ]+, void\*\)")
+
+
+def f64(x):
+    return x.astype(np.float64)
+
+
+def _shift_left(a, b):
+    return np.left_shift(a, b.astype(a.dtype))
+
+
+def _shift_right(a, b):
+    return np.right_shift(a, b.astype(a.dtype))
+
+
+def _fmod(a, b):
+    if a.dtype.kind == "f":
+        return np.fmod(f64(a), f64(b))
+    return np.fmod(a, b)
+
+
+def _prelu(a, b):
+    return np.where(a > 0, a, a * b)
+
+
+# name -> dict(launcher, regex tail, layout, inputs, expected, half, exact)
+#   layout: 'g' (gRows, gCols, tRows, tCols), 'tile_ld' / 'valid_ld' (tRows, tCols, vRows, vCols), 'nine', 'scalar7'
+#   inputs: 'any' | 'pos' | 'bits' | 'shift' | 'rem' ; half: `unsigned short` instantiations are fp16 (aclFloat16)
+SPECS = {
+    # unary, <T, gRows, gCols, tRows, tCols[, inPlace]> (tabs_kernel.cpp:17-44 and alike)
+    "tabs": dict(fn="LaunchTAbs", tail=UNARY, layout="g", nin=1, inputs="any", half=True, op=lambda a: np.abs(a)),
+    "tneg": dict(fn="LaunchTNeg", tail=UNARY, layout="g", nin=1, inputs="any", half=True, op=lambda a: -a),
+    "tnot": dict(fn="LaunchTNot", tail=UNARY, layout="g", nin=1, inputs="bits", half=False, op=lambda a: ~a),
+    "texp": dict(fn="LaunchTExp", tail=UNARY, layout="g", nin=1, inputs="any", half=True, op=lambda a: np.exp(f64(a))),
+    "tlog": dict(fn="LaunchTLog", tail=UNARY, layout="g", nin=1, inputs="pos", half=True, op=lambda a: np.log(f64(a))),
+    "tsqrt": dict(fn="LaunchTSqrt", tail=UNARY, layout="g", nin=1, inputs="pos", half=True, op=lambda a: np.sqrt(f64(a))),
+    "trsqrt": dict(fn="LaunchTRsqrt", tail=UNARY, layout="g", nin=1, inputs="pos", half=True, op=lambda a: 1.0 / np.sqrt(f64(a))),
+    "trecip": dict(fn="LaunchTRecip", tail=UNARY, layout="g", nin=1, inputs="pos", half=True, op=lambda a: 1.0 / f64(a)),
+    "trelu": dict(fn="LaunchTRelu", tail=UNARY, layout="g", nin=1, inputs="any", half=True, op=lambda a: np.maximum(a, 0)),
+    "tmov_vect": dict(fn="launchTMOV", tail=UNARY, layout="g", nin=1, inputs="any", half=True, op=lambda a: a),
+    # binary, <T, gRows, gCols, tRows, tCols> (tdiv_kernel.cpp:17-45, tmul, tsub)
+    "tsub": dict(fn="LaunchTSub", tail=BINARY5, layout="g", nin=2, inputs="any", half=True, op=lambda a, b: a - b),
+    "tmul": dict(fn="LaunchTMul", tail=BINARY5, layout="g", nin=2, inputs="any", half=True, op=lambda a, b: a * b),
+    "tdiv": dict(fn="LaunchTDiv", tail=BINARY5, layout="g", nin=2, inputs="pos", half=True, op=lambda a, b: f64(a) / f64(b)),
+    # binary, <T, tRows, tCols, vRows, vCols>
+    "tadd": dict(fn="LaunchTAdd", tail=BINARY5, layout="tile_ld", nin=2, inputs="any", half=True, op=lambda a, b: a + b),
+    "tand": dict(fn="LaunchTAnd", tail=BINARY5, layout="valid_ld", nin=2, inputs="bits", half=False, op=lambda a, b: a & b),
+    "tor": dict(fn="LaunchTOr", tail=BINARY5, layout="valid_ld", nin=2, inputs="bits", half=False, op=lambda a, b: a | b),
+    "tshl": dict(fn="LaunchTShl", tail=BINARY5, layout="valid_ld", nin=2, inputs="shift", half=False, op=_shift_left),
+    "tshr": dict(fn="LaunchTShr", tail=BINARY5, layout="valid_ld", nin=2, inputs="shift", half=False, op=_shift_right),
+    "tprelu": dict(fn="LaunchTPrelu", tail=BINARY5, layout="valid_ld", nin=2, inputs="any", half=True, op=_prelu),
+    # binary on tiles of three different widths, <T, dstH, dstW, src0H, src0W, src1H, src1W, vRows, vCols>: every buffer has
+    # its tile's width as row stride (taddplus_kernel.cpp:17-51)
+    "taddplus": dict(fn="LaunchTAdd", tail=BINARY9, layout="nine", nin=2, inputs="any", half=True, op=lambda a, b: a + b),
+    "tfmod": dict(fn="LaunchTFMOD", tail=BINARY9, layout="nine", nin=2, inputs="rem", half=True, op=_fmod),
+    # TREM: the NPU takes the sign of the divisor (a - floor(a / b) b, npu/a2a3/TRem.hpp:22-35; np.remainder in its
+    # generator), the CPU simulation that of the dividend (ElementOp.h:145-156: % and fmod), which this library follows:
+    # the two agree for dividends >= 0, which is what the case draws
+    "trem": dict(fn="LaunchTREM", tail=BINARY9, layout="nine", nin=2, inputs="rempos", half=True, op=_fmod),
+    "txor": dict(fn="LaunchTXor", tail=BINARY9, layout="nine", nin=2, inputs="bits", half=False, op=lambda a, b: a ^ b),
+    # tile (op) scalar, <T, dstH, dstW, srcH, srcW, vRows, vCols>, the scalar by value (tands_kernel.cpp:17-49)
+    "tands": dict(fn="LaunchTAndS", tail=SCALAR7, layout="scalar7", nin=1, inputs="bits", half=False, op=lambda a, k: a & k),
+    "tors": dict(fn="LaunchTOrS", tail=SCALAR7, layout="scalar7", nin=1, inputs="bits", half=False, op=lambda a, k: a | k),
+    "txors": dict(fn="LaunchTXorS", tail=SCALAR7, layout="scalar7", nin=1, inputs="bits", half=False, op=lambda a, k: a ^ k),
+    "tshls": dict(fn="LaunchTShlS", tail=SCALAR7, layout="scalar7", nin=1, inputs="shift", half=False, op=lambda a, k: np.left_shift(a, k)),
+    "tshrs": dict(fn="LaunchTShrS", tail=SCALAR7, layout="scalar7", nin=1, inputs="shift", half=False, op=lambda a, k: np.right_shift(a, k)),
+}
+
+
+def manifest():
+    path = os.path.join(ST_DIR, "manifest.json")
+    if not os.path.exists(path):
+        return {}
+    with open(path) as f:
+        return json.load(f)
+
+
+def _pattern(spec):
+    return re.compile(r"^void " + re.escape(spec["fn"]) + spec["tail"] + "$")
+
+
+def cases():
+    """[(test, mangled symbol, demangled symbol)] for every launcher instantiation of every test in SPECS that was built."""
+    out = []
+    man = manifest()
+    for test, spec in SPECS.items():
+        pat = _pattern(spec)
+        for mangled, demangled in sorted(man.get(test, {}).get("launchers", {}).items(), key=lambda kv: kv[1]):
+            if pat.match(demangled):
+                out.append((test, mangled, demangled))
+    return out
+
+
+def _elem(tname, half):
+    """numpy dtype and ctypes type of a C++ element type name (as demangled, or as written in a kernel source)."""
+    dtype, ctype = CTYPE[tname]
+    if tname in ("unsigned short", "uint16_t") and half:
+        dtype = np.float16
+    return np.dtype(dtype), ctype
+
+
+def plan(test, demangled):
+    """-> SimpleNamespace(dtype, outs [(dtype, (rows, ld))], ins [(dtype, (rows, ld))], regions [(rows, cols)] per output,
+    scalar None | (ctypes type, value), expect(ins, scalar) -> [array per output], spec)"""
+    spec = SPECS[test]
+    m = _pattern(spec).match(demangled)
+    if "planner" in spec:
+        return spec["planner"](test, spec, m)
+    dtype, ctype = _elem(m.group("T"), spec["half"])
+    lay = spec["layout"]
+    if lay == "g":
+        p = SimpleNamespace(**_ints(m, ["g0", "g1", "t0", "t1"])) if "g0" in m.groupdict() else \
+            SimpleNamespace(g0=int(m.group("a")), g1=int(m.group("b")), t0=int(m.group("c")), t1=int(m.group("d")))
+        buf, valid = (p.g0, p.g1), (p.g0, p.g1)
+        buffers = [buf] * (1 + spec["nin"])
+    elif lay in ("tile_ld", "valid_ld"):
+        t0, t1, v0, v1 = (int(m.group(k)) for k in "abcd")
+        buf = (v0, t1 if lay == "tile_ld" else v1)
+        buffers, valid = [buf] * (1 + spec["nin"]), (v0, v1)
+    elif lay == "nine":
+        q = _ints(m, ["dH", "dW", "aH", "aW", "bH", "bW", "vR", "vC"])
+        buffers, valid = [(q["dH"], q["dW"]), (q["aH"], q["aW"]), (q["bH"], q["bW"])], (q["vR"], q["vC"])
+    elif lay == "scalar7":
+        q = _ints(m, ["dH", "dW", "sH", "sW", "vR", "vC"])
+        buffers, valid = [(q["dH"], q["dW"]), (q["sH"], q["sW"])], (q["vR"], q["vC"])
+    else:
+        raise AssertionError(lay)
+    scalar = None
+    if lay == "scalar7":
+        scalar = (ctype, 3 if spec["inputs"] == "shift" else 0x5A5A & int(np.iinfo(dtype).max))
+    return _elementwise_plan(spec, dtype, buffers, valid, scalar)
+
+
+def _elementwise_plan(spec, dtype, buffers, valid, scalar, scalar_first=False):
+    """One output, spec['nin'] inputs of the same element type, the operation applied to the valid region."""
+    vr, vc = valid
+    op = spec["op"]
+
+    def expect(ins, k):
+        a = ins[0][:vr, :vc]
+        if k is not None:
+            k = dtype.type(k)
+            return [op(k, a) if scalar_first else op(a, k)]
+        return [op(a) if len(ins) == 1 else op(a, ins[1][:vr, :vc])]
+    return SimpleNamespace(dtype=dtype, outs=[(dtype, buffers[0])], ins=[(dtype, b) for b in buffers[1:]], regions=[valid],
+                           scalar=scalar, expect=expect, spec=spec)
+
+
+# ---- numbered cases: launch<OP>TestCase<N>(void *out, void *src, float scalar, stream) -> run<T, dstRows, dstCols, rows,
+# validRows, cols, validCols[, srcDivScalar]> (tadds_kernel.cpp:17-45, tdivs_kernel.cpp:17-48): output buffer [dstRows,
+# dstCols], input [rows, cols], the scalar converted from float inside the launcher
+CASE_SCALAR = r"<(?P<case>\d+)u>\(void\*, void\*, float, ihipStream_t\*\)"
+SRC_TYPES = {"float": "float", "half": "unsigned short", "aclFloat16": "unsigned short", "int32_t": "int", "int16_t": "short",
+             "uint16_t": "unsigned short", "uint32_t": "unsigned int", "int8_t": "signed char", "uint8_t": "unsigned char"}
+
+
+def case_entry(test, m):
+    return manifest()[test]["cases"][m.group("case")]
+
+
+def plan_case_scalar(test, spec, m):
+    e = case_entry(test, m)
+    t = e["targs"]
+    dtype, _ = _elem(SRC_TYPES[t[0]], True)
+    dR, dC, rows, vR, cols, vC = (int(x) for x in t[1:7])
+    scalar_first = len(t) > 7 and t[7] == "false"
+    value = 7.0 if spec["inputs"] in ("rem", "rempos") else (3.0 if dtype.kind != "f" else 1.5)
+    return _elementwise_plan(spec, dtype, [(dR, dC), (rows, cols)], (vR, vC), (C.c_float, value), scalar_first)
+
+
+def _div(a, b):
+    if np.asarray(a).dtype.kind == "f":
+        return np.asarray(a, np.float64) / np.asarray(b, np.float64)
+    return (np.asarray(a, np.int64) // np.asarray(b, np.int64)).astype(np.asarray(a).dtype)      # operands are positive
+
+
+SPECS.update({
+    "tadds": dict(fn="launchTADDSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=lambda a, k: a + k),
+    "tsubs": dict(fn="launchTSUBSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=lambda a, k: a - k),
+    "tmuls": dict(fn="launchTMULSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=lambda a, k: a * k),
+    "tdivs": dict(fn="launchTDIVSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="pos", op=_div),
+    "tmaxs": dict(fn="launchTMAXSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=lambda a, k: np.maximum(a, k)),
+    "tfmods": dict(fn="launchTFMODSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="rem", op=_fmod),
+    # TREMS: dividends >= 0, for which the NPU's floor form and the CPU simulation's truncating form agree (see "trem")
+    "trems": dict(fn="launchTREMSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="rempos", op=_fmod),
+    "tlrelu": dict(fn="launchTLRELUTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=_prelu),
+})
+
+
+def TAIL(ints, nptr, suffix="", ptr0=None):
+    """Demangled `<T, int..., suffix>(T*, ... nptr pointers ..., void*)`; ptr0: type of the first pointer if it is not T."""
+    ptrs = (re.escape(ptr0) + r"\*, " if ptr0 else "") + r"(?:[a-z ]+\*, ){%d}" % (nptr - (1 if ptr0 else 0))
+    return r"<(?P<T>[a-z ]+)" + "".join(r", (?P<%s>-?\d+)u?" % n for n in ints) + suffix + r">\(" + ptrs + r"void\*\)"
+
+
+def _plan(spec, outs, ins, regions, expect, scalar=None):
+    return SimpleNamespace(dtype=ins[0][0] if ins else outs[0][0], outs=outs, ins=ins, regions=regions, scalar=scalar,
+                           expect=lambda arrays, k: expect(arrays), spec=spec)
+
+
+# ---- column reductions: launchTCOLSUM<T, cols, srcRows, validRows[, binary]>: [validRows, cols] of a [srcRows, cols] buffer
+# reduced to [1, cols] (tcolsum_kernel.cpp:17-50)
+def plan_colreduce(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    cols, rows, vr = (int(m.group(k)) for k in ("cols", "rows", "vr"))
+    return _plan(spec, [(dt, (1, cols))], [(dt, (rows, cols))], [(1, cols)], lambda a: [spec["op"](a[0][:vr])[None, :]])
+
+
+def _sum0(a):
+    return np.sum(a, axis=0, dtype=np.float64 if a.dtype.kind == "f" else a.dtype)
+
+
+def _prod0(a):
+    return np.prod(a, axis=0, dtype=np.float64 if a.dtype.kind == "f" else a.dtype)
+
+
+# ---- TROWEXPAND: launchTROWEXPAND<T, rows, srcCols, srcValidCols, dstCols, dstValidCols>: column 0 of the source across
+# the valid columns of the destination (trowexpand_kernel.cpp:19-43; the 32-byte-row form :45-72 has srcCols == 1)
+def plan_rowexpand(test, spec, m):
+    dt, _ = _elem(m.group("T"), False)
+    rows, sc, svc, dc, dvc = (int(m.group(k)) for k in ("rows", "sc", "svc", "dc", "dvc"))
+    return _plan(spec, [(dt, (rows, dc))], [(dt, (rows, sc))], [(rows, dvc)], lambda a: [np.repeat(a[0][:, :1], dvc, axis=1)])
+
+
+# ---- dst = matrix (op) per-row operand: launchTRowExpandAdd[2]<T, validRows, validCols, rows, cols, matrixFirst>: the
+# per-row operand is a [rows32, 1] column (first form) or [rows32, 32 bytes] rows of which element (r, c mod K) is used
+# (second form), rows32 = validRows rounded up to 32 bytes of elements (trowexpandadd_kernel.cpp:17-88)
+def plan_rowexpand_bin(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    vr, vc, rows, cols = (int(m.group(k)) for k in ("vr", "vc", "rows", "cols"))
+    per = 32 // dt.itemsize
+    r32 = -(-vr // per) * per
+    K = per if m.group("two") else 1
+    mat_first = m.group("flag") == "true"
+    op = spec["op"]
+
+    def expect(a):
+        mat, row = a[0][:vr, :vc], a[1][:vr][:, np.arange(vc) % K]
+        return [op(mat, row) if mat_first else op(row, mat)]
+    return _plan(spec, [(dt, (rows, cols))], [(dt, (rows, cols)), (dt, (r32, K))], [(vr, vc)], expect)
+
+
+# ---- dst = matrix (op) per-column operand: launchTColExpandAdd<T, dstRows, dstCols, 1, cols> (tcolexpandadd_kernel.cpp:17-56)
+def plan_colexpand_bin(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    dr, dc, sr, sc = (int(m.group(k)) for k in ("dr", "dc", "sr", "sc"))
+    return _plan(spec, [(dt, (dr, dc))], [(dt, (dr, dc)), (dt, (sr, sc))], [(dr, dc)], lambda a: [spec["op"](a[0], a[1][:1, :dc])])
+
+
+def _expdif(a, b):
+    return np.exp(f64(a - b))          # the difference in the tile's element type, as the instruction forms it
+
+
+ROWBIN = r"(?P<two>2)?" + TAIL(["vr", "vc", "rows", "cols"], 3, r", (?P<flag>true|false)")
+COLBIN = TAIL(["dr", "dc", "sr", "sc"], 3)
+_ROWCOL_OPS = {"Add": ("any", lambda a, b: a + b), "Sub": ("any", lambda a, b: a - b), "Mul": ("any", lambda a, b: a * b),
+               "Div": ("pos", lambda a, b: f64(a) / f64(b)), "Max": ("any", np.maximum), "Min": ("any", np.minimum),
+               "Expdif": ("any", _expdif)}
+for _name, (_kind, _op) in _ROWCOL_OPS.items():
+    SPECS["trowexpand" + _name.lower()] = dict(fn="launchTRowExpand" + _name, tail=ROWBIN, planner=plan_rowexpand_bin, inputs=_kind, op=_op)
+    SPECS["tcolexpand" + _name.lower()] = dict(fn="TColExpand%sTest::launchTColExpand%s" % (_name, _name), tail=COLBIN,
+                                               planner=plan_colexpand_bin, inputs=_kind, op=_op)
+
+COLRED = TAIL(["cols", "rows", "vr"], 2)
+REDUCE_TOL = {"float32": 1e-5, "float16": 4e-3}            # the order of a reduction is the implementation's
+REDUCE_ATOL = {"float32": 2e-5, "float16": 2e-2}           # sums of up to 31 values of magnitude up to 4 that may cancel
+SPECS.update({
+    "tcolsum": dict(fn="launchTCOLSUM", tail=TAIL(["cols", "rows", "vr"], 2, r", (?:true|false)"), planner=plan_colreduce, inputs="any",
+                    op=_sum0, tol=REDUCE_TOL, atol=REDUCE_ATOL),
+    "tcolmax": dict(fn="launchTCOLMAX", tail=COLRED, planner=plan_colreduce, inputs="any", op=lambda a: np.max(a, axis=0)),
+    "tcolmin": dict(fn="launchTCOLMIN", tail=COLRED, planner=plan_colreduce, inputs="any", op=lambda a: np.min(a, axis=0)),
+    "tcolprod": dict(fn="launchTCOLPROD", tail=COLRED, planner=plan_colreduce, inputs="small", op=_prod0, tol=REDUCE_TOL),
+    "trowexpand": dict(fn="launchTROWEXPAND", tail=TAIL(["rows", "sc", "svc", "dc", "dvc"], 2), planner=plan_rowexpand, inputs="bits"),
+})
+
+
+# ---- comparisons into bit masks: LaunchTCmp<T, gRows, gCols, tRows, tCols, mode>(uint8 *out, T *src0, T *src1): the
+# [tRows, tCols] corner of [gRows, gCols] buffers; byte b of an output row holds columns 8b .. 8b+7, lowest bit first
+# (tcmp_kernel.cpp:17-48, gen_data.py:49-56).  LaunchTCmps compares with the scalar src1[0] (tcmps_kernel.cpp:17-42).
+CMP = [np.equal, np.not_equal, np.less, np.less_equal, np.greater, np.greater_equal]       # pto::CmpMode 0..5
+
+
+def plan_cmp(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    gr, gc, tr, tc, mode = (int(m.group(k)) for k in ("gr", "gc", "tr", "tc", "mode"))
+    scalar_form = spec["scalar_form"]
+    u8 = np.dtype(np.uint8)
+
+    def expect(a):
+        lhs, rhs = a[0][:tr, :tc], (a[1][0, 0] if scalar_form else a[1][:tr, :tc])
+        return [np.packbits(CMP[mode](lhs, rhs), axis=1, bitorder="little")]
+    return _plan(spec, [(u8, (gr, gc))], [(dt, (gr, gc)), (dt, (1, 8) if scalar_form else (gr, gc))], [(tr, tc // 8)], expect)
+
+
+# ---- TSEL: LaunchTSel<T, rows, cols, validRows, validCols>(T *out, uint8 *mask, T *src0, T *src1): bit (r, c) set takes
+# src0, clear takes src1; mask rows of ceil(validCols / 8) bytes (tsel_kernel.cpp:17-66, gen_data.py:31-47)
+def plan_sel(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    vr, vc = int(m.group("vr")), int(m.group("vc"))
+    mc = (vc + 7) // 8
+
+    def expect(a):
+        bits = np.unpackbits(a[0], axis=1, bitorder="little")[:, :vc].astype(bool)
+        return [np.where(bits, a[1], a[2])]
+    return _plan(spec, [(dt, (vr, vc))], [(np.dtype(np.uint8), (vr, mc), "bits"), (dt, (vr, vc)), (dt, (vr, vc))], [(vr, vc)], expect)
+
+
+# ---- TTRI: LaunchTTri<T, upper, diagonal, tileRows, tileCols, validRows, validCols>(T *out): ones on and above (upper) or
+# on and below (lower) the diagonal-th diagonal (ttri_kernel.cpp:17-33, gen_data.py:26-29)
+def plan_tri(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    upper, diag, vr, vc = (int(m.group(k)) for k in ("upper", "diag", "vr", "vc"))
+    ones = np.ones((vr, vc), dtype=dt)
+    return _plan(spec, [(dt, (vr, vc))], [], [(vr, vc)], lambda a: [np.triu(ones, k=diag) if upper else np.tril(ones, k=diag)])
+
+
+SPECS.update({
+    "tcmp": dict(fn="LaunchTCmp", tail=TAIL(["gr", "gc", "tr", "tc"], 3, r", \(pto::CmpMode\)(?P<mode>\d)", ptr0="unsigned char"),
+                 planner=plan_cmp, inputs="small", scalar_form=False),
+    "tcmps": dict(fn="LaunchTCmps", tail=TAIL(["gr", "gc", "tr", "tc", "mode"], 3, ptr0="unsigned char"), planner=plan_cmp, inputs="small",
+                  scalar_form=True),
+    "tsel": dict(fn="LaunchTSel", tail=r"<(?P<T>[a-z ]+), (?P<r>\d+), (?P<c>\d+), (?P<vr>\d+), (?P<vc>\d+)>\([a-z ]+\*, unsigned char\*, [a-z ]+\*, [a-z ]+\*, void\*\)",
+                 planner=plan_sel, inputs="any"),
+    "ttri": dict(fn="LaunchTTri", tail=TAIL(["upper", "diag", "tr", "tc", "vr", "vc"], 1), planner=plan_tri, inputs="any"),
+})
+
+
+# ---- row reductions, numbered cases: launchTROWSUMTestCase<N>(void *out, void *src, stream) -> run<T, rows, validRows,
+# srcCols, srcValidCols, 1>: out[r] = reduction of row r over the valid columns, as a vector of validRows elements
+# (trowsum_kernel.cpp:17-45; :47-80 stores the same vector from a column-major [rows, 1] tile viewed as [1, rows])
+CASE_UNARY = r"<(?P<case>\d+)u>\(void\*, void\*, ihipStream_t\*\)"
+
+
+def plan_rowreduce(test, spec, m):
+    t = case_entry(test, m)["targs"]
+    dt, _ = _elem(SRC_TYPES[t[0]], True)
+    rows, vr, sc, svc = (int(x) for x in t[1:5])
+    return _plan(spec, [(dt, (1, rows))], [(dt, (rows, sc))], [(1, vr)], lambda a: [spec["op"](a[0][:vr, :svc])[None, :]])
+
+
+SPECS.update({
+    "trowsum": dict(fn="launchTROWSUMTestCase", tail=CASE_UNARY, planner=plan_rowreduce, inputs="any", tol=REDUCE_TOL,
+                    atol={"float32": 2e-4, "float16": 5e-2}, op=lambda a: np.sum(a, axis=1, dtype=np.float64)),
+    "trowmax": dict(fn="launchTROWMAXTestCase", tail=CASE_UNARY, planner=plan_rowreduce, inputs="any", op=lambda a: np.max(a, axis=1)),
+    "trowmin": dict(fn="launchTROWMINTestCase", tail=CASE_UNARY, planner=plan_rowreduce, inputs="any", op=lambda a: np.min(a, axis=1)),
+})
+
+
+# ---- TCVT: launchTCVT<D, S, gRows, gCols, tRows, tCols>(D *dst, S *src): round to nearest even (CAST_RINT), values inside
+# the destination's range (tcvt_kernel.cpp:19-66; gen_data.py draws [-100, 100] and [-10000, 10000])
+def plan_cvt(test, spec, m):
+    dd, _ = _elem(m.group("D"), True)
+    sd, _ = _elem(m.group("T"), True)
+    gr, gc = int(m.group("gr")), int(m.group("gc"))
+    narrow = min(dd.itemsize, sd.itemsize) == 1
+    kind = "cvt_u" if dd.kind == "u" else ("cvt_narrow" if narrow else "cvt")
+
+    def expect(a):
+        x = a[0]
+        if sd.kind == "f" and dd.kind != "f":
+            return [np.rint(x.astype(np.float64)).astype(dd)]
+        return [x.astype(dd)]
+    return _plan(spec, [(dd, (gr, gc))], [(sd, (gr, gc), kind)], [(gr, gc)], expect)
+
+
+EXACT = {"float32": 0.0, "float16": 0.0}
+SPECS["tcvt"] = dict(fn="launchTCVT", tail=r"<(?P<D>[a-z ]+), (?P<T>[a-z ]+), (?P<gr>\d+), (?P<gc>\d+), (?P<tr>\d+), (?P<tc>\d+)>\([a-z ]+\*, [a-z ]+\*, void\*\)",
+                     planner=plan_cvt, inputs="cvt", tol=EXACT, atol=EXACT)
+
+
+def draw(rng, dt, shape, kind, j):
+    """Operand j of a test whose operation is of the given kind."""
+    bits = dt.itemsize * 8
+    if kind.startswith("cvt"):                # inside the range of every destination type of the conversion tests
+        lo, hi = (0, 100) if kind == "cvt_u" else (-100, 100)
+        if dt.kind == "f":
+            return rng.uniform(lo, hi, size=shape).astype(dt)
+        if kind == "cvt":
+            lo, hi = -10000, 10000
+        return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
+    if kind == "small":                       # few distinct values: equal pairs occur, products stay small
+        return rng.integers(-3 if dt.kind != "u" else 0, 3, size=shape, endpoint=True).astype(dt)
+    if dt.kind == "f":
+        if kind == "pos":
+            x = rng.uniform(0.5, 4.0, size=shape)
+        elif kind in ("rem", "rempos") and j == 1:
+            x = rng.integers(3, 100, size=shape).astype(np.float64)
+        elif kind in ("rem", "rempos"):
+            x = rng.integers(0 if kind == "rempos" else -1000, 1000, size=shape).astype(np.float64)
+        else:
+            x = rng.uniform(-4.0, 4.0, size=shape)
+        return x.astype(dt)
+    info = np.iinfo(dt)
+    if kind == "shift" and j == 1:
+        x = rng.integers(0, bits - 1, size=shape)
+    elif kind == "shift":
+        x = rng.integers(0, min(info.max, 1 << (bits - 2)) >> 3, size=shape)      # room to shift without sign trouble
+    elif kind in ("rem", "rempos") and j == 1:
+        x = rng.integers(3, 100, size=shape)
+    elif kind in ("rem", "rempos"):
+        x = rng.integers(0 if kind == "rempos" else max(info.min, -1000), min(info.max, 1000), size=shape)
+    elif kind == "bits":
+        x = rng.integers(info.min, info.max, size=shape, endpoint=True)
+    elif kind == "pos":
+        x = rng.integers(1, 100, size=shape)
+    else:
+        x = rng.integers(max(info.min, -100), min(info.max, 100), size=shape)
+    return x.astype(dt)
+
+
+def make_inputs(pl, seed):
+    """Input buffers (whole, with their leading dimensions), drawn for the test's kind of operation."""
+    rng = np.random.default_rng(seed)
+    return [draw(rng, dt, shape, pl.spec["inputs"] if len(entry) == 2 else entry[2], j)
+            for j, entry in enumerate(pl.ins) for dt, shape in [entry[:2]]]
+
+
+def expected(pl, ins):
+    """Per output, the valid region, in float64 for floating-point tiles (the caller rounds / compares)."""
+    return pl.expect(ins, pl.scalar[1] if pl.scalar else None)

@@ -103,18 +103,16 @@ def test_cmps_sel_vs_reference(oracle, ref, mode):
     assert np.array_equal(sel, oracle.tsel_packed(mask, 16, a, b))
 
 
-def test_tsel_running_bit_order(oracle):
-    """Bits run on across rows when the valid width is not a multiple of 8 (cpu/TSel.hpp:27-47)."""
+def test_tsel_mask_rows_when_width_is_not_a_multiple_of_8(oracle):
+    """Row i of the mask serves row i of the tiles; the unused high bits of its last byte are skipped
+    (npu/a2a3/TSel.hpp:46-57, tsel/gen_data.py:31-47: the NPU test with 54 valid columns)."""
     rng = np.random.default_rng(5)
     a, b = rng.standard_normal((6, 12)).astype(np.float32), rng.standard_normal((6, 12)).astype(np.float32)
-    flat = rng.integers(0, 2, size=72).astype(bool)
-    stream = np.packbits(flat, bitorder="little")                 # 9 bytes
-    mask = np.zeros((3, 32), dtype=np.uint8)
-    m2 = np.zeros(12, dtype=np.uint8)
-    m2[:9] = stream
-    mask[:, :4] = m2.reshape(3, 4)                                 # 4 valid mask columns per mask row
-    got = oracle.tsel_packed(mask, 4, a, b)
-    assert np.array_equal(got, np.where(flat.reshape(6, 12), a, b))
+    bits = rng.integers(0, 2, size=(6, 12)).astype(bool)
+    mask = np.full((6, 32), 0xFF, dtype=np.uint8)
+    mask[:, :2] = np.packbits(bits, axis=1, bitorder="little")
+    got = oracle.tsel_packed(mask, 2, a, b)
+    assert np.array_equal(got, np.where(bits, a, b))
 
 
 @pytest.mark.parametrize("pad_kind", [1, 2, 3])

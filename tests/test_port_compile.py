@@ -102,7 +102,7 @@ void Launch(float *out, void *stream)
     text, notes = mod.port(src, [("kSize", "128")], 4096, ("__DAV_VEC__",), None, True)
     assert "constexpr int kSize = 128;" in text
     assert "PTO_CORE_STATIC(int, calls, 0);" in text and "PTO_KERNEL_PROLOGUE();" in text
-    assert "<<<pto::host::LaunchBlocks(4, (hipStream_t)(stream)), pto::kBlockThreads, 4096, (hipStream_t)(stream)>>>" in text
+    assert "<<<pto::host::LaunchBlocks(4, (hipStream_t)(stream)), pto::kBlockThreads, pto::host::LaunchLds((const void *)(kern), 4096), (hipStream_t)(stream)>>>" in text
     assert "__global__ __launch_bounds__(pto::kBlockThreads) AICORE void kern" in text
     assert text.startswith("#define PTO_TILE_COPY_WRITEBACK 1\n#define PTO_VEC_TILES_IN_MEMORY 1\n#define __DAV_VEC__ 1\n")
     begin, end, launch = text.index("PTO_DEVICE_CODE_BEGIN"), text.index("PTO_DEVICE_CODE_END"), text.index("void Launch")
