@@ -9,6 +9,7 @@
 #include "pto/gfx950/vec_ops_ext.hpp"
 #include "pto/gfx950/fifo_ops.hpp"
 #include "pto/gfx950/sort_ops.hpp"
+#include "pto/gfx950/matmul_any.hpp"
 
 namespace pto {
 
@@ -85,6 +86,38 @@ PTO_FRONT(TMATMUL_ACC, typename C PTO_C typename A PTO_C typename B, C &cOut PTO
           (cOut, cIn, a, b))
 PTO_FRONT(TMATMUL_BIAS, typename C PTO_C typename A PTO_C typename B, C &c PTO_C A &a PTO_C B &b PTO_C BiasRow bias,
           (c, a, b, bias))
+// TMATMUL_BIAS with the bias in a [1, n] Bias tile, and the TGEMV forms: a matmul whose left operand has one valid row
+// (pto_instr.hpp:504-571 of the reference)
+template <typename C, typename A, typename B, typename Bias, typename... Ev,
+          std::enable_if_t<Bias::Loc == TileType::Bias, int> = 0>
+PTO_INST RecordEvent TMATMUL_BIAS(C &c, A &a, B &b, Bias &bias, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_BIAS_IMPL(c, a, b, bias);
+    return {};
+}
+template <typename C, typename A, typename B, typename... Ev>
+PTO_INST RecordEvent TGEMV(C &c, A &a, B &b, Ev &... ev)
+{
+    TSYNC(ev...);
+    TGEMV_IMPL(c, a, b);
+    return {};
+}
+template <typename C, typename A, typename B, typename... Ev>
+PTO_INST RecordEvent TGEMV_ACC(C &cOut, C &cIn, A &a, B &b, Ev &... ev)
+{
+    TSYNC(ev...);
+    TGEMV_ACC_IMPL(cOut, cIn, a, b);
+    return {};
+}
+template <typename C, typename A, typename B, typename Bias, typename... Ev,
+          std::enable_if_t<Bias::Loc == TileType::Bias, int> = 0>
+PTO_INST RecordEvent TGEMV_BIAS(C &c, A &a, B &b, Bias &bias, Ev &... ev)
+{
+    TSYNC(ev...);
+    TGEMV_BIAS_IMPL(c, a, b, bias);
+    return {};
+}
 PTO_FRONT(TCVT, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C RoundMode mode, (dst, src, mode))
 PTO_FRONT(TGATHER, typename D PTO_C typename S0 PTO_C typename I, D &dst PTO_C S0 &src0 PTO_C I &idx, (dst, src0, idx))
 PTO_FRONT(MGATHER, typename D PTO_C typename G PTO_C typename I, D &dst PTO_C G &src PTO_C I &idx, (dst, src, idx))

@@ -205,41 +205,70 @@ struct TileStorage<TileType::ScaleRight, T, Rows, Cols> {
 };
 
 template <typename T, int Rows, int Cols>
-struct TileStorage<TileType::Left, T, Rows, Cols> {
-    static_assert(is_mfma_operand_v<T>, "Left tiles: fp16, bf16, int8 or fp32 operands (fp8 / fp4 for TMATMUL_MX)");
-    static_assert(Rows % (kMfmaM * kWavesM) == 0, "Left tile rows must be a multiple of PTO_MFMA_M x PTO_WAVES_M");
-    static_assert(Cols % kFragK<T> == 0, "Left tile cols (K) must be a multiple of the k extent of a fragment");
+struct TileStorage<TileType::Vec, T, Rows, Cols> {
+    static constexpr int Chunks = cdiv(Rows * Cols, kVecChunk);
+    static constexpr int Slots = cdiv(Chunks, kBlockThreads);
+    T v[Slots][kVecChunk];
+};
+
+// Left / Right / Acc tiles whose extents are whole MFMA blocks per wave are fragments (below).  Any other extent (the
+// reference's own matmul tests use 48 x 64, 16 x 16, 32 x 128 ... tiles with run-time or static valid regions inside:
+// tests/cpu/st/testcase/tmatmul/tmatmul_kernel.cpp:28-45) gets the element distribution of a Vec tile, and the
+// instructions on such a tile take the general path of pto/gfx950/matmul_any.hpp: correct for every shape, far from the
+// speed of the fragment path.  Bias tiles always have it.
+template <typename T, int Rows, int Cols>
+struct PlainStorage : TileStorage<TileType::Vec, T, Rows, Cols> {
+    static constexpr bool kPlain = true;
+};
+template <typename S, typename = void>
+struct is_plain_storage : std::false_type {};
+template <typename S>
+struct is_plain_storage<S, std::void_t<decltype(S::kPlain)>> : std::true_type {};
+
+template <typename T, int Rows, int Cols>
+constexpr bool kLeftFragShaped = is_mfma_operand_v<T> && Rows % (kMfmaM * kWavesM) == 0 && Cols % kFragK<T> == 0;
+template <typename T, int Rows, int Cols>
+constexpr bool kRightFragShaped = is_mfma_operand_v<T> && Cols % (kMfmaM * kWavesN) == 0 && Rows % kFragK<T> == 0;
+template <typename T, int Rows, int Cols>
+constexpr bool kAccFragShaped = (std::is_same_v<T, float> || std::is_same_v<T, int32_t>) && Rows % (kMfmaM * kWavesM) == 0 &&
+                                Cols % (kMfmaM * kWavesN) == 0;
+
+template <typename T, int Rows, int Cols>
+struct LeftFragStorage {
     static constexpr int MB = Rows / (kMfmaM * kWavesM);
     static constexpr int KS = Cols / kFragK<T>;
     typename FragOf<T>::type f[MB][KS];
 };
-
 template <typename T, int Rows, int Cols>
-struct TileStorage<TileType::Right, T, Rows, Cols> {
-    static_assert(is_mfma_operand_v<T>, "Right tiles: fp16, bf16, int8 or fp32 operands (fp8 / fp4 for TMATMUL_MX)");
-    static_assert(Cols % (kMfmaM * kWavesN) == 0, "Right tile cols must be a multiple of PTO_MFMA_M x PTO_WAVES_N");
-    static_assert(Rows % kFragK<T> == 0, "Right tile rows (K) must be a multiple of the k extent of a fragment");
+struct RightFragStorage {
     static constexpr int NB = Cols / (kMfmaM * kWavesN);
     static constexpr int KS = Rows / kFragK<T>;
     typename FragOf<T>::type f[NB][KS];
 };
-
 template <typename T, int Rows, int Cols>
-struct TileStorage<TileType::Acc, T, Rows, Cols> {
-    static_assert(std::is_same_v<T, float> || std::is_same_v<T, int32_t>, "Acc tiles: fp32 or int32 accumulators");
-    static_assert(Rows % (kMfmaM * kWavesM) == 0 && Cols % (kMfmaM * kWavesN) == 0,
-                  "Acc tile must be a multiple of (PTO_MFMA_M x PTO_WAVES_M) x (PTO_MFMA_M x PTO_WAVES_N)");
+struct AccFragStorage {
     static constexpr int MB = Rows / (kMfmaM * kWavesM);
     static constexpr int NB = Cols / (kMfmaM * kWavesN);
     typename AccFragOf<T>::type f[MB][NB];
 };
 
 template <typename T, int Rows, int Cols>
-struct TileStorage<TileType::Vec, T, Rows, Cols> {
-    static constexpr int Chunks = cdiv(Rows * Cols, kVecChunk);
-    static constexpr int Slots = cdiv(Chunks, kBlockThreads);
-    T v[Slots][kVecChunk];
+struct TileStorage<TileType::Left, T, Rows, Cols>
+    : std::conditional_t<kLeftFragShaped<T, Rows, Cols>, LeftFragStorage<T, Rows, Cols>, PlainStorage<T, Rows, Cols>> {
+    static_assert(std::is_arithmetic_v<T> || is_mfma_operand_v<T>, "Left tiles: fp16, bf16, int8 or fp32 operands (fp8 / fp4 for TMATMUL_MX)");
 };
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Right, T, Rows, Cols>
+    : std::conditional_t<kRightFragShaped<T, Rows, Cols>, RightFragStorage<T, Rows, Cols>, PlainStorage<T, Rows, Cols>> {
+    static_assert(std::is_arithmetic_v<T> || is_mfma_operand_v<T>, "Right tiles: fp16, bf16, int8 or fp32 operands (fp8 / fp4 for TMATMUL_MX)");
+};
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Acc, T, Rows, Cols>
+    : std::conditional_t<kAccFragShaped<T, Rows, Cols>, AccFragStorage<T, Rows, Cols>, PlainStorage<T, Rows, Cols>> {
+    static_assert(std::is_same_v<T, float> || std::is_same_v<T, int32_t>, "Acc tiles: fp32 or int32 accumulators");
+};
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Bias, T, Rows, Cols> : PlainStorage<T, Rows, Cols> {};
 
 } // namespace detail
 
@@ -336,6 +365,15 @@ struct Tile {
 
     PTO_HD constexpr int GetValidRow() const { return ValidRow == DYNAMIC ? RowMaskInternal : ValidRow; }
     PTO_HD constexpr int GetValidCol() const { return ValidCol == DYNAMIC ? ColMaskInternal : ValidCol; }
+
+    // Ascend machine state that kernel sources set through a Left tile (pto_tile.hpp:1373-1401 of the reference).  TF32
+    // mode makes the cube unit round fp32 operands to 11 (a2 / a3) or 10 mantissa bits before it multiplies; the fp32
+    // MFMAs multiply fp32 operands exactly, which lies inside the TF32 product's own rounding error, so the mode has
+    // nothing to switch.  The k-alignment flag is a layout hint of the a3 cube unit.
+    PTO_HD void SetMadTF32Mode(RoundMode = RoundMode::CAST_ROUND) {}
+    PTO_HD void ResetMadMode() {}
+    PTO_HD bool GetKAligned() const { return true; }
+    PTO_HD void SetKAligned(bool) {}
 
     // Mat tiles: pointer to the LDS image (swizzled, see mem_ops.hpp).  Register tiles: their fragments.
     PTO_DEV auto data()

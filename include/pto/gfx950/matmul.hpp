@@ -14,6 +14,27 @@
 namespace pto {
 namespace detail {
 
+// The general path for tiles that are not whole MFMA blocks per wave (pto/gfx950/matmul_any.hpp, defined after the
+// memory and vector instructions it builds on).
+template <typename TileT>
+constexpr bool is_plain_v = is_plain_storage<typename TileT::Storage>::value;
+template <typename TileT>
+constexpr bool is_fully_valid_v = TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols;
+template <bool kZeroInit, typename AccT, typename LeftT, typename RightT>
+PTO_DEV void mad_any(AccT &out, AccT &in, LeftT &a, RightT &b);
+template <typename AccT, typename BiasT>
+PTO_DEV void add_bias_any(AccT &c, BiasT &bias);
+template <typename DstT, typename SrcT>
+PTO_DEV void textract_any(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCol);
+template <typename TileT, typename G>
+PTO_DEV void tload_any(TileT &dst, G &src);
+template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu>
+PTO_DEV void tstore_any(G &dst, TileT &src);
+template <typename TileT>
+PTO_DEV void zero_outside_valid(TileT &t);
+template <typename DstT, typename SrcT>
+PTO_DEV void tfillpad_mat(DstT &dst, SrcT &src);
+
 // (the accumulator type is a template parameter only so that the branch for the other MFMA shape is discarded
 // instead of type-checked)
 template <typename C>
@@ -71,7 +92,7 @@ PTO_DEV C mfma32(f32x4 a, f32x4 b, C c)
 }
 
 template <typename AccT, typename LeftT, typename RightT>
-PTO_DEV constexpr void check_mad()
+PTO_DEV constexpr void check_mad_types()
 {
     using A = typename LeftT::DType;
     using B = typename RightT::DType;
@@ -82,11 +103,18 @@ PTO_DEV constexpr void check_mad()
                   "[PTO][SA] TMATMUL on gfx950: fp16 / bf16 / fp32 operands -> fp32, or int8 x int8 -> int32");
     static_assert(LeftT::Loc == TileType::Left && RightT::Loc == TileType::Right && AccT::Loc == TileType::Acc,
                   "[PTO][SA] TMATMUL: operands must be Left, Right and Acc tiles");
+}
+template <typename AccT, typename LeftT, typename RightT>
+PTO_DEV constexpr void check_mad()
+{
+    check_mad_types<AccT, LeftT, RightT>();
     static_assert(LeftT::Rows == AccT::Rows && LeftT::Cols == RightT::Rows && RightT::Cols == AccT::Cols,
                   "[PTO][SA] TMATMUL: inconsistent m, k, n");
-    static_assert(LeftT::ValidRow == LeftT::Rows && LeftT::ValidCol == LeftT::Cols && RightT::ValidCol == RightT::Cols,
-                  "[PTO][SA] TMATMUL on gfx950: operands must be fully valid (pad the tile instead)");
 }
+// operands with a valid region inside the tile were zeroed outside it when they were extracted: the fragment path
+// multiplies whole tiles
+template <typename AccT, typename LeftT, typename RightT>
+constexpr bool any_plain_v = is_plain_v<AccT> || is_plain_v<LeftT> || is_plain_v<RightT>;
 
 template <bool kZeroInit, typename AccT, typename LeftT, typename RightT>
 PTO_DEV void mad(AccT &out, const AccT &in, const LeftT &a, const RightT &b)
@@ -119,14 +147,20 @@ template <typename AccT, typename LeftT, typename RightT>
 PTO_DEV void TMATMUL_IMPL(AccT &c, LeftT &a, RightT &b)
 {
     detail::check_mad<AccT, LeftT, RightT>();
-    detail::mad<true>(c, c, a, b);
+    if constexpr (detail::any_plain_v<AccT, LeftT, RightT>)
+        detail::mad_any<true>(c, c, a, b);
+    else
+        detail::mad<true>(c, c, a, b);
 }
 
 template <typename AccT, typename LeftT, typename RightT>
 PTO_DEV void TMATMUL_ACC_IMPL(AccT &cOut, AccT &cIn, LeftT &a, RightT &b)
 {
     detail::check_mad<AccT, LeftT, RightT>();
-    detail::mad<false>(cOut, cIn, a, b);
+    if constexpr (detail::any_plain_v<AccT, LeftT, RightT>)
+        detail::mad_any<false>(cOut, cIn, a, b);
+    else
+        detail::mad<false>(cOut, cIn, a, b);
 }
 
 // TMATMUL_MX: C (+)= (A * scaleA) x (B * scaleB) on 8-bit MX operands, one e8m0 scale per row (column) and 32-wide
@@ -202,10 +236,19 @@ struct BiasRow {
     const float *row;
 };
 
+// the reference's form: the bias is a [1, n] Bias tile (pto_instr.hpp:504-511 of the reference, cpu/TMatmul.hpp:109-115)
+template <typename AccT, typename LeftT, typename RightT, typename BiasT>
+PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasT &bias)
+{
+    TMATMUL_IMPL(c, a, b);
+    detail::add_bias_any(c, bias);
+}
+
 template <typename AccT, typename LeftT, typename RightT>
 PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasRow bias)
 {
     detail::check_mad<AccT, LeftT, RightT>();
+    static_assert(!detail::any_plain_v<AccT, LeftT, RightT>, "[PTO][SA] TMATMUL_BIAS with a bias row in memory: fragment tiles (pass a Bias tile otherwise)");
     detail::mad<true>(c, c, a, b);
     using SA = typename AccT::Storage;
     const int col0 = hw::wave_n() * (SA::NB * detail::kMfmaM) + detail::acc_lane_col((uint32_t)hw::lane());

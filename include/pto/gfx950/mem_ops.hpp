@@ -197,7 +197,8 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
         constexpr int cpr = Geo::ChunksPerRow;
         // rows that one wave instruction covers, when a row is at most one instruction long
         constexpr int rpi = (cpr <= kWaveSize && kWaveSize % cpr == 0) ? kWaveSize / cpr : 0;
-        if constexpr (rpi > 0 && (rpi * kBlockWaves) % 16 == 0 && total % perWaveInst == 0 && (nInst % kBlockWaves == 0 || SLICE < 0)) {
+        if constexpr (rpi > 0 && (rpi * kBlockWaves) % 16 == 0 && total % perWaveInst == 0 && (nInst % kBlockWaves == 0 || SLICE < 0) &&
+                      (nInst % kBlockWaves == 0 || nInst > kBlockWaves)) {
             // The swizzle repeats every 16 rows and the instructions of one wave are a multiple of 16
             // rows apart: every instruction of this wave uses the same per-lane byte offset (32 bits: a
             // tile spans less than 4 GiB of memory) on top of a wave-uniform base, which the loop
@@ -208,7 +209,6 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             const char *base = reinterpret_cast<const char *>(gm);
             constexpr int first = SLICE < 0 ? 0 : SLICE * kBlockWaves, last = SLICE < 0 ? nInst : first + kBlockWaves;
             static_assert(last <= nInst, "[PTO][SA] TLOAD slice: the tile has fewer copy instructions");
-            static_assert(nInst % kBlockWaves == 0 || nInst > kBlockWaves, "[PTO][SA] TLOAD: fewer copy instructions than waves");
 #pragma unroll
             for (int s0 = first; s0 < last; s0 += kBlockWaves) {
                 // When the last round of instructions is not full, the waves past its end repeat their instruction
@@ -426,6 +426,8 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
         detail::tload_vec(dst, src);
     else if constexpr (TileT::Loc == TileType::ScaleLeft || TileT::Loc == TileType::ScaleRight)
         detail::tload_scale(dst, src);
+    else if constexpr (TileT::Loc == TileType::Bias)
+        detail::tload_any(dst, src);
     else
         static_assert(TileT::Loc == TileType::Mat, "[PTO][SA] TLOAD: destination must be a Mat or Vec tile");
 }
@@ -543,17 +545,16 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
         } else {
             // the source is contiguous along its rows (an A operand stored transposed): element-wise gather, the slow path
             // that keeps every layout pair of the reference's TEXTRACT legal (a2a3/TExtract.hpp:537-548)
-            static_assert(sizeof(ElemT) == 2, "[PTO][SA] TEXTRACT across the contiguous dimension: 16-bit elements");
 #pragma unroll
             for (int mb = 0; mb < S::MB; ++mb)
 #pragma unroll
                 for (int ks = 0; ks < S::KS; ++ks) {
-                    Frag f;
+                    ElemT tmp[kChunkElems];
 #pragma unroll
                     for (uint32_t j = 0; j < kChunkElems; ++j)
-                        f[j] = *reinterpret_cast<const ElemT *>(
+                        tmp[j] = *reinterpret_cast<const ElemT *>(
                             lds + Geo::elem_off(row0 + mb * detail::kMfmaM, idxCol + (khalf + ks * kStepChunks) * kChunkElems + j));
-                    dst.S().f[mb][ks] = f;
+                    __builtin_memcpy(&dst.S().f[mb][ks], tmp, 16);
                 }
         }
     } else if constexpr (DstT::Loc == TileType::Right) {
@@ -570,17 +571,16 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
         } else {
             // the source is contiguous along its columns (a B operand [k, n] stored row-major, the V tile of the
             // reference's attention kernel: fa_performance_kernel.cpp:676-677): element-wise gather, the slow path
-            static_assert(sizeof(ElemT) == 2, "[PTO][SA] TEXTRACT across the contiguous dimension: 16-bit elements");
 #pragma unroll
             for (int nb = 0; nb < S::NB; ++nb)
 #pragma unroll
                 for (int ks = 0; ks < S::KS; ++ks) {
-                    Frag f;
+                    ElemT tmp[kChunkElems];
 #pragma unroll
                     for (uint32_t j = 0; j < kChunkElems; ++j)
-                        f[j] = *reinterpret_cast<const ElemT *>(
+                        tmp[j] = *reinterpret_cast<const ElemT *>(
                             lds + Geo::elem_off(idxRow + (khalf + ks * kStepChunks) * kChunkElems + j, col0 + nb * detail::kMfmaM));
-                    dst.S().f[nb][ks] = f;
+                    __builtin_memcpy(&dst.S().f[nb][ks], tmp, 16);
                 }
         }
     } else {
@@ -605,8 +605,12 @@ PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t i
                       "[PTO][SA] TEXTRACT: Mat source of the same element type");
         detail::textract_mx(dst, src, idxRow, idxCol);
         return;
+    } else if constexpr (detail::is_plain_v<DstT>) {
+        detail::textract_any(dst, src, idxRow, idxCol);
     } else {
         textract_frag(dst, src, idxRow, idxCol);
+        if constexpr (!detail::is_fully_valid_v<DstT>)
+            detail::zero_outside_valid(dst); // TMATMUL multiplies whole fragments
     }
 }
 
@@ -618,6 +622,8 @@ PTO_DEV void TMOV_IMPL(DstT &dst, SrcT &src)
 {
     if constexpr (SrcT::Loc == TileType::Mat && (DstT::Loc == TileType::Left || DstT::Loc == TileType::Right)) {
         TEXTRACT_IMPL(dst, src, 0, 0);
+    } else if constexpr (SrcT::Loc == TileType::Mat && DstT::Loc == TileType::Bias) {
+        detail::textract_any(dst, src, 0, 0); // L1 -> bias table (npu/a2a3/TMov.hpp: the Mat -> Bias pair)
     } else if constexpr (SrcT::Loc == DstT::Loc && SrcT::Rows == DstT::Rows && SrcT::Cols == DstT::Cols &&
                          std::is_same_v<typename SrcT::DType, typename DstT::DType> && SrcT::Loc != TileType::Mat) {
         dst.st = src.st;
@@ -747,7 +753,9 @@ template <typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone
 PTO_DEV void TSTORE_IMPL(G &dst, TileT &src)
 {
     static_assert(relu == ReluPreMode::NoRelu || TileT::Loc == TileType::Acc, "[PTO][SA] TSTORE: ReLU applies to Acc tiles");
-    if constexpr (TileT::Loc == TileType::Acc) {
+    if constexpr (TileT::Loc == TileType::Acc && detail::is_plain_v<TileT>) {
+        detail::tstore_any<TileT, G, atomic, relu>(dst, src);
+    } else if constexpr (TileT::Loc == TileType::Acc) {
         detail::tstore_acc<TileT, G, atomic, relu>(dst, src);
     } else if constexpr (TileT::Loc == TileType::Vec) {
         static_assert(sizeof(typename TileT::DType) == sizeof(typename G::DType), "[PTO][SA] TSTORE: element sizes differ");

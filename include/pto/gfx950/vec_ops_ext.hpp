@@ -226,16 +226,20 @@ PTO_DEV void TFILLPAD_IMPL(DstT &dst, SrcT &src)
 {
     static_assert(DstT::Rows == SrcT::Rows && DstT::Cols == SrcT::Cols && sizeof(typename DstT::DType) == sizeof(typename SrcT::DType),
                   "[PTO][SA] TFILLPAD: same shape and element size");
-    static_assert(DstT::PadVal != PadValue::Null, "[PTO][SA] TFILLPAD: the destination tile needs a pad value");
-    using T = typename DstT::DType;
-    const T pad = detail::pad_value<T>(DstT::PadVal);
-    const int vr = src.GetValidRow(), vc = src.GetValidCol();
-    detail::for_each_owned<DstT>([&](int s, int i, int e) {
-        int r, c;
-        detail::elem_rc<DstT>(e, r, c);
-        if (e < DstT::Numel)
-            dst.S().v[s][i] = (r < vr && c < vc) ? __builtin_bit_cast(T, src.S().v[s][i]) : pad;
-    });
+    if constexpr (DstT::Loc == TileType::Mat) {
+        detail::tfillpad_mat(dst, src); // an L1 tile cleared outside a ragged load (pad value Null: zero)
+    } else {
+        static_assert(DstT::PadVal != PadValue::Null, "[PTO][SA] TFILLPAD: the destination tile needs a pad value");
+        using T = typename DstT::DType;
+        const T pad = detail::pad_value<T>(DstT::PadVal);
+        const int vr = src.GetValidRow(), vc = src.GetValidCol();
+        detail::for_each_owned<DstT>([&](int s, int i, int e) {
+            int r, c;
+            detail::elem_rc<DstT>(e, r, c);
+            if (e < DstT::Numel)
+                dst.S().v[s][i] = (r < vr && c < vc) ? __builtin_bit_cast(T, src.S().v[s][i]) : pad;
+        });
+    }
 }
 
 // ------------------------------------------------------- column reductions

@@ -73,6 +73,14 @@ int pto_st_textract_windows_f16(void *stream, float *out_left, float *out_right,
 int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, const float *bias,
                                   int bf16);
 
+/* Matmul instructions on ragged tiles: [m, k] x [k, n] (both row-major in memory) with valid m, k, n inside tiles rounded
+ * up to 16 rows and 32 bytes, through TLOAD -> TFILLPAD -> TMOV / TEXTRACT -> TMATMUL / TMATMUL_ACC / TMATMUL_BIAS / TGEMV ->
+ * TSTORE, as tests/cpu/st/testcase/tmatmul/tmatmul_kernel.cpp:26-97 and tests/npu/a2a3/src/st/testcase/tmatmul/
+ * tmatmul_kernel.cpp:113-197 of the reference build them.  case_id selects element types, extents and form (the table in
+ * tests/matmul_any_cases.py); the bias forms store twice the result (once through a Bias tile loaded by TMOV from L1, once
+ * through one loaded by TLOAD, added together). */
+int pto_st_matmul_ragged(void *stream, void *out, const void *a, const void *b, const void *bias, int case_id);
+
 /* [128,128] x [128,256] int8 -> int32 and [128,32] x [32,256] fp32 -> fp32 (the other operand types of TMATMUL,
  * include/pto/cpu/TMatmul.hpp:46-51; tests/cpu/st/testcase/tmatmul/gen_data.py:92-99): a row-major, b_t = b stored
  * [256][K] (column-major b); K in two halves, TMATMUL then TMATMUL_ACC.  relu != 0: stored with

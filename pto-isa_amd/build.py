@@ -18,7 +18,7 @@ OUT = os.path.join(HERE, "libpto_amd.so")
 # the parity tests load to drive single instructions and kernel variants.  Not part of the product.
 OUT_ST = os.path.join(HERE, "libpto_st.so")
 SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_k64.hip", "pto_gemm_mx.hip", "pto_elementwise.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_fa_w8m16.hip"]
-ST_ONLY_SOURCES = ["pto_optest.hip"]
+ST_ONLY_SOURCES = ["pto_optest.hip", "pto_optest_matmul.hip"]
 # sources of libpto_st.so that differ from the product's objects (they hold a hook); the others are linked as they are
 HOOK_SOURCES = ["pto_gemm.hip", "pto_gemm_w8.hip", "pto_gemm_m16.hip", "pto_gemm_m16w4.hip", "pto_gemm_k64.hip", "pto_gemm_mx.hip", "pto_fa.hip"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -98,7 +98,7 @@ PORTED = [
 ]
 
 
-def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includes=(), defines=(), vec_in_memory=False):
+def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includes=(), defines=(), vec_in_memory=False, l1_map=None):
     """Runs a kernel source of the reference through port_ascend_source.py into a temporary directory and compiles the
     result against include/pto with hipcc; `out` ends in .o (compile only) or .so.  The ported text never enters the
     repository tree."""
@@ -109,7 +109,7 @@ def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includ
     spec.loader.exec_module(mod)
     src = os.path.join(REFERENCE, rel_src)
     with open(src) as f:
-        text, _ = mod.port(f.read(), sets, lds_bytes, defines, os.path.dirname(src), vec_in_memory)
+        text, _ = mod.port(f.read(), sets, lds_bytes, defines, os.path.dirname(src), vec_in_memory, l1_map)
     with tempfile.TemporaryDirectory() as tmp:
         hip = os.path.join(tmp, os.path.basename(rel_src).replace(".cpp", ".hip"))
         with open(hip, "w") as f:
@@ -147,16 +147,29 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolsum", "tcolmax", "tcolmin", "tcolprod", "trowexpand",
               "trowexpandadd", "trowexpandsub", "trowexpandmul", "trowexpanddiv", "trowexpandmax", "trowexpandmin", "trowexpandexpdif",
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
-              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt"]
+              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
+_ST_KEYED = re.compile(r"tilingKey\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<")
+_ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
+# options of the port script per test kernel: L1 addresses written for Ascend's 512 KiB moved inside the LDS
+ST_PORT_OPTIONS = {
+    "tmatmul": dict(l1_map={0x20000: 0x10000, 0x40000: 0x1C000}),
+}
 
 
 def st_case_table(source_text):
-    """{case number: {"run": run function, "targs": [template arguments], "params": kernel parameter list}}"""
+    """{case: {"run": run function, "targs": [template arguments], "params": kernel parameter list}} for the two ways the
+    test sources number their cases: `launch<OP>Case<N>` kernels (case = "N"), and launchers that switch on their template
+    argument, `if constexpr (tilingKey == N) { run<...><<<` (case = "<launcher>:N")."""
     table = {}
     for m in _ST_CASE.finditer(source_text):
         table[m.group(1)] = {"run": m.group(3), "targs": [a.strip() for a in m.group(4).split(",")],
                              "params": " ".join(m.group(2).replace("__gm__", "").split())}
+    launchers = [(m.start(), m.group(1)) for m in _ST_LAUNCHER.finditer(source_text)]
+    for m in _ST_KEYED.finditer(source_text):
+        owner = [name for pos, name in launchers if pos < m.start()]
+        if owner:
+            table["%s:%s" % (owner[-1], m.group(1))] = {"run": m.group(2), "targs": [a.strip() for a in m.group(3).split(",")], "params": ""}
     return table
 
 
@@ -173,7 +186,7 @@ def build_ported_st(verbose=True, jobs=8):
     def one(name):
         rel = "tests/npu/a2a3/src/st/testcase/%s/%s_kernel.cpp" % (name, name)
         lib = os.path.join(out_dir, name + ".so")
-        rc, err = port_and_compile(rel, [], 160 * 1024, lib, extra_flags=("-Wno-unknown-attributes",))
+        rc, err = port_and_compile(rel, [], 160 * 1024, lib, extra_flags=("-Wno-unknown-attributes",), **ST_PORT_OPTIONS.get(name, {}))
         if rc != 0:
             raise RuntimeError("ported build failed for %s:\n%s" % (rel, err))
         syms = subprocess.run(["nm", "-D", "--defined-only", lib], capture_output=True, text=True, check=True).stdout.split("\n")

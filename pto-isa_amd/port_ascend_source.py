@@ -2,7 +2,7 @@
 """Mechanical edits that turn a PTO kernel source written for the Ascend toolchain into a gfx950 translation unit.
 
     python pto-isa_amd/port_ascend_source.py IN.cpp OUT.hip [--set NAME=VALUE ...] [--define NAME[=VALUE] ...]
-                                             [--lds BYTES] [--vec-in-memory] [--no-inline]
+                                             [--lds BYTES] [--vec-in-memory] [--no-inline] [--l1 OLD=NEW ...]
 
 What a kernel source of the reference needs before `hipcc --offload-arch=gfx950 -I include` accepts it, and what this
 script therefore does (nothing else is touched; the tile code itself compiles as it is):
@@ -29,6 +29,9 @@ script therefore does (nothing else is touched; the tile code itself compiles as
    include/pto/common/tile.hpp) and makes every launch prepare that buffer (`pto::host::LaunchBlocks`).
 10. A source that names the Ascend compiler's built-in variables `block_idx` / `block_num` gets them as macros over
     `get_block_idx()` / `get_block_num()`, defined after the library's headers.
+11. `--l1 OLD=NEW` rewrites the literal address of `TASSIGN(tile, OLD)`: sources place their L1 tiles at addresses laid
+    out for Ascend's 512 KiB (0x20000, 0x40000 ...), which have to move inside the 160 KiB of LDS.  Register tiles ignore
+    their address, so rewriting theirs too changes nothing.
 """
 import argparse
 import os
@@ -91,7 +94,10 @@ def kernel_before(text, pos):
     return " ".join(text[start:end].split())
 
 
-def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in_memory=False):
+TASSIGN_LITERAL = re.compile(r"(TASSIGN\(\s*\w+\s*,\s*)(0[xX][0-9a-fA-F]+|\d+)(\s*\))")
+
+
+def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in_memory=False, l1_map=None):
     notes = []
     if directory is not None:
         before = text
@@ -103,6 +109,20 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
         if n == 0:
             raise SystemExit("port_ascend_source: no `constexpr ... %s = ...;` in the source" % name)
         notes.append("set %s = %s (%d place%s)" % (name, value, n, "" if n == 1 else "s"))
+
+    # 11. L1 addresses
+    if l1_map:
+        table = {int(str(k), 0): int(str(v), 0) for k, v in dict(l1_map).items()}
+        hits = [0]
+
+        def move(m):
+            a = int(m.group(2), 0)
+            if a not in table:
+                return m.group(0)
+            hits[0] += 1
+            return "%s0x%x%s" % (m.group(1), table[a], m.group(3))
+        text = TASSIGN_LITERAL.sub(move, text)
+        notes.append("%d TASSIGN address%s moved" % (hits[0], "" if hits[0] == 1 else "es"))
 
     # 2. launch statements
     blocks = "pto::host::LaunchBlocks(%s, (hipStream_t)(%s))" if vec_in_memory else "%s"
@@ -233,12 +253,13 @@ def main():
     ap.add_argument("--lds", type=int, default=160 * 1024)
     ap.add_argument("--vec-in-memory", action="store_true")
     ap.add_argument("--no-inline", action="store_true", help="leave `#include \"...\"` of files next to the source alone")
+    ap.add_argument("--l1", action="append", default=[], metavar="OLD=NEW", help="move the literal address of TASSIGN(tile, OLD)")
     args = ap.parse_args()
     sets = [tuple(s.split("=", 1)) for s in args.set]
     with open(args.src) as f:
         text = f.read()
     out, notes = port(text, sets, args.lds, args.define, None if args.no_inline else os.path.dirname(os.path.abspath(args.src)),
-                      args.vec_in_memory)
+                      args.vec_in_memory, dict(x.split("=", 1) for x in args.l1))
     with open(args.dst, "w") as f:
         f.write(out)
     for n in notes:

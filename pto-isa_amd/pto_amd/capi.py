@@ -50,6 +50,7 @@ ST_SYMBOLS = {
     "pto_st_tload_5d_f32": (C.c_int, [C.c_void_p] * 4),
     "pto_st_textract_windows_f16": (C.c_int, [C.c_void_p] * 7 + [C.c_int] * 2),
     "pto_st_matmul_bias_128x64x256": (C.c_int, [C.c_void_p] * 5 + [C.c_int]),
+    "pto_st_matmul_ragged": (C.c_int, [C.c_void_p] * 5 + [C.c_int]),
     "pto_st_matmul_s8_128x128x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_f32_128x32x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_mx_128x256x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 3),

@@ -135,7 +135,7 @@ def cases():
     man = manifest()
     for test, spec in SPECS.items():
         pat = _pattern(spec)
-        for mangled, demangled in sorted(man.get(test, {}).get("launchers", {}).items(), key=lambda kv: kv[1]):
+        for mangled, demangled in sorted(man.get(spec.get("lib", test), {}).get("launchers", {}).items(), key=lambda kv: kv[1]):
             if pat.match(demangled):
                 out.append((test, mangled, demangled))
     return out
@@ -193,7 +193,7 @@ def _elementwise_plan(spec, dtype, buffers, valid, scalar, scalar_first=False):
             return [op(k, a) if scalar_first else op(a, k)]
         return [op(a) if len(ins) == 1 else op(a, ins[1][:vr, :vc])]
     return SimpleNamespace(dtype=dtype, outs=[(dtype, buffers[0])], ins=[(dtype, b) for b in buffers[1:]], regions=[valid],
-                           scalar=scalar, expect=expect, spec=spec)
+                           scalar=scalar, expect=expect, spec=spec, compare=None)
 
 
 # ---- numbered cases: launch<OP>TestCase<N>(void *out, void *src, float scalar, stream) -> run<T, dstRows, dstCols, rows,
@@ -245,7 +245,7 @@ def TAIL(ints, nptr, suffix="", ptr0=None):
 
 def _plan(spec, outs, ins, regions, expect, scalar=None):
     return SimpleNamespace(dtype=ins[0][0] if ins else outs[0][0], outs=outs, ins=ins, regions=regions, scalar=scalar,
-                           expect=lambda arrays, k: expect(arrays), spec=spec)
+                           expect=lambda arrays, k: expect(arrays), spec=spec, compare=None)
 
 
 # ---- column reductions: launchTCOLSUM<T, cols, srcRows, validRows[, binary]>: [validRows, cols] of a [srcRows, cols] buffer
@@ -418,6 +418,57 @@ SPECS["tcvt"] = dict(fn="launchTCVT", tail=r"<(?P<D>[a-z ]+), (?P<T>[a-z ]+), (?
                      planner=plan_cvt, inputs="cvt", tol=EXACT, atol=EXACT)
 
 
+# ---- matmul: LaunchTMATMUL<N>(uint8 *out, uint8 *src0, uint8 *src1, stream) and LaunchTMATMULBIAS<N>(out, src0, src1, src2,
+# stream) -> Run...<OutT, AT, BT, BiasT, m, k, n, bias | round mode>: [m, k] x [k, n] (+ bias[n]), every matrix dense and
+# row-major in memory (tmatmul_kernel.cpp:113-197 and the split-k, GEMV and TF32 variants after it; :547-613 the cases)
+def _bf16_bits(x):
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+def _bf16_value(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def plan_matmul(test, spec, m):
+    e = manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]
+    t = e["targs"]
+    names = {"half": np.float16, "float": np.float32, "int8_t": np.int8, "int32_t": np.int32, "bfloat16_t": np.uint16}
+    out_dt, a_dt, bias_dt = np.dtype(names[t[0]]), np.dtype(names[t[1]]), np.dtype(names[t[3]])
+    vm, vk, vn = (int(x) for x in t[4:7])
+    bf16 = t[1] == "bfloat16_t"
+    kind = "bf16" if bf16 else ("bits" if a_dt.kind == "i" else "unit")
+    ins = [(a_dt, (vm, vk), kind), (a_dt, (vk, vn), kind)]
+    if spec["bias"]:
+        ins.append((bias_dt, (1, vn), "any" if bias_dt.kind == "i" else "unit"))
+
+    def values(arrays):
+        conv = (lambda x: _bf16_value(x).astype(np.float64)) if bf16 else (lambda x: x.astype(np.int64 if a_dt.kind == "i" else np.float64))
+        return conv(arrays[0]), conv(arrays[1])
+
+    def expect(arrays):
+        a, b = values(arrays)
+        c = a @ b
+        if spec["bias"]:
+            c = c + arrays[2].astype(c.dtype)
+        return [c]
+    pl = _plan(spec, [(out_dt, (vm, vn))], ins, [(vm, vn)], expect)
+    # an fp32 accumulation over k against the exact product: relative to the magnitude of the row-by-column sum
+    pl.compare = None if out_dt.kind == "i" else (
+        lambda got, want, arrays: np.max(np.abs(got.astype(np.float64) - want) / (np.abs(values(arrays)[0]) @ np.abs(values(arrays)[1]) + 1.0)) < 2e-3)
+    return pl
+
+
+CASE_MATMUL = r"<(?P<case>\d+)>\((?:unsigned char\*, ){%d}void\*\)"
+SPECS["tmatmul"] = dict(fn="LaunchTMATMUL", lib="tmatmul", tail=CASE_MATMUL % 3, planner=plan_matmul, inputs="unit", bias=False)
+SPECS["tmatmul:bias"] = dict(fn="LaunchTMATMULBIAS", lib="tmatmul", tail=CASE_MATMUL % 4, planner=plan_matmul, inputs="unit", bias=True)
+
+
+def lib_of(test):
+    """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
+    return SPECS[test].get("lib", test)
+
+
 def draw(rng, dt, shape, kind, j):
     """Operand j of a test whose operation is of the given kind."""
     bits = dt.itemsize * 8
@@ -428,6 +479,10 @@ def draw(rng, dt, shape, kind, j):
         if kind == "cvt":
             lo, hi = -10000, 10000
         return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
+    if kind == "unit":
+        return rng.uniform(-1.0, 1.0, size=shape).astype(dt)
+    if kind == "bf16":
+        return _bf16_bits(rng.uniform(-1.0, 1.0, size=shape))
     if kind == "small":                       # few distinct values: equal pairs occur, products stay small
         return rng.integers(-3 if dt.kind != "u" else 0, 3, size=shape, endpoint=True).astype(dt)
     if dt.kind == "f":

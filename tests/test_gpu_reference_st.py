@@ -19,7 +19,7 @@ CASES = S.cases()
 def test_the_test_kernel_libraries_were_built():
     if not os.path.isdir(S.ST_DIR):
         pytest.skip("oracle/_ref/st not built (reference tree absent at build time)")
-    assert len(CASES) >= 150 and {c[0] for c in CASES} == set(S.SPECS)
+    assert len(CASES) >= 700 and {c[0] for c in CASES} == set(S.SPECS)
 
 
 @pytest.mark.parametrize("test,mangled,demangled", CASES, ids=[c[2][5:].split("(")[0] for c in CASES])
@@ -27,16 +27,25 @@ def test_reference_st_kernel(test, mangled, demangled):
     import torch
     pl = S.plan(test, demangled)
     ins = S.make_inputs(pl, seed=len(demangled) + sum(map(ord, demangled)) % 997)
-    lib = C.CDLL(os.path.join(S.ST_DIR, test + ".so"))
+    lib = C.CDLL(os.path.join(S.ST_DIR, S.lib_of(test) + ".so"))
     fn = getattr(lib, mangled)
     dev = "cuda:0"
     view = {np.dtype(np.float16): np.int16, np.dtype(np.uint16): np.int16, np.dtype(np.uint32): np.int32}
 
     def to_dev(a):
         return torch.from_numpy(a.view(view.get(a.dtype, a.dtype))).to(dev)
+
+    def to_dev_padded(a):
+        # 4096 zero elements follow every input: the reference's split-k matmul case reads its matrices in blocks of 32
+        # columns with the row stride of the valid k (tmatmul_kernel.cpp:212-216, 254-255), which for k = 75 runs past the
+        # end of both; zeros there make those reads defined and leave the product what the generator computes
+        flat = a.reshape(-1)
+        buf = np.zeros(flat.size + 4096, dtype=a.dtype)
+        buf[:flat.size] = flat
+        return to_dev(buf)
     sentinel = 77
     t_out = [to_dev(np.full(shape, sentinel, dtype=dt)) for dt, shape in pl.outs]
-    t_in = [to_dev(a) for a in ins]
+    t_in = [to_dev_padded(a) for a in ins]
     args = [C.c_void_p(t.data_ptr()) for t in t_out + t_in]
     if pl.scalar:
         args.append(pl.scalar[0](pl.scalar[1]))
@@ -49,7 +58,9 @@ def test_reference_st_kernel(test, mangled, demangled):
         wants = S.expected(pl, ins)
     for t, (dt, shape), (vr, vc), want in zip(t_out, pl.outs, pl.regions, wants):
         got = t.cpu().numpy().view(dt)
-        if dt.kind == "f":
+        if pl.compare is not None:
+            assert pl.compare(got[:vr, :vc], np.asarray(want), ins), demangled
+        elif dt.kind == "f":
             want = np.asarray(want, dtype=np.float64).astype(dt)
             tol = pl.spec.get("tol", {}).get(dt.name, 2e-6 if dt == np.float32 else 1.5e-3)
             atol = pl.spec.get("atol", {}).get(dt.name, tol * 1e-2)
