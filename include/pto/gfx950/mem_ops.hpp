@@ -138,7 +138,13 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
     } else if constexpr (T::Loc == TileType::Mat) {
         const uint64_t a = (uint64_t)(uintptr_t)addr;
         const uint32_t off = (a >> 32) ? (uint32_t)a - (uint32_t)(uintptr_t)hw::lds_base() : (uint32_t)a;
-#if defined(__HIP_DEVICE_COMPILE__)
+#if defined(PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL)
+        // For translation units that hold many kernels of which a few need more L1 than a compute unit has LDS (the
+        // reference's per-instruction test sources): such a kernel ends at the TASSIGN, every wave alike, having done
+        // nothing, instead of stopping the build of the others.
+        if (off + detail::mat_tile_bytes<T>() > detail::kLdsBytes)
+            __builtin_amdgcn_endpgm();
+#elif defined(__HIP_DEVICE_COMPILE__)
         if (__builtin_constant_p(off) && off + detail::mat_tile_bytes<T>() > detail::kLdsBytes)
             detail::tassign_beyond_lds();
 #endif

@@ -147,13 +147,17 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolsum", "tcolmax", "tcolmin", "tcolprod", "trowexpand",
               "trowexpandadd", "trowexpandsub", "trowexpandmul", "trowexpanddiv", "trowexpandmax", "trowexpandmin", "trowexpandexpdif",
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
-              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul"]
+              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
 _ST_KEYED = re.compile(r"tilingKey\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
+_ST_KEYED_KERNEL = re.compile(r"tilingKey\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<<<")
+_ST_KERNEL_BODY = re.compile(r'extern "C" __global__ AICORE void (\w+)\([^)]*\)\s*\{(.*?)\n\}', re.S)
 # options of the port script per test kernel: L1 addresses written for Ascend's 512 KiB moved inside the LDS
 ST_PORT_OPTIONS = {
     "tmatmul": dict(l1_map={0x20000: 0x10000, 0x40000: 0x1C000}),
+    # four of its 46 kernels keep 64 + 128 KiB of fp32 tiles in L1: they end at their TASSIGN and are not run
+    "textract": dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL"]),
 }
 
 
@@ -170,6 +174,21 @@ def st_case_table(source_text):
         owner = [name for pos, name in launchers if pos < m.start()]
         if owner:
             table["%s:%s" % (owner[-1], m.group(1))] = {"run": m.group(2), "targs": [a.strip() for a in m.group(3).split(",")], "params": ""}
+    # ... or `if constexpr (tilingKey == N) { kernel<<<`, the kernel fixing its case through local constants
+    # (`constexpr uint32_t M = 64;`) that it hands to one run function: the constants and the run function's leading type
+    # arguments are the case
+    bodies = {m.group(1): m.group(2) for m in _ST_KERNEL_BODY.finditer(source_text)}
+    for m in _ST_KEYED_KERNEL.finditer(source_text):
+        owner = [name for pos, name in launchers if pos < m.start()]
+        body = bodies.get(m.group(2))
+        if not owner or body is None:
+            continue
+        run = re.search(r"(run\w+)\s*<([^;]*?)>\s*\(", body, re.S)
+        if run is None:
+            continue
+        table["%s:%s" % (owner[-1], m.group(1))] = {
+            "run": run.group(1), "targs": [a.strip() for a in run.group(2).split(",")], "params": "",
+            "consts": dict(re.findall(r"constexpr\s+\w+\s+(\w+)\s*=\s*(\w+)\s*;", body))}
     return table
 
 

@@ -136,7 +136,8 @@ def cases():
     for test, spec in SPECS.items():
         pat = _pattern(spec)
         for mangled, demangled in sorted(man.get(spec.get("lib", test), {}).get("launchers", {}).items(), key=lambda kv: kv[1]):
-            if pat.match(demangled):
+            m = pat.match(demangled)
+            if m and ("runnable" not in spec or spec["runnable"](spec, m)):
                 out.append((test, mangled, demangled))
     return out
 
@@ -462,6 +463,61 @@ def plan_matmul(test, spec, m):
 CASE_MATMUL = r"<(?P<case>\d+)>\((?:unsigned char\*, ){%d}void\*\)"
 SPECS["tmatmul"] = dict(fn="LaunchTMATMUL", lib="tmatmul", tail=CASE_MATMUL % 3, planner=plan_matmul, inputs="unit", bias=False)
 SPECS["tmatmul:bias"] = dict(fn="LaunchTMATMULBIAS", lib="tmatmul", tail=CASE_MATMUL % 4, planner=plan_matmul, inputs="unit", bias=True)
+
+
+# ---- TMOV / TEXTRACT windows: launchTMOV<N> / launchTEXTRACT<N> / launchTEXTRACT_COMPACT<N>(uint8 *out, uint8 *src0,
+# uint8 *src1, stream): out[M - iM, N - iN] = A[iM:M, iK:K] x B[iK:K, iN:N] with A [baseM, baseK] and B [baseK, baseN] in
+# memory (base = M, K, N where the case names none), each row-major or, "transposed", column-major (textract_kernel.cpp:
+# 17-74 runTMOV, :76-148 unaligned, :150-220 runTEXTRACT, :222-294 unaligned, :296-364 run-time valid, :366-442 compact)
+def _extract_case(spec, m):
+    return manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]
+
+
+def _extract_dims(e):
+    c = e["consts"]
+    M, N, K = int(c["M"]), int(c["N"]), int(c["K"])
+    return dict(M=M, N=N, K=K, iM=int(c.get("indexM", 0)), iN=int(c.get("indexN", 0)), iK=int(c.get("indexK", 0)),
+                bM=int(c.get("baseM", M)), bN=int(c.get("baseN", N)), bK=int(c.get("baseK", K)),
+                ta=c["isAtranspose"] == "true", tb=c["isBtranspose"] == "true")
+
+
+def extract_runnable(spec, m):
+    """False for the cases whose L1 tiles need more than a compute unit's 160 KiB of LDS (A at 0, B at 64 KiB)"""
+    e = _extract_case(spec, m)
+    d = _extract_dims(e)
+    size = {"half": 2, "bfloat16_t": 2, "float": 4, "int8_t": 1}[e["targs"][1]]
+    return 64 * 1024 + d["bK"] * d["bN"] * size <= 160 * 1024 and d["bM"] * d["bK"] * size <= 64 * 1024
+
+
+def plan_extract(test, spec, m):
+    e = _extract_case(spec, m)
+    d = _extract_dims(e)
+    names = {"half": np.float16, "float": np.float32, "int8_t": np.int8, "int32_t": np.int32, "bfloat16_t": np.uint16}
+    out_dt, a_dt = np.dtype(names[e["targs"][0]]), np.dtype(names[e["targs"][1]])
+    bf16 = e["targs"][1] == "bfloat16_t"
+    kind = "bf16" if bf16 else ("bits" if a_dt.kind == "i" else "unit")
+    shape_a = (d["bK"], d["bM"]) if d["ta"] else (d["bM"], d["bK"])
+    shape_b = (d["bN"], d["bK"]) if d["tb"] else (d["bK"], d["bN"])
+    vm, vn = d["M"] - d["iM"], d["N"] - d["iN"]
+
+    def values(arrays):
+        conv = (lambda x: _bf16_value(x).astype(np.float64)) if bf16 else (lambda x: x.astype(np.int64 if a_dt.kind == "i" else np.float64))
+        a, b = conv(arrays[0]), conv(arrays[1])
+        a = a.T if d["ta"] else a
+        b = b.T if d["tb"] else b
+        return a[d["iM"]:d["M"], d["iK"]:d["K"]], b[d["iK"]:d["K"], d["iN"]:d["N"]]
+
+    def expect(arrays):
+        a, b = values(arrays)
+        return [a @ b]
+    pl = _plan(spec, [(out_dt, (vm, vn))], [(a_dt, shape_a, kind), (a_dt, shape_b, kind)], [(vm, vn)], expect)
+    pl.compare = None if out_dt.kind == "i" else (
+        lambda got, want, arrays: np.max(np.abs(got.astype(np.float64) - want) / (np.abs(values(arrays)[0]) @ np.abs(values(arrays)[1]) + 1.0)) < 2e-3)
+    return pl
+
+
+for _fn in ("launchTMOV", "launchTEXTRACT", "launchTEXTRACT_COMPACT"):
+    SPECS["textract:" + _fn] = dict(fn=_fn, lib="textract", tail=CASE_MATMUL % 3, planner=plan_extract, inputs="unit", runnable=extract_runnable)
 
 
 def lib_of(test):
