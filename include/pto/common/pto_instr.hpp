@@ -226,7 +226,28 @@ PTO_FRONT(TCMP, typename T, T &dst PTO_C T &src0 PTO_C T &src1 PTO_C CmpMode mod
 PTO_FRONT(TCMPS, typename D PTO_C typename S PTO_C typename T, D &dst PTO_C S &src0 PTO_C T src1 PTO_C CmpMode mode,
           (dst, src0, src1, mode))
 PTO_FRONT(TSEL, typename T PTO_C typename M, T &dst PTO_C M &selMask PTO_C T &src0 PTO_C T &src1, (dst, selMask, src0, src1))
-PTO_FRONT(TSELS, typename T, T &dst PTO_C T &src0 PTO_C T &src1 PTO_C uint8_t selectMode, (dst, src0, src1, selectMode))
+// TSELS has two meanings in the reference.  Its front end (pto_instr.hpp:1014-1021) and the NPU take (dst, mask, src, scalar):
+// a tile of integers as bit mask.  Its CPU simulation implements (dst, src0, src1, selectMode) on three tiles of one type,
+// the whole of src0 or of src1.  A second operand that is a tile of integers is a mask; three floating-point tiles of one
+// type are the whole-tile form.
+template <typename T, typename... Ev, std::enable_if_t<!std::is_integral_v<typename T::DType>, int> = 0>
+PTO_INST RecordEvent TSELS(T &dst, T &src0, T &src1, uint8_t selectMode, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src0, src1, selectMode);
+    TSELS_IMPL(dst, src0, src1, selectMode);
+    detail::UbCommit(dst, src0, src1, selectMode);
+    return {};
+}
+template <typename D, typename M, typename S, typename... Ev, std::enable_if_t<std::is_integral_v<typename M::DType>, int> = 0>
+PTO_INST RecordEvent TSELS(D &dst, M &mask, S &src, typename S::DType scalar, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(mask, src);
+    TSELS_MASK_IMPL(dst, mask, src, scalar);
+    detail::UbCommit(dst);
+    return {};
+}
 PTO_FRONT(TFILLPAD, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TPUSH, typename P PTO_C typename T PTO_C typename F, P &prod PTO_C T &tile PTO_C F &fifo, (prod, tile, fifo))
 PTO_FRONT(TPOP, typename P PTO_C typename T PTO_C typename F, P &cons PTO_C T &tile PTO_C F &fifo, (cons, tile, fifo))

@@ -495,7 +495,7 @@ PTO_DEV void TGATHER_IMPL(DstT &dst, Src0T &src0, IdxT &idx)
     static_assert(std::is_same_v<T, typename Src0T::DType>, "[PTO][SA] TGATHER: dst and src0 types differ");
     static_assert(DstT::Numel == IdxT::Numel && DstT::isRowMajor == IdxT::isRowMajor,
                   "[PTO][SA] TGATHER: dst and index tiles must have the same shape");
-    static_assert(Src0T::Numel * sizeof(T) <= 64 * 1024, "[PTO][SA] TGATHER: source tile must fit 64 KiB of LDS");
+    static_assert(Src0T::Numel * sizeof(T) <= 128 * 1024, "[PTO][SA] TGATHER: source tile must fit 128 KiB of LDS");
     __shared__ T stage[Src0T::Numel]; // in (row, col) row-major order
     detail::for_each_owned<Src0T>([&](int s, int i, int e) {
         if (e < Src0T::Numel) {

@@ -218,6 +218,37 @@ PTO_DEV void TSELS_IMPL(TileT &dst, TileT &src0, TileT &src1, uint8_t selectMode
             dst.S().v[s][i] = selectMode == 1 ? src0.S().v[s][i] : src1.S().v[s][i];
 }
 
+// dst[i,j] = bit (i,j) of the mask ? src[i,j] : scalar (npu/a2a3/TSels.hpp:19-46 and its generator tsels/gen_data.py:38-45):
+// row i of the mask tile, read as bytes whatever its element type, holds the bits of row i, lowest bit first.  This is the
+// form the reference's front end has (pto_instr.hpp:1014-1021); the whole-tile form above is what its CPU simulation
+// implements.
+template <typename DstT, typename MaskT, typename SrcT>
+PTO_DEV void TSELS_MASK_IMPL(DstT &dst, MaskT &mask, SrcT &src, typename SrcT::DType scalar)
+{
+    using T = typename DstT::DType;
+    using MT = typename MaskT::DType;
+    static_assert(std::is_integral_v<MT> && DstT::isRowMajor && MaskT::isRowMajor && sizeof(T) == sizeof(typename SrcT::DType),
+                  "[PTO][SA] TSELS: row-major tiles, a mask tile of integers");
+    __shared__ MT bits[MaskT::Numel];
+    detail::for_each_owned<MaskT>([&](int s, int i, int e) {
+        if (e < MaskT::Numel)
+            bits[e] = mask.S().v[s][i];
+    });
+    hw::lds_barrier();
+    detail::Conformed<DstT, SrcT> x(src);
+    constexpr int kRowBytes = MaskT::Cols * (int)sizeof(MT);
+    const uint8_t *bytes = reinterpret_cast<const uint8_t *>(bits);
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols;
+        if (e < DstT::Numel && r < vr && c < vc && r < MaskT::Rows && (c >> 3) < kRowBytes) {
+            const uint32_t byte = bytes[r * kRowBytes + (c >> 3)];
+            dst.S().v[s][i] = ((byte >> (c & 7)) & 1u) ? (T)x.S().v[s][i] : (T)scalar;
+        }
+    });
+    hw::lds_barrier();
+}
+
 // ------------------------------------------------------------------ TFILLPAD
 // dst = src inside the source's valid region, the destination's pad value elsewhere, over the whole
 // tile (TFillPad.hpp:22-49; Max / Min pad = +/- infinity for floating types).

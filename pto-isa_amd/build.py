@@ -147,7 +147,8 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolsum", "tcolmax", "tcolmin", "tcolprod", "trowexpand",
               "trowexpandadd", "trowexpandsub", "trowexpandmul", "trowexpanddiv", "trowexpandmax", "trowexpandmin", "trowexpandexpdif",
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
-              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract"]
+              "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract",
+              "tmax", "tmin", "tmins", "texpands", "tsels"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
 _ST_KEYED = re.compile(r"tilingKey\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
@@ -159,6 +160,9 @@ ST_PORT_OPTIONS = {
     # four of its 46 kernels keep 64 + 128 KiB of fp32 tiles in L1: they end at their TASSIGN and are not run
     "textract": dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL"]),
 }
+# sources that keep their device code under the Ascend device compiler's own macro
+for _name in ("tmax", "tmin", "tmins", "texpands"):
+    ST_PORT_OPTIONS[_name] = dict(defines=["__CCE_AICORE__=220"])
 
 
 def st_case_table(source_text):

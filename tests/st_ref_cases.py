@@ -520,6 +520,66 @@ for _fn in ("launchTMOV", "launchTEXTRACT", "launchTEXTRACT_COMPACT"):
     SPECS["textract:" + _fn] = dict(fn=_fn, lib="textract", tail=CASE_MATMUL % 3, planner=plan_extract, inputs="unit", runnable=extract_runnable)
 
 
+# ---- TMAX / TMIN: LaunchTMax<T, gRows, gCols, tileRows, tileCols, validRows, validCols, pad>: the valid corner of
+# [gRows, gCols] buffers (tmax_kernel.cpp:39-66); LaunchTMins (TMIN on tiles of three widths, tmins_kernel.cpp:39-75) is the
+# nine-argument form with the pad value as a tenth
+def plan_g_valid(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    gr, gc, vr, vc = (int(m.group(k)) for k in ("gr", "gc", "vr", "vc"))
+    return _elementwise_plan(spec, dt, [(gr, gc)] * 3, (vr, vc), None)
+
+
+def plan_nine_pad(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    q = _ints(m, ["dH", "dW", "aH", "aW", "bH", "bW", "vR", "vC"])
+    return _elementwise_plan(spec, dt, [(q["dH"], q["dW"]), (q["aH"], q["aW"]), (q["bH"], q["bW"])], (q["vR"], q["vC"]), None)
+
+
+# ---- TEXPANDS: LaunchTExpandS<T, gRows, gCols, tileRows, tileCols, validRows, validCols, pad>(void *out, float scalar):
+# the scalar, converted to T, over the valid corner (texpands_kernel.cpp:38-58)
+def plan_expands(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    gr, gc, vr, vc = (int(m.group(k)) for k in ("gr", "gc", "vr", "vc"))
+    value = 2.5 if dt.kind == "f" else 7.0
+    return _plan(spec, [(dt, (gr, gc))], [], [(vr, vc)], lambda a: [np.full((vr, vc), dt.type(value))], scalar=(C.c_float, value))
+
+
+# ---- TSELS: LaunchTSels<T, TMask, dstH, dstW, maskH, maskW, srcH, srcW, validRows, validCols>(T *out, TMask *mask, T *src,
+# T scalar): bit (r, c) of mask row r, read as bytes, takes src, a clear bit the scalar (tsels_kernel.cpp:17-60,
+# gen_data.py:38-45); LaunchTSelsHalf the same on fp16 with the scalar's bit pattern by value
+def plan_sels(test, spec, m):
+    half = m.group("half") is not None
+    dt, ct = _elem("unsigned short" if half else m.group("T"), half)
+    mdt, _ = _elem(m.group("M"), False)
+    q = _ints(m, ["dH", "dW", "mH", "mW", "sH", "sW", "vR", "vC"])
+    vr, vc = q["vR"], q["vC"]
+    value = 1.5 if dt.kind == "f" else 12345
+    if half:
+        scalar = (C.c_uint16, int(np.float16(value).view(np.uint16)))
+    else:
+        scalar = (ct, value)
+
+    def expect(a):
+        bits = np.unpackbits(np.ascontiguousarray(a[0]).view(np.uint8).reshape(a[0].shape[0], -1), axis=1, bitorder="little")[:vr, :vc].astype(bool)
+        return [np.where(bits, a[1][:vr, :vc], dt.type(value))]
+    return _plan(spec, [(dt, (q["dH"], q["dW"]))], [(mdt, (q["mH"], q["mW"]), "bits"), (dt, (q["sH"], q["sW"]), "any")], [(vr, vc)],
+                 expect, scalar=scalar)
+
+
+GVALID = TAIL(["gr", "gc", "tr", "tc", "vr", "vc", "pad"], 3)
+SPECS.update({
+    "tmax": dict(fn="LaunchTMax", tail=GVALID, planner=plan_g_valid, nin=2, inputs="any", op=np.maximum),
+    "tmin": dict(fn="LaunchTMin", tail=GVALID, planner=plan_g_valid, nin=2, inputs="any", op=np.minimum),
+    "tmins": dict(fn="LaunchTMins", tail=TAIL(["dH", "dW", "aH", "aW", "bH", "bW", "vR", "vC", "pad"], 3), planner=plan_nine_pad, nin=2,
+                  inputs="any", op=np.minimum),
+    "texpands": dict(fn="LaunchTExpandS", tail=r"<(?P<T>[a-z ]+), (?P<gr>\d+), (?P<gc>\d+), (?P<tr>\d+), (?P<tc>\d+), (?P<vr>\d+), (?P<vc>\d+), -?\d+>\(void\*, float, void\*\)",
+                     planner=plan_expands, inputs="any"),
+    "tsels": dict(fn="LaunchTSels", inputs="any", planner=plan_sels,
+                  tail=r"(?P<half>Half)?<(?:(?P<T>[a-z ]+), )?(?P<M>unsigned [a-z]+), (?P<dH>\d+), (?P<dW>\d+), (?P<mH>\d+), (?P<mW>\d+), (?P<sH>\d+), "
+                       r"(?P<sW>\d+), (?P<vR>\d+), (?P<vC>\d+)>\([a-z ]+\*, [a-z ]+\*, [a-z ]+\*, [a-z ]+, void\*\)"),
+})
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
