@@ -32,8 +32,8 @@ GATHER_HBM_SIDE_BYTES = 85.0e6 + 134.3e6
 # counter reads for a plain 1 GiB device copy in the same run (--calib-copy): FETCH_SIZE reads
 # 524,300 KiB for 1,048,576 KiB actually read (factor 2.0), WRITE_SIZE reads 1,048,576 KiB for
 # 1,048,576 KiB written (factor 1.0).
-GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 295758.0, 2.0
-GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 149166.0, 1.0
+GEMM_6144_FETCH_KIB, GEMM_6144_FETCH_SCALE = 295679.0, 2.0
+GEMM_6144_WRITE_KIB, GEMM_6144_WRITE_SCALE = 149158.0, 1.0
 
 
 SETTLE_S = 0.0   # set from --settle-ms: the workloads under "extra" keep warming up until this much time has passed
