@@ -102,8 +102,9 @@ PTO_DEV void TSORT32_IMPL(DstT &dst, SrcT &src, IdxT &idx)
     uint32_t *index = reinterpret_cast<uint32_t *>(image + N);
     B *score = reinterpret_cast<B *>(index + N);
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
-    if (vr != idx.GetValidRow() || vc != idx.GetValidCol() || vc > C)
-        return; // as the reference does (cpu/TSort32.hpp:113-115); the valid extents are uniform over the workgroup
+    if (vr > idx.GetValidRow() || vc > idx.GetValidCol() || vc > C)
+        return; // the index tile must cover the scores (cpu/TSort32.hpp:113-115 asks for equal extents; the NPU's tests give
+                // the index tile the row length rounded up to 32 bytes: tsort32_kernel.cpp:47-49); uniform over the workgroup
     detail::stage_tile_rows(src, score, C);
     detail::stage_tile_rows(idx, index, C);
     hw::lds_barrier();

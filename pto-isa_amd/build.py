@@ -148,11 +148,11 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "trowexpandadd", "trowexpandsub", "trowexpandmul", "trowexpanddiv", "trowexpandmax", "trowexpandmin", "trowexpandexpdif",
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
               "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract",
-              "tmax", "tmin", "tmins", "texpands", "tsels"]
+              "tmax", "tmin", "tmins", "texpands", "tsels", "tsort32", "tgather", "tmrgsort"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
-_ST_KEYED = re.compile(r"tilingKey\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<")
+_ST_KEYED = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
-_ST_KEYED_KERNEL = re.compile(r"tilingKey\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<<<")
+_ST_KEYED_KERNEL = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<<<")
 _ST_KERNEL_BODY = re.compile(r'extern "C" __global__ AICORE void (\w+)\([^)]*\)\s*\{(.*?)\n\}', re.S)
 # options of the port script per test kernel: L1 addresses written for Ascend's 512 KiB moved inside the LDS
 ST_PORT_OPTIONS = {
@@ -160,6 +160,8 @@ ST_PORT_OPTIONS = {
     # four of its 46 kernels keep 64 + 128 KiB of fp32 tiles in L1: they end at their TASSIGN and are not run
     "textract": dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL"]),
 }
+# its top-k kernel works through Vec tiles that are views of one another (TASSIGN to the same address)
+ST_PORT_OPTIONS["tmrgsort"] = dict(vec_in_memory=True)
 # sources that keep their device code under the Ascend device compiler's own macro
 for _name in ("tmax", "tmin", "tmins", "texpands"):
     ST_PORT_OPTIONS[_name] = dict(defines=["__CCE_AICORE__=220"])
@@ -192,7 +194,7 @@ def st_case_table(source_text):
             continue
         table["%s:%s" % (owner[-1], m.group(1))] = {
             "run": run.group(1), "targs": [a.strip() for a in run.group(2).split(",")], "params": "",
-            "consts": dict(re.findall(r"constexpr\s+\w+\s+(\w+)\s*=\s*(\w+)\s*;", body))}
+            "consts": {k: " ".join(v.split()) for k, v in re.findall(r"constexpr\s+\w+\s+(\w+)\s*=\s*([^;]+);", body)}}
     return table
 
 

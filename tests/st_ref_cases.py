@@ -18,7 +18,8 @@ ST_DIR = os.path.join(ROOT, "oracle", "_ref", "st")
 
 CTYPE = {"float": (np.float32, C.c_float), "int": (np.int32, C.c_int32), "short": (np.int16, C.c_int16),
          "unsigned short": (np.uint16, C.c_uint16), "signed char": (np.int8, C.c_int8), "unsigned char": (np.uint8, C.c_uint8),
-         "unsigned int": (np.uint32, C.c_uint32), "long": (np.int64, C.c_int64)}
+         "unsigned int": (np.uint32, C.c_uint32), "long": (np.int64, C.c_int64),
+         "_Float16": (np.float16, C.c_uint16)}
 CTYPE.update({"int32_t": CTYPE["int"], "int16_t": CTYPE["short"], "uint16_t": CTYPE["unsigned short"], "uint32_t": CTYPE["unsigned int"],
               "int8_t": CTYPE["signed char"], "uint8_t": CTYPE["unsigned char"]})
 
@@ -194,7 +195,7 @@ def _elementwise_plan(spec, dtype, buffers, valid, scalar, scalar_first=False):
             return [op(k, a) if scalar_first else op(a, k)]
         return [op(a) if len(ins) == 1 else op(a, ins[1][:vr, :vc])]
     return SimpleNamespace(dtype=dtype, outs=[(dtype, buffers[0])], ins=[(dtype, b) for b in buffers[1:]], regions=[valid],
-                           scalar=scalar, expect=expect, spec=spec, compare=None)
+                           scalar=scalar, expect=expect, spec=spec, compare=None, flat_prefix=None)
 
 
 # ---- numbered cases: launch<OP>TestCase<N>(void *out, void *src, float scalar, stream) -> run<T, dstRows, dstCols, rows,
@@ -240,13 +241,13 @@ SPECS.update({
 
 def TAIL(ints, nptr, suffix="", ptr0=None):
     """Demangled `<T, int..., suffix>(T*, ... nptr pointers ..., void*)`; ptr0: type of the first pointer if it is not T."""
-    ptrs = (re.escape(ptr0) + r"\*, " if ptr0 else "") + r"(?:[a-z ]+\*, ){%d}" % (nptr - (1 if ptr0 else 0))
-    return r"<(?P<T>[a-z ]+)" + "".join(r", (?P<%s>-?\d+)u?" % n for n in ints) + suffix + r">\(" + ptrs + r"void\*\)"
+    ptrs = (re.escape(ptr0) + r"\*, " if ptr0 else "") + r"(?:[A-Za-z_0-9 ]+\*, ){%d}" % (nptr - (1 if ptr0 else 0))
+    return r"<(?P<T>[A-Za-z_0-9 ]+)" + "".join(r", (?P<%s>-?\d+)u?" % n for n in ints) + suffix + r">\(" + ptrs + r"void\*\)"
 
 
 def _plan(spec, outs, ins, regions, expect, scalar=None):
     return SimpleNamespace(dtype=ins[0][0] if ins else outs[0][0], outs=outs, ins=ins, regions=regions, scalar=scalar,
-                           expect=lambda arrays, k: expect(arrays), spec=spec, compare=None)
+                           expect=lambda arrays, k: expect(arrays), spec=spec, compare=None, flat_prefix=None)
 
 
 # ---- column reductions: launchTCOLSUM<T, cols, srcRows, validRows[, binary]>: [validRows, cols] of a [srcRows, cols] buffer
@@ -580,6 +581,164 @@ SPECS.update({
 })
 
 
+# ---- TGATHER, mask form: LaunchTGATHER<T, gRows, gCols, tileRows, tileCols, pattern>(T *out, T *src): the selected columns
+# of every row (every 2nd or 4th from a phase, or all), packed in running order from the start of the output
+# (tgather_kernel.cpp:21-46, gen_data.py:98-116); what follows the packed elements in the output is not defined
+def plan_gather_mask(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    gr, gc, p = int(m.group("gr")), int(m.group("gc")), int(m.group("pattern"))
+    step, phase = (1, 0) if p == 7 else ((2, p - 1) if p <= 2 else (4, p - 3))
+    n = gr * len(range(phase, gc, step))
+    pl = _plan(spec, [(dt, (gr, gc))], [(dt, (gr, gc), "pos")], [(gr, gc)], lambda a: [a[0][:, phase::step].reshape(-1)])
+    pl.flat_prefix = n
+    return pl
+
+
+# ---- TSORT32: launchTSORT32<N>(uint64 *out, uint64 *src, uint32 *idx, uint64 *tmp) -> runTSORT32<T, rows, cols, validRows,
+# validCols, alignedCols>: every group of 32 valid columns of a row in descending order of score, as (score, index)
+# structures of 8 bytes (tsort32_kernel.cpp:22-75; the oracle's tsort32 is the expectation)
+def _const_value(expr, consts):
+    expr = expr.replace("sizeof(float)", "4").replace("sizeof(half)", "2").replace("/", "//")
+    if not re.fullmatch(r"[\w\s+\-*/()]+", expr):
+        raise ValueError(expr)
+    names = {k: _const_value(v, consts) for k, v in consts.items() if re.search(r"\b%s\b" % k, expr)}
+    return int(eval(expr, {"__builtins__": {}}, names))
+
+
+def plan_sort32(test, spec, m):
+    e = manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]
+    c = e["consts"]
+    rows, cols, vr, vc, ac = (_const_value(c[k], c) for k in ("ROWS", "COLS", "VALID_R", "VALID_C", "ALIGN_C"))
+    dt = np.dtype(np.float32 if e["targs"][0] == "float" else np.float16)
+    per = 8 // dt.itemsize
+
+    def expect(a):
+        import sys
+        sys.path.insert(0, ROOT)
+        from oracle import oracle
+        dst = np.zeros((rows, per * cols), dtype=dt)
+        return [oracle.tsort32(dst, a[0], a[1], vr, vc)[:vr, :per * vc]]
+    pl = _plan(spec, [(dt, (rows, per * cols))], [(dt, (rows, cols), "scores"), (np.dtype(np.uint32), (rows, cols), "index"), (dt, (1, ac), "any")],
+               [(vr, per * vc)], expect)
+    bits = {2: np.uint16, 4: np.uint32}[dt.itemsize]
+    pl.compare = lambda got, want, arrays: np.array_equal(np.ascontiguousarray(got).view(bits), np.ascontiguousarray(want).view(bits))
+    return pl
+
+
+SPECS["tgather"] = dict(fn="LaunchTGATHER", tail=TAIL(["gr", "gc", "tr", "tc"], 2, r", \(pto::MaskPattern\)(?P<pattern>\d)"), planner=plan_gather_mask, inputs="pos")
+SPECS["tsort32"] = dict(fn="launchTSORT32", lib="tsort32", planner=plan_sort32, inputs="any",
+                        tail=r"<(?P<case>\d+)>\(unsigned long\*, unsigned long\*, unsigned int\*, unsigned long\*, void\*\)")
+
+
+# ---- TMRGSORT (tmrgsort_kernel.cpp): every launcher takes float pointers; T = uint16_t runs the half kernels with all column
+# counts doubled (:261-297), so a "column" below is 4 bytes and a structure (score, index) two of them.
+#   LanchTMrgsortMulti<T, gRows, gCols, rows, cols0, cols1, cols2, cols3, topk, lists, exhausted>: 2-4 sorted lists merged (:65-114)
+#   LanchTMrgsortSingle<T, gRows, gCols, rows, cols, blockLen>: every four blocks of one source merged (:116-148)
+#   LanchTMrgsortTopK<T, gRows, gCols, rows, cols, topk>: sorted blocks of 64 columns merged all the way, first topk kept (:194-258)
+def _sort_struct_lists(rng, half, counts, distinct=False):
+    """sorted lists of `counts` structures each, as arrays of the kernel's element type"""
+    import sort_cases as SC
+    out = []
+    for tag, n in enumerate(counts):
+        l = SC.sorted_list_16(rng, n, "f16", tag) if half else SC.sorted_list(rng, n, tag=tag)
+        out.append(np.ascontiguousarray(l).reshape(1, -1))
+    return out
+
+
+def _oracle():
+    import sys
+    if ROOT not in sys.path:
+        sys.path.insert(0, ROOT)
+    from oracle import oracle
+    return oracle
+
+
+def plan_mrgsort(test, spec, m):
+    half = m.group("T") == "unsigned short"
+    dt = np.dtype(np.float16 if half else np.float32)
+    coef = 2 if half else 1                     # elements of T per 4-byte column
+    bits = np.uint16 if half else np.uint32
+    form = spec["form"]
+    exact = lambda got, want, arrays: np.array_equal(np.ascontiguousarray(got).view(bits), np.ascontiguousarray(want).view(bits))
+    if form == "multi":
+        gc, c0, c1, c2, c3, topk, nl = (int(m.group(k)) for k in ("gc", "c0", "c1", "c2", "c3", "topk", "lists"))
+        exhausted = m.group("exh") == "true"
+        cols = [c0, c1, c2, c3][:nl]
+        ins = [(dt, (1, max(c, 8) * coef), ("sorted", c // 2, j)) for j, c in enumerate([c0, c1, c2, c3])]
+
+        def expect(a):
+            dst0 = np.zeros(topk * coef, dtype=dt)
+            dst, counts = _oracle().tmrgsort_lists(dst0, [a[j][0, :cols[j] * coef] for j in range(nl)], [c * coef for c in cols], topk * coef, exhausted)
+            n = int(sum(counts)) * 2 * coef
+            return [dst[:n]]
+        pl = _plan(spec, [(dt, (1, max(topk, gc * nl) * coef))], ins, [(1, topk * coef)], expect)
+        pl.flat_prefix, pl.compare = -1, exact          # -1: as long as the expectation
+        return pl
+    gc, tc = int(m.group("gc")), int(m.group("tc"))
+    if form == "single":
+        block = int(m.group("block"))
+        ins = [(dt, (1, gc * coef), ("blocks", block // 2, tc // 2))]
+        pl = _plan(spec, [(dt, (1, gc * coef))], ins, [(1, tc * coef)],
+                   lambda a: [_oracle().tmrgsort_blocks(np.zeros(tc * coef, dtype=dt), a[0][0, :tc * coef], tc * coef, block * coef)[None, :]])
+        pl.compare = exact
+        return pl
+    topk = int(m.group("topk"))
+    ins = [(dt, (1, gc * coef), ("blocks_distinct", 32, tc // 2))]
+
+    def expect_topk(a):
+        per = 2 * coef
+        structs = a[0][0, :tc * coef].reshape(-1, per)
+        order = np.argsort(-structs[:, 0].astype(np.float64), kind="stable")
+        return [structs[order][:topk // 2].reshape(-1)]
+    pl = _plan(spec, [(dt, (1, gc * coef))], ins, [(1, topk * coef)], expect_topk)
+    pl.flat_prefix, pl.compare = -1, exact
+    return pl
+
+
+def _sorted_inputs(rng, dt, shape, kind):
+    """kind = ("sorted", structures, tag) | ("blocks", structures per block, structures) | ("blocks_distinct", ...)"""
+    import sort_cases as SC
+    half = dt == np.float16
+    per = 4 if half else 2
+    buf = np.zeros(shape, dtype=dt)
+    if kind[0] == "sorted":
+        n, tag = kind[1], kind[2]
+        if n:
+            l = SC.sorted_list_16(rng, n, "f16", tag) if half else SC.sorted_list(rng, n, tag=tag)
+            buf[0, :n * per] = np.ascontiguousarray(l).reshape(-1)
+        return buf
+    blk, total = kind[1], kind[2]
+    parts = []
+    if kind[0] == "blocks":
+        for b in range(total // blk):
+            l = SC.sorted_list_16(rng, blk, "f16", b) if half else SC.sorted_list(rng, blk, tag=b)
+            parts.append(np.ascontiguousarray(l).reshape(-1))
+    else:                                      # all scores different, so that the merged order does not depend on how ties fall
+        scores = rng.permutation(total).astype(np.float64) - total // 2
+        for b in range(total // blk):
+            sc = np.sort(scores[b * blk:(b + 1) * blk])[::-1]
+            st = np.zeros((blk, per), dtype=dt)
+            st[:, 0] = sc.astype(dt)
+            ids = np.arange(b * blk, (b + 1) * blk, dtype=np.uint32)
+            if half:
+                st.view(np.uint16)[:, 2], st.view(np.uint16)[:, 3] = ids & 0xFFFF, ids >> 16
+            else:
+                st.view(np.uint32)[:, 1] = ids
+            parts.append(st.reshape(-1))
+    flat = np.concatenate(parts)
+    buf[0, :flat.size] = flat
+    return buf
+
+
+_MRG_T = r"<(?P<T>float|unsigned short), \d+, (?P<gc>\d+), \d+, "
+SPECS["tmrgsort:multi"] = dict(fn="LanchTMrgsortMulti", lib="tmrgsort", form="multi", planner=plan_mrgsort, inputs="any",
+                               tail=_MRG_T + r"(?P<c0>\d+), (?P<c1>\d+), (?P<c2>\d+), (?P<c3>\d+), (?P<topk>\d+), (?P<lists>\d), (?P<exh>true|false)>\((?:float\*, ){5}void\*\)")
+SPECS["tmrgsort:single"] = dict(fn="LanchTMrgsortSingle", lib="tmrgsort", form="single", planner=plan_mrgsort, inputs="any",
+                                tail=_MRG_T + r"(?P<tc>\d+), (?P<block>\d+)u>\((?:float\*, ){2}void\*\)")
+SPECS["tmrgsort:topk"] = dict(fn="LanchTMrgsortTopK", lib="tmrgsort", form="topk", planner=plan_mrgsort, inputs="any",
+                              tail=_MRG_T + r"(?P<tc>\d+), (?P<topk>\d+)>\((?:float\*, ){2}void\*\)")
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
@@ -587,6 +746,8 @@ def lib_of(test):
 
 def draw(rng, dt, shape, kind, j):
     """Operand j of a test whose operation is of the given kind."""
+    if isinstance(kind, tuple):
+        return _sorted_inputs(rng, dt, shape, kind)
     bits = dt.itemsize * 8
     if kind.startswith("cvt"):                # inside the range of every destination type of the conversion tests
         lo, hi = (0, 100) if kind == "cvt_u" else (-100, 100)
@@ -597,6 +758,10 @@ def draw(rng, dt, shape, kind, j):
         return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
     if kind == "unit":
         return rng.uniform(-1.0, 1.0, size=shape).astype(dt)
+    if kind == "scores":                      # few distinct values: many equal scores, whose order the index decides
+        return (rng.integers(-20, 20, size=shape) * 0.5).astype(dt)
+    if kind == "index":
+        return rng.permutation(int(np.prod(shape))).reshape(shape).astype(dt)
     if kind == "bf16":
         return _bf16_bits(rng.uniform(-1.0, 1.0, size=shape))
     if kind == "small":                       # few distinct values: equal pairs occur, products stay small
