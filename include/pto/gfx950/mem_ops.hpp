@@ -82,6 +82,33 @@ PTO_DEV int64_t gm_row_offset(const G &g, int64_t r)
     return i * g.GetStride(0) + j * g.GetStride(1) + k * g.GetStride(2) + rr * g.GetStride(3);
 }
 
+// Offset of logical element (r, c) of a 2-D tile in a 5-D GlobalTensor (TLoad.hpp:74-131 of the CPU simulation, the NZ
+// descriptors of npu/a2a3/TLoad.hpp): ND stacks the four outer dimensions along the rows, DN (column-major tiles) along
+// the columns, both with the innermost of them fastest; NZ is [col blocks 0][col blocks 1][row blocks][rows in a block]
+// [columns in a block]: row = i2 s3 + i3, column = (i0 s1 + i1) s4 + i4.
+template <typename G>
+PTO_DEV int64_t gm_elem_offset(const G &g, int64_t r, int64_t c)
+{
+    const int64_t s1 = g.GetShape(1), s2 = g.GetShape(2), s3 = g.GetShape(3), s4 = g.GetShape(4);
+    int64_t i0, i1, i2, i3, i4;
+    if constexpr (G::layout == Layout::NZ) {
+        i2 = r / s3, i3 = r % s3, i4 = c % s4;
+        const int64_t b = c / s4;
+        i1 = b % s1, i0 = b / s1;
+    } else if constexpr (G::layout == Layout::DN) {
+        i3 = r, i4 = c % s4;
+        int64_t b = c / s4;
+        i2 = b % s2, b /= s2;
+        i1 = b % s1, i0 = b / s1;
+    } else {
+        i4 = c, i3 = r % s3;
+        int64_t b = r / s3;
+        i2 = b % s2, b /= s2;
+        i1 = b % s1, i0 = b / s1;
+    }
+    return i0 * g.GetStride(0) + i1 * g.GetStride(1) + i2 * g.GetStride(2) + i3 * g.GetStride(3) + i4 * g.GetStride(4);
+}
+
 template <typename T>
 PTO_DEV T pad_value(PadValue p)
 {
@@ -263,7 +290,9 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
 {
     using T = typename TileT::DType;
     using S = typename TileT::Storage;
-    static_assert(TileT::SFractal == SLayout::NoneBox, "[PTO][SA] Vec tiles are unboxed on gfx950");
+    // (a box layout of a Vec tile names the order of its elements in Ascend's unified buffer; the register distribution
+    // holds logical elements, and only the NZ layout of the memory side shows in the addresses)
+    static_assert(TileT::SFractal == SLayout::NoneBox || !kVecTilesInMemory, "[PTO][SA] boxed Vec tiles: register tiles only");
     const T *gm = reinterpret_cast<const T *>(src.data());
     constexpr int Minor = TileT::isRowMajor ? TileT::Cols : TileT::Rows; // contiguous extent of the tile
     const int vMajor = TileT::isRowMajor ? dst.GetValidRow() : dst.GetValidCol();
@@ -272,6 +301,19 @@ PTO_DEV void tload_vec(TileT &dst, G &src)
     const bool stacked = src.GetShape(0) * src.GetShape(1) * src.GetShape(2) != 1;
     const T pad = pad_value<T>(TileT::PadVal);
     constexpr bool vecOK = Minor % kVecChunk == 0 && (kVecChunk * sizeof(T)) % 16 == 0 || Minor % kVecChunk == 0;
+    // NZ memory, or outer dimensions stacked along the columns of a column-major tile: element by element
+    if (G::layout == Layout::NZ || (!TileT::isRowMajor && stacked)) {
+        const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+#pragma unroll
+        for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i) {
+                const int e = (s * kBlockThreads + hw::tid()) * kVecChunk + i;
+                const int r = TileT::isRowMajor ? e / TileT::Cols : e % TileT::Rows, c = TileT::isRowMajor ? e % TileT::Cols : e / TileT::Rows;
+                dst.S().v[s][i] = (e < TileT::Numel && r < vr && c < vc) ? gm[gm_elem_offset(src, r, c)] : pad;
+            }
+        return;
+    }
 #pragma unroll
     for (int s = 0; s < S::Slots; ++s) {
         const int q = s * kBlockThreads + hw::tid();
@@ -698,6 +740,19 @@ PTO_DEV void tstore_vec(G &dst, TileT &src)
     const int vMinor = TileT::isRowMajor ? src.GetValidCol() : src.GetValidRow();
     const int64_t stMinor = TileT::isRowMajor ? dst.GetStride(4) : dst.GetStride(3);
     const bool stacked = dst.GetShape(0) * dst.GetShape(1) * dst.GetShape(2) != 1;
+    if (G::layout == Layout::NZ || (!TileT::isRowMajor && stacked)) { // as in tload_vec
+        const int vr = src.GetValidRow(), vc = src.GetValidCol();
+#pragma unroll
+        for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+            for (int i = 0; i < kVecChunk; ++i) {
+                const int e = (s * kBlockThreads + hw::tid()) * kVecChunk + i;
+                const int r = TileT::isRowMajor ? e / TileT::Cols : e % TileT::Rows, c = TileT::isRowMajor ? e % TileT::Cols : e / TileT::Rows;
+                if (e < TileT::Numel && r < vr && c < vc)
+                    gm[gm_elem_offset(dst, r, c)] = src.S().v[s][i];
+            }
+        return;
+    }
 #pragma unroll
     for (int s = 0; s < S::Slots; ++s) {
         const int q = s * kBlockThreads + hw::tid();

@@ -451,7 +451,10 @@ PTO_DEV void row_expand(DstT &dst, MatT &mat, RowT &row)
 template <RowOp op, typename DstT, typename A, typename B>
 PTO_DEV void row_expand_any(DstT &dst, A &src0, B &src1)
 {
-    if constexpr (kIsRowOperand<B, DstT>)
+    // as the reference decides it (npu/a2a3/TRowExpandAdd.hpp:48-66): a first operand of the destination's shape is the
+    // matrix, whatever the second looks like (a full-size column-major tile may carry the per-row values in its first
+    // column: demos/cpu/mla_attention_demo); only otherwise is the first operand the per-row one
+    if constexpr (!kIsRowOperand<A, DstT>)
         row_expand<op, false>(dst, src0, src1);
     else
         row_expand<op, true>(dst, src1, src0);

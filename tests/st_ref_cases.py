@@ -19,7 +19,7 @@ ST_DIR = os.path.join(ROOT, "oracle", "_ref", "st")
 CTYPE = {"float": (np.float32, C.c_float), "int": (np.int32, C.c_int32), "short": (np.int16, C.c_int16),
          "unsigned short": (np.uint16, C.c_uint16), "signed char": (np.int8, C.c_int8), "unsigned char": (np.uint8, C.c_uint8),
          "unsigned int": (np.uint32, C.c_uint32), "long": (np.int64, C.c_int64),
-         "_Float16": (np.float16, C.c_uint16)}
+         "_Float16": (np.float16, C.c_uint16), "unsigned long": (np.uint64, C.c_uint64)}
 CTYPE.update({"int32_t": CTYPE["int"], "int16_t": CTYPE["short"], "uint16_t": CTYPE["unsigned short"], "uint32_t": CTYPE["unsigned int"],
               "int8_t": CTYPE["signed char"], "uint8_t": CTYPE["unsigned char"]})
 
@@ -739,6 +739,33 @@ SPECS["tmrgsort:topk"] = dict(fn="LanchTMrgsortTopK", lib="tmrgsort", form="topk
                               tail=_MRG_T + r"(?P<tc>\d+), (?P<topk>\d+)>\((?:float\*, ){2}void\*\)")
 
 
+# ---- TSTORE (with the TLOAD in front of it): LaunchTStore<format, T, g0..g4, w0..w4>(T *out, T *src): the [g0..g4] corner of
+# a dense [w0..w4] array goes through a Vec tile and back to the same places of out; format 0 = ND (rows stacked), 1 = DN
+# (column-major tile, the last two dimensions swapped in memory), 2 = NZ (boxed tile) (tstore_kernel.cpp:19-117)
+def plan_store(test, spec, m):
+    dt, _ = _elem(m.group("T"), False)
+    fmt = int(m.group("fmt"))
+    g = [int(m.group("g%d" % k)) for k in range(5)]
+    w = [int(m.group("w%d" % k)) for k in range(5)]
+    total = int(np.prod(w))
+    strides = [w[1] * w[2] * w[3] * w[4], w[2] * w[3] * w[4], w[3] * w[4], w[4], 1]
+    if fmt == 1:
+        strides[3], strides[4] = 1, w[3]
+    idx = np.indices(g).reshape(5, -1)
+    offsets = (idx * np.array(strides)[:, None]).sum(axis=0)
+
+    def expect(a):
+        out = np.full(total, 77, dtype=dt)
+        out[offsets] = a[0].reshape(-1)[offsets]
+        return [out[None, :]]
+    return _plan(spec, [(dt, (1, total))], [(dt, (1, total), "bits")], [(1, total)], expect)
+
+
+SPECS["tstore"] = dict(fn="LaunchTStore", planner=plan_store, inputs="bits",
+                       tail=r"<(?P<fmt>\d), (?P<T>[a-z ]+)" + "".join(r", (?P<g%d>\d+)" % k for k in range(5)) + "".join(r", (?P<w%d>\d+)" % k for k in range(5)) +
+                            r">\((?:[a-z ]+\*, ){2}void\*\)")
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
@@ -786,6 +813,8 @@ def draw(rng, dt, shape, kind, j):
     elif kind in ("rem", "rempos"):
         x = rng.integers(0 if kind == "rempos" else max(info.min, -1000), min(info.max, 1000), size=shape)
     elif kind == "bits":
+        if dt.itemsize == 8:
+            return rng.integers(0, 2**63 - 1, size=shape, dtype=np.int64).view(dt) ^ dt.type(0x5A5A)
         x = rng.integers(info.min, info.max, size=shape, endpoint=True)
     elif kind == "pos":
         x = rng.integers(1, 100, size=shape)

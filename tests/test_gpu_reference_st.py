@@ -30,7 +30,7 @@ def test_reference_st_kernel(test, mangled, demangled):
     lib = C.CDLL(os.path.join(S.ST_DIR, S.lib_of(test) + ".so"))
     fn = getattr(lib, mangled)
     dev = "cuda:0"
-    view = {np.dtype(np.float16): np.int16, np.dtype(np.uint16): np.int16, np.dtype(np.uint32): np.int32}
+    view = {np.dtype(np.float16): np.int16, np.dtype(np.uint16): np.int16, np.dtype(np.uint32): np.int32, np.dtype(np.uint64): np.int64}
 
     def to_dev(a):
         return torch.from_numpy(a.view(view.get(a.dtype, a.dtype))).to(dev)
