@@ -353,7 +353,8 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
     static_assert(SrcT::isRowMajor && SrcT::Loc == TileType::Vec && DstT::Loc == TileType::Vec,
                   "[PTO][SA] row reduction: row-major Vec source");
     static_assert(SrcT::Cols % kVecChunk == 0, "[PTO][SA] row reduction: cols must be a multiple of 8");
-    static_assert(SrcT::Rows == DstT::Rows, "[PTO][SA] row reduction: row counts differ");
+    // (the destination may have another row count than the source, e.g. a [8, 1] column for one valid row of a [1, 8]
+    // source: tests/npu/a2a3/src/st/testcase/trowprod/trowprod_kernel.cpp:30-31; the valid rows must fit both)
     using A = float;
     using S = typename SrcT::Storage;
     constexpr int CPR = SrcT::Cols / kVecChunk; // chunks per row
@@ -379,7 +380,7 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
         if (e < DstT::Numel) {
             int r, c;
             elem_rc<DstT>(e, r, c);
-            if (c == 0 && r < vr) {
+            if (c == 0 && r < vr && r < SrcT::Rows) {
                 A acc = part[r * CPR];
                 for (int j = 1; j < CPR; ++j) {
                     const A v = part[r * CPR + j];

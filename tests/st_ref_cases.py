@@ -202,7 +202,7 @@ def _elementwise_plan(spec, dtype, buffers, valid, scalar, scalar_first=False):
 # validRows, cols, validCols[, srcDivScalar]> (tadds_kernel.cpp:17-45, tdivs_kernel.cpp:17-48): output buffer [dstRows,
 # dstCols], input [rows, cols], the scalar converted from float inside the launcher
 CASE_SCALAR = r"<(?P<case>\d+)u>\(void\*, void\*, float, ihipStream_t\*\)"
-SRC_TYPES = {"float": "float", "half": "unsigned short", "aclFloat16": "unsigned short", "int32_t": "int", "int16_t": "short",
+SRC_TYPES = {"float": "float", "half": "unsigned short", "__fp16": "unsigned short", "aclFloat16": "unsigned short", "int32_t": "int", "int16_t": "short",
              "uint16_t": "unsigned short", "uint32_t": "unsigned int", "int8_t": "signed char", "uint8_t": "unsigned char"}
 
 
@@ -766,6 +766,68 @@ SPECS["tstore"] = dict(fn="LaunchTStore", planner=plan_store, inputs="bits",
                             r">\((?:[a-z ]+\*, ){2}void\*\)")
 
 
+# ---- TCOLEXPAND: launchTCOLEXPAND<T, srcRows, srcCols, srcValidCols, dstRows, dstCols, dstValidRows, dstValidCols>: row 0 of
+# the source down the valid rows of the destination (tcolexpand_kernel.cpp:17-46)
+def plan_colexpand(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    sr, sc, dr, dc, dvr, dvc = (int(m.group(k)) for k in ("sr", "sc", "dr", "dc", "dvr", "dvc"))
+    return _plan(spec, [(dt, (dr, dc))], [(dt, (sr, sc))], [(dvr, dvc)], lambda a: [np.repeat(a[0][:1, :dvc], dvr, axis=0)])
+
+
+# ---- TTRANS: LaunchTTRANS<T, tileRows, tileCols, validRows, validCols>: out [tileCols, tileRows] gets the transpose of the
+# valid corner of src [tileRows, tileCols] (ttrans_kernel.cpp:17-66)
+def plan_trans(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    tr, tc, vr, vc = (int(m.group(k)) for k in ("tr", "tc", "vr", "vc"))
+    return _plan(spec, [(dt, (tc, tr))], [(dt, (tr, tc))], [(vc, vr)], lambda a: [a[0][:vr, :vc].T])
+
+
+# ---- TROWPROD, numbered cases -> run<T, dstRows, srcRows, validRows, srcCols, srcValidCols>: the product of every valid row as
+# a vector (trowprod_kernel.cpp:17-48)
+def plan_rowprod(test, spec, m):
+    t = case_entry(test, m)["targs"]
+    dt, _ = _elem(SRC_TYPES[t[0]], True)
+    drows, srows, vr, sc, svc = (int(x) for x in t[1:6])
+    return _plan(spec, [(dt, (1, drows))], [(dt, (srows, sc), "near1")], [(1, vr)],
+                 lambda a: [np.prod(a[0][:vr, :svc].astype(np.float64), axis=1)[None, :]])
+
+
+# ---- TPARTADD / TPARTMUL: LaunchTPartAdd<T, dstRows, dstCols, src0Rows, src0Cols, src1Rows, src1Cols> (dense buffers of
+# exactly those extents, tpartadd_kernel.cpp:17-47); TPARTMAX / TPARTMIN: the same six extents followed by the six tile
+# extents (tpartmax_kernel.cpp:17-52).  Where both sources have an element the operation, where one has it that element.
+def plan_part(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    dr, dc, ar, ac, br, bc = (int(m.group(k)) for k in ("dr", "dc", "ar", "ac", "br", "bc"))
+    op = spec["op"]
+
+    def expect(a):
+        out = np.zeros((dr, dc), dtype=np.float64 if dt.kind == "f" else dt)
+        in0 = np.zeros((dr, dc), dtype=bool)
+        in1 = np.zeros((dr, dc), dtype=bool)
+        in0[:ar, :ac] = True
+        in1[:br, :bc] = True
+        x0 = np.zeros((dr, dc), dtype=out.dtype)
+        x1 = np.zeros((dr, dc), dtype=out.dtype)
+        x0[:min(ar, dr), :min(ac, dc)] = a[0][:dr, :dc]
+        x1[:min(br, dr), :min(bc, dc)] = a[1][:dr, :dc]
+        out = np.where(in0 & in1, op(x0, x1), np.where(in0, x0, np.where(in1, x1, 0)))
+        return [out]
+    return _plan(spec, [(dt, (dr, dc))], [(dt, (ar, ac)), (dt, (br, bc))], [(dr, dc)], expect)
+
+
+PART6 = TAIL(["dr", "dc", "ar", "ac", "br", "bc"], 3)
+PART12 = TAIL(["dr", "dc", "ar", "ac", "br", "bc", "t0", "t1", "t2", "t3", "t4", "t5"], 3)[:-len(r"void\*\)")] + r"ihipStream_t\*\)"
+SPECS.update({
+    "tcolexpand": dict(fn="launchTCOLEXPAND", tail=TAIL(["sr", "sc", "svc", "dr", "dc", "dvr", "dvc"], 2), planner=plan_colexpand, inputs="any"),
+    "ttrans": dict(fn="LaunchTTRANS", tail=TAIL(["tr", "tc", "vr", "vc"], 2), planner=plan_trans, inputs="any"),
+    "trowprod": dict(fn="launchTROWPRODTestCase", tail=CASE_UNARY, planner=plan_rowprod, inputs="near1", tol=REDUCE_TOL),
+    "tpartadd": dict(fn="LaunchTPartAdd", tail=PART6, planner=plan_part, inputs="any", op=lambda a, b: a + b),
+    "tpartmul": dict(fn="LaunchTPartMul", tail=PART6, planner=plan_part, inputs="any", op=lambda a, b: a * b),
+    "tpartmax": dict(fn="LaunchTPartMax", tail=PART12, planner=plan_part, inputs="any", op=np.maximum),
+    "tpartmin": dict(fn="LaunchTPartMin", tail=PART12, planner=plan_part, inputs="any", op=np.minimum),
+})
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
@@ -785,6 +847,8 @@ def draw(rng, dt, shape, kind, j):
         return rng.integers(lo, hi, size=shape, endpoint=True).astype(dt)
     if kind == "unit":
         return rng.uniform(-1.0, 1.0, size=shape).astype(dt)
+    if kind == "near1":
+        return rng.uniform(0.9, 1.1, size=shape).astype(dt)
     if kind == "scores":                      # few distinct values: many equal scores, whose order the index decides
         return (rng.integers(-20, 20, size=shape) * 0.5).astype(dt)
     if kind == "index":
