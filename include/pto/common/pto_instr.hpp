@@ -10,6 +10,8 @@
 #include "pto/gfx950/fifo_ops.hpp"
 #include "pto/gfx950/sort_ops.hpp"
 #include "pto/gfx950/matmul_any.hpp"
+#include "pto/gfx950/fixpipe.hpp"
+#include "pto/gfx950/debug_ops.hpp"
 
 namespace pto {
 
@@ -94,6 +96,7 @@ PTO_INST RecordEvent TMATMUL_BIAS(C &c, A &a, B &b, Bias &bias, Ev &... ev)
 {
     TSYNC(ev...);
     TMATMUL_BIAS_IMPL(c, a, b, bias);
+    detail::UbCommit(c);
     return {};
 }
 template <typename C, typename A, typename B, typename... Ev>
@@ -101,13 +104,16 @@ PTO_INST RecordEvent TGEMV(C &c, A &a, B &b, Ev &... ev)
 {
     TSYNC(ev...);
     TGEMV_IMPL(c, a, b);
+    detail::UbCommit(c);
     return {};
 }
 template <typename C, typename A, typename B, typename... Ev>
 PTO_INST RecordEvent TGEMV_ACC(C &cOut, C &cIn, A &a, B &b, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(cIn);
     TGEMV_ACC_IMPL(cOut, cIn, a, b);
+    detail::UbCommit(cOut);
     return {};
 }
 template <typename C, typename A, typename B, typename Bias, typename... Ev,
@@ -116,6 +122,7 @@ PTO_INST RecordEvent TGEMV_BIAS(C &c, A &a, B &b, Bias &bias, Ev &... ev)
 {
     TSYNC(ev...);
     TGEMV_BIAS_IMPL(c, a, b, bias);
+    detail::UbCommit(c);
     return {};
 }
 PTO_FRONT(TCVT, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C RoundMode mode, (dst, src, mode))
@@ -249,6 +256,55 @@ PTO_INST RecordEvent TSELS(D &dst, M &mask, S &src, typename S::DType scalar, Ev
     return {};
 }
 PTO_FRONT(TFILLPAD, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TFILLPAD_INPLACE, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TFILLPAD_EXPAND, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+PTO_FRONT(TPACK, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
+// TPREFETCH (pto_instr.hpp:135-140 of the reference; cpu/TPrefetch.hpp copies the region into the tile): a TLOAD here
+PTO_FRONT(TPREFETCH, typename TileT PTO_C typename G, TileT &dst PTO_C G &src, (dst, src))
+// TQUANT, the row-scale form (pto_instr.hpp:1503-1510 of the reference)
+template <auto quant, typename D, typename S, typename P, typename... Ev>
+PTO_INST RecordEvent TQUANT(D &dst, S &src, P &scale, P *offset = nullptr, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src, scale);
+    if (offset != nullptr)
+        detail::UbFetch(*offset);
+    TQUANT_IMPL<quant>(dst, src, scale, offset);
+    detail::UbCommit(dst);
+    detail::UbCommit(src);
+    return {};
+}
+// TDEQUANT (pto_instr.hpp:1407-1415 of the reference)
+template <typename D, typename S, typename P, typename... Ev>
+PTO_INST RecordEvent TDEQUANT(D &dst, S &src, P &scale, P &offset, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src, scale, offset);
+    TDEQUANT_IMPL(dst, src, scale, offset);
+    detail::UbCommit(dst);
+    return {};
+}
+// TGEMV_MX (pto_instr.hpp:341-398 of the reference): TMATMUL_MX on a left operand with one valid row
+template <typename C, typename A, typename SA, typename B, typename SB, typename... Ev>
+PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TGEMV_MX(C &c, A &a, SA &sa, B &b, SB &sb, Ev &... ev)
+{
+    return TMATMUL_MX(c, a, sa, b, sb, ev...);
+}
+template <typename C, typename A, typename SA, typename B, typename SB, typename... Ev>
+PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TGEMV_MX(C &cOut, C &cIn, A &a, SA &sa, B &b, SB &sb, Ev &... ev)
+{
+    return TMATMUL_MX(cOut, cIn, a, sa, b, sb, ev...);
+}
+// TPRINT (pto_instr.hpp:316-322 of the reference): a Vec tile or a GlobalTensor written to the host's stdout
+template <typename T, typename... Ev>
+PTO_INST RecordEvent TPRINT(T &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    if constexpr (is_tile_data_v<T>)
+        detail::UbFetch(src);
+    TPRINT_IMPL(src);
+    return {};
+}
 PTO_FRONT(TPUSH, typename P PTO_C typename T PTO_C typename F, P &prod PTO_C T &tile PTO_C F &fifo, (prod, tile, fifo))
 PTO_FRONT(TPOP, typename P PTO_C typename T PTO_C typename F, P &cons PTO_C T &tile PTO_C F &fifo, (cons, tile, fifo))
 #undef PTO_FRONT
@@ -305,6 +361,10 @@ PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
     detail::UbFetch(dst, src);
     if constexpr (S::Loc == TileType::Acc && D::Loc == TileType::Vec)
         TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    else if constexpr (S::Loc == TileType::Acc && D::Loc == TileType::Mat)
+        detail::tmov_fix<relu>(dst, src, detail::FixNone{});
+    else if constexpr (S::Loc == TileType::Mat && D::Loc == TileType::Scaling)
+        TMOV_MAT2SCALING_IMPL(dst, src);
     else if constexpr ((S::Loc == TileType::Acc || S::Loc == TileType::Vec) && (D::Loc == TileType::Left || D::Loc == TileType::Right))
         TMOV_TO_OPERAND_IMPL(dst, src); // the chained matmuls of the Auto-mode programs
     else
@@ -325,6 +385,107 @@ PTO_INST RecordEvent TMOV(D &dst, S &src, Ev &... ev)
 {
     TSYNC(ev...);
     TMOV_ACC2VEC_IMPL<relu>(dst, src);
+    return {};
+}
+
+// The accumulator's way out with a conversion (pto/gfx950/fixpipe.hpp): one quantisation word for the tile, or one per
+// column in a Scaling tile (pto_instr.hpp:196-236, 625-660, 716-752, 893-915 of the reference)
+template <typename D, typename S, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TMOV(D &dst, S &src, uint64_t preQuantScalar, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tmov_fix<relu>(dst, src, detail::FixScalar{preQuantScalar});
+    return {};
+}
+template <typename D, typename S, typename Fp, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TMOV_FP(D &dst, S &src, Fp &fp, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tmov_fix<relu>(dst, src, detail::fix_vector(fp));
+    return {};
+}
+template <typename D, typename S, ReluPreMode relu, typename... Ev>
+PTO_INST RecordEvent TEXTRACT(D &dst, S &src, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::textract_fix<relu>(dst, src, idxRow, idxCol, detail::FixNone{});
+    return {};
+}
+template <typename D, typename S, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TEXTRACT(D &dst, S &src, uint64_t preQuantScalar, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::textract_fix<relu>(dst, src, idxRow, idxCol, detail::FixScalar{preQuantScalar});
+    return {};
+}
+template <typename D, typename S, typename Fp, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TEXTRACT_FP(D &dst, S &src, Fp &fp, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::textract_fix<relu>(dst, src, idxRow, idxCol, detail::fix_vector(fp));
+    return {};
+}
+template <typename D, typename S, typename... Ev>
+PTO_INST RecordEvent TINSERT(D &dst, S &src, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tinsert_fix<ReluPreMode::NoRelu>(dst, src, idxRow, idxCol, detail::FixNone{});
+    return {};
+}
+template <typename D, typename S, ReluPreMode relu, typename... Ev>
+PTO_INST RecordEvent TINSERT(D &dst, S &src, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tinsert_fix<relu>(dst, src, idxRow, idxCol, detail::FixNone{});
+    return {};
+}
+template <typename D, typename S, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TINSERT(D &dst, S &src, uint64_t preQuantScalar, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tinsert_fix<relu>(dst, src, idxRow, idxCol, detail::FixScalar{preQuantScalar});
+    return {};
+}
+template <typename D, typename S, typename Fp, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TINSERT_FP(D &dst, S &src, Fp &fp, uint16_t idxRow, uint16_t idxCol, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tinsert_fix<relu>(dst, src, idxRow, idxCol, detail::fix_vector(fp));
+    return {};
+}
+template <typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone, ReluPreMode relu = ReluPreMode::NoRelu, typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, uint64_t preQuantScalar, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tstore_fix<TileT, G, atomic, relu>(dst, src, detail::FixScalar{preQuantScalar});
+    return {};
+}
+template <STPhase Phase, typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone, ReluPreMode relu = ReluPreMode::NoRelu,
+          typename... Ev>
+PTO_INST RecordEvent TSTORE(G &dst, TileT &src, uint64_t preQuantScalar, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tstore_fix<TileT, G, atomic, relu>(dst, src, detail::FixScalar{preQuantScalar});
+    return {};
+}
+template <typename TileT, typename G, typename Fp, AtomicType atomic = AtomicType::AtomicNone, ReluPreMode relu = ReluPreMode::NoRelu,
+          typename... Ev>
+PTO_INST RecordEvent TSTORE_FP(G &dst, TileT &src, Fp &fp, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    detail::tstore_fix<TileT, G, atomic, relu>(dst, src, detail::fix_vector(fp));
     return {};
 }
 

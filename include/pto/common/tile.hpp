@@ -121,13 +121,18 @@ constexpr int cdiv(int a, int b) { return (a + b - 1) / b; }
 struct Empty {};
 
 template <TileType Loc, typename T, int Rows, int Cols>
-struct TileStorage { // Bias / Scaling / unsupported locations: no storage
+struct TileStorage { // unsupported locations: no storage
     Empty none;
 };
 
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Mat, T, Rows, Cols> {
     uint32_t lds = 0; // byte offset into the workgroup's dynamic LDS
+};
+
+template <typename T, int Rows, int Cols>
+struct TileStorage<TileType::Scaling, T, Rows, Cols> {
+    uint32_t fb = 0; // byte offset into the table of quantisation words (pto/gfx950/fixpipe.hpp)
 };
 
 // 8-bit MX operands (v_mfma_scale_f32_32x32x64_f8f6f4): a fragment is 32 rows x 64 k; lane l holds row l % 32 and the
@@ -327,6 +332,12 @@ struct Tile {
     Tile *origin_ = nullptr; // register tiles: set in a copy, the tile it was copied from (values go back on destruction)
     // the object itself is an address: Mat tiles, and Vec tiles of a translation unit that keeps them in memory
     static constexpr bool inMemory = Loc_ == TileType::Vec && detail::kVecTilesInMemory;
+    // In such a translation unit an Acc tile that was given an address is an address too: every instruction that writes
+    // it stores its [Rows, Cols] image (row-major) there and every instruction that reads it loads it from there, so that
+    // another Acc tile object TASSIGNed to the same address sees the accumulator (the reference's test kernels multiply
+    // in one function and declare the tile again in the next: tests/npu/a2a3/src/st/testcase/tmov_acc2mat).  The values
+    // still live in registers in between; the object is not a handle.
+    static constexpr bool accInMemory = Loc_ == TileType::Acc && detail::kVecTilesInMemory;
     static constexpr bool isHandle = Loc_ == TileType::Mat || inMemory;
 #if defined(PTO_VEC_TILES_IN_MEMORY)
     DType *mem_ = nullptr; // Vec tiles: element 0 of the tile in the unified buffer (nullptr: not assigned, registers only)

@@ -44,6 +44,12 @@ PTO_DEV void UbFetchTile(TileT &t)
                     t.S().v[s][i] = p[e];
             });
         }
+    } else if constexpr (TileT::accInMemory) { // the whole [Rows, Cols] image, row-major
+        if (t.mem_ != nullptr) {
+            using T = typename TileT::DType;
+            const T *p = t.mem_;
+            for_each_elem(t, [&](int r, int c, T, bool) { return p[r * TileT::Cols + c]; });
+        }
     }
 #else
     (void)t;
@@ -65,6 +71,17 @@ PTO_DEV void UbCommitTile(TileT &t)
             });
         }
         UbSyncPoint();
+    } else if constexpr (TileT::accInMemory) {
+        if (t.mem_ != nullptr) {
+            using T = typename TileT::DType;
+            T *p = t.mem_;
+            for_each_elem(t, [&](int r, int c, T v, bool owner) {
+                if (owner)
+                    p[r * TileT::Cols + c] = v;
+                return v;
+            });
+            UbSyncPoint();
+        }
     }
 #else
     (void)t;

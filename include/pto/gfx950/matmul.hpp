@@ -20,6 +20,8 @@ template <typename TileT>
 constexpr bool is_plain_v = is_plain_storage<typename TileT::Storage>::value;
 template <typename TileT>
 constexpr bool is_fully_valid_v = TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols;
+template <typename TileT, typename F>
+PTO_DEV void for_each_elem(TileT &t, F &&fn);
 template <bool kZeroInit, typename AccT, typename LeftT, typename RightT>
 PTO_DEV void mad_any(AccT &out, AccT &in, LeftT &a, RightT &b);
 template <typename AccT, typename BiasT>
@@ -32,6 +34,19 @@ template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu>
 PTO_DEV void tstore_any(G &dst, TileT &src);
 template <typename TileT>
 PTO_DEV void zero_outside_valid(TileT &t);
+// the conversion on the accumulator's way out (pto/gfx950/fixpipe.hpp): none but the cast, one quantisation word for the
+// tile, one word per column
+struct FixNone {};
+struct FixScalar {
+    uint64_t q;
+};
+struct FixVector {
+    const uint64_t *table;
+};
+template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu, typename P>
+PTO_DEV void tstore_fix(G &dst, TileT &src, const P &p);
+template <ReluPreMode relu, typename DstT, typename SrcT, typename P>
+PTO_DEV void textract_fix(DstT &dst, SrcT &src, int idxRow, int idxCol, const P &p);
 template <typename DstT, typename SrcT>
 PTO_DEV void tfillpad_mat(DstT &dst, SrcT &src);
 

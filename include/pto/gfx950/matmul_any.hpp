@@ -206,7 +206,7 @@ PTO_DEV void tstore_any(G &dst, TileT &src)
                 y = y < 0 ? 0 : y;
             GT *p = gm + (int64_t)r * st_r + (int64_t)c * st_c;
             if constexpr (atomic == AtomicType::AtomicAdd)
-                atomicAdd(p, store_cast<GT>(y));
+                atomic_add(p, store_cast<GT>(y));
             else
                 *p = store_cast<GT>(y);
         }

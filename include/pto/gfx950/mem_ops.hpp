@@ -180,6 +180,8 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
             __builtin_trap(); // the run-time form of the reference's PTO_ASSERT (debug builds only)
 #endif
         obj.st.lds = off;
+    } else if constexpr (T::Loc == TileType::Scaling) {
+        obj.st.fb = (uint32_t)(uintptr_t)addr; // offset into the table of quantisation words
     } else {
 #if defined(PTO_VEC_TILES_IN_MEMORY)
         if constexpr (T::inMemory) {
@@ -187,6 +189,12 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
             const uint64_t a = (uint64_t)(uintptr_t)addr;
             obj.mem_ = a < (uint64_t)PTO_UB_BYTES ? reinterpret_cast<typename T::DType *>(detail::ub_base() + a) :
                                                    reinterpret_cast<typename T::DType *>((uintptr_t)a);
+            return;
+        } else if constexpr (T::accInMemory) {
+            const uint64_t a = (uint64_t)(uintptr_t)addr;
+            obj.mem_ = a + sizeof(typename T::DType) * T::Numel <= (uint64_t)(PTO_UB_BYTES - PTO_ACC_ARENA_OFFSET) ?
+                           reinterpret_cast<typename T::DType *>(detail::ub_base() + PTO_ACC_ARENA_OFFSET + a) :
+                           nullptr; // beyond the arena: the tile stays in registers only
             return;
         }
 #endif
@@ -480,6 +488,13 @@ PTO_DEV void TLOAD_IMPL(TileT &dst, G &src)
         static_assert(TileT::Loc == TileType::Mat, "[PTO][SA] TLOAD: destination must be a Mat or Vec tile");
 }
 
+// TPREFETCH: the region ends up in the tile (cpu/TPrefetch.hpp:18-41), as after a TLOAD
+template <typename TileT, typename G>
+PTO_DEV void TPREFETCH_IMPL(TileT &dst, G &src)
+{
+    TLOAD_IMPL(dst, src);
+}
+
 // ----------------------------------------------------------------- TEXTRACT
 // dst[i,j] = src[idxRow+i, idxCol+j].  Mat -> Left / Right: one ds_read_b128 per row block and k step, in the
 // MFMA operand layout (lane l: row/col l % kMfmaM, the 16-byte chunk l / kMfmaM of the step: 8 fp16 / bf16, 16 int8 or
@@ -639,7 +654,10 @@ PTO_DEV void textract_frag(DstT &dst, SrcT &src, uint32_t idxRow, uint32_t idxCo
 template <typename DstT, typename SrcT>
 PTO_DEV void TEXTRACT_IMPL(DstT &dst, SrcT &src, uint32_t idxRow = 0, uint32_t idxCol = 0)
 {
-    if constexpr (DstT::Loc == TileType::ScaleLeft || DstT::Loc == TileType::ScaleRight) {
+    if constexpr (SrcT::Loc == TileType::Acc && DstT::Loc == TileType::Mat) {
+        detail::textract_fix<ReluPreMode::NoRelu>(dst, src, (int)idxRow, (int)idxCol, detail::FixNone{}); // pto/gfx950/fixpipe.hpp
+        return;
+    } else if constexpr (DstT::Loc == TileType::ScaleLeft || DstT::Loc == TileType::ScaleRight) {
         constexpr bool left = DstT::Loc == TileType::ScaleLeft;
         if constexpr (SrcT::Loc == TileType::Mat) {
             detail::textract_scale_mat(dst, src, left ? idxRow : idxCol, left ? idxCol : idxRow);
@@ -693,6 +711,34 @@ PTO_DEV D store_cast(S v)
         return static_cast<D>(v); // fp32 -> fp16 / bf16: hardware round-to-nearest-even
 }
 
+// *p += v for any element type: 32-bit types with the hardware's atomic, narrower ones with a compare-and-swap loop on
+// the aligned 32-bit word that holds them (the reference's fix pipe accumulates into fp16, bf16 and 8-bit results too:
+// tests/npu/a2a3/src/st/testcase/tstore_acc2gm)
+template <typename D>
+PTO_DEV void atomic_add(D *p, D v)
+{
+    if constexpr (std::is_same_v<D, float> || std::is_same_v<D, int32_t> || std::is_same_v<D, uint32_t>) {
+        atomicAdd(p, v);
+    } else {
+        static_assert(sizeof(D) < 4, "[PTO][SA] atomic add: 8-, 16- or 32-bit elements");
+        using Bits = std::conditional_t<sizeof(D) == 2, uint16_t, uint8_t>;
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p);
+        unsigned int *word = reinterpret_cast<unsigned int *>(a & ~(uintptr_t)3);
+        const unsigned shift = (unsigned)(a & 3) * 8;
+        const unsigned int mask = (unsigned int)(Bits)~(Bits)0 << shift;
+        unsigned int seen = *word, want;
+        do {
+            const D cur = __builtin_bit_cast(D, (Bits)((seen & mask) >> shift));
+            const D sum = (D)(cur + v);
+            want = (seen & ~mask) | ((unsigned int)__builtin_bit_cast(Bits, sum) << shift);
+            const unsigned int prev = atomicCAS(word, seen, want);
+            if (prev == seen)
+                break;
+            seen = prev;
+        } while (true);
+    }
+}
+
 // Acc fragments -> GM.  MFMA result layout: lane l, register v holds row acc_elem_row(v) + acc_lane_row(l),
 // column l % kMfmaM of the block (32 x 32: row 8*(v/4) + 4*(l/32) + v%4).
 template <typename TileT, typename G, AtomicType atomic, ReluPreMode relu = ReluPreMode::NoRelu>
@@ -721,7 +767,7 @@ PTO_DEV void tstore_acc(G &dst, TileT &src)
                     if constexpr (relu == ReluPreMode::NormalRelu)
                         x = x < 0 ? 0 : x; // before the conversion, as the fix pipe does (a2a3/TStore.hpp:328)
                     if constexpr (atomic == AtomicType::AtomicAdd)
-                        atomicAdd(p, store_cast<GT>(x));
+                        atomic_add(p, store_cast<GT>(x));
                     else
                         *p = store_cast<GT>(x);
                 }
@@ -803,8 +849,7 @@ PTO_DEV void tstore_mat(G &dst, TileT &src)
     for (int e = hw::tid(); e < TileT::Numel; e += kBlockThreads) {
         const int r = e / TileT::Cols, c = e % TileT::Cols;
         if (r < vr && c < vc)
-            gm[(int64_t)r * dst.GetStride(3) + (int64_t)c * dst.GetStride(4)] =
-                *reinterpret_cast<const T *>(lds + Geo::elem_off(r, c));
+            gm[gm_elem_offset(dst, r, c)] = *reinterpret_cast<const T *>(lds + Geo::elem_off(r, c));
     }
 }
 
@@ -814,7 +859,9 @@ template <typename TileT, typename G, AtomicType atomic = AtomicType::AtomicNone
 PTO_DEV void TSTORE_IMPL(G &dst, TileT &src)
 {
     static_assert(relu == ReluPreMode::NoRelu || TileT::Loc == TileType::Acc, "[PTO][SA] TSTORE: ReLU applies to Acc tiles");
-    if constexpr (TileT::Loc == TileType::Acc && detail::is_plain_v<TileT>) {
+    if constexpr (TileT::Loc == TileType::Acc && G::layout == Layout::NZ) {
+        detail::tstore_fix<TileT, G, atomic, relu>(dst, src, detail::FixNone{}); // pto/gfx950/fixpipe.hpp
+    } else if constexpr (TileT::Loc == TileType::Acc && detail::is_plain_v<TileT>) {
         detail::tstore_any<TileT, G, atomic, relu>(dst, src);
     } else if constexpr (TileT::Loc == TileType::Acc) {
         detail::tstore_acc<TileT, G, atomic, relu>(dst, src);

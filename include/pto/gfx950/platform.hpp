@@ -190,6 +190,14 @@ PTO_DEV int64_t get_subblockdim() { return 1; }
 PTO_DEV int64_t get_coreid() { return static_cast<int64_t>(blockIdx.x); }
 PTO_DEV int64_t get_sys_cnt() { return static_cast<int64_t>(wall_clock64()); }
 
+// ---- cache maintenance of the Ascend scalar core (the preamble of the reference's tfillpad / tload test kernels:
+// tests/npu/a2a3/src/st/testcase/tfillpad/tfillpad_kernel.cpp:124-139): a data barrier, an instruction-cache preload and
+// its status.  A wave's own stores are visible to its later loads, and there is no instruction cache to warm by hand.
+enum dsb_mode_t { DSB_ALL = 0, DSB_DDR, DSB_UB };
+PTO_DEV void dsb(dsb_mode_t) { __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup"); }
+PTO_DEV void preload(const void *, int64_t) {}
+PTO_DEV int64_t get_icache_prl_st() { return 0; }
+
 // ---- cross-core flags of the Cube / Vec kernels (fa_performance_kernel.cpp:617, TPush.hpp:140-160 of the reference) ----
 // On Ascend a Cube core and its Vec cores are separate instruction streams that signal each other through FFTS flags.
 // Here one workgroup runs both roles in program order, so the producer's code has always run before the consumer's: what

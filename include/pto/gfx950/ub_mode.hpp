@@ -16,6 +16,11 @@
 #ifndef PTO_UB_BYTES
 #define PTO_UB_BYTES (512 * 1024)
 #endif
+// Acc tiles that were given an address keep their image in the upper part of the same arena: address a of the
+// accumulator memory is byte PTO_ACC_ARENA_OFFSET + a of the workgroup's unified buffer
+#ifndef PTO_ACC_ARENA_OFFSET
+#define PTO_ACC_ARENA_OFFSET (256 * 1024)
+#endif
 
 namespace pto {
 namespace detail {

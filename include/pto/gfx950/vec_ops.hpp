@@ -13,6 +13,11 @@
 #include "pto/common/global_tensor.hpp"
 #include "pto/common/tile.hpp"
 
+// Every tile instruction rounds on its own, as the reference's do: a multiplication in one instruction and an addition in
+// the next (TMUL then TADD, the two halves of TQUANT) must not be contracted into one fused multiply-add once both are
+// inlined into a kernel.  Contraction is switched off for the instruction bodies of this header and back to hipcc's
+// default for device code at its end.
+#pragma clang fp contract(off)
 namespace pto {
 namespace detail {
 
@@ -608,3 +613,4 @@ PTO_DEV void MGATHER_ROWS_IMPL(DstT &dst, G &table, IdxT &rowIdx, int tableRows)
 }
 
 } // namespace pto
+#pragma clang fp contract(fast)

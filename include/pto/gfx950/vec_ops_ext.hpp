@@ -5,6 +5,7 @@
 #pragma once
 #include "pto/gfx950/vec_ops.hpp"
 
+#pragma clang fp contract(off) // as in vec_ops.hpp: instructions round on their own
 namespace pto {
 
 // ------------------------------------------------------------------ unary
@@ -273,6 +274,102 @@ PTO_DEV void TFILLPAD_IMPL(DstT &dst, SrcT &src)
     }
 }
 
+// TFILLPAD_INPLACE: source and destination are the same buffer on the NPU; here the destination keeps the source's
+// elements inside the source's valid region like TFILLPAD (npu/a2a3/TFillPad.hpp:264-271).
+template <typename DstT, typename SrcT>
+PTO_DEV void TFILLPAD_INPLACE_IMPL(DstT &dst, SrcT &src)
+{
+    TFILLPAD_IMPL(dst, src);
+}
+// TFILLPAD_EXPAND: the destination has at least the source's rows and columns (npu/a2a3/TFillPad.hpp:273-280)
+template <typename DstT, typename SrcT>
+PTO_DEV void TFILLPAD_EXPAND_IMPL(DstT &dst, SrcT &src)
+{
+    static_assert(DstT::Rows >= SrcT::Rows && DstT::Cols >= SrcT::Cols && sizeof(typename DstT::DType) == sizeof(typename SrcT::DType),
+                  "[PTO][SA] TFILLPAD_EXPAND: the destination is at least as large as the source, one element size");
+    static_assert(DstT::PadVal != PadValue::Null, "[PTO][SA] TFILLPAD: the destination tile needs a pad value");
+    using T = typename DstT::DType;
+    const T pad = detail::pad_value<T>(DstT::PadVal);
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    detail::Conformed<DstT, SrcT> c(src);
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        int r, col;
+        detail::elem_rc<DstT>(e, r, col);
+        if (e < DstT::Numel)
+            dst.S().v[s][i] = (r < vr && col < vc) ? __builtin_bit_cast(T, c.S().v[s][i]) : pad;
+    });
+}
+
+// TPACK: every element cut to the low bits that fit the narrower destination type: 32 -> 16, 32 -> 8, 16 -> 8 bits
+// (npu/a5/TPack.hpp:21-72: a store that keeps the low half / quarter of every register element)
+template <typename DstT, typename SrcT>
+PTO_DEV void TPACK_IMPL(DstT &dst, SrcT &src)
+{
+    using T = typename DstT::DType;
+    using U = typename SrcT::DType;
+    static_assert(sizeof(U) > sizeof(T) && (sizeof(U) == 4 || sizeof(U) == 2) && (sizeof(T) == 2 || sizeof(T) == 1),
+                  "[PTO][SA] TPACK: 32 -> 16, 32 -> 8 or 16 -> 8 bits");
+    using UB = std::conditional_t<sizeof(U) == 4, uint32_t, uint16_t>;
+    using TB = std::conditional_t<sizeof(T) == 2, uint16_t, uint8_t>;
+    using S = typename DstT::Storage;
+    detail::Conformed<DstT, SrcT> c(src);
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i)
+            dst.S().v[s][i] = __builtin_bit_cast(T, (TB)__builtin_bit_cast(UB, (U)c.S().v[s][i]));
+}
+
+// TQUANT (the a2a3 form, npu/a2a3/TQuant.hpp:26-52): src = src * scale[row] (+ offset[row]), in place as there, then
+// rounded to the nearest integer (ties to even) and saturated to int8 (symmetric) or uint8 (asymmetric)
+enum class QuantType { INT8_SYM, INT8_ASYM };
+template <QuantType quant, typename DstT, typename SrcT, typename ParaT>
+PTO_DEV void TQUANT_IMPL(DstT &dst, SrcT &src, ParaT &scale, ParaT *offset = nullptr)
+{
+    using U = typename DstT::DType;
+    static_assert(std::is_same_v<typename SrcT::DType, float>, "[PTO][SA] TQUANT: fp32 source");
+    static_assert(quant == QuantType::INT8_SYM ? std::is_same_v<U, int8_t> : std::is_same_v<U, uint8_t>,
+                  "[PTO][SA] TQUANT: int8 (symmetric) or uint8 (asymmetric) destination");
+    TROWEXPANDMUL_IMPL(src, src, scale);
+    if constexpr (quant == QuantType::INT8_ASYM)
+        TROWEXPANDADD_IMPL(src, src, *offset);
+    using S = typename DstT::Storage;
+    detail::Conformed<DstT, SrcT> c(src);
+    constexpr float lo = quant == QuantType::INT8_SYM ? -128.0f : 0.0f, hi = quant == QuantType::INT8_SYM ? 127.0f : 255.0f;
+#pragma unroll
+    for (int s = 0; s < S::Slots; ++s)
+#pragma unroll
+        for (int i = 0; i < detail::kVecChunk; ++i) {
+            const float t = __builtin_rintf(c.S().v[s][i]);
+            dst.S().v[s][i] = (U)(int)(t < lo ? lo : t > hi ? hi : t); // a NaN compares false twice and converts to 0
+        }
+}
+
+// TDEQUANT: dst = (float(src) - offset[row]) * scale[row] over the destination's valid region, the two steps rounded
+// separately; scale and offset are column 0 of their tiles (npu/a2a3/TDequant.hpp:193-202 and the generator of its test,
+// tests/npu/a2a3/src/st/testcase/tdequant/gen_data.py:40-46)
+template <typename DstT, typename SrcT, typename ParaT>
+PTO_DEV void TDEQUANT_IMPL(DstT &dst, SrcT &src, ParaT &scale, ParaT &offset)
+{
+    using U = typename SrcT::DType;
+    static_assert(std::is_same_v<typename DstT::DType, float> && std::is_same_v<typename ParaT::DType, float> &&
+                      (std::is_same_v<U, int8_t> || std::is_same_v<U, int16_t>),
+                  "[PTO][SA] TDEQUANT: int8 or int16 source, fp32 destination, scale and offset");
+    __shared__ float sc[DstT::Rows], of[DstT::Rows];
+    detail::stage_row_values<ParaT, DstT::Rows>(scale, sc);
+    detail::stage_row_values<ParaT, DstT::Rows>(offset, of);
+    hw::lds_barrier();
+    detail::Conformed<DstT, SrcT> c(src);
+    const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        int r, col;
+        detail::elem_rc<DstT>(e, r, col);
+        if (e < DstT::Numel && r < vr && col < vc)
+            dst.S().v[s][i] = ((float)c.S().v[s][i] - of[r]) * sc[r];
+    });
+    hw::lds_barrier();
+}
+
 // ------------------------------------------------------- column reductions
 namespace detail {
 enum class Red { Max, Min, Sum, Prod };
@@ -460,14 +557,16 @@ PTO_DEV char *stage_buffer()
     __shared__ __attribute__((aligned(16))) char buf[Bytes];
     return buf;
 }
-// a Vec tile's elements as 32-bit words in row-major order
+// a Vec tile's elements in row-major order, as they lie in a buffer of the reference
 template <typename TileT>
-PTO_DEV void stage_tile_rows_raw(TileT &t, uint32_t *lds)
+PTO_DEV void stage_tile_rows_raw(TileT &t, void *lds)
 {
-    static_assert(sizeof(typename TileT::DType) == 4 && TileT::isRowMajor, "4-byte elements, row-major");
+    static_assert(TileT::isRowMajor, "row-major tile");
+    using T = typename TileT::DType;
+    T *p = static_cast<T *>(lds);
     for_each_owned<TileT>([&](int s, int i, int e) {
         if (e < TileT::Numel)
-            lds[e] = __builtin_bit_cast(uint32_t, t.S().v[s][i]);
+            p[e] = t.S().v[s][i];
     });
 }
 } // namespace detail
@@ -785,17 +884,17 @@ PTO_DEV void TCI_IMPL(TileT &dst, T start)
 // TSCATTER (cpu/TScatter.hpp:21-44): dst[indexes[i, j], j] = src[i, j] over the source's valid region.  The reference
 // walks the rows in order, so where several rows send an element to the same place the last one wins: the winner is
 // found with an atomic maximum over the source row numbers in LDS.  Rows outside the tile are dropped (the reference
-// writes out of bounds there).  4-byte elements.
+// writes out of bounds there).
 template <typename TileT, typename IdxT>
 PTO_DEV void TSCATTER_IMPL(TileT &dst, TileT &src, IdxT &indexes)
 {
     using T = typename TileT::DType;
-    static_assert(TileT::Loc == TileType::Vec && IdxT::Loc == TileType::Vec && TileT::isRowMajor && IdxT::isRowMajor && sizeof(T) == 4 &&
+    static_assert(TileT::Loc == TileType::Vec && IdxT::Loc == TileType::Vec && TileT::isRowMajor && IdxT::isRowMajor &&
                       std::is_integral_v<typename IdxT::DType> && IdxT::Rows == TileT::Rows && IdxT::Cols == TileT::Cols,
-                  "[PTO][SA] TSCATTER: row-major Vec tiles of 4-byte elements, integer index tile of the same shape");
+                  "[PTO][SA] TSCATTER: row-major Vec tiles, integer index tile of the same shape");
     constexpr int N = TileT::Numel;
-    int *owner = reinterpret_cast<int *>(detail::stage_buffer<detail::stage_bytes(8 * N)>());
-    uint32_t *value = reinterpret_cast<uint32_t *>(owner + N);
+    int *owner = reinterpret_cast<int *>(detail::stage_buffer<detail::stage_bytes((4 + (int)sizeof(T)) * N)>());
+    T *value = reinterpret_cast<T *>(owner + N);
     for (int e = hw::tid(); e < N; e += kBlockThreads)
         owner[e] = -1;
     hw::lds_barrier();
@@ -811,12 +910,12 @@ PTO_DEV void TSCATTER_IMPL(TileT &dst, TileT &src, IdxT &indexes)
         const int r = e / TileT::Cols, c = e % TileT::Cols;
         const uint32_t row = (uint32_t)indexes.S().v[s][i];
         if (e < N && r < vr && c < vc && row < (uint32_t)TileT::Rows && owner[row * TileT::Cols + c] == r)
-            value[row * TileT::Cols + c] = __builtin_bit_cast(uint32_t, src.S().v[s][i]);
+            value[row * TileT::Cols + c] = src.S().v[s][i];
     });
     hw::lds_barrier();
     detail::for_each_owned<TileT>([&](int s, int i, int e) {
         if (e < N && owner[e] >= 0)
-            dst.S().v[s][i] = __builtin_bit_cast(T, value[e]);
+            dst.S().v[s][i] = value[e];
     });
     hw::lds_barrier();
 }
@@ -844,7 +943,7 @@ PTO_DEV void MSCATTER_IMPL(G &dst, SrcT &src, IdxT &indexes)
 // ---------------------------------------------------------------------- TGATHERB
 // Block gather (cpu/TGatherB.hpp:21-60): for every row r and every 32-byte block c of the destination's valid region,
 // dst block (r, c) = the 32 bytes of the source tile's storage that start at byte offset[r, c]; blocks whose source range
-// does not lie inside the source tile are left as they are.  4-byte elements: a block is one 8-element chunk of a lane.
+// does not lie inside the source tile are left as they are.
 template <typename DstT, typename SrcT, typename OffT>
 PTO_DEV void TGATHERB_IMPL(DstT &dst, SrcT &src, OffT &offset)
 {
@@ -852,33 +951,28 @@ PTO_DEV void TGATHERB_IMPL(DstT &dst, SrcT &src, OffT &offset)
     static_assert(DstT::Loc == TileType::Vec && SrcT::Loc == TileType::Vec && OffT::Loc == TileType::Vec && DstT::isRowMajor && SrcT::isRowMajor &&
                       OffT::isRowMajor,
                   "[PTO][SA] TGATHERB: row-major Vec tiles");
-    static_assert(sizeof(T) == 4 && sizeof(typename SrcT::DType) == 4 && sizeof(typename OffT::DType) == 4 && DstT::Cols % detail::kVecChunk == 0 &&
-                      OffT::Rows == DstT::Rows,
-                  "[PTO][SA] TGATHERB: 4-byte elements, 32-bit offsets, one offset row per destination row");
-    constexpr int kSrcBytes = SrcT::Numel * 4, kOffs = OffT::Numel;
-    char *bytes = detail::stage_buffer<detail::stage_bytes(kSrcBytes + 4 * kOffs)>();
-    uint32_t *offs = reinterpret_cast<uint32_t *>(bytes + kSrcBytes);
-    detail::stage_tile_rows_raw(src, reinterpret_cast<uint32_t *>(bytes));
+    static_assert(sizeof(typename SrcT::DType) == sizeof(T) && sizeof(typename OffT::DType) == 4 && OffT::Rows == DstT::Rows,
+                  "[PTO][SA] TGATHERB: one element size, 32-bit offsets, one offset row per destination row");
+    constexpr int kSrcBytes = SrcT::Numel * (int)sizeof(T), kOffs = OffT::Numel, kPerBlock = 32 / (int)sizeof(T);
+    char *bytes = detail::stage_buffer<detail::stage_bytes(kSrcBytes + 4 + 4 * kOffs)>();
+    uint32_t *offs = reinterpret_cast<uint32_t *>(bytes + (kSrcBytes + 3) / 4 * 4);
+    detail::stage_tile_rows_raw(src, bytes);
     detail::stage_tile_rows_raw(offset, offs);
     hw::lds_barrier();
     const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
-    using S = typename DstT::Storage;
-#pragma unroll
-    for (int s = 0; s < S::Slots; ++s) {
-        const int q = s * kBlockThreads + hw::tid(), e0 = q * detail::kVecChunk;
-        const int r = e0 / DstT::Cols, c = (e0 % DstT::Cols) / detail::kVecChunk;
-        if (e0 < DstT::Numel && r < vr && (c + 1) * detail::kVecChunk <= vc && c < OffT::Cols) {
-            const uint32_t off = offs[r * OffT::Cols + c];
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        const int r = e / DstT::Cols, c = e % DstT::Cols, cb = c / kPerBlock;
+        if (e < DstT::Numel && r < vr && (cb + 1) * kPerBlock <= vc && cb < OffT::Cols) {
+            const uint32_t off = offs[r * OffT::Cols + cb];
             if (off <= (uint32_t)kSrcBytes - 32u) {
-                T v[detail::kVecChunk];
-                __builtin_memcpy(v, bytes + off, 32); // any byte alignment
-#pragma unroll
-                for (int i = 0; i < detail::kVecChunk; ++i)
-                    dst.S().v[s][i] = v[i];
+                T v;
+                __builtin_memcpy(&v, bytes + off + (uint32_t)(c % kPerBlock) * sizeof(T), sizeof(T)); // any byte alignment
+                dst.S().v[s][i] = v;
             }
         }
-    }
+    });
     hw::lds_barrier();
 }
 
 } // namespace pto
+#pragma clang fp contract(fast)

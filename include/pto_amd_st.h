@@ -183,6 +183,10 @@ int pto_st_tmrgsort_lists_16(void *stream, void *out, uint32_t *executed, const 
 int pto_st_matmul_vec_operands_f16_64x64x128(void *stream, float *out, float *mid, const uint16_t *a, const uint16_t *b);
 /* TTRANS on fp32: out [128,64] = in [64,128] transposed. */
 int pto_st_ttrans_f32_64x128(void *stream, float *out, const float *in);
+/* TPREFETCH of an int32 [16,64] matrix into a tile, TPACK to int16 (out16) and on to int8 (out8): the low bits of every
+ * element (npu/a5/TPack.hpp:21-72); print != 0: TPRINT of a [4,16] tile with a [3,10] valid region and of a [2,4] view of
+ * the input, in the reference's format (npu/a2a3/TPrint.hpp:44-190), on the process's standard output. */
+int pto_st_prefetch_pack_print_s32_16x64(void *stream, int16_t *out16, int8_t *out8, const int32_t *in, int print);
 int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, int relu, float scale);
 
 /* Two-stage pipeline through TPUSH / TPOP FIFOs (common/fifo.hpp, cpu/TPush.hpp, cpu/TPop.hpp; the hand-offs of

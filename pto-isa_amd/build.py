@@ -149,9 +149,9 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
               "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract",
               "tmax", "tmin", "tmins", "texpands", "tsels", "tsort32", "tgather", "tmrgsort", "tstore",
-              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin"]
+              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
-_ST_KEYED = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<")
+_ST_KEYED = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<[^;]*?>>>\s*\(([^;]*)\)\s*;")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
 _ST_KEYED_KERNEL = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<<<")
 _ST_KERNEL_BODY = re.compile(r'extern "C" __global__ AICORE void (\w+)\([^)]*\)\s*\{(.*?)\n\}', re.S)
@@ -163,13 +163,16 @@ ST_PORT_OPTIONS = {
 }
 # its top-k kernel works through Vec tiles that are views of one another (TASSIGN to the same address)
 ST_PORT_OPTIONS["tmrgsort"] = dict(vec_in_memory=True)
+# multiplies in one function and declares the accumulator tile again, at the same address, in the next: tiles as addresses
+ST_PORT_OPTIONS["tmov_acc2mat"] = dict(vec_in_memory=True)
 # sources that keep their device code under the Ascend device compiler's own macro
 for _name in ("tmax", "tmin", "tmins", "texpands"):
     ST_PORT_OPTIONS[_name] = dict(defines=["__CCE_AICORE__=220"])
 
 
 def st_case_table(source_text):
-    """{case: {"run": run function, "targs": [template arguments], "params": kernel parameter list}} for the two ways the
+    """{case: {"run": run function, "targs": [template arguments], "params": kernel parameter list, "args": the launch's
+    arguments where the source writes them}} for the ways the
     test sources number their cases: `launch<OP>Case<N>` kernels (case = "N"), and launchers that switch on their template
     argument, `if constexpr (tilingKey == N) { run<...><<<` (case = "<launcher>:N")."""
     table = {}
@@ -180,7 +183,8 @@ def st_case_table(source_text):
     for m in _ST_KEYED.finditer(source_text):
         owner = [name for pos, name in launchers if pos < m.start()]
         if owner:
-            table["%s:%s" % (owner[-1], m.group(1))] = {"run": m.group(2), "targs": [a.strip() for a in m.group(3).split(",")], "params": ""}
+            table["%s:%s" % (owner[-1], m.group(1))] = {"run": m.group(2), "targs": [a.strip() for a in m.group(3).split(",")], "params": "",
+                                                        "args": " ".join(m.group(4).split())}
     # ... or `if constexpr (tilingKey == N) { kernel<<<`, the kernel fixing its case through local constants
     # (`constexpr uint32_t M = 64;`) that it hands to one run function: the constants and the run function's leading type
     # arguments are the case

@@ -1046,6 +1046,31 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void TransKernel(__gm__ float
     TSTORE(go, y);
 }
 
+// TPREFETCH (the tile then holds the region, as after a TLOAD), TPACK to 16 and to 8 bits, and, when asked, TPRINT of
+// the [4, 16] corner tile and of the matching corner of the input in memory
+__global__ __launch_bounds__(kBlockThreads) AICORE void PackKernel(__gm__ int16_t *out16, __gm__ int8_t *out8, __gm__ const int32_t *in, int print)
+{
+    Tile<TileType::Vec, int32_t, 16, 64, BLayout::RowMajor> x;
+    Tile<TileType::Vec, int16_t, 16, 64, BLayout::RowMajor> y16;
+    Tile<TileType::Vec, int8_t, 16, 64, BLayout::RowMajor> y8;
+    GmND<int32_t, 16, 64> gi(const_cast<int32_t *>(in));
+    GmND<int16_t, 16, 64> go16(out16);
+    GmND<int8_t, 16, 64> go8(out8);
+    TPREFETCH(x, gi);
+    TPACK(y16, x);
+    TPACK(y8, y16);
+    TSTORE(go16, y16);
+    TSTORE(go8, y8);
+    if (print) {
+        Tile<TileType::Vec, int32_t, 4, 16, BLayout::RowMajor, -1, -1> corner(3, 10);
+        GlobalTensor<int32_t, Shape<1, 1, 1, 4, 16>, Stride<64 * 16, 64 * 16, 64 * 16, 64, 1>> gc(const_cast<int32_t *>(in));
+        TLOAD(corner, gc);
+        TPRINT(corner);
+        GlobalTensor<int32_t, Shape<1, 1, 1, 2, 4>, Stride<64 * 16, 64 * 16, 64 * 16, 64, 1>> gs(const_cast<int32_t *>(in));
+        TPRINT(gs);
+    }
+}
+
 // ---- TSORT32 on an [8, 128] tile with valid region [vr, vc]; out [8, 256] (4-byte scores) or [8, 512] (2-byte) is loaded first so that the elements the
 // instruction leaves alone keep what the caller put there ----
 template <typename T>
@@ -1388,6 +1413,13 @@ extern "C" int pto_st_ttrans_f32_64x128(void *stream, float *out, const float *i
 {
     PTO_ST_NONNULL(out, in);
     TransKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, in);
+    return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_prefetch_pack_print_s32_16x64(void *stream, int16_t *out16, int8_t *out8, const int32_t *in, int print)
+{
+    PTO_ST_NONNULL(out16, out8, in);
+    PackKernel<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out16, out8, in, print);
     return pto_amd::check_launch();
 }
 

@@ -32,6 +32,9 @@ script therefore does (nothing else is touched; the tile code itself compiles as
 11. `--l1 OLD=NEW` rewrites the literal address of `TASSIGN(tile, OLD)`: sources place their L1 tiles at addresses laid
     out for Ascend's 512 KiB (0x20000, 0x40000 ...), which have to move inside the 160 KiB of LDS.  Register tiles ignore
     their address, so rewriting theirs too changes nothing.
+12. Reads of Ascend's special scalar registers written as inline assembly, `asm volatile("MOV %0, SYS_CNT\n" : "+l"(x));`
+    and `... PC ...`, become `x = get_sys_cnt();` and `x = 0;` (time stamps that the test kernels log, and the program
+    counter they hand to an instruction-cache preload, which is a no-op here).
 """
 import argparse
 import os
@@ -94,6 +97,7 @@ def kernel_before(text, pos):
     return " ".join(text[start:end].split())
 
 
+ASCEND_SREG_READ = re.compile(r'asm\s+volatile\s*\(\s*"MOV %0, (SYS_CNT|PC)\\n"\s*:\s*"\+l"\s*\(\s*(\w+)\s*\)\s*\)\s*;')
 TASSIGN_LITERAL = re.compile(r"(TASSIGN\(\s*\w+\s*,\s*)(0[xX][0-9a-fA-F]+|\d+)(\s*\))")
 
 
@@ -123,6 +127,11 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
             return "%s0x%x%s" % (m.group(1), table[a], m.group(3))
         text = TASSIGN_LITERAL.sub(move, text)
         notes.append("%d TASSIGN address%s moved" % (hits[0], "" if hits[0] == 1 else "es"))
+
+    # 12. special-register reads
+    text, n = ASCEND_SREG_READ.subn(lambda m: "%s = %s;" % (m.group(2), "get_sys_cnt()" if m.group(1) == "SYS_CNT" else "0"), text)
+    if n:
+        notes.append("%d special-register read%s rewritten" % (n, "" if n == 1 else "s"))
 
     # 2. launch statements
     blocks = "pto::host::LaunchBlocks(%s, (hipStream_t)(%s))" if vec_in_memory else "%s"

@@ -66,6 +66,7 @@ ST_SYMBOLS = {
     "pto_st_tmrgsort_blocks_16_1x2048": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 3),
     "pto_st_tmrgsort_lists_16": (C.c_int, [C.c_void_p] * 7 + [C.c_int] * 8),
     "pto_st_ttrans_f32_64x128": (C.c_int, [C.c_void_p] * 3),
+    "pto_st_prefetch_pack_print_s32_16x64": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_vec_bitop_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int, C.c_int]),
     "pto_st_vec_op_f32_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int]),
     "pto_st_reduce_f32_64x128": (C.c_int, [C.c_void_p] * 3 + [C.c_int] * 3),

@@ -195,7 +195,7 @@ def _elementwise_plan(spec, dtype, buffers, valid, scalar, scalar_first=False):
             return [op(k, a) if scalar_first else op(a, k)]
         return [op(a) if len(ins) == 1 else op(a, ins[1][:vr, :vc])]
     return SimpleNamespace(dtype=dtype, outs=[(dtype, buffers[0])], ins=[(dtype, b) for b in buffers[1:]], regions=[valid],
-                           scalar=scalar, expect=expect, spec=spec, compare=None, flat_prefix=None)
+                           scalar=scalar, expect=expect, spec=spec, compare=None, flat_prefix=None, scalar_after_stream=False, ins_after_stream=0)
 
 
 # ---- numbered cases: launch<OP>TestCase<N>(void *out, void *src, float scalar, stream) -> run<T, dstRows, dstCols, rows,
@@ -247,7 +247,7 @@ def TAIL(ints, nptr, suffix="", ptr0=None):
 
 def _plan(spec, outs, ins, regions, expect, scalar=None):
     return SimpleNamespace(dtype=ins[0][0] if ins else outs[0][0], outs=outs, ins=ins, regions=regions, scalar=scalar,
-                           expect=lambda arrays, k: expect(arrays), spec=spec, compare=None, flat_prefix=None)
+                           expect=lambda arrays, k: expect(arrays), spec=spec, compare=None, flat_prefix=None, scalar_after_stream=False, ins_after_stream=0)
 
 
 # ---- column reductions: launchTCOLSUM<T, cols, srcRows, validRows[, binary]>: [validRows, cols] of a [srcRows, cols] buffer
@@ -828,6 +828,234 @@ SPECS.update({
 })
 
 
+# ---- the accumulator's way out with a conversion (the fix pipe): tmov_acc2mat (Acc -> Mat by TMOV / TEXTRACT / TINSERT,
+# then Mat -> NZ memory) and tstore_acc2gm (Acc -> ND or NZ memory), plain, with one quantisation word, with one per column.
+# The numpy model restates the generators' decoding of the word (tmov_acc2mat/gen_data.py:27-100, tstore_acc2gm/gen_data.py):
+# bits 31..13 a float scale cut to 10 mantissa bits, 35..32 the int16 shift - 1, 45..37 an offset, 46 signed 8-bit result.
+_FIX_NAMES = {"half": np.float16, "float": np.float32, "int8_t": np.int8, "uint8_t": np.uint8, "int16_t": np.int16, "int32_t": np.int32,
+              "bfloat16_t": np.uint16, "uint64_t": np.uint64}
+
+
+def fix_quant_model(acc, words, out_name):
+    """acc [m, n] (float32 or int32), words: one uint64 or [n] of them -> the converted matrix (bf16 as its bits)"""
+    q = np.broadcast_to(np.asarray(words, dtype=np.uint64), (acc.shape[1],))
+    if out_name == "int16_t":
+        shift = ((q >> np.uint64(32)) & np.uint64(0xF)).astype(np.int64) + 1
+        return np.clip(acc.astype(np.int64) >> shift[None, :], -32768, 32767).astype(np.int16)
+    scale = (q & np.uint64(0xFFFFE000)).astype(np.uint32).view(np.float32)
+    y = acc.astype(np.float32) * scale[None, :]
+    if out_name in ("int8_t", "uint8_t"):
+        t = np.clip(np.rint(y), -256, 255).astype(np.int64) + ((q >> np.uint64(37)) & np.uint64(0x1FF)).astype(np.int64)[None, :]
+        signed = ((q >> np.uint64(46)) & np.uint64(1)).astype(bool)[None, :]
+        return np.where(signed, np.clip(t, -128, 127), np.clip(t, 0, 255)).astype(_FIX_NAMES[out_name])
+    if out_name == "half":
+        return np.clip(y, -65504, 65504).astype(np.float16)
+    return _bf16_bits(y.astype(np.float64))
+
+
+def fix_plain_model(acc, out_name):
+    if out_name == "bfloat16_t":
+        return _bf16_bits(acc.astype(np.float64))
+    return acc.astype(_FIX_NAMES[out_name])
+
+
+def fix_scalar_word(scalar, out_name):
+    """the word the test kernels build from their float argument (tmov_acc2mat_kernel.cpp:270-283, tstore_acc2gm_kernel.cpp:230-234)"""
+    if out_name == "int16_t":
+        return np.uint64(((int(scalar) - 1) & 0xF) << 32)
+    w = int(np.float32(scalar).view(np.uint32))
+    if out_name in ("int8_t", "uint8_t"):
+        w |= int(out_name == "int8_t") << 46
+    return np.uint64(w)
+
+
+def _nz(mat, block_cols):
+    """[R, C] -> the NZ image [C / bc][R / 16][16][bc] as rows of bc"""
+    r, c = mat.shape
+    return mat.reshape(r // 16, 16, c // block_cols, block_cols).transpose(2, 0, 1, 3).reshape(-1, block_cols)
+
+
+def _acc_of(arrays, a_name, vm, vk, vn):
+    """the accumulator of the valid product (inputs are zero outside it): int32 for int8 operands, else float32 (exact: small integers)"""
+    conv = (lambda x: _bf16_value(x).astype(np.int64)) if a_name == "bfloat16_t" else (lambda x: x.astype(np.int64))
+    a, b = conv(arrays[0]), conv(arrays[1])
+    c = a @ b
+    return c.astype(np.int32 if a_name == "int8_t" else np.float32)
+
+
+def plan_acc2mat(test, spec, m):
+    e = manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]
+    t = list(e["targs"])
+    form = spec["form"]
+    out_name, a_name = t[0], t[1]
+    if form == "vector":
+        del t[3]
+    M, K, N, vm, vk, vn = (int(x) for x in t[3:9])
+    opt = t[9:] + ["false", "0", "0", "false", "0", "0"][len(t) - 9:]
+    relu, ir, ic, insert, drow, dcol = opt[0] == "true", int(opt[1]), int(opt[2]), opt[3] == "true", int(opt[4]), int(opt[5])
+    out_dt, a_dt = np.dtype(_FIX_NAMES[out_name]), np.dtype(_FIX_NAMES[a_name])
+    bc = 512 // (16 * out_dt.itemsize)
+    rows, cols = (drow, dcol) if insert else (M - ir, N - ic)
+    ins = [(a_dt, (M, K), ("corner", vm, vk)), (a_dt, (K, N), ("corner", vk, vn))]
+    if form == "vector":
+        ins.append((np.dtype(np.uint64), (1, N), ("words", out_name)))
+    init_dt = out_dt if out_dt.kind != "f" and out_dt != np.uint16 else out_dt
+    ins.append((init_dt, (rows, cols) if insert else (1, 16), "bits" if out_dt.kind in "iu" else "unit"))
+    scalar = float(e["args"].rsplit(",", 1)[1]) if form == "scalar" else None
+
+    def expect(arrays):
+        acc = _acc_of(arrays, a_name, vm, vk, vn)
+        if relu:
+            acc = np.maximum(acc, 0)
+        if form == "plain":
+            g = fix_plain_model(acc, out_name)
+        else:
+            g = fix_quant_model(acc, arrays[2].reshape(-1) if form == "vector" else fix_scalar_word(scalar, out_name), out_name)
+        if insert:
+            full = arrays[-1].copy()
+            full[ir:ir + M, ic:ic + N] = g
+            g = full
+        else:
+            g = g[ir:, ic:]
+        return [_nz(g, bc)]
+    pl = _plan(spec, [(out_dt, (rows * cols // bc, bc))], ins, [(rows * cols // bc, bc)], expect)
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(want.dtype), want)
+    return pl
+
+
+for _fn, _form, _n in (("launchTMOVAcc2MatNZ2NZ", "plain", 4), ("launchTMOVAcc2MatSCQuantNz", "scalar", 4), ("launchTMOVAcc2MatFBQuantNz", "vector", 5)):
+    SPECS["tmov_acc2mat:" + _fn] = dict(fn=_fn, lib="tmov_acc2mat", tail=CASE_MATMUL % _n, planner=plan_acc2mat, inputs="small", form=_form)
+
+
+def plan_acc2gm(test, spec, m):
+    e = manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]
+    t = e["targs"]
+    form, nz = spec["form"], spec["nz"]
+    atomic, out_name, a_name = t[0] == "1", t[2], t[3]
+    g = [int(x) for x in t[4:9]]
+    w = [int(x) for x in t[9:14]]
+    vm, vn, vk = (int(x) for x in t[14:17])
+    relu = len(t) > 17 and t[17] == "1"
+    out_dt, a_dt = np.dtype(_FIX_NAMES[out_name]), np.dtype(_FIX_NAMES[a_name])
+    kind = ("corner", vm, vk, "bf16") if a_name == "bfloat16_t" else "small"
+    ins = [(a_dt, (vm, vk), kind), (a_dt, (vk, vn), ("corner", vk, vn, "bf16") if a_name == "bfloat16_t" else "small")]
+    if form == "vector":
+        align = (vn * 8 + 127) // 128 * 128 // 8
+        ins.append((np.dtype(np.uint64), (1, align), ("words", out_name)))
+    scalar = 2.0 if form == "scalar" else None
+    if nz:
+        assert g == w
+        rows, cols = g[2] * g[3], g[0] * g[1] * g[4]
+        shape = region = (g[0] * g[1] * g[2] * g[3], g[4])
+    else:
+        assert g[:3] == [1, 1, 1] and w[:3] == [1, 1, 1]
+        rows, cols = g[3], g[4]
+        shape, region = (w[3], w[4]), (rows, cols)
+
+    def expect(arrays):
+        acc = _acc_of(arrays, a_name, vm, vk, vn)[:rows, :cols]
+        if relu:
+            acc = np.maximum(acc, 0)
+        if form == "plain":
+            r = fix_plain_model(acc, out_name)
+        else:
+            r = fix_quant_model(acc, arrays[2].reshape(-1)[:cols] if form == "vector" else fix_scalar_word(scalar, out_name), out_name)
+        if atomic and out_name == "bfloat16_t":
+            # the harness fills the output with the bits 77, a bf16 denormal of 7e-39: it is what is left where 0 is added
+            # to it and vanishes in the rounding of every other sum
+            r = np.where(_bf16_value(r) == 0, np.uint16(77), r)
+        elif atomic:    # the harness fills the output with 77 before the launch
+            r = (r.astype(np.float64 if out_dt.kind == "f" else np.int64) + 77).astype(out_dt)
+        if nz:          # [col blocks][row blocks][rows of a block][columns of a block]
+            r = r.reshape(rows, cols // g[4], g[4]).transpose(1, 0, 2).reshape(-1, g[4])
+        return [r]
+    pl = _plan(spec, [(out_dt, shape)], ins, [region], expect, scalar=(C.c_float, scalar) if form == "scalar" else None)
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(want.dtype), want)
+    pl.scalar_after_stream = True
+    return pl
+
+
+for _fn, _form, _nzflag, _n in (("LaunchTStoreAcc2gmNz2nd", "plain", False, 3), ("LaunchTStoreAcc2gmNz2nz", "plain", True, 3),
+                               ("LaunchTStoreAcc2gmVectorNz2nd", "vector", False, 4), ("LaunchTStoreAcc2gmVectorNz2nz", "vector", True, 4)):
+    SPECS["tstore_acc2gm:" + _fn] = dict(fn=_fn, lib="tstore_acc2gm", tail=CASE_MATMUL % _n, planner=plan_acc2gm, inputs="small", form=_form, nz=_nzflag)
+for _fn, _nzflag in (("LaunchTStoreAcc2gmScalarNz2nd", False), ("LaunchTStoreAcc2gmScalarNz2nz", True)):
+    SPECS["tstore_acc2gm:" + _fn] = dict(fn=_fn, lib="tstore_acc2gm", tail=r"<(?P<case>\d+)>\((?:unsigned char\*, ){3}void\*, float\)", planner=plan_acc2gm,
+                                         inputs="small", form="scalar", nz=_nzflag)
+
+
+# ---- TFILLPAD / TFILLPAD_INPLACE / TFILLPAD_EXPAND: launchTFILLPAD<N>(out, src, log, stream); kernel N fixes
+# <T, 1, 1, 1, rows, cols, tileRows, tileCols, dyn, load pad, fill pad[, inplace[, expand]]>: a [rows, cols] matrix in the
+# corner of a [tileRows, tileCols] tile, the fill pad value around it (tfillpad_kernel.cpp:113-194; golden :316-363).  The
+# kernel also writes three time stamps into `log`.
+def _pad_value(dt, which):
+    if dt.kind == "f":
+        return dt.type(np.inf if which == "Max" else -np.inf)
+    info = np.iinfo(dt)
+    return dt.type(info.max if which == "Max" else info.min)
+
+
+def plan_fillpad(test, spec, m):
+    e = manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]
+    t = e["targs"]
+    dt = np.dtype({"float": np.float32, "uint16_t": np.uint16, "int16_t": np.int16, "int8_t": np.int8, "int32_t": np.int32}[t[0]])
+    rows, cols, trows, tcols = (int(x) for x in t[4:8])
+    pad = _pad_value(dt, t[10].split("::")[1])
+
+    def expect(arrays):
+        out = np.full((trows, tcols), pad, dtype=dt)
+        out[:rows, :cols] = arrays[0]
+        return [out]
+    pl = _plan(spec, [(dt, (trows, tcols))], [(dt, (rows, cols), "any"), (np.dtype(np.uint64), (1, 128), "any")], [(trows, tcols)], expect)
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    return pl
+
+
+SPECS["tfillpad"] = dict(fn="launchTFILLPAD", lib="tfillpad", tail=r"<(?P<case>\d+)>\(unsigned char\*, unsigned char\*, unsigned long\*, void\*\)", planner=plan_fillpad, inputs="any")
+
+
+# ---- TQUANT, the a2a3 form: TQuantTest::LaunchTQuantInt8<rows, cols, mode, type>(dst, src, scale, stream, offset):
+# int8 = clamp(rint(src * scale[row])), uint8 = clamp(rint(src * scale[row] + offset[row])), each step rounded to fp32
+# (tquant_kernel.cpp:24-95, tquant/gen_data.py:22-60)
+def plan_quant(test, spec, m):
+    rows, cols, asym = int(m.group("r")), int(m.group("c")), m.group("q") == "1"
+    dt = np.dtype(np.uint8 if asym else np.int8)
+
+    def expect(arrays):
+        y = arrays[0] * arrays[1]
+        if asym:
+            y = y + arrays[2]
+        return [np.clip(np.rint(y), 0 if asym else -128, 255 if asym else 127).astype(dt)]
+    f32 = np.dtype(np.float32)
+    pl = _plan(spec, [(dt, (rows, cols))], [(f32, (rows, cols), ("range", -2.0, 2.0)), (f32, (rows, 1), ("range", 20.0, 90.0)),
+                                             (f32, (rows, 1), ("range", 60.0, 160.0))], [(rows, cols)], expect)
+    pl.ins_after_stream = 1
+    return pl
+
+
+SPECS["tquant"] = dict(fn="TQuantTest::LaunchTQuantInt8", planner=plan_quant, inputs="any",
+                       tail=r"<(?P<r>\d+), (?P<c>\d+), 0, \(pto::QuantType\)(?P<q>[01])>\(std::conditional<.*>::type\*, float\*, float\*, void\*, float\*\)")
+
+
+# ---- TDEQUANT: LaunchTDequant<float, S, dstRows, dstCols, srcRows, srcCols, validRows, validCols, paraRows, paraCols>(out, src,
+# scale, offset, stream): out = (float(src) - offset[row]) * scale[row] on the valid region; every matrix has the row stride
+# dstCols in memory, scale and offset paraCols (tdequant_kernel.cpp:20-57, tdequant/gen_data.py:12-46)
+def plan_dequant(test, spec, m):
+    src_dt, _ = _elem(m.group("T"), False)
+    q = _ints(m, ["dr", "dc", "sr", "sc", "vr", "vc", "pr", "pc"])
+    vr, vc = q["vr"], q["vc"]
+    f32 = np.dtype(np.float32)
+
+    def expect(arrays):
+        return [(arrays[0][:, :vc].astype(np.float32) - arrays[2][:, :1]) * arrays[1][:, :1]]
+    return _plan(spec, [(f32, (vr, q["dc"]))], [(src_dt, (vr, q["dc"]), "bits"), (f32, (vr, q["pc"]), ("range", 0.001, 1.0)),
+                                                 (f32, (vr, q["pc"]), ("range", -128.0, 127.0))], [(vr, vc)], expect)
+
+
+SPECS["tdequant"] = dict(fn="LaunchTDequant", planner=plan_dequant, inputs="any",
+                         tail=r"<float, (?P<T>[a-z ]+)" + "".join(r", (?P<%s>\d+)" % k for k in ("dr", "dc", "sr", "sc", "vr", "vc", "pr", "pc")) +
+                         r">\(float\*, [a-z ]+\*, float\*, float\*, void\*\)")
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
@@ -835,6 +1063,22 @@ def lib_of(test):
 
 def draw(rng, dt, shape, kind, j):
     """Operand j of a test whose operation is of the given kind."""
+    if isinstance(kind, tuple) and kind[0] == "range":
+        return rng.uniform(kind[1], kind[2], size=shape).astype(dt)
+    if isinstance(kind, tuple) and kind[0] == "corner":      # small integers in the [vr, vc] corner, zeros around it
+        x = np.zeros(shape, dtype=dt)
+        v = rng.integers(-1, 2, size=(kind[1], kind[2]), endpoint=True)
+        x[:kind[1], :kind[2]] = _bf16_bits(v.astype(np.float64)) if len(kind) > 3 and kind[3] == "bf16" else v.astype(dt)
+        return x
+    if isinstance(kind, tuple) and kind[0] == "words":       # quantisation words for results of type kind[1]
+        n = int(np.prod(shape))
+        if kind[1] == "int16_t":
+            return (rng.integers(0, 7, size=n, endpoint=True).astype(np.uint64) << np.uint64(32)).reshape(shape)
+        w = rng.choice(np.array([0.5, 1.0, 1.5, 2.0], dtype=np.float32), size=n).view(np.uint32).astype(np.uint64)
+        if kind[1] in ("int8_t", "uint8_t"):
+            w |= rng.integers(0, 3, size=n, endpoint=True).astype(np.uint64) << np.uint64(37)
+            w |= np.uint64(int(kind[1] == "int8_t")) << np.uint64(46)
+        return w.reshape(shape)
     if isinstance(kind, tuple):
         return _sorted_inputs(rng, dt, shape, kind)
     bits = dt.itemsize * 8

@@ -46,10 +46,14 @@ def test_reference_st_kernel(test, mangled, demangled):
     sentinel = 77
     t_out = [to_dev(np.full(shape, sentinel, dtype=dt)) for dt, shape in pl.outs]
     t_in = [to_dev_padded(a) for a in ins]
-    args = [C.c_void_p(t.data_ptr()) for t in t_out + t_in]
-    if pl.scalar:
+    late = pl.ins_after_stream      # buffers that the launcher takes after its stream argument
+    args = [C.c_void_p(t.data_ptr()) for t in t_out + t_in[:len(t_in) - late]]
+    if pl.scalar and not pl.scalar_after_stream:
         args.append(pl.scalar[0](pl.scalar[1]))
     args.append(C.c_void_p(0))
+    if pl.scalar and pl.scalar_after_stream:
+        args.append(pl.scalar[0](pl.scalar[1]))
+    args += [C.c_void_p(t.data_ptr()) for t in t_in[len(t_in) - late:]]
     fn.restype = None
     print("launch", demangled, flush=True)
     fn(*args)

@@ -40,3 +40,35 @@ def test_plan_and_formula(test, mangled, demangled):
         assert want.shape == (vr, vc) or (pl.flat_prefix is not None and want.ndim == 1 and want.size in (pl.flat_prefix, want.size if pl.flat_prefix < 0 else -1))
         if dt.kind == "f" and pl.compare is None:
             assert np.isfinite(want.astype(np.float64)).all()
+
+
+def test_fix_pipe_model_known_answers():
+    """The numpy model of the quantising conversions against values worked out by hand from the word layout of the
+    reference's generator (tests/npu/a2a3/src/st/testcase/tmov_acc2mat/gen_data.py:27-100)."""
+    f32 = lambda x: int(np.float32(x).view(np.uint32))
+    acc = np.array([[100, -3, 10, -200, 5]], dtype=np.int32)
+    signed = 1 << 46
+    # scale 2, signed: 200 -> 127, -6, 20, -400 -> -256 -> -128, 10
+    assert S.fix_quant_model(acc, np.uint64(f32(2.0) | signed), "int8_t").tolist() == [[127, -6, 20, -128, 10]]
+    # unsigned: negatives clamp to 0, 200 stays
+    assert S.fix_quant_model(acc, np.uint64(f32(2.0)), "uint8_t").tolist() == [[200, 0, 20, 0, 10]]
+    # halves round to even: -1.5 -> -2, 2.5 -> 2; offset 3 is added after the rounding
+    assert S.fix_quant_model(acc, np.uint64(f32(0.5) | signed | (3 << 37)), "int8_t").tolist() == [[53, 1, 8, -97, 5]]
+    # one word per column
+    words = np.array([f32(1.0) | signed, f32(2.0) | signed, f32(0.5) | signed, f32(1.0) | signed, f32(1.5) | signed], dtype=np.uint64)
+    assert S.fix_quant_model(acc, words, "int8_t").tolist() == [[100, -6, 5, -128, 8]]
+    # the scale keeps 10 mantissa bits: 1 + 2^-10 survives, 1 + 2^-11 is cut to 1
+    big = np.array([[2048, 2048]], dtype=np.float32)
+    got = S.fix_quant_model(big, np.array([f32(1 + 2.0**-10), f32(1 + 2.0**-11)], dtype=np.uint64), "half")
+    assert got.tolist() == [[2050.0, 2048.0]]
+    assert S.fix_quant_model(np.array([[1e6, -1e6]], dtype=np.float32), np.uint64(f32(1.0)), "half").tolist() == [[65504.0, -65504.0]]
+    # int32 -> int16: shift by n + 1 (arithmetic), then clamp
+    acc16 = np.array([[1000, -1000, 1 << 20, -(1 << 20)]], dtype=np.int32)
+    assert S.fix_quant_model(acc16, np.uint64(1 << 32), "int16_t").tolist() == [[250, -250, 32767, -32768]]
+    # the word the kernels build from their float argument
+    assert S.fix_scalar_word(2.0, "int8_t") == np.uint64(0x40000000 | signed) and S.fix_scalar_word(2.0, "uint8_t") == np.uint64(0x40000000)
+    assert S.fix_scalar_word(2.0, "int16_t") == np.uint64(1 << 32) and S.fix_scalar_word(2.0, "half") == np.uint64(0x40000000)
+    # NZ image: [col blocks][row blocks][16][bc]
+    mat = np.arange(32 * 32).reshape(32, 32)
+    nz = S._nz(mat, 16)
+    assert nz.shape == (64, 16) and nz[0].tolist() == list(range(16)) and nz[1].tolist() == list(range(32, 48)) and nz[32].tolist() == list(range(16, 32))
