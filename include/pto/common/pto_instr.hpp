@@ -194,7 +194,20 @@ PTO_FRONT(TREM, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a 
 PTO_FRONT(TFMOD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TNOT, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 PTO_FRONT(TGATHERB, typename D PTO_C typename S PTO_C typename O, D &dst PTO_C S &src PTO_C O &offset, (dst, src, offset))
+#if defined(PTO_TSCATTER_FLAT_INDEX)
+// the NPU implementation's TSCATTER: indices are element numbers of the destination (npu/a2a3/TScatter.hpp:17-36)
+template <typename D, typename S, typename I, typename... Ev>
+PTO_INST RecordEvent TSCATTER(D &dst, S &src, I &indexes, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(dst, src, indexes);
+    TSCATTER_FLAT_IMPL(dst, src, indexes);
+    detail::UbCommit(dst);
+    return {};
+}
+#else
 PTO_FRONT(TSCATTER, typename D PTO_C typename I, D &dst PTO_C D &src PTO_C I &indexes, (dst, src, indexes))
+#endif
 PTO_FRONT(MSCATTER, typename G PTO_C typename S PTO_C typename I, G &dst PTO_C S &src PTO_C I &indexes, (dst, src, indexes))
 PTO_FRONT(TPARTADD, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))
 PTO_FRONT(TPARTMAX, typename D PTO_C typename A PTO_C typename B, D &dst PTO_C A &a PTO_C B &b, (dst, a, b))

@@ -284,7 +284,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             const int r = e / TileT::Cols, c = e % TileT::Cols;
             T v = pad;
             if (r < vr && c < vc)
-                v = gm[(int64_t)r * st_r + (int64_t)c * st_c];
+                v = gm[gm_elem_offset(src, r, c)]; // ND / DN views with stacked outer dimensions, NZ memory
             *reinterpret_cast<T *>(lds + Geo::elem_off(r, c)) = v;
         }
     }

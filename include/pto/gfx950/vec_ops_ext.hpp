@@ -920,6 +920,47 @@ PTO_DEV void TSCATTER_IMPL(TileT &dst, TileT &src, IdxT &indexes)
     hw::lds_barrier();
 }
 
+// TSCATTER as the NPU implementation defines it (npu/a2a3/TScatter.hpp:17-36): the index tile holds element numbers of the
+// destination's storage, dst[indexes[i, j]] = src[i, j] over the index tile's valid region, walked in row-major order (the
+// last writer of an element wins: found with an atomic maximum over i * cols + j).  The index tile may have another shape
+// than the source.  Translation units choose this form with PTO_TSCATTER_FLAT_INDEX; the default is the CPU simulation's
+// row-index form above.
+template <typename DstT, typename SrcT, typename IdxT>
+PTO_DEV void TSCATTER_FLAT_IMPL(DstT &dst, SrcT &src, IdxT &indexes)
+{
+    using T = typename DstT::DType;
+    static_assert(DstT::Loc == TileType::Vec && SrcT::Loc == TileType::Vec && IdxT::Loc == TileType::Vec && DstT::isRowMajor && SrcT::isRowMajor &&
+                      IdxT::isRowMajor && std::is_same_v<T, typename SrcT::DType> && std::is_integral_v<typename IdxT::DType>,
+                  "[PTO][SA] TSCATTER: row-major Vec tiles, destination and source of one type, integer indices");
+    constexpr int N = DstT::Numel;
+    int *owner = reinterpret_cast<int *>(detail::stage_buffer<detail::stage_bytes((4 + (int)sizeof(T)) * N)>());
+    T *value = reinterpret_cast<T *>(owner + N);
+    for (int e = hw::tid(); e < N; e += kBlockThreads)
+        owner[e] = -1;
+    detail::Conformed<IdxT, SrcT> c(src); // src (i, j) in the lane that holds index (i, j)
+    hw::lds_barrier();
+    const int vr = indexes.GetValidRow(), vc = indexes.GetValidCol();
+    detail::for_each_owned<IdxT>([&](int s, int i, int e) {
+        const int r = e / IdxT::Cols, col = e % IdxT::Cols;
+        const uint32_t to = (uint32_t)(int)indexes.S().v[s][i];
+        if (e < IdxT::Numel && r < vr && col < vc && to < (uint32_t)N)
+            atomicMax(&owner[to], e);
+    });
+    hw::lds_barrier();
+    detail::for_each_owned<IdxT>([&](int s, int i, int e) {
+        const int r = e / IdxT::Cols, col = e % IdxT::Cols;
+        const uint32_t to = (uint32_t)(int)indexes.S().v[s][i];
+        if (e < IdxT::Numel && r < vr && col < vc && to < (uint32_t)N && owner[to] == e)
+            value[to] = c.S().v[s][i];
+    });
+    hw::lds_barrier();
+    detail::for_each_owned<DstT>([&](int s, int i, int e) {
+        if (e < N && owner[e] >= 0)
+            dst.S().v[s][i] = value[e];
+    });
+    hw::lds_barrier();
+}
+
 // MSCATTER (cpu/MGatherScatter.hpp:46-69): memory[indexes[i, j]] = src[i, j] over the source's valid region, the dual of
 // MGATHER.  Elements sent to the same address: the reference keeps the last in row-major order, here one of them
 // arrives last - callers that need the reference's result pass distinct indices.

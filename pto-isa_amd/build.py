@@ -149,7 +149,7 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
               "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract",
               "tmax", "tmin", "tmins", "texpands", "tsels", "tsort32", "tgather", "tmrgsort", "tstore",
-              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant"]
+              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant", "tscatter", "tgatherb", "tstore_mat2gm"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
 _ST_KEYED = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<[^;]*?>>>\s*\(([^;]*)\)\s*;")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
@@ -163,6 +163,10 @@ ST_PORT_OPTIONS = {
 }
 # its top-k kernel works through Vec tiles that are views of one another (TASSIGN to the same address)
 ST_PORT_OPTIONS["tmrgsort"] = dict(vec_in_memory=True)
+# the NPU form of TSCATTER (indices are element numbers of the destination; the CPU simulation's are row numbers)
+ST_PORT_OPTIONS["tscatter"] = dict(defines=["PTO_TSCATTER_FLAT_INDEX"])
+# three of its kernels keep more than 160 KiB of L1 tiles: they end at their TASSIGN and are not run
+ST_PORT_OPTIONS["tstore_mat2gm"] = dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL"])
 # multiplies in one function and declares the accumulator tile again, at the same address, in the next: tiles as addresses
 ST_PORT_OPTIONS["tmov_acc2mat"] = dict(vec_in_memory=True)
 # sources that keep their device code under the Ascend device compiler's own macro

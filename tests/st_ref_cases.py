@@ -1056,6 +1056,79 @@ SPECS["tdequant"] = dict(fn="LaunchTDequant", planner=plan_dequant, inputs="any"
                          r">\(float\*, [a-z ]+\*, float\*, float\*, void\*\)")
 
 
+# ---- TSTORE of Mat tiles: the tstore launcher and cases again, through L1 (tstore_mat2gm_kernel.cpp:17-121); cases whose
+# tile is larger than a compute unit's LDS end at their TASSIGN and are not run
+def store_mat_runnable(spec, m):
+    g = [int(m.group("g%d" % k)) for k in range(5)]
+    size = {"long": 8, "float": 4, "short": 2, "signed char": 1, "unsigned short": 2}[m.group("T")]
+    block = 32 // size
+    up = lambda x: (x + block - 1) // block * block
+    fmt = int(m.group("fmt"))
+    if fmt == 0:
+        numel = g[0] * g[1] * g[2] * g[3] * up(g[4])
+    elif fmt == 1:
+        numel = up(g[3]) * g[0] * g[1] * g[2] * g[4]
+    else:
+        numel = g[2] * g[3] * g[0] * g[1] * g[4]
+    return numel * size <= 160 * 1024
+
+
+SPECS["tstore_mat2gm"] = dict(SPECS["tstore"], lib="tstore_mat2gm", runnable=store_mat_runnable)
+
+
+# ---- TSCATTER, the NPU form: launchTScatterTestCase<N>(out, src, indexes, stream); kernel N fixes <T, TI, rows, cols, idxRows,
+# idxCols, ...>: out.flat[indexes[i, j]] = src[i, j] in row-major order of (i, j); what no index names is not defined
+# (tscatter_kernel.cpp:17-57, tscatter/gen_data.py:11-22)
+def plan_scatter_flat(test, spec, m):
+    t = manifest()[spec["lib"]]["cases"][m.group("case")]["targs"]
+    dt = np.dtype({"int16_t": np.int16, "half": np.float16, "int32_t": np.int32, "float": np.float32, "int8_t": np.int8}[t[0]])
+    it = np.dtype({"uint16_t": np.uint16, "int16_t": np.int16, "uint32_t": np.uint32, "int32_t": np.int32}[t[1]])
+    r0, c0, r1, c1 = (int(x) for x in t[2:6])
+
+    def scatter(arrays):
+        out = np.zeros(r0 * c0, dtype=dt)
+        written = np.zeros(r0 * c0, dtype=bool)
+        src, idx = arrays[0], arrays[1]
+        for i in range(r1):
+            for j in range(c1):
+                out[int(idx[i, j])] = src[i, j]
+                written[int(idx[i, j])] = True
+        return out.reshape(r0, c0), written.reshape(r0, c0)
+
+    pl = _plan(spec, [(dt, (r0, c0))], [(dt, (r0, c0), "any"), (it, (r1, c1), ("below", r0 * c0))], [(r0, c0)], lambda a: [scatter(a)[0]])
+    pl.compare = lambda got, want, arrays: np.array_equal(got[scatter(arrays)[1]].view(np.uint8), want[scatter(arrays)[1]].view(np.uint8))
+    return pl
+
+
+SPECS["tscatter"] = dict(fn="launchTScatterTestCase", lib="tscatter", planner=plan_scatter_flat, inputs="any",
+                         tail=r"<(?P<case>\d+)u>\(void\*, void\*, void\*, (?:ihipStream_t|void)\*\)")
+
+
+# ---- TGATHERB: LaunchTGatherB<T, dstRows, dstCols, offRows, offCols, srcRows, srcCols>(out, src, offset, stream): every 32-byte
+# block of out = the 32 bytes at byte offset[r, block] of src (tgatherb_kernel.cpp:17-60, tgatherb/gen_data.py:12-40)
+def plan_gatherb(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    q = _ints(m, ["dr", "dc", "orr", "oc", "sr", "sc"])
+    per = 32 // dt.itemsize
+    src_bytes = q["sr"] * q["sc"] * dt.itemsize
+
+    def expect(arrays):
+        raw = arrays[0].reshape(-1).view(np.uint8)
+        off = arrays[1].astype(np.int64)
+        blocks = raw[(off[:, :, None] + np.arange(32)[None, None, :])]          # [rows, blocks, 32]
+        return [blocks.reshape(q["dr"], -1).view(dt)[:, :q["dc"]]]
+    pl = _plan(spec, [(dt, (q["dr"], q["dc"]))], [(dt, (q["sr"], q["sc"]), "bits" if dt.kind in "iu" else "any"),
+                                                   (np.dtype(np.uint32), (q["orr"], q["oc"]), ("blocks", src_bytes))], [(q["dr"], q["dc"])], expect)
+    assert q["oc"] * per == q["dc"] and q["orr"] == q["dr"]
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    return pl
+
+
+SPECS["tgatherb"] = dict(fn="LaunchTGatherB", planner=plan_gatherb, inputs="any",
+                         tail=r"<(?P<T>[A-Za-z_0-9 ]+)" + "".join(r", (?P<%s>\d+)ul?" % k for k in ("dr", "dc", "orr", "oc", "sr", "sc")) +
+                         r">\([A-Za-z_0-9 ]+\*, [A-Za-z_0-9 ]+\*, unsigned int\*, void\*\)")
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
@@ -1063,6 +1136,10 @@ def lib_of(test):
 
 def draw(rng, dt, shape, kind, j):
     """Operand j of a test whose operation is of the given kind."""
+    if isinstance(kind, tuple) and kind[0] == "below":       # indices below kind[1]
+        return rng.integers(0, kind[1], size=shape).astype(dt)
+    if isinstance(kind, tuple) and kind[0] == "blocks":      # byte offsets of whole 32-byte blocks inside kind[1] bytes
+        return (rng.integers(0, kind[1] // 32, size=shape) * 32).astype(dt)
     if isinstance(kind, tuple) and kind[0] == "range":
         return rng.uniform(kind[1], kind[2], size=shape).astype(dt)
     if isinstance(kind, tuple) and kind[0] == "corner":      # small integers in the [vr, vc] corner, zeros around it
