@@ -149,7 +149,9 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
               "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract",
               "tmax", "tmin", "tmins", "texpands", "tsels", "tsort32", "tgather", "tmrgsort", "tstore",
-              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant", "tscatter", "tgatherb", "tstore_mat2gm"]
+              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant", "tscatter", "tgatherb", "tstore_mat2gm",
+              "a5_tadd_tdiv", "a5_tmul_tadds", "a5_tmuls_trowsum", "a5_trowsum_trowexpand", "a5_trowexpand_tdiv", "a5_trowexpand_tsqrt",
+              "a5_trowexpand_trowsum", "a5_tsub_texp"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
 _ST_KEYED = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<[^;]*?>>>\s*\(([^;]*)\)\s*;")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)
@@ -218,7 +220,9 @@ def build_ported_st(verbose=True, jobs=8):
     os.makedirs(out_dir, exist_ok=True)
 
     def one(name):
-        rel = "tests/npu/a2a3/src/st/testcase/%s/%s_kernel.cpp" % (name, name)
+        # "a5_<op>": the test source of that name in the a5 tree (instruction sequences that the a2a3 tree does not have)
+        arch, op = ("a5", name[3:]) if name.startswith("a5_") else ("a2a3", name)
+        rel = "tests/npu/%s/src/st/testcase/%s/%s_kernel.cpp" % (arch, op, op)
         lib = os.path.join(out_dir, name + ".so")
         rc, err = port_and_compile(rel, [], 160 * 1024, lib, extra_flags=("-Wno-unknown-attributes",), **ST_PORT_OPTIONS.get(name, {}))
         if rc != 0:

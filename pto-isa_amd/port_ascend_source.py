@@ -89,6 +89,21 @@ def kernel_before(text, pos):
             return None
         while i > 0 and text[i - 1].isspace():
             i -= 1
+    # a name that a macro call pastes together (`CONCAT(run, CASENAME)<...>`): the call belongs to the expression
+    if i > 0 and text[i - 1] == ")":
+        depth = 0
+        while i > 0:
+            i -= 1
+            if text[i] == ")":
+                depth += 1
+            elif text[i] == "(":
+                depth -= 1
+                if depth == 0:
+                    break
+            elif text[i] in ";{}":
+                return None
+        if depth != 0:
+            return None
     start = i
     while start > 0 and (text[start - 1].isalnum() or text[start - 1] in "_:"):
         start -= 1

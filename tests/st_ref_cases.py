@@ -1129,6 +1129,37 @@ SPECS["tgatherb"] = dict(fn="LaunchTGatherB", planner=plan_gatherb, inputs="any"
                          r">\([A-Za-z_0-9 ]+\*, [A-Za-z_0-9 ]+\*, unsigned int\*, void\*\)")
 
 
+# ---- pairs of instructions from the a5 tree: Launch<A>_<B><T, tileRows, tileCols, validRows, validCols>(out, src0, src1[, src2],
+# stream): all tiles [tileRows, tileCols], memory rows tileCols apart; every instruction rounds to T on its own
+# (tests/npu/a5/src/st/testcase/tadd_tdiv/tadd_tdiv_kernel.cpp:20-55 and its seven siblings, and their gen_data.py)
+def plan_pair(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    tr, tc, vr, vc = (int(m.group(k)) for k in ("tr", "tc", "vr", "vc"))
+    rnd = (lambda x: x.astype(dt)) if dt.kind == "f" else (lambda x: x.astype(np.int64).astype(dt))
+    wide = (lambda x: x.astype(np.float64)) if dt.kind == "f" else (lambda x: x.astype(np.int64))
+    f = spec["formula"]
+
+    def expect(arrays):
+        return [f(*[wide(a[:, :vc]) for a in arrays], rnd=lambda x: wide(rnd(x)), vc=vc)]
+    region = (vr, 1) if spec["col0"] else (vr, vc)
+    return _plan(spec, [(dt, (vr, tc))], [(dt, (vr, tc))] * spec["nin"], [region], expect)
+
+
+_PAIRS = {
+    "tadd_tdiv": ("LaunchTADD_TDIV", 3, False, lambda a, b, c, rnd, vc: rnd(a + b) / c),
+    "tmul_tadds": ("LaunchTMUL_TADDS", 3, False, lambda a, b, c, rnd, vc: rnd(a * b) + c[0, 0]),
+    "tmuls_trowsum": ("LaunchTMULS_TROWSUM", 3, True, lambda a, b, c, rnd, vc: rnd(a * b[0, 0]).sum(axis=1, keepdims=True)),
+    "trowsum_trowexpand": ("LaunchTROWSUM_TROWEXPAND", 2, False, lambda a, b, rnd, vc: np.repeat(rnd(a.sum(axis=1, keepdims=True)), vc, axis=1)),
+    "trowexpand_tdiv": ("LaunchTROWEXPAND_TDIV", 2, False, lambda a, b, rnd, vc: a[:, :1] / b),
+    "trowexpand_tsqrt": ("LaunchTROWEXPAND_TSQRT", 2, False, lambda a, b, rnd, vc: np.repeat(np.sqrt(a[:, :1]), vc, axis=1)),
+    "trowexpand_trowsum": ("LaunchTROWEXPAND_TROWSUM", 2, True, lambda a, b, rnd, vc: a[:, :1] * vc),
+    "tsub_texp": ("LaunchTSUB_TEXP", 2, False, lambda a, b, rnd, vc: np.exp(rnd(a - b))),
+}
+for _name, (_fn, _nin, _col0, _formula) in _PAIRS.items():
+    SPECS["a5_" + _name] = dict(fn=_fn, lib="a5_" + _name, planner=plan_pair, inputs="pos", nin=_nin, col0=_col0, formula=_formula,
+                                tail=TAIL(["tr", "tc", "vr", "vc"], _nin + 1), tol=REDUCE_TOL, atol=REDUCE_ATOL)
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)

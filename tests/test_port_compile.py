@@ -107,6 +107,14 @@ void Launch(float *out, void *stream)
     assert text.startswith("#define PTO_TILE_COPY_WRITEBACK 1\n#define PTO_VEC_TILES_IN_MEMORY 1\n#define __DAV_VEC__ 1\n")
     begin, end, launch = text.index("PTO_DEVICE_CODE_BEGIN"), text.index("PTO_DEVICE_CODE_END"), text.index("void Launch")
     assert begin < text.index("AICORE inline int counter") and text.index("void kern") < end < launch
+    # the kernel expression in front of a launch: plain, with template arguments, with a name pasted by a macro call
+    # (tests/npu/a5/src/st/testcase/tmuls_trowsum/tmuls_trowsum_kernel.cpp:59-63) - each gets its static LDS taken off
+    for expr in ("kern", "ns::kern<float, 4>", "CONCAT(run, CASENAME)<half, kRows, kCols>"):
+        line = "    %s<<<1, nullptr, stream>>>(out);" % expr
+        assert mod.kernel_before(line, line.index("<<<")) == expr
+    asm = 'uint64_t t; asm volatile("MOV %0, SYS_CNT\\n" : "+l"(t)); asm volatile("MOV %0, PC\\n" : "+l"(pc));'
+    assert mod.ASCEND_SREG_READ.sub(lambda m: "%s = %s;" % (m.group(2), "get_sys_cnt()" if m.group(1) == "SYS_CNT" else "0"), asm) == \
+        "uint64_t t; t = get_sys_cnt(); pc = 0;"
 
 
 SNIPPET = r"""
