@@ -80,7 +80,15 @@ PTO_DEV void UbCommit(T &dst, Rest &...)
     }
 #define PTO_C ,
 
-PTO_FRONT(TLOAD, typename TileT PTO_C typename G, TileT &dst PTO_C G &src, (dst, src))
+template <typename TileT, typename G, typename... Ev>
+PTO_INST RecordEvent TLOAD(TileT &dst, G &src, Ev &... ev)
+{
+    TSYNC(ev...);
+    TLOAD_IMPL(dst, src);
+    if constexpr (is_tile_data_v<TileT>)
+        detail::UbCommitLoaded(dst);
+    return {};
+}
 PTO_FRONT(TEXTRACT, typename D PTO_C typename S, D &dst PTO_C S &src PTO_C uint16_t idxRow PTO_C uint16_t idxCol,
           (dst, src, idxRow, idxCol))
 PTO_FRONT(TMATMUL, typename C PTO_C typename A PTO_C typename B, C &c PTO_C A &a PTO_C B &b, (c, a, b))

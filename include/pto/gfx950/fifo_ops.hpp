@@ -55,6 +55,32 @@ PTO_DEV void UbFetchTile(TileT &t)
     (void)t;
 #endif
 }
+// after a TLOAD: the valid region and, as the NPU's copy into the unified buffer does, the pad value up to the end of the
+// last 32-byte block of every valid row (column, for a column-major tile): what another tile object at the same address
+// then finds there (tests/npu/a2a3/src/st/testcase/tload/tload_kernel.cpp:121-150 stores through such a second tile)
+template <typename TileT>
+PTO_DEV void UbCommitLoaded(TileT &t)
+{
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+    if constexpr (TileT::inMemory) {
+        if (t.mem_ != nullptr) {
+            typename TileT::DType *p = t.mem_;
+            constexpr int kBlock = 32 / (int)sizeof(typename TileT::DType) > 0 ? 32 / (int)sizeof(typename TileT::DType) : 1;
+            const int vr = t.GetValidRow(), vc = t.GetValidCol();
+            const int pr = TileT::isRowMajor ? vr : (vr + kBlock - 1) / kBlock * kBlock, pc = TileT::isRowMajor ? (vc + kBlock - 1) / kBlock * kBlock : vc;
+            for_each_owned<TileT>([&](int s, int i, int e) {
+                int r, c;
+                elem_rc<TileT>(e, r, c);
+                if (e < TileT::Numel && r < pr && c < pc)
+                    p[e] = t.S().v[s][i];
+            });
+        }
+        UbSyncPoint();
+    }
+#else
+    (void)t;
+#endif
+}
 template <typename TileT>
 PTO_DEV void UbCommitTile(TileT &t)
 {

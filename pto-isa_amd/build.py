@@ -149,7 +149,7 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tcolexpandadd", "tcolexpandsub", "tcolexpandmul", "tcolexpanddiv", "tcolexpandmax", "tcolexpandmin", "tcolexpandexpdif",
               "tcmp", "tcmps", "tsel", "ttri", "trowsum", "trowmax", "trowmin", "tcvt", "tmatmul", "textract",
               "tmax", "tmin", "tmins", "texpands", "tsels", "tsort32", "tgather", "tmrgsort", "tstore",
-              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant", "tscatter", "tgatherb", "tstore_mat2gm",
+              "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant", "tscatter", "tgatherb", "tstore_mat2gm", "tci", "tload",
               "a5_tadd_tdiv", "a5_tmul_tadds", "a5_tmuls_trowsum", "a5_trowsum_trowexpand", "a5_trowexpand_tdiv", "a5_trowexpand_tsqrt",
               "a5_trowexpand_trowsum", "a5_tsub_texp"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
@@ -169,6 +169,8 @@ ST_PORT_OPTIONS["tmrgsort"] = dict(vec_in_memory=True)
 ST_PORT_OPTIONS["tscatter"] = dict(defines=["PTO_TSCATTER_FLAT_INDEX"])
 # three of its kernels keep more than 160 KiB of L1 tiles: they end at their TASSIGN and are not run
 ST_PORT_OPTIONS["tstore_mat2gm"] = dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL"])
+# stores through a second tile object at the address of the one it loaded: tiles as addresses
+ST_PORT_OPTIONS["tload"] = dict(vec_in_memory=True)
 # multiplies in one function and declares the accumulator tile again, at the same address, in the next: tiles as addresses
 ST_PORT_OPTIONS["tmov_acc2mat"] = dict(vec_in_memory=True)
 # sources that keep their device code under the Ascend device compiler's own macro

@@ -1160,6 +1160,49 @@ for _name, (_fn, _nin, _col0, _formula) in _PAIRS.items():
                                 tail=TAIL(["tr", "tc", "vr", "vc"], _nin + 1), tol=REDUCE_TOL, atol=REDUCE_ATOL)
 
 
+# ---- TCI: launchTCI_demo_b32_case<N><d>(out, stream) / ..._b16_...: out[0, j] = START +- j; the kernels fix columns and
+# direction through macros (tci_common.h:11-26: START 0; b32 columns 128, 600, 32, 2000, b16 256, 800, 64, 5120;
+# tci_kernel.cpp:36-67: b32 cases 3 and 4, b16 cases 2 and 4 count down); the launcher's template argument is not used
+_TCI = {("b32", 1): (128, 0), ("b32", 2): (600, 0), ("b32", 3): (32, 1), ("b32", 4): (2000, 1),
+        ("b16", 1): (256, 0), ("b16", 2): (800, 1), ("b16", 3): (64, 0), ("b16", 4): (5120, 1)}
+
+
+def plan_ci(test, spec, m):
+    cols, down = _TCI[(m.group("w"), int(m.group("case")))]
+    dt = np.dtype(np.int32 if m.group("w") == "b32" else np.int16)
+    return _plan(spec, [(dt, (1, cols))], [], [(1, cols)], lambda a: [((-1 if down else 1) * np.arange(cols)).astype(dt)[None, :]])
+
+
+SPECS["tci"] = dict(fn="launchTCI_demo_", lib="tci", planner=plan_ci, inputs="any", tail=r"(?P<w>b32|b16)_case(?P<case>\d)<[01]u>\((?:int|short)\*, void\*\)")
+
+
+# ---- TLOAD: launchTLOAD<N>(out, src, log, stream); kernel N fixes <T, s0, s1, s2, s3, s4, tileRows, tileCols, dyn, pad>: the
+# [s0, s1, s2, s3, s4] tensor, in as many blocks as the launcher asks for, each loading its rows of every slab into one
+# tile and storing it through a second tile object at the same address; out is [s0, s1, s2, s3, s4 rounded up to 32 bytes]
+# with the pad value in the added columns (tload_kernel.cpp:97-150; golden :253-300)
+def plan_load(test, spec, m):
+    t = manifest()[spec["lib"]]["cases"]["%s:%s" % (spec["fn"], m.group("case"))]["targs"]
+    dt = np.dtype({"float": np.float32, "int16_t": np.int16, "uint8_t": np.uint8, "int64_t": np.int64, "uint64_t": np.uint64}[t[0]])
+    s = [int(x) for x in t[1:6]]
+    per = 32 // dt.itemsize
+    aligned = (s[4] + per - 1) // per * per
+    which = t[9].split("::")[1]
+    pad = _pad_value(dt, which) if which in ("Max", "Min") else dt.type(0)
+    rows = s[0] * s[1] * s[2] * s[3]
+
+    def expect(arrays):
+        out = np.full((rows, aligned), pad, dtype=dt)
+        out[:, :s[4]] = arrays[0]
+        return [out]
+    pl = _plan(spec, [(dt, (rows, aligned))], [(dt, (rows, s[4]), "bits" if dt.kind in "iu" else "any"), (np.dtype(np.uint64), (1, 128 * 32), "any")],
+               [(rows, aligned)], expect)
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(np.uint8), want.view(np.uint8))
+    return pl
+
+
+SPECS["tload"] = dict(fn="launchTLOAD", lib="tload", tail=r"<(?P<case>\d+)>\(unsigned char\*, unsigned char\*, unsigned long\*, void\*\)", planner=plan_load, inputs="any")
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
