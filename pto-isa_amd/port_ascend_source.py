@@ -230,6 +230,12 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
             host = "<<<" in body or re.match(r"\s*template\s+(?!<)", lines[start]) is not None or \
                 re.match(r'\s*extern\s+"C"\s+(?!.*__global__)', lines[start]) is not None and "AICORE" not in lines[start]
             marked = re.search(r"\b(AICORE|__aicore__|__global__|PTO_INTERNAL|PTO_INST)\b", body.split("{", 1)[0]) is not None
+            # the declaration of a host function (no body, no device marker: `template <...> void Launch(T *out, void *stream);`,
+            # specialised further down with the launches in the bodies) is host code too
+            flat = " ".join(strip_code(x) for x in lines[start:i + 1]).strip()
+            if not host and not marked and "{" not in flat and \
+                    re.match(r"^(template\s*<[^;{}]*>\s*)?(?!static_assert|using|typedef|return)[\w:]+[\w:<>,\*&\s]*?\b\w+\s*\([^;{}]*\)\s*;$", flat):
+                host = True
             chunks.append((start, i, host, marked))
             start = None
     res, pos, open_region, regions = lines[:first_dev], first_dev, False, 0

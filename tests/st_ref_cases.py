@@ -1118,7 +1118,7 @@ def plan_gatherb(test, spec, m):
         blocks = raw[(off[:, :, None] + np.arange(32)[None, None, :])]          # [rows, blocks, 32]
         return [blocks.reshape(q["dr"], -1).view(dt)[:, :q["dc"]]]
     pl = _plan(spec, [(dt, (q["dr"], q["dc"]))], [(dt, (q["sr"], q["sc"]), "bits" if dt.kind in "iu" else "any"),
-                                                   (np.dtype(np.uint32), (q["orr"], q["oc"]), ("blocks", src_bytes))], [(q["dr"], q["dc"])], expect)
+                                                   (np.dtype(np.uint32), (q["orr"], q["oc"]), ("block_offsets", src_bytes))], [(q["dr"], q["dc"])], expect)
     assert q["oc"] * per == q["dc"] and q["orr"] == q["dr"]
     pl.compare = lambda got, want, arrays: np.array_equal(got.view(np.uint8), want.view(np.uint8))
     return pl
@@ -1203,6 +1203,44 @@ def plan_load(test, spec, m):
 SPECS["tload"] = dict(fn="launchTLOAD", lib="tload", tail=r"<(?P<case>\d+)>\(unsigned char\*, unsigned char\*, unsigned long\*, void\*\)", planner=plan_load, inputs="any")
 
 
+# ---- MGATHER / MSCATTER (a5 tree): LaunchMGATHER<T, TIdx, tableRows, tableCols, outRows, outCols>(out, table, indices, stream),
+# out[i, j] = table.flat[indices[i, j]]; LaunchMSCATTER<T, TIdx, srcRows, srcCols, outSize>(out, src, indices, stream),
+# out[indices[i, j]] = src[i, j], the rest of out untouched; the Half launchers take fp16 as uint16
+# (tests/npu/a5/src/st/testcase/mgather/mgather_kernel.cpp:17-46, mscatter/mscatter_kernel.cpp:19-60 and their gen_data.py)
+def plan_mgather(test, spec, m):
+    dt = np.dtype(np.float16) if spec["half"] else _elem(m.group("T"), False)[0]
+    tr, tc, orr, oc = (int(m.group(k)) for k in ("tr", "tc", "orr", "oc"))
+    pl = _plan(spec, [(dt, (orr, oc))], [(dt, (tr, tc), "bits" if dt.kind in "iu" else "any"), (np.dtype(np.int32), (orr, oc), ("below", tr * tc))],
+               [(orr, oc)], lambda a: [a[0].reshape(-1)[a[1]]])
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(np.uint8), np.ascontiguousarray(want).view(np.uint8))
+    return pl
+
+
+def plan_mscatter(test, spec, m):
+    dt = np.dtype(np.float16) if spec["half"] else _elem(m.group("T"), False)[0]
+    sr, sc, n = (int(m.group(k)) for k in ("sr", "sc", "n"))
+
+    def expect(a):
+        out = np.full(n, 77, dtype=dt)
+        out[a[1].reshape(-1)] = a[0].reshape(-1)
+        return [out[None, :]]
+    pl = _plan(spec, [(dt, (1, n))], [(dt, (sr, sc), "bits" if dt.kind in "iu" else "any"), (np.dtype(np.int32), (sr, sc), ("distinct", n))], [(1, n)], expect)
+    pl.compare = lambda got, want, arrays: np.array_equal(got.view(np.uint8), np.ascontiguousarray(want).view(np.uint8))
+    return pl
+
+
+_G4 = "".join(r", (?P<%s>\d+)" % k for k in ("tr", "tc", "orr", "oc"))
+_S3 = "".join(r", (?P<%s>\d+)" % k for k in ("sr", "sc", "n"))
+SPECS["a5_mgather"] = dict(fn="LaunchMGATHER", lib="a5_mgather", planner=plan_mgather, inputs="any", half=False,
+                           tail=r"<(?P<T>[a-z ]+), int" + _G4 + r">\((?:[a-z ]+\*, ){2}int\*, void\*\)")
+SPECS["a5_mgather:half"] = dict(fn="LaunchMGATHERHalf", lib="a5_mgather", planner=plan_mgather, inputs="any", half=True,
+                                tail=r"<" + _G4[2:] + r">\((?:unsigned short\*, ){2}int\*, void\*\)")
+SPECS["a5_mscatter"] = dict(fn="LaunchMSCATTER", lib="a5_mscatter", planner=plan_mscatter, inputs="any", half=False,
+                            tail=r"<(?P<T>[a-z ]+), int" + _S3 + r">\((?:[a-z ]+\*, ){2}int\*, void\*\)")
+SPECS["a5_mscatter:half"] = dict(fn="LaunchMSCATTERHalf", lib="a5_mscatter", planner=plan_mscatter, inputs="any", half=True,
+                                 tail=r"<" + _S3[2:] + r">\((?:unsigned short\*, ){2}int\*, void\*\)")
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
@@ -1210,9 +1248,11 @@ def lib_of(test):
 
 def draw(rng, dt, shape, kind, j):
     """Operand j of a test whose operation is of the given kind."""
+    if isinstance(kind, tuple) and kind[0] == "distinct":    # distinct indices below kind[1]
+        return rng.permutation(kind[1])[:int(np.prod(shape))].reshape(shape).astype(dt)
     if isinstance(kind, tuple) and kind[0] == "below":       # indices below kind[1]
         return rng.integers(0, kind[1], size=shape).astype(dt)
-    if isinstance(kind, tuple) and kind[0] == "blocks":      # byte offsets of whole 32-byte blocks inside kind[1] bytes
+    if isinstance(kind, tuple) and kind[0] == "block_offsets":      # byte offsets of whole 32-byte blocks inside kind[1] bytes
         return (rng.integers(0, kind[1] // 32, size=shape) * 32).astype(dt)
     if isinstance(kind, tuple) and kind[0] == "range":
         return rng.uniform(kind[1], kind[2], size=shape).astype(dt)
