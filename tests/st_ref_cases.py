@@ -1241,6 +1241,31 @@ SPECS["a5_mscatter:half"] = dict(fn="LaunchMSCATTERHalf", lib="a5_mscatter", pla
                                  tail=r"<" + _S3[2:] + r">\((?:unsigned short\*, ){2}int\*, void\*\)")
 
 
+# ---- TPACK (a5 tree): TPackTest::LaunchTPack<rows, cols, Src, Dst>(dst, src, stream): the low bytes of every element
+# (tests/npu/a5/src/st/testcase/tpack/tpack_kernel.cpp:20-50, tpack/gen_data.py:10-38)
+def plan_pack(test, spec, m):
+    rows, cols = int(m.group("r")), int(m.group("c"))
+    sdt, ddt = _elem(m.group("S"), False)[0], _elem(m.group("D"), False)[0]
+    return _plan(spec, [(ddt, (rows, cols))], [(sdt, (rows, cols), "bits")], [(rows, cols)],
+                 lambda a: [(a[0].astype(np.uint64) & np.uint64((1 << (8 * ddt.itemsize)) - 1)).astype(ddt)])
+
+
+SPECS["a5_tpack"] = dict(fn="TPackTest::LaunchTPack", lib="a5_tpack", planner=plan_pack, inputs="bits",
+                         tail=r"<(?P<r>\d+), (?P<c>\d+), (?P<S>[a-z ]+), (?P<D>[a-z ]+)>\([a-z ]+\*, [a-z ]+\*, void\*\)")
+
+
+# ---- TROWEXPAND from a column tile (a5 tree): TRowExpandTest::launchTROWEXPAND<T, rows, cols>(out, src, stream):
+# out[r, c] = src[r] (tests/npu/a5/src/st/testcase/trowexpandbrcb/trowexpandbrcb_kernel.cpp:16-45)
+def plan_rowexpand_col(test, spec, m):
+    dt, _ = _elem(m.group("T"), True)
+    rows, cols = int(m.group("r")), int(m.group("c"))
+    return _plan(spec, [(dt, (rows, cols))], [(dt, (rows, 1), "any")], [(rows, cols)], lambda a: [np.repeat(a[0], cols, axis=1)])
+
+
+SPECS["a5_trowexpandbrcb"] = dict(fn="TRowExpandTest::launchTROWEXPAND", lib="a5_trowexpandbrcb", planner=plan_rowexpand_col, inputs="any",
+                                  tail=r"<(?P<T>[a-z ]+), (?P<r>\d+)u, (?P<c>\d+)u>\([a-z ]+\*, [a-z ]+\*, void\*\)", tol=EXACT)
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
