@@ -151,15 +151,22 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
     # 2. launch statements
     blocks = "pto::host::LaunchBlocks(%s, (hipStream_t)(%s))" if vec_in_memory else "%s"
 
+    unnamed = [0]
+
     def launch(m):
         b = blocks % (m.group(1), m.group(2)) if vec_in_memory else m.group(1)
         kernel = kernel_before(m.string, m.start())
         # the kernel's own static LDS (staging buffers of the tile library, PTO_CORE_STATIC slots) comes out of the same
         # 160 KiB: the dynamic part shrinks by it, or the dispatch would be refused by the hardware queue
         lds = "pto::host::LaunchLds((const void *)(%s), %d)" % (kernel, lds_bytes) if kernel else "%d" % lds_bytes
+        if not kernel:
+            unnamed[0] += 1
         return "<<<%s, pto::kBlockThreads, %s, (hipStream_t)(%s)>>>" % (b, lds, m.group(2))
     text, n = LAUNCH.subn(launch, text)
     notes.append("%d launch statement%s rewritten" % (n, "" if n == 1 else "s"))
+    if unnamed[0]:
+        notes.append("WARNING: %d launch%s whose kernel expression was not recognised keep the full dynamic LDS size; a kernel with "
+                     "__shared__ variables of its own then asks for more than a compute unit has" % (unnamed[0], "" if unnamed[0] == 1 else "es"))
 
     # 9. kernels are launched with pto::kBlockThreads threads: tell the compiler (it assumes 1024 otherwise and has half the
     # registers per thread to work with)
