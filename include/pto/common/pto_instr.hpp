@@ -682,20 +682,25 @@ PTO_INST RecordEvent TMATMUL(C &c, A &a, B &b, Ev &... ev)
 {
     TSYNC(ev...);
     TMATMUL_IMPL(c, a, b);
+    detail::UbCommit(c);
     return {};
 }
 template <AccPhase Phase, typename C, typename A, typename B, typename... Ev>
 PTO_INST RecordEvent TMATMUL_ACC(C &cOut, C &cIn, A &a, B &b, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(cIn);
     TMATMUL_ACC_IMPL(cOut, cIn, a, b);
+    detail::UbCommit(cOut);
     return {};
 }
 template <AccPhase Phase = AccPhase::Unspecified, typename C, typename A, typename B, typename... Ev>
 PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TMATMUL_ACC(C &c, A &a, B &b, Ev &... ev)
 {
     TSYNC(ev...);
+    detail::UbFetch(c);
     TMATMUL_ACC_IMPL(c, c, a, b);
+    detail::UbCommit(c);
     return {};
 }
 // TMATMUL_MX(c, a, aScale, b, bScale) and the accumulating form (cOut, cIn, a, aScale, b, bScale)  (pto_instr.hpp:403-440)

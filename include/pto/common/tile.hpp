@@ -60,6 +60,14 @@ constexpr bool kVecTilesInMemory = true;
 #else
 constexpr bool kVecTilesInMemory = false;
 #endif
+#if defined(PTO_ACC_TILES_IN_MEMORY)
+#if !defined(PTO_VEC_TILES_IN_MEMORY)
+#error "PTO_ACC_TILES_IN_MEMORY needs PTO_VEC_TILES_IN_MEMORY (the accumulator images live in the same per-workgroup arena)"
+#endif
+constexpr bool kAccTilesInMemory = true;
+#else
+constexpr bool kAccTilesInMemory = false;
+#endif
 
 static_assert(PTO_MFMA_M == 32 || PTO_MFMA_M == 16, "v_mfma_f32_32x32x16 or v_mfma_f32_16x16x32");
 constexpr int kMfmaM = PTO_MFMA_M;                     // the MFMA's output block is kMfmaM x kMfmaM
@@ -332,12 +340,12 @@ struct Tile {
     Tile *origin_ = nullptr; // register tiles: set in a copy, the tile it was copied from (values go back on destruction)
     // the object itself is an address: Mat tiles, and Vec tiles of a translation unit that keeps them in memory
     static constexpr bool inMemory = Loc_ == TileType::Vec && detail::kVecTilesInMemory;
-    // In such a translation unit an Acc tile that was given an address is an address too: every instruction that writes
+    // With PTO_ACC_TILES_IN_MEMORY as well, an Acc tile that was given an address is an address too: every instruction that writes
     // it stores its [Rows, Cols] image (row-major) there and every instruction that reads it loads it from there, so that
     // another Acc tile object TASSIGNed to the same address sees the accumulator (the reference's test kernels multiply
     // in one function and declare the tile again in the next: tests/npu/a2a3/src/st/testcase/tmov_acc2mat).  The values
     // still live in registers in between; the object is not a handle.
-    static constexpr bool accInMemory = Loc_ == TileType::Acc && detail::kVecTilesInMemory;
+    static constexpr bool accInMemory = Loc_ == TileType::Acc && detail::kAccTilesInMemory;
     static constexpr bool isHandle = Loc_ == TileType::Mat || inMemory;
 #if defined(PTO_VEC_TILES_IN_MEMORY)
     DType *mem_ = nullptr; // Vec tiles: element 0 of the tile in the unified buffer (nullptr: not assigned, registers only)

@@ -280,11 +280,12 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
         // general path: element by element, pad outside the valid region (TLoad.hpp:151-152)
         const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
         const T pad = pad_value<T>(TileT::PadVal);
+        const bool stacked = src.GetShape(0) * src.GetShape(1) * src.GetShape(2) != 1;
         for (int e = hw::tid(); e < TileT::Numel; e += kBlockThreads) {
             const int r = e / TileT::Cols, c = e % TileT::Cols;
             T v = pad;
-            if (r < vr && c < vc)
-                v = gm[gm_elem_offset(src, r, c)]; // ND / DN views with stacked outer dimensions, NZ memory
+            if (r < vr && c < vc) // views with stacked outer dimensions and NZ memory: by the 5-D rule; else rows and columns
+                v = (G::layout == Layout::NZ || stacked) ? gm[gm_elem_offset(src, r, c)] : gm[(int64_t)r * st_r + (int64_t)c * st_c];
             *reinterpret_cast<T *>(lds + Geo::elem_off(r, c)) = v;
         }
     }
@@ -846,10 +847,12 @@ PTO_DEV void tstore_mat(G &dst, TileT &src)
     const char *lds = hw::lds_base() + src.st.lds;
     T *gm = reinterpret_cast<T *>(dst.data());
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    const bool stacked = dst.GetShape(0) * dst.GetShape(1) * dst.GetShape(2) != 1;
     for (int e = hw::tid(); e < TileT::Numel; e += kBlockThreads) {
         const int r = e / TileT::Cols, c = e % TileT::Cols;
         if (r < vr && c < vc)
-            gm[gm_elem_offset(dst, r, c)] = *reinterpret_cast<const T *>(lds + Geo::elem_off(r, c));
+            gm[(G::layout == Layout::NZ || stacked) ? gm_elem_offset(dst, r, c) : (int64_t)r * dst.GetStride(3) + (int64_t)c * dst.GetStride(4)] =
+                *reinterpret_cast<const T *>(lds + Geo::elem_off(r, c));
     }
 }
 

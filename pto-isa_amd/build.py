@@ -172,7 +172,7 @@ ST_PORT_OPTIONS["tstore_mat2gm"] = dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KE
 # stores through a second tile object at the address of the one it loaded: tiles as addresses
 ST_PORT_OPTIONS["tload"] = dict(vec_in_memory=True)
 # multiplies in one function and declares the accumulator tile again, at the same address, in the next: tiles as addresses
-ST_PORT_OPTIONS["tmov_acc2mat"] = dict(vec_in_memory=True)
+ST_PORT_OPTIONS["tmov_acc2mat"] = dict(vec_in_memory=True, defines=["PTO_ACC_TILES_IN_MEMORY"])
 # sources that keep their device code under the Ascend device compiler's own macro
 for _name in ("tmax", "tmin", "tmins", "texpands"):
     ST_PORT_OPTIONS[_name] = dict(defines=["__CCE_AICORE__=220"])
