@@ -19,7 +19,7 @@ CASES = S.cases()
 def test_the_test_kernel_libraries_were_built():
     if not os.path.isdir(S.ST_DIR):
         pytest.skip("oracle/_ref/st not built (reference tree absent at build time)")
-    assert len(CASES) >= 700 and {c[0] for c in CASES} == set(S.SPECS)
+    assert len(CASES) >= 1100 and {c[0] for c in CASES} == set(S.SPECS)
 
 
 @pytest.mark.parametrize("test,mangled,demangled", CASES, ids=[c[2][5:].split("(")[0] for c in CASES])
