@@ -363,8 +363,43 @@ PTO_DEV void row_reduce(DstT &dst, SrcT &src)
     using A = float;
     using S = typename SrcT::Storage;
     constexpr int CPR = SrcT::Cols / kVecChunk; // chunks per row
-    __shared__ A part[S::Chunks];
     const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    // A row of at most 64 chunks whose count is a power of two lies in consecutive lanes of one wavefront: the lanes
+    // combine their chunks' partial results with a butterfly of wavefront shuffles (every lane of the row ends with the
+    // row's result), and one value per row goes through LDS to the lane that holds element (r, 0) of the destination.
+    if constexpr (CPR <= kWaveSize && (CPR & (CPR - 1)) == 0) {
+        __shared__ A rowval[SrcT::Rows];
+        auto op = [](A a, A b) { return KIND == 1 ? (a < b ? b : a) : KIND == 2 ? (b < a ? b : a) : KIND == 3 ? a * b : a + b; };
+#pragma unroll
+        for (int s = 0; s < S::Slots; ++s) {
+            const int q = s * kBlockThreads + hw::tid();
+            const int c0 = (q % CPR) * kVecChunk;
+            A acc = KIND == 1 ? -__builtin_huge_valf() : KIND == 2 ? __builtin_huge_valf() : KIND == 3 ? 1.0f : 0.0f;
+            if (q < S::Chunks) {
+#pragma unroll
+                for (int i = 0; i < kVecChunk; ++i)
+                    if (c0 + i < vc)
+                        acc = op(acc, (A)src.S().v[s][i]);
+            }
+#pragma unroll
+            for (int off = CPR / 2; off >= 1; off >>= 1)
+                acc = op(acc, __shfl_xor(acc, off, kWaveSize));
+            if (q < S::Chunks && q % CPR == 0)
+                rowval[q / CPR] = acc;
+        }
+        hw::lds_barrier();
+        for_each_owned<DstT>([&](int s, int i, int e) {
+            if (e < DstT::Numel) {
+                int r, c;
+                elem_rc<DstT>(e, r, c);
+                if (c == 0 && r < vr && r < SrcT::Rows)
+                    dst.S().v[s][i] = (typename DstT::DType)rowval[r];
+            }
+        });
+        hw::lds_barrier();
+        return;
+    }
+    __shared__ A part[S::Chunks];
 #pragma unroll
     for (int s = 0; s < S::Slots; ++s) {
         const int q = s * kBlockThreads + hw::tid();
