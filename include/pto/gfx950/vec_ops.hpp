@@ -3,8 +3,9 @@
 //
 // A Vec tile is spread over the workgroup's lanes in chunks of 8 consecutive elements of its
 // linear order (common/tile.hpp), so every elementwise instruction between tiles of equal shape
-// is lane-local VALU work.  Instructions that move data across lanes (row reductions, row
-// broadcasts, gathers) stage through a small statically allocated LDS buffer sized by the tile.
+// is lane-local VALU work.  Row reductions combine the chunks of a row with wavefront shuffles where a
+// row lies inside one wavefront; the other instructions that move data across lanes (row broadcasts,
+// gathers) stage through a small statically allocated LDS buffer sized by the tile.
 //
 // Reference semantics: include/pto/cpu/TCvt.hpp:65-92, TGather.hpp:58-129, MGatherScatter.hpp:21-44,
 // TRowMax.hpp:20-59, TRowSum.hpp:17-63, TRowExpandOp.hpp:37-96, TExp.hpp:22-60, TBinSOps.hpp,
