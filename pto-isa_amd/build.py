@@ -151,7 +151,7 @@ ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip
               "tmax", "tmin", "tmins", "texpands", "tsels", "tsort32", "tgather", "tmrgsort", "tstore",
               "tcolexpand", "ttrans", "trowprod", "tpartadd", "tpartmul", "tpartmax", "tpartmin", "tmov_acc2mat", "tstore_acc2gm", "tfillpad", "tquant", "tdequant", "tscatter", "tgatherb", "tstore_mat2gm", "tci", "tload",
               "a5_tadd_tdiv", "a5_tmul_tadds", "a5_tmuls_trowsum", "a5_trowsum_trowexpand", "a5_trowexpand_tdiv", "a5_trowexpand_tsqrt",
-              "a5_trowexpand_trowsum", "a5_tsub_texp", "a5_mgather", "a5_mscatter", "a5_tpack", "a5_trowexpandbrcb"]
+              "a5_trowexpand_trowsum", "a5_tsub_texp", "a5_mgather", "a5_mscatter", "a5_tpack", "a5_trowexpandbrcb", "a5_tpartmul", "a5_tfmods", "a5_tmov_vect"]
 _ST_CASE = re.compile(r"void\s+launch\w+?Case(\d+)\s*\(([^)]*)\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*\(")
 _ST_KEYED = re.compile(r"(?:tilingKey|testKey)\s*==\s*(\d+)\s*\)\s*\{\s*(\w+)\s*<([^;{}]*?)>\s*<<<[^;]*?>>>\s*\(([^;]*)\)\s*;")
 _ST_LAUNCHER = re.compile(r"^void\s+(\w+)\s*\(", re.M)

@@ -1266,6 +1266,11 @@ SPECS["a5_trowexpandbrcb"] = dict(fn="TRowExpandTest::launchTROWEXPAND", lib="a5
                                   tail=r"<(?P<T>[a-z ]+), (?P<r>\d+)u, (?P<c>\d+)u>\([a-z ]+\*, [a-z ]+\*, void\*\)", tol=EXACT)
 
 
+# ---- sources of the a5 tree whose launchers have the form of their a2a3 namesakes: the same planners
+for _name in ("tpartmul", "tfmods", "tmov_vect"):
+    SPECS["a5_" + _name] = dict(SPECS[_name], lib="a5_" + _name)
+
+
 def lib_of(test):
     """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
