@@ -14,16 +14,11 @@ extern "C" {
 
 /* ---- tuning hooks: one kernel variant each, whatever the dispatch of the public entry point would pick -------------
  * PTO_ERR_UNSUPPORTED where the variant has no tiling for the shape, PTO_ERR_BAD_ARG for an unknown variant. */
-/* four-wave / 128 x 256-block kernels on 32 x 32 x 16 MFMAs: tiling and pipeline depth by number (csrc/pto_gemm.hip) */
+/* the 128 x 256 / 256 x 256 block kernels on 32 x 32 x 16 MFMAs: tiling and pipeline depth by number (csrc/pto_gemm.hip) */
 int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
-/* the same kernels for workgroups of eight wavefronts (csrc/pto_gemm_w8.hip) */
-int pto_gemm_f16f32_w8_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
-/* eight wavefronts on 16 x 16 x 32 MFMAs: 0 / 3 = 256 x 256 tiles with / without quarter tiles in the last round,
- * 10 = 256 x 192, 12 = 384 x 192 (csrc/pto_gemm_m16.hip) */
-int pto_gemm_f16f32_m16_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
-/* four wavefronts on 16 x 16 x 32 MFMAs: 0 / 1 = 256 x 256 with / without quarter tiles, 2 = 192 x 256, 3 = 256 x 192,
- * 4 = 192 x 192 (csrc/pto_gemm_m16w4.hip) */
-int pto_gemm_f16f32_m16w4_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
+/* four wavefronts, 256-row tiles, K-steps of 64, A in a ring per wave: 0 = 256 x 256 tiles, 1 = 256 x 192, 2 = 256 x 128
+ * (csrc/pto_gemm_w4.hip) */
+int pto_gemm_f16f32_w4_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
 /* eight wavefronts on a 4 x 2 wave grid, K-steps of 64 (whole 128-byte lines), two LDS stages: 0 = 384 x 192 tiles,
  * 1 = 256 x 256, 2 = 256 x 192 (csrc/pto_gemm_k64.hip) */
 int pto_gemm_f16f32_k64_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);

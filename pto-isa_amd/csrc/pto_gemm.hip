@@ -1,6 +1,7 @@
 // fp16 x fp16 -> fp32 GEMM for MI355X written with PTO tile instructions:
 //   TLOAD (HBM -> LDS, async 16-byte copies)  ->  TEXTRACT (LDS -> MFMA operand fragments)
-//   ->  TMATMUL / TMATMUL_ACC (v_mfma_f32_32x32x16_f16)  ->  TSTORE (accumulators -> HBM).
+//   ->  TMATMUL / TMATMUL_ACC (v_mfma_f32_32x32x16_f16)  ->  TSTORE (accumulators -> HBM);
+// and the entry point that picks among it, the K-64 kernel of pto_gemm_k64.hip and the four-wave kernel of pto_gemm_w4.hip.
 //
 // Same decomposition as the reference's manual kernel
 // (kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp:67-230): each "core" owns
@@ -33,13 +34,6 @@ extern "C" int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a
     case 9: return launch_gemm<256, 256, 32, 3, 1, 8>(st, c, ha, hb, m, n, k);
     case 10: return launch_gemm<256, 256, 32, 4, 1, 4>(st, c, ha, hb, m, n, k);
     case 11: return launch_gemm<256, 256, 32, 2, 1, 8>(st, c, ha, hb, m, n, k);
-    case 30: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 2);
-    case 31: return launch_gemm_mix<256, 256, 3, 8>(st, c, ha, hb, m, n, k, 2);
-    case 32: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 2);
-    case 33: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 0);
-    case 35: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 3);
-    case 36: return launch_gemm_mix<256, 256, 4, 8>(st, c, ha, hb, m, n, k, 3);
-    case 34: return launch_gemm_mix<256, 256, 4, 4>(st, c, ha, hb, m, n, k, 0);
     default: return PTO_ERR_BAD_ARG;
     }
 }
@@ -51,27 +45,19 @@ extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const 
         return PTO_ERR_BAD_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
-    // Large problems: 256 x 256 C tiles (two thirds of the operand traffic per flop of the 128 x 256
-    // block), one workgroup of eight wavefronts per compute unit.  Problems with too few such tiles
-    // to fill the machine, or with extents that are not multiples of them: the 128 x 256 block of
-    // the reference kernel, two workgroups of four wavefronts per compute unit.
-    const bool big = m % 256 == 0 && n % 256 == 0 && k % 128 == 0 && k / 32 >= 8 &&
-                     (long long)(m / 256) * (n / 256) * 2 >= compute_units();
-    if (big) {
-        // tiles that (nearly) fill whole rounds over the compute units: the kernel with K-steps of 64 (every operand row a
-        // whole 128-byte line per step; interleaved runs: 6144^3 1336 against 1254 TFLOP/s, 8192^3 1329 against 1298)
+    // Problems with enough work for every compute unit: 256-row tiles on four wavefronts with K-steps of 64, the width
+    // chosen from 256 / 192 / 128 by the number of rounds it gives (pto_gemm_w4.hip).  Everything else (small problems,
+    // extents that are not multiples of those tiles): the 128 x 256 block of the reference kernel with K-steps of 32,
+    // two workgroups of four wavefronts per compute unit.
+    if ((long long)m * n >= (long long)compute_units() * 32768) {
+        const int rc = pto_amd::gemm_f16f32_w4(st, c, ha, hb, m, n, k);
+        if (rc != PTO_ERR_UNSUPPORTED)
+            return rc;
+        // shapes those tiles do not divide: the K-64 kernel written with the tile instructions (eight wavefronts, 256 x 256,
+        // 384 x 192 or 256 x 192 tiles), where its tiles fill the rounds
         const int rc64 = pto_amd::gemm_f16f32_k64(st, c, ha, hb, m, n, k);
         if (rc64 != PTO_ERR_UNSUPPORTED)
             return rc64;
-        // otherwise four wavefronts with the K-step written fragment by fragment where that kernel has a tile shape for
-        // the problem and is the faster one (uneven rounds, or 192 x 192 tiles for a single round), else eight wavefronts
-        const int rc384 = pto_amd::gemm_f16f32_tile384x192_w8(st, c, ha, hb, m, n, k); // whole rounds of 384 x 192 tiles, k % 128 != 0
-        if (rc384 != PTO_ERR_UNSUPPORTED)
-            return rc384;
-        const int rc = pto_amd::gemm_f16f32_tile256_w4(st, c, ha, hb, m, n, k);
-        if (rc != PTO_ERR_UNSUPPORTED)
-            return rc;
-        return pto_amd::gemm_f16f32_tile256_w8(st, c, ha, hb, m, n, k);
     }
     return launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
 }

@@ -35,9 +35,7 @@ ST_LIB_PATH = os.path.join(_HERE, "libpto_st.so")
 _V = [C.c_void_p] * 4 + [C.c_int] * 4
 ST_SYMBOLS = {
     "pto_gemm_f16f32_variant": (C.c_int, _V),
-    "pto_gemm_f16f32_w8_variant": (C.c_int, _V),
-    "pto_gemm_f16f32_m16_variant": (C.c_int, _V),
-    "pto_gemm_f16f32_m16w4_variant": (C.c_int, _V),
+    "pto_gemm_f16f32_w4_variant": (C.c_int, _V),
     "pto_gemm_f16f32_k64_variant": (C.c_int, _V),
     "pto_gemm_mxfp8_variant": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 6),
     "pto_fa_fwd_f16_variant": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 7),
