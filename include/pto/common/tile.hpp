@@ -135,7 +135,8 @@ struct TileStorage { // unsupported locations: no storage
 
 template <typename T, int Rows, int Cols>
 struct TileStorage<TileType::Mat, T, Rows, Cols> {
-    uint32_t lds = 0; // byte offset into the workgroup's dynamic LDS
+    uint32_t lds = 0;   // byte offset into the workgroup's dynamic LDS ("L1" address 0 = its first byte)
+    bool bound = false; // a TASSIGN has given the tile its address
 };
 
 template <typename T, int Rows, int Cols>
@@ -155,6 +156,8 @@ constexpr bool is_mx_operand_v = is_mx8_v<T> || is_mx4_v<T>;
 template <typename T>
 constexpr int elem_bits = is_mx4_v<T> ? 4 : 8 * (int)sizeof(T);
 constexpr int kMxM = 32, kMxK = 64, kMxBlock = 32;
+// upper half of the value that data() of a Mat tile returns (the lower half is the tile's L1 byte offset)
+constexpr uint64_t kMatHandleTag = 0x4D41540000000000ull; // "MAT"
 
 template <int Rows, int Cols>
 struct TileStorage<TileType::Left, float8_e4m3_t, Rows, Cols> {
@@ -398,7 +401,10 @@ struct Tile {
     PTO_DEV auto data()
     {
         if constexpr (Loc_ == TileType::Mat) {
-            return reinterpret_cast<DType *>(hw::lds_base() + st.lds);
+            // A handle, not an address to read through (the LDS image is swizzled; TEXTRACT / TMOV / TSTORE read it): the
+            // tile's byte offset in the workgroup's "L1" under a tag in the upper half, so that TASSIGN can take
+            // `data() + n` apart again with integer arithmetic that the compiler folds.
+            return reinterpret_cast<DType *>((uintptr_t)(detail::kMatHandleTag | (uint64_t)st.lds));
         } else {
 #if defined(PTO_VEC_TILES_IN_MEMORY)
             if constexpr (inMemory)

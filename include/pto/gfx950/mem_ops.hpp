@@ -155,6 +155,8 @@ constexpr uint32_t mat_tile_bytes()
 // (the reference checks its compile-time form the same way, tassign_check.hpp:18-30).
 #if defined(__HIP_DEVICE_COMPILE__)
 __device__ void tassign_beyond_lds() __attribute__((error("[PTO][SA] TASSIGN: the Mat tile ends beyond the 160 KiB LDS of a compute unit")));
+__device__ void tassign_beyond_ub() __attribute__((error("[PTO][SA] TASSIGN: the Vec tile ends beyond the part of the workgroup's unified buffer that Vec tiles may use")));
+__device__ void tassign_moves_mat_view() __attribute__((error("[PTO][SA] TASSIGN: a Mat tile that has an address is moved by a pointer taken from data(): the LDS image of a tile is not the L1 layout, a part of it is not a tile")));
 #endif
 } // namespace detail
 template <typename T, typename AddrType>
@@ -164,7 +166,8 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
         obj.SetAddr(reinterpret_cast<typename T::DType *>(addr));
     } else if constexpr (T::Loc == TileType::Mat) {
         const uint64_t a = (uint64_t)(uintptr_t)addr;
-        const uint32_t off = (a >> 32) ? (uint32_t)a - (uint32_t)(uintptr_t)hw::lds_base() : (uint32_t)a;
+        // a literal L1 byte offset, or a value made from a Mat tile's data() (tag in the upper half, offset in the lower)
+        const uint32_t off = (uint32_t)a;
 #if defined(PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL)
         // For translation units that hold many kernels of which a few need more L1 than a compute unit has LDS (the
         // reference's per-instruction test sources): such a kernel ends at the TASSIGN, every wave alike, having done
@@ -179,7 +182,23 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
         if (off + detail::mat_tile_bytes<T>() > detail::kLdsBytes)
             __builtin_trap(); // the run-time form of the reference's PTO_ASSERT (debug builds only)
 #endif
+        // A tile that already has an address, moved by an address computed from a tile's data(): the reference's stage
+        // macros walk a large L1 tile in chunks this way (pto_macro_matmul.hpp:176-177: data() + k * Cube_K * Cube_M).  The
+        // LDS image of a Mat tile is swizzled row-major, not Nz: a chunk of it is not the image of a smaller tile, so the
+        // second and later chunks would read another part of the data.  Stops the build where the compiler knows both
+        // addresses; otherwise the kernel reports it and ends (every wave makes the same call).
+        if ((a >> 32) != 0 && obj.st.bound && off != obj.st.lds) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            if (__builtin_constant_p(off) && __builtin_constant_p(obj.st.lds))
+                detail::tassign_moves_mat_view();
+#endif
+            if (hw::tid() == 0)
+                printf("[PTO][RT] TASSIGN: a Mat tile at LDS offset %u is moved to %u by a pointer taken from data(); a part of a "
+                       "tile's LDS image is not a tile (block %d)\n", obj.st.lds, off, (int)blockIdx.x);
+            __builtin_amdgcn_endpgm();
+        }
         obj.st.lds = off;
+        obj.st.bound = true;
     } else if constexpr (T::Loc == TileType::Scaling) {
         obj.st.fb = (uint32_t)(uintptr_t)addr; // offset into the table of quantisation words
     } else {
@@ -187,6 +206,23 @@ PTO_DEV void TASSIGN_IMPL(T &obj, AddrType addr)
         if constexpr (T::inMemory) {
             // a byte offset into the workgroup's unified buffer, or a pointer obtained from another Vec tile's data()
             const uint64_t a = (uint64_t)(uintptr_t)addr;
+            // offset form: the tile has to end inside this workgroup's buffer, and below the accumulator images when
+            // those live in its upper part
+#if defined(PTO_ACC_TILES_IN_MEMORY)
+            constexpr uint64_t vecLimit = PTO_ACC_ARENA_OFFSET;
+#else
+            constexpr uint64_t vecLimit = PTO_UB_BYTES;
+#endif
+            constexpr uint64_t bytes = (uint64_t)T::Numel * sizeof(typename T::DType);
+            if (a < (uint64_t)PTO_UB_BYTES && a + bytes > vecLimit) {
+#if defined(__HIP_DEVICE_COMPILE__)
+                if (__builtin_constant_p(a))
+                    detail::tassign_beyond_ub();
+#endif
+#if defined(_DEBUG) || defined(PTO_DEBUG)
+                __builtin_trap();
+#endif
+            }
             obj.mem_ = a < (uint64_t)PTO_UB_BYTES ? reinterpret_cast<typename T::DType *>(detail::ub_base() + a) :
                                                    reinterpret_cast<typename T::DType *>((uintptr_t)a);
             return;

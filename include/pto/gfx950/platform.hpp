@@ -218,7 +218,7 @@ PTO_DEV void wait_flag_dev(int64_t)
 // ---- function-local `static` variables of a core (pto_macro_matmul.hpp:58-65, fa_performance_kernel.cpp:263-275) ----
 // On Ascend such a variable is private to the core and keeps its value between calls for the length of the kernel.  A GPU
 // function cannot hold a `static` in a register; port_ascend_source.py rewrites `static T name = init;` inside device
-// functions into PTO_CORE_STATIC(T, name, init): `name` becomes a reference to one of 32 eight-byte slots in LDS, private
+// functions into PTO_CORE_STATIC(T, name, init, number): `name` becomes a reference to one of 32 eight-byte slots in LDS, private
 // to the wave (every wave runs the same scalar program, so each keeps its own copy and no barrier is needed), initialised
 // on first use after PTO_KERNEL_PROLOGUE(), which the script puts at the top of every kernel.  Instantiations of one
 // template share the slot of the declaration.
@@ -249,4 +249,5 @@ PTO_DEV T &core_static(T init)
 } // namespace detail
 } // namespace pto
 #define PTO_KERNEL_PROLOGUE() (pto::detail::core_static_area().inited[pto::hw::wave()] = 0u)
-#define PTO_CORE_STATIC(T, NAME, INIT) T &NAME = pto::detail::core_static<T, __COUNTER__ % 32>(INIT)
+// ID: the variable's number in its translation unit (0 .. 31), which port_ascend_source.py counts itself
+#define PTO_CORE_STATIC(T, NAME, INIT, ID) T &NAME = pto::detail::core_static<T, ID>(INIT)

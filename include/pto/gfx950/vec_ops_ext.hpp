@@ -733,6 +733,34 @@ PTO_DEV T elem_rem(T a, T b)
     else
         return (T)::fmod((double)a, (double)b);
 }
+// TREM / TREMS exist in two meanings in the reference.  The CPU simulation takes C's % and fmod (cpu/ElementOp.h:145-156):
+// the result has the sign of the dividend; that is elem_rem above and the default here, as for every instruction.  The
+// NPU computes a - floor(a / b) b in the tile's own floating-point type, integer tiles through a conversion to that type
+// and back by rounding (npu/a2a3/TRem.hpp:17-95, TRemS.hpp:17-56, and np.remainder in the generators of its tests): the
+// result has the sign of the divisor.  A translation unit that defines PTO_TREM_FLOOR_FORM gets the NPU's meaning.
+template <typename T>
+PTO_DEV T elem_rem_floor(T a, T b)
+{
+    if constexpr (std::is_integral_v<T>) {
+        using F = std::conditional_t<sizeof(T) == 2, half, float>;
+        const F r = elem_rem_floor<F>((F)a, (F)b);
+        return (T)__builtin_rintf((float)r);
+    } else {
+        const T q = (T)(a / b);
+        const T f = (T)__builtin_floorf((float)q);
+        const T p = (T)(f * b);
+        return (T)(a - p);
+    }
+}
+template <typename T>
+PTO_DEV T elem_trem(T a, T b)
+{
+#if defined(PTO_TREM_FLOOR_FORM)
+    return elem_rem_floor<T>(a, b);
+#else
+    return elem_rem<T>(a, b);
+#endif
+}
 } // namespace detail
 
 #define PTO_DEFINE_BINARY_EXT(NAME, INT_ONLY, EXPR)                                                     \
@@ -755,7 +783,7 @@ PTO_DEFINE_BINARY_EXT(TOR, false, detail::bitwise(a, b, [](auto x, auto y) { ret
 PTO_DEFINE_BINARY_EXT(TXOR, false, detail::bitwise(a, b, [](auto x, auto y) { return x ^ y; }))
 PTO_DEFINE_BINARY_EXT(TSHL, true, a << b)
 PTO_DEFINE_BINARY_EXT(TSHR, true, a >> b)
-PTO_DEFINE_BINARY_EXT(TREM, false, detail::elem_rem<T>(a, b))
+PTO_DEFINE_BINARY_EXT(TREM, false, detail::elem_trem<T>(a, b))
 PTO_DEFINE_BINARY_EXT(TFMOD, false, detail::elem_rem<T>(a, b)) // C fmod / integer %: the sign of the dividend (tfmod/gen_data.py:32)
 #undef PTO_DEFINE_BINARY_EXT
 
@@ -778,7 +806,7 @@ PTO_DEFINE_SCALAR_EXT(TORS, false, detail::bitwise(a, (T)k, [](auto x, auto y) {
 PTO_DEFINE_SCALAR_EXT(TXORS, false, detail::bitwise(a, (T)k, [](auto x, auto y) { return x ^ y; }))
 PTO_DEFINE_SCALAR_EXT(TSHLS, true, a << k)
 PTO_DEFINE_SCALAR_EXT(TSHRS, true, a >> k)
-PTO_DEFINE_SCALAR_EXT(TREMS, false, detail::elem_rem<T>(a, k))
+PTO_DEFINE_SCALAR_EXT(TREMS, false, detail::elem_trem<T>(a, k))
 PTO_DEFINE_SCALAR_EXT(TFMODS, false, detail::elem_rem<T>(a, k))
 #undef PTO_DEFINE_SCALAR_EXT
 

@@ -193,6 +193,12 @@ int pto_st_matmul_tmov_f16_64x64x128(void *stream, float *out, const uint16_t *a
 int pto_st_pushpop_f16_64x64x128(void *stream, float *out, const uint16_t *a, const uint16_t *b_t, const uint16_t *v_t,
                                  float *qk_fifo, uint16_t *p_fifo, int lds_fifo);
 
+/* The guard of TASSIGN against walking a Mat tile over a larger one by `data() + k * bytes` (pto_macro_matmul.hpp:176-177
+ * of the reference does so over an L1 panel; an LDS image is swizzled row-major, a part of it is not a tile).  One
+ * workgroup makes `chunks` (1 or 2) such TASSIGNs: flags[0] = 1 once it has started, flags[1] = 1 once it has reached
+ * its end, which it does for one chunk only; with two it prints a "[PTO][RT] TASSIGN" line and ends at the second. */
+int pto_st_mat_view_walk(void *stream, uint32_t *flags, int chunks);
+
 #ifdef __cplusplus
 }
 #endif

@@ -77,7 +77,9 @@ def build_host(verbose=True):
 
 
 REFERENCE = os.environ.get("PTO_REFERENCE", "/root/reference")
-PORTED_DIR = os.path.join(ROOT, "oracle", "_ref")
+# the reference's kernel sources compiled against this library's headers are the thing under test, not the checker: they are
+# kept apart from oracle/_ref (the compiled reference that the oracle is pinned against)
+PORTED_DIR = os.path.join(ROOT, "build", "ported")
 # (library, reference source, constants rewritten for 160 KiB of LDS, dynamic LDS bytes of the launch, further options)
 PORTED = [
     ("libpto_ported_gemm.so", "kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp",
@@ -123,7 +125,7 @@ def port_and_compile(rel_src, sets, lds_bytes, out, extra_flags=(), extra_includ
 
 def build_ported(verbose=True):
     """The reference's own kernel sources compiled against this library's headers (only where the reference tree is
-    mounted; the libraries go to oracle/_ref/, which is kept out of the history)."""
+    mounted; the libraries go to build/ported/, which is kept out of the history)."""
     if not os.path.isdir(REFERENCE):
         return
     os.makedirs(PORTED_DIR, exist_ok=True)
@@ -137,8 +139,8 @@ def build_ported(verbose=True):
 
 
 # Per-instruction test kernels of the reference (tests/npu/a2a3/src/st/testcase/<op>/<op>_kernel.cpp) that tests/st_ref_cases.py
-# runs on the GPU: each compiled unchanged (register tiles; no constant rewritten) into oracle/_ref/st/<op>.so.
-# oracle/_ref/st/manifest.json holds, per test, the launcher symbols (mangled -> demangled, so that the tests need no
+# runs on the GPU: each compiled unchanged (register tiles; no constant rewritten) into build/ported/st/<op>.so.
+# build/ported/st/manifest.json holds, per test, the launcher symbols (mangled -> demangled, so that the tests need no
 # binutils) and, for sources whose launchers are numbered cases (`launch<OP>Case<N>` kernels that fix the template arguments
 # of one run function each), the table case number -> [run function, template arguments] read from the source.
 ST_KERNELS = ["tabs", "tneg", "tnot", "texp", "tlog", "tsqrt", "trsqrt", "trecip", "trelu", "tmov_vect", "tsub", "tmul", "tdiv", "tadd",
@@ -167,6 +169,9 @@ ST_PORT_OPTIONS = {
 ST_PORT_OPTIONS["tmrgsort"] = dict(vec_in_memory=True)
 # the NPU form of TSCATTER (indices are element numbers of the destination; the CPU simulation's are row numbers)
 ST_PORT_OPTIONS["tscatter"] = dict(defines=["PTO_TSCATTER_FLAT_INDEX"])
+# the NPU form of TREM / TREMS (the sign of the divisor; the CPU simulation's % / fmod take the dividend's)
+ST_PORT_OPTIONS["trem"] = dict(defines=["PTO_TREM_FLOOR_FORM"])
+ST_PORT_OPTIONS["trems"] = dict(defines=["PTO_TREM_FLOOR_FORM"])
 # three of its kernels keep more than 160 KiB of L1 tiles: they end at their TASSIGN and are not run
 ST_PORT_OPTIONS["tstore_mat2gm"] = dict(defines=["PTO_TASSIGN_BEYOND_LDS_ENDS_KERNEL"])
 # stores through a second tile object at the address of the one it loaded: tiles as addresses

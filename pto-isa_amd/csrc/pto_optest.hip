@@ -1451,3 +1451,32 @@ extern "C" int pto_st_pushpop_f16_64x64x128(void *stream, float *out, const uint
     }
     return pto_amd::check_launch();
 }
+
+// A Mat tile walked over a larger one by `data() + k * bytes`, the way pto_macro_matmul.hpp:176-177 of the reference walks an
+// L1 panel: chunk 0 is accepted (the start of an image is an image), a later chunk ends the kernel with a message.
+// flags[0] = 1 when the kernel has started, flags[1] = 1 when it has reached its end.
+PTO_DEVICE_CODE_BEGIN
+__global__ __launch_bounds__(kBlockThreads) AICORE void MatViewWalk(__gm__ uint32_t *flags, int chunks, uint32_t step)
+{
+    using Whole = Tile<TileType::Mat, half, 128, 128, BLayout::ColMajor, 128, 128, SLayout::RowMajor>;
+    using Chunk = Tile<TileType::Mat, half, 128, 64, BLayout::ColMajor, 128, 64, SLayout::RowMajor>;
+    Whole whole;
+    Chunk chunk;
+    TASSIGN(whole, 0x0);
+    if (hw::tid() == 0)
+        flags[0] = 1;
+    for (int k = 0; k < chunks; ++k)
+        TASSIGN(chunk, (uint64_t)whole.data() + (uint64_t)k * step); // (a step the compiler does not know: the run-time form)
+    if (hw::tid() == 0)
+        flags[1] = 1 + (uint32_t)(chunk.data() - whole.data());
+}
+PTO_DEVICE_CODE_END
+
+extern "C" int pto_st_mat_view_walk(void *stream, uint32_t *flags, int chunks)
+{
+    PTO_ST_NONNULL(flags);
+    if (chunks < 1 || chunks > 2)
+        return PTO_ERR_UNSUPPORTED;
+    MatViewWalk<<<dim3(1), dim3(kBlockThreads), 128 * 128 * sizeof(half), static_cast<hipStream_t>(stream)>>>(flags, chunks, 128 * 64 * (uint32_t)sizeof(half));
+    return pto_amd::check_launch();
+}

@@ -20,8 +20,8 @@ script therefore does (nothing else is touched; the tile code itself compiles as
    to fit the 160 KiB of LDS (the TASSIGN of a tile that does not fit is a compile error, not a silent overrun).
 5. Headers that sit next to the source (`#include "name"`) are inlined so that the edits reach them; an inlined `.hpp`
    is device code as a whole.
-6. `static T name = init;` inside a function becomes `PTO_CORE_STATIC(T, name, init);` (a per-wave slot in LDS: a GPU
-   function cannot keep a core-private `static`), and every `__global__` function starts with `PTO_KERNEL_PROLOGUE();`.
+6. `static T name = init;` inside a function becomes `PTO_CORE_STATIC(T, name, init, number);` (a per-wave slot in LDS,
+   numbered per translation unit, at most 32: a GPU function cannot keep a core-private `static`), and every `__global__` function starts with `PTO_KERNEL_PROLOGUE();`.
 7. `--define NAME[=VALUE]` puts `#define`s in front of everything (the `__DAV_*` macros by which a source asks which
    kind of core it is compiled for: a workgroup plays both, so both may be defined).
 8. `__global__` becomes `__global__ __launch_bounds__(pto::kBlockThreads)`.
@@ -35,6 +35,10 @@ script therefore does (nothing else is touched; the tile code itself compiles as
 12. Reads of Ascend's special scalar registers written as inline assembly, `asm volatile("MOV %0, SYS_CNT\n" : "+l"(x));`
     and `... PC ...`, become `x = get_sys_cnt();` and `x = 0;` (time stamps that the test kernels log, and the program
     counter they hand to an instruction-cache preload, which is a no-op here).
+13. A kernel template over `S1`, `CUBE_S1`, `TILE_S1` and `QK_PRELOAD` (the flash-attention kernel `runTFA`) gets a
+    `static_assert(TILE_S1 == CUBE_S1 || S1 <= QK_PRELOAD * TILE_S1)` at the top of its body: one workgroup plays the Cube
+    and the Vec role of a block in program order, and a Vec-side score tile wider than what the Cube side has produced
+    would be read half-written.  Such a case stops the build instead of returning wrong output.
 """
 import argparse
 import os
@@ -45,6 +49,10 @@ LAUNCH = re.compile(r"<<<\s*([^,<>]+?)\s*,\s*nullptr\s*,\s*([^<>]+?)\s*>>>")
 LOCAL_INCLUDE = re.compile(r'^[ \t]*#include[ \t]+"([^"]+)"[ \t]*$', re.M)
 STATIC_LOCAL = re.compile(r"^([ \t]+)static[ \t]+([A-Za-z_][\w:]*(?:[ \t]+[A-Za-z_][\w:]*)*)[ \t]+([A-Za-z_]\w*)[ \t]*=[ \t]*([^;]+);", re.M)
 KERNEL_HEAD = re.compile(r"__global__[^;{}]*?\)\s*\{")
+# a kernel template over CUBE_S1, TILE_S1 and QK_PRELOAD (runTFA of fa_performance_kernel.cpp:607-609), up to its opening brace
+TFA_KERNEL = re.compile(r"template\s*<[^<>{};]*\bS1\b[^<>{};]*\bCUBE_S1\b[^<>{};]*\bTILE_S1\b[^<>{};]*\bQK_PRELOAD\b[^<>{};]*>\s*__global__[^;{}]*?\)\s*\{")
+TFA_ASSERT = ('static_assert(TILE_S1 == CUBE_S1 || S1 <= QK_PRELOAD * TILE_S1, "[PTO][SA] flash-attention kernel on gfx950: the Vec role runs '
+              'after the Cube role in program order; TILE_S1 > CUBE_S1 needs the whole key range inside the preload (S1 <= QK_PRELOAD * TILE_S1)");')
 BEGIN_MARK, END_MARK = "//@@PTO_INLINED_BEGIN ", "//@@PTO_INLINED_END "
 
 
@@ -173,11 +181,22 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
     text, n = re.subn(r"__global__(?!\s*__launch_bounds__)", "__global__ __launch_bounds__(pto::kBlockThreads)", text)
 
     # 5. function-local statics of device functions, and the prologue that resets them
-    text, n = STATIC_LOCAL.subn(lambda m: "%sPTO_CORE_STATIC(%s, %s, %s);" % (m.group(1), m.group(2), m.group(3), m.group(4).strip()), text)
+    numbered = [0]
+
+    def core_static(m):
+        numbered[0] += 1
+        return "%sPTO_CORE_STATIC(%s, %s, %s, %d);" % (m.group(1), m.group(2), m.group(3), m.group(4).strip(), numbered[0] - 1)
+    text, n = STATIC_LOCAL.subn(core_static, text)
+    if n > 32:
+        raise SystemExit("port_ascend_source: %d function-local statics, the per-wave area has 32 slots" % n)
     if n:
         notes.append("%d function-local static%s rewritten" % (n, "" if n == 1 else "s"))
         text, k = KERNEL_HEAD.subn(lambda m: m.group(0) + "\n    PTO_KERNEL_PROLOGUE();", text)
         notes.append("%d kernel prologue%s inserted" % (k, "" if k == 1 else "s"))
+    # 13. the flash-attention kernel: one workgroup plays the Cube and the Vec role of a block in program order
+    text, k13 = TFA_KERNEL.subn(lambda m: m.group(0) + "\n    " + TFA_ASSERT, text)
+    if k13:
+        notes.append("%d flash-attention kernel%s: schedule checked at compile time" % (k13, "" if k13 == 1 else "s"))
 
     # 1. brackets.  Inlined .hpp files are device code as a whole; in the main file the device code opens after the
     # prologue (comments, includes, using-directives, macro definitions and file-scope constants come first in these

@@ -46,6 +46,7 @@ ST_SYMBOLS = {
     "pto_st_mgather_b16_8x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_tload_pad_f32_16x32": (C.c_int, [C.c_void_p] * 3),
     "pto_st_tload_5d_f32": (C.c_int, [C.c_void_p] * 4),
+    "pto_st_mat_view_walk": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int]),
     "pto_st_textract_windows_f16": (C.c_int, [C.c_void_p] * 7 + [C.c_int] * 2),
     "pto_st_matmul_bias_128x64x256": (C.c_int, [C.c_void_p] * 5 + [C.c_int]),
     "pto_st_matmul_ragged": (C.c_int, [C.c_void_p] * 5 + [C.c_int]),

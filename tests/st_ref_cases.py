@@ -1,5 +1,5 @@
 """Cases for running the reference's own per-instruction NPU test kernels (tests/npu/a2a3/src/st/testcase/<op>/<op>_kernel.cpp,
-compiled unchanged through pto-isa_amd/port_ascend_source.py into oracle/_ref/st/<op>.so by pto-isa_amd/build.py) on the
+compiled unchanged through pto-isa_amd/port_ascend_source.py into build/ported/st/<op>.so by pto-isa_amd/build.py) on the
 GPU.  Every explicit instantiation of a launcher that a kernel source exports is one case; its template arguments, read
 from the demangled symbol, give the element type, the tile shapes and the valid region; launchers that are numbered cases
 (`launch<OP>TestCase<N>`) take them from the case table that the build reads from the kernel source (manifest.json).  What
@@ -14,7 +14,7 @@ from types import SimpleNamespace
 import numpy as np
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-ST_DIR = os.path.join(ROOT, "oracle", "_ref", "st")
+ST_DIR = os.path.join(ROOT, "build", "ported", "st")
 
 CTYPE = {"float": (np.float32, C.c_float), "int": (np.int32, C.c_int32), "short": (np.int16, C.c_int16),
          "unsigned short": (np.uint16, C.c_uint16), "signed char": (np.int8, C.c_int8), "unsigned char": (np.uint8, C.c_uint8),
@@ -70,6 +70,12 @@ def _fmod(a, b):
     return np.fmod(a, b)
 
 
+def _remainder(a, b):
+    if a.dtype.kind == "f":
+        return np.remainder(f64(a), f64(b))
+    return np.remainder(a, b)
+
+
 def _prelu(a, b):
     return np.where(a > 0, a, a * b)
 
@@ -105,9 +111,9 @@ SPECS = {
     "taddplus": dict(fn="LaunchTAdd", tail=BINARY9, layout="nine", nin=2, inputs="any", half=True, op=lambda a, b: a + b),
     "tfmod": dict(fn="LaunchTFMOD", tail=BINARY9, layout="nine", nin=2, inputs="rem", half=True, op=_fmod),
     # TREM: the NPU takes the sign of the divisor (a - floor(a / b) b, npu/a2a3/TRem.hpp:22-35; np.remainder in its
-    # generator), the CPU simulation that of the dividend (ElementOp.h:145-156: % and fmod), which this library follows:
-    # the two agree for dividends >= 0, which is what the case draws
-    "trem": dict(fn="LaunchTREM", tail=BINARY9, layout="nine", nin=2, inputs="rempos", half=True, op=_fmod),
+    # generator), the CPU simulation that of the dividend (ElementOp.h:145-156: % and fmod).  The test source is built
+    # with PTO_TREM_FLOOR_FORM (the NPU's meaning) and runs the generator's range: dividends in [-1000, 1000)
+    "trem": dict(fn="LaunchTREM", tail=BINARY9, layout="nine", nin=2, inputs="rem", half=True, op=_remainder),
     "txor": dict(fn="LaunchTXor", tail=BINARY9, layout="nine", nin=2, inputs="bits", half=False, op=lambda a, b: a ^ b),
     # tile (op) scalar, <T, dstH, dstW, srcH, srcW, vRows, vCols>, the scalar by value (tands_kernel.cpp:17-49)
     "tands": dict(fn="LaunchTAndS", tail=SCALAR7, layout="scalar7", nin=1, inputs="bits", half=False, op=lambda a, k: a & k),
@@ -233,8 +239,8 @@ SPECS.update({
     "tdivs": dict(fn="launchTDIVSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="pos", op=_div),
     "tmaxs": dict(fn="launchTMAXSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=lambda a, k: np.maximum(a, k)),
     "tfmods": dict(fn="launchTFMODSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="rem", op=_fmod),
-    # TREMS: dividends >= 0, for which the NPU's floor form and the CPU simulation's truncating form agree (see "trem")
-    "trems": dict(fn="launchTREMSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="rempos", op=_fmod),
+    # TREMS: the NPU's meaning (the sign of the divisor), as "trem"
+    "trems": dict(fn="launchTREMSTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="rem", op=_remainder),
     "tlrelu": dict(fn="launchTLRELUTestCase", tail=CASE_SCALAR, planner=plan_case_scalar, nin=1, inputs="any", op=_prelu),
 })
 
@@ -1272,7 +1278,7 @@ for _name in ("tpartmul", "tfmods", "tmov_vect"):
 
 
 def lib_of(test):
-    """name of the library (oracle/_ref/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
+    """name of the library (build/ported/st/<name>.so, and of the manifest entry) that holds a test's launchers"""
     return SPECS[test].get("lib", test)
 
 

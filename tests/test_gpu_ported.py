@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-PORTED = os.path.join(ROOT, "oracle", "_ref")
+PORTED = os.path.join(ROOT, "build", "ported")
 
 pytestmark = pytest.mark.gpu
 
@@ -16,6 +16,8 @@ pytestmark = pytest.mark.gpu
 def _ported(name):
     path = os.path.join(PORTED, name)
     if not os.path.exists(path):
+        # a run that is meant to cover the ported kernels (PTO_REQUIRE_PORTED=1) must not pass without them
+        assert os.environ.get("PTO_REQUIRE_PORTED") != "1", "%s is missing and PTO_REQUIRE_PORTED=1" % path
         pytest.skip("%s not built (reference tree absent at build time)" % name)
     return C.CDLL(path)
 

@@ -161,6 +161,20 @@ def test_tload_tstore_5d(oracle):
     assert np.array_equal(strided.cpu().numpy(), back)
 
 
+def test_mat_tile_walked_through_data_pointer_ends_the_kernel(capfd):
+    """TASSIGN of a Mat tile that has an address to `data() + n` of another: n == 0 is the image itself, n != 0 is a part of
+    a swizzled image and not a tile (the reference's L1 layout allows it, pto_macro_matmul.hpp:176-177) - the kernel
+    says so and ends there, in every wave, instead of computing on other data."""
+    lib = capi.load_st()
+    for chunks, reached in ((1, 1), (2, 0)):
+        flags = torch.zeros(2, dtype=torch.int32, device="cuda")
+        capi.check(lib.pto_st_mat_view_walk(st(), flags.data_ptr(), chunks), "walk")
+        torch.cuda.synchronize()
+        assert flags.cpu().tolist() == [1, reached], (chunks, flags.cpu().tolist())
+    out = capfd.readouterr().out
+    assert "[PTO][RT] TASSIGN: a Mat tile at LDS offset 0 is moved to 16384" in out, out
+
+
 @pytest.mark.parametrize("col0,row0", [(0, 0), (64, 128), (192, 192), (8, 40)])
 def test_textract_windows(oracle, col0, row0):
     """dst[i,j] = src[r0+i, c0+j] for windows that are not the suffix (the reference CPU simulation only

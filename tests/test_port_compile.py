@@ -88,7 +88,8 @@ constexpr int kSize = 512;
 AICORE inline int counter()
 {
     static int calls = 0;
-    return ++calls;
+    static uint64_t ticks = 7;
+    return ++calls + (int)ticks;
 }
 __global__ AICORE void kern(__gm__ float *out)
 {
@@ -101,7 +102,23 @@ void Launch(float *out, void *stream)
 """
     text, notes = mod.port(src, [("kSize", "128")], 4096, ("__DAV_VEC__",), None, True)
     assert "constexpr int kSize = 128;" in text
-    assert "PTO_CORE_STATIC(int, calls, 0);" in text and "PTO_KERNEL_PROLOGUE();" in text
+    # statics are numbered in the order of the source, one LDS slot each
+    assert "PTO_CORE_STATIC(int, calls, 0, 0);" in text and "PTO_CORE_STATIC(uint64_t, ticks, 7, 1);" in text
+    assert "PTO_KERNEL_PROLOGUE();" in text
+    many = src.replace("    static int calls = 0;\n", "".join("    static int c%d = 0;\n" % i for i in range(32)) + "    int calls = 0;\n")
+    with pytest.raises(SystemExit, match="33 function-local statics"):
+        mod.port(many, [("kSize", "128")], 4096, ("__DAV_VEC__",), None, True)
+    # a flash-attention kernel (a __global__ runTFA with the reference's template parameters) gets the check of its schedule
+    tfa = """#include <pto/pto-inst.hpp>
+template <int S0, int HEAD_SIZE, int S1, int CUBE_S0, int CUBE_S1, int TILE_S1, int QK_PRELOAD>
+__global__ AICORE void runTFA(__gm__ half *q)
+{
+    q[0] = 0;
+}
+"""
+    text2, notes2 = mod.port(tfa, [], 4096, (), None, True)
+    assert "static_assert(TILE_S1 == CUBE_S1 || S1 <= QK_PRELOAD * TILE_S1" in text2
+    assert text2.index("static_assert(TILE_S1 == CUBE_S1") < text2.index("q[0] = 0;")
     assert "<<<pto::host::LaunchBlocks(4, (hipStream_t)(stream)), pto::kBlockThreads, pto::host::LaunchLds((const void *)(kern), 4096), (hipStream_t)(stream)>>>" in text
     assert "__global__ __launch_bounds__(pto::kBlockThreads) AICORE void kern" in text
     assert text.startswith("#define PTO_TILE_COPY_WRITEBACK 1\n#define PTO_VEC_TILES_IN_MEMORY 1\n#define __DAV_VEC__ 1\n")
@@ -162,6 +179,70 @@ def test_register_tile_by_value_compiles_in_write_back_mode(tmp_path):
     values back to the tile it was copied from)."""
     rc, err = _hipcc_snippet(tmp_path, SNIPPET, defines=["PTO_TILE_COPY_WRITEBACK=1"])
     assert rc == 0, err
+
+
+MOVED_MAT = r"""
+#include <hip/hip_runtime.h>
+#include <pto/pto-inst.hpp>
+using namespace pto;
+PTO_DEVICE_CODE_BEGIN
+template <typename ChunkT, typename WholeT>
+AICORE inline void Chunks(ChunkT &chunk, WholeT &whole, half *src)
+{
+    GlobalTensor<half, pto::Shape<1, 1, 1, 128, 64>, pto::Stride<1, 1, 1, 64, 1>> g(src);
+    for (int k = 0; k < KCHUNKS; ++k) {
+        TASSIGN(chunk, (uint64_t)whole.data() + k * 128 * 64 * 2);
+        TLOAD(chunk, g);
+    }
+}
+__global__ void k(half *src)
+{
+    using Whole = Tile<TileType::Mat, half, 128, 128, BLayout::ColMajor, 128, 128, SLayout::RowMajor>;
+    using Chunk = Tile<TileType::Mat, half, 128, 64, BLayout::ColMajor, 128, 64, SLayout::RowMajor>;
+    Whole w; Chunk c;
+    TASSIGN(w, 0x0);
+    Chunks(c, w, src);
+}
+PTO_DEVICE_CODE_END
+"""
+
+
+def test_mat_tile_moved_through_data_pointer_is_a_compile_error(tmp_path):
+    """The walk of pto_macro_matmul.hpp:176-177 (one Mat tile re-addressed to data() + k * chunk bytes): accepted for one
+    chunk (offset 0 of the image is the image), stopped at compile time for two."""
+    rc, err = _hipcc_snippet(tmp_path, MOVED_MAT, defines=["KCHUNKS=1"])
+    assert rc == 0, err
+    rc, err = _hipcc_snippet(tmp_path, MOVED_MAT, defines=["KCHUNKS=2"])
+    assert rc != 0 and "[PTO][SA] TASSIGN: a Mat tile that has an address is moved" in err, err
+
+
+VEC_BEYOND = r"""
+#include <hip/hip_runtime.h>
+#include <pto/pto-inst.hpp>
+using namespace pto;
+PTO_DEVICE_CODE_BEGIN
+__global__ void k(float *out)
+{
+    Tile<TileType::Vec, float, 64, 64, BLayout::RowMajor, 64, 64> t;
+    TASSIGN(t, VEC_ADDR);
+    TEXPANDS(t, 1.0f);
+    GlobalTensor<float, pto::Shape<1, 1, 1, 64, 64>, pto::Stride<1, 1, 1, 64, 1>> g(out);
+    TSTORE(g, t);
+}
+PTO_DEVICE_CODE_END
+"""
+
+
+def test_vec_tile_beyond_unified_buffer_is_a_compile_error(tmp_path):
+    """A Vec tile in the unified buffer has to end inside the workgroup's share of it (512 KiB), and below the accumulator
+    images (from 256 KiB) when those live there too."""
+    ok = ["PTO_VEC_TILES_IN_MEMORY=1", "VEC_ADDR=0x7C000"]          # ends at 512 KiB exactly
+    rc, err = _hipcc_snippet(tmp_path, VEC_BEYOND, defines=ok)
+    assert rc == 0, err
+    rc, err = _hipcc_snippet(tmp_path, VEC_BEYOND, defines=["PTO_VEC_TILES_IN_MEMORY=1", "VEC_ADDR=0x7C040"])
+    assert rc != 0 and "[PTO][SA] TASSIGN: the Vec tile ends beyond" in err, err
+    rc, err = _hipcc_snippet(tmp_path, VEC_BEYOND, defines=ok + ["PTO_ACC_TILES_IN_MEMORY=1"])
+    assert rc != 0 and "[PTO][SA] TASSIGN: the Vec tile ends beyond" in err, err
 
 
 def test_forwarding_headers_exist():

@@ -14,7 +14,7 @@ CASES = S.cases()
 
 def test_case_table_covers_every_built_test():
     if not os.path.isdir(S.ST_DIR):
-        pytest.skip("oracle/_ref/st not built (reference tree absent at build time)")
+        pytest.skip("build/ported/st not built (reference tree absent at build time)")
     man = S.manifest()
     assert {S.lib_of(t) for t in S.SPECS} <= set(man)
     # every exported launcher of a listed test is a case: none is dropped by the symbol patterns
