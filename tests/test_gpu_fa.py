@@ -120,11 +120,23 @@ def test_fa_invariants():
     assert rel(o3[0, 0], want) <= TOL
 
 
-def test_fa_config3_noncausal_b1_h16_s4096_d128():
-    """Full-size config: Q/K/V ~ N(0,1)/sqrt(128), fp16 output.  Two heads checked in full against fp64."""
+def check_head_against_streaming_oracle(oracle, q, k, v, b, h, causal):
+    """One whole head of a full-size configuration against the oracle's streaming recurrence with the kernel's key tile (64)
+    and the RNE cast of P: what is left is the order of the fp32 sums (5e-4 of the largest |O|).  The fp32 output of the
+    same launch shape is compared, so that the fp16 rounding of O (2^-11) does not eat the tolerance."""
+    o32, lse = fa_gpu(q, k, v, causal=causal, o_fp32=True)
+    oo, m, l = oracle.fa_stream_f16(q[b, h], k[b, h], v[b, h], tile_s1=64, causal=causal, q_offset=0, round_away=False)
+    assert rel(o32[b, h], oo) <= 5e-4
+    assert np.max(np.abs(lse[b, h] - (m / np.sqrt(q.shape[-1]) + np.log(l)))) <= 1e-4
+
+
+def test_fa_config3_noncausal_b1_h16_s4096_d128(oracle):
+    """Full-size config: Q/K/V ~ N(0,1)/sqrt(128), fp16 output.  Two heads checked in full against fp64, one against the
+    streaming oracle."""
     B, H, S, D = 1, 16, 4096, 128
     q, k, v = datagen.fa_inputs(B, H, S, S, D, scale=1.0 / np.sqrt(D))
     o, lse = fa_gpu(q, k, v, causal=False, o_fp32=False)
+    check_head_against_streaming_oracle(oracle, q, k, v, 0, 5, False)
     for h in (0, 11):
         want, want_lse = dense_fp64(q[0, h], k[0, h], v[0, h])
         assert rel(o[0, h], want) <= TOL
@@ -243,11 +255,13 @@ def test_fa_kernel_variants_of_the_test_library(D, causal, variant):
         assert np.max(np.abs(lse[0, h] - want_lse)) <= 1e-3
 
 
-def test_fa_config4_causal_b4_h32_s2048_d64():
-    """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row."""
+def test_fa_config4_causal_b4_h32_s2048_d64(oracle):
+    """Full-size config: N(0,1) inputs, causal, fp16 output plus fp32 log-sum-exp per row.  Three heads in full against
+    fp64, one against the streaming oracle."""
     B, H, S, D = 4, 32, 2048, 64
     q, k, v = datagen.fa_inputs(B, H, S, S, D, scale=1.0)
     o, lse = fa_gpu(q, k, v, causal=True, o_fp32=False)
+    check_head_against_streaming_oracle(oracle, q, k, v, 2, 9, True)
     for b, h in ((0, 0), (3, 31), (1, 17)):
         want, want_lse = dense_fp64(q[b, h], k[b, h], v[b, h], causal=True)
         assert rel(o[b, h], want) <= TOL
