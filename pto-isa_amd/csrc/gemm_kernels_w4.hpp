@@ -344,15 +344,19 @@ AICORE inline __attribute__((always_inline)) void W4StoreTile(float *out, int64_
     });
 }
 
-// One 256 x BN tile of C per workgroup.
+// One 256 x BN tile of C per workgroup.  Where 256 does not divide m (BN does not divide n) the last tile row (column) is
+// moved back so that it ends with the matrix: it computes some rows (columns) of its neighbour a second time and stores
+// the same values.
 template <int BN, int GROUP_M>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     void GemmF16F32W4(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k)
 {
-    const int tilesM = m / kW4TileM, tilesN = n / BN;
+    const int tilesM = (m + kW4TileM - 1) / kW4TileM, tilesN = (n + BN - 1) / BN;
     int tm, tn;
     TileOfId<GROUP_M>(RegroupXcd((int)get_block_idx(), tilesM * tilesN), tilesM, tilesN, tm, tn);
-    const int row0 = __builtin_amdgcn_readfirstlane(tm * kW4TileM), col0 = __builtin_amdgcn_readfirstlane(tn * BN);
+    const int r = tm * kW4TileM, c = tn * BN;
+    const int row0 = __builtin_amdgcn_readfirstlane(r + kW4TileM <= m ? r : m - kW4TileM);
+    const int col0 = __builtin_amdgcn_readfirstlane(c + BN <= n ? c : n - BN);
     W4TileCompute<BN>(src0, src1, k, row0, col0);
     W4StoreTile<BN>(out, n, row0, col0);
 }
@@ -364,14 +368,15 @@ namespace {
 template <int BN>
 int launch_gemm_w4(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k)
 {
-    if (m % kW4TileM || n % BN || k % 128 || k < 128)
+    // (n % 4: the accumulator blocks are stored 16 bytes at a time)
+    if (m < kW4TileM || n < BN || n % 4 || k % 128 || k < 128)
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = 3 * 64 * BN * (int)sizeof(half) + 4 * 2 * 64 * 64 * (int)sizeof(half); // three B stages + two A slots per wave
     auto kernel = GemmF16F32W4<BN, 4>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
-    const int tiles = (m / kW4TileM) * (n / BN);
+    const int tiles = ((m + kW4TileM - 1) / kW4TileM) * ((n + BN - 1) / BN);
     kernel<<<dim3((unsigned)tiles), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k);
     return pto_amd::check_launch();
 }

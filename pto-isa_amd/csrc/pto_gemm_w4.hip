@@ -12,7 +12,7 @@ namespace pto_amd {
 // 256 x 192.  Times in microseconds as measured at 6144^3 and 7680^3 (96 and 120 K-steps); only their ratios matter.
 int gemm_f16f32_w4(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k)
 {
-    if (m % kW4TileM || k % 128 || k < 128)
+    if (m < kW4TileM || n % 4 || k % 128 || k < 128)
         return PTO_ERR_UNSUPPORTED;
     struct Width { int bn; double step, fixed; };
     const Width widths[3] = {{256, 1.31, 10.0}, {192, 1.03, 10.0}, {128, 0.70, 7.0}};
@@ -20,9 +20,10 @@ int gemm_f16f32_w4(hipStream_t st, float *c, const _Float16 *a, const _Float16 *
     int best = -1;
     double bestTime = 0.0;
     for (int i = 0; i < 3; ++i) {
-        if (n % widths[i].bn)
+        if (n < widths[i].bn)
             continue;
-        const long long tiles = (long long)(m / kW4TileM) * (n / widths[i].bn), rounds = (tiles + cus - 1) / cus;
+        const long long tiles = (long long)((m + kW4TileM - 1) / kW4TileM) * ((n + widths[i].bn - 1) / widths[i].bn);
+        const long long rounds = (tiles + cus - 1) / cus;
         const double time = (double)rounds * ((k / 64) * widths[i].step + widths[i].fixed);
         if (best < 0 || time < bestTime) {
             best = i;

@@ -63,8 +63,36 @@ def test_gemm_four_wave_tile_widths_exact():
             assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
     p = ta.data_ptr()
     assert fn(0, p, p, p, 256, 768, 192, 0) == capi.ERR_UNSUPPORTED      # k not a multiple of 128
-    assert fn(0, p, p, p, 384, 768, 256, 0) == capi.ERR_UNSUPPORTED      # m not a multiple of 256
-    assert fn(0, p, p, p, 256, 640, 256, 1) == capi.ERR_UNSUPPORTED      # n not a multiple of the width
+    assert fn(0, p, p, p, 192, 768, 256, 0) == capi.ERR_UNSUPPORTED      # fewer rows than a tile
+    assert fn(0, p, p, p, 256, 160, 256, 1) == capi.ERR_UNSUPPORTED      # fewer columns than the width
+    assert fn(0, p, p, p, 256, 770, 256, 1) == capi.ERR_UNSUPPORTED      # rows of C not a multiple of 16 bytes
+
+
+def test_gemm_ragged_m_and_n_exact():
+    """Extents that the tiles do not divide: the last tile row / column is moved back to end with the matrix.  Integer
+    operands, every element exact: each width of the four-wave kernel on small shapes (one tile that is also the moved
+    one, several, m or n alone ragged), then 6000 x 6100 x 6144 through the public entry point."""
+    import torch
+    from gpu_util import to_dev, stream
+    fn = capi.load_st().pto_gemm_f16f32_w4_variant
+    for m, n, k in ((300, 772, 256), (256, 260, 128), (1000, 1100, 384), (512, 1000, 640), (777, 768, 256)):
+        a, b = datagen.gemm_inputs_integer(m, n, k)
+        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
+        ta, tb = to_dev(a), to_dev(b)
+        for variant in (0, 1, 2):
+            tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "four-wave GEMM width %d" % variant)
+            torch.cuda.synchronize()
+            assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
+    lib = capi.load()
+    for m, n, k in ((6000, 6100, 6144), (300, 772, 256)):   # the second: too small for the size rule, taken because nothing else fits
+        a, b = datagen.gemm_inputs_integer(m, n, k)
+        ta, tb = to_dev(a), to_dev(b)
+        tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
+        capi.check(lib.pto_gemm_f16f32(stream(), tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k), "pto_gemm_f16f32")
+        torch.cuda.synchronize()
+        want = ta.view(torch.float16).double() @ tb.view(torch.float16).double().T
+        assert torch.equal(tc.double(), want), (m, n, k)
 
 
 def test_gemm_k64_tile_shapes_exact():
