@@ -53,7 +53,7 @@ int pto_last_hip_error(void);
 
 /* C[m,n] fp32 row-major = A[m,k] fp16 row-major x B, where B is stored [n,k] fp16 (a column-major
  * k x n operand), fp32 accumulation.  Accepted extents: m % 128 == 0, n % 256 == 0, k % 32 == 0 (multiples of the
- * 128 x 256 block of the reference kernel), or any m >= 256 and n >= 128 with n % 4 == 0 and k % 128 == 0 (256-row
+ * 128 x 256 block of the reference kernel), or any m >= 192 and n >= 128 with n % 4 == 0 and k % 128 == 0 (256- or 192-row
  * tiles whose last row / column of tiles is moved back to end with the matrix).  Anything else: PTO_ERR_UNSUPPORTED. */
 int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k);
 

@@ -16,12 +16,9 @@ extern "C" {
  * PTO_ERR_UNSUPPORTED where the variant has no tiling for the shape, PTO_ERR_BAD_ARG for an unknown variant. */
 /* the 128 x 256 / 256 x 256 block kernels on 32 x 32 x 16 MFMAs: tiling and pipeline depth by number (csrc/pto_gemm.hip) */
 int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
-/* four wavefronts, 256-row tiles, K-steps of 64, A in a ring per wave: 0 = 256 x 256 tiles, 1 = 256 x 192, 2 = 256 x 128
- * (csrc/pto_gemm_w4.hip) */
+/* four wavefronts, K-steps of 64, A in a ring per wave: 0 = 256 x 256 tiles, 1 = 256 x 192, 2 = 256 x 128, 3 = 192 x 256,
+ * 4 = 192 x 192, 5 = 192 x 128 (csrc/pto_gemm_w4.hip) */
 int pto_gemm_f16f32_w4_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
-/* eight wavefronts on a 4 x 2 wave grid, K-steps of 64 (whole 128-byte lines), two LDS stages: 0 = 384 x 192 tiles,
- * 1 = 256 x 256, 2 = 256 x 192 (csrc/pto_gemm_k64.hip) */
-int pto_gemm_f16f32_k64_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
 /* MX GEMM: variant bit 0 = quarter tiles in the last round, bit 1 = the shallower copy pipeline (csrc/pto_gemm_mx.hip) */
 int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                            const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant);

@@ -36,9 +36,6 @@ inline int allow_lds(K kernel, int bytes)
 // defined in pto_gemm_w4.hip (256 x 256 / 192 / 128 tiles on four wavefronts, K-steps of 64); PTO_ERR_UNSUPPORTED unless m is a
 // multiple of 256, n of one of the widths and k of 128
 int gemm_f16f32_w4(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
-// defined in pto_gemm_k64.hip (eight wavefronts, K-steps of 64, written with the tile instructions); PTO_ERR_UNSUPPORTED unless one
-// of its tile shapes keeps the compute units busy in at least 85 % of the rounds' tile slots
-int gemm_f16f32_k64(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
 // defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries, two groups of four waves in
 // opposite MFMA / softmax phases)
 int fa_fwd_d128_w8(hipStream_t st, void *o, float *lse, const _Float16 *q, const _Float16 *k, const _Float16 *v, int batch, int heads,

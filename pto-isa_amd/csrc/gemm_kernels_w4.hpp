@@ -1,5 +1,7 @@
-// fp16 x fp16 -> fp32 GEMM tile of 256 x BN (BN = 256, 192 or 128) on four wavefronts, wave grid 4 x 1, one wave per SIMD,
-// 64 x BN of C per wave; K-steps of 64 on v_mfma_f32_16x16x32_f16.
+// fp16 x fp16 -> fp32 GEMM tile of 256 x BN or 192 x BN (BN = 256, 192 or 128) on four wavefronts, wave grid 4 x 1, one wave
+// per SIMD, NMB = 4 or 3 row blocks of 16 = 64 or 48 rows x BN of C per wave; K-steps of 64 on v_mfma_f32_16x16x32_f16.
+// (What follows is written for NMB = 4; with three row blocks a wave copies 48 rows in six instructions and a slot is
+// 3 f + mb.)
 //
 // A wave's 64 rows of A are used by no other wave: each wave copies them into a ring of its own in the LDS (two slots of
 // 8 KiB) and reads its fragments back from there, so A needs no workgroup barrier, only the wave's own counters.  B
@@ -99,16 +101,16 @@ PTO_DEV detail::AccFrag W4ReadAcc()
     return v;
 }
 
-// Issue slots of a K-step for NFRAG B fragments (see the head of the file).
-template <int NFRAG, int NCOPY>
+// Issue slots of a K-step for NFRAG B fragments and NMB row blocks per wave (see the head of the file; slot = NMB f + mb).
+template <int NFRAG, int NCOPY, int NMB>
 struct W4Sched {
-    static constexpr int kPD = 4, kSlots = 4 * NFRAG;
-    static constexpr int kBarrier1 = 4 * (NFRAG - kPD) - 1, kBarrier2 = kSlots - 3;
-    static constexpr int aReadSlot(int q) { return 4 * (NFRAG / 4 + q * (NFRAG / 2) / 8) + 1; }
-    static constexpr int copySlot(int j) { return 4 * (j * NFRAG / NCOPY) + 3; }
+    static constexpr int kPD = 4, kSlots = NMB * NFRAG, kAReads = 2 * NMB;
+    static constexpr int kBarrier1 = NMB * (NFRAG - kPD) - 1, kBarrier2 = NMB * (NFRAG - 1) + 1;
+    static constexpr int aReadSlot(int q) { return NMB * (NFRAG / 4 + q * (NFRAG / 2) / kAReads) + 1; }
+    static constexpr int copySlot(int j) { return NMB * (j * NFRAG / NCOPY) + NMB - 1; }
     static constexpr int aReadAt(int idx) // the A read issued at slot idx, or -1
     {
-        for (int q = 0; q < 8; ++q)
+        for (int q = 0; q < kAReads; ++q)
             if (aReadSlot(q) == idx)
                 return q;
         return -1;
@@ -123,7 +125,7 @@ struct W4Sched {
     static constexpr int aReadsIn(int lo, int hi) // A reads at slots in (lo, hi)
     {
         int n = 0;
-        for (int q = 0; q < 8; ++q)
+        for (int q = 0; q < kAReads; ++q)
             if (aReadSlot(q) > lo && aReadSlot(q) < hi)
                 ++n;
         return n;
@@ -136,10 +138,19 @@ struct W4Sched {
                 ++n;
         return n;
     }
-    static_assert(NFRAG >= NCOPY && aReadSlot(7) < kBarrier1 && copySlot(NCOPY - 1) < kSlots, "order of the step");
+    static constexpr bool distinct() // no two A reads and no two copies in one slot
+    {
+        for (int q = 1; q < kAReads; ++q)
+            if (aReadSlot(q) == aReadSlot(q - 1))
+                return false;
+        for (int j = 1; j < NCOPY; ++j)
+            if (copySlot(j) == copySlot(j - 1))
+                return false;
+        return true;
+    }
+    static_assert(NFRAG >= NCOPY && aReadSlot(kAReads - 1) < kBarrier1 && copySlot(NCOPY - 1) < kSlots && distinct(), "order of the step");
 };
 
-constexpr int kW4TileM = 256;
 constexpr int kW4Group = 6; // K-steps of 64 come in groups of six (three B stages x two A slots)
 
 // accumulators += A[row0 .. + 256, 64 kFirst .. 64 (kFirst + kLoop)) x B[col0 .. + BN, the same k]^T, block (mb, nb) of this
@@ -147,16 +158,16 @@ constexpr int kW4Group = 6; // K-steps of 64 come in groups of six (three B stag
 // groups of six steps; TAIL > 0: exactly kLoop == TAIL steps in straight-line code (the steps that a K extent leaves over
 // after its whole groups: conditions around single steps of the loop would make the compiler join register
 // assignments of fragments that are still on their way from the LDS).
-template <int BN, int TAIL>
+template <int BN, int TAIL, int NMB>
 AICORE inline __attribute__((always_inline)) void W4Pass(__gm__ const half *src0, __gm__ const half *src1, int k, int row0, int col0, int kFirst,
                                                          int kLoop)
 {
-    constexpr int BK = 64, NMB = 4, NNB = BN / 16, NBUF = 8, BSTAGES = 3;
-    constexpr int NFRAG = 2 * NNB, NM = NFRAG * NMB, NCB = BN / 32, NCOPY = 8 + NCB;
-    using S = W4Sched<NFRAG, NCOPY>;
+    constexpr int BK = 64, NNB = BN / 16, NBUF = 8, BSTAGES = 3, NA = 2 * NMB; // NA: A copies (of eight rows) and A fragments per step
+    constexpr int NFRAG = 2 * NNB, NM = NFRAG * NMB, NCB = BN / 32, NCOPY = NA + NCB;
+    using S = W4Sched<NFRAG, NCOPY, NMB>;
     constexpr int PD = S::kPD;
-    constexpr uint32_t kBBytes = BK * BN * sizeof(half), kASlot = 64 * BK * sizeof(half), kABase = BSTAGES * kBBytes;
-    static_assert(BN % 32 == 0 && BN <= 256 && kABase + 8 * kASlot <= 160 * 1024, "tile width");
+    constexpr uint32_t kBBytes = BK * BN * sizeof(half), kASlot = 16 * NMB * BK * sizeof(half), kABase = BSTAGES * kBBytes;
+    static_assert((NMB == 3 || NMB == 4) && BN % 32 == 0 && BN <= 256 && kABase + 8 * kASlot <= 160 * 1024, "tile shape");
 
     const int wave = hw::wave();
     const uint32_t lane = (uint32_t)hw::lane();
@@ -164,7 +175,7 @@ AICORE inline __attribute__((always_inline)) void W4Pass(__gm__ const half *src0
     const int64_t ld = (int64_t)k * 2; // bytes between rows of A and between columns of B
     // A: this wave's 64 rows.  Copy t takes rows 8 t .. 8 t + 7: lane l copies the 16-byte chunk (l % 8) ^ swz(row) of row
     // 8 t + l / 8 to position l % 8 of that row's LDS image (swz(r) = (r / 2) % 8 as in a Mat tile: 4 t + l / 16).
-    const char *aWave = reinterpret_cast<const char *>(src0 + ((int64_t)row0 + 64 * wave) * k + (int64_t)kFirst * BK);
+    const char *aWave = reinterpret_cast<const char *>(src0 + ((int64_t)row0 + 16 * NMB * wave) * k + (int64_t)kFirst * BK);
     const char *bPanel = reinterpret_cast<const char *>(src1 + (int64_t)col0 * k + (int64_t)kFirst * BK);
     const uint32_t chunkEven = (lane % 8) ^ (lane / 16);
     const uint32_t aCopyOff[2] = {(lane / 8) * (uint32_t)ld + chunkEven * 16u, (lane / 8) * (uint32_t)ld + (chunkEven ^ 4u) * 16u};
@@ -189,9 +200,9 @@ AICORE inline __attribute__((always_inline)) void W4Pass(__gm__ const half *src0
     }
     // a copy in two halves: the LDS address (M0), and one slot later the copy itself; bases per copy in scalar registers,
     // the K offset of the step in the lane offsets
-    const char *aBase[8], *bBase[NCB];
+    const char *aBase[NA], *bBase[NCB];
 #pragma unroll
-    for (int t = 0; t < 8; ++t)
+    for (int t = 0; t < NA; ++t)
         aBase[t] = detail::uniform_ptr(aWave + (int64_t)(8 * t) * ld);
 #pragma unroll
     for (int t = 0; t < NCB; ++t)
@@ -223,21 +234,21 @@ AICORE inline __attribute__((always_inline)) void W4Pass(__gm__ const half *src0
         const uint32_t kOff = (uint32_t)clampStep(s) * (BK * 2);
         W4For<0, NCOPY>([&](auto jTag) __attribute__((always_inline)) {
             constexpr int j = decltype(jTag)::value;
-            if constexpr (j < 8)
+            if constexpr (j < NA)
                 setLds(aLdsWave, integral_constant<int, s * kASlot + j * 1024>());
             else
-                setLds(bLdsWave, integral_constant<int, s * kBBytes + (j - 8) * 4096>());
+                setLds(bLdsWave, integral_constant<int, s * kBBytes + (j - NA) * 4096>());
             asm volatile("s_nop 0" ::: "memory");
-            if constexpr (j < 8)
+            if constexpr (j < NA)
                 copyAsm(aCopyOff[j % 2] + kOff, aBase[j]);
             else
-                copyAsm(bCopyOff + kOff, bBase[j - 8]);
+                copyAsm(bCopyOff + kOff, bBase[j - NA]);
         });
     });
     hw::wait_vm<NCOPY>();
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    W4For<0, 8>([&](auto qTag) __attribute__((always_inline)) { readA(integral_constant<int, 0>(), qTag); });
+    W4For<0, NA>([&](auto qTag) __attribute__((always_inline)) { readA(integral_constant<int, 0>(), qTag); });
     W4For<0, PD>([&](auto fTag) __attribute__((always_inline)) {
         readB(integral_constant<int, decltype(fTag)::value % NBUF>(), integral_constant<int, 0>(), fTag);
     });
@@ -275,20 +286,20 @@ AICORE inline __attribute__((always_inline)) void W4Pass(__gm__ const half *src0
             }
             if constexpr (S::copyAt(idx + 1) >= 0) {
                 constexpr int j = S::copyAt(idx + 1);
-                if constexpr (j < 8)
+                if constexpr (j < NA)
                     setLds(aLdsWave, integral_constant<int, par * kASlot + j * 1024>());
                 else
-                    setLds(bLdsWave, integral_constant<int, sCopy * kBBytes + (j - 8) * 4096>());
+                    setLds(bLdsWave, integral_constant<int, sCopy * kBBytes + (j - NA) * 4096>());
             }
             if constexpr (S::copyAt(idx) >= 0) {
                 constexpr int j = S::copyAt(idx);
-                if constexpr (j < 8)
+                if constexpr (j < NA)
                     copyAsm(voffA[j % 2], aBase[j]);
                 else
-                    copyAsm(voffB, bBase[j - 8]);
+                    copyAsm(voffB, bBase[j - NA]);
             }
             if constexpr (mb == 0) // B fragment f has arrived; the reads issued after it may be under way
-                asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(PD + S::aReadsIn(4 * (f - PD), 4 * f)) : "memory");
+                asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(PD + S::aReadsIn(NMB * (f - PD), NMB * f)) : "memory");
             if constexpr (idx == S::kBarrier2) {
                 __builtin_amdgcn_s_barrier(); // every wave has the last B fragment of this step: the stage is dead
                 __builtin_amdgcn_sched_barrier(0);
@@ -317,66 +328,69 @@ AICORE inline __attribute__((always_inline)) void W4Pass(__gm__ const half *src0
     asm volatile("s_waitcnt lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
 }
 
-// accumulators = A[row0 .. + 256, :] x B[col0 .. + BN, :]^T over the whole K extent (k % 128 == 0, k >= 128)
-template <int BN>
+// accumulators = A[row0 .. + 64 NMB, :] x B[col0 .. + BN, :]^T over the whole K extent (k % 128 == 0, k >= 128)
+template <int BN, int NMB>
 AICORE inline __attribute__((always_inline)) void W4TileCompute(__gm__ const half *src0, __gm__ const half *src1, int k, int row0, int col0)
 {
     const int steps = k / 64, whole = steps / kW4Group * kW4Group, left = steps - whole;
-    W4ZeroAcc<BN / 4>();
+    W4ZeroAcc<NMB * BN / 16>();
     if (whole > 0)
-        W4Pass<BN, 0>(src0, src1, k, row0, col0, 0, whole);
+        W4Pass<BN, 0, NMB>(src0, src1, k, row0, col0, 0, whole);
     if (left == 2)
-        W4Pass<BN, 2>(src0, src1, k, row0, col0, whole, 2);
+        W4Pass<BN, 2, NMB>(src0, src1, k, row0, col0, whole, 2);
     else if (left == 4)
-        W4Pass<BN, 4>(src0, src1, k, row0, col0, whole, 4);
+        W4Pass<BN, 4, NMB>(src0, src1, k, row0, col0, whole, 4);
 }
 
 // this wave's accumulator blocks to C (row-major, n floats between rows)
-template <int BN>
+template <int BN, int NMB>
 AICORE inline __attribute__((always_inline)) void W4StoreTile(float *out, int64_t n, int row0, int col0)
 {
     constexpr int NNB = BN / 16;
     const uint32_t lane = (uint32_t)hw::lane();
-    float *cWave = out + ((int64_t)row0 + 64 * hw::wave() + lane % 16) * n + col0 + 4 * (lane / 16);
-    W4For<0, 4 * NNB>([&](auto idxTag) __attribute__((always_inline)) {
+    float *cWave = out + ((int64_t)row0 + 16 * NMB * hw::wave() + lane % 16) * n + col0 + 4 * (lane / 16);
+    W4For<0, NMB * NNB>([&](auto idxTag) __attribute__((always_inline)) {
         constexpr int idx = decltype(idxTag)::value, mb = idx / NNB, nb = idx % NNB;
         *reinterpret_cast<detail::AccFrag *>(cWave + (int64_t)(16 * mb) * n + 16 * nb) = W4ReadAcc<idx>();
     });
 }
 
-// One 256 x BN tile of C per workgroup.  Where 256 does not divide m (BN does not divide n) the last tile row (column) is
-// moved back so that it ends with the matrix: it computes some rows (columns) of its neighbour a second time and stores
-// the same values.
-template <int BN, int GROUP_M>
+// One 64 NMB x BN tile of C per workgroup.  Where the tile height does not divide m (BN does not divide n) the last tile
+// row (column) is moved back so that it ends with the matrix: it computes some rows (columns) of its neighbour a second
+// time and stores the same values.
+template <int BN, int GROUP_M, int NMB>
 __global__ __launch_bounds__(kBlockThreads, 1) AICORE
     void GemmF16F32W4(__gm__ float *out, __gm__ const half *src0, __gm__ const half *src1, int m, int n, int k)
 {
-    const int tilesM = (m + kW4TileM - 1) / kW4TileM, tilesN = (n + BN - 1) / BN;
+    constexpr int TM = 64 * NMB;
+    const int tilesM = (m + TM - 1) / TM, tilesN = (n + BN - 1) / BN;
     int tm, tn;
     TileOfId<GROUP_M>(RegroupXcd((int)get_block_idx(), tilesM * tilesN), tilesM, tilesN, tm, tn);
-    const int r = tm * kW4TileM, c = tn * BN;
-    const int row0 = __builtin_amdgcn_readfirstlane(r + kW4TileM <= m ? r : m - kW4TileM);
+    const int r = tm * TM, c = tn * BN;
+    const int row0 = __builtin_amdgcn_readfirstlane(r + TM <= m ? r : m - TM);
     const int col0 = __builtin_amdgcn_readfirstlane(c + BN <= n ? c : n - BN);
-    W4TileCompute<BN>(src0, src1, k, row0, col0);
-    W4StoreTile<BN>(out, n, row0, col0);
+    W4TileCompute<BN, NMB>(src0, src1, k, row0, col0);
+    W4StoreTile<BN, NMB>(out, n, row0, col0);
 }
 
 } // namespace
 PTO_DEVICE_CODE_END
 
 namespace {
-template <int BN>
+// NMB row blocks of 16 per wave: tiles of 256 (NMB = 4) or 192 (NMB = 3) rows
+template <int BN, int NMB = 4>
 int launch_gemm_w4(hipStream_t st, float *c, const half *a, const half *b, int m, int n, int k)
 {
+    constexpr int TM = 64 * NMB;
     // (n % 4: the accumulator blocks are stored 16 bytes at a time)
-    if (m < kW4TileM || n < BN || n % 4 || k % 128 || k < 128)
+    if (m < TM || n < BN || n % 4 || k % 128 || k < 128)
         return PTO_ERR_UNSUPPORTED;
-    constexpr int lds = 3 * 64 * BN * (int)sizeof(half) + 4 * 2 * 64 * 64 * (int)sizeof(half); // three B stages + two A slots per wave
-    auto kernel = GemmF16F32W4<BN, 4>;
+    constexpr int lds = 3 * 64 * BN * (int)sizeof(half) + 4 * 2 * (16 * NMB) * 64 * (int)sizeof(half); // three B stages + two A slots per wave
+    auto kernel = GemmF16F32W4<BN, 4, NMB>;
     static const int attr = pto_amd::allow_lds(kernel, lds);
     if (attr != PTO_OK)
         return attr;
-    const int tiles = ((m + kW4TileM - 1) / kW4TileM) * ((n + BN - 1) / BN);
+    const int tiles = ((m + TM - 1) / TM) * ((n + BN - 1) / BN);
     kernel<<<dim3((unsigned)tiles), dim3(kBlockThreads), lds, st>>>(c, a, b, m, n, k);
     return pto_amd::check_launch();
 }

@@ -1,7 +1,7 @@
 // fp16 x fp16 -> fp32 GEMM for MI355X written with PTO tile instructions:
 //   TLOAD (HBM -> LDS, async 16-byte copies)  ->  TEXTRACT (LDS -> MFMA operand fragments)
 //   ->  TMATMUL / TMATMUL_ACC (v_mfma_f32_32x32x16_f16)  ->  TSTORE (accumulators -> HBM);
-// and the entry point that picks among it, the K-64 kernel of pto_gemm_k64.hip and the four-wave kernel of pto_gemm_w4.hip.
+// and the entry point that picks between it and the four-wave kernel of pto_gemm_w4.hip.
 //
 // Same decomposition as the reference's manual kernel
 // (kernels/manual/a2a3/gemm_performance/gemm_performance_kernel.cpp:67-230): each "core" owns
@@ -46,18 +46,13 @@ extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const 
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
     // Problems with enough work for every compute unit: 256-row tiles on four wavefronts with K-steps of 64, the width
-    // chosen from 256 / 192 / 128 by the number of rounds it gives (pto_gemm_w4.hip; m >= 256, n >= 128, n % 4 == 0,
+    // chosen from 256 / 192 / 128 and the height from 256 / 192 by the number of rounds they give (pto_gemm_w4.hip; m >= 192, n >= 128, n % 4 == 0,
     // k % 128 == 0).  Small problems: the 128 x 256 block of the reference kernel with K-steps of 32, two workgroups of
     // four wavefronts per compute unit (m % 128 == 0, n % 256 == 0, k % 32 == 0).
     if ((long long)m * n >= (long long)compute_units() * 32768) {
         const int rc = pto_amd::gemm_f16f32_w4(st, c, ha, hb, m, n, k);
         if (rc != PTO_ERR_UNSUPPORTED)
             return rc;
-        // shapes those tiles do not divide: the K-64 kernel written with the tile instructions (eight wavefronts, 256 x 256,
-        // 384 x 192 or 256 x 192 tiles), where its tiles fill the rounds
-        const int rc64 = pto_amd::gemm_f16f32_k64(st, c, ha, hb, m, n, k);
-        if (rc64 != PTO_ERR_UNSUPPORTED)
-            return rc64;
     }
     const int rc = launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
     if (rc != PTO_ERR_UNSUPPORTED)

@@ -36,7 +36,6 @@ _V = [C.c_void_p] * 4 + [C.c_int] * 4
 ST_SYMBOLS = {
     "pto_gemm_f16f32_variant": (C.c_int, _V),
     "pto_gemm_f16f32_w4_variant": (C.c_int, _V),
-    "pto_gemm_f16f32_k64_variant": (C.c_int, _V),
     "pto_gemm_mxfp8_variant": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 6),
     "pto_fa_fwd_f16_variant": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 7),
     "pto_st_softmax_step_f32_64x256": (C.c_int, [C.c_void_p] * 8 + [C.c_float, C.c_int, C.c_int]),

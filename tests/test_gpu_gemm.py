@@ -30,11 +30,11 @@ def test_gemm_small_vs_oracle(oracle, m, n, k):
 
 
 def test_gemm_every_dispatch_path_agrees_with_integer_reference():
-    """4096 x 4096 selects the four-wave kernel with 256 x 256 tiles, 4096 x 4224 the same kernel with 256 x 192 tiles,
-    4224 x 4224 (rows not a multiple of 256) the K-64 kernel written with the tile instructions (384 x 192 tiles),
+    """4096 x 4096 selects the four-wave kernel with 256 x 256 tiles, 4096 x 4224 and 4224 x 4224 (rows not a multiple of
+    256: the last tile row is moved back) the same kernel with 256 x 192 tiles, 3072 x 3072 its 192 x 192 tiles,
     1024 x 1024 the 128 x 256-block kernel: all exact on integer inputs."""
     from gpu_util import gemm
-    for m, n, k in ((4096, 4096, 512), (4096, 4224, 512), (4224, 4224, 512), (1024, 1024, 512)):
+    for m, n, k in ((4096, 4096, 512), (4096, 4224, 512), (4224, 4224, 512), (3072, 3072, 512), (1024, 1024, 512)):
         a, b = datagen.gemm_inputs_integer(m, n, k)
         got = gemm(a, b)
         rows = np.r_[0:64, m // 2:m // 2 + 64, m - 64:m]
@@ -45,7 +45,7 @@ def test_gemm_every_dispatch_path_agrees_with_integer_reference():
 
 
 def test_gemm_four_wave_tile_widths_exact():
-    """Every tile width of the four-wave kernel (tuning hook: 256 x 256, 256 x 192, 256 x 128) on integer inputs, the whole
+    """Every tile shape of the four-wave kernel (tuning hook: 256 or 192 rows x 256 / 192 / 128 columns) on integer inputs, the whole
     matrix exactly, with K extents of whole groups of six K-steps (384, 768), of groups plus two or four steps (512, 640,
     1152 + 128) and of a tail alone (128, 256); one tile and several; and the shapes that the kernel refuses."""
     import torch
@@ -56,14 +56,15 @@ def test_gemm_four_wave_tile_widths_exact():
         a, b = datagen.gemm_inputs_integer(m, n, k)
         want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
         ta, tb = to_dev(a), to_dev(b)
-        for variant in (0, 1, 2):
+        for variant in range(6):
             tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
-            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "four-wave GEMM width %d" % variant)
+            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "four-wave GEMM shape %d" % variant)
             torch.cuda.synchronize()
             assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
     p = ta.data_ptr()
     assert fn(0, p, p, p, 256, 768, 192, 0) == capi.ERR_UNSUPPORTED      # k not a multiple of 128
     assert fn(0, p, p, p, 192, 768, 256, 0) == capi.ERR_UNSUPPORTED      # fewer rows than a tile
+    assert fn(0, p, p, p, 128, 768, 256, 4) == capi.ERR_UNSUPPORTED
     assert fn(0, p, p, p, 256, 160, 256, 1) == capi.ERR_UNSUPPORTED      # fewer columns than the width
     assert fn(0, p, p, p, 256, 770, 256, 1) == capi.ERR_UNSUPPORTED      # rows of C not a multiple of 16 bytes
 
@@ -79,9 +80,9 @@ def test_gemm_ragged_m_and_n_exact():
         a, b = datagen.gemm_inputs_integer(m, n, k)
         want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
         ta, tb = to_dev(a), to_dev(b)
-        for variant in (0, 1, 2):
+        for variant in range(6):
             tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
-            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "four-wave GEMM width %d" % variant)
+            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "four-wave GEMM shape %d" % variant)
             torch.cuda.synchronize()
             assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
     lib = capi.load()
@@ -93,24 +94,6 @@ def test_gemm_ragged_m_and_n_exact():
         torch.cuda.synchronize()
         want = ta.view(torch.float16).double() @ tb.view(torch.float16).double().T
         assert torch.equal(tc.double(), want), (m, n, k)
-
-
-def test_gemm_k64_tile_shapes_exact():
-    """Every tile shape of the kernel with K-steps of 64 that is written with the tile instructions (384 x 192, 256 x 256,
-    256 x 192) on integer inputs, two and six K-steps: the whole matrix, exactly; and an unsupported K."""
-    import torch
-    from gpu_util import to_dev
-    fn = capi.load_st().pto_gemm_f16f32_k64_variant
-    for m, n, k in ((768, 768, 128), (1536, 2304, 384)):
-        a, b = datagen.gemm_inputs_integer(m, n, k)
-        want = (a.astype(np.int64) @ b.astype(np.int64).T).astype(np.float32)
-        ta, tb = to_dev(a), to_dev(b)
-        for variant in (0, 1, 2):
-            tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0")
-            capi.check(fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k, variant), "K-64 GEMM variant %d" % variant)
-            torch.cuda.synchronize()
-            assert np.array_equal(tc.cpu().numpy(), want), (m, n, k, variant)
-        assert fn(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), m, n, k + 64, 0) == capi.ERR_UNSUPPORTED
 
 
 def test_gemm_6144_every_element_exact():
