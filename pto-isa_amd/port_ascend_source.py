@@ -35,10 +35,14 @@ script therefore does (nothing else is touched; the tile code itself compiles as
 12. Reads of Ascend's special scalar registers written as inline assembly, `asm volatile("MOV %0, SYS_CNT\n" : "+l"(x));`
     and `... PC ...`, become `x = get_sys_cnt();` and `x = 0;` (time stamps that the test kernels log, and the program
     counter they hand to an instruction-cache preload, which is a no-op here).
-13. A kernel template over `S1`, `CUBE_S1`, `TILE_S1` and `QK_PRELOAD` (the flash-attention kernel `runTFA`) gets a
-    `static_assert(TILE_S1 == CUBE_S1 || S1 <= QK_PRELOAD * TILE_S1)` at the top of its body: one workgroup plays the Cube
-    and the Vec role of a block in program order, and a Vec-side score tile wider than what the Cube side has produced
-    would be read half-written.  Such a case stops the build instead of returning wrong output.
+13. Loops over role blocks are split.  A source written for a Cube core and its Vec cores interleaves their work in one
+    loop, `for (...) { if constexpr (DAV_CUBE) {A} if constexpr (DAV_VEC) {B} if constexpr (DAV_CUBE) {C} }`, and relies
+    on the cores running side by side: B of an iteration may wait (through a FIFO) for what A produces in later
+    iterations (the flash-attention kernel's Vec side takes a row slice of a whole score tile of which each iteration of
+    its Cube side produces one column block, fa_performance_kernel.cpp:862-907).  One workgroup plays both roles in
+    program order, so an innermost loop whose body is nothing but such blocks becomes one loop per block with the same
+    header, `for (...) {A}  for (...) {B}  for (...) {C}`: every producer has then run before its consumer.  The blocks
+    talk to each other through FIFOs only, which is what makes the order of different roles' blocks free on the NPU too.
 """
 import argparse
 import os
@@ -49,11 +53,56 @@ LAUNCH = re.compile(r"<<<\s*([^,<>]+?)\s*,\s*nullptr\s*,\s*([^<>]+?)\s*>>>")
 LOCAL_INCLUDE = re.compile(r'^[ \t]*#include[ \t]+"([^"]+)"[ \t]*$', re.M)
 STATIC_LOCAL = re.compile(r"^([ \t]+)static[ \t]+([A-Za-z_][\w:]*(?:[ \t]+[A-Za-z_][\w:]*)*)[ \t]+([A-Za-z_]\w*)[ \t]*=[ \t]*([^;]+);", re.M)
 KERNEL_HEAD = re.compile(r"__global__[^;{}]*?\)\s*\{")
-# a kernel template over CUBE_S1, TILE_S1 and QK_PRELOAD (runTFA of fa_performance_kernel.cpp:607-609), up to its opening brace
-TFA_KERNEL = re.compile(r"template\s*<[^<>{};]*\bS1\b[^<>{};]*\bCUBE_S1\b[^<>{};]*\bTILE_S1\b[^<>{};]*\bQK_PRELOAD\b[^<>{};]*>\s*__global__[^;{}]*?\)\s*\{")
-TFA_ASSERT = ('static_assert(TILE_S1 == CUBE_S1 || S1 <= QK_PRELOAD * TILE_S1, "[PTO][SA] flash-attention kernel on gfx950: the Vec role runs '
-              'after the Cube role in program order; TILE_S1 > CUBE_S1 needs the whole key range inside the preload (S1 <= QK_PRELOAD * TILE_S1)");')
+ROLE_BLOCK = re.compile(r"\s*if\s+constexpr\s*\(\s*DAV_(?:CUBE|VEC)\s*\)\s*\{")
+FOR_HEAD = re.compile(r"^([ \t]*)for\s*\(", re.M)
 BEGIN_MARK, END_MARK = "//@@PTO_INLINED_BEGIN ", "//@@PTO_INLINED_END "
+
+
+def _match(text, pos, open_ch, close_ch):
+    """Index just behind the bracket that closes the one at text[pos] (comments and literals of the sources this script
+    sees hold no unbalanced brackets)."""
+    depth = 0
+    for i in range(pos, len(text)):
+        c = text[i]
+        if c == open_ch:
+            depth += 1
+        elif c == close_ch:
+            depth -= 1
+            if depth == 0:
+                return i + 1
+    raise SystemExit("port_ascend_source: unbalanced %s" % open_ch)
+
+
+def split_role_loops(text):
+    """Rule 13: innermost `for` loops whose body consists of two or more `if constexpr (DAV_CUBE / DAV_VEC) {...}` blocks
+    and nothing else become one loop per block.  Returns the new text and the number of loops split."""
+    out, pos, count = [], 0, 0
+    for m in FOR_HEAD.finditer(text):
+        if m.start() < pos:
+            continue
+        head_end = _match(text, text.index("(", m.start()), "(", ")")
+        brace = re.compile(r"\s*\{").match(text, head_end)
+        if not brace:
+            continue
+        body_begin, body_end = brace.end(), _match(text, brace.end() - 1, "{", "}") - 1
+        body = text[body_begin:body_end]
+        blocks, at = [], 0
+        while True:
+            rb = ROLE_BLOCK.match(body, at)
+            if not rb:
+                break
+            end = _match(body, rb.end() - 1, "{", "}")
+            blocks.append(body[at:end])
+            at = end
+        if len(blocks) < 2 or body[at:].strip() or any(re.search(r"\bfor\s*\(", blk) for blk in blocks):
+            continue
+        indent, header = m.group(1), text[m.start():head_end].lstrip()
+        loops = "\n".join("%s%s {%s\n%s}" % (indent, header, blk.rstrip(), indent) for blk in blocks)
+        out.append(text[pos:m.start()] + loops)
+        pos = body_end + 1
+        count += 1
+    out.append(text[pos:])
+    return "".join(out), count
 
 
 def inline_local_includes(text, directory, seen=None):
@@ -194,9 +243,9 @@ def port(text, sets=(), lds_bytes=160 * 1024, defines=(), directory=None, vec_in
         text, k = KERNEL_HEAD.subn(lambda m: m.group(0) + "\n    PTO_KERNEL_PROLOGUE();", text)
         notes.append("%d kernel prologue%s inserted" % (k, "" if k == 1 else "s"))
     # 13. the flash-attention kernel: one workgroup plays the Cube and the Vec role of a block in program order
-    text, k13 = TFA_KERNEL.subn(lambda m: m.group(0) + "\n    " + TFA_ASSERT, text)
+    text, k13 = split_role_loops(text)
     if k13:
-        notes.append("%d flash-attention kernel%s: schedule checked at compile time" % (k13, "" if k13 == 1 else "s"))
+        notes.append("%d loop%s over Cube / Vec role blocks split into one loop per block" % (k13, "" if k13 == 1 else "s"))
 
     # 1. brackets.  Inlined .hpp files are device code as a whole; in the main file the device code opens after the
     # prologue (comments, includes, using-directives, macro definitions and file-scope constants come first in these

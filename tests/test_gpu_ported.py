@@ -50,12 +50,16 @@ def test_reference_gemm_performance_kernel_6144(oracle):
     assert np.abs(got[rows] - want).max() <= 2e-3 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("S0,S1,causal,tile_s1,preload", [(128, 1024, False, 256, 4), (256, 2048, False, 128, 4),
+@pytest.mark.parametrize("S0,S1,causal,tile_s1,preload", [(128, 1024, False, 256, 4), (128, 2048, False, 256, 4),
+                                                          (128, 8192, False, 256, 4), (512, 2048, False, 256, 4),
+                                                          (256, 2048, True, 256, 2), (256, 2048, False, 128, 4),
                                                           (256, 1024, True, 128, 4), (512, 2048, True, 128, 2)])
 def test_reference_flash_attention_kernel(oracle, S0, S1, causal, tile_s1, preload):
     """fa_performance_kernel.cpp: runTFA with its Cube / Vec stage functions, stage macros, TPipe FIFOs in global memory and
     Vec tiles as views of a unified buffer, launched through its own LaunchTFA<S0, 128, S1, 128, 128, TILE_S1, QK_PRELOAD, 8,
-    false, CAUSAL, 4> with the workspace its host program allocates (main.cpp:126-207).  O [S0, 128] fp32 against a dense
+    false, CAUSAL, 4> with the workspace its host program allocates (main.cpp:126-207).  The first four cases are the
+    reference generator's default schedule (score tiles of 256 keys made of two 128-wide cube tiles, preload 4) at 1024, 2048
+    and 8192 keys.  O [S0, 128] fp32 against a dense
     float64 softmax (2e-3 of the largest |O|) and against the oracle's restatement of the streaming recurrence with the same
     key tile and the NPU's round-half-away cast of P (5e-4: rounding only).  Data as the reference's generator draws them
     (scripts/gen_data.py:26-35: seed 7, N(0,1) * 1.5 / 1.2 / 1)."""

@@ -108,17 +108,44 @@ void Launch(float *out, void *stream)
     many = src.replace("    static int calls = 0;\n", "".join("    static int c%d = 0;\n" % i for i in range(32)) + "    int calls = 0;\n")
     with pytest.raises(SystemExit, match="33 function-local statics"):
         mod.port(many, [("kSize", "128")], 4096, ("__DAV_VEC__",), None, True)
-    # a flash-attention kernel (a __global__ runTFA with the reference's template parameters) gets the check of its schedule
-    tfa = """#include <pto/pto-inst.hpp>
-template <int S0, int HEAD_SIZE, int S1, int CUBE_S0, int CUBE_S1, int TILE_S1, int QK_PRELOAD>
-__global__ AICORE void runTFA(__gm__ half *q)
+    # an innermost loop over Cube / Vec role blocks becomes one loop per block; loops with anything else in the body, or whose
+    # blocks hold loops themselves, stay
+    roles = """#include <pto/pto-inst.hpp>
+__global__ AICORE void k(__gm__ float *o)
 {
-    q[0] = 0;
+    for (int t = 0; t < 4; ++t) {
+        int next = t + 1;
+        for (int s = 0; s < 2; ++s) {
+            if constexpr (DAV_CUBE) {
+                o[0] += s;
+            }
+            if constexpr (DAV_VEC) {
+                o[1] += next;
+            }
+            if constexpr (DAV_CUBE) {
+                o[2] += t;
+            }
+        }
+        if constexpr (DAV_VEC) {
+            o[3] += 1;
+        }
+    }
+    for (int p = 0; p < 4; ++p) {
+        if constexpr (DAV_CUBE) {
+            for (int s = 0; s < 2; ++s)
+                o[4] += s;
+        }
+        if constexpr (DAV_VEC) {
+            o[5] += p;
+        }
+    }
 }
 """
-    text2, notes2 = mod.port(tfa, [], 4096, (), None, True)
-    assert "static_assert(TILE_S1 == CUBE_S1 || S1 <= QK_PRELOAD * TILE_S1" in text2
-    assert text2.index("static_assert(TILE_S1 == CUBE_S1") < text2.index("q[0] = 0;")
+    text2, notes2 = mod.port(roles, [], 4096, ("DAV_CUBE=1", "DAV_VEC=1"), None, True)
+    assert any("1 loop over Cube / Vec role blocks split" in n for n in notes2), notes2
+    assert text2.count("for (int s = 0; s < 2; ++s) {") == 3 and text2.count("for (int p = 0; p < 4; ++p) {") == 1
+    cube0, vec1, cube2 = text2.index("o[0] += s;"), text2.index("o[1] += next;"), text2.index("o[2] += t;")
+    assert cube0 < text2.index("for (int s = 0; s < 2; ++s) {", cube0) < vec1 < text2.index("for (int s = 0; s < 2; ++s) {", vec1) < cube2
     assert "<<<pto::host::LaunchBlocks(4, (hipStream_t)(stream)), pto::kBlockThreads, pto::host::LaunchLds((const void *)(kern), 4096), (hipStream_t)(stream)>>>" in text
     assert "__global__ __launch_bounds__(pto::kBlockThreads) AICORE void kern" in text
     assert text.startswith("#define PTO_TILE_COPY_WRITEBACK 1\n#define PTO_VEC_TILES_IN_MEMORY 1\n#define __DAV_VEC__ 1\n")
