@@ -6,12 +6,14 @@
 // The arena is one device allocation, `blocks * PTO_UB_BYTES` bytes, made by pto::host::PrepareUnifiedBuffer before a
 // launch (port_ascend_source.py puts the call in front of every launch statement); the kernels of the translation unit
 // find it through a device variable.  Launches of one translation unit that overlap in time share the arena: keep them on
-// one stream.
+// one stream.  Host threads may call concurrently (one lock around the bookkeeping); when the arena has to grow, the
+// whole device is synchronised before the old one is freed, whichever streams still use it.
 #pragma once
 #include <hip/hip_runtime.h>
 
 #include <cstddef>
 #include <cstdint>
+#include <mutex>
 
 #ifndef PTO_UB_BYTES
 #define PTO_UB_BYTES (512 * 1024)
@@ -38,13 +40,15 @@ namespace host {
 // Returns hipSuccess or the first HIP error.  The arena only grows and is kept until the process ends.
 inline hipError_t PrepareUnifiedBuffer(unsigned blocks, hipStream_t stream)
 {
+    static std::mutex lock;
     static char *arena = nullptr;
     static size_t capacity = 0;
+    const std::lock_guard<std::mutex> guard(lock);
     const size_t need = (size_t)blocks * (size_t)PTO_UB_BYTES;
     hipError_t e = hipSuccess;
     if (need > capacity) {
         if (arena) {
-            e = hipStreamSynchronize(stream);
+            e = hipDeviceSynchronize();
             if (e == hipSuccess)
                 e = hipFree(arena);
             if (e != hipSuccess)
