@@ -63,7 +63,8 @@ int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b
  * format per operand).  scale_a [m,k/32] and scale_b stored [n,k/32] hold one e8m0 exponent per row
  * (column) and 32 consecutive k (the reference's x1_gm / x2_gm / x1_scale_gm / x2_scale_gm files).  c: bf16
  * (c_fp32 == 0, round-to-nearest-even of the fp32 sum) or fp32.  m >= 256, n >= 256 (any value: the last tile row /
- * column is moved back to end at m / n and recomputes what it overlaps), k % 512 == 0. */
+ * column is moved back to end at m / n and recomputes what it overlaps; fp8 also 128 <= n < 256 when n % 4 == 0),
+ * k % 512 == 0. */
 int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
                    int m, int n, int k, int format, int c_fp32);
 

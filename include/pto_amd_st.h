@@ -19,7 +19,9 @@ int pto_gemm_f16f32_variant(void *stream, float *c, const uint16_t *a, const uin
 /* four wavefronts, K-steps of 64, A in a ring per wave: 0 = 256 x 256 tiles, 1 = 256 x 192, 2 = 256 x 128, 3 = 192 x 256,
  * 4 = 192 x 192, 5 = 192 x 128 (csrc/pto_gemm_w4.hip) */
 int pto_gemm_f16f32_w4_variant(void *stream, float *c, const uint16_t *a, const uint16_t *b, int m, int n, int k, int variant);
-/* MX GEMM: variant bit 0 = quarter tiles in the last round, bit 1 = the shallower copy pipeline (csrc/pto_gemm_mx.hip) */
+/* MX GEMM: variant 0 .. 3: bit 0 = quarter tiles in the last round, bit 1 = the shallower copy pipeline (csrc/pto_gemm_mx.hip);
+ * fp8 formats only: 4 = the four-wave kernel with the width its estimate picks, 5 = its 256 x 192 tiles, 6 = 256 x 128
+ * (csrc/pto_gemm_mxw4.hip) */
 int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                            const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant);
 /* flash attention: workgroup size, occupancy, queries per wave and MFMA shape by number (csrc/pto_fa.hip: 1 / 2 / 5 = four

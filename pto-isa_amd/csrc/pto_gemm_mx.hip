@@ -24,6 +24,8 @@
 #define PTO_WAVES_N 4
 #include "gemm_kernels.hpp"
 
+#include <algorithm>
+
 PTO_DEVICE_CODE_BEGIN
 
 namespace {
@@ -352,6 +354,23 @@ extern "C" int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uin
         return PTO_ERR_BAD_ARG;
     if (format < 0 || format > 3)
         return PTO_ERR_UNSUPPORTED;
+    // Two kernels: 256 x 256 tiles on eight wavefronts (this file; quarter tiles in a last partial round) and 256 x 192 /
+    // 256 x 128 tiles on four wavefronts (pto_gemm_mxw4.hip: the faster engine, the smaller tile).  Estimated times in
+    // microseconds, rounds over the compute units x (K-steps of 128 x step time + fixed time) as measured at 4096^3,
+    // 6144^3 and 8192^3: 6144^3 is 2.25 rounds of 256 x 256 and 3 of 256 x 192 (2335 against 2610 TFLOP/s), 8192^3 is 4
+    // whole rounds of 256 x 256 (2600 against 2440).
+    if (m >= 256 && n >= 128 && n % 4 == 0 && k % 512 == 0) {
+        const int cus = compute_units(), steps = k / 128;
+        const double t4 = std::min(pto_amd::mxfp8_w4_time(m, n, k, 192), pto_amd::mxfp8_w4_time(m, n, k, 128));
+        double t8 = 1e30;
+        if (n >= 256) {
+            const long long tiles = (long long)((m + 255) / 256) * ((n + 255) / 256), full = tiles / cus, rest = tiles - full * cus;
+            const bool quarters = rest > 0 && full > 0 && rest * 4 <= cus && m % 256 == 0 && n % 256 == 0;
+            t8 = (double)full * (steps * 1.4 + 16.0) + (rest == 0 ? 0.0 : (quarters ? steps * 0.34 + 16.0 : steps * 1.4 + 16.0));
+        }
+        if (t4 < t8)
+            return pto_amd::gemm_mxfp8_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 0);
+    }
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 1);
 }
 
@@ -369,8 +388,11 @@ extern "C" int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uin
 extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                                       const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32, int variant)
 {
-    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0 || variant < 0 || variant > 3)
+    if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0 || variant < 0 || variant > 6)
         return PTO_ERR_BAD_ARG;
+    if (variant >= 4) // the four-wave engine: 4 = width by rounds, 5 = 256 x 192 tiles, 6 = 256 x 128
+        return pto_amd::gemm_mxfp8_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32,
+                                      variant == 4 ? 0 : (variant == 5 ? 192 : 128));
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, variant);
 }
 #endif // PTO_ST_HOOKS

@@ -128,6 +128,76 @@ def test_mx_gemm_ragged_m_n(oracle, fmt, m, n, k):
     assert np.array_equal(got16, bf16_rne(got))
 
 
+def _mx_variant(a, b, sa, sb, fmt, variant, c_fp32=True):
+    """pto_gemm_mxfp8_variant of the test library: one kernel whatever the public entry point would pick."""
+    import torch
+    from gpu_util import to_dev
+    lib = capi.load_st()
+    (m, k), n = a.shape, b.shape[0]
+    ta, tb, tsa, tsb = (to_dev(x) for x in (a, b, sa, sb))
+    tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0") if c_fp32 else \
+        torch.full((m, n), -1, dtype=torch.int16, device="cuda:0")
+    rc = lib.pto_gemm_mxfp8_variant(0, tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), m, n, k, fmt,
+                                    int(c_fp32), variant)
+    torch.cuda.synchronize()
+    out = tc.cpu().numpy()
+    return rc, (out if c_fp32 else out.view(np.uint16))
+
+
+@pytest.mark.parametrize("variant", [5, 6])
+@pytest.mark.parametrize("m,n,k", [(256, 192, 512), (256, 512, 1024), (512, 384, 1536), (768, 768, 2048), (300, 260, 512),
+                                   (1000, 1100, 1024)])
+def test_mx_gemm_four_wave_kernel(oracle, m, n, k, variant):
+    """The MXFP8 kernel on four wavefronts (256 x 192 and 256 x 128 tiles; one, two and four groups of four K-steps; m and n
+    that the tiles do not divide): integer operands exactly, the generator's distribution to the GEMM tolerance, both fp8
+    formats and a mixed pair, the bf16 result = RNE of the fp32 one."""
+    for fmt in (0, 1):
+        a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt, dist="integer")
+        rc, got = _mx_variant(a, b, sa, sb, fmt, variant)
+        capi.check(rc, "four-wave MX kernel")
+        assert np.array_equal(got, oracle.mx_gemm(a, b, sa, sb, fmt)), (fmt, "integer")
+        a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt)
+        rc, got = _mx_variant(a, b, sa, sb, fmt, variant)
+        assert rc == 0 and np.all(np.isfinite(got)) and rel_err(got, oracle.mx_gemm(a, b, sa, sb, fmt)) <= TOL
+        rc, got16 = _mx_variant(a, b, sa, sb, fmt, variant, c_fp32=False)
+        assert rc == 0 and np.array_equal(got16, bf16_rne(got))
+    a, _, sa, sb = datagen.mx_inputs(m, n, k, 0, dist="bytes")
+    _, b, _, _ = datagen.mx_inputs(m, n, k, 1, dist="bytes")
+    rc, got = _mx_variant(a, b, sa, sb, 2, variant)
+    assert rc == 0 and np.all(np.isfinite(got)) and rel_err(got, oracle.mx_gemm(a, b, sa, sb, 0, 1)) <= TOL
+    a3, _, sa3, sb3 = datagen.mx_inputs(m, n, k, 1, dist="bytes")
+    _, b3, _, _ = datagen.mx_inputs(m, n, k, 0, dist="bytes")
+    rc, got = _mx_variant(a3, b3, sa3, sb3, 3, variant)
+    assert rc == 0 and np.all(np.isfinite(got)) and rel_err(got, oracle.mx_gemm(a3, b3, sa3, sb3, 1, 0)) <= TOL
+
+
+def test_mx_gemm_four_wave_kernel_scale_of_every_block(oracle):
+    """Every (row, k block) scale of A and every (column, k block) scale of B reaches its products: operands of ones, scales
+    drawn per block from {2^-2 .. 2^3}, so that C[i, j] = 32 sum_b 2^(sa[i, b] + sb[j, b] - 254) exactly."""
+    m, n, k = 512, 384, 2048
+    rng = np.random.default_rng(77)
+    one = 0x38  # 1.0 in e4m3
+    a = np.full((m, k), one, dtype=np.uint8)
+    b = np.full((n, k), one, dtype=np.uint8)
+    sa = rng.integers(125, 131, size=(m, k // 32)).astype(np.uint8)
+    sb = rng.integers(125, 131, size=(n, k // 32)).astype(np.uint8)
+    want = 32.0 * (np.exp2(sa.astype(np.float64) - 127) @ np.exp2(sb.astype(np.float64) - 127).T)
+    for variant in (5, 6):
+        rc, got = _mx_variant(a, b, sa, sb, 0, variant)
+        assert rc == 0 and np.array_equal(got.astype(np.float64), want), variant
+    assert np.array_equal(want, oracle.mx_gemm(a, b, sa, sb, 0).astype(np.float64))
+
+
+def test_mx_gemm_four_wave_kernel_refuses():
+    import torch
+    p = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda:0").data_ptr()
+    fn = capi.load_st().pto_gemm_mxfp8_variant
+    assert fn(0, p, p, p, p, p, 128, 512, 512, 0, 1, 5) == capi.ERR_UNSUPPORTED     # fewer than 256 rows
+    assert fn(0, p, p, p, p, p, 256, 160, 512, 0, 1, 5) == capi.ERR_UNSUPPORTED     # narrower than the tile
+    assert fn(0, p, p, p, p, p, 256, 258, 512, 0, 1, 6) == capi.ERR_UNSUPPORTED     # rows of C not a multiple of four elements
+    assert fn(0, p, p, p, p, p, 256, 256, 640, 0, 1, 6) == capi.ERR_UNSUPPORTED     # k not whole groups of four steps
+
+
 def test_mxfp4_gemm_reference_config_2040_8192_8100(oracle):
     """The reference's matmul_mxfp4_performance case: e2m1 operands, m, k, n = 2040, 8192, 8100, bf16 result, its generator's
     integer distribution in [-6, 6) and scales 2^0 .. 2^2: partial sums stay below 2^24, so the fp32 result is exact."""
