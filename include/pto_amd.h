@@ -63,14 +63,15 @@ int pto_gemm_f16f32(void *stream, float *c, const uint16_t *a, const uint16_t *b
  * format per operand).  scale_a [m,k/32] and scale_b stored [n,k/32] hold one e8m0 exponent per row
  * (column) and 32 consecutive k (the reference's x1_gm / x2_gm / x1_scale_gm / x2_scale_gm files).  c: bf16
  * (c_fp32 == 0, round-to-nearest-even of the fp32 sum) or fp32.  m >= 256, n >= 256 (any value: the last tile row /
- * column is moved back to end at m / n and recomputes what it overlaps; fp8 also 128 <= n < 256 when n % 4 == 0),
+ * column is moved back to end at m / n and recomputes what it overlaps; also 128 <= n < 256 when n % 4 == 0),
  * k % 512 == 0. */
 int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
                    int m, int n, int k, int format, int c_fp32);
 
 /* MXFP4 GEMM: as pto_gemm_mxfp8 with 4-bit e2m1 operands packed two per byte, element 2i in bits 0-3 (the reference's
  * pack_two_fp4): a [m,k/2] bytes, b stored [n,k/2] bytes (LaunchMxMatmul of
- * kernels/manual/a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp).  Same limits. */
+ * kernels/manual/a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp).  Same limits (128 <= n < 256 only
+ * when k % 1024 == 0 as well). */
 int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
                    int m, int n, int k, int c_fp32);
 

@@ -36,11 +36,11 @@ inline int allow_lds(K kernel, int bytes)
 // defined in pto_gemm_w4.hip (256 x 256 / 192 / 128 tiles on four wavefronts, K-steps of 64); PTO_ERR_UNSUPPORTED unless m is a
 // multiple of 256, n of one of the widths and k of 128
 int gemm_f16f32_w4(hipStream_t st, float *c, const _Float16 *a, const _Float16 *b, int m, int n, int k);
-// defined in pto_gemm_mxw4.hip (MXFP8 on the four-wave engine: 256 x 192 or 256 x 128 tiles, width 0 = chosen by rounds);
-// PTO_ERR_UNSUPPORTED unless m >= 256, n >= 128, n % 4 == 0, k % 512 == 0
-int gemm_mxfp8_w4(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n, int k,
+// defined in pto_gemm_mxw4.hip (MXFP8 / MXFP4 on the four-wave engine: 256 x 192 or 256 x 128 tiles, width 0 = chosen by
+// rounds); PTO_ERR_UNSUPPORTED unless m >= 256, n >= 128, n % 4 == 0, k % 512 == 0 (fp4, format 4: k % 1024 == 0)
+int gemm_mx_w4(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n, int k,
                   int format, int c_fp32, int width);
-double mxfp8_w4_time(int m, int n, int k, int width);
+double mx_w4_time(int m, int n, int k_bytes, int width, bool fp4);
 // defined in pto_fa_w8.hip (head_dim 128, workgroups of eight wavefronts = 256 queries, two groups of four waves in
 // opposite MFMA / softmax phases)
 int fa_fwd_d128_w8(hipStream_t st, void *o, float *lse, const _Float16 *q, const _Float16 *k, const _Float16 *v, int batch, int heads,

@@ -11,6 +11,9 @@
 //   * four B stages (96 + 64 KiB = the whole LDS at BN = 192), which makes the step's second barrier unnecessary: a
 //     stage is overwritten two steps after its last read, with the barrier of the step in between.
 // Steps come in groups of four (B stage, A slot and scale byte repeat): k % 512 == 0.
+// MXFP4 (format 4, two e2m1 per byte): a K-step of 128 bytes is 256 k = two MFMAs (4 passes each, 16-byte operands: lane group
+// g holds bytes 16 g .. + 15 of the MFMA's 64) and eight scale blocks per row, so the 16 scale bytes of a row last two steps
+// and the MFMA of step j % 2 and half kk selects byte 2 (j % 2) + kk of the picked register: k % 1024 == 0.
 #pragma once
 #include "gemm_kernels_w4.hpp"
 
@@ -31,6 +34,20 @@ PTO_DEV void MxW4Mfma(i32x8 first, i32x8 second, uint32_t scaleFirst, uint32_t s
 #undef X
 }
 
+// the same with 4-bit operands: 16 rows x 128 k = 64 bytes per row, 16 per lane
+template <int BLK, int SEL>
+PTO_DEV void MxW4MfmaFp4(u32x4 first, u32x4 second, uint32_t scaleFirst, uint32_t scaleSecond)
+{
+#define X(b, r0, r1, r2, r3)                                                                                                          \
+    if constexpr (BLK == b)                                                                                                           \
+        asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 a[" #r0 ":" #r3 "], %0, %1, a[" #r0 ":" #r3 "], %2, %3 op_sel:[%4,%4,0] "       \
+                     "op_sel_hi:[%5,%5,0] cbsz:4 blgp:4" ::"v"(first),                                                                \
+                     "v"(second), "v"(scaleFirst), "v"(scaleSecond), "n"(SEL & 1), "n"(SEL >> 1)                                      \
+                     : "a" #r0, "a" #r1, "a" #r2, "a" #r3);
+    PTO_W4_ACC_BLOCKS(X)
+#undef X
+}
+
 // 16 bytes per lane from memory as assembly (counted by the kernel's own waits); use the result only behind such a wait
 PTO_DEV u32x4 MxW4Load16(const char *base, uint32_t voff)
 {
@@ -46,7 +63,7 @@ PTO_DEV void MxW4WaitLoads(u32x4 &x) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(
 // Issue slots of a K-step: slot = 4 nb + mb (nb: 16-column block, outer; mb: 16-row block of the wave's 64 rows).
 template <int NNB, int NCOPY>
 struct MxW4Sched {
-    static constexpr int kPD = 2, kSlots = 4 * NNB, kBarrier = 4 * (NNB - kPD) - 1, kScaleLoads = 4;
+    static constexpr int kPD = 2, kSlots = 4 * NNB, kBarrier = 4 * (NNB - kPD) - 1;
     // the eight A reads of the next step
     static constexpr int aReadSlot(int q) { return NNB >= 10 ? 4 * (q + 1) + 3 : 4 * (q / 2 + 1) + 2 + q % 2; }
     static constexpr int copySlot(int j) { return 2 + j * (kSlots - 6) / NCOPY; }
@@ -93,8 +110,9 @@ struct MxW4Sched {
     static_assert(aReadSlot(7) < kBarrier && copySlot(NCOPY - 1) < kSlots && copySlot(0) >= 2 && distinct(), "order of the step");
 };
 
-// accumulators = (A .* scales)[row0 .. + 256, :] x (B .* scales)[col0 .. + BN, :]^T over the whole K extent (k % 512 == 0);
-// block (mb, nb) of this wave's 64 rows in accumulator block (BN / 16) mb + nb.  FMT: 0 = e4m3, 1 = e5m2.
+// accumulators = (A .* scales)[row0 .. + 256, :] x (B .* scales)[col0 .. + BN, :]^T over the whole K extent (k elements, four
+// K-steps of 128 bytes per row at a time); block (mb, nb) of this wave's 64 rows in accumulator block (BN / 16) mb + nb.
+// FMT: 0 = e4m3, 1 = e5m2, 4 = e2m1 (both operands then).
 template <int FMT_A, int FMT_B, int BN>
 AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const uint8_t *src0, __gm__ const uint8_t *src1,
                                                                   __gm__ const uint8_t *scale0, __gm__ const uint8_t *scale1, int k,
@@ -102,16 +120,19 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
 {
     constexpr int NMB = 4, NNB = BN / 16, NBUF = 4, BSTAGES = 4, NA = 8, NCB = BN / 32, NCOPY = NA + NCB;
     using S = MxW4Sched<NNB, NCOPY>;
-    constexpr int PD = S::kPD, kScales = NMB + NNB;
+    constexpr bool FP4 = FMT_A == 4;
+    static_assert((FMT_A == 4) == (FMT_B == 4), "fp4 with fp4");
+    // steps that the 16 scale bytes of a row last, and rows loaded in each of them
+    constexpr int PD = S::kPD, kScales = NMB + NNB, kGroupSteps = FP4 ? 2 : 4, kScaleLoads = (kScales + kGroupSteps - 1) / kGroupSteps;
     constexpr uint32_t kStepBytes = 128, kBBytes = kStepBytes * BN, kASlot = 64 * kStepBytes, kABase = BSTAGES * kBBytes;
-    static_assert(BN % 32 == 0 && kABase + 8 * kASlot <= 160 * 1024 && kScales <= 4 * S::kScaleLoads, "tile width");
+    static_assert(BN % 32 == 0 && kABase + 8 * kASlot <= 160 * 1024, "tile width");
     using std::integral_constant;
 
     const int wave = hw::wave();
     const uint32_t lane = (uint32_t)hw::lane();
     const uint32_t ldsBase = (uint32_t)(uintptr_t)hw::lds_base();
-    const int64_t ld = k; // bytes between rows of A and between columns of B
-    const int kLoop = k / 128, groups = kLoop / 4;
+    const int64_t ld = FP4 ? k / 2 : k; // bytes between rows of A and between columns of B
+    const int kLoop = (int)(ld / 128), groups = kLoop / 4, scaleGroups = kLoop / kGroupSteps;
     const char *aWave = reinterpret_cast<const char *>(src0) + ((int64_t)row0 + 64 * wave) * ld;
     const char *bPanel = reinterpret_cast<const char *>(src1) + (int64_t)col0 * ld;
     auto chunkOf = [](uint32_t q) { return q; };
@@ -142,7 +163,7 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     for (int t = 0; t < NCB; ++t)
         bBase[t] = detail::uniform_ptr(bPanel + (int64_t)(32 * t) * ld);
     // scales: scale row i < NMB is block row i of this wave (row 16 i + lane % 16), i >= NMB block column i - NMB of the tile;
-    // 16 bytes per four steps, k / 32 bytes between rows
+    // 16 bytes per kGroupSteps steps, k / 32 bytes between rows
     const int64_t ldScale = k / 32;
     const char *saWave = detail::uniform_ptr(reinterpret_cast<const char *>(scale0) + ((int64_t)row0 + 64 * wave) * ldScale);
     const char *sbPanel = detail::uniform_ptr(reinterpret_cast<const char *>(scale1) + (int64_t)col0 * ldScale);
@@ -170,7 +191,7 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     };
     Pair aF[2][NMB], bF[NBUF];
     uint32_t sc[kScales], scNext[kScales]; // scales of the current four steps and of the next four
-    u32x4 raw[S::kScaleLoads];
+    u32x4 raw[kScaleLoads];
     auto readA = [&](auto setTag, auto qTag) __attribute__((always_inline)) {
         constexpr int set = decltype(setTag)::value, q = decltype(qTag)::value, mb = q / 2, kk = q % 2;
         aF[set][mb].h[kk] = W4LdsRead16<mb * 2048>(aAddr[kk][set]);
@@ -225,15 +246,17 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     // of the next group are loaded at the start of the step and picked apart behind its barrier.
     auto step = [&](auto jTag, int it, int group) __attribute__((always_inline)) {
         constexpr int j = decltype(jTag)::value, s = j, par = j % 2, sNext = (j + 1) % BSTAGES, sCopy = (j + 2) % BSTAGES;
-        constexpr int nLoads = (kScales - 4 * j) < 0 ? 0 : ((kScales - 4 * j) < S::kScaleLoads ? (kScales - 4 * j) : S::kScaleLoads);
+        constexpr int jj = j % kGroupSteps, left = kScales - kScaleLoads * jj;
+        constexpr int nLoads = left < 0 ? 0 : (left < kScaleLoads ? left : kScaleLoads);
         const uint32_t kOff = (uint32_t)clampStep(it + 2) * kStepBytes;
-        const int nextGroup = group + 1 < groups ? group + 1 : groups - 1;
+        const int scaleGroup = group * (4 / kGroupSteps) + j / kGroupSteps;
+        const int nextGroup = scaleGroup + 1 < scaleGroups ? scaleGroup + 1 : scaleGroups - 1;
         W4For<0, S::kSlots>([&](auto idxTag) __attribute__((always_inline)) {
             constexpr int idx = decltype(idxTag)::value, nb = idx / NMB, mb = idx % NMB;
             if constexpr (idx == 0) { // (older than every copy of this step)
                 W4For<0, nLoads>([&](auto uTag) __attribute__((always_inline)) {
                     constexpr int u = decltype(uTag)::value;
-                    raw[u] = scaleLoad(integral_constant<int, 4 * j + u>(), nextGroup);
+                    raw[u] = scaleLoad(integral_constant<int, kScaleLoads * jj + u>(), nextGroup);
                 });
             }
             if constexpr (idx == 1) {
@@ -249,7 +272,7 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
                 W4For<0, nLoads>([&](auto uTag) __attribute__((always_inline)) {
                     constexpr int u = decltype(uTag)::value;
                     MxW4Pin(raw[u]); // (not before the wait above)
-                    scNext[4 * j + u] = scalePick(raw[u]);
+                    scNext[kScaleLoads * jj + u] = scalePick(raw[u]);
                 });
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -283,9 +306,21 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
                 constexpr int lo = 4 * (nb - PD) + 1;
                 asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(2 * (PD - 1) + 1 + (lo > 0 ? S::aReadsIn(lo, idx) : 0)) : "memory");
             }
-            MxW4Mfma<mb * NNB + nb, j, FMT_B, FMT_A>(operand(bF[nb % NBUF]), operand(aF[par][mb]), sc[NMB + nb], sc[mb]);
+            if constexpr (FP4) {
+                MxW4MfmaFp4<mb * NNB + nb, 2 * jj>(__builtin_bit_cast(u32x4, bF[nb % NBUF].h[0]), __builtin_bit_cast(u32x4, aF[par][mb].h[0]),
+                                                   sc[NMB + nb], sc[mb]);
+                MxW4MfmaFp4<mb * NNB + nb, 2 * jj + 1>(__builtin_bit_cast(u32x4, bF[nb % NBUF].h[1]),
+                                                       __builtin_bit_cast(u32x4, aF[par][mb].h[1]), sc[NMB + nb], sc[mb]);
+            } else {
+                MxW4Mfma<mb * NNB + nb, j, FMT_B, FMT_A>(operand(bF[nb % NBUF]), operand(aF[par][mb]), sc[NMB + nb], sc[mb]);
+            }
             __builtin_amdgcn_sched_barrier(0);
         });
+        if constexpr (jj == kGroupSteps - 1) { // the next steps multiply with the scales loaded during this group
+#pragma unroll
+            for (int i = 0; i < kScales; ++i)
+                sc[i] = scNext[i];
+        }
     };
     for (int group = 0; group < groups; ++group) {
         const int it = 4 * group;
@@ -293,9 +328,6 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
         step(integral_constant<int, 1>(), it + 1, group);
         step(integral_constant<int, 2>(), it + 2, group);
         step(integral_constant<int, 3>(), it + 3, group);
-#pragma unroll
-        for (int i = 0; i < kScales; ++i)
-            sc[i] = scNext[i];
     }
     hw::wait_vm0(); // the copies issued past the end of K
     // the last MFMAs have written their accumulators
@@ -350,7 +382,7 @@ template <int FMT_A, int FMT_B, typename OutT, int BN>
 int launch_gemm_mxw4(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *sa, const uint8_t *sb, int m, int n, int k)
 {
     // (n % 4: a lane stores four consecutive elements of a row, 16 or 8 bytes, at once)
-    if (m < 256 || n < BN || n % 4 || k % 512 || k < 512)
+    if (m < 256 || n < BN || n % 4 || k % (FMT_A == 4 ? 1024 : 512) || k <= 0)
         return PTO_ERR_UNSUPPORTED;
     constexpr int lds = 4 * 128 * BN + 4 * 2 * 64 * 128; // four B stages + two A slots per wave
     auto kernel = GemmMxW4<FMT_A, FMT_B, OutT, BN, 4>;

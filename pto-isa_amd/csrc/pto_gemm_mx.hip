@@ -347,6 +347,30 @@ int gemm_mx_dispatch(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b
 
 } // namespace
 
+namespace {
+// Two kernels: 256 x 256 tiles on eight wavefronts (this file; quarter tiles in a last partial round) and 256 x 192 /
+// 256 x 128 tiles on four wavefronts (pto_gemm_mxw4.hip: the faster engine, the smaller tile).  Estimated times in
+// microseconds, rounds over the compute units x (K-steps of 128 bytes x step time + fixed time) as measured at 4096^3,
+// 6144^3 and 8192^3.  fp8: 6144^3 is 2.25 rounds of 256 x 256 and 3 of 256 x 192 (2335 against 2610 TFLOP/s), 8192^3 is 4
+// whole rounds of 256 x 256 (2600 against 2440).  fp4: 6144^3 3330 against 3470, 8192^3 3780 against 3280, m, k, n = 2040,
+// 8192, 8100 (one round of 256 x 256) 3430 against 3000.
+bool mx_four_wave_is_faster(int m, int n, int k, int k_bytes, bool fp4)
+{
+    if (m < 256 || n < 128 || n % 4 != 0 || k % (fp4 ? 1024 : 512) != 0)
+        return false;
+    const int cus = compute_units(), steps = k_bytes / 128;
+    const double t4 = std::min(pto_amd::mx_w4_time(m, n, k_bytes, 192, fp4), pto_amd::mx_w4_time(m, n, k_bytes, 128, fp4));
+    double t8 = 1e30;
+    if (n >= 256) {
+        const double step = fp4 ? 1.77 : 1.4, quarter = fp4 ? 0.43 : 0.34;
+        const long long tiles = (long long)((m + 255) / 256) * ((n + 255) / 256), full = tiles / cus, rest = tiles - full * cus;
+        const bool quarters = rest > 0 && full > 0 && rest * 4 <= cus && m % 256 == 0 && n % 256 == 0;
+        t8 = (double)full * (steps * step + 16.0) + (rest == 0 ? 0.0 : (quarters ? steps * quarter + 16.0 : steps * step + 16.0));
+    }
+    return t4 < t8;
+}
+} // namespace
+
 extern "C" int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a,
                               const uint8_t *scale_b, int m, int n, int k, int format, int c_fp32)
 {
@@ -354,23 +378,8 @@ extern "C" int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uin
         return PTO_ERR_BAD_ARG;
     if (format < 0 || format > 3)
         return PTO_ERR_UNSUPPORTED;
-    // Two kernels: 256 x 256 tiles on eight wavefronts (this file; quarter tiles in a last partial round) and 256 x 192 /
-    // 256 x 128 tiles on four wavefronts (pto_gemm_mxw4.hip: the faster engine, the smaller tile).  Estimated times in
-    // microseconds, rounds over the compute units x (K-steps of 128 x step time + fixed time) as measured at 4096^3,
-    // 6144^3 and 8192^3: 6144^3 is 2.25 rounds of 256 x 256 and 3 of 256 x 192 (2335 against 2610 TFLOP/s), 8192^3 is 4
-    // whole rounds of 256 x 256 (2600 against 2440).
-    if (m >= 256 && n >= 128 && n % 4 == 0 && k % 512 == 0) {
-        const int cus = compute_units(), steps = k / 128;
-        const double t4 = std::min(pto_amd::mxfp8_w4_time(m, n, k, 192), pto_amd::mxfp8_w4_time(m, n, k, 128));
-        double t8 = 1e30;
-        if (n >= 256) {
-            const long long tiles = (long long)((m + 255) / 256) * ((n + 255) / 256), full = tiles / cus, rest = tiles - full * cus;
-            const bool quarters = rest > 0 && full > 0 && rest * 4 <= cus && m % 256 == 0 && n % 256 == 0;
-            t8 = (double)full * (steps * 1.4 + 16.0) + (rest == 0 ? 0.0 : (quarters ? steps * 0.34 + 16.0 : steps * 1.4 + 16.0));
-        }
-        if (t4 < t8)
-            return pto_amd::gemm_mxfp8_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 0);
-    }
+    if (mx_four_wave_is_faster(m, n, k, k, false))
+        return pto_amd::gemm_mx_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 0);
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, 1);
 }
 
@@ -379,6 +388,8 @@ extern "C" int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uin
 {
     if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0)
         return PTO_ERR_BAD_ARG;
+    if (mx_four_wave_is_faster(m, n, k, k / 2, true))
+        return pto_amd::gemm_mx_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, 4, c_fp32, 0);
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, 4, c_fp32, 1);
 }
 
@@ -391,7 +402,7 @@ extern "C" int pto_gemm_mxfp8_variant(void *stream, void *c, const uint8_t *a, c
     if (!c || !a || !b || !scale_a || !scale_b || m <= 0 || n <= 0 || k <= 0 || variant < 0 || variant > 6)
         return PTO_ERR_BAD_ARG;
     if (variant >= 4) // the four-wave engine: 4 = width by rounds, 5 = 256 x 192 tiles, 6 = 256 x 128
-        return pto_amd::gemm_mxfp8_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32,
+        return pto_amd::gemm_mx_w4(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32,
                                       variant == 4 ? 0 : (variant == 5 ? 192 : 128));
     return gemm_mx_dispatch(static_cast<hipStream_t>(stream), c, a, b, scale_a, scale_b, m, n, k, format, c_fp32, variant);
 }

@@ -134,6 +134,8 @@ def _mx_variant(a, b, sa, sb, fmt, variant, c_fp32=True):
     from gpu_util import to_dev
     lib = capi.load_st()
     (m, k), n = a.shape, b.shape[0]
+    if fmt == 4:
+        k *= 2      # two e2m1 per byte
     ta, tb, tsa, tsb = (to_dev(x) for x in (a, b, sa, sb))
     tc = torch.full((m, n), float("nan"), dtype=torch.float32, device="cuda:0") if c_fp32 else \
         torch.full((m, n), -1, dtype=torch.int16, device="cuda:0")
@@ -188,6 +190,38 @@ def test_mx_gemm_four_wave_kernel_scale_of_every_block(oracle):
     assert np.array_equal(want, oracle.mx_gemm(a, b, sa, sb, 0).astype(np.float64))
 
 
+@pytest.mark.parametrize("variant", [5, 6])
+@pytest.mark.parametrize("m,n,k", [(256, 192, 1024), (256, 512, 2048), (512, 384, 3072), (300, 260, 1024), (1000, 1100, 2048)])
+def test_mxfp4_gemm_four_wave_kernel(oracle, m, n, k, variant):
+    """The four-wave kernel with e2m1 operands (two matrix instructions per 16 x 16 block and K-step of 256 k, the 16 scale
+    bytes of a row last two steps): the generator's integers exactly, every encoding with a wide range of scales to the GEMM
+    tolerance, the bf16 result = RNE of the fp32 one."""
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 4)
+    rc, got = _mx_variant(a, b, sa, sb, 4, variant)
+    capi.check(rc, "four-wave MX kernel, fp4")
+    assert np.array_equal(got, oracle.mx_gemm(a, b, sa, sb, 4))
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 4, dist="bytes", scale_lo=110, scale_hi=140)
+    rc, got = _mx_variant(a, b, sa, sb, 4, variant)
+    assert rc == 0 and np.all(np.isfinite(got)) and rel_err(got, oracle.mx_gemm(a, b, sa, sb, 4)) <= TOL
+    rc, got16 = _mx_variant(a, b, sa, sb, 4, variant, c_fp32=False)
+    assert rc == 0 and np.array_equal(got16, bf16_rne(got))
+
+
+def test_mxfp4_gemm_four_wave_kernel_scale_of_every_block(oracle):
+    """As for fp8: operands of ones, scales drawn per block, C[i, j] = 32 sum_b 2^(sa[i, b] + sb[j, b] - 254) exactly."""
+    m, n, k = 512, 384, 4096
+    rng = np.random.default_rng(78)
+    ones = datagen.fp4_pack(np.full((1, k), datagen.fp8_encode(np.ones(1), 4)[0], dtype=np.uint8))
+    a, b = np.repeat(ones, m, axis=0), np.repeat(ones, n, axis=0)
+    sa = rng.integers(125, 131, size=(m, k // 32)).astype(np.uint8)
+    sb = rng.integers(125, 131, size=(n, k // 32)).astype(np.uint8)
+    want = 32.0 * (np.exp2(sa.astype(np.float64) - 127) @ np.exp2(sb.astype(np.float64) - 127).T)
+    for variant in (5, 6):
+        rc, got = _mx_variant(a, b, sa, sb, 4, variant)
+        assert rc == 0 and np.array_equal(got.astype(np.float64), want), variant
+    assert np.array_equal(want, oracle.mx_gemm(a, b, sa, sb, 4).astype(np.float64))
+
+
 def test_mx_gemm_four_wave_kernel_refuses():
     import torch
     p = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda:0").data_ptr()
@@ -196,6 +230,7 @@ def test_mx_gemm_four_wave_kernel_refuses():
     assert fn(0, p, p, p, p, p, 256, 160, 512, 0, 1, 5) == capi.ERR_UNSUPPORTED     # narrower than the tile
     assert fn(0, p, p, p, p, p, 256, 258, 512, 0, 1, 6) == capi.ERR_UNSUPPORTED     # rows of C not a multiple of four elements
     assert fn(0, p, p, p, p, p, 256, 256, 640, 0, 1, 6) == capi.ERR_UNSUPPORTED     # k not whole groups of four steps
+    assert fn(0, p, p, p, p, p, 256, 256, 1536, 4, 1, 6) == capi.ERR_UNSUPPORTED    # the same for fp4 (a step is 256 k)
 
 
 def test_mxfp4_gemm_reference_config_2040_8192_8100(oracle):
