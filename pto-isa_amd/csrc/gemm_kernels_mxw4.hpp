@@ -4,16 +4,21 @@
 //   * one v_mfma_scale_f32_16x16x128_f8f6f4 (8 passes) per 16 x 16 block and step instead of two v_mfma_f32_16x16x32_f16
 //     (4 passes each).  Its operand registers hold, for lane group g = lane / 16, bytes 16 g .. + 15 of the row's first 64
 //     k and bytes 64 + 16 g .. + 15 of its second 64 k: exactly the two reads of the fp16 kernel;
-//   * the block scales (one e8m0 byte per row and 32 k = per lane and MFMA exactly one byte): a lane loads the 16 scale
-//     bytes of its row for four K-steps (512 k) straight from memory, once per four steps and block row / column, picks
-//     byte 4 j + g for j = 0 .. 3 with three byte permutes, and the MFMA of step j selects byte j of that register
-//     (op_sel).  Loads at the start of a step, permutes behind the step's barrier, into the set of the next four steps;
+//   * the block scales (one e8m0 byte per row and 32 k = per lane and MFMA exactly one byte).  The MFMAs of four steps
+//     (512 k = 16 scale bytes of a row) take theirs from one register per block row / column: byte j = the scale of the
+//     lane's k block g in step j (op_sel selects j).  These registers are made for 16 steps (64 scale bytes of a row) at
+//     once: lane group g loads bytes 16 g .. + 15 of the 64 straight from memory (one instruction and one cache line per
+//     row for 16 steps), transposes its 4 x 4 bytes (register u = byte u of each k-block quadruple: what lane group u
+//     needs) and the four lane groups exchange register u of group g with register g of group u (two
+//     v_permlane32_swap, two v_permlane16_swap).  One block row / column per step: load at the start of the step,
+//     permutes and swaps behind its barrier, into the set of the next 16 steps;
 //   * four B stages (96 + 64 KiB = the whole LDS at BN = 192), which makes the step's second barrier unnecessary: a
 //     stage is overwritten two steps after its last read, with the barrier of the step in between.
 // Steps come in groups of four (B stage, A slot and scale byte repeat): k % 512 == 0.
 // MXFP4 (format 4, two e2m1 per byte): a K-step of 128 bytes is 256 k = two MFMAs (4 passes each, 16-byte operands: lane group
-// g holds bytes 16 g .. + 15 of the MFMA's 64) and eight scale blocks per row, so the 16 scale bytes of a row last two steps
-// and the MFMA of step j % 2 and half kk selects byte 2 (j % 2) + kk of the picked register: k % 1024 == 0.
+// g holds bytes 16 g .. + 15 of the MFMA's 64) and eight scale blocks per row, so a scale register lasts two steps (the MFMA of
+// step j % 2 and half kk selects byte 2 (j % 2) + kk), the 64 scale bytes of a row eight steps, and two block rows / columns
+// are loaded per step: k % 1024 == 0.
 #pragma once
 #include "gemm_kernels_w4.hpp"
 
@@ -59,6 +64,41 @@ PTO_DEV u32x4 MxW4Load16(const char *base, uint32_t voff)
 // (the compiler does not see that the load above is still on its way: a value is used only behind one of these)
 PTO_DEV void MxW4Pin(u32x4 &x) { asm volatile("" : "+v"(x)); }
 PTO_DEV void MxW4WaitLoads(u32x4 &x) { asm volatile("s_waitcnt vmcnt(0)" : "+v"(x)::"memory"); }
+
+// w = the 16 scale bytes that this lane's group g loaded (bytes 16 g .. + 15 of the 64 of its row) -> out[u] = bytes g, 4 + g,
+// 8 + g, 12 + g of the 16 bytes that group u loaded: the scales of the lane's k block in the four MFMA rounds of quarter u
+// In four parts, each a few instructions between two MFMAs; w is worked on in place and holds out[0 .. 3] after part 3.
+template <int PART>
+PTO_DEV void MxW4ScaleSpreadPart(u32x4 &w)
+{
+    if constexpr (PART == 0) { // bytes transposed within the lane: register u = byte u of w[0], w[1], w[2], w[3], in two rounds
+        const uint32_t t0 = __builtin_amdgcn_perm(w[1], w[0], 0x05010400u), t1 = __builtin_amdgcn_perm(w[1], w[0], 0x07030602u);
+        const uint32_t t2 = __builtin_amdgcn_perm(w[3], w[2], 0x05010400u), t3 = __builtin_amdgcn_perm(w[3], w[2], 0x07030602u);
+        w = u32x4{t0, t1, t2, t3};
+    } else if constexpr (PART == 1) {
+        const uint32_t p0 = __builtin_amdgcn_perm(w[2], w[0], 0x05040100u), p1 = __builtin_amdgcn_perm(w[2], w[0], 0x07060302u);
+        const uint32_t p2 = __builtin_amdgcn_perm(w[3], w[1], 0x05040100u), p3 = __builtin_amdgcn_perm(w[3], w[1], 0x07060302u);
+        w = u32x4{p0, p1, p2, p3};
+    } else if constexpr (PART == 2) { // registers transposed against lane groups: (register u of group g) <-> (register g of group u)
+        const auto a = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false), b = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+        w = u32x4{a[0], b[0], a[1], b[1]};
+    } else {
+        const auto c = __builtin_amdgcn_permlane16_swap(w[0], w[1], false, false), d = __builtin_amdgcn_permlane16_swap(w[2], w[3], false, false);
+        w = u32x4{c[0], c[1], d[0], d[1]};
+    }
+}
+
+PTO_DEV void MxW4ScaleSpread(u32x4 w, uint32_t (&out)[4])
+{
+    MxW4ScaleSpreadPart<0>(w);
+    MxW4ScaleSpreadPart<1>(w);
+    MxW4ScaleSpreadPart<2>(w);
+    MxW4ScaleSpreadPart<3>(w);
+    out[0] = w[0];
+    out[1] = w[1];
+    out[2] = w[2];
+    out[3] = w[3];
+}
 
 // Issue slots of a K-step: slot = 4 nb + mb (nb: 16-column block, outer; mb: 16-row block of the wave's 64 rows).
 template <int NNB, int NCOPY>
@@ -108,6 +148,7 @@ struct MxW4Sched {
         return true;
     }
     static_assert(aReadSlot(7) < kBarrier && copySlot(NCOPY - 1) < kSlots && copySlot(0) >= 2 && distinct(), "order of the step");
+    static_assert(kBarrier + 8 < kSlots, "two scale rows are spread in the slots behind the barrier");
 };
 
 // accumulators = (A .* scales)[row0 .. + 256, :] x (B .* scales)[col0 .. + BN, :]^T over the whole K extent (k elements, four
@@ -122,8 +163,10 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     using S = MxW4Sched<NNB, NCOPY>;
     constexpr bool FP4 = FMT_A == 4;
     static_assert((FMT_A == 4) == (FMT_B == 4), "fp4 with fp4");
-    // steps that the 16 scale bytes of a row last, and rows loaded in each of them
-    constexpr int PD = S::kPD, kScales = NMB + NNB, kGroupSteps = FP4 ? 2 : 4, kScaleLoads = (kScales + kGroupSteps - 1) / kGroupSteps;
+    // steps that a scale register (16 scale bytes of a row) lasts, steps that the 64 bytes loaded at once last, and block rows /
+    // columns loaded in each of these
+    constexpr int PD = S::kPD, kScales = NMB + NNB, kGroupSteps = FP4 ? 2 : 4, kSuperSteps = 4 * kGroupSteps;
+    constexpr int kScaleLoads = (kScales + kSuperSteps - 1) / kSuperSteps;
     constexpr uint32_t kStepBytes = 128, kBBytes = kStepBytes * BN, kASlot = 64 * kStepBytes, kABase = BSTAGES * kBBytes;
     static_assert(BN % 32 == 0 && kABase + 8 * kASlot <= 160 * 1024, "tile width");
     using std::integral_constant;
@@ -132,7 +175,7 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     const uint32_t lane = (uint32_t)hw::lane();
     const uint32_t ldsBase = (uint32_t)(uintptr_t)hw::lds_base();
     const int64_t ld = FP4 ? k / 2 : k; // bytes between rows of A and between columns of B
-    const int kLoop = (int)(ld / 128), groups = kLoop / 4, scaleGroups = kLoop / kGroupSteps;
+    const int kLoop = (int)(ld / 128), supers = (kLoop + kSuperSteps - 1) / kSuperSteps;
     const char *aWave = reinterpret_cast<const char *>(src0) + ((int64_t)row0 + 64 * wave) * ld;
     const char *bPanel = reinterpret_cast<const char *>(src1) + (int64_t)col0 * ld;
     auto chunkOf = [](uint32_t q) { return q; };
@@ -163,20 +206,17 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     for (int t = 0; t < NCB; ++t)
         bBase[t] = detail::uniform_ptr(bPanel + (int64_t)(32 * t) * ld);
     // scales: scale row i < NMB is block row i of this wave (row 16 i + lane % 16), i >= NMB block column i - NMB of the tile;
-    // 16 bytes per kGroupSteps steps, k / 32 bytes between rows
-    const int64_t ldScale = k / 32;
+    // k / 32 bytes between rows, 64 bytes per kSuperSteps steps of which lane group g loads bytes 16 g .. + 15 (the last 16 of
+    // the row where that is past its end: scales of steps beyond K)
+    const uint32_t ldScale = (uint32_t)(k / 32);
     const char *saWave = detail::uniform_ptr(reinterpret_cast<const char *>(scale0) + ((int64_t)row0 + 64 * wave) * ldScale);
     const char *sbPanel = detail::uniform_ptr(reinterpret_cast<const char *>(scale1) + (int64_t)col0 * ldScale);
-    const uint32_t scaleRowOff = (lane % 16) * (uint32_t)ldScale;
-    const uint32_t pick01 = (lane / 16) | ((4u + lane / 16) << 8); // bytes g of the first and of the second source register
-    auto scaleLoad = [&](auto iTag, int group) __attribute__((always_inline)) {
+    const uint32_t scaleRowOff = (lane % 16) * ldScale;
+    auto scaleLoad = [&](auto iTag, int super) __attribute__((always_inline)) {
         constexpr int i = decltype(iTag)::value;
-        const uint32_t voff = scaleRowOff + (uint32_t)((i < NMB ? i : i - NMB) * 16) * (uint32_t)ldScale + (uint32_t)group * 16u;
+        const uint32_t chunk = (uint32_t)super * 64u + (lane / 16) * 16u;
+        const uint32_t voff = scaleRowOff + (uint32_t)((i < NMB ? i : i - NMB) * 16) * ldScale + (chunk < ldScale - 16u ? chunk : ldScale - 16u);
         return MxW4Load16(i < NMB ? saWave : sbPanel, voff);
-    };
-    auto scalePick = [&](u32x4 raw) { // bytes g, 4 + g, 8 + g, 12 + g of the 16: the lane's k block in steps 0 .. 3
-        const uint32_t lo = __builtin_amdgcn_perm(raw[1], raw[0], pick01), hi = __builtin_amdgcn_perm(raw[3], raw[2], pick01);
-        return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
     };
 
     uint32_t voffA[2], voffB;
@@ -190,7 +230,7 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
         f16x8 h[2];
     };
     Pair aF[2][NMB], bF[NBUF];
-    uint32_t sc[kScales], scNext[kScales]; // scales of the current four steps and of the next four
+    uint32_t sc[kScales][4], scNext[kScales][4] = {}; // scales of the current kSuperSteps steps and of the next, a register per quarter
     u32x4 raw[kScaleLoads];
     auto readA = [&](auto setTag, auto qTag) __attribute__((always_inline)) {
         constexpr int set = decltype(setTag)::value, q = decltype(qTag)::value, mb = q / 2, kk = q % 2;
@@ -232,7 +272,7 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
     W4For<0, kScales>([&](auto iTag) __attribute__((always_inline)) {
         constexpr int i = decltype(iTag)::value;
         MxW4Pin(first[i]); // (older than the copies waited for above)
-        sc[i] = scalePick(first[i]);
+        MxW4ScaleSpread(first[i], sc[i]);
     });
     __builtin_amdgcn_sched_barrier(0);
     W4For<0, NA>([&](auto qTag) __attribute__((always_inline)) { readA(integral_constant<int, 0>(), qTag); });
@@ -241,22 +281,22 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
         readB(integral_constant<int, 0>(), integral_constant<int, f / 2>(), integral_constant<int, f % 2>());
     });
 
-    // ---- K-step `it`, number j = it % 4 of its group: B stage j, A register set and LDS slot j % 2, scale byte j.  The
-    // copies of A of step it + 2 go to this step's A slot, those of B to the stage of step it - 2; scale rows 4 j .. 4 j + 3
-    // of the next group are loaded at the start of the step and picked apart behind its barrier.
-    auto step = [&](auto jTag, int it, int group) __attribute__((always_inline)) {
-        constexpr int j = decltype(jTag)::value, s = j, par = j % 2, sNext = (j + 1) % BSTAGES, sCopy = (j + 2) % BSTAGES;
-        constexpr int jj = j % kGroupSteps, left = kScales - kScaleLoads * jj;
+    // ---- K-step `it`, number t = it % kSuperSteps of its scale period: B stage t % 4, A register set and LDS slot t % 2, scale
+    // register t / kGroupSteps, byte t % kGroupSteps (fp4: two bytes).  The copies of A of step it + 2 go to this step's A slot,
+    // those of B to the stage of step it - 2; scale rows kScaleLoads t .. of the next period are loaded at the start of the step
+    // and spread over the lane groups behind its barrier.
+    auto step = [&](auto tTag, int it, int super) __attribute__((always_inline)) {
+        constexpr int t = decltype(tTag)::value, j = t % 4, s = j, par = j % 2, sNext = (j + 1) % BSTAGES, sCopy = (j + 2) % BSTAGES;
+        constexpr int quarter = t / kGroupSteps, jj = t % kGroupSteps, left = kScales - kScaleLoads * t;
         constexpr int nLoads = left < 0 ? 0 : (left < kScaleLoads ? left : kScaleLoads);
         const uint32_t kOff = (uint32_t)clampStep(it + 2) * kStepBytes;
-        const int scaleGroup = group * (4 / kGroupSteps) + j / kGroupSteps;
-        const int nextGroup = scaleGroup + 1 < scaleGroups ? scaleGroup + 1 : scaleGroups - 1;
+        const int nextSuper = super + 1 < supers ? super + 1 : supers - 1;
         W4For<0, S::kSlots>([&](auto idxTag) __attribute__((always_inline)) {
             constexpr int idx = decltype(idxTag)::value, nb = idx / NMB, mb = idx % NMB;
             if constexpr (idx == 0) { // (older than every copy of this step)
                 W4For<0, nLoads>([&](auto uTag) __attribute__((always_inline)) {
                     constexpr int u = decltype(uTag)::value;
-                    raw[u] = scaleLoad(integral_constant<int, kScaleLoads * jj + u>(), nextGroup);
+                    raw[u] = scaleLoad(integral_constant<int, kScaleLoads * t + u>(), nextSuper);
                 });
             }
             if constexpr (idx == 1) {
@@ -269,12 +309,18 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
                 hw::wait_vm<S::copiesBefore(S::kBarrier)>();
                 __builtin_amdgcn_s_barrier();
                 __builtin_amdgcn_sched_barrier(0);
-                W4For<0, nLoads>([&](auto uTag) __attribute__((always_inline)) {
-                    constexpr int u = decltype(uTag)::value;
+            }
+            if constexpr (idx > S::kBarrier && idx <= S::kBarrier + 4 * nLoads) { // a part of the spreading of a loaded scale row
+                constexpr int u = (idx - S::kBarrier - 1) / 4, part = (idx - S::kBarrier - 1) % 4;
+                if constexpr (part == 0)
                     MxW4Pin(raw[u]); // (not before the wait above)
-                    scNext[kScaleLoads * jj + u] = scalePick(raw[u]);
-                });
-                __builtin_amdgcn_sched_barrier(0);
+                MxW4ScaleSpreadPart<part>(raw[u]);
+                if constexpr (part == 3) {
+                    scNext[kScaleLoads * t + u][0] = raw[u][0];
+                    scNext[kScaleLoads * t + u][1] = raw[u][1];
+                    scNext[kScaleLoads * t + u][2] = raw[u][2];
+                    scNext[kScaleLoads * t + u][3] = raw[u][3];
+                }
             }
             if constexpr (mb < 2) { // half mb of the B operand of block column nb + PD
                 constexpr int g = nb + PD;
@@ -308,26 +354,32 @@ AICORE inline __attribute__((always_inline)) void MxW4TileCompute(__gm__ const u
             }
             if constexpr (FP4) {
                 MxW4MfmaFp4<mb * NNB + nb, 2 * jj>(__builtin_bit_cast(u32x4, bF[nb % NBUF].h[0]), __builtin_bit_cast(u32x4, aF[par][mb].h[0]),
-                                                   sc[NMB + nb], sc[mb]);
+                                                   sc[NMB + nb][quarter], sc[mb][quarter]);
                 MxW4MfmaFp4<mb * NNB + nb, 2 * jj + 1>(__builtin_bit_cast(u32x4, bF[nb % NBUF].h[1]),
-                                                       __builtin_bit_cast(u32x4, aF[par][mb].h[1]), sc[NMB + nb], sc[mb]);
+                                                       __builtin_bit_cast(u32x4, aF[par][mb].h[1]), sc[NMB + nb][quarter], sc[mb][quarter]);
             } else {
-                MxW4Mfma<mb * NNB + nb, j, FMT_B, FMT_A>(operand(bF[nb % NBUF]), operand(aF[par][mb]), sc[NMB + nb], sc[mb]);
+                MxW4Mfma<mb * NNB + nb, jj, FMT_B, FMT_A>(operand(bF[nb % NBUF]), operand(aF[par][mb]), sc[NMB + nb][quarter],
+                                                          sc[mb][quarter]);
             }
             __builtin_amdgcn_sched_barrier(0);
         });
-        if constexpr (jj == kGroupSteps - 1) { // the next steps multiply with the scales loaded during this group
-#pragma unroll
-            for (int i = 0; i < kScales; ++i)
-                sc[i] = scNext[i];
-        }
     };
-    for (int group = 0; group < groups; ++group) {
-        const int it = 4 * group;
-        step(integral_constant<int, 0>(), it, group);
-        step(integral_constant<int, 1>(), it + 1, group);
-        step(integral_constant<int, 2>(), it + 2, group);
-        step(integral_constant<int, 3>(), it + 3, group);
+    for (int super = 0; super < supers; ++super) {
+        const int it0 = super * kSuperSteps;
+        W4For<0, kSuperSteps / 4>([&](auto qTag) __attribute__((always_inline)) {
+            constexpr int q = decltype(qTag)::value;
+            if (it0 + 4 * q < kLoop) { // (K is whole groups of four steps, not whole scale periods)
+                step(integral_constant<int, 4 * q>(), it0 + 4 * q, super);
+                step(integral_constant<int, 4 * q + 1>(), it0 + 4 * q + 1, super);
+                step(integral_constant<int, 4 * q + 2>(), it0 + 4 * q + 2, super);
+                step(integral_constant<int, 4 * q + 3>(), it0 + 4 * q + 3, super);
+            }
+        });
+#pragma unroll
+        for (int i = 0; i < kScales; ++i)
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                sc[i][u] = scNext[i][u];
     }
     hw::wait_vm0(); // the copies issued past the end of K
     // the last MFMAs have written their accumulators

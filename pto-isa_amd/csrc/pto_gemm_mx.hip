@@ -350,10 +350,10 @@ int gemm_mx_dispatch(hipStream_t st, void *c, const uint8_t *a, const uint8_t *b
 namespace {
 // Two kernels: 256 x 256 tiles on eight wavefronts (this file; quarter tiles in a last partial round) and 256 x 192 /
 // 256 x 128 tiles on four wavefronts (pto_gemm_mxw4.hip: the faster engine, the smaller tile).  Estimated times in
-// microseconds, rounds over the compute units x (K-steps of 128 bytes x step time + fixed time) as measured at 4096^3,
-// 6144^3 and 8192^3.  fp8: 6144^3 is 2.25 rounds of 256 x 256 and 3 of 256 x 192 (2335 against 2610 TFLOP/s), 8192^3 is 4
-// whole rounds of 256 x 256 (2600 against 2440).  fp4: 6144^3 3330 against 3470, 8192^3 3780 against 3280, m, k, n = 2040,
-// 8192, 8100 (one round of 256 x 256) 3430 against 3000.
+// microseconds, rounds over the compute units x (K-steps of 128 bytes x step time + fixed time) as measured in one run at
+// 4096^3, 6144^3 and 8192^3 (eight against four wavefronts).  fp8: 6144^3 2240 against 2590 TFLOP/s, 8192^3 2460 against
+// 2545, 4096^3 2150 against 2165.  fp4: 6144^3 3600 against 4020, 8192^3 4030 against 4090, m, k, n = 2040, 8192, 8100
+// (one round of 256 x 256) 3680 against 3910.
 bool mx_four_wave_is_faster(int m, int n, int k, int k_bytes, bool fp4)
 {
     if (m < 256 || n < 128 || n % 4 != 0 || k % (fp4 ? 1024 : 512) != 0)
@@ -362,7 +362,7 @@ bool mx_four_wave_is_faster(int m, int n, int k, int k_bytes, bool fp4)
     const double t4 = std::min(pto_amd::mx_w4_time(m, n, k_bytes, 192, fp4), pto_amd::mx_w4_time(m, n, k_bytes, 128, fp4));
     double t8 = 1e30;
     if (n >= 256) {
-        const double step = fp4 ? 1.77 : 1.4, quarter = fp4 ? 0.43 : 0.34;
+        const double step = fp4 ? 1.63 : 1.5, quarter = fp4 ? 0.25 : 0.34;
         const long long tiles = (long long)((m + 255) / 256) * ((n + 255) / 256), full = tiles / cus, rest = tiles - full * cus;
         const bool quarters = rest > 0 && full > 0 && rest * 4 <= cus && m % 256 == 0 && n % 256 == 0;
         t8 = (double)full * (steps * step + 16.0) + (rest == 0 ? 0.0 : (quarters ? steps * quarter + 16.0 : steps * step + 16.0));

@@ -6,17 +6,18 @@
 
 namespace pto_amd {
 // Estimated time (microseconds) of the four-wave kernel with 256 x width tiles: rounds over the compute units x (K-steps
-// of 128 bytes x step time + fixed time), the times as measured at 4096^3, 6144^3 and 8192^3; a huge value where the width
-// does not fit.  k_bytes: bytes of a row of A (k for fp8, k / 2 for fp4).  The fp4 steps are slower (twice the matrix
-// instructions, of half the length, and twice the scale rows per step: 1.42 / 1.10 us against 0.99 / 0.70).
+// of 128 bytes x step time + fixed time), the times as measured at 4096^3, 6144^3 and 8192^3; a last round that does not
+// fill the chip counts as half a round plus half its share of the compute units (the others finish early and the clock
+// rises).  A huge value where the width does not fit.  k_bytes: bytes of a row of A (k for fp8, k / 2 for fp4).
 double mx_w4_time(int m, int n, int k_bytes, int width, bool fp4)
 {
     if (m < 256 || n < width || (width != 192 && width != 128))
         return 1e30;
     const int cus = compute_units();
-    const long long tiles = (long long)((m + 255) / 256) * ((n + width - 1) / width), rounds = (tiles + cus - 1) / cus;
-    const double step = width == 192 ? (fp4 ? 1.42 : 0.99) : (fp4 ? 1.10 : 0.70);
-    return (double)rounds * ((k_bytes / 128) * step + (width == 192 ? 11.5 : 9.0));
+    const long long tiles = (long long)((m + 255) / 256) * ((n + width - 1) / width), full = tiles / cus, rest = tiles - full * cus;
+    const double rounds = (double)full + (rest ? 0.5 + 0.5 * (double)rest / cus : 0.0);
+    const double step = width == 192 ? (fp4 ? 1.16 : 1.0) : 0.78, fixed = width == 192 ? 11.0 : (fp4 ? 8.7 : 6.0);
+    return rounds * ((k_bytes / 128) * step + fixed);
 }
 
 // format: 0 = e4m3 x e4m3, 1 = e5m2 x e5m2, 2 = A e4m3 x B e5m2, 3 = A e5m2 x B e4m3, 4 = e2m1 x e2m1 (k then counts 4-bit
