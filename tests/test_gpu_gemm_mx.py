@@ -222,6 +222,16 @@ def test_mxfp4_gemm_four_wave_kernel_scale_of_every_block(oracle):
     assert np.array_equal(want, oracle.mx_gemm(a, b, sa, sb, 4).astype(np.float64))
 
 
+@pytest.mark.parametrize("fmt", [0, 4])
+def test_mx_gemm_public_entry_narrow_n_and_kernel_choice(oracle, fmt):
+    """128 <= n < 256 (four-wave kernel only) and shapes on either side of the entry points' choice between the kernels:
+    the same exact result on integer data whichever runs."""
+    from gpu_util import gemm_mx
+    for m, n, k in ((256, 160, 1024), (512, 252, 2048), (1024, 1024, 1024), (2048, 3072, 1024), (512, 258, 1024)):
+        a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt, dist="integer")
+        assert np.array_equal(gemm_mx(a, b, sa, sb, fmt), oracle.mx_gemm(a, b, sa, sb, fmt)), (m, n, k)
+
+
 def test_mx_gemm_four_wave_kernel_refuses():
     import torch
     p = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda:0").data_ptr()
