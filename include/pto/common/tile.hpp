@@ -363,6 +363,23 @@ struct Tile {
         Bind(o);
         return *this;
     }
+    // `tile = TileT(validRows, validCols)`: a temporary that no TASSIGN has given an address (and whose registers hold
+    // nothing yet) brings its valid extents only; the tile stays where it is.  (The reference's kernels re-shape their
+    // TASSIGNed tiles this way per block: mxmatmul_performance_kernel.cpp of a5/matmul_mxfp4_performance :297-307.)
+    PTO_HD Tile &operator=(Tile &&o)
+    {
+        RowMaskInternal = o.RowMaskInternal;
+        ColMaskInternal = o.ColMaskInternal;
+        if constexpr (Loc_ == TileType::Mat && !inMemory) {
+            if (o.st.bound)
+                st = o.st;
+        }
+#if defined(PTO_VEC_TILES_IN_MEMORY)
+        if (o.mem_)
+            mem_ = o.mem_;
+#endif
+        return *this;
+    }
 #if defined(PTO_TILE_COPY_WRITEBACK)
     PTO_HD ~Tile()
     {
@@ -501,6 +518,12 @@ template <typename E, int R, int C, int RV = R, int CV = C>
 using TileLeftScale = Tile<TileType::ScaleLeft, E, R, C, BLayout::RowMajor, RV, CV, SLayout::NoneBox>;
 template <typename E, int R, int C, int RV = R, int CV = C>
 using TileRightScale = Tile<TileType::ScaleRight, E, R, C, BLayout::ColMajor, RV, CV, SLayout::NoneBox>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileLeftScaleCompact = Tile<TileType::ScaleLeft, E, R, C, BLayout::RowMajor, RV, CV, SLayout::NoneBox, TileConfig::fractalABSize,
+                                  PadValue::Null, CompactMode::Normal>;
+template <typename E, int R, int C, int RV = R, int CV = C>
+using TileRightScaleCompact = Tile<TileType::ScaleRight, E, R, C, BLayout::ColMajor, RV, CV, SLayout::NoneBox, TileConfig::fractalABSize,
+                                   PadValue::Null, CompactMode::Normal>;
 template <typename E, int R, int C, int RV = R, int CV = C>
 using TileAccCompact = Tile<TileType::Acc, E, R, C, BLayout::ColMajor, RV, CV, SLayout::RowMajor,
                             TileConfig::fractalCSize, PadValue::Null, CompactMode::Normal>;

@@ -312,9 +312,40 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
         }
     } else {
         static_assert(SLICE < 0, "[PTO][SA] TLOAD slice: only for fully valid, unit-stride Mat tiles");
-        static_assert(elem_bits<T> >= 8, "[PTO][SA] TLOAD of 4-bit elements: fully valid, unit-stride Mat tiles only");
-        // general path: element by element, pad outside the valid region (TLoad.hpp:151-152)
         const int vr = dst.GetValidRow(), vc = dst.GetValidCol();
+        if constexpr (staticUnit && TileT::PadVal == PadValue::Null && G::layout != Layout::NZ) {
+            // Run-time valid extents with whole rows of the contiguous dimension (the last row / column block of a matrix
+            // that the tiles do not divide): the same 16-byte copies; rows past the valid ones repeat the last valid row
+            // (memory past it may not exist, and what a tile holds outside its valid region is unspecified).
+            const int vMajor = Geo::colsK ? vr : vc, vMinor = Geo::colsK ? vc : vr;
+            const bool plain2d = src.GetShape(0) * src.GetShape(1) * src.GetShape(2) == 1; // (no stacked outer dimensions)
+            if (plain2d && vMinor == (Geo::colsK ? TileT::Cols : TileT::Rows) && vMajor > 0) {
+                const int64_t ld = (Geo::colsK ? st_r : st_c) * elem_bits<T> / 8;
+                constexpr int total = Geo::Major * Geo::ChunksPerRow, nInst = cdiv(total, kWaveSize);
+                const int lane = hw::lane(), wave = hw::wave();
+#pragma unroll
+                for (int s0 = 0; s0 < nInst; s0 += kBlockWaves) {
+                    const int s = s0 + wave;
+                    const uint32_t q = (uint32_t)(s * kWaveSize + lane);
+                    constexpr bool evenInst = nInst % kBlockWaves == 0, evenTotal = total % kWaveSize == 0;
+                    if ((evenInst || s < nInst) && (evenTotal || q < (uint32_t)total)) {
+                        const uint32_t major = q / Geo::ChunksPerRow, cpos = q % Geo::ChunksPerRow;
+                        const uint32_t chunk = cpos ^ mat_swz<Geo::RowBytes>(major);
+                        const uint32_t from = major < (uint32_t)vMajor ? major : (uint32_t)vMajor - 1u;
+                        const char *g = reinterpret_cast<const char *>(gm) + (int64_t)from * ld + chunk * 16;
+                        __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(g), PTO_LDS_PTR(lds + s * (kWaveSize * 16)), 16, 0, 0);
+                    }
+                }
+                return;
+            }
+        }
+        if constexpr (elem_bits<T> < 8) {
+            // (4-bit elements have no address of their own)
+            if (hw::tid() == 0)
+                printf("[PTO][RT] TLOAD of 4-bit elements into a Mat tile: whole rows of the contiguous dimension only\n");
+            __builtin_amdgcn_endpgm();
+        } else {
+        // general path: element by element, pad outside the valid region (TLoad.hpp:151-152)
         const T pad = pad_value<T>(TileT::PadVal);
         const bool stacked = src.GetShape(0) * src.GetShape(1) * src.GetShape(2) != 1;
         for (int e = hw::tid(); e < TileT::Numel; e += kBlockThreads) {
@@ -323,6 +354,7 @@ PTO_DEV void tload_mat(TileT &dst, G &src)
             if (r < vr && c < vc) // views with stacked outer dimensions and NZ memory: by the 5-D rule; else rows and columns
                 v = (G::layout == Layout::NZ || stacked) ? gm[gm_elem_offset(src, r, c)] : gm[(int64_t)r * st_r + (int64_t)c * st_c];
             *reinterpret_cast<T *>(lds + Geo::elem_off(r, c)) = v;
+        }
         }
     }
 }
@@ -443,19 +475,26 @@ PTO_DEV void tload_scale_mat(TileT &dst, G &src)
 {
     using Geo = ScaleMatGeom<TileT>;
     static_assert(Geo::left ? G::staticStride[4] == 1 : G::staticStride[3] == 1, "[PTO][SA] TLOAD of block scales: k blocks must be contiguous");
-    static_assert(TileT::ValidRow == TileT::Rows && TileT::ValidCol == TileT::Cols, "[PTO][SA] TLOAD of block scales: fully valid tiles");
+    // (run-time valid extents: every k block of the tile, any number of rows / columns; those past the valid ones repeat the
+    // last valid one, as for operand tiles)
+    const int vMajor = Geo::left ? dst.GetValidRow() : dst.GetValidCol();
     char *lds = hw::lds_base() + dst.st.lds;
     const char *gm = reinterpret_cast<const char *>(src.data());
     const int64_t ld = Geo::left ? src.GetStride(3) : src.GetStride(4);
     const int lane = hw::lane(), wave = hw::wave();
-    const uint32_t laneOff = (uint32_t)lane * (uint32_t)ld;
     static_assert(Geo::nInst % kBlockWaves == 0 || Geo::nInst > kBlockWaves, "[PTO][SA] TLOAD: fewer copy instructions than waves");
 #pragma unroll
     for (int s0 = 0; s0 < Geo::nInst; s0 += kBlockWaves) {
         // (waves past the end of an incomplete last round repeat their previous instruction, as for operand tiles)
         const int s = ((Geo::nInst % kBlockWaves != 0 && s0 + wave >= Geo::nInst) ? s0 - kBlockWaves : s0) + wave;
         const int q = s / (Geo::Major / kWaveSize), g = s % (Geo::Major / kWaveSize);
-        const char *p = uniform_ptr(gm + (int64_t)(g * kWaveSize) * ld + 4 * q) + laneOff;
+        const char *p;
+        if constexpr (TileT::ValidRow != TileT::Rows || TileT::ValidCol != TileT::Cols) {
+            const int major = g * kWaveSize + lane;
+            p = gm + (int64_t)(major < vMajor ? major : vMajor - 1) * ld + 4 * q;
+        } else {
+            p = uniform_ptr(gm + (int64_t)(g * kWaveSize) * ld + 4 * q) + (uint32_t)lane * (uint32_t)ld;
+        }
         __builtin_amdgcn_global_load_lds(PTO_GLOBAL_PTR(p), PTO_LDS_PTR(lds + s * (kWaveSize * 4)), 4, 0, 0);
     }
 }

@@ -97,6 +97,10 @@ PORTED = [
     # the MXFP8 matmul kernel (e5m2 operands, e8m0 block scales, bf16 output): one K-128 step per L1 panel instead of four
     ("libpto_ported_mxfp8.so", "kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp",
      [("stepKa", "1"), ("stepKb", "1")], 160 * 1024, dict(extra_flags=("-Wno-unknown-attributes",))),
+    # the MXFP4 matmul kernel (e2m1 operands, m = 2040 and n = 8100 through run-time valid extents of its Mat, operand, scale
+    # and accumulator tiles): one K-256 step per L1 panel instead of two
+    ("libpto_ported_mxfp4.so", "kernels/manual/a5/matmul_mxfp4_performance/mxmatmul_performance_kernel.cpp",
+     [("stepKa", "1"), ("stepKb", "1")], 160 * 1024, dict(extra_flags=("-Wno-unknown-attributes",))),
 ]
 
 

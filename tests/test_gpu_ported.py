@@ -163,3 +163,36 @@ def test_reference_mxfp8_matmul_kernel(oracle):
     rows = np.array([0, 127, 128, 1535, 1536, 3000, 4607, 6143])
     want = oracle.mx_gemm(a[rows], b, sa[rows], sb, 1)
     assert np.abs(got[rows] - want).max() <= 2.0 ** -7 * np.abs(want).max()
+
+
+def test_reference_mxfp4_matmul_kernel(oracle):
+    """mxmatmul_performance_kernel.cpp of a5/matmul_mxfp4_performance (LaunchMxMatmul: m, k, n = 2040, 8192, 8100, e2m1
+    operands two per byte, bf16 output, 32 blocks of 512 x 1024 in 256 x 256 tiles) with stepKa = stepKb = 1.  The last row
+    block has 248 valid rows and the last column block 164 valid columns: every tile of the kernel carries run-time valid
+    extents (`tile = TileT(validRows, validCols)` on TASSIGNed tiles, TLOAD / TEXTRACT / TMATMUL_MX / TSTORE on them).  On
+    the generator's data every sum is exact in fp32, so every element equals the native kernel's bf16 result; nothing is
+    written outside C."""
+    import torch
+    import gpu_util as G
+    from pto_amd import capi, datagen
+    lib = _ported("libpto_ported_mxfp4.so")
+    fn = lib._Z14LaunchMxMatmulPhS_S_S_S_Pv         # void LaunchMxMatmul(uint8_t*, uint8_t*, uint8_t*, uint8_t*, uint8_t*, void*)
+    fn.argtypes, fn.restype = [C.c_void_p] * 6, None
+    m, k, n = 2040, 8192, 8100
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, 4)
+    ta, tb, tsa, tsb = (torch.from_numpy(x).to(G.DEV) for x in (a, b, sa, sb))
+    guard = 4096                                     # elements before and after C that must keep their pattern
+    buf = torch.full((m * n + 2 * guard,), 0x7FC1, dtype=torch.int16, device=G.DEV)
+    tc = buf[guard:guard + m * n].view(m, n)
+    print("ported mxfp4 launch", flush=True)
+    fn(tc.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(), None)
+    torch.cuda.synchronize()
+    got = tc.cpu().numpy().view(np.uint16)
+    edges = torch.cat((buf[:guard], buf[guard + m * n:])).cpu().numpy()
+    assert np.all(edges == 0x7FC1)
+    native = G.gemm_mx(a, b, sa, sb, 4, c_fp32=False)
+    assert np.array_equal(got, native)
+    rows = np.array([0, 255, 256, 511, 512, 1791, 1792, 2039])
+    want = oracle.mx_gemm(a[rows], b, sa[rows], sb, 4)
+    u = np.ascontiguousarray(want, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    assert np.array_equal(got[rows], ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16))    # RNE to bf16

@@ -77,6 +77,46 @@ def test_reference_mxfp8_matmul_kernel_compiles(tmp_path):
     assert rc == 0, err
 
 
+@needs_reference
+def test_reference_mxfp4_matmul_kernel_compiles(tmp_path):
+    """mxmatmul_performance_kernel.cpp of a5/matmul_mxfp4_performance with stepKa = stepKb = 1: e2m1 Mat / Left / Right
+    tiles, TileLeftScaleCompact / TileRightScaleCompact, every tile with run-time valid extents set by assigning a
+    temporary `TileT(validRows, validCols)` to a TASSIGNed tile."""
+    lib, rel_src, sets, lds, opts = [p for p in B.PORTED if p[0] == "libpto_ported_mxfp4.so"][0]
+    rc, err = B.port_and_compile(rel_src, sets, lds, str(tmp_path / "mx4.o"), **opts)
+    assert rc == 0, err
+
+
+def test_assigning_a_temporary_tile_keeps_the_address(tmp_path):
+    """`tile = TileT(vr, vc)` on a TASSIGNed Mat tile takes the valid extents and keeps the address (host-side check of the
+    tile object; the reference's MXFP4 kernel re-shapes its tiles this way per block)."""
+    src = tmp_path / "assign.hip"
+    src.write_text("""
+#include <pto/pto-inst.hpp>
+#include <cstdio>
+using namespace pto;
+int main()
+{
+    using T = Tile<TileType::Mat, half, 64, 64, BLayout::ColMajor, -1, -1, SLayout::RowMajor>;
+    T a(64, 64), b(64, 64);
+    a.S().lds = 4096; a.S().bound = true;
+    a = T(17, 33);
+    if (a.GetValidRow() != 17 || a.GetValidCol() != 33 || a.S().lds != 4096u) { std::printf("moved: %u\\n", a.S().lds); return 1; }
+    b.S().lds = 8192; b.S().bound = true;
+    a = b;                      // a named, TASSIGNed tile: the address comes along
+    if (a.S().lds != 8192u) return 2;
+    std::printf("ok\\n");
+    return 0;
+}
+""")
+    exe = tmp_path / "assign"
+    r = subprocess.run([B.HIPCC, "--offload-arch=gfx950", "-std=c++17", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe)],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    r = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert r.returncode == 0 and "ok" in r.stdout, (r.returncode, r.stdout, r.stderr)
+
+
 def test_port_script_rewrites():
     """The mechanical edits on a synthetic source: launch statement, function-local static, kernel prologue, brackets."""
     spec = importlib.util.spec_from_file_location("port_ascend_source", os.path.join(PKG, "port_ascend_source.py"))
