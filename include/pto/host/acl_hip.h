@@ -11,6 +11,49 @@
 typedef hipStream_t aclrtStream;
 typedef int aclError;
 typedef uint16_t aclFloat16; /* fp16 bit pattern on the host, as in the reference's host code */
+/* conversions of the Ascend runtime between that pattern and float (every value of fp16 is a float; to fp16 rounds to nearest even) */
+static inline float aclFloat16ToFloat(aclFloat16 value)
+{
+    const uint32_t sign = (uint32_t)(value & 0x8000u) << 16, exp = (value >> 10) & 0x1Fu, man = value & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0x1Fu) {
+        bits = sign | 0x7F800000u | (man << 13); /* infinity, NaN */
+    } else if (exp != 0) {
+        bits = sign | ((exp + 112u) << 23) | (man << 13);
+    } else if (man == 0) {
+        bits = sign;
+    } else { /* subnormal: man x 2^-24 */
+        uint32_t m = man, e = 113u;
+        while ((m & 0x400u) == 0) {
+            m <<= 1;
+            --e;
+        }
+        bits = sign | (e << 23) | ((m & 0x3FFu) << 13);
+    }
+    float f;
+    __builtin_memcpy(&f, &bits, sizeof f);
+    return f;
+}
+static inline aclFloat16 aclFloatToFloat16(float value)
+{
+    uint32_t x;
+    __builtin_memcpy(&x, &value, sizeof x);
+    const uint32_t sign = (x >> 16) & 0x8000u, mag = x & 0x7FFFFFFFu;
+    if (mag >= 0x7F800000u) /* infinity, NaN */
+        return (aclFloat16)(sign | 0x7C00u | (mag > 0x7F800000u ? 0x200u : 0u));
+    if (mag >= 0x477FF000u) /* rounds to 65520 or more: infinity */
+        return (aclFloat16)(sign | 0x7C00u);
+    if (mag < 0x33000001u) /* at most 2^-25: zero */
+        return (aclFloat16)sign;
+    const int e = (int)(mag >> 23) - 127;
+    const uint32_t man = (mag & 0x7FFFFFu) | 0x800000u;
+    const int shift = e >= -14 ? 13 : 13 + (-14 - e); /* bits dropped below the fp16 mantissa */
+    const uint32_t kept = man >> shift, rest = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    uint32_t r = kept + ((rest > half || (rest == half && (kept & 1u))) ? 1u : 0u);
+    /* normal: implicit bit of `kept` adds one to the exponent field; subnormal: the field starts at 0 and a carry makes it 1 */
+    const uint32_t bits = e >= -14 ? (((uint32_t)(e + 14) << 10) + r) : r;
+    return (aclFloat16)(sign | bits);
+}
 enum { ACL_SUCCESS = 0 };
 typedef enum aclrtMemMallocPolicy {
     ACL_MEM_MALLOC_HUGE_FIRST = 0,

@@ -2,8 +2,12 @@
 // WriteFile :112-150, ResultCmp :211-301), written for this back end's host programs and tests.
 #ifndef PTO_HOST_TEST_COMMON_H
 #define PTO_HOST_TEST_COMMON_H
+#include <cassert>
 #include <cmath>
 #include <cstdio>
+#include <fstream>
+#include <iomanip>
+#include <iostream> // (the reference's host programs count on this header for their stream output)
 #include <string>
 #include <vector>
 

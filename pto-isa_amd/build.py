@@ -142,6 +142,38 @@ def build_ported(verbose=True):
             print("built", out)
 
 
+# The reference's host programs (main.cpp beside each manual kernel: Ascend runtime calls, the file protocol, ResultCmp),
+# compiled where they lie against this library's runtime shim (include/acl/acl.h, include/pto/host/test_common.h) and linked
+# with the ported kernel library that holds their launcher: build/ported/host/<name>.
+PORTED_HOSTS = [
+    ("gemm_performance_main", "kernels/manual/a2a3/gemm_performance/main.cpp", "pto_ported_gemm"),
+    ("matmul_mxfp8_performance_main", "kernels/manual/a5/matmul_mxfp8_performance/main.cpp", "pto_ported_mxfp8"),
+    ("matmul_mxfp4_performance_main", "kernels/manual/a5/matmul_mxfp4_performance/main.cpp", "pto_ported_mxfp4"),
+    ("topk_main", "kernels/manual/a2a3/topk/main.cpp", "pto_ported_topk"),
+    # the flash-attention program takes its case list from generated_cases.h (written by the reference's build from a
+    # case string; here the list the ported kernel library is built with) and runs the cases named with --case=
+    ("flash_atten_main", "kernels/manual/common/flash_atten/main.cpp", "pto_ported_fa"),
+]
+
+
+def build_ported_hosts(verbose=True):
+    if not os.path.isdir(REFERENCE):
+        return
+    out_dir = os.path.join(PORTED_DIR, "host")
+    os.makedirs(out_dir, exist_ok=True)
+    for name, rel_src, lib in PORTED_HOSTS:
+        out = os.path.join(out_dir, name)
+        cmd = ["g++", "-O2", "-std=c++17", "-w", "-I" + os.path.join(ROOT, "include"), "-I" + os.path.join(ROOT, "include", "pto", "host"),
+               "-I/opt/rocm/include", "-I" + os.path.dirname(os.path.join(REFERENCE, rel_src)), "-I" + os.path.join(HERE, "host", "port_cases"),
+               "-D__HIP_PLATFORM_AMD__", os.path.join(REFERENCE, rel_src), "-o", out,
+               "-L" + PORTED_DIR, "-l" + lib, "-Wl,-rpath,$ORIGIN/..", "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError("host program build failed for %s:\n%s" % (rel_src, r.stderr))
+        if verbose:
+            print("built", out)
+
+
 # Per-instruction test kernels of the reference (tests/npu/a2a3/src/st/testcase/<op>/<op>_kernel.cpp) that tests/st_ref_cases.py
 # runs on the GPU: each compiled unchanged (register tiles; no constant rewritten) into build/ported/st/<op>.so.
 # build/ported/st/manifest.json holds, per test, the launcher symbols (mangled -> demangled, so that the tests need no
@@ -258,5 +290,6 @@ def build_ported_st(verbose=True, jobs=8):
 if __name__ == "__main__":
     build()
     build_ported()
+    build_ported_hosts()
     build_ported_st()
     sys.exit(0)

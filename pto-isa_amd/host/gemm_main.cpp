@@ -1,95 +1,71 @@
-// Host program of the GEMM kernel with the reference's file protocol
-// (kernels/manual/a2a3/gemm_performance/main.cpp:17-105): reads <dir>/input/x1_gm.bin (A [m,k] fp16) and
-// <dir>/input/x2_gm.bin (B stored [n,k] fp16), runs the kernel, writes <dir>/output/output_z.bin (C [m,n] fp32) and
-// compares it with <dir>/output/golden.bin (ResultCmp, eps 1e-3).  Prints "test success" or "test failed".
+// GEMM through the C ABI on files in the layout of the reference's gemm_performance example
+// (kernels/manual/a2a3/gemm_performance/main.cpp:42-78; scripts/gen_data.py): <dir>/input/x1_gm.bin = A [m,k] fp16,
+// <dir>/input/x2_gm.bin = B stored [n,k] fp16 -> <dir>/output/output_z.bin = C [m,n] fp32, compared with
+// <dir>/output/golden.bin by the reference's rule (ResultCmp, eps 1e-3).  Prints "test success" or "test failed".
+// (The reference's own main.cpp, compiled where it lies against include/acl/acl.h, is build/ported/host/gemm_performance_main.)
 //
-//   gemm_main [dir [m k n]]        defaults: dir = "..", m = k = n = 6144 (the reference's build)
-#include <cstdint>
-#include <cstdio>
+//   gemm_main [dir [m k n]]        defaults: dir = "..", m = k = n = 6144
 #include <cstdlib>
-#include <string>
-#include <vector>
 
-#include <pto/host/acl_hip.h>
 #include <pto/host/test_common.h>
 
+#include "host_util.hpp"
 #include "pto_amd.h"
 
-using namespace PtoTestCommon;
-
 namespace {
-uint32_t gM = 6144, gK = 6144, gN = 6144;
-int gStatus = PTO_OK;
+struct Problem {
+    std::string dir = "..";
+    int m = 6144, k = 6144, n = 6144;
+};
+
+Problem ParseArgs(int argc, char **argv)
+{
+    Problem p;
+    if (argc > 1)
+        p.dir = argv[1];
+    if (argc > 4) {
+        p.m = std::atoi(argv[2]);
+        p.k = std::atoi(argv[3]);
+        p.n = std::atoi(argv[4]);
+    }
+    return p;
 }
 
-// same name and argument meaning as the reference's launcher (gemm_performance_kernel.cpp:243-264)
-template <typename T>
-void LaunchGEMME2E(uint8_t *out, uint8_t *src0, uint8_t *src1, void *stream)
+// 0: matches the golden file, 1: does not; exceptions: the set-up failed or the kernel refused the shape
+int Run(const Problem &p)
 {
-    gStatus = pto_gemm_f16f32(stream, reinterpret_cast<float *>(out), reinterpret_cast<const uint16_t *>(src0),
-                              reinterpret_cast<const uint16_t *>(src1), (int)gM, (int)gN, (int)gK);
+    using namespace host_util;
+    const size_t elemsC = (size_t)p.m * p.n;
+    DeviceBuffer a(ReadExactly(p.dir + "/input/x1_gm.bin", (size_t)p.m * p.k * sizeof(uint16_t)));
+    DeviceBuffer b(ReadExactly(p.dir + "/input/x2_gm.bin", (size_t)p.n * p.k * sizeof(uint16_t)));
+    DeviceBuffer c(elemsC * sizeof(float));
+    hipStream_t stream;
+    Check(hipStreamCreate(&stream), "hipStreamCreate");
+    const int status = pto_gemm_f16f32(stream, c.as<float>(), a.as<uint16_t>(), b.as<uint16_t>(), p.m, p.n, p.k);
+    Check(hipStreamSynchronize(stream), "hipStreamSynchronize");
+    Check(hipStreamDestroy(stream), "hipStreamDestroy");
+    if (status != PTO_OK)
+        throw std::runtime_error("pto_gemm_f16f32 returned " + std::to_string(status));
+    const std::vector<float> result = c.ToHost<float>();
+    WriteAll(p.dir + "/output/output_z.bin", result.data(), result.size() * sizeof(float));
+    const std::vector<uint8_t> goldenBytes = ReadExactly(p.dir + "/output/golden.bin", elemsC * sizeof(float));
+    const float *golden = reinterpret_cast<const float *>(goldenBytes.data());
+    return PtoTestCommon::ResultCmp(std::vector<float>(golden, golden + elemsC), result, 0.001f) ? 0 : 1;
 }
+} // namespace
 
 int main(int argc, char **argv)
 {
-    const std::string dir = argc > 1 ? argv[1] : "..";
-    if (argc > 4) {
-        gM = (uint32_t)std::atoi(argv[2]);
-        gK = (uint32_t)std::atoi(argv[3]);
-        gN = (uint32_t)std::atoi(argv[4]);
-    }
-    size_t aFileSize = (size_t)gM * gK * sizeof(uint16_t), bFileSize = (size_t)gK * gN * sizeof(uint16_t);
-    size_t cFileSize = (size_t)gM * gN * sizeof(float);
-
-    aclInit(nullptr);
-    aclrtSetDevice(0);
     if (pto_init() != PTO_OK) {
         std::printf("test failed (pto_init: not a gfx950 device)\n");
         return 2;
     }
-    aclrtStream stream;
-    aclrtCreateStream(&stream);
-
-    uint8_t *dstHost, *src0Host, *src1Host, *dstDevice, *src0Device, *src1Device;
-    aclrtMallocHost((void **)(&dstHost), cFileSize);
-    aclrtMallocHost((void **)(&src0Host), aFileSize);
-    aclrtMallocHost((void **)(&src1Host), bFileSize);
-    aclrtMalloc((void **)&dstDevice, cFileSize, ACL_MEM_MALLOC_HUGE_FIRST);
-    aclrtMalloc((void **)&src0Device, aFileSize, ACL_MEM_MALLOC_HUGE_FIRST);
-    aclrtMalloc((void **)&src1Device, bFileSize, ACL_MEM_MALLOC_HUGE_FIRST);
-
-    bool ok = ReadFile(dir + "/input/x1_gm.bin", aFileSize, src0Host, aFileSize);
-    ok = ReadFile(dir + "/input/x2_gm.bin", bFileSize, src1Host, bFileSize) && ok;
-    if (!ok) {
-        std::printf("test failed (inputs)\n");
+    try {
+        const int rc = Run(ParseArgs(argc, argv));
+        std::printf(rc == 0 ? "test success\n" : "test failed\n");
+        return rc;
+    } catch (const std::exception &e) {
+        std::printf("test failed (%s)\n", e.what());
         return 2;
     }
-    aclrtMemcpy(src0Device, aFileSize, src0Host, aFileSize, ACL_MEMCPY_HOST_TO_DEVICE);
-    aclrtMemcpy(src1Device, bFileSize, src1Host, bFileSize, ACL_MEMCPY_HOST_TO_DEVICE);
-    LaunchGEMME2E<uint16_t>(dstDevice, src0Device, src1Device, stream);
-    aclrtSynchronizeStream(stream);
-    aclrtMemcpy(dstHost, cFileSize, dstDevice, cFileSize, ACL_MEMCPY_DEVICE_TO_HOST);
-    WriteFile(dir + "/output/output_z.bin", dstHost, cFileSize);
-
-    aclrtFree(dstDevice);
-    aclrtFree(src0Device);
-    aclrtFree(src1Device);
-    aclrtFreeHost(dstHost);
-    aclrtFreeHost(src0Host);
-    aclrtFreeHost(src1Host);
-    aclrtDestroyStream(stream);
-    aclrtResetDevice(0);
-    aclFinalize();
-    if (gStatus != PTO_OK) {
-        std::printf("test failed (pto_gemm_f16f32 returned %d)\n", gStatus);
-        return 1;
-    }
-
-    const size_t count = (size_t)gM * gN;
-    std::vector<float> golden(count), devFinal(count);
-    ok = ReadFile(dir + "/output/golden.bin", cFileSize, golden.data(), cFileSize);
-    ok = ReadFile(dir + "/output/output_z.bin", cFileSize, devFinal.data(), cFileSize) && ok;
-    const bool ret = ok && ResultCmp(golden, devFinal, 0.001f);
-    std::printf(ret ? "test success\n" : "test failed\n");
-    return ret ? 0 : 1;
 }

@@ -170,3 +170,57 @@ def test_call_kernel_flash_attention_causal_rule_of_the_reference(oracle, s0, s1
     assert np.max(np.abs(got - want)) / np.max(np.abs(want)) < 2e-3
     oo, _, _ = oracle.fa_stream_f16(q, k, v, tile_s1=64, causal=True, q_offset=0, round_away=False)
     assert np.max(np.abs(got - oo)) / np.max(np.abs(oo)) < 5e-4
+
+
+def test_acl_fp16_conversions_match_ieee(tmp_path):
+    """aclFloatToFloat16 / aclFloat16ToFloat of the runtime shim (what the reference's flash-attention host program converts
+    its fp16 files with): every fp16 pattern to float and back, and float -> fp16 equal to numpy's round-to-nearest-even on
+    normals, subnormals, ties, overflow and the specials."""
+    src = tmp_path / "cvt.cpp"
+    src.write_text("""
+#include <acl/acl.h>
+#include <cstdio>
+#include <vector>
+int main(int argc, char **argv)
+{
+    std::FILE *f = std::fopen(argv[1], "rb");
+    std::vector<float> in(1 << 20);
+    const size_t n = std::fread(in.data(), sizeof(float), in.size(), f);
+    std::fclose(f);
+    std::vector<unsigned short> out(n);
+    for (size_t i = 0; i < n; ++i)
+        out[i] = aclFloatToFloat16(in[i]);
+    f = std::fopen(argv[2], "wb");
+    std::fwrite(out.data(), 2, n, f);
+    std::fclose(f);
+    std::vector<float> all(65536);
+    for (unsigned h = 0; h < 65536; ++h)
+        all[h] = aclFloat16ToFloat((aclFloat16)h);
+    f = std::fopen(argv[3], "wb");
+    std::fwrite(all.data(), 4, all.size(), f);
+    std::fclose(f);
+    return 0;
+}
+""")
+    exe = tmp_path / "cvt"
+    r = subprocess.run(["g++", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "include"), "-I/opt/rocm/include", "-D__HIP_PLATFORM_AMD__",
+                        str(src), "-o", str(exe), "-L/opt/rocm/lib", "-lamdhip64", "-Wl,-rpath,/opt/rocm/lib"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    rng = np.random.default_rng(5)
+    every = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    finite = every[np.isfinite(every)]
+    mids = ((finite[:-1].astype(np.float64) + np.sort(finite)[1:].astype(np.float64)) / 2).astype(np.float32)   # includes exact ties
+    x = np.concatenate([rng.normal(size=200000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, size=200000).astype(np.float32),
+                        every, mids, np.sort(finite)[:-1] + np.float32(0), np.float32([65504, 65519.99, 65520, 1e9, -1e9, 2.0 ** -25,
+                                                                                      2.0 ** -25 * 1.0001, 2.0 ** -24, 0.0, -0.0, np.inf, -np.inf])])
+    x = x[:1 << 20].astype(np.float32)
+    x.tofile(tmp_path / "in.bin")
+    subprocess.run([str(exe), str(tmp_path / "in.bin"), str(tmp_path / "out.bin"), str(tmp_path / "all.bin")], check=True)
+    got = np.fromfile(tmp_path / "out.bin", dtype=np.uint16)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    nan = np.isnan(x)
+    assert np.array_equal(got[~nan], want[~nan])
+    assert np.all(np.isnan(got[nan].view(np.float16)))
+    back = np.fromfile(tmp_path / "all.bin", dtype=np.float32)
+    assert np.array_equal(back.view(np.uint32)[~np.isnan(every)], every.view(np.uint32)[~np.isnan(every)]) and np.all(np.isnan(back[np.isnan(every)]))
