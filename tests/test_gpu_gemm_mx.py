@@ -232,6 +232,28 @@ def test_mx_gemm_public_entry_narrow_n_and_kernel_choice(oracle, fmt):
         assert np.array_equal(gemm_mx(a, b, sa, sb, fmt), oracle.mx_gemm(a, b, sa, sb, fmt)), (m, n, k)
 
 
+@pytest.mark.parametrize("variant", [5, 6])
+@pytest.mark.parametrize("fmt,m,n,k", [(0, 256, 192, 2560), (1, 512, 384, 3584), (0, 256, 256, 4608), (4, 256, 192, 5120),
+                                       (4, 512, 384, 7168), (4, 256, 256, 9216)])
+def test_mx_gemm_four_wave_kernel_scale_periods(oracle, fmt, m, n, k, variant):
+    """K extents that end inside a scale period of the four-wave kernel (64 scale bytes of a row = 16 K-steps of fp8, 8 of
+    fp4, loaded at once; K is whole groups of four steps only): scales drawn per block from a wide range with operands of
+    ones, so that a scale register taken from the wrong quarter or period shows, then the generator's data exactly."""
+    rng = np.random.default_rng(k + fmt)
+    one = datagen.fp8_encode(np.ones(1), fmt)[0]
+    a, b = np.full((m, k), one, dtype=np.uint8), np.full((n, k), one, dtype=np.uint8)
+    if fmt == 4:
+        a, b = datagen.fp4_pack(a), datagen.fp4_pack(b)
+    sa = rng.integers(124, 131, size=(m, k // 32)).astype(np.uint8)
+    sb = rng.integers(124, 131, size=(n, k // 32)).astype(np.uint8)
+    want = 32.0 * (np.exp2(sa.astype(np.float64) - 127) @ np.exp2(sb.astype(np.float64) - 127).T)
+    rc, got = _mx_variant(a, b, sa, sb, fmt, variant)
+    assert rc == 0 and np.array_equal(got.astype(np.float64), want)
+    a, b, sa, sb = datagen.mx_inputs(m, n, k, fmt, dist="integer")
+    rc, got = _mx_variant(a, b, sa, sb, fmt, variant)
+    assert rc == 0 and np.array_equal(got, oracle.mx_gemm(a, b, sa, sb, fmt))
+
+
 def test_mx_gemm_four_wave_kernel_refuses():
     import torch
     p = torch.zeros(1 << 20, dtype=torch.uint8, device="cuda:0").data_ptr()
