@@ -719,6 +719,15 @@ PTO_INST std::enable_if_t<A::Loc == TileType::Left, RecordEvent> TMATMUL_MX(C &c
     TMATMUL_MX_IMPL(cOut, cIn, a, aScale, b, bScale);
     return {};
 }
+// TMATMUL_MX with a [1, n] Bias tile: c = a x b + bias  (pto_instr.hpp:444-451 of the reference)
+template <typename C, typename A, typename AS, typename B, typename BS, typename Bias, typename... Ev,
+          std::enable_if_t<A::Loc == TileType::Left && Bias::Loc == TileType::Bias, int> = 0>
+PTO_INST RecordEvent TMATMUL_MX(C &c, A &a, AS &aScale, B &b, BS &bScale, Bias &bias, Ev &... ev)
+{
+    TSYNC(ev...);
+    TMATMUL_MX_IMPL(c, a, aScale, b, bScale, bias);
+    return {};
+}
 template <typename D, typename S, typename... Ev>
 PTO_INST RecordEvent TCVT(D &dst, S &src, RoundMode mode, SaturationMode sat, Ev &... ev)
 {

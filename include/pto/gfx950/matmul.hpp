@@ -258,6 +258,14 @@ PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasT &bias)
     TMATMUL_IMPL(c, a, b);
     detail::add_bias_any(c, bias);
 }
+// the same for MX operands: the scaled product, then the bias row added to every row of the result
+template <typename AccT, typename LeftT, typename LeftScaleT, typename RightT, typename RightScaleT, typename BiasT>
+PTO_DEV std::enable_if_t<BiasT::Loc == TileType::Bias> TMATMUL_MX_IMPL(AccT &c, LeftT &a, LeftScaleT &sa, RightT &b, RightScaleT &sb,
+                                                                     BiasT &bias)
+{
+    detail::mad_mx<true>(c, c, a, sa, b, sb);
+    detail::add_bias_any(c, bias);
+}
 
 template <typename AccT, typename LeftT, typename RightT>
 PTO_DEV void TMATMUL_BIAS_IMPL(AccT &c, LeftT &a, RightT &b, BiasRow bias)

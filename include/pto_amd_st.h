@@ -89,6 +89,10 @@ int pto_st_matmul_f32_128x32x256(void *stream, float *out, const float *a, const
  * L1) instead of being loaded from memory into scale tiles directly. */
 int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
                                  const uint8_t *scale_b_t, int format_a, int format_b, int scales_via_lds);
+/* The same with a bias row [128] fp32 added: the first k half through the bias form of TMATMUL_MX (a [1, n] Bias tile;
+ * pto_instr.hpp:444-451 of the reference), the second through the accumulating form.  Scales from registers. */
+int pto_st_matmul_mx_bias_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
+                                      const uint8_t *scale_b_t, const float *bias, int format_a, int format_b);
 
 /* One Vec instruction on [64,128] fp32 tiles: out = OP(a [, b | scalar | vec]).  vec is a per-row [64] operand for
  * the TROWEXPAND* ops and a per-column [128] operand for the TCOLEXPAND* ops.  op codes (PTO_VOP_*): unary

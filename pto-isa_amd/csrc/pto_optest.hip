@@ -316,9 +316,11 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulTyped(__gm__ CT *o
 // in two halves of 128: TMATMUL_MX on the first, the accumulating form on the second.  VIA_MAT == false: the scale tiles
 // are loaded whole from memory (MX_A_ND / MX_B_DN) into registers and windowed per half; true: the scales are TLOADed
 // into Mat tiles (as the reference kernels stage them in L1) and each half's scale tiles TEXTRACTed from there.
+// bias != nullptr: the first half is the bias form of TMATMUL_MX with the row bias[0 .. 127] in a Bias tile.
 template <typename FA, typename FB, bool VIA_MAT>
 __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMx(__gm__ float *out, __gm__ const FA *a, __gm__ const FB *bT,
-                                                                 __gm__ const float8_e8m0_t *sa, __gm__ const float8_e8m0_t *sbT)
+                                                                 __gm__ const float8_e8m0_t *sa, __gm__ const float8_e8m0_t *sbT,
+                                                                 __gm__ const float *bias)
 {
     constexpr int M = 128, N = 128, K = 256, KH = 128, KB = K / 32;
     using X = float8_e8m0_t;
@@ -364,7 +366,14 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void MatmulMx(__gm__ float *o
         TEXTRACT(ls, lsAll, 0, 0);
         TEXTRACT(rs, rsAll, 0, 0);
     }
-    TMATMUL_MX(c, l, ls, r, rs);
+    if (bias != nullptr) {
+        Tile<TileType::Bias, float, 1, N, BLayout::RowMajor, 1, N> biasTile;
+        GlobalTensor<float, Shape<1, 1, 1, 1, N>, Stride<N, N, N, N, 1>> gBias(const_cast<float *>(bias));
+        TLOAD(biasTile, gBias);
+        TMATMUL_MX(c, l, ls, r, rs, biasTile);
+    } else {
+        TMATMUL_MX(c, l, ls, r, rs);
+    }
     TEXTRACT(l, am, 0, KH);
     TEXTRACT(r, bm, KH, 0);
     if constexpr (VIA_MAT) {
@@ -739,8 +748,8 @@ extern "C" int pto_st_matmul_f32_128x32x256(void *stream, float *out, const floa
     return pto_amd::check_launch();
 }
 
-extern "C" int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
-                                            const uint8_t *scale_b_t, int format_a, int format_b, int scales_via_lds)
+static int matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
+                                 const uint8_t *scale_b_t, const float *bias, int format_a, int format_b, int scales_via_lds)
 {
     PTO_ST_NONNULL(out, a, b_t, scale_a, scale_b_t);
     if (format_a < 0 || format_a > 1 || format_b < 0 || format_b > 1)
@@ -756,10 +765,10 @@ extern "C" int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint
             return attr0 != PTO_OK ? attr0 : attr1;                                                                           \
         if (scales_via_lds)                                                                                                   \
             MatmulMx<FA, FB, true><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const FA *>(a),           \
-                                                                              reinterpret_cast<const FB *>(b_t), sa, sb);    \
+                                                                              reinterpret_cast<const FB *>(b_t), sa, sb, bias); \
         else                                                                                                                  \
             MatmulMx<FA, FB, false><<<dim3(1), dim3(kBlockThreads), lds, st>>>(out, reinterpret_cast<const FA *>(a),          \
-                                                                               reinterpret_cast<const FB *>(b_t), sa, sb);   \
+                                                                               reinterpret_cast<const FB *>(b_t), sa, sb, bias); \
     } while (0)
     if (format_a == 0 && format_b == 0)
         PTO_ST_MX(float8_e4m3_t, float8_e4m3_t);
@@ -771,6 +780,19 @@ extern "C" int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint
         PTO_ST_MX(float8_e5m2_t, float8_e5m2_t);
 #undef PTO_ST_MX
     return pto_amd::check_launch();
+}
+
+extern "C" int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
+                                            const uint8_t *scale_b_t, int format_a, int format_b, int scales_via_lds)
+{
+    return matmul_mx_128x256x128(stream, out, a, b_t, scale_a, scale_b_t, nullptr, format_a, format_b, scales_via_lds);
+}
+
+extern "C" int pto_st_matmul_mx_bias_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
+                                                 const uint8_t *scale_b_t, const float *bias, int format_a, int format_b)
+{
+    PTO_ST_NONNULL(bias);
+    return matmul_mx_128x256x128(stream, out, a, b_t, scale_a, scale_b_t, bias, format_a, format_b, 0);
 }
 
 extern "C" int pto_st_matmul_bias_128x64x256(void *stream, float *out, const uint16_t *a, const uint16_t *b_t,

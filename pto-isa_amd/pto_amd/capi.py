@@ -52,6 +52,7 @@ ST_SYMBOLS = {
     "pto_st_matmul_s8_128x128x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_f32_128x32x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_mx_128x256x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 3),
+    "pto_st_matmul_mx_bias_128x256x128": (C.c_int, [C.c_void_p] * 7 + [C.c_int] * 2),
     "pto_st_vec_op_typed_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int]),
     "pto_st_matmul_vec_operands_f16_64x64x128": (C.c_int, [C.c_void_p] * 5),
     "pto_st_tpart_f32_64x128": (C.c_int, [C.c_void_p] * 4 + [C.c_int] * 7),

@@ -294,6 +294,24 @@ def test_tmatmul_mx_single_tile(oracle, fmt_a, fmt_b, via_lds):
             assert np.max(np.abs(got - want)) <= 2e-3 * np.max(np.abs(want)), (dist, fmt_a, fmt_b)
 
 
+@pytest.mark.parametrize("fmt", [0, 1])
+def test_tmatmul_mx_bias_form(oracle, fmt):
+    """TMATMUL_MX(c, a, aScale, b, bScale, bias) with a [1, n] Bias tile (the reference's bias form, pto_instr.hpp:444-451;
+    its generator adds the bias row to every row of the product: tmatmul_mx/gen_data.py): integer operands and an integer
+    bias row, exact."""
+    from pto_amd import datagen
+    lib = capi.load_st()
+    a, b, sa, sb = datagen.mx_inputs(128, 128, 256, fmt, dist="integer", scale_lo=126, scale_hi=130)
+    bias = np.random.default_rng(9).integers(-10, 10, size=128).astype(np.float32)
+    out = torch.full((128, 128), float("nan"), device=DEV)
+    ta, tb, tsa, tsb, tbias = (torch.from_numpy(x).to(DEV) for x in (a, b, sa, sb, bias))
+    capi.check(lib.pto_st_matmul_mx_bias_128x256x128(st(), out.data_ptr(), ta.data_ptr(), tb.data_ptr(), tsa.data_ptr(), tsb.data_ptr(),
+                                                     tbias.data_ptr(), fmt, fmt), "matmul mx bias")
+    torch.cuda.synchronize()
+    want = oracle.mx_gemm(a, b, sa, sb, fmt, fmt) + bias[None, :]
+    assert np.array_equal(out.cpu().numpy(), want.astype(np.float32))
+
+
 def test_tmatmul_int8_to_int32(oracle):
     """int8 x int8 -> int32 (v_mfma_i32_32x32x32_i8), TMATMUL then TMATMUL_ACC over two k halves: exact."""
     lib = capi.load_st()
