@@ -146,8 +146,11 @@ __global__ __launch_bounds__(kBlockThreads, 1) AICORE void FlashAttnFwdM16(__gm_
     }
     const int q0 = qt * kBQ;
     __gm__ half *qBase = const_cast<half *>(qAll) + ((int64_t)bh * seqQ + q0) * D;
-    __gm__ half *kBase = const_cast<half *>(kAll) + (int64_t)bh * seqKv * D;
-    __gm__ half *vBase = const_cast<half *>(vAll) + (int64_t)bh * seqKv * D;
+    // (the same in every lane: kept in scalar registers, so that the tile addresses of the copies are scalar arithmetic)
+    __gm__ half *kBase = reinterpret_cast<half *>(const_cast<char *>(
+        detail::uniform_ptr(reinterpret_cast<const char *>(kAll + (int64_t)bh * seqKv * D))));
+    __gm__ half *vBase = reinterpret_cast<half *>(const_cast<char *>(
+        detail::uniform_ptr(reinterpret_cast<const char *>(vAll + (int64_t)bh * seqKv * D))));
     int numTiles = seqKv / kBKV;
     if (CAUSAL) {
         const int lim = (q0 + kBQ - 1 + causalOff) / kBKV + 1;
