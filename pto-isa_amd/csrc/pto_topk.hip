@@ -30,12 +30,14 @@ __device__ inline uint32_t ScoreBits(uint32_t ord) { return (ord & 0x80000000u) 
 template <int M>
 __device__ inline uint32_t LaneXor(uint32_t v, int lane)
 {
+    // (every lane has a source lane in these three patterns, so the destination needs no initial value: mov_dpp, not
+    // update_dpp with a zero that costs a move per call)
     if constexpr (M == 1)
-        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false); // quad_perm [1,0,3,2]
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0xB1, 0xf, 0xf, true); // quad_perm [1,0,3,2]
     else if constexpr (M == 2)
-        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false); // quad_perm [2,3,0,1]
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x4E, 0xf, 0xf, true); // quad_perm [2,3,0,1]
     else if constexpr (M == 8)
-        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128, 0xf, 0xf, false); // row_ror:8 (rows of 16 lanes)
+        return (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x128, 0xf, 0xf, true); // row_ror:8 (rows of 16 lanes)
     else if constexpr (M < 32)
         return (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, (M << 10) | 0x1f); // bit mode: lane ^ M within 32 lanes
     else
@@ -60,8 +62,15 @@ __device__ inline void StaticFor(F &&f)
 template <int E>
 __device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
 {
-    constexpr int N = kTopkThreads * E, kLogN = __builtin_ctz(N);
+    constexpr int N = kTopkThreads * E, kLogN = __builtin_ctz(N), kLogE = __builtin_ctz(E);
     const int lane = tid & 63;
+    // The lane predicates of the network, once: bit s of the key's rank for every run length and partner distance that
+    // spans threads (as lane masks they live in scalar registers; computed per stage they were an eighth of the vector
+    // instructions).
+    bool rankBitClear[kLogN + 1];
+#pragma unroll
+    for (int s = 0; s <= kLogN; ++s)
+        rankBitClear[s] = s < kLogE ? true : ((tid >> (s - kLogE)) & 1) == 0;
     StaticFor<1, kLogN + 1>([&](auto sizeTag) {
         constexpr int kk = 1 << decltype(sizeTag)::value; // the network sorts runs of kk keys, alternating direction
         StaticFor<0, decltype(sizeTag)::value>([&](auto strideTag) {
@@ -70,7 +79,8 @@ __device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
 #pragma unroll
                 for (int e = 0; e < E; ++e)
                     if ((e & j) == 0) {
-                        const bool descending = ((tid * E + e) & kk) == 0;
+                        // (run lengths below E: the direction is a property of the register, not of the lane)
+                        const bool descending = kk < E ? (e & kk) == 0 : (kk == N ? true : rankBitClear[decltype(sizeTag)::value]);
                         const uint64_t a = k[e], b = k[e | j];
                         const bool swap = descending ? a < b : a > b;
                         k[e] = swap ? b : a;
@@ -95,7 +105,8 @@ __device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
                         other[e] = lds[e * kTopkThreads + (tid ^ (j / E))];
                 }
                 // the lower rank of a pair keeps the larger key where the run is descending
-                const bool lower = ((tid * E) & j) == 0, descending = ((tid * E) & kk) == 0;
+                const bool lower = rankBitClear[__builtin_ctz(j)];
+                const bool descending = kk == N ? true : rankBitClear[decltype(sizeTag)::value];
                 const bool keepMax = lower == descending;
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
