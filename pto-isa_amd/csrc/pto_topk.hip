@@ -49,6 +49,27 @@ __device__ inline uint64_t LaneXor64(uint64_t v, int lane)
     return ((uint64_t)LaneXor<M>((uint32_t)(v >> 32), lane) << 32) | LaneXor<M>((uint32_t)v, lane);
 }
 
+// Compare and select on wave masks held in scalar register pairs.  (Measured on gfx950: a conditional move that takes its
+// mask from VCC issues at a fifth of the rate of one that takes it from a scalar register pair, so the selects of the
+// network name their masks themselves instead of leaving the choice to the compiler.)  All 64 lanes are active here.
+__device__ inline uint64_t MaskLess(uint64_t a, uint64_t b)
+{
+    uint64_t m;
+    asm("v_cmp_lt_u64_e64 %0, %1, %2" : "=s"(m) : "v"(a), "v"(b));
+    return m;
+}
+__device__ inline uint32_t SelectWord(uint64_t mask, uint32_t ifSet, uint32_t ifClear)
+{
+    uint32_t r;
+    asm("v_cndmask_b32_e64 %0, %1, %2, %3" : "=v"(r) : "v"(ifClear), "v"(ifSet), "s"(mask));
+    return r;
+}
+__device__ inline uint64_t Select(uint64_t mask, uint64_t ifSet, uint64_t ifClear)
+{
+    return ((uint64_t)SelectWord(mask, (uint32_t)(ifSet >> 32), (uint32_t)(ifClear >> 32)) << 32) |
+           SelectWord(mask, (uint32_t)ifSet, (uint32_t)ifClear);
+}
+
 template <int FIRST, int LAST, typename F>
 __device__ inline void StaticFor(F &&f)
 {
@@ -67,24 +88,28 @@ __device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
     // The lane predicates of the network, once: bit s of the key's rank for every run length and partner distance that
     // spans threads (as lane masks they live in scalar registers; computed per stage they were an eighth of the vector
     // instructions).
-    bool rankBitClear[kLogN + 1];
+    uint64_t rankBitClear[kLogN + 1]; // wave masks
 #pragma unroll
     for (int s = 0; s <= kLogN; ++s)
-        rankBitClear[s] = s < kLogE ? true : ((tid >> (s - kLogE)) & 1) == 0;
+        rankBitClear[s] = s < kLogE ? ~0ull : __builtin_amdgcn_ballot_w64(((tid >> (s - kLogE)) & 1) == 0);
     StaticFor<1, kLogN + 1>([&](auto sizeTag) {
         constexpr int kk = 1 << decltype(sizeTag)::value; // the network sorts runs of kk keys, alternating direction
+        // lanes whose run is descending (the last stage sorts the whole row downwards)
+        const uint64_t descending = kk == N ? ~0ull : rankBitClear[decltype(sizeTag)::value];
         StaticFor<0, decltype(sizeTag)::value>([&](auto strideTag) {
             constexpr int j = kk >> (decltype(strideTag)::value + 1); // distance between partners
             if constexpr (j < E) {
 #pragma unroll
                 for (int e = 0; e < E; ++e)
                     if ((e & j) == 0) {
-                        // (run lengths below E: the direction is a property of the register, not of the lane)
-                        const bool descending = kk < E ? (e & kk) == 0 : (kk == N ? true : rankBitClear[decltype(sizeTag)::value]);
                         const uint64_t a = k[e], b = k[e | j];
-                        const bool swap = descending ? a < b : a > b;
-                        k[e] = swap ? b : a;
-                        k[e | j] = swap ? a : b;
+                        const uint64_t less = MaskLess(a, b);
+                        // descending runs swap where a < b, ascending ones where a >= b (equal keys are the padding:
+                        // swapping them changes nothing).  Run lengths below E: the direction is a property of the
+                        // register, not of the lane.
+                        const uint64_t swap = kk < E ? ((e & kk) == 0 ? less : ~less) : ~(less ^ descending);
+                        k[e] = Select(swap, b, a);
+                        k[e | j] = Select(swap, a, b);
                     }
             } else {
                 uint64_t other[E];
@@ -105,13 +130,11 @@ __device__ inline void SortInRegisters(uint64_t (&k)[E], uint64_t *lds, int tid)
                         other[e] = lds[e * kTopkThreads + (tid ^ (j / E))];
                 }
                 // the lower rank of a pair keeps the larger key where the run is descending
-                const bool lower = rankBitClear[__builtin_ctz(j)];
-                const bool descending = kk == N ? true : rankBitClear[decltype(sizeTag)::value];
-                const bool keepMax = lower == descending;
+                const uint64_t keepMax = ~(rankBitClear[__builtin_ctz(j)] ^ descending);
 #pragma unroll
                 for (int e = 0; e < E; ++e) {
-                    const bool otherLarger = other[e] > k[e];
-                    k[e] = (otherLarger == keepMax) ? other[e] : k[e];
+                    const uint64_t otherLarger = MaskLess(k[e], other[e]);
+                    k[e] = Select(~(otherLarger ^ keepMax), other[e], k[e]);
                 }
             }
         });
