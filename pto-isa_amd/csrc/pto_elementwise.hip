@@ -53,6 +53,34 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void CvtF32(__gm__ D *dst, __
     TSTORE(dstGlobal, dstTile);
 }
 
+// Whole tiles in the default rounding mode take a streaming form of the same conversion below the tile instructions:
+// a lane loads 16 bytes and stores 8, so that every load instruction of a wave covers 1 KiB of consecutive addresses and
+// every store 512 bytes (a Vec tile gives a lane eight consecutive elements, i.e. two loads 32 bytes apart per lane and
+// half-used lines per instruction), all eight loads of a lane are in flight before the first conversion, and there is
+// no barrier; the stores are non-temporal (measured with inputs and outputs that no cache holds: 6.5 against 6.2 TB/s
+// with plain stores).  Same element function as TCVT (detail::convert), so the results are the same bits.
+template <typename D>
+__global__ __launch_bounds__(kBlockThreads) void CvtF32Stream(D *dst, const float *src, size_t firstTile)
+{
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef uint16_t u16x4 __attribute__((ext_vector_type(4)));
+    constexpr int kPerStep = kBlockThreads * 4, kSteps = kCvtTile / kPerStep;
+    static_assert(kCvtTile % kPerStep == 0 && sizeof(D) == 2, "whole steps of 16-bit results");
+    const size_t base = (firstTile + blockIdx.x) * (size_t)kCvtTile + 4 * threadIdx.x;
+    f32x4 x[kSteps];
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i)
+        x[i] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(src + base + (size_t)i * kPerStep));
+#pragma unroll
+    for (int i = 0; i < kSteps; ++i) {
+        u16x4 y;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            y[j] = __builtin_bit_cast(uint16_t, ::pto::detail::convert<D, float>(x[i][j], RoundMode::CAST_RINT));
+        __builtin_nontemporal_store(y, reinterpret_cast<u16x4 *>(dst + base + (size_t)i * kPerStep));
+    }
+}
+
 constexpr int kGatherRows = 32, kGatherCols = 256; // one Vec tile: 8192 elements
 
 template <typename T, bool kTailCols>
@@ -122,7 +150,10 @@ int launch_cvt(void *stream, D *dst, const float *src, size_t n, int mode)
     constexpr size_t kMaxBlocks = 1u << 30;
     for (size_t t0 = 0; t0 < full; t0 += kMaxBlocks) {
         const size_t nb = full - t0 < kMaxBlocks ? full - t0 : kMaxBlocks;
-        CvtF32<D, false><<<dim3((unsigned)nb), dim3(kBlockThreads), 0, st>>>(dst, src, n, t0, mode);
+        if (mode == PTO_CAST_RINT)
+            CvtF32Stream<D><<<dim3((unsigned)nb), dim3(kBlockThreads), 0, st>>>(dst, src, t0);
+        else
+            CvtF32<D, false><<<dim3((unsigned)nb), dim3(kBlockThreads), 0, st>>>(dst, src, n, t0, mode);
     }
     if (tail)
         CvtF32<D, true><<<dim3(1), dim3(kBlockThreads), 0, st>>>(dst, src, n, full, mode);
