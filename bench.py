@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the PTO tile compute path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|mx|fa|tcvt|gather|topk]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--only gemm|mx|fa|tcvt|quant|gather|topk]
 
 A step is one pass of the hot path over one batch of synthetic input, resident in HBM before the
 timed region: one fp16 -> fp32 GEMM at m=n=k=6144 (the configuration the headline metric is quoted
@@ -167,6 +167,27 @@ def bench_tcvt(torch, lib, capi, datagen, steps, warmup, kind):
     return {"ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9, "bytes": nbytes}
 
 
+def bench_quant(torch, lib, capi, datagen, steps, warmup):
+    """MXFP8 quantisation (the a5 TQUANT) of a 16384 x 8192 fp32 matrix: 4 bytes read, 1 + 1/32 written per element; two
+    buffer sets, alternated, so that no launch finds its input in cache."""
+    rows, cols = 16384, 8192
+    n = rows * cols
+    x0 = torch.from_numpy(datagen.quant_input(rows, cols, specials=True)).cuda()
+    xs = [x0, x0.flip(0).contiguous()]
+    qs = [torch.empty((rows, cols), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    ss = [torch.empty((rows, cols // 32), dtype=torch.uint8, device="cuda") for _ in range(2)]
+    st = torch.cuda.current_stream().cuda_stream
+    i = [0]
+
+    def step():
+        j = i[0] & 1
+        i[0] += 1
+        capi.check(lib.pto_quant_mxfp8_f32(st, qs[j].data_ptr(), ss[j].data_ptr(), xs[j].data_ptr(), rows, cols), "quant")
+    ms = time_launches(torch, step, steps, warmup)
+    nbytes = n * (4.0 + 1.0 + 1.0 / 32)
+    return {"ms": ms, "gbs": nbytes / (ms * 1e-3) / 1e9, "bytes": nbytes}
+
+
 def bench_gather(torch, lib, capi, datagen, steps, warmup):
     import numpy as np
     table, idx = datagen.gather_inputs(16384, 1024, 65536)
@@ -237,6 +258,11 @@ def cpu_baselines_extra(datagen, cores):
     oracle.tcvt_f32_f16(x)
     dt = time.perf_counter() - t0
     out["tcvt_f32_f16"] = {"gbs": x.size * 6.0 / dt / 1e9, "cores": 1, "kind": "port", "sample": "%d elements, %.2f s" % (x.size, dt)}
+    xq = datagen.quant_input(2048, 8192)
+    t0 = time.perf_counter()
+    oracle.quant_mxfp8(xq)
+    dt = time.perf_counter() - t0
+    out["quant_mxfp8_f32"] = {"gbs": xq.size * (5.0 + 1.0 / 32) / dt / 1e9, "cores": 1, "kind": "port", "sample": "%d elements, %.2f s" % (xq.size, dt)}
     table, idx = datagen.gather_inputs(16384, 1024, 8192)
     t0 = time.perf_counter()
     oracle.gather_rows(table, idx)
@@ -265,7 +291,7 @@ def main():
     ap.add_argument("--settle-ms", type=float, default=300.0,
                     help="workloads under \"extra\": after the warm-up launches keep launching untimed until this much time has passed")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--only", default="", help="gemm | mx | fa | tcvt | gather | topk: time just that workload")
+    ap.add_argument("--only", default="", help="gemm | mx | fa | tcvt | quant | gather | topk: time just that workload")
     ap.add_argument("--size", type=int, default=6144)
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run a plain 1 GiB device copy a few times (reference point for FETCH_SIZE / WRITE_SIZE counters)")
@@ -323,6 +349,9 @@ def main():
         for kind in ("f16", "bf16"):
             r = bench_tcvt(torch, lib, capi, datagen, args.steps, args.warmup, kind)
             extra["tcvt_f32_%s_16384x8192" % kind] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS}
+    if only in ("", "quant") and hasattr(lib, "pto_quant_mxfp8_f32"):
+        r = bench_quant(torch, lib, capi, datagen, args.steps, args.warmup)
+        extra["quant_mxfp8_f32_16384x8192"] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS}
     if only in ("", "topk"):
         r = bench_topk(torch, lib, capi, datagen, args.steps, args.warmup)
         extra["topk_4800x1024_top1000_f32"] = {"ms": r["ms"], "gbs": r["gbs"], "frac_hbm_peak": r["gbs"] / PEAK_HBM_GBS,

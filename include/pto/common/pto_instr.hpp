@@ -282,6 +282,19 @@ PTO_FRONT(TFILLPAD_EXPAND, typename D PTO_C typename S, D &dst PTO_C S &src, (ds
 PTO_FRONT(TPACK, typename D PTO_C typename S, D &dst PTO_C S &src, (dst, src))
 // TPREFETCH (pto_instr.hpp:135-140 of the reference; cpu/TPrefetch.hpp copies the region into the tile): a TLOAD here
 PTO_FRONT(TPREFETCH, typename TileT PTO_C typename G, TileT &dst PTO_C G &src, (dst, src))
+// TQUANT, the block-scaled MXFP8 form (pto_instr.hpp:1481-1490 of the reference): exponent, maximum and scaling tiles by address
+template <auto quant, typename D, typename S, typename E, typename M, typename... Ev>
+PTO_INST RecordEvent TQUANT(D &dst, S &src, E *exp, M *max, S *scaling, Ev &... ev)
+{
+    TSYNC(ev...);
+    detail::UbFetch(src);
+    TQUANT_IMPL<quant>(dst, src, exp, max, scaling);
+    detail::UbCommit(dst);
+    detail::UbCommit(*exp);
+    detail::UbCommit(*max);
+    detail::UbCommit(*scaling);
+    return {};
+}
 // TQUANT, the row-scale form (pto_instr.hpp:1503-1510 of the reference)
 template <auto quant, typename D, typename S, typename P, typename... Ev>
 PTO_INST RecordEvent TQUANT(D &dst, S &src, P &scale, P *offset = nullptr, Ev &... ev)

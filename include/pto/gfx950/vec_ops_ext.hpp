@@ -322,7 +322,8 @@ PTO_DEV void TPACK_IMPL(DstT &dst, SrcT &src)
 
 // TQUANT (the a2a3 form, npu/a2a3/TQuant.hpp:26-52): src = src * scale[row] (+ offset[row]), in place as there, then
 // rounded to the nearest integer (ties to even) and saturated to int8 (symmetric) or uint8 (asymmetric)
-enum class QuantType { INT8_SYM, INT8_ASYM };
+enum class QuantType { MXFP8, INT8_SYM, INT8_ASYM }; // npu/a5/TQuant.hpp:22-27
+enum class VecStoreMode { ND, NZ };                  // npu/a5/TQuant.hpp:29-33
 template <QuantType quant, typename DstT, typename SrcT, typename ParaT>
 PTO_DEV void TQUANT_IMPL(DstT &dst, SrcT &src, ParaT &scale, ParaT *offset = nullptr)
 {
@@ -343,6 +344,84 @@ PTO_DEV void TQUANT_IMPL(DstT &dst, SrcT &src, ParaT &scale, ParaT *offset = nul
             const float t = __builtin_rintf(c.S().v[s][i]);
             dst.S().v[s][i] = (U)(int)(t < lo ? lo : t > hi ? hi : t); // a NaN compares false twice and converts to 0
         }
+}
+
+// TQUANT<QuantType::MXFP8>(dst, src, &exp, &max, &scaling), the block-scaled form (npu/a5/TQuant.hpp:262-322, ND store
+// mode): every 32 consecutive elements of the fp32 source tile (row-major, Cols a multiple of 32) share one e8m0 exponent.
+//   max[g]     = largest |x| of group g                                   (TQuant.hpp:35-126)
+//   exp[g]     = E - 8, E the biased fp32 exponent of max[g]              (:147-151; 8 = exponent of e4m3's top binade)
+//   scaling[g] = 2^(127 - exp[g]) = the float with bits (254 - exp[g]) << 23   (:153-155)
+//   dst        = e4m3(clip(src * scaling[group], +-448)), round to nearest even (:182-203; the generator of the
+//                reference's test clips and casts: tests/npu/a5/src/st/testcase/tquant/gen_data.py:27-33)
+// Elements outside the source's valid region count as zeros.  A group with an infinity or NaN gets exp 0xff (:158-160) and
+// NaN -> NaN, +-inf -> +-448, finite -> +-0; a group whose maximum is below 2^-119 gets exp 0 (:163-165 store that byte)
+// and the factor 2^127 that this byte stands for (the reference multiplies by its clamp constant 0x7f800000 there).
+// exp, max and scaling are linear arrays of one entry per group in their tiles' element order.  The NZ store mode (fp8 in
+// the fractal layout, exponents reordered through an index tile) is not built.
+namespace detail {
+PTO_DEV uint8_t f32_to_e4m3_bits_sat(float y) // |y| <= 448, not NaN: the hardware conversion rounds to nearest even
+{
+    return (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(y, 0.0f, 0, false) & 0xff);
+}
+} // namespace detail
+template <QuantType quant, typename DstT, typename SrcT, typename ExpT, typename MaxT>
+PTO_DEV void TQUANT_IMPL(DstT &dst, SrcT &src, ExpT *exp, MaxT *max, SrcT *scaling)
+{
+    static_assert(quant == QuantType::MXFP8, "[PTO][SA] TQUANT with exponent, maximum and scaling tiles is the MXFP8 form");
+    static_assert(std::is_same_v<typename SrcT::DType, float> && SrcT::isRowMajor && SrcT::Cols % 32 == 0,
+                  "[PTO][SA] TQUANT MXFP8: fp32 row-major source whose row length is a multiple of 32");
+    static_assert(sizeof(typename DstT::DType) == 1 && DstT::Rows == SrcT::Rows && DstT::Cols == SrcT::Cols && DstT::isRowMajor,
+                  "[PTO][SA] TQUANT MXFP8: one byte per element, the source's shape");
+    static_assert(sizeof(typename ExpT::DType) == 1 && std::is_same_v<typename MaxT::DType, float>,
+                  "[PTO][SA] TQUANT MXFP8: e8m0 bytes and fp32 maxima");
+    constexpr int G = SrcT::Numel / 32;
+    static_assert(ExpT::Numel >= G && MaxT::Numel >= G && G <= 8192, "[PTO][SA] TQUANT MXFP8: one entry per group of 32");
+    __shared__ uint32_t groupMax[G]; // |x| as integers: a NaN is above every number
+    for (int g = hw::tid(); g < G; g += kBlockThreads)
+        groupMax[g] = 0;
+    hw::lds_barrier();
+    const int vr = src.GetValidRow(), vc = src.GetValidCol();
+    detail::for_each_owned<SrcT>([&](int s, int i, int e) {
+        int r, c;
+        detail::elem_rc<SrcT>(e, r, c);
+        if (e < SrcT::Numel && r < vr && c < vc) {
+            const uint32_t a = __builtin_bit_cast(uint32_t, src.S().v[s][i]) & 0x7fffffffu;
+            if (a != 0)
+                atomicMax(&groupMax[e / 32], a);
+        }
+    });
+    hw::lds_barrier();
+    auto expOf = [](uint32_t a) { return (a >> 23) == 255u ? 0xffu : (a >> 23) < 8u ? 0u : (a >> 23) - 8u; };
+    auto scaleOf = [&](uint32_t a) { return __builtin_bit_cast(float, (a >> 23) == 255u ? 0xffu : (254u - expOf(a)) << 23); };
+    using U = typename DstT::DType;
+    detail::for_each_owned<SrcT>([&](int s, int i, int e) {
+        if (e >= SrcT::Numel)
+            return;
+        int r, c;
+        detail::elem_rc<SrcT>(e, r, c);
+        const float x = (r < vr && c < vc) ? src.S().v[s][i] : 0.0f;
+        const uint32_t a = groupMax[e / 32], u = __builtin_bit_cast(uint32_t, x), mag = u & 0x7fffffffu;
+        uint8_t code;
+        if ((a >> 23) == 255u)
+            code = (uint8_t)(((u >> 24) & 0x80u) | (mag > 0x7f800000u ? 0x7fu : mag == 0x7f800000u ? 0x7eu : 0u));
+        else
+            code = detail::f32_to_e4m3_bits_sat(__builtin_fminf(__builtin_fmaxf(x * scaleOf(a), -448.0f), 448.0f));
+        dst.S().v[s][i] = __builtin_bit_cast(U, code);
+    });
+    using EU = typename ExpT::DType;
+    detail::for_each_owned<ExpT>([&](int s, int i, int e) {
+        if (e < G)
+            exp->S().v[s][i] = __builtin_bit_cast(EU, (uint8_t)expOf(groupMax[e]));
+    });
+    detail::for_each_owned<MaxT>([&](int s, int i, int e) {
+        if (e < G)
+            max->S().v[s][i] = __builtin_bit_cast(float, groupMax[e]);
+    });
+    detail::for_each_owned<SrcT>([&](int s, int i, int e) {
+        if (e < G)
+            scaling->S().v[s][i] = scaleOf(groupMax[e]);
+    });
+    hw::lds_barrier();
 }
 
 // TDEQUANT: dst = (float(src) - offset[row]) * scale[row] over the destination's valid region, the two steps rounded

@@ -12,6 +12,9 @@
  *                        ctypes entry call_kernel(blockDim, stream, out, src0, src1) demos/torch_jit/gemm/gemm_kernel.cpp:259-262
  *   pto_gemm_mxfp8       LaunchMxMatmul(uint8_t *out, uint8_t *src0, uint8_t *src1, uint8_t *src2, uint8_t *src3, void *stream)
  *                        kernels/manual/a5/matmul_mxfp8_performance/mxmatmul_performance_kernel.cpp:344-364
+ *   pto_quant_mxfp8_f32  TQUANT<QuantType::MXFP8>(dst, src, &exp, &max, &scaling) include/pto/common/pto_instr.hpp:1481-1490,
+ *                        include/pto/npu/a5/TQuant.hpp:262-322, as launched by runTQuant<rows, cols, 0>
+ *                        tests/npu/a5/src/st/testcase/tquant/tquant_kernel.cpp:27-80 (TLOAD -> TQUANT -> TSTORE of both outputs)
  *   pto_topk_f32         launchTopk<float>(uint8_t *out, uint8_t *index, uint8_t *src, uint8_t *inIdx, void *stream)
  *                        kernels/manual/a2a3/topk/topk_kernel.cpp:334-345
  *   pto_mla_attention_*  mla_pto(q, k, v, wq, wk, wv, wo, out) demos/cpu/mla_attention_demo/mla_attention_demo.cpp:227-397
@@ -74,6 +77,15 @@ int pto_gemm_mxfp8(void *stream, void *c, const uint8_t *a, const uint8_t *b, co
  * when k % 1024 == 0 as well). */
 int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, const uint8_t *scale_a, const uint8_t *scale_b,
                    int m, int n, int k, int c_fp32);
+
+/* MXFP8 quantisation: src [rows, cols] fp32 contiguous, cols % 32 == 0 -> q [rows, cols] float8_e4m3fn bytes and
+ * scale [rows, cols / 32] e8m0 bytes, one per 32 consecutive elements of a row: the operand and scale layout that
+ * pto_gemm_mxfp8 takes for A (rows = m, cols = k) and for B stored [n, k].  Per group: E = biased fp32 exponent of the
+ * largest |x|, scale byte = E - 8, q = e4m3(clip(x * 2^(127 - scale byte), +-448)) rounded to nearest even, so that the
+ * group's largest element lands in [256, 448].  Groups holding an infinity or a NaN: scale byte 0xff, NaN -> NaN (0x7f
+ * with the sign), +-inf -> +-448, finite -> +-0.  Groups whose largest |x| is below 2^-119 (all zeros included): scale
+ * byte 0, factor 2^127. */
+int pto_quant_mxfp8_f32(void *stream, uint8_t *q, uint8_t *scale, const float *src, size_t rows, size_t cols);
 
 /* Row-wise top-k.  src [rows, ld] fp32, the first valid_cols columns of every row are scored; in_idx [valid_cols] uint32
  * gives the index reported for a column (the reference passes 0, 1, 2, ...).  Per row the (score, index) pairs are put in

@@ -91,6 +91,12 @@ int pto_st_matmul_mx_128x256x128(void *stream, float *out, const uint8_t *a, con
                                  const uint8_t *scale_b_t, int format_a, int format_b, int scales_via_lds);
 /* The same with a bias row [128] fp32 added: the first k half through the bias form of TMATMUL_MX (a [1, n] Bias tile;
  * pto_instr.hpp:444-451 of the reference), the second through the accumulating form.  Scales from registers. */
+/* TQUANT<QuantType::MXFP8> on one Vec tile: TLOAD -> TQUANT -> TSTORE, the ND-mode program of the reference's test
+ * (tests/npu/a5/src/st/testcase/tquant/tquant_kernel.cpp:27-80).  shape 0..3 = 32 x 32, 32 x 64, 64 x 128, 128 x 128 (its ND
+ * cases); src [valid_rows, valid_cols] contiguous, elements outside it count as zeros.  out_fp8 [R, C] bytes, out_e8m0 and
+ * out_max [R * C / 32], out_scaling [R, C] floats of which the first R * C / 32 are the groups' factors. */
+int pto_st_tquant_mxfp8(void *stream, uint8_t *out_e8m0, uint8_t *out_fp8, float *out_max, float *out_scaling, const float *src,
+                        int shape, int valid_rows, int valid_cols);
 int pto_st_matmul_mx_bias_128x256x128(void *stream, float *out, const uint8_t *a, const uint8_t *b_t, const uint8_t *scale_a,
                                       const uint8_t *scale_b_t, const float *bias, int format_a, int format_b);
 

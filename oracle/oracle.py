@@ -67,6 +67,10 @@ def lib():
         L.po_topk_f32.restype = None
         L.po_mx_gemm.argtypes = [C.c_void_p] * 5 + [C.c_int] * 6
         L.po_mx_gemm.restype = None
+        L.po_f32_to_fp8_e4m3fn.argtypes = [C.c_float]
+        L.po_f32_to_fp8_e4m3fn.restype = C.c_uint8
+        L.po_quant_mxfp8_e4m3.argtypes = [C.c_void_p] * 5 + [C.c_size_t]
+        L.po_quant_mxfp8_e4m3.restype = None
         L.po_fp8_e4m3fn_to_f32.argtypes = [C.c_uint8]
         L.po_fp8_e4m3fn_to_f32.restype = C.c_float
         L.po_fp8_e5m2_to_f32.argtypes = [C.c_uint8]
@@ -355,6 +359,27 @@ def mx_gemm(A, B, SA, SB, fmt_a=0, fmt_b=None, threads=0):
     Cm = np.empty((m, n), dtype=np.float32)
     lib().po_mx_gemm(_p(Cm), _p(A), _p(B), _p(SA), _p(SB), m, n, k, fmt_a, fmt_b, threads)
     return Cm
+
+
+def quant_mxfp8(x, with_stats=False):
+    """x [..., cols] fp32, cols a multiple of 32 -> (q uint8 e4m3 bytes of x's shape, e8m0 uint8 [..., cols/32]); with_stats
+    adds the per-group absolute maximum and the factor the group was multiplied by."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.shape[-1] % 32 == 0
+    q = np.empty(x.shape, dtype=np.uint8)
+    gshape = x.shape[:-1] + (x.shape[-1] // 32,)
+    e = np.empty(gshape, dtype=np.uint8)
+    amax = np.empty(gshape, dtype=np.float32)
+    scale = np.empty(gshape, dtype=np.float32)
+    lib().po_quant_mxfp8_e4m3(_p(q), _p(e), _p(amax), _p(scale), _p(x), x.size)
+    return (q, e, amax, scale) if with_stats else (q, e)
+
+
+def fp8_e4m3_encode(x):
+    """fp32 array -> e4m3fn bytes, nearest even, saturating, element by element (small arrays)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    f = lib().po_f32_to_fp8_e4m3fn
+    return np.array([f(float(v)) for v in x.reshape(-1)], dtype=np.uint8).reshape(x.shape)
 
 
 # --------------------------------------------------------------- conversion

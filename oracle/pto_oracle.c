@@ -586,6 +586,106 @@ void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA,
     free(Bd);
 }
 
+/* ------------------------------------------------------------------ MXFP8 quantisation */
+/* fp32 -> float8_e4m3fn, round to nearest even, magnitudes above 448 (infinities included) saturate to +-448, NaN ->
+ * sign | 0x7f.  (The reference converts with ROUND_R, RS_ENABLE and the saturation control bit set:
+ * include/pto/npu/a5/TQuant.hpp:198, :283; its generator clips to +-448 and casts to ml_dtypes float8_e4m3fn, which
+ * rounds to nearest even: tests/npu/a5/src/st/testcase/tquant/gen_data.py:27-33.) */
+uint8_t po_f32_to_fp8_e4m3fn(float x)
+{
+    uint32_t u;
+    memcpy(&u, &x, 4);
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u)
+        return (uint8_t)(sign | 0x7fu);
+    if (a >= 0x43e00000u) /* 448 and above */
+        return (uint8_t)(sign | 0x7eu);
+    const int e = (int)(a >> 23) - 127;
+    if (e < -6) { /* below the smallest normal 2^-6: multiples of 2^-9; 8 of them is that normal's code */
+        float mag;
+        memcpy(&mag, &a, 4);
+        return (uint8_t)(sign | (uint8_t)lrintf(mag * 512.0f)); /* exact product, nearest-even under the default mode */
+    }
+    uint32_t m = (a >> 20) & 7u, ex = (uint32_t)(e + 7);
+    const uint32_t rem = a & 0xfffffu;
+    if (rem > 0x80000u || (rem == 0x80000u && (m & 1u))) {
+        if (++m == 8u) {
+            m = 0;
+            ++ex;
+        }
+    }
+    uint32_t code = (ex << 3) | m;
+    if (code > 0x7eu)
+        code = 0x7eu;
+    return (uint8_t)(sign | code);
+}
+
+/* Block-scaled quantisation of fp32 to MXFP8 (e4m3 elements, one e8m0 scale per 32 consecutive elements), the rule of
+ * TQUANT<QuantType::MXFP8> (include/pto/npu/a5/TQuant.hpp:128-180 ExtractB8ExponentAndScaling, :182-203
+ * CalcQuantizedFP8Values) and of its generator (gen_data.py:43-57 fp32_to_fp8_element, :27-33 scale_data):
+ *   amax  = largest |x| of the group, E = its biased fp32 exponent
+ *   e8m0  = E - 8                          (8 = exponent of the largest e4m3 binade: 448 = 1.75 * 2^8)
+ *   scale = 2^(127 - e8m0)                 (fp32 bits (254 - e8m0) << 23), q = e4m3(clip(x * scale, +-448))
+ * so that amax * scale lies in [256, 512).  Outside what the generator's data reaches:
+ *   E == 255 (an infinity or NaN in the group): e8m0 = 0xff as the reference stores; elements: NaN -> NaN, +-inf -> +-448,
+ *       finite -> +-0 (the reference multiplies by the bit pattern 0xff read as a float, 3.6e-43);
+ *   E < 8 (amax < 2^-119, all-zero groups included): e8m0 = 0 as the reference stores, scale = 2^127.  (The reference
+ *       kernel's clamp constant for this case is 0x7f800000, +inf as a factor, which turns a zero group into NaNs; its
+ *       generator wraps the exponent to 248 and yields zeros.  2^127 is the scale that e8m0 = 0 stands for.)
+ * q [n] bytes, e8m0 [n / 32] bytes, amax / scale [n / 32] floats or NULL; n a multiple of 32. */
+void po_quant_mxfp8_e4m3(uint8_t *q, uint8_t *e8m0, float *amax_out, float *scale_out, const float *src, size_t n)
+{
+    for (size_t g = 0; g < n / 32; ++g) {
+        const float *x = src + g * 32;
+        uint32_t amax = 0;
+        for (int i = 0; i < 32; ++i) {
+            uint32_t u;
+            memcpy(&u, &x[i], 4);
+            u &= 0x7fffffffu;
+            if (u > amax)
+                amax = u; /* as integers: a NaN is above every number */
+        }
+        const uint32_t E = amax >> 23;
+        uint32_t scale_bits;
+        uint8_t se;
+        if (E == 255u) {
+            se = 0xffu;
+            scale_bits = 0xffu;
+        } else if (E < 8u) {
+            se = 0;
+            scale_bits = 254u << 23;
+        } else {
+            se = (uint8_t)(E - 8u);
+            scale_bits = (254u - (E - 8u)) << 23;
+        }
+        float scale, am;
+        memcpy(&scale, &scale_bits, 4);
+        memcpy(&am, &amax, 4);
+        e8m0[g] = se;
+        if (amax_out)
+            amax_out[g] = am;
+        if (scale_out)
+            scale_out[g] = scale;
+        for (int i = 0; i < 32; ++i) {
+            uint32_t u;
+            memcpy(&u, &x[i], 4);
+            if (E == 255u) {
+                const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+                const uint32_t a = u & 0x7fffffffu;
+                q[g * 32 + i] = (uint8_t)(sign | (a > 0x7f800000u ? 0x7fu : a == 0x7f800000u ? 0x7eu : 0u));
+            } else {
+                float y = x[i] * scale; /* a power of two: exact unless it underflows, far below the smallest e4m3 */
+                if (y > 448.0f)
+                    y = 448.0f;
+                if (y < -448.0f)
+                    y = -448.0f;
+                q[g * 32 + i] = po_f32_to_fp8_e4m3fn(y);
+            }
+        }
+    }
+}
+
 /* -------------------------------------------------------------------- top-k */
 typedef struct {
     float score;

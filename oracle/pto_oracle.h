@@ -98,6 +98,8 @@ void po_gemm_f16f32(float *C, const uint16_t *A, const uint16_t *B, int m, int n
  * packed two per byte, element 2i in the low nibble (pack_two_fp4, tmatmul_mx/gen_data.py:74-84; the operand then has
  * k/2 bytes per row). */
 float po_fp8_e4m3fn_to_f32(uint8_t v);
+uint8_t po_f32_to_fp8_e4m3fn(float x);
+void po_quant_mxfp8_e4m3(uint8_t *q, uint8_t *e8m0, float *amax_out, float *scale_out, const float *src, size_t n);
 float po_fp8_e5m2_to_f32(uint8_t v);
 float po_fp4_e2m1_to_f32(uint8_t nibble);
 void po_mx_gemm(float *C, const uint8_t *A, const uint8_t *B, const uint8_t *SA, const uint8_t *SB, int m, int n, int k,

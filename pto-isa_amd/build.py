@@ -17,7 +17,7 @@ OUT = os.path.join(HERE, "libpto_amd.so")
 # libpto_st.so: the same sources with the tuning hooks compiled in (PTO_ST_HOOKS) plus the single-tile test programs; what
 # the parity tests load to drive single instructions and kernel variants.  Not part of the product.
 OUT_ST = os.path.join(HERE, "libpto_st.so")
-SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w4.hip", "pto_gemm_mx.hip", "pto_gemm_mxw4.hip", "pto_elementwise.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_fa_w8m16.hip"]
+SOURCES = ["pto_core.hip", "pto_gemm.hip", "pto_gemm_w4.hip", "pto_gemm_mx.hip", "pto_gemm_mxw4.hip", "pto_elementwise.hip", "pto_quant.hip", "pto_topk.hip", "pto_mla.hip", "pto_fa.hip", "pto_fa_w8.hip", "pto_fa_w8m16.hip"]
 ST_ONLY_SOURCES = ["pto_optest.hip", "pto_optest_matmul.hip"]
 # sources of libpto_st.so that differ from the product's objects (they hold a hook); the others are linked as they are
 HOOK_SOURCES = ["pto_gemm.hip", "pto_gemm_w4.hip", "pto_gemm_mx.hip", "pto_fa.hip"]

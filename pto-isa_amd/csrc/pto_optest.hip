@@ -115,6 +115,43 @@ __global__ __launch_bounds__(kBlockThreads) AICORE void TriMask(__gm__ float *ou
     TSTORE(go, x);
 }
 
+// ---- TQUANT<QuantType::MXFP8>: the ND-mode program of the reference's test (runTQuant<rows, cols, 0>,
+// tests/npu/a5/src/st/testcase/tquant/tquant_kernel.cpp:27-80): TLOAD -> TQUANT -> TSTORE of the exponents and of the fp8 tile ----
+template <int R, int C>
+__global__ __launch_bounds__(kBlockThreads) AICORE void TQuantMx(__gm__ uint8_t *outE8, __gm__ uint8_t *outFp8, __gm__ float *outMax,
+                                                                 __gm__ float *outScaling, __gm__ const float *in, int validRows,
+                                                                 int validCols)
+{
+    constexpr int kGroups = R * (C / 32);
+    using SrcTile = Tile<TileType::Vec, float, R, C, BLayout::RowMajor, -1, -1, SLayout::NoneBox, 512, PadValue::Zero>;
+    using Fp8Tile = Tile<TileType::Vec, int8_t, R, C, BLayout::RowMajor, R, C, SLayout::NoneBox, 512, PadValue::Zero>;
+    using E8Tile = Tile<TileType::Vec, uint8_t, 1, kGroups, BLayout::RowMajor, -1, -1, SLayout::NoneBox, 512, PadValue::Zero>;
+    using MaxTile = Tile<TileType::Vec, float, 1, kGroups, BLayout::RowMajor, -1, -1>;
+    using SrcGlobal = GlobalTensor<float, Shape<1, 1, 1, DYNAMIC, DYNAMIC>, Stride<1, 1, 1, DYNAMIC, 1>>;
+    SrcTile srcTile(validRows, validCols), scalingTile(validRows, validCols);
+    Fp8Tile fp8Tile;
+    E8Tile e8Tile(1, kGroups);
+    MaxTile maxTile(1, kGroups);
+    SrcGlobal srcGlobal(const_cast<float *>(in), Shape<1, 1, 1, DYNAMIC, DYNAMIC>(validRows, validCols),
+                        Stride<1, 1, 1, DYNAMIC, 1>(validCols));
+    GmND<uint8_t, 1, kGroups> e8Global(outE8);
+    GmND<int8_t, R, C> fp8Global(reinterpret_cast<__gm__ int8_t *>(outFp8));
+    GmND<float, 1, kGroups> maxGlobal(outMax);
+    GmND<float, R, C> scalingGlobal(outScaling);
+    TLOAD(srcTile, srcGlobal);
+    TLOAD(scalingTile, srcGlobal); // defined contents beyond the first kGroups entries
+    set_flag(PIPE_MTE2, PIPE_V, EVENT_ID0);
+    wait_flag(PIPE_MTE2, PIPE_V, EVENT_ID0);
+    TQUANT<QuantType::MXFP8, Fp8Tile, SrcTile, E8Tile, MaxTile>(fp8Tile, srcTile, &e8Tile, &maxTile, &scalingTile);
+    set_flag(PIPE_V, PIPE_MTE3, EVENT_ID0);
+    wait_flag(PIPE_V, PIPE_MTE3, EVENT_ID0);
+    TSTORE(e8Global, e8Tile);
+    TSTORE(fp8Global, fp8Tile);
+    TSTORE(maxGlobal, maxTile);
+    scalingTile = SrcTile(R, C);
+    TSTORE(scalingGlobal, scalingTile);
+}
+
 // ---- mask-form TGATHER on a [16, 64] tile of 16-bit elements ----
 template <MaskPattern P, int DIV>
 AICORE inline void GatherMaskBody(__gm__ uint16_t *out, __gm__ const uint16_t *in)
@@ -693,6 +730,27 @@ extern "C" int pto_st_tgather_mask_b16_16x64(void *stream, uint16_t *out, const 
         return PTO_ERR_BAD_ARG;
     GatherMask<<<dim3(1), dim3(kBlockThreads), 0, static_cast<hipStream_t>(stream)>>>(out, src, pattern);
     return pto_amd::check_launch();
+}
+
+// shape: 0 = 32 x 32, 1 = 32 x 64, 2 = 64 x 128, 3 = 128 x 128 (the ND cases of the reference's test, tquant/main.cpp:236-251)
+extern "C" int pto_st_tquant_mxfp8(void *stream, uint8_t *out_e8m0, uint8_t *out_fp8, float *out_max, float *out_scaling, const float *src,
+                                   int shape, int valid_rows, int valid_cols)
+{
+    PTO_ST_NONNULL(out_e8m0, out_fp8, out_max, out_scaling, src);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define PTO_ST_TQUANT_CASE(ID, R, C)                                                                                          \
+    if (shape == ID) {                                                                                                        \
+        if (valid_rows < 1 || valid_rows > R || valid_cols < 1 || valid_cols > C)                                             \
+            return PTO_ERR_BAD_ARG;                                                                                           \
+        TQuantMx<R, C><<<dim3(1), dim3(kBlockThreads), 0, st>>>(out_e8m0, out_fp8, out_max, out_scaling, src, valid_rows, valid_cols); \
+        return pto_amd::check_launch();                                                                                       \
+    }
+    PTO_ST_TQUANT_CASE(0, 32, 32)
+    PTO_ST_TQUANT_CASE(1, 32, 64)
+    PTO_ST_TQUANT_CASE(2, 64, 128)
+    PTO_ST_TQUANT_CASE(3, 128, 128)
+#undef PTO_ST_TQUANT_CASE
+    return PTO_ERR_BAD_ARG;
 }
 
 extern "C" int pto_st_mgather_b16_8x128(void *stream, uint16_t *out, const uint16_t *gm, const int32_t *idx, int gm_elems)

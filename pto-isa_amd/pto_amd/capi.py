@@ -21,6 +21,7 @@ SYMBOLS = {
     "pto_gemm_mxfp8": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 5),
     "pto_gemm_mxfp4": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 4),
     "pto_topk_f32": (C.c_int, [C.c_void_p] * 5 + [C.c_int] * 4),
+    "pto_quant_mxfp8_f32": (C.c_int, [C.c_void_p] * 4 + [C.c_size_t] * 2),
     "pto_attention_auto_f32": (C.c_int, [C.c_void_p] * 5 + [C.c_int] * 4),
     "pto_mla_attention_f32_s64_d32_r16": (C.c_int, [C.c_void_p] * 9 + [C.c_int] * 2),
     "pto_fa_fwd_f16": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 7),
@@ -52,6 +53,7 @@ ST_SYMBOLS = {
     "pto_st_matmul_s8_128x128x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_f32_128x32x256": (C.c_int, [C.c_void_p] * 4 + [C.c_int]),
     "pto_st_matmul_mx_128x256x128": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 3),
+    "pto_st_tquant_mxfp8": (C.c_int, [C.c_void_p] * 6 + [C.c_int] * 3),
     "pto_st_matmul_mx_bias_128x256x128": (C.c_int, [C.c_void_p] * 7 + [C.c_int] * 2),
     "pto_st_vec_op_typed_64x128": (C.c_int, [C.c_void_p] * 5 + [C.c_float, C.c_int, C.c_int]),
     "pto_st_matmul_vec_operands_f16_64x64x128": (C.c_int, [C.c_void_p] * 5),

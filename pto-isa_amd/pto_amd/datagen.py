@@ -120,6 +120,43 @@ def fp8_encode(x, fmt):
     return order[pick].astype(np.uint8)
 
 
+SEED_QUANT = 20260131
+
+
+def quant_input(rows, cols, spread=12, specials=True):
+    """fp32 [rows, cols] for the MXFP8 quantiser: N(0, 1) with every group of 32 multiplied by its own power of two in
+    2^[-spread, spread]; with `specials`, a few groups are made all zero, tiny (below 2^-119, fp32 denormals included),
+    huge, or get an infinity, a NaN or a -0."""
+    assert cols % 32 == 0
+    r = _rng(SEED_QUANT + rows * 131 + cols)
+    x = r.standard_normal(size=(rows, cols // 32, 32), dtype=np.float32)
+    x *= np.exp2(r.integers(-spread, spread + 1, size=(rows, cols // 32, 1))).astype(np.float32)
+    if specials:
+        g = x.reshape(-1, 32)
+        n = g.shape[0]
+        pick = r.permutation(n)[:min(n, 48)]
+        for j, gi in enumerate(pick):
+            kind = j % 8
+            if kind == 0:
+                g[gi] = 0.0
+            elif kind == 1:
+                g[gi] = (r.standard_normal(32) * 1e-40).astype(np.float32)
+            elif kind == 2:
+                g[gi] = (r.standard_normal(32) * 2.0 ** -122).astype(np.float32)
+            elif kind == 3:
+                g[gi] = (r.standard_normal(32) * 1e38).clip(-3.4e38, 3.4e38).astype(np.float32)
+            elif kind == 4:
+                g[gi, r.integers(0, 32)] = np.inf if j % 16 < 8 else -np.inf
+            elif kind == 5:
+                g[gi, r.integers(0, 32)] = np.nan
+                g[gi, r.integers(0, 32)] = -np.inf
+            elif kind == 6:
+                g[gi, ::3] = -0.0
+            else:
+                g[gi] = np.float32(448.0) * np.sign(g[gi])          # every element at the top of the range
+    return x.reshape(rows, cols)
+
+
 def mx_inputs(m, n, k, fmt, dist="uniform", scale_lo=127, scale_hi=130):
     """Operands of the MX GEMMs: A [m,k], B [n,k] fp8 bytes (fmt 0 e4m3, 1 e5m2) or [m,k/2], [n,k/2] packed fp4 (fmt 4),
     SA [m,k/32], SB [n,k/32] e8m0 bytes.  For fp4 "uniform" and "integer" draw integers in [-6, 6) as the reference's

@@ -631,3 +631,83 @@ def test_mla_oracle_closed_forms(oracle):
     assert np.max(np.abs(out - np.broadcast_to(want, out.shape))) < 1e-6
     # the acceptance test counts what it should
     assert oracle.mla_verify_allclose(np.array([1.0, 2.0, np.nan, 0.0]), np.array([1.0001, 2.1, 0.0, 0.0])) == 2
+
+
+# ---------------------------------------------------------------- MXFP8 quantisation (TQUANT<QuantType::MXFP8>)
+def _e4m3_grid():
+    tab = datagen.fp8_values(0)
+    vals = np.sort(np.unique(tab[np.isfinite(tab)]))
+    return tab, vals
+
+
+def test_fp8_e4m3_encoder_against_torch_and_the_value_table(oracle):
+    """The oracle's fp32 -> e4m3fn encoder: every representable value maps to its own byte, every midpoint between two
+    neighbours goes to the one with the even code (ties) and its fp32 neighbours to the nearer value, random values agree
+    with torch's float8_e4m3fn cast, magnitudes above 448 saturate, NaN keeps its sign."""
+    import torch
+    tab, vals = _e4m3_grid()
+    mids = ((vals[:-1] + vals[1:]) / 2).astype(np.float32)            # exact in fp32
+    rng = np.random.default_rng(3)
+    x = np.concatenate([vals.astype(np.float32), mids, np.nextafter(mids, np.float32(np.inf)), np.nextafter(mids, np.float32(-np.inf)),
+                        rng.uniform(-448, 448, 30000).astype(np.float32), (rng.standard_normal(30000) * 0.02).astype(np.float32)])
+    got = oracle.fp8_e4m3_encode(x)
+    want = torch.from_numpy(x).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(got, want)
+    # nearest value by brute force over the table (independent of any cast); at a tie the even code
+    dec = tab[got].astype(np.float64)
+    best = np.min(np.abs(x.astype(np.float64)[:, None] - vals[None, :]), axis=1)
+    assert np.array_equal(np.abs(dec - x.astype(np.float64)), best)
+    tie = oracle.fp8_e4m3_encode(mids)
+    assert not (tie & 1).any()
+    sat = oracle.fp8_e4m3_encode(np.array([448, 448.5, 479, 480, 1e30, np.inf, -449, -np.inf], dtype=np.float32))
+    assert list(sat) == [0x7e] * 6 + [0xfe] * 2
+    nan = oracle.fp8_e4m3_encode(np.array([np.nan, -np.nan], dtype=np.float32))
+    assert list(nan & 0x7f) == [0x7f, 0x7f]
+
+
+def test_quant_mxfp8_oracle_closed_forms(oracle):
+    """Scale byte = floor(log2(amax)) + 119; elements = e4m3(x * 2^(127 - scale byte)) computed with torch's cast; the
+    largest element of a group lands in [256, 448]; dequantised values are within 2^-4 relative (half a step of a 3-bit
+    mantissa) of every element that is not far below its group's maximum; scaling a group by a power of two moves only
+    the scale byte."""
+    import torch
+    rows, cols = 37, 1024
+    x = datagen.quant_input(rows, cols, specials=False)
+    q, s, amax, scale = oracle.quant_mxfp8(x, with_stats=True)
+    g = np.abs(x).reshape(rows, cols // 32, 32).max(axis=2)
+    assert np.array_equal(amax, g)
+    _, ex = np.frexp(g)
+    assert np.array_equal(s, (ex - 1 + 119).astype(np.uint8))
+    assert np.array_equal(scale, np.exp2(127.0 - s.astype(np.float64)).astype(np.float32))
+    y = np.clip(x.astype(np.float64) * np.repeat(np.exp2(127.0 - s.astype(np.float64)), 32, axis=1), -448, 448).astype(np.float32)
+    assert np.array_equal(q, torch.from_numpy(y).to(torch.float8_e4m3fn).view(torch.uint8).numpy())
+    tab = datagen.fp8_values(0)
+    top = np.abs(tab[q]).reshape(rows, cols // 32, 32).max(axis=2)
+    assert top.min() >= 256 and top.max() <= 448
+    deq = tab[q] * np.repeat(np.exp2(s.astype(np.float64) - 127.0), 32, axis=1)
+    big = np.abs(x) >= np.repeat(g, 32, axis=1) * 2.0 ** -7          # normal e4m3 range below the group's top
+    clipped = np.abs(y) >= 448
+    err = np.abs(deq - x)[big & ~clipped] / np.abs(x)[big & ~clipped]
+    assert err.max() <= 2.0 ** -4
+    q2, s2 = oracle.quant_mxfp8(x * np.float32(2.0 ** 5))
+    assert np.array_equal(q2, q) and np.array_equal(s2.astype(int), s.astype(int) + 5)
+
+
+def test_quant_mxfp8_oracle_special_groups(oracle):
+    """Zero and tiny groups: scale byte 0, factor 2^127; groups with an infinity or NaN: scale byte 0xff, NaN -> NaN,
+    infinities -> +-448, finite -> signed zero; an element at -0 stays -0."""
+    z = np.zeros((1, 32), dtype=np.float32)
+    q, s = oracle.quant_mxfp8(z)
+    assert s[0, 0] == 0 and not q.any()
+    t = np.full((1, 32), 2.0 ** -125, dtype=np.float32)
+    t[0, 1] = -2.0 ** -121
+    q, s, _, scale = oracle.quant_mxfp8(t, with_stats=True)
+    assert s[0, 0] == 0 and scale[0, 0] == np.float32(2.0 ** 127)
+    assert q[0, 0] == 0x48 and q[0, 1] == 0xe8          # 2^-125 * 2^127 = 4 -> 0.1001.000; -2^-121 * 2^127 = -64 -> 1.1101.000
+    w = np.ones((1, 64), dtype=np.float32)
+    w[0, 3], w[0, 4], w[0, 5], w[0, 6] = np.inf, -np.inf, np.nan, -5.0
+    w[0, 40] = -0.0
+    q, s = oracle.quant_mxfp8(w)
+    assert s[0, 0] == 0xff and s[0, 1] == 127 - 8
+    assert q[0, 3] == 0x7e and q[0, 4] == 0xfe and (q[0, 5] & 0x7f) == 0x7f and q[0, 6] == 0x80 and q[0, 0] == 0
+    assert q[0, 40] == 0x80 and q[0, 41] == 0x78         # 1.0 * 2^8 = 256 -> 0.1111.000
