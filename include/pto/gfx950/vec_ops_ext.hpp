@@ -322,7 +322,9 @@ PTO_DEV void TPACK_IMPL(DstT &dst, SrcT &src)
 
 // TQUANT (the a2a3 form, npu/a2a3/TQuant.hpp:26-52): src = src * scale[row] (+ offset[row]), in place as there, then
 // rounded to the nearest integer (ties to even) and saturated to int8 (symmetric) or uint8 (asymmetric)
-enum class QuantType { MXFP8, INT8_SYM, INT8_ASYM }; // npu/a5/TQuant.hpp:22-27
+// (the a2a3 tree's enumerators keep their values, which appear in the names of its launchers' instantiations; the a5 tree
+// puts MXFP8 first: npu/a5/TQuant.hpp:22-27, npu/a2a3/TQuant.hpp)
+enum class QuantType { INT8_SYM, INT8_ASYM, MXFP8 };
 enum class VecStoreMode { ND, NZ };                  // npu/a5/TQuant.hpp:29-33
 template <QuantType quant, typename DstT, typename SrcT, typename ParaT>
 PTO_DEV void TQUANT_IMPL(DstT &dst, SrcT &src, ParaT &scale, ParaT *offset = nullptr)
