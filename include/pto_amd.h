@@ -84,7 +84,7 @@ int pto_gemm_mxfp4(void *stream, void *c, const uint8_t *a, const uint8_t *b, co
  * largest |x|, scale byte = E - 8, q = e4m3(clip(x * 2^(127 - scale byte), +-448)) rounded to nearest even, so that the
  * group's largest element lands in [256, 448].  Groups holding an infinity or a NaN: scale byte 0xff, NaN -> NaN (0x7f
  * with the sign), +-inf -> +-448, finite -> +-0.  Groups whose largest |x| is below 2^-119 (all zeros included): scale
- * byte 0, factor 2^127. */
+ * byte 0, factor 2^127.  src aligned to 16 bytes, q to 4 (else PTO_ERR_UNSUPPORTED). */
 int pto_quant_mxfp8_f32(void *stream, uint8_t *q, uint8_t *scale, const float *src, size_t rows, size_t cols);
 
 /* Row-wise top-k.  src [rows, ld] fp32, the first valid_cols columns of every row are scored; in_idx [valid_cols] uint32

@@ -146,11 +146,13 @@ int launch_cvt(void *stream, D *dst, const float *src, size_t n, int mode)
         return PTO_ERR_BAD_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const size_t full = n / kCvtTile, tail = n % kCvtTile;
+    // (the streaming kernel for buffers aligned to its accesses: 16-byte loads, 8-byte stores)
+    const bool aligned = reinterpret_cast<uintptr_t>(src) % 16 == 0 && reinterpret_cast<uintptr_t>(dst) % 8 == 0;
     // the grid's x extent is limited to 2^31-1 blocks; stay far below it per launch
     constexpr size_t kMaxBlocks = 1u << 30;
     for (size_t t0 = 0; t0 < full; t0 += kMaxBlocks) {
         const size_t nb = full - t0 < kMaxBlocks ? full - t0 : kMaxBlocks;
-        if (mode == PTO_CAST_RINT)
+        if (mode == PTO_CAST_RINT && aligned)
             CvtF32Stream<D><<<dim3((unsigned)nb), dim3(kBlockThreads), 0, st>>>(dst, src, t0);
         else
             CvtF32<D, false><<<dim3((unsigned)nb), dim3(kBlockThreads), 0, st>>>(dst, src, n, t0, mode);

@@ -102,8 +102,8 @@ extern "C" int pto_quant_mxfp8_f32(void *stream, uint8_t *q, uint8_t *scale, con
         return PTO_OK;
     if (!q || !scale || !src)
         return PTO_ERR_BAD_ARG;
-    if (cols % 32)
-        return PTO_ERR_UNSUPPORTED;
+    if (cols % 32 || reinterpret_cast<uintptr_t>(src) % 16 || reinterpret_cast<uintptr_t>(q) % 4)
+        return PTO_ERR_UNSUPPORTED; // whole groups; 16-byte loads and 4-byte stores at their natural alignment
     if (rows > ((size_t)1 << 62) / cols)
         return PTO_ERR_UNSUPPORTED;
     const size_t n = rows * cols, full = n / kQuantTile, tail = n % kQuantTile;

@@ -124,3 +124,13 @@ def test_tquant_mxfp8_tile_instruction(oracle, shape, R, C, vr, vc):
     ordinary = we.reshape(-1) != 0xff                      # a group with inf / NaN: the factor is the bit pattern 0xff
     assert np.array_equal(got_scale[ordinary], wscale.reshape(-1)[ordinary])
     assert np.all(got_scale[~ordinary].view(np.uint32) == 0xff)
+
+
+def test_quant_mxfp8_refuses_pointers_below_the_alignment_of_its_accesses():
+    lib = capi.load()
+    d = torch.zeros(128, dtype=torch.float32, device="cuda:0")
+    o = torch.zeros(128, dtype=torch.uint8, device="cuda:0")
+    assert lib.pto_quant_mxfp8_f32(None, o.data_ptr(), o.data_ptr(), d.data_ptr() + 4, 1, 64) == capi.ERR_UNSUPPORTED
+    assert lib.pto_quant_mxfp8_f32(None, o.data_ptr() + 2, o.data_ptr(), d.data_ptr(), 1, 64) == capi.ERR_UNSUPPORTED
+    assert lib.pto_quant_mxfp8_f32(None, o.data_ptr(), o.data_ptr() + 1, d.data_ptr(), 1, 64) == capi.OK
+    torch.cuda.synchronize()
